@@ -1,0 +1,108 @@
+/*
+ * libkeops_hip - C ABI of the MI355X (gfx950) map-reduce backend.
+ *
+ * These entry points are what the reference's two FFI surfaces for its GPU path bind to:
+ *   (1) the ctypes call  Compile(target_file, cu_code, use_half, use_fast_math, device_id,
+ *       cuda_include_path)  of keopscore/keopscore/binders/nvrtc/nvrtc_jit.cpp:38-136
+ *       (called from keopscore/keopscore/binders/nvrtc/Gpu_link_compile.py:78-91), and
+ *   (2) the pybind11 class KeOps_module_{float,double}(device_id, nargs, target_file) with its
+ *       __call__  (pykeops/pykeops/common/keops_io/pykeops_nvrtc.cpp:13-103), i.e.
+ *       KeOps_module<TYPE>::launch_kernel of keopscore/keopscore/binders/nvrtc/keops_nvrtc.cpp:328-643.
+ *
+ * Conventions: plain C types only; every pointer argument is borrowed for the duration of the
+ * call; functions return 0 on success and a non-zero code on failure, with a human-readable
+ * message available from keops_hip_last_error() (thread-local).  No exceptions cross the ABI.
+ * A module must not be launched from two threads at once (same rule as the reference, whose
+ * module owns a per-module argument buffer); distinct modules are independent.
+ */
+#ifndef KEOPS_HIP_H
+#define KEOPS_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Version of this ABI (bumped on any signature change). */
+int keops_hip_abi_version(void);
+
+/* sha256 of the embedded kernel templates and host code this library was built from; part of the
+   key of the on-disk JIT cache (the reference hashes its own version into the tag,
+   keopscore/keopscore/binders/LinkCompile.py:19-35). */
+const char* keops_hip_templates_digest(void);
+
+/* Number of visible HIP devices (0 when no GPU / no driver). */
+int keops_hip_device_count(void);
+
+/*
+ * JIT-compile a kernel module with hiprtc and write it to target_file.
+ * Replaces Compile() of nvrtc_jit.cpp:38-136.  hip_src is the generated plug-in (formula body +
+ * geometry macros) that #includes one of the library's embedded kernel templates
+ * ("keops_conv.h", ...).  The target architecture is taken from device_id when a device is
+ * present, else from the environment variable KEOPS_HIP_ARCH, else "gfx950".
+ * File format: [u64 code_size][code object][u64 meta_size][meta text]; the meta text is the
+ * "//@keops key=value" lines of hip_src.  Returns 0 or the hiprtcResult.
+ */
+int keops_hip_compile(const char* target_file, const char* hip_src, int use_fast_math, int device_id);
+
+/*
+ * Load a compiled module on a device.  Replaces the KeOps_module<TYPE> constructor
+ * (keops_nvrtc.cpp:354-380).  Returns an opaque handle, or NULL on error.
+ */
+void* keops_hip_module_create(int device_id, int nargs, const char* target_file);
+
+/* Unload the module and free what it owns (keops_nvrtc.cpp:382-388). */
+void keops_hip_module_destroy(void* module);
+
+/*
+ * Run one map-reduce.  Replaces KeOps_module<TYPE>::launch_kernel (keops_nvrtc.cpp:390-643);
+ * arguments keep the reference's meaning and order:
+ *   tagHostDevice     must be 1 (all data pointers are device pointers)
+ *   dimY              total dimension of the reduced-index variables
+ *   nx, ny            sizes M and N of the i and j axes (per batch)
+ *   tagI              0: output indexed by i (reduce over j); 1: output indexed by j
+ *   tagZero           1: the formula is identically zero, out is filled with zeros
+ *   tag1D2D           0: one pass over the reduced axis; 1: force the column-slab (2D) scheme
+ *   dimred, dimout    accumulator and output dimensions per row
+ *   block_size        upper bound for the workgroup size (0 = module default)
+ *   use_chunk_mode    0 plain, 1 chunked inner reduction, 2 final chunks
+ *   indsi/j/p, dims*  argument indices and dimensions of the i, j and parameter variables
+ *   ranges            7 pointers: ranges_i, slices_i, redranges_j, ranges_j, slices_j, redranges_i
+ *                     (int64, on the data's device) and a HOST int64[6] with their row counts;
+ *                     ranges[6][0] == -1 means "no ranges" (LoadKeOps.py:11-12,194-202)
+ *   shapeout          shape of out; out has prod(shapeout) elements
+ *   args, argshapes   nargs device pointers; their shapes are concatenated in argshapes_flat,
+ *                     argndims[k] entries each
+ *   hip_stream        hipStream_t to launch on (NULL = default stream)
+ *   sync              non-zero: wait for completion before returning (the reference always does)
+ * Returns 0 or a hipError_t / negative library code.
+ */
+int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, int64_t ny, int tagI,
+                     int tagZero, int tag1D2D, int64_t dimred, int64_t block_size, int use_chunk_mode,
+                     const int* indsi, int ni, const int* indsj, int nj, const int* indsp, int np,
+                     int64_t dimout, const int64_t* dimsx, const int64_t* dimsy, const int64_t* dimsp,
+                     int64_t* const* ranges, const int64_t* shapeout, int nshapeout, void* out,
+                     void* const* args, const int64_t* argshapes_flat, const int* argndims,
+                     void* hip_stream, int sync);
+
+/* Message describing the last failure on the calling thread ("" if none). */
+const char* keops_hip_last_error(void);
+
+/* Text of a "//@keops" metadata entry of a loaded module (NULL if absent); for diagnostics. */
+const char* keops_hip_module_meta(void* module, const char* key);
+
+/*
+ * Average duration in milliseconds of the kernels launched by the most recent
+ * keops_hip_launch on this module, measured with HIP events on the launch stream when
+ * timing has been enabled with keops_hip_module_set_timing(module, 1); -1 if unavailable.
+ * No counterpart in the reference (it only has commented-out clock() stamps,
+ * keops_nvrtc.cpp:402-412); used by the benchmark's roofline measurement.
+ */
+void keops_hip_module_set_timing(void* module, int enabled);
+double keops_hip_module_last_kernel_ms(void* module);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KEOPS_HIP_H */

@@ -1,0 +1,119 @@
+"""ctypes binding of libkeops_hip.so (the C ABI of include/keops_hip.h).
+
+Plays the role of the reference's two native bindings: the ctypes call into nvrtc_jit.so
+(keopscore/keopscore/binders/nvrtc/Gpu_link_compile.py:78-91) and the pybind11 module
+pykeops_nvrtc (pykeops/pykeops/common/keops_io/pykeops_nvrtc.cpp:13-103).  The library is built
+in-tree by keops_amd/csrc/build_lib.py; a missing library is an error, there is no fallback.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libkeops_hip.so")
+_lib = None
+
+
+class KeOpsHipError(RuntimeError):
+    pass
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            from .csrc import build_lib
+
+            build_lib.build()
+        L = ctypes.CDLL(LIB_PATH)
+        L.keops_hip_last_error.restype = ctypes.c_char_p
+        L.keops_hip_templates_digest.restype = ctypes.c_char_p
+        L.keops_hip_module_create.restype = ctypes.c_void_p
+        L.keops_hip_module_create.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_char_p]
+        L.keops_hip_module_destroy.argtypes = [ctypes.c_void_p]
+        L.keops_hip_module_meta.restype = ctypes.c_char_p
+        L.keops_hip_module_meta.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
+        L.keops_hip_module_set_timing.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        L.keops_hip_module_last_kernel_ms.restype = ctypes.c_double
+        L.keops_hip_module_last_kernel_ms.argtypes = [ctypes.c_void_p]
+        L.keops_hip_compile.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int]
+        I64, P = ctypes.c_int64, ctypes.c_void_p
+        L.keops_hip_launch.argtypes = [
+            P, ctypes.c_int, I64, I64, I64, ctypes.c_int, ctypes.c_int, ctypes.c_int, I64, I64, ctypes.c_int,
+            P, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, I64, P, P, P, P, P, ctypes.c_int, P, P, P, P, P,
+            ctypes.c_int,
+        ]
+        _lib = L
+    return _lib
+
+
+def last_error():
+    return lib().keops_hip_last_error().decode(errors="replace")
+
+
+def device_count():
+    return lib().keops_hip_device_count()
+
+
+def templates_digest():
+    return lib().keops_hip_templates_digest().decode()
+
+
+def compile_module(target_file, source, use_fast_math=True, device_id=0):
+    rc = lib().keops_hip_compile(target_file.encode(), source.encode(), int(bool(use_fast_math)), int(device_id))
+    if rc != 0:
+        raise KeOpsHipError(f"kernel compilation failed (code {rc}): {last_error()}")
+
+
+def _iarr(ctype, values):
+    values = list(values)
+    return (ctype * max(1, len(values)))(*values)
+
+
+class Module:
+    """A loaded kernel module (KeOps_module_float/double of the reference)."""
+
+    def __init__(self, device_id, nargs, target_file):
+        self.handle = lib().keops_hip_module_create(int(device_id), int(nargs), target_file.encode())
+        if not self.handle:
+            raise KeOpsHipError(f"cannot load kernel module: {last_error()}")
+        self.nargs = nargs
+
+    def __del__(self):
+        h, self.handle = getattr(self, "handle", None), None
+        if h and _lib is not None:
+            _lib.keops_hip_module_destroy(h)
+
+    def meta(self, key):
+        v = lib().keops_hip_module_meta(self.handle, key.encode())
+        return None if v is None else v.decode()
+
+    def set_timing(self, enabled):
+        lib().keops_hip_module_set_timing(self.handle, int(bool(enabled)))
+
+    def last_kernel_ms(self):
+        return lib().keops_hip_module_last_kernel_ms(self.handle)
+
+    def __call__(self, tagHostDevice, dimy, nx, ny, tagI, tagZero, use_half, tag1D2D, dimred, block_size,
+                 use_chunk_mode, indsi, indsj, indsp, dimout, dimsx, dimsy, dimsp, ranges_ptr, shapeout,
+                 out_ptr, args_ptr, argshapes, stream=0, sync=False):
+        """Same positional arguments as KeOps_module_python::operator() (pykeops_nvrtc.cpp:17-23),
+        plus the stream to launch on and whether to wait for completion."""
+        if use_half:
+            raise KeOpsHipError("float16 data is not supported")
+        ci, cj, cp = _iarr(ctypes.c_int, indsi), _iarr(ctypes.c_int, indsj), _iarr(ctypes.c_int, indsp)
+        dx, dy, dp = _iarr(ctypes.c_int64, dimsx), _iarr(ctypes.c_int64, dimsy), _iarr(ctypes.c_int64, dimsp)
+        rp = (ctypes.c_void_p * 7)(*ranges_ptr)
+        so = _iarr(ctypes.c_int64, shapeout)
+        ap = (ctypes.c_void_p * max(1, len(args_ptr)))(*args_ptr)
+        flat = [int(d) for shp in argshapes for d in shp]
+        sh = _iarr(ctypes.c_int64, flat)
+        nd = _iarr(ctypes.c_int, [len(shp) for shp in argshapes])
+        rc = lib().keops_hip_launch(
+            self.handle, int(tagHostDevice), int(dimy), int(nx), int(ny), int(tagI), int(tagZero), int(tag1D2D),
+            int(dimred), int(block_size), int(use_chunk_mode), ci, len(indsi), cj, len(indsj), cp, len(indsp),
+            int(dimout), dx, dy, dp, rp, so, len(shapeout), ctypes.c_void_p(out_ptr), ap, sh, nd,
+            ctypes.c_void_p(stream), int(bool(sync)),
+        )
+        if rc != 0:
+            raise KeOpsHipError(f"kernel launch failed (code {rc}): {last_error()}")
+        return 0

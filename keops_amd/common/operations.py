@@ -1,0 +1,46 @@
+"""User-level reductions that are built on an internal one, and the matching output fix-up.
+
+Same behaviour as pykeops/pykeops/common/operations.py:7-35 (preprocess) and :38-87 (postprocess),
+written for torch tensors only.
+"""
+import torch
+
+
+def preprocess(reduction_op, formula2):
+    if reduction_op in ("SumSoftMaxWeight", "SoftMax"):
+        # sum_j exp(f_ij - m_i) [1, g_ij] through Max_SumShiftExpWeight, divided afterwards
+        return "Max_SumShiftExpWeight", "Concat(IntCst(1)," + formula2 + ")"
+    if reduction_op == "LogSumExp":
+        return ("Max_SumShiftExpWeight" if formula2 else "Max_SumShiftExp"), formula2
+    if reduction_op == "LogSumExpWeight":
+        if not formula2:
+            raise ValueError("LogSumExpWeight reduction requires a weight formula (given as formula2 kwarg)")
+        return "Max_SumShiftExpWeight", formula2
+    return reduction_op, formula2
+
+
+def postprocess(out, binding, reduction_op, nout, opt_arg, dtype):
+    if reduction_op in ("SumSoftMaxWeight", "SoftMax"):
+        return out[..., 2:] / out[..., 1][..., None]
+    if reduction_op in ("ArgMin", "ArgMax"):
+        return out.long()
+    if reduction_op in ("Min_ArgMin", "MinArgMin", "Max_ArgMax", "MaxArgMax"):
+        tmp = out.view(out.shape[:-1] + (2, -1))
+        return tmp[..., 0, :], tmp[..., 1, :].long()
+    if reduction_op == "KMin":
+        out = out.view(out.shape[:-1] + (opt_arg, -1))
+        return out.squeeze(-1) if out.shape[-1] == 1 else out
+    if reduction_op == "ArgKMin":
+        out = out.long().view(out.shape[:-1] + (opt_arg, -1))
+        return out.squeeze(-1) if out.shape[-1] == 1 else out
+    if reduction_op in ("KMin_ArgKMin", "KMinArgKMin"):
+        tmp = out.view(out.shape[:-1] + (opt_arg, 2, -1))
+        vals, idx = tmp[..., 0, :], tmp[..., 1, :].long()
+        if vals.shape[-1] == 1:
+            return vals.squeeze(-1), idx.squeeze(-1)
+        return vals, idx
+    if reduction_op in ("LogSumExp", "LogSumExpWeight"):
+        if out.shape[-1] == 2:
+            return (out[..., 0] + torch.log(out[..., 1]))[..., None]
+        return out[..., 0][..., None] + torch.log(out[..., 1:])
+    return out

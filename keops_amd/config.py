@@ -1,0 +1,35 @@
+"""Run-time knobs of the backend (counterpart of keopscore/keopscore/config: only the settings
+that still mean something on ROCm are kept; CUDA discovery has no equivalent here).
+
+Environment variables:
+  KEOPS_AMD_CACHE     folder of the on-disk JIT cache (default: <package>/build)
+  KEOPS_AMD_VERBOSE   "0" silences the informational messages
+  KEOPS_HIP_ARCH      offload architecture used when no GPU is visible (default gfx950)
+"""
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+
+verbose = os.environ.get("KEOPS_AMD_VERBOSE", "1") != "0"
+
+# chunked-mode thresholds, same values as keopscore/keopscore/config/chunks.py:19-35
+dimchunk = 64
+dim_treshold_chunk = 146
+specdims_use_chunk = [99, 100, 102, 120, 133, 138, 139, 140, 141, 142]
+dimfinalchunk = 64
+
+# workgroup geometry of the tiled kernels
+block_size = 256           # threads per workgroup (4 wavefronts)
+max_rows_per_lane = 4      # output rows held in the registers of one lane
+lds_tile_bytes = 16384     # LDS bytes of one staged column tile
+
+
+def get_build_folder():
+    folder = os.environ.get("KEOPS_AMD_CACHE") or os.path.join(_PKG, "build")
+    os.makedirs(folder, exist_ok=True)
+    return folder
+
+
+def message(*args, **kwargs):
+    if verbose:
+        print("[keops_amd]", *args, **kwargs)

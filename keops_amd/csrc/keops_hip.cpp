@@ -1,0 +1,670 @@
+// libkeops_hip: hiprtc JIT, module loading, shape/range preprocessing and kernel launches for the
+// MI355X map-reduce backend.  C ABI declared in include/keops_hip.h.
+//
+// Host-side counterpart of the reference's nvrtc binder:
+//   keopscore/keopscore/binders/nvrtc/nvrtc_jit.cpp:38-136      -> keops_hip_compile
+//   keopscore/keopscore/binders/nvrtc/keops_nvrtc.cpp:328-388   -> keops_hip_module_create/destroy
+//   keopscore/keopscore/binders/nvrtc/keops_nvrtc.cpp:390-643   -> keops_hip_launch
+//   keopscore/keopscore/include/Sizes.h, Ranges.h, ranges_utils.h -> ShapeTable / RangeSet below
+#include "../../include/keops_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <map>
+#include <mutex>
+#include <numeric>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include <unistd.h>
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string& msg) {
+  g_last_error = "[KeOps-HIP] " + msg;
+  return code == 0 ? -1 : code;
+}
+
+#define HIP_TRY(expr)                                                                          \
+  do {                                                                                         \
+    hipError_t e_ = (expr);                                                                    \
+    if (e_ != hipSuccess)                                                                      \
+      return fail((int)e_, std::string(#expr) + " failed: " + hipGetErrorString(e_));          \
+  } while (0)
+
+// ---- embedded kernel templates (generated from csrc/kernels/*.h at build time) -------------
+struct EmbeddedHeader {
+  const char* name;
+  const char* text;
+};
+#include "kernels_embedded.inc"
+
+// ---- module file -----------------------------------------------------------------------------
+
+std::string collect_meta(const char* src) {
+  std::istringstream in(src);
+  std::string line, meta;
+  while (std::getline(in, line)) {
+    if (line.rfind("//@keops ", 0) == 0) meta += line.substr(9) + "\n";
+  }
+  return meta;
+}
+
+std::map<std::string, std::string> parse_meta(const std::string& meta) {
+  std::map<std::string, std::string> kv;
+  std::istringstream in(meta);
+  std::string tok;
+  while (in >> tok) {
+    size_t eq = tok.find('=');
+    if (eq != std::string::npos) kv[tok.substr(0, eq)] = tok.substr(eq + 1);
+  }
+  return kv;
+}
+
+std::string target_arch(int device_id) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) == hipSuccess && n > 0) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device_id >= 0 && device_id < n ? device_id : 0) == hipSuccess) {
+      std::string a = prop.gcnArchName;  // e.g. "gfx950:sramecc+:xnack-"
+      return a.substr(0, a.find(':'));
+    }
+  } else {
+    (void)hipGetLastError();
+  }
+  const char* env = std::getenv("KEOPS_HIP_ARCH");
+  return env && *env ? env : "gfx950";
+}
+
+// ---- shape table: Sizes.h ----------------------------------------------------------------------
+
+struct ShapeTable {
+  int nargs = 0, nbatchdims = 0;
+  int64_t M = 0, N = 0, nbatches = 1;
+  std::vector<int64_t> shapes;  // (nargs+1) x (nbatchdims+3): [batch.., M, N, D]
+
+  int64_t* row(int k) { return shapes.data() + (size_t)k * (nbatchdims + 3); }
+
+  // Mirrors Sizes<TYPE>::Sizes / fill_shape / check_ranges (Sizes.h:86-150,176-330) with the
+  // checks enabled: a mismatch is an error instead of undefined behaviour.
+  int build(int nargs_, const std::vector<std::vector<int64_t>>& argshapes, int64_t nx, int64_t ny,
+            int64_t dimout, const std::vector<int>& indsI, const std::vector<int>& indsJ,
+            const std::vector<int>& indsP, const std::vector<int64_t>& dimsX,
+            const std::vector<int64_t>& dimsY, const std::vector<int64_t>& dimsP, std::string& err) {
+    nargs = nargs_;
+    int posI = indsI.empty() ? -1 : *std::min_element(indsI.begin(), indsI.end());
+    int posJ = indsJ.empty() ? -1 : *std::min_element(indsJ.begin(), indsJ.end());
+    int pos = std::max(posI, posJ);
+    nbatchdims = pos > -1 ? (int)argshapes[pos].size() - 2 : 0;
+    if (nbatchdims < 0) {
+      err = "argument " + std::to_string(pos) + " must have at least 2 dimensions";
+      return -2;
+    }
+    const int W = nbatchdims + 3;
+    shapes.assign((size_t)(nargs + 1) * W, 1);
+    shapes[nbatchdims] = nx;
+    shapes[nbatchdims + 1] = ny;
+    shapes[nbatchdims + 2] = dimout;
+
+    auto batch = [&](int i, const std::vector<int64_t>& shp) -> bool {
+      int64_t* r = row(i + 1);
+      for (int b = 0; b < nbatchdims; b++) {
+        r[b] = shp[b];
+        if (r[b] != 1) {
+          if (shapes[b] == 1) shapes[b] = r[b];
+          else if (shapes[b] != r[b]) {
+            err = "batch dimension " + std::to_string(b) + " of argument " + std::to_string(i) + " is " +
+                  std::to_string(r[b]) + " but was " + std::to_string(shapes[b]) + " or 1 in previous arguments";
+            return false;
+          }
+        }
+      }
+      return true;
+    };
+    auto check_var = [&](int i, int64_t dim, int cat, int64_t len) -> bool {
+      if (i < 0 || i >= nargs) { err = "variable index " + std::to_string(i) + " out of range"; return false; }
+      const auto& shp = argshapes[i];
+      const int want = cat == 2 ? nbatchdims + 1 : nbatchdims + 2;
+      if ((int)shp.size() != want) {
+        err = "argument " + std::to_string(i) + " has " + std::to_string(shp.size()) + " dimensions, expected " +
+              std::to_string(want);
+        return false;
+      }
+      if (!batch(i, shp)) return false;
+      int64_t* r = row(i + 1);
+      if (cat == 2) {
+        r[nbatchdims + 2] = shp[nbatchdims];
+      } else {
+        r[nbatchdims + cat] = shp[nbatchdims];
+        r[nbatchdims + 2] = shp[nbatchdims + 1];
+        if (shp[nbatchdims] != len) {
+          err = "argument " + std::to_string(i) + " has " + std::to_string(shp[nbatchdims]) + " rows, expected " +
+                std::to_string(len);
+          return false;
+        }
+      }
+      if (r[nbatchdims + 2] != dim) {
+        err = "argument " + std::to_string(i) + " has vector size " + std::to_string(r[nbatchdims + 2]) +
+              " but the formula expects " + std::to_string(dim);
+        return false;
+      }
+      return true;
+    };
+    for (size_t k = 0; k < indsI.size(); k++) if (!check_var(indsI[k], dimsX[k], 0, nx)) return -2;
+    for (size_t k = 0; k < indsJ.size(); k++) if (!check_var(indsJ[k], dimsY[k], 1, ny)) return -2;
+    for (size_t k = 0; k < indsP.size(); k++) if (!check_var(indsP[k], dimsP[k], 2, 0)) return -2;
+    M = shapes[nbatchdims];
+    N = shapes[nbatchdims + 1];
+    nbatches = 1;
+    for (int b = 0; b < nbatchdims; b++) nbatches *= shapes[b];
+    return 0;
+  }
+};
+
+// ranges_utils.h:3-15: flat index of row i of the full batch grid inside a variable whose batch
+// dimensions may be 1 (broadcast)
+int64_t broadcast_index(int64_t i, int nbatchdims, const int64_t* full_shape, const int64_t* shape) {
+  int64_t MN = shape[nbatchdims];
+  int64_t res = i % MN, step = MN, full_step = MN;
+  for (int b = nbatchdims; b > 0; b--) {
+    if (shape[b - 1] != 1) res += ((i / full_step) % shape[b - 1]) * step;
+    full_step *= full_shape[b - 1];
+    step *= shape[b - 1];
+  }
+  return res;
+}
+
+// ---- module ------------------------------------------------------------------------------------
+
+struct DeviceBuffer {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+  int reserve(size_t n) {
+    if (n <= bytes) return 0;
+    if (ptr) (void)hipFree(ptr);
+    ptr = nullptr;
+    bytes = 0;
+    hipError_t e = hipMalloc(&ptr, n);
+    if (e != hipSuccess) return fail((int)e, std::string("hipMalloc of workspace failed: ") + hipGetErrorString(e));
+    bytes = n;
+    return 0;
+  }
+  void release() {
+    if (ptr) (void)hipFree(ptr);
+    ptr = nullptr;
+    bytes = 0;
+  }
+};
+
+struct Module {
+  int device = 0, nargs = 0;
+  hipModule_t mod = nullptr;
+  std::map<std::string, std::string> meta;
+  std::map<std::string, hipFunction_t> fns;
+  int cu_count = 256;
+  // geometry baked into the code object
+  int block = 256, rows = 1, tile_j = 256, dimred = 1, dimout = 1, sizeof_t = 4, sizeof_acc = 4;
+  int nrowvars = 0, ncolvars = 0, nparvars = 0;
+  std::string scheme;
+  DeviceBuffer partial;  // column-slab partial accumulators
+  DeviceBuffer tables;   // lookup / offsets / synthesized ranges
+  void* pinned = nullptr;  // staging for the tables
+  size_t pinned_bytes = 0;
+  hipEvent_t tables_copied = nullptr;
+  bool tables_in_flight = false;
+  std::vector<int64_t> tables_key;  // batch mode: shape signature of the cached tables
+  int64_t cached_nblocks = 0;
+  // timing
+  bool timing = false;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  double last_ms = -1.0;
+
+  int meta_int(const char* k, int dflt) const {
+    auto it = meta.find(k);
+    return it == meta.end() ? dflt : std::atoi(it->second.c_str());
+  }
+  int fn(const char* name, hipFunction_t* f) {
+    auto it = fns.find(name);
+    if (it != fns.end()) { *f = it->second; return 0; }
+    hipError_t e = hipModuleGetFunction(f, mod, name);
+    if (e != hipSuccess) return fail((int)e, std::string("kernel '") + name + "' not found in module: " + hipGetErrorString(e));
+    fns[name] = *f;
+    return 0;
+  }
+};
+
+// Kernel argument block: must match struct KeopsParams of kernels/keops_conv.h.
+struct LaunchHeader {
+  int64_t nx, ny;
+  void* out;
+  void* partial;
+  int64_t slab_len;
+  int32_t nslabs, nbatchdims;
+  const int64_t* lookup;
+  const int64_t* slices_x;
+  const int64_t* ranges_y;
+  const int64_t* offsets;
+};
+
+int launch(Module& m, const char* kernel, unsigned gx, unsigned gy, const LaunchHeader& h, void* const* args,
+           hipStream_t stream) {
+  hipFunction_t f;
+  if (int rc = m.fn(kernel, &f)) return rc;
+  std::vector<char> buf(sizeof(LaunchHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs));
+  std::memcpy(buf.data(), &h, sizeof(h));
+  for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
+  size_t size = buf.size();
+  void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, buf.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+  if (gx == 0 || gy == 0) return 0;
+  HIP_TRY(hipModuleLaunchKernel(f, gx, gy, 1, (unsigned)m.block, 1, 1, 0, stream, nullptr, extra));
+  return 0;
+}
+
+int ensure_pinned(Module& m, size_t bytes) {
+  if (bytes <= m.pinned_bytes) return 0;
+  if (m.pinned) (void)hipHostFree(m.pinned);
+  m.pinned = nullptr;
+  m.pinned_bytes = 0;
+  HIP_TRY(hipHostMalloc(&m.pinned, bytes, hipHostMallocDefault));
+  m.pinned_bytes = bytes;
+  return 0;
+}
+
+}  // namespace
+
+// =================================================================================================
+
+extern "C" {
+
+int keops_hip_abi_version(void) { return 1; }
+
+const char* keops_hip_templates_digest(void) { return keops_templates_digest; }
+
+int keops_hip_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+const char* keops_hip_last_error(void) { return g_last_error.c_str(); }
+
+int keops_hip_compile(const char* target_file, const char* hip_src, int use_fast_math, int device_id) {
+  if (!target_file || !hip_src) return fail(-1, "keops_hip_compile: null argument");
+  std::vector<const char*> hdr_text, hdr_name;
+  for (const EmbeddedHeader* h = keops_embedded_headers; h->name; ++h) {
+    hdr_name.push_back(h->name);
+    hdr_text.push_back(h->text);
+  }
+  hiprtcProgram prog;
+  hiprtcResult r = hiprtcCreateProgram(&prog, hip_src, "keops_module.hip", (int)hdr_name.size(), hdr_text.data(), hdr_name.data());
+  if (r != HIPRTC_SUCCESS) return fail((int)r, std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r));
+  const std::string arch = "--offload-arch=" + target_arch(device_id);
+  std::vector<const char*> opts = {arch.c_str(), "-O3", "-std=c++17", "-fno-math-errno", "-ffp-contract=fast",
+                                   // packed FP32 instructions are kept out of every kernel of this library
+                                   "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  const std::string fm = std::string("-DKEOPS_FAST_MATH=") + (use_fast_math ? "1" : "0");
+  opts.push_back(fm.c_str());
+  r = hiprtcCompileProgram(prog, (int)opts.size(), opts.data());
+  if (r != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    hiprtcGetProgramLogSize(prog, &n);
+    std::string log(n, '\0');
+    if (n) hiprtcGetProgramLog(prog, &log[0]);
+    hiprtcDestroyProgram(&prog);
+    return fail((int)r, std::string("hiprtc compilation failed (") + hiprtcGetErrorString(r) + "):\n" + log);
+  }
+  size_t n = 0;
+  hiprtcGetCodeSize(prog, &n);
+  std::vector<char> code(n);
+  hiprtcGetCode(prog, code.data());
+  hiprtcDestroyProgram(&prog);
+
+  const std::string meta = collect_meta(hip_src);
+  const std::string tmp = std::string(target_file) + ".tmp" + std::to_string((long)getpid());
+  {
+    std::ofstream out(tmp, std::ios::binary);
+    if (!out) return fail(-1, "cannot write " + tmp);
+    uint64_t cs = code.size(), ms = meta.size();
+    out.write((const char*)&cs, sizeof(cs));
+    out.write(code.data(), (std::streamsize)cs);
+    out.write((const char*)&ms, sizeof(ms));
+    out.write(meta.data(), (std::streamsize)ms);
+  }
+  if (std::rename(tmp.c_str(), target_file) != 0) return fail(-1, std::string("cannot rename to ") + target_file);
+  return 0;
+}
+
+void* keops_hip_module_create(int device_id, int nargs, const char* target_file) {
+  std::ifstream in(target_file, std::ios::binary);
+  if (!in) {
+    fail(-1, std::string("cannot open module file ") + target_file);
+    return nullptr;
+  }
+  uint64_t cs = 0, ms = 0;
+  in.read((char*)&cs, sizeof(cs));
+  std::vector<char> code(cs);
+  in.read(code.data(), (std::streamsize)cs);
+  in.read((char*)&ms, sizeof(ms));
+  std::string meta(ms, '\0');
+  if (ms) in.read(&meta[0], (std::streamsize)ms);
+  if (!in) {
+    fail(-1, std::string("truncated module file ") + target_file);
+    return nullptr;
+  }
+  Module* m = new Module();
+  m->device = device_id < 0 ? 0 : device_id;
+  m->nargs = nargs;
+  m->meta = parse_meta(meta);
+  hipError_t e = hipSetDevice(m->device);
+  if (e == hipSuccess) e = hipModuleLoadData(&m->mod, code.data());
+  if (e != hipSuccess) {
+    fail((int)e, std::string("loading module on device ") + std::to_string(m->device) + " failed: " + hipGetErrorString(e));
+    delete m;
+    return nullptr;
+  }
+  int cus = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, m->device) == hipSuccess && cus > 0) m->cu_count = cus;
+  m->block = m->meta_int("block", 256);
+  m->rows = m->meta_int("rows", 1);
+  m->tile_j = m->meta_int("tile_j", 256);
+  m->dimred = m->meta_int("dimred", 1);
+  m->dimout = m->meta_int("dimout", 1);
+  m->sizeof_t = m->meta_int("sizeof_t", 4);
+  m->sizeof_acc = m->meta_int("sizeof_acc", 4);
+  m->nrowvars = m->meta_int("nrowvars", 0);
+  m->ncolvars = m->meta_int("ncolvars", 0);
+  m->nparvars = m->meta_int("nparvars", 0);
+  m->scheme = m->meta.count("scheme") ? m->meta["scheme"] : "conv";
+  return m;
+}
+
+void keops_hip_module_destroy(void* module) {
+  Module* m = (Module*)module;
+  if (!m) return;
+  (void)hipSetDevice(m->device);
+  if (m->tables_in_flight && m->tables_copied) (void)hipEventSynchronize(m->tables_copied);
+  m->partial.release();
+  m->tables.release();
+  if (m->pinned) (void)hipHostFree(m->pinned);
+  if (m->tables_copied) (void)hipEventDestroy(m->tables_copied);
+  if (m->ev0) (void)hipEventDestroy(m->ev0);
+  if (m->ev1) (void)hipEventDestroy(m->ev1);
+  if (m->mod) (void)hipModuleUnload(m->mod);
+  delete m;
+}
+
+const char* keops_hip_module_meta(void* module, const char* key) {
+  Module* m = (Module*)module;
+  if (!m || !key) return nullptr;
+  auto it = m->meta.find(key);
+  return it == m->meta.end() ? nullptr : it->second.c_str();
+}
+
+void keops_hip_module_set_timing(void* module, int enabled) {
+  Module* m = (Module*)module;
+  if (m) m->timing = enabled != 0;
+}
+
+double keops_hip_module_last_kernel_ms(void* module) {
+  Module* m = (Module*)module;
+  return m ? m->last_ms : -1.0;
+}
+
+int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, int64_t ny, int tagI,
+                     int tagZero, int tag1D2D, int64_t dimred, int64_t block_size, int use_chunk_mode,
+                     const int* indsi, int ni, const int* indsj, int nj, const int* indsp, int np,
+                     int64_t dimout, const int64_t* dimsx, const int64_t* dimsy, const int64_t* dimsp,
+                     int64_t* const* ranges, const int64_t* shapeout, int nshapeout, void* out,
+                     void* const* args, const int64_t* argshapes_flat, const int* argndims,
+                     void* hip_stream, int sync) {
+  (void)dimY; (void)block_size; (void)use_chunk_mode;
+  Module* mp = (Module*)module;
+  if (!mp) return fail(-1, "keops_hip_launch: null module");
+  Module& m = *mp;
+  if (tagHostDevice != 1) return fail(-1, "only device-resident arguments are supported (tagHostDevice must be 1)");
+  if (dimred != m.dimred || dimout != m.dimout)
+    return fail(-1, "dimred/dimout do not match the compiled module");
+  hipStream_t stream = (hipStream_t)hip_stream;
+  HIP_TRY(hipSetDevice(m.device));
+
+  int64_t sizeout = 1;
+  for (int k = 0; k < nshapeout; k++) sizeout *= shapeout[k];
+
+  if (tagZero) {
+    HIP_TRY(hipMemsetAsync(out, 0, (size_t)sizeout * m.sizeof_t, stream));
+    if (sync) HIP_TRY(hipStreamSynchronize(stream));
+    return 0;
+  }
+
+  // ---- shapes (Sizes.h) ----
+  std::vector<int> vI(indsi, indsi + ni), vJ(indsj, indsj + nj), vP(indsp, indsp + np);
+  std::vector<int64_t> dX(dimsx, dimsx + ni), dY(dimsy, dimsy + nj), dP(dimsp, dimsp + np);
+  std::vector<std::vector<int64_t>> argshapes(m.nargs);
+  {
+    const int64_t* p = argshapes_flat;
+    for (int k = 0; k < m.nargs; k++) {
+      argshapes[k].assign(p, p + argndims[k]);
+      p += argndims[k];
+    }
+  }
+  ShapeTable S;
+  std::string err;
+  if (int rc = S.build(m.nargs, argshapes, nx, ny, dimout, vI, vJ, vP, dX, dY, dP, err)) return fail(rc, err);
+  const int nb = S.nbatchdims;
+  const int64_t NX = S.nbatches * S.M, NY = S.nbatches * S.N;
+
+  // the kernel's "rows" are the output-indexed variables, its "columns" the reduced ones
+  const int64_t rows_total = tagI == 0 ? NX : NY;
+  const int64_t cols_total = tagI == 0 ? NY : NX;
+  const std::vector<int>& rowvars = tagI == 0 ? vI : vJ;
+  const std::vector<int>& colvars = tagI == 0 ? vJ : vI;
+  if ((int)rowvars.size() != m.nrowvars || (int)colvars.size() != m.ncolvars || (int)vP.size() != m.nparvars)
+    return fail(-1, "variable lists do not match the compiled module");
+  if (sizeout != rows_total * dimout)
+    return fail(-1, "output has " + std::to_string(sizeout) + " elements, expected " + std::to_string(rows_total * dimout));
+  if (rows_total == 0) return 0;
+
+  const bool user_ranges = ranges && ranges[6] && ranges[6][0] != -1;
+  if (user_ranges && nb > 0)
+    return fail(-1, "the 'ranges' argument (block-sparse mode) is not supported with batch processing");
+  const bool use_ranges = user_ranges || nb > 0;
+  const int64_t rows_per_block = (int64_t)m.block * m.rows;
+
+  if (m.timing) {
+    if (!m.ev0) { HIP_TRY(hipEventCreate(&m.ev0)); HIP_TRY(hipEventCreate(&m.ev1)); }
+  }
+  m.last_ms = -1.0;
+
+  LaunchHeader h{};
+  h.nx = rows_total;
+  h.ny = cols_total;
+  h.out = out;
+  h.nbatchdims = nb;
+  h.nslabs = 1;
+  h.slab_len = cols_total;
+
+  if (!use_ranges) {
+    // ---- dense scheme, optionally cut in column slabs ----
+    const int64_t row_blocks = (rows_total + rows_per_block - 1) / rows_per_block;
+    int64_t nslabs = 1;
+    const int64_t target_blocks = 4 * (int64_t)m.cu_count;
+    if (tag1D2D == 1 || row_blocks * 2 <= target_blocks) {
+      const int64_t max_slabs = std::max<int64_t>(1, cols_total / (4 * (int64_t)m.tile_j));
+      nslabs = std::min<int64_t>(max_slabs, (target_blocks + row_blocks - 1) / row_blocks);
+      if (tag1D2D == 1) nslabs = std::max<int64_t>(nslabs, std::min<int64_t>(max_slabs, 2));
+      nslabs = std::min<int64_t>(nslabs, 65535);
+    }
+    if (nslabs > 1) {
+      int64_t len = (cols_total + nslabs - 1) / nslabs;
+      len = ((len + m.tile_j - 1) / m.tile_j) * m.tile_j;
+      nslabs = (cols_total + len - 1) / len;
+      h.slab_len = len;
+    }
+    h.nslabs = (int32_t)nslabs;
+    if (nslabs > 1) {
+      if (int rc = m.partial.reserve((size_t)nslabs * rows_total * m.dimred * m.sizeof_acc)) return rc;
+      h.partial = m.partial.ptr;
+    }
+    if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
+    if (int rc = launch(m, "keops_conv_dense", (unsigned)row_blocks, (unsigned)nslabs, h, args, stream)) return rc;
+    if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
+    if (nslabs > 1) {
+      const int64_t gb = (rows_total + m.block - 1) / m.block;
+      if (int rc = launch(m, "keops_reduce_partials", (unsigned)gb, 1, h, args, stream)) return rc;
+    }
+  } else {
+    // ---- block-sparse / batched scheme (Ranges.h, keops_nvrtc.cpp:152-248) ----
+    const int64_t* rx_dev = nullptr;  // row ranges, device (user ranges only)
+    std::vector<int64_t> rx_host;     // row ranges on the host
+    int64_t nranges = 0;
+    const int64_t *slices_dev = nullptr, *ry_dev = nullptr;
+    const int nvars = m.nrowvars + m.ncolvars + m.nparvars;
+    std::vector<int64_t> synth;  // batch mode: [slices (nbatches)] [ranges_y (2*nbatches)]
+
+    if (user_ranges) {
+      const int sel = tagI == 0 ? 0 : 3;
+      nranges = ranges[6][sel];
+      rx_dev = ranges[sel];
+      slices_dev = ranges[sel + 1];
+      ry_dev = ranges[sel + 2];
+      rx_host.resize((size_t)2 * nranges);
+      // same synchronous read-back as the reference (keops_nvrtc.cpp:195-197)
+      if (nranges) HIP_TRY(hipMemcpyAsync(rx_host.data(), rx_dev, sizeof(int64_t) * 2 * nranges, hipMemcpyDeviceToHost, stream));
+      HIP_TRY(hipStreamSynchronize(stream));
+    } else {
+      // block-diagonal pattern, one range per batch (Ranges.h:40-86)
+      nranges = S.nbatches;
+      const int64_t R = tagI == 0 ? S.M : S.N, C = tagI == 0 ? S.N : S.M;
+      rx_host.resize((size_t)2 * nranges);
+      synth.resize((size_t)3 * nranges);
+      for (int64_t b = 0; b < nranges; b++) {
+        rx_host[2 * b] = b * R;
+        rx_host[2 * b + 1] = (b + 1) * R;
+        synth[b] = b + 1;
+        synth[nranges + 2 * b] = b * C;
+        synth[nranges + 2 * b + 1] = (b + 1) * C;
+      }
+    }
+
+    // lookup table: one entry per workgroup (keops_nvrtc.cpp:210-231)
+    int64_t nblocks = 0;
+    for (int64_t r = 0; r < nranges; r++) {
+      const int64_t len = rx_host[2 * r + 1] - rx_host[2 * r];
+      if (len < 0 || rx_host[2 * r] < 0 || rx_host[2 * r + 1] > rows_total)
+        return fail(-1, "row range " + std::to_string(r) + " is out of bounds");
+      nblocks += (len + rows_per_block - 1) / rows_per_block;
+    }
+
+    // batch mode tables only depend on the shapes: reuse them across calls
+    std::vector<int64_t> key;
+    bool reuse = false;
+    if (!user_ranges) {
+      key.push_back(tagI);
+      key.push_back(rows_per_block);
+      key.insert(key.end(), S.shapes.begin(), S.shapes.end());
+      reuse = key == m.tables_key && m.tables.ptr != nullptr;
+    }
+    const size_t n_lookup = (size_t)3 * nblocks, n_off = nb > 0 ? (size_t)nblocks * nvars : 0, n_syn = synth.size();
+    const size_t total = n_lookup + n_off + n_syn;
+    if (!reuse && total > 0) {
+      if (m.tables_in_flight) {
+        HIP_TRY(hipEventSynchronize(m.tables_copied));
+        m.tables_in_flight = false;
+      }
+      if (int rc = ensure_pinned(m, total * sizeof(int64_t))) return rc;
+      int64_t* lk = (int64_t*)m.pinned;
+      int64_t* off = lk + n_lookup;
+      int64_t* syn = off + n_off;
+      int64_t idx = 0;
+      for (int64_t r = 0; r < nranges; r++) {
+        const int64_t s = rx_host[2 * r], len = rx_host[2 * r + 1] - s;
+        for (int64_t j = 0; j < len; j += rows_per_block) {
+          lk[3 * idx] = r;
+          lk[3 * idx + 1] = s + j;
+          lk[3 * idx + 2] = s + j + std::min(rows_per_block, len - j);
+          idx++;
+        }
+      }
+      if (nb > 0) {
+        // per-block first-row offsets of every variable (keops_nvrtc.cpp:75-149, ranges_utils.h:27-91)
+        const int W = nb + 3;
+        const int64_t R = tagI == 0 ? S.M : S.N, C = tagI == 0 ? S.N : S.M;
+        const int rpos = tagI == 0 ? nb : nb + 1, cpos = tagI == 0 ? nb + 1 : nb;
+        std::vector<int64_t> shp(nb + 1);
+        for (int64_t k = 0; k < nblocks; k++) {
+          const int64_t rid = lk[3 * k];
+          const int64_t patch = lk[3 * k + 1] - rid * R;
+          int64_t* o = off + k * nvars;
+          int c = 0;
+          for (int v : rowvars) {
+            const int64_t* r = S.row(v + 1);
+            for (int b = 0; b < nb; b++) shp[b] = r[b];
+            shp[nb] = r[rpos];
+            o[c++] = patch + broadcast_index(rid * R, nb, S.shapes.data(), shp.data());
+          }
+          for (int v : colvars) {
+            const int64_t* r = S.row(v + 1);
+            for (int b = 0; b < nb; b++) shp[b] = r[b];
+            shp[nb] = r[cpos];
+            o[c++] = broadcast_index(rid * C, nb, S.shapes.data(), shp.data());
+          }
+          for (int v : vP) {
+            const int64_t* r = S.row(v + 1);
+            for (int b = 0; b < nb; b++) shp[b] = r[b];
+            shp[nb] = 1;
+            o[c++] = broadcast_index(rid, nb, S.shapes.data(), shp.data());
+          }
+          (void)W;
+        }
+      }
+      if (n_syn) std::memcpy(syn, synth.data(), n_syn * sizeof(int64_t));
+      if (int rc = m.tables.reserve(total * sizeof(int64_t))) return rc;
+      HIP_TRY(hipMemcpyAsync(m.tables.ptr, m.pinned, total * sizeof(int64_t), hipMemcpyHostToDevice, stream));
+      if (!m.tables_copied) HIP_TRY(hipEventCreateWithFlags(&m.tables_copied, hipEventDisableTiming));
+      HIP_TRY(hipEventRecord(m.tables_copied, stream));
+      m.tables_in_flight = true;
+      m.tables_key = key;
+      m.cached_nblocks = nblocks;
+    }
+    const int64_t* tab = (const int64_t*)m.tables.ptr;
+    h.lookup = tab;
+    h.offsets = nb > 0 ? tab + n_lookup : nullptr;
+    if (user_ranges) {
+      h.slices_x = slices_dev;
+      h.ranges_y = ry_dev;
+    } else {
+      h.slices_x = tab + n_lookup + n_off;
+      h.ranges_y = tab + n_lookup + n_off + nranges;
+    }
+    if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
+    if (user_ranges) {
+      const int64_t gb = (rows_total + m.block - 1) / m.block;
+      if (int rc = launch(m, "keops_fill_neutral", (unsigned)gb, 1, h, args, stream)) return rc;
+    }
+    if (int rc = launch(m, "keops_conv_ranges", (unsigned)nblocks, 1, h, args, stream)) return rc;
+    if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
+  }
+
+  if (m.timing) {
+    HIP_TRY(hipEventSynchronize(m.ev1));
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, m.ev0, m.ev1));
+    m.last_ms = ms;
+  }
+  if (sync) HIP_TRY(hipStreamSynchronize(stream));
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,328 @@
+"""Scalar SSA program ("low-level IR") that a formula tree lowers to.
+
+Every value is one scalar; vector-valued formula nodes become Python lists of value ids.  Values
+are hash-consed (common sub-expressions are shared), constants are folded, and a few algebraic
+peepholes keep the per-pair instruction count of the generated HIP code minimal:
+
+* ``exp(u)`` is emitted as the hardware base-2 exponential ``exp2(u * log2(e))`` and, when fast
+  math is allowed, the ``log2(e)`` factor is merged into any uniform (parameter-only) factor of
+  ``u``; the merged product is invariant in the pair loop, so one multiply per pair disappears.
+* negations are pushed outwards (they are free source modifiers on the VALU).
+
+The program is printed as straight-line C++ (``const T t7 = t3 * t5;``): with every index a
+compile-time constant the compiler keeps all values in VGPRs.
+"""
+from __future__ import annotations
+
+import math
+
+LOG2E = 1.4426950408889634
+LN2 = 0.6931471805599453
+
+# value "levels": how often a value changes in the map-reduce loop nest
+UNIFORM, PER_ROW, PER_PAIR = 0, 1, 2
+
+
+class Lir:
+    def __init__(self, row_cat=0, fast_math=True, dtype="float"):
+        self.row_cat = row_cat  # category (0 = i, 1 = j) of the variables indexed like the output
+        self.fast = bool(fast_math)
+        self.dtype = dtype
+        self.nodes = []  # (op, args...) tuples
+        self.level = []
+        self.index = {}
+        self.loads = {}  # (cat, ind) -> set of component indices actually read
+
+    # ------------------------------------------------------------------ construction
+    def _mk(self, key, level):
+        i = self.index.get(key)
+        if i is None:
+            i = len(self.nodes)
+            self.nodes.append(key)
+            self.level.append(level)
+            self.index[key] = i
+        return i
+
+    def _lvl(self, *ids):
+        return max(self.level[i] for i in ids)
+
+    def const(self, v):
+        v = float(v)
+        if v == 0.0:
+            v = 0.0  # merge -0.0
+        return self._mk(("const", v), UNIFORM)
+
+    def is_const(self, i, v=None):
+        n = self.nodes[i]
+        return n[0] == "const" and (v is None or n[1] == v)
+
+    def cval(self, i):
+        return self.nodes[i][1]
+
+    def load(self, cat, ind, k):
+        self.loads.setdefault((cat, ind), set()).add(k)
+        if cat == 2:
+            lvl = UNIFORM
+        elif cat == 3:
+            lvl = PER_PAIR  # chunk accumulator input (value computed by the kernel per pair)
+        else:
+            lvl = PER_ROW if cat == self.row_cat else PER_PAIR
+        return self._mk(("load", cat, ind, k), lvl)
+
+    def neg(self, a):
+        n = self.nodes[a]
+        if n[0] == "const":
+            return self.const(-n[1])
+        if n[0] == "neg":
+            return n[1]
+        if n[0] == "sub":
+            return self.sub(n[2], n[1])
+        return self._mk(("neg", a), self.level[a])
+
+    def add(self, a, b):
+        if self.is_const(a) and self.is_const(b):
+            return self.const(self.cval(a) + self.cval(b))
+        if self.is_const(a, 0.0):
+            return b
+        if self.is_const(b, 0.0):
+            return a
+        if self.nodes[b][0] == "neg":
+            return self.sub(a, self.nodes[b][1])
+        if self.nodes[a][0] == "neg":
+            return self.sub(b, self.nodes[a][1])
+        return self._mk(("add", a, b), self._lvl(a, b))
+
+    def sub(self, a, b):
+        if self.is_const(a) and self.is_const(b):
+            return self.const(self.cval(a) - self.cval(b))
+        if self.is_const(b, 0.0):
+            return a
+        if self.is_const(a, 0.0):
+            return self.neg(b)
+        if self.nodes[b][0] == "neg":
+            return self.add(a, self.nodes[b][1])
+        if a == b and self.fast:
+            return self.const(0.0)
+        return self._mk(("sub", a, b), self._lvl(a, b))
+
+    def mul(self, a, b):
+        na, nb = self.nodes[a], self.nodes[b]
+        if na[0] == "const" and nb[0] == "const":
+            return self.const(na[1] * nb[1])
+        for p, q in ((a, b), (b, a)):
+            if self.is_const(p, 1.0):
+                return q
+            if self.is_const(p, -1.0):
+                return self.neg(q)
+            if self.is_const(p, 0.0) and self.fast:
+                return self.const(0.0)
+        if na[0] == "neg" and nb[0] == "neg":
+            return self.mul(na[1], nb[1])
+        if na[0] == "neg":
+            return self.neg(self.mul(na[1], b))
+        if nb[0] == "neg":
+            return self.neg(self.mul(a, nb[1]))
+        if self.fast:
+            # hoisting: a factor that changes less often than its partner joins the partner's own
+            # slow-changing sub-factor, (u * (v * w)) -> ((u * v) * w) when level(u), level(v) < level(w),
+            # so that the slow product is computed outside the pair loop.
+            for p, q in ((a, b), (b, a)):
+                nq = self.nodes[q]
+                if nq[0] == "mul" and self.level[p] < self.level[q]:
+                    for lo, hi in ((nq[1], nq[2]), (nq[2], nq[1])):
+                        if self.level[lo] < self.level[q] and self.level[hi] == self.level[q]:
+                            return self.mul(self.mul(p, lo), hi)
+        if a > b:
+            a, b = b, a
+        return self._mk(("mul", a, b), self._lvl(a, b))
+
+    def fma(self, a, b, c):
+        """a*b + c; printed as a plain multiply-add (the compiler contracts it)."""
+        return self.add(self.mul(a, b), c)
+
+    def div(self, a, b):
+        if self.is_const(a) and self.is_const(b) and self.cval(b) != 0.0:
+            return self.const(self.cval(a) / self.cval(b))
+        if self.is_const(b, 1.0):
+            return a
+        if self.fast:
+            return self.mul(a, self.rcp(b))
+        return self._mk(("div", a, b), self._lvl(a, b))
+
+    def rcp(self, a):
+        if self.is_const(a) and self.cval(a) != 0.0:
+            return self.const(1.0 / self.cval(a))
+        return self._mk(("rcp", a), self.level[a])
+
+    def exp(self, a):
+        if self.is_const(a):
+            return self.const(math.exp(self.cval(a)))
+        if self.dtype == "float" and self.fast:
+            return self._mk(("exp2", self.mul(a, self.const(LOG2E))), self.level[a])
+        return self._mk(("exp", a), self.level[a])
+
+    def log(self, a):
+        if self.is_const(a) and self.cval(a) > 0:
+            return self.const(math.log(self.cval(a)))
+        if self.dtype == "float" and self.fast:
+            return self.mul(self._mk(("log2", a), self.level[a]), self.const(LN2))
+        return self._mk(("log", a), self.level[a])
+
+    def sqrt(self, a):
+        if self.is_const(a) and self.cval(a) >= 0:
+            return self.const(math.sqrt(self.cval(a)))
+        return self._mk(("sqrt", a), self.level[a])
+
+    def rsqrt0(self, a):
+        """x == 0 ? 0 : 1/sqrt(x)  (keops_rsqrt, math_functions.py:104-108)."""
+        if self.is_const(a):
+            v = self.cval(a)
+            return self.const(0.0 if v == 0 else 1.0 / math.sqrt(v))
+        return self._mk(("rsqrt0", a), self.level[a])
+
+    def abs(self, a):
+        if self.is_const(a):
+            return self.const(abs(self.cval(a)))
+        if self.nodes[a][0] == "neg":
+            return self.abs(self.nodes[a][1])
+        return self._mk(("abs", a), self.level[a])
+
+    def sign(self, a):
+        return self._mk(("sign", a), self.level[a])
+
+    def powi(self, a, m):
+        if m < 0:
+            return self.rcp(self.powi(a, -m))
+        if m == 0:
+            return self.const(1.0)
+        # square-and-multiply
+        result, base = None, a
+        while m:
+            if m & 1:
+                result = base if result is None else self.mul(result, base)
+            m >>= 1
+            if m:
+                base = self.mul(base, base)
+        return result
+
+    def call(self, fn, *args):
+        return self._mk(("call", fn) + tuple(args), self._lvl(*args))
+
+    # comparisons produce boolean values, only usable as the first argument of select
+    def lt(self, a, b):
+        return self._mk(("lt", a, b), self._lvl(a, b))
+
+    def le(self, a, b):
+        return self._mk(("le", a, b), self._lvl(a, b))
+
+    def eq(self, a, b):
+        return self._mk(("eq", a, b), self._lvl(a, b))
+
+    def ne(self, a, b):
+        return self._mk(("ne", a, b), self._lvl(a, b))
+
+    def select(self, c, a, b):
+        if a == b:
+            return a
+        return self._mk(("select", c, a, b), self._lvl(c, a, b))
+
+    # ------------------------------------------------------------------ printing
+    def live(self, outputs):
+        seen = set()
+        stack = list(outputs)
+        while stack:
+            i = stack.pop()
+            if i in seen:
+                continue
+            seen.add(i)
+            n = self.nodes[i]
+            if n[0] == "const" or n[0] == "load":
+                continue
+            start = 2 if n[0] == "call" else 1
+            stack.extend(n[start:])
+        return seen
+
+    def count_ops(self, outputs, level=PER_PAIR):
+        """Number of arithmetic values at a given level (a proxy for VALU work per pair)."""
+        live = self.live(outputs)
+        return sum(1 for i in live if self.level[i] == level and self.nodes[i][0] not in ("const", "load", "neg"))
+
+    def _lit(self, v):
+        if v != v:
+            return "(T)NAN"
+        if v in (float("inf"), float("-inf")):
+            return "(T)INFINITY" if v > 0 else "-(T)INFINITY"
+        return f"(T){v!r}" if self.dtype == "double" else f"{float(v)!r}f".replace("e+", "e")
+
+    def emit(self, outputs, names, indent="    "):
+        """C++ statements computing ``outputs`` (value ids).
+
+        ``names`` maps a load key (cat, ind, k) to the C++ expression that reads it.
+        Returns (lines, exprs) where exprs[k] is the C++ expression of outputs[k].
+        """
+        live = self.live(outputs)
+        f32 = self.dtype == "float"
+        ref = {}
+        lines = []
+        for i in sorted(live):
+            n = self.nodes[i]
+            op = n[0]
+            if op == "const":
+                ref[i] = self._lit(n[1])
+                continue
+            if op == "load":
+                ref[i] = names[(n[1], n[2], n[3])]
+                continue
+            a = [ref[j] for j in (n[2:] if op == "call" else n[1:])]
+            boolean = False
+            if op == "neg":
+                e = f"-{a[0]}"
+            elif op in ("add", "sub", "mul", "div"):
+                e = f"{a[0]} {dict(add='+', sub='-', mul='*', div='/')[op]} {a[1]}"
+            elif op == "rcp":
+                e = f"__builtin_amdgcn_rcpf({a[0]})" if f32 and self.fast else f"(T)1 / {a[0]}"
+            elif op == "exp2":
+                e = f"__builtin_amdgcn_exp2f({a[0]})"
+            elif op == "exp":
+                e = f"keops_exp({a[0]})"
+            elif op == "log2":
+                e = f"__builtin_amdgcn_logf({a[0]})"
+            elif op == "log":
+                e = f"keops_log({a[0]})"
+            elif op == "sqrt":
+                e = f"__builtin_amdgcn_sqrtf({a[0]})" if f32 and self.fast else f"keops_sqrt({a[0]})"
+            elif op == "rsqrt0":
+                r = f"__builtin_amdgcn_rsqf({a[0]})" if f32 and self.fast else f"(T)1 / keops_sqrt({a[0]})"
+                e = f"({a[0]} == (T)0) ? (T)0 : {r}"
+            elif op == "abs":
+                e = f"keops_abs({a[0]})"
+            elif op == "sign":
+                e = f"({a[0]} > (T)0) ? (T)1 : (({a[0]} < (T)0) ? -(T)1 : (T)0)"
+            elif op == "call":
+                e = f"keops_{n[1]}({', '.join(a)})"
+            elif op in ("lt", "le", "eq", "ne"):
+                e = f"{a[0]} {dict(lt='<', le='<=', eq='==', ne='!=')[op]} {a[1]}"
+                boolean = True
+            elif op == "select":
+                e = f"{a[0]} ? {a[1]} : {a[2]}"
+            else:
+                raise AssertionError(op)
+            ref[i] = f"t{i}"
+            lines.append(f"{indent}const {'bool' if boolean else 'T'} t{i} = {e};")
+        return lines, [ref[o] if self.nodes[o][0] not in ("const",) else ref[o] for o in outputs]
+
+
+def lower(formula, L: Lir):
+    """Lower a formula tree into ``L``; returns the list of output value ids (memoised per node)."""
+    memo = {}
+
+    def rec(node):
+        r = memo.get(node)
+        if r is None:
+            kids = [rec(c) for c in node.children]
+            r = node.lower(L, kids)
+            assert len(r) == node.dim, (node.name, len(r), node.dim)
+            memo[node] = r
+        return r
+
+    return rec(formula)

@@ -1,0 +1,186 @@
+"""Engine entry: formula string -> compiled kernel module + launch metadata.
+
+Counterpart of keopscore/keopscore/get_keops_dll.py:78-159 (scheme selection, zero-formula
+bypass, metadata tuple) and keopscore/keopscore/binders/LinkCompile.py:19-125 (sha256 tag,
+compile-if-absent).  Instead of emitting a whole CUDA kernel as text, the engine emits a short
+"plug-in" - the straight-line formula body plus geometry macros - that is prepended to one of
+the hand-written HIP templates embedded in libkeops_hip.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import threading
+
+from . import binder, config
+from .formulas import Lir, lower, parse_reduction
+from .formulas.ops import Zero
+from .formulas.reductions import KIND_ZERO, Reduction, Sum_Reduction, Zero_Reduction
+
+SUM_SCHEMES = dict(direct_sum=0, block_sum=1, kahan_scheme=2)
+
+_cache = {}
+_lock = threading.Lock()
+
+
+class VarLayout:
+    """Which argument goes where in the packed x_i / y_j / p arrays of the kernels
+    (code_gen_utils.py:531-564 Var_loader).  "row" variables are indexed like the output."""
+
+    def __init__(self, red: Reduction):
+        tagI = red.tagI
+        vs = red.formula.variables
+        self.rowvars = [v for v in vs if v.cat == tagI]
+        self.colvars = [v for v in vs if v.cat == 1 - tagI]
+        self.parvars = [v for v in vs if v.cat == 2]
+        self.dimx = sum(v.dim for v in self.rowvars)
+        self.dimy = sum(v.dim for v in self.colvars)
+        self.dimp = sum(v.dim for v in self.parvars)
+        self.names = {}
+        for group, arr in ((self.rowvars, "xi"), (self.colvars, "yj"), (self.parvars, "p")):
+            off = 0
+            for v in group:
+                for k in range(v.dim):
+                    self.names[(v.cat, v.ind, k)] = f"{arr}[{off + k}]"
+                off += v.dim
+
+    @staticmethod
+    def table(group):
+        args = [v.ind for v in group] or [0]
+        dims = [v.dim for v in group] or [0]
+        offs, o = [], 0
+        for v in group:
+            offs.append(o)
+            o += v.dim
+        offs = offs or [0]
+        return args, dims, offs
+
+
+def _c_list(xs):
+    return "{" + ", ".join(str(int(x)) for x in xs) + "}"
+
+
+def choose_geometry(red, layout, nops, sizeof_t, nx=None):
+    """Rows per lane / tile length: register budget first, then enough workgroups for the chip."""
+    block = config.block_size
+    dimy_pad = 0 if layout.dimy == 0 else -(-layout.dimy // (16 // sizeof_t)) * (16 // sizeof_t)
+    per_row = layout.dimx + 2 * red.dimred * (2 if sizeof_t == 8 else 1) + min(nops, 32)
+    rows = config.max_rows_per_lane
+    while rows > 1 and rows * per_row + 2 * dimy_pad + 24 > 128:
+        rows //= 2
+    if nx is not None:
+        # keep at least ~2 workgroups per compute unit when the row count allows it
+        while rows > 1 and nx < 2 * 256 * block * rows:
+            rows //= 2
+    tile_j = config.lds_tile_bytes // max(1, dimy_pad * sizeof_t)
+    tile_j = max(64, min(1024, 1 << (tile_j.bit_length() - 1)))
+    unroll = 2 if nops * rows <= 128 else 1
+    return dict(block=block, rows=rows, tile_j=tile_j, dimy_pad=dimy_pad, unroll=unroll)
+
+
+def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=None, geometry=None):
+    """HIP source of the kernel module for a reduction; returns (source, meta dict)."""
+    sizeof_t = 8 if dtype == "double" else 4
+    layout = VarLayout(red)
+    L = Lir(row_cat=red.tagI, fast_math=use_fast_math, dtype=dtype)
+    outs = lower(red.formula, L)
+    lines, exprs = L.emit(outs, layout.names, indent="    ")
+    nops = L.count_ops(outs)
+    geo = choose_geometry(red, layout, nops, sizeof_t, nx)
+    if geometry:
+        geo.update(geometry)
+    ra, rd, ro = VarLayout.table(layout.rowvars)
+    ca, cd, co = VarLayout.table(layout.colvars)
+    pa, pd, po = VarLayout.table(layout.parvars)
+    meta = dict(
+        scheme="conv", block=geo["block"], rows=geo["rows"], tile_j=geo["tile_j"], dimred=red.dimred, dimout=red.dim,
+        sizeof_t=sizeof_t, sizeof_acc=8 if dtypeacc == "double" else 4, nrowvars=len(layout.rowvars),
+        ncolvars=len(layout.colvars), nparvars=len(layout.parvars), nops=nops,
+    )
+    src = []
+    src.append("//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()))
+    src.append(f"// reduction: {red!r}")
+    src.append(f"typedef {dtype} T;\ntypedef {dtypeacc} TACC;")
+    defs = dict(
+        KEOPS_NARGS=nargs, KEOPS_DIMX=layout.dimx, KEOPS_DIMY=layout.dimy, KEOPS_DIMY_PAD=geo["dimy_pad"],
+        KEOPS_DIMP=layout.dimp, KEOPS_DIMFOUT=red.formula.dim, KEOPS_DIMRED=red.dimred, KEOPS_DIMOUT=red.dim,
+        KEOPS_RED_KIND=red.kind, KEOPS_RED_KEEP=red.keep, KEOPS_RED_K=red.K, KEOPS_SUM_SCHEME=SUM_SCHEMES[sum_scheme],
+        KEOPS_BLOCK=geo["block"], KEOPS_ROWS=geo["rows"], KEOPS_TILE_J=geo["tile_j"], KEOPS_UNROLL_J=geo["unroll"],
+        KEOPS_NROWVARS=len(layout.rowvars), KEOPS_NCOLVARS=len(layout.colvars), KEOPS_NPARVARS=len(layout.parvars),
+    )
+    src += [f"#define {k} {v}" for k, v in defs.items()]
+    for name, vals in (("row_arg", ra), ("row_dim", rd), ("row_off", ro), ("col_arg", ca), ("col_dim", cd),
+                       ("col_off", co), ("par_arg", pa), ("par_dim", pd), ("par_off", po)):
+        src.append(f"static __device__ constexpr int keops_{name}[] = {_c_list(vals)};")
+    dx, dy, dp = max(1, layout.dimx), max(1, geo["dimy_pad"]), max(1, layout.dimp)
+    src.append("struct KeopsFormula {")
+    src.append(
+        f"  static __device__ __forceinline__ void eval(const T (&xi)[{dx}], const T (&yj)[{dy}], "
+        f"const T (&p)[{dp}], T (&fout)[{red.formula.dim}]) {{"
+    )
+    src += lines
+    src += [f"    fout[{k}] = {e};" for k, e in enumerate(exprs)]
+    src.append("  }\n};")
+    src.append('#include "keops_conv.h"')
+    return "\n".join(src) + "\n", meta
+
+
+def get_keops_dll(
+    map_reduce_id, red_formula_string, enable_chunks, enable_finalchunks, mul_var_highdim, aliases, nargs, dtype,
+    dtypeacc, sum_scheme_string, tagHostDevice, tagCPUGPU, tag1D2D, use_half, use_fast_math, device_id, nx=None,
+):
+    """Same arguments and same 19-tuple as the reference's get_keops_dll (get_keops_dll.py:78-159),
+    plus ``nx``: the number of output rows of the call being prepared, used to pick the number of
+    rows per lane.  ``dtype`` / ``dtypeacc`` are C type names ("float" | "double")."""
+    if use_half or dtype not in ("float", "double"):
+        raise ValueError("[KeOps] only float32 and float64 data are supported by the HIP backend")
+    if "Gpu" not in map_reduce_id:
+        raise ValueError("[KeOps] the HIP engine only builds Gpu map-reduce schemes")
+    red = parse_reduction(red_formula_string, aliases)
+    layout = VarLayout(red)
+    sizeof_t = 8 if dtype == "double" else 4
+    rows_hint = None
+    if nx is not None:
+        # only the bucket matters for the cache key
+        rows_hint = nx if nx < 8 * 256 * config.block_size else None
+    key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
+           use_fast_math, _rows_bucket(rows_hint), binder.templates_digest())
+    with _lock:
+        hit = _cache.get(key)
+    if hit is not None:
+        return hit
+
+    tagZero = int(isinstance(red, Zero_Reduction) or (isinstance(red.formula, Zero) and isinstance(red, Sum_Reduction)))
+    use_chunk_mode = 0
+    if tagZero:
+        target, tag, src_file = "", "zero", ""
+    else:
+        source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint)
+        tag = hashlib.sha256((source + binder.templates_digest() + str(use_fast_math)).encode()).hexdigest()[:16]
+        folder = config.get_build_folder()
+        target = os.path.join(folder, f"hsaco_{tag}")
+        src_file = os.path.join(folder, f"{tag}.hip")
+        if not os.path.exists(target):
+            config.message(f"Compiling formula {red_formula_string} ... ", end="", flush=True)
+            with open(src_file, "w") as f:
+                f.write(source)
+            binder.compile_module(target, source, use_fast_math, max(0, device_id))
+            config.message("OK", flush=True)
+    res = (
+        tag, src_file, target, red.tagI, tagZero, 0, int(bool(use_fast_math)), config.block_size, use_chunk_mode,
+        0 if tagZero else tag1D2D, red.dimred, red.dim, layout.dimy,
+        tuple(v.ind for v in layout.rowvars), tuple(v.ind for v in layout.colvars), tuple(v.ind for v in layout.parvars),
+        tuple(v.dim for v in layout.rowvars), tuple(v.dim for v in layout.colvars), tuple(v.dim for v in layout.parvars),
+    )
+    with _lock:
+        _cache[key] = res
+    return res
+
+
+def _rows_bucket(nx):
+    if nx is None:
+        return -1
+    b = 0
+    while (2 * 256 * config.block_size) << b <= nx:
+        b += 1
+    return b

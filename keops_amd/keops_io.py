@@ -1,0 +1,111 @@
+"""Binding layer between the user-level Genred and the native library.
+
+Counterpart of pykeops/pykeops/common/keops_io/LoadKeOps.py:33-243 (alias -> Var rewrite, dtype
+map, scheme id, output allocation, pointer/shape tuples) and LoadKeOps_nvrtc.py:18-72 (module
+object + call).  The native side is libkeops_hip through ctypes (keops_amd/binder.py).
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from . import binder
+from .common.parse_type import parse_dtype_acc
+from .formulas.parse import parse_alias
+from .get_keops_dll import get_keops_dll
+
+_NULL_RANGE = np.array([-1], dtype=np.int64)
+_modules = {}
+
+
+class LoadKeOps_hip:
+    empty_ranges = tuple([_NULL_RANGE.ctypes.data] * 7)
+
+    def __init__(self, tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula, aliases, nargs,
+                 dtype, lang, optional_flags, nx=None):
+        if lang not in ("torch", "pytorch"):
+            raise ValueError("[KeOps] the HIP backend binds torch tensors only")
+        if tagCPUGPU != 1 or tagHostDevice != 1:
+            raise ValueError(
+                "[KeOps] the HIP backend computes on device-resident tensors only "
+                "(backend 'CPU' and host-memory inputs are not available)"
+            )
+        aliases_new = []
+        for k, alias in enumerate(aliases):
+            name, var = parse_alias(alias, k)
+            if name is not None:
+                aliases_new.append(f"{name}=Var({var.ind},{var.dim},{var.cat})")
+        p = self.params = type("Params", (), {})()
+        p.aliases_old, p.aliases = list(aliases), aliases_new
+        p.red_formula_string = formula
+        p.dtype = dtype
+        p.c_dtype = dict(float32="float", float64="double").get(dtype)
+        if p.c_dtype is None:
+            raise ValueError("not implemented")
+        p.c_dtype_acc = parse_dtype_acc(optional_flags["dtype_acc"], dtype)
+        p.sum_scheme = optional_flags["sum_scheme"]
+        p.enable_chunks = optional_flags["enable_chunks"]
+        p.mult_var_highdim = optional_flags.get("multVar_highdim", 0)
+        p.tagHostDevice, p.tagCPUGPU = tagHostDevice, tagCPUGPU
+        map_reduce_id = "GpuReduc" + ("1D" if tag1D2D == 0 else "2D") + ("_ranges" if use_ranges else "")
+        (p.tag, p.source_name, p.low_level_code_file, p.tagI, p.tagZero, p.use_half, p.use_fast_math,
+         p.cuda_block_size, p.use_chunk_mode, p.tag1D2D, p.dimred, p.dim, p.dimy, indsi, indsj, indsp, dimsx,
+         dimsy, dimsp) = get_keops_dll(
+            map_reduce_id, formula, p.enable_chunks, -1, p.mult_var_highdim, p.aliases, nargs, p.c_dtype,
+            p.c_dtype_acc, p.sum_scheme, tagHostDevice, tagCPUGPU, tag1D2D, False, optional_flags["use_fast_math"],
+            device_id_request, nx=nx,
+        )
+        # the engine reports (output-indexed, reduced) variable lists; the ABI takes (i, j) lists
+        if p.tagI == 1:
+            indsi, indsj, dimsx, dimsy = indsj, indsi, dimsy, dimsx
+        p.indsi, p.indsj, p.indsp, p.dimsx, p.dimsy, p.dimsp = indsi, indsj, indsp, dimsx, dimsy, dimsp
+        p.device_id_request, p.nargs = device_id_request, nargs
+        p.reduction_op = formula.split("(")[0]
+        p.axis = 1 - p.tagI
+        self.dimout, self.tagIJ = p.dim, p.tagI
+        self.module = None
+        if not p.tagZero:
+            key = (p.low_level_code_file, device_id_request, nargs)
+            self.module = _modules.get(key)
+            if self.module is None:
+                self.module = _modules[key] = binder.Module(max(0, device_id_request), nargs, p.low_level_code_file)
+
+    def genred_pytorch(self, device_args, ranges, nx, ny, nbatchdims, out, *args):
+        p = self.params
+        if not ranges:
+            ranges_ptr, keep = self.empty_ranges, None
+        else:
+            shapes = np.array([r.shape[0] for r in ranges], dtype=np.int64)
+            keep = (ranges, shapes)
+            ranges_ptr = tuple(int(r.data_ptr()) for r in ranges) + (shapes.ctypes.data,)
+        args_ptr = tuple(int(a.data_ptr()) for a in args)
+        argshapes = tuple(tuple(a.shape) for a in args)
+        M = nx if p.tagI == 0 else ny
+        if nbatchdims:
+            bshape = np.maximum.reduce([list(a.shape[:nbatchdims]) for a in args])
+            shapeout = tuple(int(b) for b in bshape) + (M, p.dim)
+        else:
+            shapeout = (M, p.dim)
+        if out is None:
+            out = torch.empty(shapeout, dtype=args[0].dtype, device=device_args)
+        elif tuple(out.shape) != shapeout or not out.is_contiguous():
+            raise ValueError(f"[KeOps] 'out' must be a contiguous tensor of shape {shapeout}")
+        if p.tagZero:
+            out.zero_()
+            return out
+        stream = torch.cuda.current_stream(out.device).cuda_stream
+        self.module(
+            p.tagHostDevice, p.dimy, nx, ny, p.tagI, p.tagZero, p.use_half, p.tag1D2D, p.dimred, p.cuda_block_size,
+            p.use_chunk_mode, p.indsi, p.indsj, p.indsp, p.dim, p.dimsx, p.dimsy, p.dimsp, ranges_ptr, tuple(out.shape),
+            int(out.data_ptr()), args_ptr, argshapes, stream=stream, sync=False,
+        )
+        del keep
+        return out
+
+    genred = genred_pytorch
+
+    def import_module(self):
+        return self
+
+
+keops_binder = {"hip": LoadKeOps_hip}
