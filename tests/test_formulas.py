@@ -1,0 +1,206 @@
+"""Host-logic tests of the formula layer: grammar, simplification, autodiff and scalar lowering,
+checked against dense torch expressions (the reference's own test style, keopscore/keopscore/
+test/test_op.py:18-188: M=300, N=500-like random inputs, forward and gradient vs torch)."""
+import numpy as np
+import pytest
+import torch
+
+from keops_amd.formulas import FormulaError, Lir, lower, parse, parse_reduction
+from keops_amd.formulas import ops as O
+
+from host_eval import dense_eval
+
+M, N = 7, 9
+torch.manual_seed(0)
+
+
+def _t(*shape, lo=-1.0, hi=1.0):
+    return (torch.rand(*shape, dtype=torch.float64) * (hi - lo) + lo)
+
+
+def _check(formula, aliases, targs, torch_fn, grad_wrt=(), tol=1e-10):
+    """targs: torch tensors shaped (M,d)/(N,d)/(d,); torch_fn gets broadcastable views."""
+    views = []
+    for a, al in zip(targs, aliases):
+        cat = parse(al.split("=")[1] if "=" in al else al, []).cat
+        views.append(a[:, None, :] if cat == 0 else (a[None, :, :] if cat == 1 else a[None, None, :]))
+    leaves = [v.detach().clone().requires_grad_(True) for v in views]
+    ref = torch_fn(*leaves)
+    got = dense_eval(formula, aliases, [a.numpy() for a in targs], M, N)
+    ref_b = torch.broadcast_to(ref, (M, N, ref.shape[-1])).detach().numpy()
+    assert got.shape == ref_b.shape, (got.shape, ref_b.shape)
+    assert np.allclose(got, ref_b, rtol=tol, atol=tol), formula
+    op = parse(formula, aliases)
+    for k in grad_wrt:
+        v = op.variables[[w.ind for w in op.variables].index(k)]
+        eta = O.Var(len(targs), op.dim, 1 - v.cat if v.cat < 2 else 0)
+        gop = O.Grad(op, v, eta)
+        E = _t(M if eta.cat == 0 else N, op.dim)
+        gdense = dense_eval(gop, None, [a.numpy() for a in targs] + [E.numpy()], M, N)
+        Ev = E[:, None, :] if eta.cat == 0 else E[None, :, :]
+        (gref,) = torch.autograd.grad((torch.broadcast_to(ref, (M, N, ref.shape[-1])) * Ev).sum(), leaves[k], retain_graph=True)
+        # dense pairwise gradient summed over the axis the variable does not depend on
+        if v.cat == 0:
+            g = gdense.sum(1)
+            gr = gref.reshape(M, -1).numpy()
+        elif v.cat == 1:
+            g = gdense.sum(0)
+            gr = gref.reshape(N, -1).numpy()
+        else:
+            g = gdense.sum((0, 1))
+            gr = gref.reshape(-1).numpy()
+        assert np.allclose(g, gr, rtol=1e-8, atol=1e-8), (formula, k)
+
+
+AL = ["x=Vi(0,3)", "y=Vj(1,3)", "p=Pm(2,1)", "b=Vj(3,2)"]
+
+
+def _args():
+    return [_t(M, 3), _t(N, 3), _t(1, lo=0.5, hi=1.5), _t(N, 2)]
+
+
+UNARY = {
+    "Exp": (torch.exp, (-1, 1)), "Log": (torch.log, (0.5, 2)), "Sqrt": (torch.sqrt, (0.5, 2)),
+    "Rsqrt": (torch.rsqrt, (0.5, 2)), "Inv": (lambda t: 1 / t, (0.5, 2)), "Square": (lambda t: t * t, (-1, 1)),
+    "Abs": (torch.abs, (-1, 1)), "Sign": (torch.sign, (-1, 1)), "Step": (lambda t: (t >= 0).double(), (-1, 1)),
+    "ReLU": (torch.relu, (-1, 1)), "Sin": (torch.sin, (-1, 1)), "Cos": (torch.cos, (-1, 1)),
+    "Asin": (torch.asin, (-0.9, 0.9)), "Acos": (torch.acos, (-0.9, 0.9)), "Atan": (torch.atan, (-1, 1)),
+    "Floor": (torch.floor, (-3, 3)), "XLogX": (lambda t: t * torch.log(t), (0.5, 2)),
+    "SinXDivX": (lambda t: torch.sin(t) / t, (0.2, 2)), "Minus": (lambda t: -t, (-1, 1)),
+}
+
+
+@pytest.mark.parametrize("name", sorted(UNARY))
+def test_unary_ops(name):
+    fn, (lo, hi) = UNARY[name]
+    targs = [_t(M, 3, lo=lo, hi=hi), _t(N, 3, lo=lo, hi=hi)]
+    al = ["x=Vi(0,3)", "y=Vj(1,3)"]
+    grad = () if name in ("Sign", "Step", "Floor") else (0, 1)
+    # x*y keeps products inside the op's domain for positive ranges; use a sum for signed ones
+    if lo > 0:
+        _check(f"{name}(x*y)", al, targs, lambda x, y: fn(x * y), grad)
+    else:
+        _check(f"{name}((x+y)/2)", al, targs, lambda x, y: fn((x + y) / 2), grad)
+
+
+def test_binary_and_broadcast_ops():
+    a = _args()
+    _check("(x-y)*p + y/(p+2)", AL, a, lambda x, y, p, b: (x - y) * p + y / (p + 2), (0, 1, 2))
+    _check("(x|y)*b", AL, a, lambda x, y, p, b: (x * y).sum(-1, keepdim=True) * b, (0, 1, 3))
+    _check("Powf(Abs(x)+1, y)", AL, a, lambda x, y, p, b: torch.pow(x.abs() + 1, y), (0, 1))
+    _check("Pow(x,3)+Pow(y,-2)", AL, [_t(M, 3), _t(N, 3, lo=0.5, hi=1.5), a[2], a[3]],
+           lambda x, y, p, b: x**3 + y**-2.0, (0, 1))
+    _check("Atan2(x,y+3)", AL, a, lambda x, y, p, b: torch.atan2(x, y + 3), (0, 1))
+    _check("x/SumT(p+Sum(y*y),3)", AL, a, lambda x, y, p, b: x / (p + (y * y).sum(-1, keepdim=True)), (0, 1, 2))
+    _check("IfElse(x-y, x*2, y*p)", AL, a, lambda x, y, p, b: torch.where(x - y >= 0, x * 2, y * p), (0, 1, 2))
+    _check("Clamp(x, y-1, y+1)", AL, a, lambda x, y, p, b: torch.minimum(torch.maximum(x, y - 1), y + 1), (0, 1))
+    _check("ClampInt(3*x, -1, 1)", AL, a, lambda x, y, p, b: torch.clamp(3 * x, -1, 1), (0,))
+    _check("Mod(5*x, 2, 0)", AL, a, lambda x, y, p, b: 5 * x - 2 * torch.floor(5 * x / 2))
+    _check("Round(3*x, 1)", AL, a, lambda x, y, p, b: torch.round(30 * x) / 10)
+    _check("(x<y) + (x<=y)*2 + Equal(x,x) + NotEqual(x,y)", AL, a,
+           lambda x, y, p, b: (x < y).double() + 2 * (x <= y).double() + 1 + (x != y).double())
+
+
+def test_vector_ops():
+    a = _args()
+    _check("SqDist(x,y)", AL, a, lambda x, y, p, b: ((x - y) ** 2).sum(-1, keepdim=True), (0, 1))
+    _check("Norm2(x-y)", AL, a, lambda x, y, p, b: (x - y).norm(dim=-1, keepdim=True), (0, 1))
+    _check("Normalize(x+y)", AL, a, lambda x, y, p, b: (x + y) / (x + y).norm(dim=-1, keepdim=True), (0, 1))
+    _check("SqNorm2(x)*y", AL, a, lambda x, y, p, b: (x * x).sum(-1, keepdim=True) * y, (0, 1))
+    _check("Concat(x, b)", AL, a, lambda x, y, p, b: torch.cat([x.expand(M, N, 3), b.expand(M, N, 2)], -1), (0, 3))
+    _check("Extract(Concat(x*y, b), 2, 3)", AL, a,
+           lambda x, y, p, b: torch.cat([(x * y).expand(M, N, 3), b.expand(M, N, 2)], -1)[..., 2:5], (0, 1, 3))
+    _check("ExtractT(b*p, 1, 4)", AL, a,
+           lambda x, y, p, b: torch.cat([0 * b[..., :1], b * p, 0 * b[..., :1]], -1), (2, 3))
+    _check("Elem(x,1)*ElemT(Elem(y,2), 3, 0)", AL, a,
+           lambda x, y, p, b: x[..., 1:2] * torch.cat([y[..., 2:3], 0 * y[..., :2]], -1), (0, 1))
+    _check("Max(x*y)+Min(x-y)", AL, a,
+           lambda x, y, p, b: (x * y).max(-1, keepdim=True)[0] + (x - y).min(-1, keepdim=True)[0], (0, 1))
+    _check("ArgMax(x*y)+2*ArgMin(x*y)", AL, a,
+           lambda x, y, p, b: ((x * y).argmax(-1, keepdim=True) + 2 * (x * y).argmin(-1, keepdim=True)).double())
+    _check("OneHot(Floor(Abs(2*Elem(x,0))), 3)", AL, a,
+           lambda x, y, p, b: torch.nn.functional.one_hot(torch.floor((2 * x[..., 0]).abs()).long(), 3).double())
+    _check("WeightedSqDist(p, x, y)", AL, a, lambda x, y, p, b: p * ((x - y) ** 2).sum(-1, keepdim=True), (0, 1, 2))
+    _check("WeightedSqNorm(y, x)", AL, a, lambda x, y, p, b: (y * x * x).sum(-1, keepdim=True), (0, 1))
+    al2 = ["A=Vi(0,6)", "v=Vj(1,2)", "w=Vj(2,3)"]
+    t2 = [_t(M, 6), _t(N, 2), _t(N, 3)]
+    # A is a (3 x 2) matrix stored column-major: out_i = sum_k A[k*3+i] v_k
+    _check("MatVecMult(A, v)", al2, t2,
+           lambda A, v, w: (A.expand(M, N, 6).reshape(M, N, 2, 3) * v.expand(M, N, 2)[..., None]).sum(-2), (0, 1))
+    _check("VecMatMult(w, A)", al2, t2,
+           lambda A, v, w: (A.expand(M, N, 6).reshape(M, N, 2, 3) * w.expand(M, N, 3)[..., None, :]).sum(-1), (0, 2))
+    _check("TensorProd(v, w)", al2, t2,
+           lambda A, v, w: (v.expand(M, N, 2)[..., :, None] * w.expand(M, N, 3)[..., None, :]).reshape(M, N, 6), (1, 2))
+    _check("WeightedSqNorm(Concat(Concat(v,v),v)+1, v)" if False else "SqNorm2(MatVecMult(A, v))", al2, t2,
+           lambda A, v, w: ((A.expand(M, N, 6).reshape(M, N, 2, 3) * v.expand(M, N, 2)[..., None]).sum(-2) ** 2).sum(-1, keepdim=True), (0, 1))
+
+
+def test_gaussian_and_its_gradients():
+    al = ["x=Vi(0,3)", "y=Vj(1,3)", "b=Vj(2,2)", "g=Pm(3,1)"]
+    a = [_t(M, 3), _t(N, 3), _t(N, 2), _t(1, lo=0.5, hi=1.5)]
+    _check("Exp(-g*SqDist(x,y))*b", al, a, lambda x, y, b, g: torch.exp(-g * ((x - y) ** 2).sum(-1, keepdim=True)) * b,
+           (0, 1, 2, 3), tol=1e-12)
+    _check("Exp(-Norm2(x-y))*b", al, a, lambda x, y, b, g: torch.exp(-(x - y).norm(dim=-1, keepdim=True)) * b, (0, 1, 2))
+    # second order: gradient of the gradient formula (cf. pykeops/test/test_lazytensor_gaussian_cpu.py)
+    op = parse("Exp(-g*SqDist(x,y))*b", al)
+    x, y, b, g = op.variables
+    e = O.Var(4, 2, 0)
+    g1 = O.Grad(op, x, e)          # dim 3, depends on x,y,b,g,e
+    e2 = O.Var(5, 3, 0)
+    g2 = O.Grad(g1, x, e2)
+    E, E2 = _t(M, 2), _t(M, 3)
+    dense = dense_eval(g2, None, [t.numpy() for t in a] + [E.numpy(), E2.numpy()], M, N).sum(1)
+    xt = a[0].clone().requires_grad_(True)
+    K = torch.exp(-a[3] * ((xt[:, None] - a[1][None]) ** 2).sum(-1, keepdim=True)) * a[2][None]
+    (gx,) = torch.autograd.grad((K * E[:, None]).sum(), xt, create_graph=True)
+    (ggx,) = torch.autograd.grad((gx * E2).sum(), xt)
+    assert np.allclose(dense, ggx.numpy(), rtol=1e-8, atol=1e-10)
+
+
+def test_simplifications():
+    al = ["x=Vi(0,3)", "y=Vj(1,3)", "s=Pm(2,1)"]
+    x, y, s = parse("x", al), parse("y", al), parse("s", al)
+    assert isinstance(x - x, O.Zero) and (x - x).dim == 3
+    assert x * 1 == x and 1 * x == x and x + O.Zero(3) == x
+    assert repr(-(-x)) == repr(x)
+    assert repr(x * x) == repr(O.Square(x))
+    assert isinstance(O.Grad(parse("Exp(s)*y", al), x, O.Var(3, 3, 1)), O.Zero)
+    assert repr(parse("SqDist(x,y)", al)) == "Sum(Square(Subtract(Var(0,3,0),Var(1,3,1))))"
+    assert repr(parse("2*(3*x)", al)) == repr(parse("6*x", al))
+    assert repr(parse("IntInv(2)*IntCst(4)", al)) == "IntCst(2)"
+    assert parse("Sum(s*x)", al) == parse("s*Sum(x)", al)
+    # Exp(a)*Exp(b) -> Exp(a+b): one exponential per pair
+    e = parse("Exp(-s*SqNorm2(x))*Exp(-SqNorm2(y))", al)
+    assert sum(1 for n in e.walk() if n.name == "Exp") == 1
+
+
+def test_gaussian_lowering_is_minimal():
+    """The Gaussian kernel must cost 3 sub + 3 mul/fma + 1 scale + exp + weight per pair."""
+    al = ["x=Var(0,3,0)", "y=Var(1,3,1)", "b=Var(2,1,1)", "g=Var(3,1,2)"]
+    red = parse_reduction("Sum_Reduction(Exp(-g*SqDist(x,y))*b,0)", al)
+    L = Lir(row_cat=0, fast_math=True)
+    outs = lower(red.formula, L)
+    assert L.count_ops(outs) == 11  # sub x3, mul x3, add x2, scale, exp2, weight (mul+add fuse to fma)
+    g = parse_reduction("Grad_WithSavedForward(Sum_Reduction(Exp(-g*SqDist(x,y))*b,0),Var(0,3,0),Var(4,1,0),Var(5,1,0))", al)
+    L = Lir(row_cat=0, fast_math=True)
+    assert L.count_ops(lower(g.formula, L)) <= 16
+
+
+def test_parser_errors_and_aliases():
+    with pytest.raises(FormulaError):
+        parse("Foo(x)", ["x=Vi(3)"])
+    with pytest.raises(FormulaError):
+        parse("x+z", ["x=Vi(3)"])
+    with pytest.raises(FormulaError):
+        parse("x+y", ["x=Vi(3)", "y=Vj(2)"])
+    with pytest.raises(FormulaError):
+        parse("__import__('os')", [])
+    with pytest.raises(FormulaError):
+        parse_reduction("Exp(x)", ["x=Vi(3)"])
+    assert repr(parse("Vi(0,3)+Vj(1,3)*Pm(2,1)", [])) == "Add(Var(0,3,0),Mult(Var(2,1,2),Var(1,3,1)))"
+    r = parse_reduction("KMin_ArgKMin_Reduction(SqDist(x,y),10,0)", ["x=Vi(64)", "y=Vj(64)"])
+    assert (r.K, r.dim, r.dimred, r.tagI) == (10, 20, 20, 0)
+    r = parse_reduction("Max_SumShiftExp_Reduction(l-SqDist(x,y)*e,0)", ["x=Vi(3)", "y=Vj(3)", "l=Vj(1)", "e=Pm(1)"])
+    assert (r.dim, r.dimred) == (2, 2)
+    r = parse_reduction("Max_SumShiftExpWeight_Reduction(SqDist(x,y),1,Concat(IntCst(1),x))", ["x=Vi(3)", "y=Vj(3)"])
+    assert (r.dim, r.tagI) == (5, 1)
