@@ -38,6 +38,8 @@ __device__ __forceinline__ float keops_atan2(float y, float x) { return __ocml_a
 __device__ __forceinline__ double keops_atan2(double y, double x) { return __ocml_atan2_f64(y, x); }
 __device__ __forceinline__ float keops_pow(float x, float y) { return __ocml_pow_f32(x, y); }
 __device__ __forceinline__ double keops_pow(double x, double y) { return __ocml_pow_f64(x, y); }
+__device__ __forceinline__ float keops_fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double keops_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
 __device__ __forceinline__ float keops_floor(float x) { return __builtin_floorf(x); }
 __device__ __forceinline__ double keops_floor(double x) { return __builtin_floor(x); }
 __device__ __forceinline__ float keops_round(float x) { return __builtin_roundf(x); }

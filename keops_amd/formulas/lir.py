@@ -24,9 +24,14 @@ UNIFORM, PER_ROW, PER_PAIR = 0, 1, 2
 
 
 class Lir:
-    def __init__(self, row_cat=0, fast_math=True, dtype="float"):
+    def __init__(self, row_cat=0, fast_math=True, dtype="float", exact_order=False):
         self.row_cat = row_cat  # category (0 = i, 1 = j) of the variables indexed like the output
-        self.fast = bool(fast_math)
+        # exact_order: keep the reference's operation order and roundings (explicit fused
+        # multiply-adds only where the reference calls fma, no re-association); used when the
+        # reduction returns indices, whose parity is bit-exact
+        self.exact = bool(exact_order)
+        self.fast = bool(fast_math) and not self.exact
+        self.fast_fn = bool(fast_math)  # hardware exp2/log2/rcp/sqrt approximations allowed
         self.dtype = dtype
         self.nodes = []  # (op, args...) tuples
         self.level = []
@@ -137,7 +142,10 @@ class Lir:
         return self._mk(("mul", a, b), self._lvl(a, b))
 
     def fma(self, a, b, c):
-        """a*b + c; printed as a plain multiply-add (the compiler contracts it)."""
+        """a*b + c; printed as a plain multiply-add (the compiler contracts it) unless the exact
+        operation order is requested, where it is a genuine single-rounding fma."""
+        if self.exact:
+            return self._mk(("fma", a, b, c), self._lvl(a, b, c))
         return self.add(self.mul(a, b), c)
 
     def div(self, a, b):
@@ -145,7 +153,7 @@ class Lir:
             return self.const(self.cval(a) / self.cval(b))
         if self.is_const(b, 1.0):
             return a
-        if self.fast:
+        if self.fast_fn and not self.exact:
             return self.mul(a, self.rcp(b))
         return self._mk(("div", a, b), self._lvl(a, b))
 
@@ -157,14 +165,14 @@ class Lir:
     def exp(self, a):
         if self.is_const(a):
             return self.const(math.exp(self.cval(a)))
-        if self.dtype == "float" and self.fast:
+        if self.dtype == "float" and self.fast_fn:
             return self._mk(("exp2", self.mul(a, self.const(LOG2E))), self.level[a])
         return self._mk(("exp", a), self.level[a])
 
     def log(self, a):
         if self.is_const(a) and self.cval(a) > 0:
             return self.const(math.log(self.cval(a)))
-        if self.dtype == "float" and self.fast:
+        if self.dtype == "float" and self.fast_fn:
             return self.mul(self._mk(("log2", a), self.level[a]), self.const(LN2))
         return self._mk(("log", a), self.level[a])
 
@@ -279,8 +287,10 @@ class Lir:
                 e = f"-{a[0]}"
             elif op in ("add", "sub", "mul", "div"):
                 e = f"{a[0]} {dict(add='+', sub='-', mul='*', div='/')[op]} {a[1]}"
+            elif op == "fma":
+                e = f"keops_fma({a[0]}, {a[1]}, {a[2]})"
             elif op == "rcp":
-                e = f"__builtin_amdgcn_rcpf({a[0]})" if f32 and self.fast else f"(T)1 / {a[0]}"
+                e = f"__builtin_amdgcn_rcpf({a[0]})" if f32 and self.fast_fn else f"(T)1 / {a[0]}"
             elif op == "exp2":
                 e = f"__builtin_amdgcn_exp2f({a[0]})"
             elif op == "exp":
@@ -290,9 +300,9 @@ class Lir:
             elif op == "log":
                 e = f"keops_log({a[0]})"
             elif op == "sqrt":
-                e = f"__builtin_amdgcn_sqrtf({a[0]})" if f32 and self.fast else f"keops_sqrt({a[0]})"
+                e = f"__builtin_amdgcn_sqrtf({a[0]})" if f32 and self.fast_fn and not self.exact else f"keops_sqrt({a[0]})"
             elif op == "rsqrt0":
-                r = f"__builtin_amdgcn_rsqf({a[0]})" if f32 and self.fast else f"(T)1 / keops_sqrt({a[0]})"
+                r = f"__builtin_amdgcn_rsqf({a[0]})" if f32 and self.fast_fn and not self.exact else f"(T)1 / keops_sqrt({a[0]})"
                 e = f"({a[0]} == (T)0) ? (T)0 : {r}"
             elif op == "abs":
                 e = f"keops_abs({a[0]})"

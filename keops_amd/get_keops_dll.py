@@ -15,7 +15,7 @@ import threading
 from . import binder, config
 from .formulas import Lir, lower, parse_reduction
 from .formulas.ops import Zero
-from .formulas.reductions import KIND_ZERO, Reduction, Sum_Reduction, Zero_Reduction
+from .formulas.reductions import KIND_KMIN, KIND_MAX, KIND_MIN, Reduction, Sum_Reduction, Zero_Reduction
 
 SUM_SCHEMES = dict(direct_sum=0, block_sum=1, kahan_scheme=2)
 
@@ -82,9 +82,14 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
     """HIP source of the kernel module for a reduction; returns (source, meta dict)."""
     sizeof_t = 8 if dtype == "double" else 4
     layout = VarLayout(red)
-    L = Lir(row_cat=red.tagI, fast_math=use_fast_math, dtype=dtype)
+    # reductions that return indices are compared bit for bit: their pair values keep the
+    # reference's operation order, without fused multiply-add contraction
+    exact = red.kind in (KIND_MIN, KIND_MAX, KIND_KMIN)
+    L = Lir(row_cat=red.tagI, fast_math=use_fast_math, dtype=dtype, exact_order=exact)
     outs = lower(red.formula, L)
     lines, exprs = L.emit(outs, layout.names, indent="    ")
+    if exact:
+        lines = ["    #pragma clang fp contract(off)"] + lines
     nops = L.count_ops(outs)
     geo = choose_geometry(red, layout, nops, sizeof_t, nx)
     if geometry:
@@ -101,6 +106,7 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
     src.append("//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()))
     src.append(f"// reduction: {red!r}")
     src.append(f"typedef {dtype} T;\ntypedef {dtypeacc} TACC;")
+    src.append('#include "keops_common.h"')
     defs = dict(
         KEOPS_NARGS=nargs, KEOPS_DIMX=layout.dimx, KEOPS_DIMY=layout.dimy, KEOPS_DIMY_PAD=geo["dimy_pad"],
         KEOPS_DIMP=layout.dimp, KEOPS_DIMFOUT=red.formula.dim, KEOPS_DIMRED=red.dimred, KEOPS_DIMOUT=red.dim,

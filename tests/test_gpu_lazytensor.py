@@ -1,0 +1,86 @@
+"""LazyTensor front end on the GPU, against dense torch (the reference's test style:
+pykeops/test/test_lazytensor_gaussian_cpu.py, test_lazytensor_gaussian_batch.py, test_torch.py)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def test_gaussian_matvec_and_two_orders_of_gradients():
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(0)
+    M, N, D, DV = 1000, 1001, 3, 2
+    x = torch.randn(M, D, device="cuda", dtype=torch.float64, requires_grad=True)
+    y = torch.randn(N, D, device="cuda", dtype=torch.float64)
+    b = torch.randn(N, DV, device="cuda", dtype=torch.float64)
+
+    def fun(x, y, b, lazy):
+        if lazy:
+            xi, yj = LazyTensor(x[:, None, :]), LazyTensor(y[None, :, :])
+        else:
+            xi, yj = x[:, None, :], y[None, :, :]
+        K = (-((xi - yj) ** 2).sum(dim=2) / 2).exp()
+        return K @ b if lazy else K @ b
+
+    outs = []
+    for lazy in (True, False):
+        o = fun(x, y, b, lazy)
+        (g1,) = torch.autograd.grad((o**2).sum(), [x], create_graph=True)
+        (g2,) = torch.autograd.grad((g1**2).sum(), [x])
+        outs.append((o, g1, g2))
+    for a, r in zip(*outs):
+        assert torch.allclose(a, r, rtol=1e-9, atol=1e-9)
+
+
+def test_batch_lazytensor_logsumexp_argkmin_and_ops():
+    from keops_amd.torch import LazyTensor, Pm, Vi, Vj
+
+    torch.manual_seed(1)
+    B, M, N = 3, 200, 300
+    x = torch.randn(B, M, 1, 3, device="cuda")
+    y = torch.randn(1, 1, N, 3, device="cuda")
+    p = torch.rand(B, 1, 1, 1, device="cuda") + 0.5
+    xi, yj, pp = LazyTensor(x), LazyTensor(y), LazyTensor(p)
+    D = ((xi - yj) ** 2).sum(-1)
+    lse = (-D * pp).logsumexp(dim=2)
+    dd = ((x - y) ** 2).sum(-1)
+    assert tuple(lse.shape) == (B, M, 1)
+    assert torch.allclose(lse[..., 0], torch.logsumexp(-dd * p[..., 0], dim=2), rtol=1e-5, atol=1e-5)
+    idx = D.argKmin(4, dim=2)
+    assert tuple(idx.shape) == (B, M, 4)
+    assert (idx == dd.topk(4, dim=2, largest=False).indices).float().mean() > 0.999
+    # plain 2D constructors, scalar arithmetic, Scalprod, abs, clamp, elementwise ops, sum over i
+    x2, y2 = torch.randn(M, 3, device="cuda"), torch.randn(N, 3, device="cuda")
+    F = ((Vi(x2) | Vj(y2)).abs() * 0.5 + (Vi(x2) - Vj(y2)).clamp(-1, 1).sum(-1) - 2 * Pm(torch.tensor([0.25], device="cuda")))
+    got = F.sum(dim=0)
+    dense = ((x2 @ y2.T).abs() * 0.5 + (x2[:, None] - y2[None]).clamp(-1, 1).sum(-1) - 0.5).sum(0)[:, None]
+    assert torch.allclose(got, dense, rtol=1e-4, atol=1e-3)
+    vals, arg = (Vi(x2).sqdist(Vj(y2))).min_argmin(dim=1)
+    d2 = ((x2[:, None] - y2[None]) ** 2).sum(-1)
+    assert torch.allclose(vals[:, 0], d2.min(1).values, rtol=1e-5, atol=1e-6)
+
+
+def test_lazytensor_ranges_and_symbolic_variables():
+    from keops_amd.torch import LazyTensor, Vi, Vj
+    from keops_amd.torch.cluster import cluster_ranges, from_matrix, grid_cluster, sort_clusters
+
+    torch.manual_seed(2)
+    x = torch.rand(3000, 2, device="cuda")
+    b = torch.randn(3000, 1, device="cuda")
+    lab = grid_cluster(x, 0.25).long()
+    (x, b), lab = sort_clusters((x, b), lab)
+    r = cluster_ranges(lab)
+    keep = torch.ones(len(r), len(r), dtype=torch.bool, device="cuda")
+    keep[0, 1:] = False
+    K = (-Vi(x).sqdist(Vj(x)) * 10.0).exp()
+    K.ranges = from_matrix(r, r, keep)
+    got = K @ b
+    dense = torch.exp(-10 * torch.cdist(x, x) ** 2)
+    mask = keep[lab][:, lab]
+    assert torch.allclose(got, (dense * mask) @ b, rtol=1e-4, atol=1e-4)
+    # symbolic variables are bound at call time
+    f = (Vi(0, 2) - Vj(1, 2)).sqnorm2().exp().sum(dim=1, call=False) if False else (
+        (-(LazyTensor((0, 2, 0)) - LazyTensor((1, 2, 1))).sqnorm2()).exp().reduction("Sum", axis=1))
+    out = f(x, x)
+    assert torch.allclose(out[:, 0], torch.exp(-torch.cdist(x, x) ** 2).sum(1), rtol=1e-4)
