@@ -1,0 +1,194 @@
+"""Benchmark of the map-reduce hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
+HBM.  The default workload is BASELINE.json's headline configuration: the Gaussian kernel sum
+a_i = sum_j exp(-|x_i-y_j|^2/sigma^2) b_j at M = N = 1,000,000, D = 3, Dv = 1, float32.
+The last line printed is ONE JSON object with the throughput (pair interactions per second), the
+roofline of the dominant kernel (algorithmic flops / kernel time measured with HIP events on the
+launch stream) and, for the default run, the CPU oracle timed on the host cores on a bounded sample
+of the same workload.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# published MI355X peaks
+PEAK_FP32_VECTOR_TFLOPS = 157.3
+PEAK_FP32_MFMA_TFLOPS = 157.3
+# reference number for this metric: PyKeOps Gaussian conv, M=N=1M, RTX 2080 Ti, 1.39 s
+# (reference benchmarks/README.md:14) -> 7.2e11 pairs/s
+PUBLISHED_PAIRS_PER_S = 1e12 / 1.39
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/);
+# None until measured for a workload
+MEASURED_TRAFFIC_BYTES = {}
+
+WORKLOADS = {
+    # name: (description, algorithmic flop per pair, roofline bound)
+    "gauss_1m_dv1": ("Gaussian kernel sum 1e6 x 1e6, D=3, Dv=1, float32 (BASELINE config 2)", 14, "valu"),
+    "gauss_1m_dv8": ("Gaussian kernel sum 1e6 x 1e6, D=3, Dv=8, float32 (BASELINE config 2)", 28, "valu"),
+    "gauss_1m_grad": ("gradient wrt x of the Gaussian kernel sum 1e6 x 1e6, D=3, Dv=1 (BASELINE config 2)", 21, "valu"),
+    "gauss_10k": ("Gaussian kernel sum 1e4 x 1e4, D=3, Dv=1, float32 (BASELINE config 1)", 14, "valu"),
+    "knn_d64": ("ArgKMin K=10, 1e5 queries x 1e6 references, D=64 (BASELINE config 3)", 130, "mfma"),
+    "sparse_100x10k": ("block-sparse Gaussian sum, 100 clusters x 10,000 points (BASELINE config 4)", 14, "valu"),
+    "lse_b16": ("batched LogSumExp softmin B=16, 50,000 x 50,000, D=3 (BASELINE config 5a)", 17, "valu"),
+    "laplace_d256": ("Laplace kernel sum 2e5 x 2e5, D=256, Dv=16 (BASELINE config 5b)", 547, "mfma"),
+}
+
+
+def _np_inputs(name):
+    import numpy as np
+
+    if name.startswith("gauss_1m") or name == "gauss_10k":
+        M = N = 10_000 if name == "gauss_10k" else 1_000_000
+        Dv = 8 if name.endswith("dv8") else 1
+        rng = np.random.default_rng(0 if name == "gauss_10k" else 1)
+        x = rng.standard_normal((M, 3)).astype(np.float32)
+        y = rng.standard_normal((N, 3)).astype(np.float32)
+        b = rng.standard_normal((N, Dv)).astype(np.float32)
+        return dict(M=M, N=N, Dv=Dv, arrays=[x, y, b, np.array([1.0], np.float32)])
+    raise SystemExit(f"workload {name} is not available in this build")
+
+
+def build_step(name):
+    """Returns (step callable, pairs per step, loaded module handle or None, numpy inputs)."""
+    import torch
+
+    from keops_amd.torch import Genred
+
+    inp = _np_inputs(name)
+    dev = [torch.from_numpy(a).cuda() for a in inp["arrays"]]
+    M, N, Dv = inp["M"], inp["N"], inp["Dv"]
+    conv = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", f"b=Vj({Dv})", "g=Pm(1)"], reduction_op="Sum", axis=1)
+    if name == "gauss_1m_grad":
+        # the gradient is another map-reduce (pykeops generic_red.py:165-214): run the forward once,
+        # then every step back-propagates G = ones through it, which launches the gradient kernel only
+        dev[0].requires_grad_(True)
+        a = conv(*dev)
+        G = torch.ones_like(a)
+
+        def step():
+            return torch.autograd.grad(a, [dev[0]], G, retain_graph=True)[0]
+    else:
+        def step():
+            return conv(*dev)
+
+    return step, M * N, inp
+
+
+def kernel_modules():
+    from keops_amd import keops_io
+
+    return list(keops_io._modules.values())
+
+
+def cpu_baseline(name, inp):
+    """The CPU oracle (restatement of the reference's CpuReduc loop) timed on the host cores on a
+    bounded sample of the same workload: a subset of output rows against all columns."""
+    import numpy as np
+
+    from oracle.cpu_oracle import cpu_reduc, lib
+
+    M, N, Dv = inp["M"], inp["N"], inp["Dv"]
+    x, y, b, g = inp["arrays"]
+    try:
+        threads = ctypes.CDLL(None).omp_get_max_threads()
+    except Exception:
+        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    lib()
+    # calibrate on 64 rows, then size the sample for about 10 s of CPU work
+    rows = np.arange(64, dtype=np.int64)
+    t0 = time.perf_counter()
+    cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
+    rate = 64 * N / (time.perf_counter() - t0)
+    nrows = int(min(M, max(256, (10.0 * rate / N) // 256 * 256)))
+    rows = np.sort(np.random.default_rng(0).choice(M, nrows, replace=False)).astype(np.int64)
+    t0 = time.perf_counter()
+    cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
+    dt = time.perf_counter() - t0
+    return dict(value=nrows * N / dt, unit="pairs/s", cores=int(threads), kind="port",
+                sample=f"{nrows} random output rows x {N} columns of the same inputs ({dt:.1f} s, OpenMP over rows)")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="gauss_1m_dv1", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a HIP device")
+    desc, flop_per_pair, bound = WORKLOADS[args.workload]
+    step, pairs, inp = build_step(args.workload)
+
+    for _ in range(max(1, args.warmup)):
+        step()
+    torch.cuda.synchronize()
+    # kernel-only time: HIP events recorded by the library around the launch, on the launch stream
+    mods = kernel_modules()
+    for m in mods:
+        m.set_timing(True)
+    kernel_ms = []
+    for _ in range(min(3, args.steps)):
+        step()
+        kernel_ms.append(max(m.last_kernel_ms() for m in mods))
+    for m in mods:
+        m.set_timing(False)
+    torch.cuda.synchronize()
+
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+
+    kms = sum(kernel_ms) / len(kernel_ms)
+    achieved = pairs * flop_per_pair / (kms * 1e-3) / 1e12
+    peak = PEAK_FP32_VECTOR_TFLOPS if bound == "valu" else PEAK_FP32_MFMA_TFLOPS
+    out = {
+        "metric": "pair interactions/sec (M*N/s), 1e6x1e6 D=3 Gauss sum" if args.workload == "gauss_1m_dv1"
+        else "pair interactions/sec (M*N/s)",
+        "value": pairs / dt,
+        "unit": "pairs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": (pairs / dt) / PUBLISHED_PAIRS_PER_S if args.workload == "gauss_1m_dv1" else None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": desc, "M": inp["M"], "N": inp["N"], "D": 3, "Dv": inp["Dv"],
+                   "baseline_hardware": "RTX 2080 Ti (reference benchmarks/README.md:14)"},
+        "roofline": {
+            "bound": bound, "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "kernel_ms": kms, "flop_per_pair": flop_per_pair,
+            "note": "peak is the packed-FP32 vector figure; kernels here issue scalar FP32 VALU ops only "
+                    "(packed FP32 is disabled), whose ceiling is 78.6 TFLOP/s",
+        },
+    }
+    if args.workload == "gauss_1m_dv1" and not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.workload, inp)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -132,8 +132,10 @@ struct ShapeTable {
     };
     auto check_var = [&](int i, int64_t dim, int cat, int64_t len) -> bool {
       if (i < 0 || i >= nargs) { err = "variable index " + std::to_string(i) + " out of range"; return false; }
-      const auto& shp = argshapes[i];
       const int want = cat == 2 ? nbatchdims + 1 : nbatchdims + 2;
+      // an argument with fewer leading dimensions is broadcast over the missing batch dimensions
+      std::vector<int64_t> shp = argshapes[i];
+      if ((int)shp.size() < want && (int)shp.size() >= (cat == 2 ? 1 : 2)) shp.insert(shp.begin(), want - shp.size(), 1);
       if ((int)shp.size() != want) {
         err = "argument " + std::to_string(i) + " has " + std::to_string(shp.size()) + " dimensions, expected " +
               std::to_string(want);
@@ -311,7 +313,7 @@ int keops_hip_compile(const char* target_file, const char* hip_src, int use_fast
   hiprtcResult r = hiprtcCreateProgram(&prog, hip_src, "keops_module.hip", (int)hdr_name.size(), hdr_text.data(), hdr_name.data());
   if (r != HIPRTC_SUCCESS) return fail((int)r, std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r));
   const std::string arch = "--offload-arch=" + target_arch(device_id);
-  std::vector<const char*> opts = {arch.c_str(), "-O3", "-std=c++17", "-fno-math-errno", "-ffp-contract=fast",
+  std::vector<const char*> opts = {arch.c_str(), "-O3", "-std=c++17", "-fno-math-errno", "-ffp-contract=fast-honor-pragmas",
                                    // packed FP32 instructions are kept out of every kernel of this library
                                    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
   const std::string fm = std::string("-DKEOPS_FAST_MATH=") + (use_fast_math ? "1" : "0");

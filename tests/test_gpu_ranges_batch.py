@@ -118,7 +118,7 @@ def test_batch_broadcasting_two_batch_dims_and_gradients():
     conv = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)", "g=Pm(1)"], reduction_op="Sum", axis=1)
     out = conv(x, y, b, g)
     assert tuple(out.shape) == (A, B, M, 2)
-    K = torch.exp(-g[..., None, :] * ((x[:, :, :, None, :] - y[:, :, None, :, :]) ** 2).sum(-1, keepdim=True))
+    K = torch.exp(-g[:, :, None, None, :] * ((x[:, :, :, None, :] - y[:, :, None, :, :]) ** 2).sum(-1, keepdim=True))
     ref = (K * b[:, :, None, :, :]).sum(3)
     assert rel_l2(out.detach().cpu().numpy(), ref.detach().cpu().numpy()) < 1e-12
     E = torch.from_numpy(rng.standard_normal((A, B, M, 2))).cuda()
