@@ -30,7 +30,10 @@ PUBLISHED_PAIRS_PER_S = 1e12 / 1.39
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/);
 # None until measured for a workload
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/keops_conv_dense__gauss_1m_dv1.md: FETCH_SIZE 230808 KiB x 2.0 (copy calibration) + WRITE_SIZE 3906.25 KiB
+    "gauss_1m_dv1": int((230808 * 2.0 + 3906.25) * 1024),
+}
 
 WORKLOADS = {
     # name: (description, algorithmic flop per pair, roofline bound)
@@ -126,6 +129,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="gauss_1m_dv1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run a plain 1 GiB device copy instead of a workload (reference point for the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -134,6 +140,14 @@ def main():
 
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a HIP device")
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4, "copies": args.steps}))
+        return
     desc, flop_per_pair, bound = WORKLOADS[args.workload]
     step, pairs, inp = build_step(args.workload)
 
