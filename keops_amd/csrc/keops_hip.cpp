@@ -257,17 +257,87 @@ struct LaunchHeader {
   const int64_t* offsets;
 };
 
-int launch(Module& m, const char* kernel, unsigned gx, unsigned gy, const LaunchHeader& h, void* const* args,
-           hipStream_t stream) {
+int launch_raw(Module& m, const char* kernel, unsigned gx, unsigned gy, unsigned block, void* params, size_t size,
+               hipStream_t stream) {
   hipFunction_t f;
   if (int rc = m.fn(kernel, &f)) return rc;
+  void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, params, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+  if (gx == 0 || gy == 0) return 0;
+  HIP_TRY(hipModuleLaunchKernel(f, gx, gy, 1, block, 1, 1, 0, stream, nullptr, extra));
+  return 0;
+}
+
+int launch(Module& m, const char* kernel, unsigned gx, unsigned gy, const LaunchHeader& h, void* const* args,
+           hipStream_t stream) {
   std::vector<char> buf(sizeof(LaunchHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs));
   std::memcpy(buf.data(), &h, sizeof(h));
   for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
-  size_t size = buf.size();
-  void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, buf.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
-  if (gx == 0 || gy == 0) return 0;
-  HIP_TRY(hipModuleLaunchKernel(f, gx, gy, 1, (unsigned)m.block, 1, 1, 0, stream, nullptr, extra));
+  return launch_raw(m, kernel, gx, gy, (unsigned)m.block, buf.data(), buf.size(), stream);
+}
+
+// ---- K-nearest-neighbour scheme (kernels/keops_knn_mfma.h) ---------------------------------------
+
+// must match struct KnnParams of kernels/keops_knn_mfma.h
+struct KnnHeader {
+  int64_t nq, nr;
+  const void* xq;
+  const void* yr;
+  void* xh;
+  void* yh;
+  void* xkey;
+  void* ykey;
+  void* colsum;
+  void* plist_d;
+  void* plist_i;
+  int64_t slab_len;
+  int32_t nslabs, pad_;
+  void* out;
+};
+
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr, void* out, int tag1D2D,
+               hipStream_t stream) {
+  const int64_t D = m.meta_int("knn_d", 0), DP = m.meta_int("knn_dpad", 0), K = m.meta_int("knn_k", 0);
+  const int64_t QB = m.meta_int("knn_qb", 256), TJ = m.tile_j;
+  if (D <= 0 || DP <= 0 || K <= 0) return fail(-1, "corrupt knn module metadata");
+  if (nr > 2147483647LL) return fail(-1, "too many reference rows for 32-bit indices");
+  const int64_t qblocks = (nq + QB - 1) / QB;
+  int64_t nslabs = 1;
+  const int64_t target = 6 * (int64_t)m.cu_count;
+  if (qblocks < target || tag1D2D == 1) {
+    nslabs = std::min<int64_t>((target + qblocks - 1) / qblocks, std::max<int64_t>(1, nr / (16 * TJ)));
+    nslabs = std::max<int64_t>(1, std::min<int64_t>(nslabs, 1024));
+  }
+  int64_t slab_len = (nr + nslabs - 1) / nslabs;
+  slab_len = (slab_len + TJ - 1) / TJ * TJ;
+  nslabs = std::max<int64_t>(1, (nr + slab_len - 1) / slab_len);
+
+  // workspace layout
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+  const size_t o_colsum = take((size_t)DP * 4), o_xh = take((size_t)nq * DP * 2), o_yh = take((size_t)nr * DP * 2);
+  const size_t o_xkey = take((size_t)nq * 4), o_ykey = take((size_t)nr * 4);
+  const size_t o_pd = take((size_t)nslabs * nq * K * 4), o_pi = take((size_t)nslabs * nq * K * 4);
+  if (int rc = m.partial.reserve(off)) return rc;
+  char* ws = (char*)m.partial.ptr;
+  struct { KnnHeader h; int32_t which; int32_t pad; } p{};
+  p.h.nq = nq; p.h.nr = nr; p.h.xq = xq; p.h.yr = yr;
+  p.h.xh = ws + o_xh; p.h.yh = ws + o_yh; p.h.xkey = ws + o_xkey; p.h.ykey = ws + o_ykey; p.h.colsum = ws + o_colsum;
+  p.h.plist_d = ws + o_pd; p.h.plist_i = ws + o_pi; p.h.slab_len = slab_len; p.h.nslabs = (int32_t)nslabs; p.h.out = out;
+
+  HIP_TRY(hipMemsetAsync(p.h.colsum, 0, (size_t)DP * 4, stream));
+  const unsigned cs_blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(1024, nr / 64));
+  if (int rc = launch_raw(m, "keops_knn_colsum", cs_blocks, 1, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
+  const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
+  p.which = 0;
+  if (int rc = launch_raw(m, "keops_knn_prep", (unsigned)((nq * lpr + 255) / 256), 1, 256, &p, sizeof(KnnHeader) + 4, stream)) return rc;
+  p.which = 1;
+  if (int rc = launch_raw(m, "keops_knn_prep", (unsigned)((nr * lpr + 255) / 256), 1, 256, &p, sizeof(KnnHeader) + 4, stream)) return rc;
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
+  if (int rc = launch_raw(m, "keops_knn_main", (unsigned)qblocks, (unsigned)nslabs, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
+  if (int rc = launch_raw(m, "keops_knn_merge", (unsigned)((nq + 255) / 256), 1, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
   return 0;
 }
 
@@ -497,7 +567,11 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
   h.nslabs = 1;
   h.slab_len = cols_total;
 
-  if (!use_ranges) {
+  if (m.scheme == "knn") {
+    if (use_ranges) return fail(-1, "the matrix-core KNN module does not handle ranges or batch dimensions");
+    const int rowarg = m.meta_int("rowarg", 0), colarg = m.meta_int("colarg", 1);
+    if (int rc = launch_knn(m, rows_total, cols_total, args[rowarg], args[colarg], out, tag1D2D, stream)) return rc;
+  } else if (!use_ranges) {
     // ---- dense scheme, optionally cut in column slabs ----
     const int64_t row_blocks = (rows_total + rows_per_block - 1) / rows_per_block;
     int64_t nslabs = 1;

@@ -131,6 +131,40 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
     return "\n".join(src) + "\n", meta
 
 
+def match_knn_sqdist(red, dtype, map_reduce_id):
+    """(row variable, column variable) when ``red`` is a K-min family reduction of SqDist between an
+    output-indexed and a reduced-index variable of dimension 32..256 in float32, on the dense
+    scheme; None otherwise.  Such reductions run on the matrix-core filter + exact re-rank kernels."""
+    from .formulas import ops as O
+
+    if red.kind != KIND_KMIN or dtype != "float" or "_ranges" in map_reduce_id or red.K > 64:
+        return None
+    f = red.formula
+    if f.name != "Sum" or f.children[0].name != "Square" or f.children[0].children[0].name != "Subtract":
+        return None
+    a, b = f.children[0].children[0].children
+    if not (isinstance(a, O.Var) and isinstance(b, O.Var)) or a.dim != b.dim or not 32 <= a.dim <= 256:
+        return None
+    if {a.cat, b.cat} != {0, 1}:
+        return None
+    return (a, b) if a.cat == red.tagI else (b, a)
+
+
+def generate_knn_plugin(red, rowvar, colvar, nargs):
+    D = rowvar.dim
+    dpad = -(-D // 16) * 16
+    qsets, tj = 2, 128
+    meta = dict(scheme="knn", block=256, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4, sizeof_acc=4,
+                nrowvars=1, ncolvars=1, nparvars=0, knn_d=D, knn_dpad=dpad, knn_k=red.K, knn_qb=4 * 32 * qsets,
+                rowarg=rowvar.ind, colarg=colvar.ind)
+    src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}", "typedef float T;"]
+    defs = dict(KEOPS_NARGS=nargs, KNN_D=D, KNN_DPAD=dpad, KNN_K=red.K, KEOPS_RED_KEEP=red.keep, KEOPS_DIMOUT=red.dim,
+                KNN_QSETS=qsets, KNN_TJ=tj)
+    src += [f"#define {k} {v}" for k, v in defs.items()]
+    src.append('#include "keops_knn_mfma.h"')
+    return "\n".join(src) + "\n", meta
+
+
 def get_keops_dll(
     map_reduce_id, red_formula_string, enable_chunks, enable_finalchunks, mul_var_highdim, aliases, nargs, dtype,
     dtypeacc, sum_scheme_string, tagHostDevice, tagCPUGPU, tag1D2D, use_half, use_fast_math, device_id, nx=None,
@@ -150,7 +184,7 @@ def get_keops_dll(
         # only the bucket matters for the cache key
         rows_hint = nx if nx < 8 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
-           use_fast_math, _rows_bucket(rows_hint), binder.templates_digest())
+           use_fast_math, _rows_bucket(rows_hint), bool(enable_chunks), binder.templates_digest())
     with _lock:
         hit = _cache.get(key)
     if hit is not None:
@@ -161,7 +195,12 @@ def get_keops_dll(
     if tagZero:
         target, tag, src_file = "", "zero", ""
     else:
-        source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint)
+        knn = match_knn_sqdist(red, dtype, map_reduce_id) if enable_chunks else None
+        if knn is not None:
+            source, meta = generate_knn_plugin(red, knn[0], knn[1], nargs)
+            use_chunk_mode = 3  # matrix-core filter scheme (no counterpart among the reference's chunk modes)
+        else:
+            source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint)
         tag = hashlib.sha256((source + binder.templates_digest() + str(use_fast_math)).encode()).hexdigest()[:16]
         folder = config.get_build_folder()
         target = os.path.join(folder, f"hsaco_{tag}")
