@@ -23,6 +23,12 @@ block_size = 256           # threads per workgroup (4 wavefronts)
 max_rows_per_lane = 4      # output rows held in the registers of one lane
 lds_tile_bytes = 16384     # LDS bytes of one staged column tile
 
+# matrix-core KNN kernel (csrc/kernels/keops_knn_mfma.h)
+knn_tile_j = int(os.environ.get("KEOPS_AMD_KNN_TJ", 128))          # reference rows per LDS tile (<= 256)
+knn_max_waves = int(os.environ.get("KEOPS_AMD_KNN_WAVES", 8))     # wavefronts per workgroup sharing one staged tile
+knn_lds_budget = 150 * 1024                                        # LDS bytes a KNN workgroup may use (160 KB per CU)
+knn_qsets = int(os.environ.get("KEOPS_AMD_KNN_QSETS", 1))          # 32-query operand sets per wavefront (<= 2)
+
 
 def get_build_folder():
     folder = os.environ.get("KEOPS_AMD_CACHE") or os.path.join(_PKG, "build")

@@ -303,12 +303,11 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   if (D <= 0 || DP <= 0 || K <= 0) return fail(-1, "corrupt knn module metadata");
   if (nr > 2147483647LL) return fail(-1, "too many reference rows for 32-bit indices");
   const int64_t qblocks = (nq + QB - 1) / QB;
-  int64_t nslabs = 1;
-  const int64_t target = 6 * (int64_t)m.cu_count;
-  if (qblocks < target || tag1D2D == 1) {
-    nslabs = std::min<int64_t>((target + qblocks - 1) / qblocks, std::max<int64_t>(1, nr / (16 * TJ)));
-    nslabs = std::max<int64_t>(1, std::min<int64_t>(nslabs, 1024));
-  }
+  // cut the reference axis in slabs until about two workgroups per compute unit exist
+  int64_t nslabs = std::max<int64_t>(1, (2 * (int64_t)m.cu_count) / qblocks);
+  if (tag1D2D == 1) nslabs = std::max<int64_t>(nslabs, 2);
+  nslabs = std::max<int64_t>(1, std::min<int64_t>(nslabs, std::max<int64_t>(1, nr / (16 * TJ))));
+  nslabs = std::min<int64_t>(nslabs, 1024);
   int64_t slab_len = (nr + nslabs - 1) / nslabs;
   slab_len = (slab_len + TJ - 1) / TJ * TJ;
   nslabs = std::max<int64_t>(1, (nr + slab_len - 1) / slab_len);
@@ -326,7 +325,7 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   p.h.xh = ws + o_xh; p.h.yh = ws + o_yh; p.h.xkey = ws + o_xkey; p.h.ykey = ws + o_ykey; p.h.colsum = ws + o_colsum;
   p.h.plist_d = ws + o_pd; p.h.plist_i = ws + o_pi; p.h.slab_len = slab_len; p.h.nslabs = (int32_t)nslabs; p.h.out = out;
 
-  HIP_TRY(hipMemsetAsync(p.h.colsum, 0, (size_t)DP * 4, stream));
+  if (int rc = launch_raw(m, "keops_knn_zero", 1, 1, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
   const unsigned cs_blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(1024, nr / 64));
   if (int rc = launch_raw(m, "keops_knn_colsum", cs_blocks, 1, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
   const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
@@ -335,7 +334,7 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   p.which = 1;
   if (int rc = launch_raw(m, "keops_knn_prep", (unsigned)((nr * lpr + 255) / 256), 1, 256, &p, sizeof(KnnHeader) + 4, stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
-  if (int rc = launch_raw(m, "keops_knn_main", (unsigned)qblocks, (unsigned)nslabs, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
+  if (int rc = launch_raw(m, "keops_knn_main", (unsigned)qblocks, (unsigned)nslabs, (unsigned)m.block, &p.h, sizeof(KnnHeader), stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
   if (int rc = launch_raw(m, "keops_knn_merge", (unsigned)((nq + 255) / 256), 1, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
   return 0;

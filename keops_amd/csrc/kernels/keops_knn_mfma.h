@@ -29,7 +29,7 @@
 //      lists under the same key and writes the output in the reference's layout.
 //
 // The plug-in defines: T (float), KEOPS_NARGS, KNN_D, KNN_DPAD (D rounded up to 16), KNN_K,
-// KEOPS_RED_KEEP, KEOPS_DIMOUT, KNN_QSETS, KNN_TJ, KNN_ROWARG, KNN_COLARG.
+// KEOPS_RED_KEEP, KEOPS_DIMOUT, KNN_QSETS, KNN_WAVES (wavefronts per workgroup), KNN_TJ.
 #pragma once
 #include "keops_common.h"
 
@@ -38,7 +38,6 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 knn_bf16x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float knn_f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float knn_f32x4;
 
-#define KNN_WAVES 4
 #define KNN_BLOCK (64 * KNN_WAVES)
 #define KNN_QW (32 * KNN_QSETS)        // queries per wavefront
 #define KNN_QB (KNN_WAVES * KNN_QW)    // queries per workgroup
@@ -47,6 +46,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float knn_f32x4;
 // filter slack: 4u(1+3u) + 2(D+1) 2^-24 with u = 2^-9, rounded up (see header comment)
 #define KNN_C 0.0082f
 #define KNN_DELTA 2e-5f
+#define KNN_FLT_MAX 3.402823466e38f
 
 struct KnnParams {
   i64 nq, nr;            // queries (output rows), references (reduced rows)
@@ -66,6 +66,10 @@ struct KnnParams {
 };
 
 // ---- pre-pass ---------------------------------------------------------------------------------
+
+extern "C" __global__ void __launch_bounds__(256) keops_knn_zero(const KnnParams P) {
+  if (threadIdx.x < KNN_DPAD) P.colsum[threadIdx.x] = 0.f;
+}
 
 extern "C" __global__ void __launch_bounds__(256) keops_knn_colsum(const KnnParams P) {
   // each workgroup sums a block of rows; 256 threads = (256 / KNN_DPAD) row lanes x KNN_DPAD columns
@@ -101,6 +105,9 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_prep(const KnnParams
       h[e] = (__bf16)v;
       const float r = (float)h[e];
       nrm += r * r;
+      // queries are stored as -2 x^ (exact in bf16) so that the MFMA accumulator, initialised with
+      // the reference keys, directly holds (1-c)|y^|^2 - 2 <y^, x^>
+      if (!which) h[e] = (__bf16)(-2.0f * r);
     }
     *reinterpret_cast<knn_bf16x4*>(dst + row * KNN_DPAD + sub * 4) = h;
   }
@@ -181,7 +188,7 @@ extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const Knn
     for (int kb = 0; kb < KNN_KB; kb++)
       bq[h][kb] = *reinterpret_cast<const knn_bf16x8*>(P.xh + q * KNN_DPAD + kb * 16 + 8 * half);
     xk[h] = P.xkey[q];
-    t[h] = valid[h] ? inf : -inf;
+    t[h] = valid[h] ? KNN_FLT_MAX : -inf;  // finite: padded rows carry an infinite key and never pass
   }
   for (int e = tid; e < KNN_QB * KNN_K; e += KNN_BLOCK) {
     (&lv[0][0])[e] = inf;
@@ -215,34 +222,55 @@ extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const Knn
 #pragma unroll
     for (int h = 0; h < KNN_QSETS; h++) {
       const float tau = lv[wave * KNN_QW + h * 32 + col][KNN_K - 1];
-      t[h] = valid[h] ? (tau + tau * KNN_DELTA) - xk[h] : -inf;
+      t[h] = valid[h] ? __builtin_fminf((tau + tau * KNN_DELTA) - xk[h], KNN_FLT_MAX) : -inf;
     }
   };
 
   const i64 jbeg = (i64)blockIdx.y * P.slab_len;
   const i64 jend = keops_min(P.nr, jbeg + P.slab_len);
+  // software pipeline: the rows of tile t+1 travel from HBM/L2 to registers while tile t is consumed
+  constexpr int CH = KNN_DPAD / 8;                              // 16-byte chunks per staged row
+  constexpr int NPF = (KNN_TJ * CH + KNN_BLOCK - 1) / KNN_BLOCK; // chunks per thread and tile
+  uint4 pf[NPF];
+  float pfkey = inf;
+  auto prefetch = [&](i64 j0) {
+    const int n = (int)keops_min((i64)KNN_TJ, jend - j0);
+    const uint4* src = reinterpret_cast<const uint4*>(P.yh + j0 * KNN_DPAD);
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * KNN_BLOCK;
+      pf[u] = (e < n * CH) ? src[e] : make_uint4(0u, 0u, 0u, 0u);
+    }
+    pfkey = (tid < n) ? P.ykey[j0 + tid] : inf;
+  };
+  static_assert(KNN_TJ <= KNN_BLOCK, "one key per thread");
+  if (jbeg < jend) prefetch(jbeg);
   for (i64 j0 = jbeg; j0 < jend; j0 += KNN_TJ) {
     const int n = (int)keops_min((i64)KNN_TJ, jend - j0);
-    __syncthreads();
-    {  // stage n reference rows (contiguous in yh) into padded LDS rows, 16 bytes per thread-step
-      constexpr int CH = KNN_DPAD / 8;  // 16-byte chunks per row
-      const uint4* src = reinterpret_cast<const uint4*>(P.yh + j0 * KNN_DPAD);
-      for (int e = tid; e < KNN_TJ * CH; e += KNN_BLOCK) {
+    __syncthreads();  // every wavefront is done with the previous tile
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * KNN_BLOCK;
+      if (e < KNN_TJ * CH) {
         const int row = e / CH, c = e - row * CH;
-        uint4 w = make_uint4(0u, 0u, 0u, 0u);
-        if (row < n) w = src[e];
-        *reinterpret_cast<uint4*>(ys + row * KNN_STRIDE + c * 16) = w;
+        *reinterpret_cast<uint4*>(ys + row * KNN_STRIDE + c * 16) = pf[u];
       }
-      for (int e = tid; e < KNN_TJ; e += KNN_BLOCK) ykey_s[e] = e < n ? P.ykey[j0 + e] : inf;
     }
+    if (tid < KNN_TJ) ykey_s[tid] = pfkey;
     __syncthreads();
+    if (j0 + KNN_TJ < jend) prefetch(j0 + KNN_TJ);
     const int nsub = (n + 31) / 32;
     for (int sub = 0; sub < nsub; sub++) {
+      // accumulator register v of this lane is reference row 8*(v/4) + 4*half + v%4 of the sub-tile:
+      // start from the keys of those rows
+      knn_f32x4 kk[4];
+#pragma unroll
+      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const knn_f32x4*>(ykey_s + sub * 32 + 8 * b + 4 * half);
       knn_f32x16 acc[KNN_QSETS];
 #pragma unroll
       for (int h = 0; h < KNN_QSETS; h++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) acc[h][v] = 0.f;
+        for (int v = 0; v < 16; v++) acc[h][v] = kk[v >> 2][v & 3];
       const unsigned char* arow = ys + (sub * 32 + col) * KNN_STRIDE + 16 * half;
 #pragma unroll
       for (int kb = 0; kb < KNN_KB; kb++) {
@@ -250,22 +278,12 @@ extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const Knn
 #pragma unroll
         for (int h = 0; h < KNN_QSETS; h++) acc[h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bq[h][kb], acc[h], 0, 0, 0);
       }
-      // accumulator register v of this lane is reference row 8*(v/4) + 4*half + v%4 of the sub-tile
-      knn_f32x4 kk[4];
-#pragma unroll
-      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const knn_f32x4*>(ykey_s + sub * 32 + 8 * b + 4 * half);
       unsigned mask = 0u;
       bool hit = false;
 #pragma unroll
-      for (int h = 0; h < KNN_QSETS; h++) {
-        float m = inf;
+      for (int h = 0; h < KNN_QSETS; h++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-          acc[h][v] = __builtin_fmaf(acc[h][v], -2.0f, kk[v >> 2][v & 3]);
-          m = __builtin_fminf(m, acc[h][v]);
-        }
-        hit = hit || (m <= t[h]);
-      }
+        for (int v = 0; v < 16; v++) hit |= acc[h][v] <= t[h];  // one v_cmp each, OR-ed on the scalar unit
       if (__any(hit)) {
 #pragma unroll
         for (int h = 0; h < KNN_QSETS; h++)

@@ -153,13 +153,19 @@ def match_knn_sqdist(red, dtype, map_reduce_id):
 def generate_knn_plugin(red, rowvar, colvar, nargs):
     D = rowvar.dim
     dpad = -(-D // 16) * 16
-    qsets, tj = 2, 128
-    meta = dict(scheme="knn", block=256, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4, sizeof_acc=4,
-                nrowvars=1, ncolvars=1, nparvars=0, knn_d=D, knn_dpad=dpad, knn_k=red.K, knn_qb=4 * 32 * qsets,
-                rowarg=rowvar.ind, colarg=colvar.ind)
+    qsets, tj = config.knn_qsets, config.knn_tile_j
+    # as many wavefronts as the LDS budget allows share one staged reference tile: the K-lists of the
+    # 32*qsets queries of every wavefront live in LDS (8 bytes per entry)
+    fixed = tj * (dpad * 2 + 16) + tj * 4
+    waves = config.knn_max_waves
+    while waves > 1 and fixed + waves * (32 * qsets * (red.K * 8 + 4) + 512) > config.knn_lds_budget:
+        waves //= 2
+    meta = dict(scheme="knn", block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
+                sizeof_acc=4, nrowvars=1, ncolvars=1, nparvars=0, knn_d=D, knn_dpad=dpad, knn_k=red.K,
+                knn_qb=waves * 32 * qsets, rowarg=rowvar.ind, colarg=colvar.ind)
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}", "typedef float T;"]
     defs = dict(KEOPS_NARGS=nargs, KNN_D=D, KNN_DPAD=dpad, KNN_K=red.K, KEOPS_RED_KEEP=red.keep, KEOPS_DIMOUT=red.dim,
-                KNN_QSETS=qsets, KNN_TJ=tj)
+                KNN_QSETS=qsets, KNN_TJ=tj, KNN_WAVES=waves)
     src += [f"#define {k} {v}" for k, v in defs.items()]
     src.append('#include "keops_knn_mfma.h"')
     return "\n".join(src) + "\n", meta
