@@ -46,6 +46,7 @@ WORKLOADS = {
     "knn_d64": ("KMin_ArgKMin K=10, 1e5 queries x 1e6 references, D=64 (BASELINE config 3)", 128, "mfma"),
     "sparse_100x10k": ("block-sparse Gaussian sum, 100 clusters x 10,000 points (BASELINE config 4)", 14, "valu"),
     "lse_b16": ("batched LogSumExp softmin B=16, 50,000 x 50,000, D=3 (BASELINE config 5a)", 17, "valu"),
+    # 2*D flop of the contraction + sqrt, neg, exp + 2*Dv of the weighted accumulation
     "laplace_d256": ("Laplace kernel sum 2e5 x 2e5, D=256, Dv=16 (BASELINE config 5b)", 547, "mfma"),
 }
 
@@ -65,6 +66,12 @@ def _np_inputs(name):
         M, N, D = 100_000, 1_000_000, 64
         rng = np.random.default_rng(2)
         return dict(M=M, N=N, Dv=0, D=D, arrays=[rng.random((M, D), dtype=np.float32), rng.random((N, D), dtype=np.float32)])
+    if name == "laplace_d256":
+        M = N = 200_000
+        rng = np.random.default_rng(5)
+        x = (rng.standard_normal((M, 256)) / 16).astype(np.float32)
+        y = (rng.standard_normal((N, 256)) / 16).astype(np.float32)
+        return dict(M=M, N=N, Dv=16, D=256, arrays=[x, y, rng.standard_normal((N, 16)).astype(np.float32)])
     raise SystemExit(f"workload {name} is not available in this build")
 
 
@@ -80,6 +87,9 @@ def build_step(name):
     if name == "knn_d64":
         knn = Genred("SqDist(x,y)", ["x=Vi(64)", "y=Vj(64)"], reduction_op="KMin_ArgKMin", axis=1, opt_arg=10)
         return (lambda: knn(*dev)), M * N, inp
+    if name == "laplace_d256":
+        lap = Genred("Exp(-Norm2(x-y))*b", ["x=Vi(256)", "y=Vj(256)", "b=Vj(16)"], reduction_op="Sum", axis=1)
+        return (lambda: lap(*dev)), M * N, inp
     conv = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", f"b=Vj({Dv})", "g=Pm(1)"], reduction_op="Sum", axis=1)
     if name == "gauss_1m_grad":
         # the gradient is another map-reduce (pykeops generic_red.py:165-214): run the forward once,
@@ -183,7 +193,7 @@ def main():
 
     kms = sum(kernel_ms) / len(kernel_ms)
     achieved = pairs * flop_per_pair / (kms * 1e-3) / 1e12
-    peak = PEAK_FP32_VECTOR_TFLOPS if bound == "valu" else (PEAK_BF16_MFMA_TFLOPS if args.workload == "knn_d64" else PEAK_FP32_MFMA_TFLOPS)
+    peak = PEAK_FP32_VECTOR_TFLOPS if bound == "valu" else (PEAK_BF16_MFMA_TFLOPS if args.workload in ("knn_d64", "laplace_d256") else PEAK_FP32_MFMA_TFLOPS)
     out = {
         "metric": "pair interactions/sec (M*N/s), 1e6x1e6 D=3 Gauss sum" if args.workload == "gauss_1m_dv1"
         else "pair interactions/sec (M*N/s)",

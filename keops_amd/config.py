@@ -23,6 +23,9 @@ block_size = 256           # threads per workgroup (4 wavefronts)
 max_rows_per_lane = 4      # output rows held in the registers of one lane
 lds_tile_bytes = 16384     # LDS bytes of one staged column tile
 
+# matrix-core chunked scheme (csrc/kernels/keops_chunk_mfma.h): wavefronts (32 output rows each) per workgroup
+chunk_waves = int(os.environ.get("KEOPS_AMD_CHUNK_WAVES", 8))
+
 # matrix-core KNN kernel (csrc/kernels/keops_knn_mfma.h)
 knn_tile_j = int(os.environ.get("KEOPS_AMD_KNN_TJ", 128))          # reference rows per LDS tile (<= 256)
 knn_max_waves = int(os.environ.get("KEOPS_AMD_KNN_WAVES", 8))     # wavefronts per workgroup sharing one staged tile

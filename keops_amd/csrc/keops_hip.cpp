@@ -287,6 +287,7 @@ struct KnnHeader {
   void* xkey;
   void* ykey;
   void* colsum;
+  void* colpart;
   void* plist_d;
   void* plist_i;
   int64_t slab_len;
@@ -315,19 +316,21 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   // workspace layout
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
-  const size_t o_colsum = take((size_t)DP * 4), o_xh = take((size_t)nq * DP * 2), o_yh = take((size_t)nr * DP * 2);
+  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(1024, nr / 64));
+  const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
+  const size_t o_xh = take((size_t)nq * DP * 2), o_yh = take((size_t)nr * DP * 2);
   const size_t o_xkey = take((size_t)nq * 4), o_ykey = take((size_t)nr * 4);
   const size_t o_pd = take((size_t)nslabs * nq * K * 4), o_pi = take((size_t)nslabs * nq * K * 4);
   if (int rc = m.partial.reserve(off)) return rc;
   char* ws = (char*)m.partial.ptr;
   struct { KnnHeader h; int32_t which; int32_t pad; } p{};
   p.h.nq = nq; p.h.nr = nr; p.h.xq = xq; p.h.yr = yr;
-  p.h.xh = ws + o_xh; p.h.yh = ws + o_yh; p.h.xkey = ws + o_xkey; p.h.ykey = ws + o_ykey; p.h.colsum = ws + o_colsum;
+  p.h.xh = ws + o_xh; p.h.yh = ws + o_yh; p.h.xkey = ws + o_xkey; p.h.ykey = ws + o_ykey; p.h.colsum = ws + o_colsum; p.h.colpart = ws + o_colpart;
   p.h.plist_d = ws + o_pd; p.h.plist_i = ws + o_pi; p.h.slab_len = slab_len; p.h.nslabs = (int32_t)nslabs; p.h.out = out;
 
-  if (int rc = launch_raw(m, "keops_knn_zero", 1, 1, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
-  const unsigned cs_blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(1024, nr / 64));
-  if (int rc = launch_raw(m, "keops_knn_colsum", cs_blocks, 1, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
+  if (int rc = launch_raw(m, "keops_knn_colsum", (unsigned)nparts, 1, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
+  p.which = nparts;
+  if (int rc = launch_raw(m, "keops_knn_colsum_final", 1, 1, 256, &p, sizeof(KnnHeader) + 4, stream)) return rc;
   const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
   p.which = 0;
   if (int rc = launch_raw(m, "keops_knn_prep", (unsigned)((nq * lpr + 255) / 256), 1, 256, &p, sizeof(KnnHeader) + 4, stream)) return rc;
@@ -347,6 +350,57 @@ int ensure_pinned(Module& m, size_t bytes) {
   m.pinned_bytes = 0;
   HIP_TRY(hipHostMalloc(&m.pinned, bytes, hipHostMallocDefault));
   m.pinned_bytes = bytes;
+  return 0;
+}
+
+// ---- matrix-core chunked scheme (kernels/keops_chunk_mfma.h) ---------------------------------------
+
+// must match struct ChkParams of kernels/keops_chunk_mfma.h (argument pointers follow)
+struct ChkHeader {
+  int64_t nx, ny;
+  void* xs;
+  void* ys;
+  void* xn;
+  void* yn;
+  void* colsum;
+  void* colpart;
+  void* out;
+};
+
+int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, hipStream_t stream) {
+  const int64_t D = m.meta_int("chk_d", 0), DP = m.meta_int("chk_dpad", 0), QB = m.meta_int("chk_qb", 128);
+  const int mode = m.meta_int("chk_mode", 0);
+  if (D <= 0 || DP <= 0) return fail(-1, "corrupt chunk module metadata");
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(2048, ny / 32));
+  const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
+  const size_t o_xs = take((size_t)nx * DP * 4), o_ys = take((size_t)ny * DP * 4);
+  const size_t o_xn = take((size_t)nx * 4), o_yn = take((size_t)ny * 4);
+  if (int rc = m.partial.reserve(off)) return rc;
+  char* ws = (char*)m.partial.ptr;
+  std::vector<char> buf(sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 8);
+  ChkHeader h{};
+  h.nx = nx; h.ny = ny; h.xs = ws + o_xs; h.ys = ws + o_ys; h.xn = ws + o_xn; h.yn = ws + o_yn; h.colsum = ws + o_colsum;
+  h.colpart = ws + o_colpart; h.out = out;
+  std::memcpy(buf.data(), &h, sizeof(h));
+  for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
+  const size_t psize = sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs);
+  int32_t which = 0;
+  auto with_which = [&](int w) { which = w; std::memcpy(buf.data() + psize, &which, 4); return psize + 4; };
+  if (mode == 0) {
+    if (int rc = launch_raw(m, "keops_chk_colsum", (unsigned)nparts, 1, 256, buf.data(), psize, stream)) return rc;
+    const size_t szp = with_which(nparts);
+    if (int rc = launch_raw(m, "keops_chk_colsum_final", 1, 1, 256, buf.data(), szp, stream)) return rc;
+  }
+  const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
+  size_t sz = with_which(0);
+  if (int rc = launch_raw(m, "keops_chk_prep", (unsigned)((nx * lpr + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  sz = with_which(1);
+  if (int rc = launch_raw(m, "keops_chk_prep", (unsigned)((ny * lpr + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
+  if (int rc = launch_raw(m, "keops_chk_main", (unsigned)((nx + QB - 1) / QB), 1, (unsigned)m.block, buf.data(), psize, stream)) return rc;
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
   return 0;
 }
 
@@ -570,6 +624,9 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
     if (use_ranges) return fail(-1, "the matrix-core KNN module does not handle ranges or batch dimensions");
     const int rowarg = m.meta_int("rowarg", 0), colarg = m.meta_int("colarg", 1);
     if (int rc = launch_knn(m, rows_total, cols_total, args[rowarg], args[colarg], out, tag1D2D, stream)) return rc;
+  } else if (m.scheme == "chunk") {
+    if (use_ranges) return fail(-1, "the matrix-core chunked module does not handle ranges or batch dimensions");
+    if (int rc = launch_chunk(m, rows_total, cols_total, out, args, stream)) return rc;
   } else if (!use_ranges) {
     // ---- dense scheme, optionally cut in column slabs ----
     const int64_t row_blocks = (rows_total + rows_per_block - 1) / rows_per_block;

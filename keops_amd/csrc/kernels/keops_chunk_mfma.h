@@ -1,0 +1,267 @@
+// High-dimensional map-reduce: the inner contraction over a large vector dimension runs on the
+// matrix cores, the rest of the formula and the reduction on the vector ALU.
+//
+// Counterpart of the reference's "chunked" schemes
+//   keopscore/keopscore/mapreduce/gpu/GpuReduc1D_chunks.py:19-118,255-330
+//   keopscore/keopscore/mapreduce/Chunk_Mode_Constants.py:6-140
+// which cut a Sum / Scalprod over a dimension >= 146 into 64-wide chunks accumulated per thread in
+// a local array, and then evaluate the "post-chunk" formula in which the chunked sub-formula has
+// become a scalar variable.  Here the chunked sub-formula
+//     s_ij = SqDist(x_i, y_j) = |x_i|^2 + |y_j|^2 - 2 <x_i, y_j>      (CHK_MODE 0)
+//     s_ij = <x_i, y_j>                                                (CHK_MODE 1)
+// is produced for a 32 x 32 tile of pairs by v_mfma_f32_32x32x16_bf16, and the post-chunk formula
+// F'(s_ij, other variables) is the generated straight-line code of KeopsFormula::eval.
+//
+// Precision: every float32 operand is split once as x = hi + lo with hi = bf16(x), lo = bf16(x - hi)
+// (a 16-bit significand in total) and <x, y> is accumulated in float32 from the three products
+// hi*hi + hi*lo + lo*hi; the dropped lo*lo term and the split residuals are below 2^-16 |x||y|.
+// For SqDist the rows are first centred on the column mean of y, which keeps |x|^2 + |y|^2 - 2<x,y>
+// well conditioned.  This is the accuracy class of the fast-math build; with use_fast_math=False
+// the engine does not select this scheme.
+//
+// Work decomposition: a wavefront owns 32 output rows ("queries") whose split operands stay in
+// VGPRs as the MFMA B matrix; the workgroup stages 32 reduced rows at a time in LDS (A matrix plus
+// the other reduced-index variables of the formula).  After the MFMAs lane l holds, for output row
+// l % 32, the 16 values s of reduced rows 8*(v/4) + 4*(l/32) + v%4; it evaluates the formula and
+// folds them in its private accumulator; the two lanes of a row merge their accumulators at the end
+// (ReducePair), so sums are deterministic.
+//
+// The plug-in defines: T (float), TACC, KEOPS_NARGS, CHK_D, CHK_DPAD, CHK_MODE, CHK_XARG, CHK_YARG,
+// CHK_WAVES, the KEOPS_DIM* / KEOPS_RED_* / KEOPS_SUM_SCHEME macros, the row/col/par variable
+// tables of the *other* variables, and KeopsFormula::eval(xi, yj, p, s, fout).
+#pragma once
+#include "keops_reductions.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 chk_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 chk_bf16x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float chk_f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float chk_f32x4;
+
+#define CHK_BLOCK (64 * CHK_WAVES)
+#define CHK_QB (32 * CHK_WAVES)              // output rows per workgroup
+#define CHK_KB (CHK_DPAD / 16)
+#define CHK_ROWBYTES (CHK_DPAD * 4)          // hi part then lo part, bf16 each
+#define CHK_STRIDE (CHK_ROWBYTES + 16)       // padded LDS row
+#define CHK_TJ 32                            // reduced rows per staged tile
+#define CHK_DY (KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1)
+
+struct ChkParams {
+  i64 nx, ny;           // output rows, reduced rows
+  __bf16* xs;           // [nx][2*CHK_DPAD] split (and centred, scaled) rows of the chunked row variable
+  __bf16* ys;           // [ny][2*CHK_DPAD]
+  float* xn;            // [nx] |x - mu|^2      (CHK_MODE 0)
+  float* yn;            // [ny]
+  float* colsum;        // [CHK_DPAD]
+  float* colpart;       // [nparts][CHK_DPAD] partial column sums
+  T* out;               // [nx][KEOPS_DIMOUT]
+  const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
+};
+
+// ---- pre-pass -----------------------------------------------------------------------------------
+
+// Column sums of the chunked column variable in two deterministic stages: per-workgroup partial
+// sums, then one workgroup adds the partials in a fixed order (no atomics: the same inputs always
+// give the same centring, hence bit-identical results from call to call).
+extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum(const ChkParams P) {
+  const i64 rows_per_block = (P.ny + gridDim.x - 1) / gridDim.x;
+  const i64 r0 = (i64)blockIdx.x * rows_per_block, r1 = keops_min(P.ny, r0 + rows_per_block);
+  const T* y = P.arg[CHK_YARG];
+  for (int c = threadIdx.x; c < CHK_DPAD; c += 256) {
+    float s = 0.f;
+    if (c < CHK_D)
+      for (i64 r = r0; r < r1; r++) s += y[r * CHK_D + c];
+    P.colpart[(i64)blockIdx.x * CHK_DPAD + c] = s;
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum_final(const ChkParams P, int nparts) {
+  for (int c = threadIdx.x; c < CHK_DPAD; c += 256) {
+    float s = 0.f;
+    for (int b = 0; b < nparts; b++) s += P.colpart[(i64)b * CHK_DPAD + c];
+    P.colsum[c] = s;
+  }
+}
+
+// One row per group of CHK_LPR lanes, 4 columns per lane; which = 0: row variable (stored times -2
+// in CHK_MODE 0), 1: column variable.  The squared norm is reduced inside the lane group
+// (deterministic).
+#define CHK_LPR (CHK_DPAD / 4 <= 4 ? 4 : (CHK_DPAD / 4 <= 8 ? 8 : (CHK_DPAD / 4 <= 16 ? 16 : (CHK_DPAD / 4 <= 32 ? 32 : 64))))
+extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams P, int which) {
+  const i64 n = which ? P.ny : P.nx;
+  const T* src = P.arg[which ? CHK_YARG : CHK_XARG];
+  __bf16* dst = which ? P.ys : P.xs;
+  const int q = threadIdx.x % CHK_LPR;
+  const i64 row = ((i64)blockIdx.x * 256 + threadIdx.x) / CHK_LPR;
+  const bool live = row < n && q * 4 < CHK_DPAD;
+  const float inv = 1.0f / (float)P.ny;
+  const float scale = (CHK_MODE == 0 && !which) ? -2.0f : 1.0f;
+  float nrm = 0.f;
+  if (live) {
+    chk_bf16x4 hi, lo;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const int c = q * 4 + e;
+      float v = 0.f;
+      if (c < CHK_D) {
+        v = src[row * CHK_D + c];
+        if (CHK_MODE == 0) v -= P.colsum[c] * inv;
+      }
+      nrm += v * v;
+      v *= scale;
+      hi[e] = (__bf16)v;
+      lo[e] = (__bf16)(v - (float)hi[e]);
+    }
+    *reinterpret_cast<chk_bf16x4*>(dst + row * 2 * CHK_DPAD + q * 4) = hi;
+    *reinterpret_cast<chk_bf16x4*>(dst + row * 2 * CHK_DPAD + CHK_DPAD + q * 4) = lo;
+  }
+#pragma unroll
+  for (int o = CHK_LPR / 2; o > 0; o >>= 1) nrm += __shfl_xor(nrm, o, CHK_LPR);
+  if (CHK_MODE == 0 && live && q == 0) (which ? P.yn : P.xn)[row] = nrm;
+}
+
+// ---- main kernel --------------------------------------------------------------------------------
+
+extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const ChkParams P) {
+  __shared__ __attribute__((aligned(16))) unsigned char as[CHK_TJ * CHK_STRIDE];  // A tile (hi|lo)
+  __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
+  __shared__ __attribute__((aligned(16))) T yo_s[CHK_TJ * CHK_DY];                // other column variables
+  __shared__ TACC merge_s[CHK_QB][KEOPS_DIMRED];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  i64 q = (i64)blockIdx.x * CHK_QB + wave * 32 + col;
+  const bool valid = q < P.nx;
+  if (!valid) q = P.nx - 1;
+
+  // B operands: split rows of the chunked row variable
+  chk_bf16x8 bh[CHK_KB], bl[CHK_KB];
+#pragma unroll
+  for (int kb = 0; kb < CHK_KB; kb++) {
+    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + kb * 16 + 8 * half);
+    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+  }
+  const float xnq = CHK_MODE == 0 ? P.xn[q] : 0.f;
+  // other row variables and parameters of the post-chunk formula
+  T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
+#pragma unroll
+  for (int v = 0; v < KEOPS_NROWVARS; v++) {
+    const T* src = P.arg[keops_row_arg[v]] + q * keops_row_dim[v];
+#pragma unroll
+    for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
+  }
+  T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+#pragma unroll
+  for (int v = 0; v < KEOPS_NPARVARS; v++) {
+    const T* src = P.arg[keops_par_arg[v]];
+#pragma unroll
+    for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
+  }
+  KeopsAcc<TACC> acc;
+  acc.init();
+
+  // software pipeline: tile t+1 travels to registers while tile t is consumed
+  constexpr int CH = CHK_ROWBYTES / 16;
+  constexpr int NPF = (CHK_TJ * CH + CHK_BLOCK - 1) / CHK_BLOCK;
+  uint4 pf[NPF];
+  float pfn = 0.f;
+  auto prefetch = [&](i64 j0) {
+    const int n = (int)keops_min((i64)CHK_TJ, P.ny - j0);
+    const uint4* src = reinterpret_cast<const uint4*>(P.ys + j0 * 2 * CHK_DPAD);
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * CHK_BLOCK;
+      pf[u] = (e < n * CH) ? src[e] : make_uint4(0u, 0u, 0u, 0u);
+    }
+    if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[j0 + tid] : 0.f;
+  };
+  if (P.ny > 0) prefetch(0);
+  for (i64 j0 = 0; j0 < P.ny; j0 += CHK_TJ) {
+    const int n = (int)keops_min((i64)CHK_TJ, P.ny - j0);
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * CHK_BLOCK;
+      if (e < CHK_TJ * CH) {
+        const int row = e / CH, c = e - row * CH;
+        *reinterpret_cast<uint4*>(as + row * CHK_STRIDE + c * 16) = pf[u];
+      }
+    }
+    if (CHK_MODE == 0 && tid < CHK_TJ) yn_s[tid] = pfn;
+    // the other reduced-index variables of this tile (small: loaded directly)
+#pragma unroll
+    for (int v = 0; v < KEOPS_NCOLVARS; v++) {
+      const int dim = keops_col_dim[v];
+      const T* src = P.arg[keops_col_arg[v]] + j0 * dim;
+      for (int e = tid; e < n * dim; e += CHK_BLOCK) {
+        const int row = e / dim, c = e - row * dim;
+        yo_s[row * CHK_DY + keops_col_off[v] + c] = src[e];
+      }
+    }
+    __syncthreads();
+    if (j0 + CHK_TJ < P.ny) prefetch(j0 + CHK_TJ);
+
+    // s tile: accumulator register v of this lane is reduced row 8*(v/4) + 4*half + v%4
+    chk_f32x16 s;
+    if (CHK_MODE == 0) {
+      chk_f32x4 kk[4];
+#pragma unroll
+      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const chk_f32x4*>(yn_s + 8 * b + 4 * half);
+#pragma unroll
+      for (int v = 0; v < 16; v++) s[v] = kk[v >> 2][v & 3];
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; v++) s[v] = 0.f;
+    }
+    const unsigned char* arow = as + col * CHK_STRIDE + 16 * half;
+#pragma unroll
+    for (int kb = 0; kb < CHK_KB; kb++) {
+      const chk_bf16x8 ah = *reinterpret_cast<const chk_bf16x8*>(arow + kb * 32);
+      const chk_bf16x8 al = *reinterpret_cast<const chk_bf16x8*>(arow + CHK_DPAD * 2 + kb * 32);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
+    }
+#if KEOPS_USE_TILE_TMP
+    KeopsAcc<T> tmp;
+    tmp.init();
+#endif
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int r = 8 * (v >> 2) + 4 * half + (v & 3);
+      if (r < n) {
+        T sv = s[v];
+        if (CHK_MODE == 0) sv = __builtin_fmaxf(sv + xnq, 0.f);
+        T yj[CHK_DY];
+        constexpr int VEC = 16 / sizeof(T);
+        typedef T vecT __attribute__((ext_vector_type(VEC)));
+#pragma unroll
+        for (int c4 = 0; c4 < KEOPS_DIMY_PAD / VEC; c4++) {
+          const vecT w = *reinterpret_cast<const vecT*>(yo_s + r * CHK_DY + c4 * VEC);
+#pragma unroll
+          for (int c = 0; c < VEC; c++) yj[c4 * VEC + c] = w[c];
+        }
+        T fout[KEOPS_DIMFOUT];
+        KeopsFormula::eval(xi, yj, p, sv, fout);
+#if KEOPS_USE_TILE_TMP
+        tmp.push(fout, j0 + r);
+#else
+        acc.push(fout, j0 + r);
+#endif
+      }
+    }
+#if KEOPS_USE_TILE_TMP
+    acc.merge(tmp);
+#endif
+  }
+
+  // the two lanes of an output row merge their accumulators (lower reduced rows first)
+  __syncthreads();
+  if (half == 1) acc.store_partial(merge_s[wave * 32 + col]);
+  __syncthreads();
+  if (half == 0) {
+    KeopsAcc<TACC> other;
+    other.load_partial(merge_s[wave * 32 + col]);
+    acc.merge(other);
+    if (valid) acc.finalize(P.out + q * KEOPS_DIMOUT);
+  }
+}

@@ -57,6 +57,7 @@ struct KnnParams {
   float* xkey;           // [nq]  (1-c)|x^|^2
   float* ykey;           // [nr]
   float* colsum;         // [KNN_DPAD] column sums of the references
+  float* colpart;        // [nparts][KNN_DPAD] partial column sums
   float* plist_d;        // [nslabs][nq][K] partial lists: distances
   int* plist_i;          //                                indices
   i64 slab_len;
@@ -67,20 +68,25 @@ struct KnnParams {
 
 // ---- pre-pass ---------------------------------------------------------------------------------
 
-extern "C" __global__ void __launch_bounds__(256) keops_knn_zero(const KnnParams P) {
-  if (threadIdx.x < KNN_DPAD) P.colsum[threadIdx.x] = 0.f;
-}
-
+// Column sums of the references in two deterministic stages (per-workgroup partials, then a
+// fixed-order final sum): no atomics.
 extern "C" __global__ void __launch_bounds__(256) keops_knn_colsum(const KnnParams P) {
-  // each workgroup sums a block of rows; 256 threads = (256 / KNN_DPAD) row lanes x KNN_DPAD columns
-  constexpr int RL = 256 / (KNN_DPAD <= 256 ? KNN_DPAD : 256);
-  const int c = threadIdx.x % KNN_DPAD, rl = threadIdx.x / KNN_DPAD;
-  if (rl >= RL || c >= KNN_D) return;
   const i64 rows_per_block = (P.nr + gridDim.x - 1) / gridDim.x;
   const i64 r0 = (i64)blockIdx.x * rows_per_block, r1 = keops_min(P.nr, r0 + rows_per_block);
-  float s = 0.f;
-  for (i64 r = r0 + rl; r < r1; r += RL) s += P.yr[r * KNN_D + c];
-  atomicAdd(&P.colsum[c], s);
+  for (int c = threadIdx.x; c < KNN_DPAD; c += 256) {
+    float s = 0.f;
+    if (c < KNN_D)
+      for (i64 r = r0; r < r1; r++) s += P.yr[r * KNN_D + c];
+    P.colpart[(i64)blockIdx.x * KNN_DPAD + c] = s;
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(256) keops_knn_colsum_final(const KnnParams P, int nparts) {
+  for (int c = threadIdx.x; c < KNN_DPAD; c += 256) {
+    float s = 0.f;
+    for (int b = 0; b < nparts; b++) s += P.colpart[(i64)b * KNN_DPAD + c];
+    P.colsum[c] = s;
+  }
 }
 
 // which = 0: queries, 1: references.  One row per group of KNN_LPR lanes, 4 columns per lane.

@@ -171,6 +171,90 @@ def generate_knn_plugin(red, rowvar, colvar, nargs):
     return "\n".join(src) + "\n", meta
 
 
+def match_chunk(red, dtype, map_reduce_id, use_fast_math):
+    """(mode, node, row variable, column variable) when the formula of a Sum / log-sum-exp reduction
+    contains exactly one high-dimensional contraction SqDist(x_i, y_j) (mode 0) or <x_i, y_j> (mode 1)
+    between plain variables of dimension 32..256 that appear nowhere else in the formula (the
+    reference's conditions, Chunkable_Op.py:20-41 and Chunk_Mode_Constants.py:56-60, with the
+    matrix-core dimension range instead of its >= 146 threshold).  None otherwise."""
+    from .formulas import ops as O
+    from .formulas.reductions import KIND_LSE, KIND_SUM
+
+    if red.kind not in (KIND_SUM, KIND_LSE) or dtype != "float" or not use_fast_math or "_ranges" in map_reduce_id:
+        return None
+    found = []
+    for node in red.formula.walk():
+        mode = pair = None
+        if node.name == "Sum" and node.children[0].name == "Square" and node.children[0].children[0].name == "Subtract":
+            mode, pair = 0, node.children[0].children[0].children
+        elif node.name == "Scalprod":
+            mode, pair = 1, node.children
+        if mode is None:
+            continue
+        a, b = pair
+        if isinstance(a, O.Var) and isinstance(b, O.Var) and a.dim == b.dim and 32 <= a.dim <= 256 and {a.cat, b.cat} == {0, 1}:
+            if node not in [f[1] for f in found]:
+                found.append((mode, node, a, b))
+    if len(found) != 1:
+        return None
+    mode, node, a, b = found[0]
+    post = red.formula.replace(node, O.Var(1 << 30, 1, 3))
+    if any(v == a or v == b for v in post.variables):
+        return None  # the chunked variables also appear outside the contraction
+    return (mode, node) + ((a, b) if a.cat == red.tagI else (b, a))
+
+
+def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
+    """Module source for the matrix-core chunked scheme (kernels/keops_chunk_mfma.h)."""
+    from .formulas import ops as O
+    from .formulas.reductions import Reduction
+
+    mode, node, xvar, yvar = match
+    svar = O.Var(1 << 30, 1, 3)
+    post = red.formula.replace(node, svar)
+
+    class _Post:  # what VarLayout needs: the post-chunk formula with the reduction's orientation
+        formula, tagI = post, red.tagI
+
+    layout = VarLayout(_Post)
+    layout.names[(3, svar.ind, 0)] = "s"
+    L = Lir(row_cat=red.tagI, fast_math=True, dtype="float")
+    outs = lower(post, L)
+    lines, exprs = L.emit(outs, layout.names, indent="    ")
+    D = xvar.dim
+    dpad = -(-D // 16) * 16
+    dimy_pad = 0 if layout.dimy == 0 else -(-layout.dimy // 4) * 4
+    waves = config.chunk_waves
+    ra, rd, ro = VarLayout.table(layout.rowvars)
+    ca, cd, co = VarLayout.table(layout.colvars)
+    pa, pd, po = VarLayout.table(layout.parvars)
+    meta = dict(scheme="chunk", block=64 * waves, rows=1, tile_j=32, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
+                sizeof_acc=8 if dtypeacc == "double" else 4, nrowvars=len(layout.rowvars) + 1,
+                ncolvars=len(layout.colvars) + 1, nparvars=len(layout.parvars), chk_d=D, chk_dpad=dpad, chk_mode=mode,
+                chk_qb=32 * waves, nops=L.count_ops(outs))
+    src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
+           f"typedef float T;\ntypedef {dtypeacc} TACC;", '#include "keops_common.h"']
+    defs = dict(
+        KEOPS_NARGS=nargs, CHK_D=D, CHK_DPAD=dpad, CHK_MODE=mode, CHK_XARG=xvar.ind, CHK_YARG=yvar.ind, CHK_WAVES=waves,
+        KEOPS_DIMX=layout.dimx, KEOPS_DIMY=layout.dimy, KEOPS_DIMY_PAD=dimy_pad, KEOPS_DIMP=layout.dimp,
+        KEOPS_DIMFOUT=post.dim, KEOPS_DIMRED=red.dimred, KEOPS_DIMOUT=red.dim, KEOPS_RED_KIND=red.kind,
+        KEOPS_RED_KEEP=red.keep, KEOPS_RED_K=red.K, KEOPS_SUM_SCHEME=SUM_SCHEMES[sum_scheme],
+        KEOPS_NROWVARS=len(layout.rowvars), KEOPS_NCOLVARS=len(layout.colvars), KEOPS_NPARVARS=len(layout.parvars),
+    )
+    src += [f"#define {k} {v}" for k, v in defs.items()]
+    for name, vals in (("row_arg", ra), ("row_dim", rd), ("row_off", ro), ("col_arg", ca), ("col_dim", cd),
+                       ("col_off", co), ("par_arg", pa), ("par_dim", pd), ("par_off", po)):
+        src.append(f"static __device__ constexpr int keops_{name}[] = {_c_list(vals)};")
+    dx, dy, dp = max(1, layout.dimx), max(1, dimy_pad), max(1, layout.dimp)
+    src.append("struct KeopsFormula {")
+    src.append(f"  static __device__ __forceinline__ void eval(const T (&xi)[{dx}], const T (&yj)[{dy}], "
+               f"const T (&p)[{dp}], const T s, T (&fout)[{post.dim}]) {{")
+    src += lines + [f"    fout[{k}] = {e};" for k, e in enumerate(exprs)]
+    src.append("  }\n};")
+    src.append('#include "keops_chunk_mfma.h"')
+    return "\n".join(src) + "\n", meta
+
+
 def get_keops_dll(
     map_reduce_id, red_formula_string, enable_chunks, enable_finalchunks, mul_var_highdim, aliases, nargs, dtype,
     dtypeacc, sum_scheme_string, tagHostDevice, tagCPUGPU, tag1D2D, use_half, use_fast_math, device_id, nx=None,
@@ -202,9 +286,13 @@ def get_keops_dll(
         target, tag, src_file = "", "zero", ""
     else:
         knn = match_knn_sqdist(red, dtype, map_reduce_id) if enable_chunks else None
+        chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
         if knn is not None:
             source, meta = generate_knn_plugin(red, knn[0], knn[1], nargs)
             use_chunk_mode = 3  # matrix-core filter scheme (no counterpart among the reference's chunk modes)
+        elif chk is not None:
+            source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs)
+            use_chunk_mode = 1
         else:
             source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint)
         tag = hashlib.sha256((source + binder.templates_digest() + str(use_fast_math)).encode()).hexdigest()[:16]

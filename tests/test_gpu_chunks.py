@@ -1,0 +1,104 @@
+"""GPU parity of the matrix-core chunked scheme (keops_chunk_mfma.h) for high-dimensional formulas:
+the result must equal the un-chunked formula (the scheme is only a schedule), cf. the reference's
+pykeops/test/test_chunks.py (D=300-style tests, atol 1e-4)."""
+import numpy as np
+import pytest
+import torch
+
+from common import assert_sum_parity, rel_l2, to_dev
+from oracle.cpu_oracle import cpu_reduc
+
+pytestmark = pytest.mark.gpu
+
+
+def _laplace_inputs(M, N, D, Dv, seed):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((M, D)) / np.sqrt(D)).astype(np.float32)
+    y = (rng.standard_normal((N, D)) / np.sqrt(D)).astype(np.float32)
+    b = rng.standard_normal((N, Dv)).astype(np.float32)
+    return x, y, b
+
+
+def _scheme_used(name):
+    from keops_amd import keops_io
+
+    return any(m.meta("scheme") == name for m in keops_io._modules.values())
+
+
+@pytest.mark.parametrize("M,N,D,Dv", [(1000, 1500, 256, 16), (333, 4097, 64, 3), (2049, 31, 100, 1), (50, 70, 32, 2)])
+def test_laplace_chunked_vs_oracle(M, N, D, Dv):
+    from keops_amd.torch import Genred
+
+    x, y, b = _laplace_inputs(M, N, D, Dv, 5)
+    conv = Genred("Exp(-Norm2(x-y))*b", [f"x=Vi({D})", f"y=Vj({D})", f"b=Vj({Dv})"], reduction_op="Sum", axis=1)
+    got = conv(*to_dev(x, y, b)).cpu().numpy()
+    assert _scheme_used("chunk")
+    ref = cpu_reduc("laplace", [x, y, b], M, N, Dv)
+    scale = cpu_reduc("laplace", [x, y, np.abs(b)], M, N, Dv)
+    assert_sum_parity(got, ref, scale)
+    # the un-chunked generic kernel (enable_chunks=False) is the same function
+    plain = Genred("Exp(-Norm2(x-y))*b", [f"x=Vi({D})", f"y=Vj({D})", f"b=Vj({Dv})"], reduction_op="Sum", axis=1,
+                   enable_chunks=False)(*to_dev(x, y, b)).cpu().numpy()
+    assert_sum_parity(plain, ref, scale)
+
+
+def test_config5b_laplace_d256_row_subset():
+    # BASELINE config 5b: M=N=200,000, D=256, Dv=16, x,y ~ N(0,1/D), seed 5
+    M = N = 200_000
+    from keops_amd.torch import Genred
+
+    x, y, b = _laplace_inputs(M, N, 256, 16, 5)
+    conv = Genred("Exp(-Norm2(x-y))*b", ["x=Vi(256)", "y=Vj(256)", "b=Vj(16)"], reduction_op="Sum", axis=1)
+    got = conv(*to_dev(x, y, b))
+    rows = np.sort(np.random.default_rng(9).choice(M, 512, replace=False)).astype(np.int64)
+    ref = cpu_reduc("laplace", [x, y, b], M, N, 16, rows=rows)
+    scale = cpu_reduc("laplace", [x, y, np.abs(b)], M, N, 16, rows=rows)
+    assert_sum_parity(got[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
+    twice = conv(*[t * s for t, s in zip(to_dev(x, y, b), (1, 1, 2))])
+    assert torch.equal(twice, 2 * got)  # linearity in b holds exactly
+
+
+def test_scalprod_mode_uncentred_data_axis0_and_lse():
+    from keops_amd.torch import Genred
+
+    M, N, D = 700, 900, 128
+    rng = np.random.default_rng(7)
+    x = (rng.standard_normal((M, D)) / np.sqrt(D) + 0.05).astype(np.float32)
+    y = (rng.standard_normal((N, D)) / np.sqrt(D) + 0.05).astype(np.float32)
+    b = rng.standard_normal((M, 2)).astype(np.float32)
+    p = np.array([0.7], np.float32)
+    xd, yd, bd, pd_ = to_dev(x, y, b, p)
+    x64, y64, b64 = (torch.from_numpy(t).double() for t in (x, y, b))
+    # reduction over i of exp(p * <x,y>) * b_i : Scalprod contraction, output indexed by j
+    conv = Genred("Exp(p*(x|y))*b", [f"x=Vi({D})", f"y=Vj({D})", "b=Vi(2)", "p=Pm(1)"], reduction_op="Sum", axis=0)
+    got = conv(xd, yd, bd, pd_).cpu().double()
+    K = torch.exp(0.7 * (x64 @ y64.T))  # (M,N)
+    ref = K.T @ b64
+    scale = K.T @ b64.abs()
+    assert_sum_parity(got.numpy(), ref.numpy(), scale.numpy())
+    # log-sum-exp of -SqDist/ (2 sigma^2) over a high-dimensional feature space, far from the origin
+    xs = (rng.standard_normal((M, D)) + 3.0).astype(np.float32)
+    ys = (rng.standard_normal((N, D)) + 3.0).astype(np.float32)
+    lse = Genred("-SqDist(x,y)*p", [f"x=Vi({D})", f"y=Vj({D})", "p=Pm(1)"], reduction_op="LogSumExp", axis=1)
+    got = lse(*to_dev(xs, ys, np.array([0.01], np.float32))).cpu().double()
+    d2 = torch.cdist(torch.from_numpy(xs).double(), torch.from_numpy(ys).double()) ** 2
+    ref = torch.logsumexp(-0.01 * d2, dim=1, keepdim=True)
+    assert float((got - ref).abs().max()) <= 1e-5 * max(1.0, float(ref.abs().max()))
+    assert _scheme_used("chunk")
+
+
+def test_gradient_through_chunked_formula():
+    from keops_amd.torch import Genred
+
+    M, N, D = 300, 400, 64
+    rng = np.random.default_rng(8)
+    x = torch.from_numpy((rng.standard_normal((M, D)) / 8).astype(np.float32)).cuda().requires_grad_(True)
+    y = torch.from_numpy((rng.standard_normal((N, D)) / 8).astype(np.float32)).cuda()
+    b = torch.from_numpy(rng.standard_normal((N, 1)).astype(np.float32)).cuda()
+    conv = Genred("Exp(-SqDist(x,y))*b", [f"x=Vi({D})", f"y=Vj({D})", "b=Vj(1)"], reduction_op="Sum", axis=1)
+    out = conv(x, y, b)
+    (gx,) = torch.autograd.grad(out.sum(), [x])
+    xt = x.detach().double().requires_grad_(True)
+    ref = (torch.exp(-torch.cdist(xt, y.double()) ** 2) @ b.double()).sum()
+    (rx,) = torch.autograd.grad(ref, [xt])
+    assert rel_l2(gx.cpu().numpy(), rx.cpu().numpy()) < 1e-5
