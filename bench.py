@@ -72,6 +72,22 @@ def _np_inputs(name):
         x = (rng.standard_normal((M, 256)) / 16).astype(np.float32)
         y = (rng.standard_normal((N, 256)) / 16).astype(np.float32)
         return dict(M=M, N=N, Dv=16, D=256, arrays=[x, y, rng.standard_normal((N, 16)).astype(np.float32)])
+    if name == "sparse_100x10k":
+        # 100 clusters x 10,000 points N(c_k, 0.05^2), c_k ~ U[0,10)^3, sigma = 0.1, centre distance < 1 kept
+        rng = np.random.default_rng(3)
+        C, per = 100, 10_000
+        c = (10 * rng.random((C, 3))).astype(np.float32)
+        x = (np.repeat(c, per, 0) + 0.05 * rng.standard_normal((C * per, 3))).astype(np.float32)
+        y = (np.repeat(c, per, 0) + 0.05 * rng.standard_normal((C * per, 3))).astype(np.float32)
+        b = rng.standard_normal((C * per, 1)).astype(np.float32)
+        return dict(M=C * per, N=C * per, Dv=1, centres=c, per=per, arrays=[x, y, b, np.array([100.0], np.float32)])
+    if name == "lse_b16":
+        rng = np.random.default_rng(4)
+        B, M, N = 16, 50_000, 50_000
+        x = rng.standard_normal((B, M, 3)).astype(np.float32)
+        y = rng.standard_normal((B, N, 3)).astype(np.float32)
+        l = rng.standard_normal((B, N, 1)).astype(np.float32)
+        return dict(M=M, N=N, Dv=1, B=B, arrays=[x, y, l, np.array([20.0], np.float32)])
     raise SystemExit(f"workload {name} is not available in this build")
 
 
@@ -90,6 +106,20 @@ def build_step(name):
     if name == "laplace_d256":
         lap = Genred("Exp(-Norm2(x-y))*b", ["x=Vi(256)", "y=Vj(256)", "b=Vj(16)"], reduction_op="Sum", axis=1)
         return (lambda: lap(*dev)), M * N, inp
+    if name == "lse_b16":
+        lse = Genred("l-SqDist(x,y)*e", ["x=Vi(3)", "y=Vj(3)", "l=Vj(1)", "e=Pm(1)"], reduction_op="LogSumExp", axis=1)
+        return (lambda: lse(*dev)), inp["B"] * M * N, inp
+    if name == "sparse_100x10k":
+        from keops_amd.torch.cluster import from_matrix
+
+        per, C = inp["per"], inp["centres"].shape[0]
+        r = torch.tensor([[per * k, per * (k + 1)] for k in range(C)], dtype=torch.int64, device="cuda")
+        ct = torch.from_numpy(inp["centres"]).cuda()
+        keep = torch.cdist(ct, ct) < 1.0
+        ranges = from_matrix(r, r, keep)
+        sp = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(1)", "g=Pm(1)"], reduction_op="Sum", axis=1)
+        kept_pairs = int(keep.sum().item()) * per * per  # effective pairs: kept cluster pairs only
+        return (lambda: sp(*dev, ranges=ranges)), kept_pairs, inp
     conv = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", f"b=Vj({Dv})", "g=Pm(1)"], reduction_op="Sum", axis=1)
     if name == "gauss_1m_grad":
         # the gradient is another map-reduce (pykeops generic_red.py:165-214): run the forward once,
