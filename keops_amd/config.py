@@ -29,6 +29,9 @@ chunk_waves = int(os.environ.get("KEOPS_AMD_CHUNK_WAVES", 8))
 # matrix-core KNN kernel (csrc/kernels/keops_knn_mfma.h)
 knn_tile_j = int(os.environ.get("KEOPS_AMD_KNN_TJ", 128))          # reference rows per LDS tile (<= 256)
 knn_max_waves = int(os.environ.get("KEOPS_AMD_KNN_WAVES", 8))     # wavefronts per workgroup sharing one staged tile
+knn_filter_waves = int(os.environ.get("KEOPS_AMD_KNN_FWAVES", 16))  # fixed-threshold filter: wavefronts per workgroup
+knn_filter_qsets = int(os.environ.get("KEOPS_AMD_KNN_FQSETS", 2))   # and 32-query operand sets per wavefront
+knn_sample = 16                                                    # sampling pass: every 16th reference
 knn_lds_budget = 150 * 1024                                        # LDS bytes a KNN workgroup may use (160 KB per CU)
 knn_qsets = int(os.environ.get("KEOPS_AMD_KNN_QSETS", 1))          # 32-query operand sets per wavefront (<= 2)
 

@@ -275,6 +275,16 @@ int launch(Module& m, const char* kernel, unsigned gx, unsigned gy, const Launch
   return launch_raw(m, kernel, gx, gy, (unsigned)m.block, buf.data(), buf.size(), stream);
 }
 
+int ensure_pinned(Module& m, size_t bytes) {
+  if (bytes <= m.pinned_bytes) return 0;
+  if (m.pinned) (void)hipHostFree(m.pinned);
+  m.pinned = nullptr;
+  m.pinned_bytes = 0;
+  HIP_TRY(hipHostMalloc(&m.pinned, bytes, hipHostMallocDefault));
+  m.pinned_bytes = bytes;
+  return 0;
+}
+
 // ---- K-nearest-neighbour scheme (kernels/keops_knn_mfma.h) ---------------------------------------
 
 // must match struct KnnParams of kernels/keops_knn_mfma.h
@@ -291,65 +301,132 @@ struct KnnHeader {
   void* plist_d;
   void* plist_i;
   int64_t slab_len;
-  int32_t nslabs, pad_;
+  int32_t nslabs, ref_step;
   void* out;
+  void* thr;
+  void* log;
+  void* logcount;
+  void* overflow;
+  int64_t logcap;
 };
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// number of reference slabs that gives about `per_cu` workgroups per compute unit
+int64_t pick_slabs(int64_t qblocks, int64_t nr, int64_t tile, int64_t cus, int64_t per_cu, int forced_min) {
+  int64_t n = std::max<int64_t>(1, (per_cu * cus) / std::max<int64_t>(1, qblocks));
+  n = std::max<int64_t>(n, forced_min);
+  n = std::min<int64_t>(n, std::max<int64_t>(1, nr / (16 * tile)));
+  return std::max<int64_t>(1, std::min<int64_t>(n, 1024));
+}
 
 int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr, void* out, int tag1D2D,
                hipStream_t stream) {
   const int64_t D = m.meta_int("knn_d", 0), DP = m.meta_int("knn_dpad", 0), K = m.meta_int("knn_k", 0);
   const int64_t QB = m.meta_int("knn_qb", 256), TJ = m.tile_j;
+  const int64_t FW = m.meta_int("knn_fwaves", 16), FQW = 32 * m.meta_int("knn_fqsets", 2), SAMPLE = m.meta_int("knn_sample", 16);
+  const int64_t FQB = FW * FQW;
   if (D <= 0 || DP <= 0 || K <= 0) return fail(-1, "corrupt knn module metadata");
   if (nr > 2147483647LL) return fail(-1, "too many reference rows for 32-bit indices");
-  const int64_t qblocks = (nq + QB - 1) / QB;
-  // cut the reference axis in slabs until about two workgroups per compute unit exist
-  int64_t nslabs = std::max<int64_t>(1, (2 * (int64_t)m.cu_count) / qblocks);
-  if (tag1D2D == 1) nslabs = std::max<int64_t>(nslabs, 2);
-  nslabs = std::max<int64_t>(1, std::min<int64_t>(nslabs, std::max<int64_t>(1, nr / (16 * TJ))));
-  nslabs = std::min<int64_t>(nslabs, 1024);
-  int64_t slab_len = (nr + nslabs - 1) / nslabs;
-  slab_len = (slab_len + TJ - 1) / TJ * TJ;
-  nslabs = std::max<int64_t>(1, (nr + slab_len - 1) / slab_len);
+  const bool two_phase = nr >= 32768 && nr / SAMPLE >= 8 * K && nq >= 1024;
+  const int64_t nsample = two_phase ? (nr + SAMPLE - 1) / SAMPLE : 0;
+
+  // adaptive pass: over the sample (two-phase) or over everything
+  const int64_t a_nr = two_phase ? nsample : nr;
+  const int64_t a_qblocks = (nq + QB - 1) / QB;
+  int64_t a_slabs = pick_slabs(a_qblocks, a_nr, TJ, m.cu_count, 2, tag1D2D == 1 && !two_phase ? 2 : 1);
+  int64_t a_len = ((a_nr + a_slabs - 1) / a_slabs + TJ - 1) / TJ * TJ;
+  a_slabs = std::max<int64_t>(1, (a_nr + a_len - 1) / a_len);
+  // filter pass
+  const int64_t f_qblocks = (nq + FQB - 1) / FQB;
+  int64_t f_slabs = pick_slabs(f_qblocks, nr, TJ, m.cu_count, 2, 1);
+  {
+    // one filter workgroup fills a CU and all of them take the same time: prefer a slab count whose
+    // grid is close to a whole number of rounds over the CUs
+    const int64_t cap = std::max<int64_t>(1, nr / (16 * TJ));
+    int64_t best = f_slabs;
+    double best_eff = 0.0;
+    for (int64_t n = f_slabs; n <= std::min<int64_t>(4 * f_slabs, cap); n++) {
+      const int64_t blocks = f_qblocks * n, rounds = (blocks + m.cu_count - 1) / m.cu_count;
+      const double eff = (double)blocks / (double)(rounds * m.cu_count);
+      if (eff > best_eff + 0.015) { best_eff = eff; best = n; }
+    }
+    f_slabs = best;
+  }
+  int64_t f_len = ((nr + f_slabs - 1) / f_slabs + TJ - 1) / TJ * TJ;
+  f_slabs = std::max<int64_t>(1, (nr + f_len - 1) / f_len);
+  const int64_t nlogs = f_qblocks * f_slabs * FW;
+  // expected survivors per query: SAMPLE * K (the sample's K-th neighbour is about the (SAMPLE*K)-th overall)
+  const int64_t logcap = two_phase ? align_up((size_t)(4 * FQW * SAMPLE * K / f_slabs + 512), 64) : 0;
+  const int64_t list_slabs = std::max<int64_t>(a_slabs, two_phase ? f_slabs : 1);
 
   // workspace layout
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
-  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(1024, nr / 64));
+  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(512, nr / 64));
   const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
   const size_t o_xh = take((size_t)nq * DP * 2), o_yh = take((size_t)nr * DP * 2);
   const size_t o_xkey = take((size_t)nq * 4), o_ykey = take((size_t)nr * 4);
-  const size_t o_pd = take((size_t)nslabs * nq * K * 4), o_pi = take((size_t)nslabs * nq * K * 4);
+  const size_t o_pd = take((size_t)list_slabs * nq * K * 4), o_pi = take((size_t)list_slabs * nq * K * 4);
+  const size_t o_yhs = take((size_t)nsample * DP * 2), o_ykeys = take((size_t)nsample * 4);
+  const size_t o_thr = take((size_t)nq * 4), o_flag = take(256);
+  const size_t o_logcount = take((size_t)(two_phase ? nlogs : 0) * 4), o_log = take((size_t)(two_phase ? nlogs : 0) * logcap * 8);
   if (int rc = m.partial.reserve(off)) return rc;
   char* ws = (char*)m.partial.ptr;
-  struct { KnnHeader h; int32_t which; int32_t pad; } p{};
-  p.h.nq = nq; p.h.nr = nr; p.h.xq = xq; p.h.yr = yr;
-  p.h.xh = ws + o_xh; p.h.yh = ws + o_yh; p.h.xkey = ws + o_xkey; p.h.ykey = ws + o_ykey; p.h.colsum = ws + o_colsum; p.h.colpart = ws + o_colpart;
-  p.h.plist_d = ws + o_pd; p.h.plist_i = ws + o_pi; p.h.slab_len = slab_len; p.h.nslabs = (int32_t)nslabs; p.h.out = out;
+  struct Packed { KnnHeader h; int64_t extra[3]; } p{};
+  KnnHeader& h = p.h;
+  h.nq = nq; h.nr = nr; h.xq = xq; h.yr = yr;
+  h.xh = ws + o_xh; h.yh = ws + o_yh; h.xkey = ws + o_xkey; h.ykey = ws + o_ykey; h.colsum = ws + o_colsum; h.colpart = ws + o_colpart;
+  h.plist_d = ws + o_pd; h.plist_i = ws + o_pi; h.out = out; h.ref_step = 1;
+  h.thr = ws + o_thr; h.log = ws + o_log; h.logcount = ws + o_logcount; h.overflow = ws + o_flag; h.logcap = logcap;
+  const size_t HS = sizeof(KnnHeader);
+  auto run = [&](const char* k, unsigned gx, unsigned gy, unsigned block, size_t size) {
+    return launch_raw(m, k, gx, gy, block, &p, size, stream);
+  };
+  auto with_int = [&](int v) { std::memcpy(p.extra, &v, 4); return HS + 4; };
 
-  if (int rc = launch_raw(m, "keops_knn_colsum", (unsigned)nparts, 1, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
-  p.which = nparts;
-  if (int rc = launch_raw(m, "keops_knn_colsum_final", 1, 1, 256, &p, sizeof(KnnHeader) + 4, stream)) return rc;
+  // pre-pass: centring, bf16 copies, keys
+  if (int rc = run("keops_knn_colsum", (unsigned)nparts, 1, 256, HS)) return rc;
+  if (int rc = run("keops_knn_colsum_final", 1, 1, 256, with_int(nparts))) return rc;
   const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
-  p.which = 0;
-  if (int rc = launch_raw(m, "keops_knn_prep", (unsigned)((nq * lpr + 255) / 256), 1, 256, &p, sizeof(KnnHeader) + 4, stream)) return rc;
-  p.which = 1;
-  if (int rc = launch_raw(m, "keops_knn_prep", (unsigned)((nr * lpr + 255) / 256), 1, 256, &p, sizeof(KnnHeader) + 4, stream)) return rc;
+  if (int rc = run("keops_knn_prep", (unsigned)((nq * lpr + 255) / 256), 1, 256, with_int(0))) return rc;
+  if (int rc = run("keops_knn_prep", (unsigned)((nr * lpr + 255) / 256), 1, 256, with_int(1))) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
-  if (int rc = launch_raw(m, "keops_knn_main", (unsigned)qblocks, (unsigned)nslabs, (unsigned)m.block, &p.h, sizeof(KnnHeader), stream)) return rc;
-  if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
-  if (int rc = launch_raw(m, "keops_knn_merge", (unsigned)((nq + 255) / 256), 1, 256, &p.h, sizeof(KnnHeader), stream)) return rc;
-  return 0;
-}
 
-int ensure_pinned(Module& m, size_t bytes) {
-  if (bytes <= m.pinned_bytes) return 0;
-  if (m.pinned) (void)hipHostFree(m.pinned);
-  m.pinned = nullptr;
-  m.pinned_bytes = 0;
-  HIP_TRY(hipHostMalloc(&m.pinned, bytes, hipHostMallocDefault));
-  m.pinned_bytes = bytes;
+  auto adaptive = [&](int64_t refs, void* yh, void* ykey, int step, int64_t slabs, int64_t len) -> int {
+    h.nr = refs; h.yh = yh; h.ykey = ykey; h.ref_step = step; h.nslabs = (int32_t)slabs; h.slab_len = len;
+    return run("keops_knn_main", (unsigned)a_qblocks, (unsigned)slabs, (unsigned)m.block, HS);
+  };
+  bool done = false;
+  if (two_phase) {
+    // (a) thresholds from every SAMPLE-th reference
+    void* gargs[3] = {ws + o_yhs, ws + o_ykeys, nullptr};
+    std::memcpy(&p.extra[0], &gargs[0], 8);
+    std::memcpy(&p.extra[1], &gargs[1], 8);
+    p.extra[2] = nsample;
+    const int64_t chunks = nsample * (DP / 8);
+    if (int rc = run("keops_knn_gather_sample", (unsigned)((chunks + 255) / 256), 1, 256, HS + 24)) return rc;
+    if (int rc = adaptive(nsample, ws + o_yhs, ws + o_ykeys, (int)SAMPLE, a_slabs, a_len)) return rc;
+    if (int rc = run("keops_knn_thresholds", (unsigned)((nq + 255) / 256), 1, 256, HS)) return rc;
+    // (b) fixed-threshold filter over all references, survivors logged per wavefront
+    h.nr = nr; h.yh = ws + o_yh; h.ykey = ws + o_ykey; h.ref_step = 1; h.nslabs = (int32_t)f_slabs; h.slab_len = f_len;
+    if (int rc = run("keops_knn_filter", (unsigned)f_qblocks, (unsigned)f_slabs, (unsigned)(64 * FW), HS)) return rc;
+    // (c) exact replay of the logs
+    if (int rc = run("keops_knn_rerank", (unsigned)nlogs, 1, 64, with_int((int)f_qblocks))) return rc;
+    if (int rc = ensure_pinned(m, 64)) return rc;
+    HIP_TRY(hipMemcpyAsync(m.pinned, h.overflow, 4, hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipStreamSynchronize(stream));
+    done = *(volatile int*)m.pinned == 0;  // a log overflowed (pathological ties): redo adaptively
+  }
+  if (!done) {
+    int64_t slabs = pick_slabs(a_qblocks, nr, TJ, m.cu_count, 2, tag1D2D == 1 ? 2 : 1);
+    slabs = std::min<int64_t>(slabs, list_slabs);
+    int64_t len = ((nr + slabs - 1) / slabs + TJ - 1) / TJ * TJ;
+    slabs = std::max<int64_t>(1, (nr + len - 1) / len);
+    if (int rc = adaptive(nr, ws + o_yh, ws + o_ykey, 1, slabs, len)) return rc;
+  }
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
+  if (int rc = run("keops_knn_merge", (unsigned)((nq + 255) / 256), 1, 256, HS)) return rc;
   return 0;
 }
 
@@ -373,7 +450,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (D <= 0 || DP <= 0) return fail(-1, "corrupt chunk module metadata");
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
-  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(2048, ny / 32));
+  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(512, ny / 64));
   const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
   const size_t o_xs = take((size_t)nx * DP * 4), o_ys = take((size_t)ny * DP * 4);
   const size_t o_xn = take((size_t)nx * 4), o_yn = take((size_t)ny * 4);

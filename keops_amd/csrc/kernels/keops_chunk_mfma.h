@@ -62,23 +62,58 @@ struct ChkParams {
 // Column sums of the chunked column variable in two deterministic stages: per-workgroup partial
 // sums, then one workgroup adds the partials in a fixed order (no atomics: the same inputs always
 // give the same centring, hence bit-identical results from call to call).
+#define CHK_CW (CHK_D > 128 ? 256 : (CHK_D > 64 ? 128 : (CHK_D > 32 ? 64 : 32)))
 extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum(const ChkParams P) {
+  // lanes run along the columns (coalesced rows), 256 / CHK_CW row groups per block
+  __shared__ float part[256];
+  constexpr int RG = 256 / CHK_CW;
+  const int cw = threadIdx.x % CHK_CW, rg = threadIdx.x / CHK_CW;
   const i64 rows_per_block = (P.ny + gridDim.x - 1) / gridDim.x;
   const i64 r0 = (i64)blockIdx.x * rows_per_block, r1 = keops_min(P.ny, r0 + rows_per_block);
   const T* y = P.arg[CHK_YARG];
-  for (int c = threadIdx.x; c < CHK_DPAD; c += 256) {
-    float s = 0.f;
-    if (c < CHK_D)
-      for (i64 r = r0; r < r1; r++) s += y[r * CHK_D + c];
-    P.colpart[(i64)blockIdx.x * CHK_DPAD + c] = s;
+  for (int c0 = 0; c0 < CHK_DPAD; c0 += CHK_CW) {
+    const int c = c0 + cw;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (c < CHK_D) {
+      i64 r = r0 + rg;
+      for (; r + 3 * RG < r1; r += 4 * RG) {
+        s0 += (float)y[r * CHK_D + c];
+        s1 += (float)y[(r + RG) * CHK_D + c];
+        s2 += (float)y[(r + 2 * RG) * CHK_D + c];
+        s3 += (float)y[(r + 3 * RG) * CHK_D + c];
+      }
+      for (; r < r1; r += RG) s0 += (float)y[r * CHK_D + c];
+    }
+    part[threadIdx.x] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (rg == 0 && c < CHK_DPAD) {
+      float s = 0.f;
+#pragma unroll
+      for (int g = 0; g < RG; g++) s += part[g * CHK_CW + cw];
+      P.colpart[(i64)blockIdx.x * CHK_DPAD + c] = s;
+    }
+    __syncthreads();
   }
 }
 
 extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum_final(const ChkParams P, int nparts) {
-  for (int c = threadIdx.x; c < CHK_DPAD; c += 256) {
+  __shared__ float part[256];
+  constexpr int RG = 256 / CHK_CW;
+  const int cw = threadIdx.x % CHK_CW, rg = threadIdx.x / CHK_CW;
+  for (int c0 = 0; c0 < CHK_DPAD; c0 += CHK_CW) {
+    const int c = c0 + cw;
     float s = 0.f;
-    for (int b = 0; b < nparts; b++) s += P.colpart[(i64)b * CHK_DPAD + c];
-    P.colsum[c] = s;
+    if (c < CHK_DPAD)
+      for (int b = rg; b < nparts; b += RG) s += P.colpart[(i64)b * CHK_DPAD + c];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    if (rg == 0 && c < CHK_DPAD) {
+      float t = 0.f;
+#pragma unroll
+      for (int g = 0; g < RG; g++) t += part[g * CHK_CW + cw];
+      P.colsum[c] = t;
+    }
+    __syncthreads();
   }
 }
 

@@ -27,6 +27,14 @@
 //      indices and distances are bit-identical to the CPU path.
 //   4. The reference axis can be cut in slabs (blockIdx.y); keops_knn_merge merges the per-slab
 //      lists under the same key and writes the output in the reference's layout.
+//   5. Large problems run in two phases so that the matrix-core sweep never waits for a re-rank:
+//      (a) the adaptive kernel of steps 2-3 runs on every KNN_SAMPLE-th reference only; the K-th
+//      distance it finds is an upper bound of the final one and becomes a *fixed* threshold;
+//      (b) keops_knn_filter sweeps all references against the fixed thresholds and only logs the
+//      surviving (query, reference) pairs, each wavefront in a private region of global memory (no
+//      atomics, no list updates); (c) keops_knn_rerank replays every log with the exact distance and
+//      the same K-list insertion.  If a log overflows (pathological ties) the host falls back to the
+//      adaptive kernel over all references.
 //
 // The plug-in defines: T (float), KEOPS_NARGS, KNN_D, KNN_DPAD (D rounded up to 16), KNN_K,
 // KEOPS_RED_KEEP, KEOPS_DIMOUT, KNN_QSETS, KNN_WAVES (wavefronts per workgroup), KNN_TJ.
@@ -38,9 +46,6 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 knn_bf16x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float knn_f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float knn_f32x4;
 
-#define KNN_BLOCK (64 * KNN_WAVES)
-#define KNN_QW (32 * KNN_QSETS)        // queries per wavefront
-#define KNN_QB (KNN_WAVES * KNN_QW)    // queries per workgroup
 #define KNN_KB (KNN_DPAD / 16)         // 16-wide k blocks
 #define KNN_STRIDE (KNN_DPAD * 2 + 16) // bytes per staged reference row (16 B pad: conflict-free b128 reads)
 // filter slack: 4u(1+3u) + 2(D+1) 2^-24 with u = 2^-9, rounded up (see header comment)
@@ -62,30 +67,70 @@ struct KnnParams {
   int* plist_i;          //                                indices
   i64 slab_len;
   int nslabs;
-  int pad_;
+  int ref_step;          // reference row j of this pass is row j*ref_step of yr (sub-sampled pass: > 1)
   T* out;                // [nq][KEOPS_DIMOUT]
+  float* thr;            // [nq] fixed filter thresholds of the two-phase scheme
+  int2* log;             // candidate logs of the filter pass: [nlogs][logcap] (local query, reference)
+  int* logcount;         // [nlogs] entries written (clamped to logcap)
+  int* overflow;         // set to 1 when a log was too small
+  i64 logcap;
 };
 
 // ---- pre-pass ---------------------------------------------------------------------------------
 
 // Column sums of the references in two deterministic stages (per-workgroup partials, then a
 // fixed-order final sum): no atomics.
+#define KNN_CW (KNN_D > 128 ? 256 : (KNN_D > 64 ? 128 : (KNN_D > 32 ? 64 : 32)))
 extern "C" __global__ void __launch_bounds__(256) keops_knn_colsum(const KnnParams P) {
+  // lanes run along the columns (coalesced rows), 256 / KNN_CW row groups per block; fixed summation order
+  __shared__ float part[256];
+  constexpr int RG = 256 / KNN_CW;
+  const int cw = threadIdx.x % KNN_CW, rg = threadIdx.x / KNN_CW;
   const i64 rows_per_block = (P.nr + gridDim.x - 1) / gridDim.x;
   const i64 r0 = (i64)blockIdx.x * rows_per_block, r1 = keops_min(P.nr, r0 + rows_per_block);
-  for (int c = threadIdx.x; c < KNN_DPAD; c += 256) {
-    float s = 0.f;
-    if (c < KNN_D)
-      for (i64 r = r0; r < r1; r++) s += P.yr[r * KNN_D + c];
-    P.colpart[(i64)blockIdx.x * KNN_DPAD + c] = s;
+  for (int c0 = 0; c0 < KNN_DPAD; c0 += KNN_CW) {
+    const int c = c0 + cw;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (c < KNN_D) {
+      i64 r = r0 + rg;
+      for (; r + 3 * RG < r1; r += 4 * RG) {
+        s0 += P.yr[r * KNN_D + c];
+        s1 += P.yr[(r + RG) * KNN_D + c];
+        s2 += P.yr[(r + 2 * RG) * KNN_D + c];
+        s3 += P.yr[(r + 3 * RG) * KNN_D + c];
+      }
+      for (; r < r1; r += RG) s0 += P.yr[r * KNN_D + c];
+    }
+    part[threadIdx.x] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (rg == 0 && c < KNN_DPAD) {
+      float s = 0.f;
+#pragma unroll
+      for (int g = 0; g < RG; g++) s += part[g * KNN_CW + cw];
+      P.colpart[(i64)blockIdx.x * KNN_DPAD + c] = s;
+    }
+    __syncthreads();
   }
 }
 
 extern "C" __global__ void __launch_bounds__(256) keops_knn_colsum_final(const KnnParams P, int nparts) {
-  for (int c = threadIdx.x; c < KNN_DPAD; c += 256) {
+  __shared__ float part[256];
+  constexpr int RG = 256 / KNN_CW;
+  const int cw = threadIdx.x % KNN_CW, rg = threadIdx.x / KNN_CW;
+  for (int c0 = 0; c0 < KNN_DPAD; c0 += KNN_CW) {
+    const int c = c0 + cw;
     float s = 0.f;
-    for (int b = 0; b < nparts; b++) s += P.colpart[(i64)b * KNN_DPAD + c];
-    P.colsum[c] = s;
+    if (c < KNN_DPAD)
+      for (int b = rg; b < nparts; b += RG) s += P.colpart[(i64)b * KNN_DPAD + c];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    if (rg == 0 && c < KNN_DPAD) {
+      float t = 0.f;
+#pragma unroll
+      for (int g = 0; g < RG; g++) t += part[g * KNN_CW + cw];
+      P.colsum[c] = t;
+    }
+    __syncthreads();
   }
 }
 
@@ -165,28 +210,25 @@ __device__ __forceinline__ void knn_insert(float* lv, int* li, float d, int j) {
   li[pos] = j;
 }
 
-// ---- main kernel ------------------------------------------------------------------------------
+// ---- sweep of the references: staging, MFMA filter, candidate queue ----------------------------
 
-extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const KnnParams P) {
-  __shared__ __attribute__((aligned(16))) unsigned char ys[KNN_TJ * KNN_STRIDE];
-  __shared__ __attribute__((aligned(16))) float ykey_s[KNN_TJ];
-  __shared__ float lv[KNN_QB][KNN_K];
-  __shared__ int li[KNN_QB][KNN_K];
-  __shared__ int owner[KNN_QB];
-  __shared__ int qq[KNN_WAVES][64];  // queued candidates: local query
-  __shared__ int qj[KNN_WAVES][64];  //                    reference index
-
+// MODE 0 (adaptive): thresholds follow the K-lists, full queues are re-examined at once.
+// MODE 1 (fixed thresholds): full queues are appended to the wavefront's log in global memory.
+template <int MODE, int WAVES, int QSETS>
+__device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys, float* ykey_s, float (*lv)[KNN_K],
+                                          int (*li)[KNN_K], int* owner, int (*qq)[64], int (*qj)[64]) {
+  constexpr int BLOCK = 64 * WAVES, QW = 32 * QSETS, QB = WAVES * QW;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
-  const i64 qw0 = (i64)blockIdx.x * KNN_QB + (i64)wave * KNN_QW;  // first query of this wavefront
+  const i64 qw0 = (i64)blockIdx.x * QB + (i64)wave * QW;  // first query of this wavefront
   const float inf = __builtin_huge_valf();
 
   // queries of this wavefront as MFMA B operands
-  knn_bf16x8 bq[KNN_QSETS][KNN_KB];
-  float xk[KNN_QSETS], t[KNN_QSETS];
-  bool valid[KNN_QSETS];
+  knn_bf16x8 bq[QSETS][KNN_KB];
+  float xk[QSETS], t[QSETS];
+  bool valid[QSETS];
 #pragma unroll
-  for (int h = 0; h < KNN_QSETS; h++) {
+  for (int h = 0; h < QSETS; h++) {
     i64 q = qw0 + h * 32 + col;
     valid[h] = q < P.nq;
     if (!valid[h]) q = P.nq - 1;
@@ -194,15 +236,22 @@ extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const Knn
     for (int kb = 0; kb < KNN_KB; kb++)
       bq[h][kb] = *reinterpret_cast<const knn_bf16x8*>(P.xh + q * KNN_DPAD + kb * 16 + 8 * half);
     xk[h] = P.xkey[q];
-    t[h] = valid[h] ? KNN_FLT_MAX : -inf;  // finite: padded rows carry an infinite key and never pass
+    // finite start value: padded rows carry an infinite key and never pass
+    if (MODE == 0) t[h] = valid[h] ? KNN_FLT_MAX : -inf;
+    else t[h] = valid[h] ? P.thr[q] : -inf;
   }
-  for (int e = tid; e < KNN_QB * KNN_K; e += KNN_BLOCK) {
-    (&lv[0][0])[e] = inf;
-    (&li[0][0])[e] = 0;
+  if (MODE == 0) {
+    for (int e = tid; e < QB * KNN_K; e += BLOCK) {
+      (&lv[0][0])[e] = inf;
+      (&li[0][0])[e] = 0;
+    }
   }
-  int qcount = 0;  // wave-uniform number of queued candidates
+  int qcount = 0;    // wave-uniform number of queued candidates
+  i64 logged = 0;    // wave-uniform number of entries already in this wavefront's log
+  const i64 logid = ((i64)blockIdx.y * gridDim.x + blockIdx.x) * WAVES + wave;
+  int2* mylog = MODE == 1 ? P.log + logid * P.logcap : nullptr;
 
-  // re-examine the queued candidates (one per lane) and refresh the thresholds
+  // MODE 0: re-examine the queued candidates (one per lane) and refresh the thresholds
   auto process = [&](int nb) {
     const bool act = lane < nb;
     int ql = 0, j = 0;
@@ -213,7 +262,7 @@ extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const Knn
       d = knn_exact_sqdist(P.xq + (qw0 + ql) * KNN_D, P.yr + (i64)j * KNN_D);
     }
     // several lanes may hold candidates of the same query: elect one owner per query and round
-    const int slot = wave * KNN_QW + ql;
+    const int slot = wave * QW + ql;
     volatile int* ow = owner;
     bool done = !act;
     while (__any(!done)) {
@@ -226,17 +275,26 @@ extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const Knn
       __threadfence_block();
     }
 #pragma unroll
-    for (int h = 0; h < KNN_QSETS; h++) {
-      const float tau = lv[wave * KNN_QW + h * 32 + col][KNN_K - 1];
+    for (int h = 0; h < QSETS; h++) {
+      const float tau = lv[wave * QW + h * 32 + col][KNN_K - 1];
       t[h] = valid[h] ? __builtin_fminf((tau + tau * KNN_DELTA) - xk[h], KNN_FLT_MAX) : -inf;
+    }
+  };
+  // MODE 1: append the queued candidates to the log (coalesced 8-byte stores, fire and forget)
+  auto flush = [&](int nb) {
+    if (logged + nb <= P.logcap) {
+      if (lane < nb) mylog[logged + lane] = make_int2(qq[wave][lane], qj[wave][lane]);
+      logged += nb;
+    } else {
+      if (lane == 0) *P.overflow = 1;
     }
   };
 
   const i64 jbeg = (i64)blockIdx.y * P.slab_len;
   const i64 jend = keops_min(P.nr, jbeg + P.slab_len);
   // software pipeline: the rows of tile t+1 travel from HBM/L2 to registers while tile t is consumed
-  constexpr int CH = KNN_DPAD / 8;                              // 16-byte chunks per staged row
-  constexpr int NPF = (KNN_TJ * CH + KNN_BLOCK - 1) / KNN_BLOCK; // chunks per thread and tile
+  constexpr int CH = KNN_DPAD / 8;                          // 16-byte chunks per staged row
+  constexpr int NPF = (KNN_TJ * CH + BLOCK - 1) / BLOCK;    // chunks per thread and tile
   uint4 pf[NPF];
   float pfkey = inf;
   auto prefetch = [&](i64 j0) {
@@ -244,19 +302,19 @@ extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const Knn
     const uint4* src = reinterpret_cast<const uint4*>(P.yh + j0 * KNN_DPAD);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
-      const int e = tid + u * KNN_BLOCK;
+      const int e = tid + u * BLOCK;
       pf[u] = (e < n * CH) ? src[e] : make_uint4(0u, 0u, 0u, 0u);
     }
     pfkey = (tid < n) ? P.ykey[j0 + tid] : inf;
   };
-  static_assert(KNN_TJ <= KNN_BLOCK, "one key per thread");
+  static_assert(KNN_TJ <= BLOCK, "one key per thread");
   if (jbeg < jend) prefetch(jbeg);
   for (i64 j0 = jbeg; j0 < jend; j0 += KNN_TJ) {
     const int n = (int)keops_min((i64)KNN_TJ, jend - j0);
     __syncthreads();  // every wavefront is done with the previous tile
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
-      const int e = tid + u * KNN_BLOCK;
+      const int e = tid + u * BLOCK;
       if (e < KNN_TJ * CH) {
         const int row = e / CH, c = e - row * CH;
         *reinterpret_cast<uint4*>(ys + row * KNN_STRIDE + c * 16) = pf[u];
@@ -272,9 +330,9 @@ extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const Knn
       knn_f32x4 kk[4];
 #pragma unroll
       for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const knn_f32x4*>(ykey_s + sub * 32 + 8 * b + 4 * half);
-      knn_f32x16 acc[KNN_QSETS];
+      knn_f32x16 acc[QSETS];
 #pragma unroll
-      for (int h = 0; h < KNN_QSETS; h++)
+      for (int h = 0; h < QSETS; h++)
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[h][v] = kk[v >> 2][v & 3];
       const unsigned char* arow = ys + (sub * 32 + col) * KNN_STRIDE + 16 * half;
@@ -282,54 +340,62 @@ extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const Knn
       for (int kb = 0; kb < KNN_KB; kb++) {
         const knn_bf16x8 a = *reinterpret_cast<const knn_bf16x8*>(arow + kb * 32);
 #pragma unroll
-        for (int h = 0; h < KNN_QSETS; h++) acc[h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bq[h][kb], acc[h], 0, 0, 0);
+        for (int h = 0; h < QSETS; h++) acc[h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bq[h][kb], acc[h], 0, 0, 0);
       }
-      unsigned mask = 0u;
-      bool hit = false;
+      // one v_cmp per pair; its wave-wide result lands in an SGPR pair and is tested on the scalar
+      // unit, so the common case (no survivor) costs no further vector work
 #pragma unroll
-      for (int h = 0; h < KNN_QSETS; h++)
+      for (int h = 0; h < QSETS; h++) {
+        // cheap screen first: the smallest of the lane's 16 values against the threshold (min3 tree)
+        float m = acc[h][0];
 #pragma unroll
-        for (int v = 0; v < 16; v++) hit |= acc[h][v] <= t[h];  // one v_cmp each, OR-ed on the scalar unit
-      if (__any(hit)) {
+        for (int v = 1; v < 16; v += 2)
+          m = __builtin_fminf(__builtin_fminf(m, acc[h][v]), v + 1 < 16 ? acc[h][v + 1] : acc[h][v]);
+        if (__builtin_expect(!__any(m <= t[h]), 1)) continue;
+        // all 16 compares first (independent, pipelined), then scalar tests of their wave-wide masks
+        unsigned long long bals[16];
 #pragma unroll
-        for (int h = 0; h < KNN_QSETS; h++)
+        for (int v = 0; v < 16; v++) bals[v] = __ballot(acc[h][v] <= t[h]);
 #pragma unroll
-          for (int v = 0; v < 16; v++)
-            if (acc[h][v] <= t[h]) mask |= 1u << (h * 16 + v);
-        // KNN_QSETS <= 2 keeps the mask in 32 bits
-        while (true) {
-          const bool has = mask != 0u;
-          const unsigned long long bal = __ballot(has);
-          if (bal == 0ull) break;
-          const int slot = qcount + __popcll(bal & ((1ull << lane) - 1ull));
-          if (has && slot < 64) {
-            const int bit = __ffs(mask) - 1;
-            mask &= mask - 1u;
-            const int h = bit >> 4, v = bit & 15;
-            qq[wave][slot] = h * 32 + col;
-            qj[wave][slot] = (int)(j0 + sub * 32 + 8 * (v >> 2) + 4 * half + (v & 3));
-          }
-          qcount += __popcll(bal);
-          if (qcount >= 64) {
-            process(64);
-            qcount = 0;
-            // candidates that found the queue full retry; drop those the new thresholds exclude
-#pragma unroll
-            for (int h = 0; h < KNN_QSETS; h++)
-#pragma unroll
-              for (int v = 0; v < 16; v++)
-                if (!(acc[h][v] <= t[h])) mask &= ~(1u << (h * 16 + v));
+        for (int v = 0; v < 16; v++) {
+          unsigned long long bal = bals[v];
+          bool mine = (bal >> lane) & 1ull;
+          while (__builtin_expect(bal != 0ull, 0)) {
+            const int slot = qcount + __popcll(bal & ((1ull << lane) - 1ull));
+            if (mine && slot < 64) {
+              qq[wave][slot] = h * 32 + col;
+              qj[wave][slot] = (int)(j0 + sub * 32 + 8 * (v >> 2) + 4 * half + (v & 3)) * P.ref_step;
+              mine = false;
+            }
+            qcount += __popcll(bal);
+            if (qcount >= 64) {
+              if (MODE == 0) process(64);
+              else flush(64);
+              qcount = 0;
+              // lanes that found the queue full retry (MODE 0: unless the new threshold excludes them)
+              if (MODE == 0) mine = mine && (acc[h][v] <= t[h]);
+              bal = __ballot(mine);
+            } else {
+              bal = 0ull;
+            }
           }
         }
       }
     }
   }
-  if (qcount > 0) process(qcount);
+  if (qcount > 0) {
+    if (MODE == 0) process(qcount);
+    else flush(qcount);
+  }
+  if (MODE == 1) {
+    if (lane == 0) P.logcount[logid] = (int)logged;
+    return;
+  }
   __syncthreads();
   // partial lists of this slab
-  for (int e = tid; e < KNN_QB * KNN_K; e += KNN_BLOCK) {
+  for (int e = tid; e < QB * KNN_K; e += BLOCK) {
     const int ql = e / KNN_K, l = e - ql * KNN_K;
-    const i64 q = (i64)blockIdx.x * KNN_QB + ql;
+    const i64 q = (i64)blockIdx.x * QB + ql;
     if (q < P.nq) {
       const i64 o = ((i64)blockIdx.y * P.nq + q) * KNN_K + l;
       P.plist_d[o] = lv[ql][l];
@@ -338,13 +404,42 @@ extern "C" __global__ void __launch_bounds__(KNN_BLOCK) keops_knn_main(const Knn
   }
 }
 
-// ---- merge of the per-slab lists and output ---------------------------------------------------
+// adaptive kernel: KNN_WAVES wavefronts of 32*KNN_QSETS queries
+extern "C" __global__ void __launch_bounds__(64 * KNN_WAVES) keops_knn_main(const KnnParams P) {
+  __shared__ __attribute__((aligned(16))) unsigned char ys[KNN_TJ * KNN_STRIDE];
+  __shared__ __attribute__((aligned(16))) float ykey_s[KNN_TJ];
+  __shared__ float lv[KNN_WAVES * 32 * KNN_QSETS][KNN_K];
+  __shared__ int li[KNN_WAVES * 32 * KNN_QSETS][KNN_K];
+  __shared__ int owner[KNN_WAVES * 32 * KNN_QSETS];
+  __shared__ int qq[KNN_WAVES][64];  // queued candidates: local query
+  __shared__ int qj[KNN_WAVES][64];  //                    reference index
+  knn_sweep<0, KNN_WAVES, KNN_QSETS>(P, ys, ykey_s, lv, li, owner, qq, qj);
+}
 
-extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParams P) {
-  const i64 q = (i64)blockIdx.x * 256 + threadIdx.x;
-  if (q >= P.nq) return;
-  float bv[KNN_K];
-  int bi[KNN_K];
+// fixed-threshold filter: KNN_FWAVES wavefronts of 32*KNN_FQSETS queries share every staged tile
+extern "C" __global__ void __launch_bounds__(64 * KNN_FWAVES) keops_knn_filter(const KnnParams P) {
+  __shared__ __attribute__((aligned(16))) unsigned char ys[KNN_TJ * KNN_STRIDE];
+  __shared__ __attribute__((aligned(16))) float ykey_s[KNN_TJ];
+  __shared__ int qq[KNN_FWAVES][64];
+  __shared__ int qj[KNN_FWAVES][64];
+  knn_sweep<1, KNN_FWAVES, KNN_FQSETS>(P, ys, ykey_s, nullptr, nullptr, nullptr, qq, qj);
+}
+
+// every KNN_SAMPLE-th reference row (bf16 row + key) gathered in a compact array for the sampling pass
+extern "C" __global__ void __launch_bounds__(256) keops_knn_gather_sample(const KnnParams P, __bf16* yh_s, float* ykey_sm,
+                                                                           i64 nsample) {
+  constexpr int CH = KNN_DPAD / 8;
+  const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
+  const i64 row = e / CH;
+  const int c = (int)(e - row * CH);
+  if (row >= nsample) return;
+  reinterpret_cast<uint4*>(yh_s)[e] = reinterpret_cast<const uint4*>(P.yh)[row * KNN_SAMPLE * CH + c];
+  if (c == 0) ykey_sm[row] = P.ykey[row * KNN_SAMPLE];
+}
+
+// ---- merge of the per-slab lists ----------------------------------------------------------------
+
+__device__ __forceinline__ void knn_merge_lists(const KnnParams& P, i64 q, float (&bv)[KNN_K], int (&bi)[KNN_K]) {
 #pragma unroll
   for (int l = 0; l < KNN_K; l++) {
     bv[l] = P.plist_d[q * KNN_K + l];
@@ -370,6 +465,14 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParam
       }
     }
   }
+}
+
+extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParams P) {
+  const i64 q = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (q >= P.nq) return;
+  float bv[KNN_K];
+  int bi[KNN_K];
+  knn_merge_lists(P, q, bv, bi);
   T* out = P.out + q * KEOPS_DIMOUT;
 #pragma unroll
   for (int l = 0; l < KNN_K; l++) {
@@ -381,5 +484,74 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParam
 #else
     out[l] = (T)bi[l];
 #endif
+  }
+}
+
+// thresholds of the filter pass from the K-lists of the sampling pass
+extern "C" __global__ void __launch_bounds__(256) keops_knn_thresholds(const KnnParams P) {
+  const i64 q = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (q == 0) *P.overflow = 0;  // reset before the filter pass (a fill kernel would be one more launch)
+  if (q >= P.nq) return;
+  float bv[KNN_K];
+  int bi[KNN_K];
+  knn_merge_lists(P, q, bv, bi);
+  const float tau = bv[KNN_K - 1];
+  P.thr[q] = __builtin_fminf((tau + tau * KNN_DELTA) - P.xkey[q], KNN_FLT_MAX);
+}
+
+// ---- replay of the candidate logs ---------------------------------------------------------------
+
+// One wavefront per log (= per filter wavefront and slab): exact distances and K-list insertion for
+// its 32*KNN_FQSETS queries, then the partial lists of that slab.
+extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParams P, int fgrid_x) {
+  constexpr int QW = 32 * KNN_FQSETS;
+  __shared__ float lv[QW][KNN_K];
+  __shared__ int li[QW][KNN_K];
+  __shared__ int owner[QW];
+  const int lane = threadIdx.x;
+  const i64 logid = blockIdx.x;
+  const int wave = (int)(logid % KNN_FWAVES);
+  const i64 rest = logid / KNN_FWAVES;
+  const i64 bx = rest % fgrid_x, slab = rest / fgrid_x;
+  const i64 qw0 = bx * (KNN_FWAVES * QW) + (i64)wave * QW;
+  const float inf = __builtin_huge_valf();
+  for (int e = lane; e < QW * KNN_K; e += 64) {
+    (&lv[0][0])[e] = inf;
+    (&li[0][0])[e] = 0;
+  }
+  __syncthreads();
+  const int count = P.logcount[logid];
+  const int2* mylog = P.log + logid * P.logcap;
+  volatile int* ow = owner;
+  for (int base = 0; base < count; base += 64) {
+    const bool act = base + lane < count;
+    int ql = 0, j = 0;
+    float d = inf;
+    if (act) {
+      const int2 e = mylog[base + lane];
+      ql = e.x;
+      j = e.y;
+      d = knn_exact_sqdist(P.xq + (qw0 + ql) * KNN_D, P.yr + (i64)j * KNN_D);
+    }
+    bool done = !act;
+    while (__any(!done)) {
+      if (!done) ow[ql] = lane;
+      __threadfence_block();
+      if (!done && ow[ql] == lane) {
+        knn_insert(lv[ql], li[ql], d, j);
+        done = true;
+      }
+      __threadfence_block();
+    }
+  }
+  __syncthreads();
+  for (int e = lane; e < QW * KNN_K; e += 64) {
+    const int ql = e / KNN_K, l = e - ql * KNN_K;
+    const i64 q = qw0 + ql;
+    if (q < P.nq) {
+      const i64 o = (slab * P.nq + q) * KNN_K + l;
+      P.plist_d[o] = lv[ql][l];
+      P.plist_i[o] = li[ql][l];
+    }
   }
 }
