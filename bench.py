@@ -48,15 +48,17 @@ WORKLOADS = {
     "lse_b16": ("batched LogSumExp softmin B=16, 50,000 x 50,000, D=3 (BASELINE config 5a)", 17, "valu"),
     # 2*D flop of the contraction + sqrt, neg, exp + 2*Dv of the weighted accumulation
     "laplace_d256": ("Laplace kernel sum 2e5 x 2e5, D=256, Dv=16 (BASELINE config 5b)", 547, "mfma"),
+    # 12 flop of the Gaussian kernel + 2*Dv of the product with the 256-dimensional variable (float32 matrix cores)
+    "gauss_dv256": ("Gaussian kernel times a 256-dimensional variable, 2e5 x 2e5, D=3 (final-product scheme)", 524, "mfma32"),
 }
 
 
 def _np_inputs(name):
     import numpy as np
 
-    if name.startswith("gauss_1m") or name == "gauss_10k":
-        M = N = 10_000 if name == "gauss_10k" else 1_000_000
-        Dv = 8 if name.endswith("dv8") else 1
+    if name.startswith("gauss_1m") or name in ("gauss_10k", "gauss_dv256"):
+        M = N = 10_000 if name == "gauss_10k" else (200_000 if name == "gauss_dv256" else 1_000_000)
+        Dv = 8 if name.endswith("dv8") else (256 if name == "gauss_dv256" else 1)
         rng = np.random.default_rng(0 if name == "gauss_10k" else 1)
         x = rng.standard_normal((M, 3)).astype(np.float32)
         y = rng.standard_normal((N, 3)).astype(np.float32)
@@ -223,7 +225,10 @@ def main():
 
     kms = sum(kernel_ms) / len(kernel_ms)
     achieved = pairs * flop_per_pair / (kms * 1e-3) / 1e12
-    peak = PEAK_FP32_VECTOR_TFLOPS if bound == "valu" else (PEAK_BF16_MFMA_TFLOPS if args.workload in ("knn_d64", "laplace_d256") else PEAK_FP32_MFMA_TFLOPS)
+    peak = {"valu": PEAK_FP32_VECTOR_TFLOPS, "mfma": PEAK_BF16_MFMA_TFLOPS, "mfma32": PEAK_FP32_MFMA_TFLOPS}[bound]
+    note = {"valu": "peak is the packed-FP32 vector figure; kernels here issue scalar FP32 VALU ops only "
+                    "(packed FP32 is disabled), whose ceiling is 78.6 TFLOP/s",
+            "mfma": "peak is the dense bf16 matrix figure", "mfma32": "peak is the dense fp32 matrix figure"}[bound]
     out = {
         "metric": "pair interactions/sec (M*N/s), 1e6x1e6 D=3 Gauss sum" if args.workload == "gauss_1m_dv1"
         else "pair interactions/sec (M*N/s)",
@@ -241,11 +246,10 @@ def main():
         "config": {"workload": desc, "M": inp["M"], "N": inp["N"], "D": inp.get("D", 3), "Dv": inp["Dv"],
                    "baseline_hardware": "RTX 2080 Ti (reference benchmarks/README.md:14)"},
         "roofline": {
-            "bound": bound, "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
+            "bound": "mfma" if bound.startswith("mfma") else bound, "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "kernel_ms": kms, "flop_per_pair": flop_per_pair,
-            "note": "peak is the packed-FP32 vector figure; kernels here issue scalar FP32 VALU ops only "
-                    "(packed FP32 is disabled), whose ceiling is 78.6 TFLOP/s",
+            "note": note,
         },
     }
     if args.workload == "gauss_1m_dv1" and not args.no_cpu_baseline:

@@ -66,7 +66,8 @@ void keops_hip_module_destroy(void* module);
  *   tag1D2D           0: one pass over the reduced axis; 1: force the column-slab (2D) scheme
  *   dimred, dimout    accumulator and output dimensions per row
  *   block_size        upper bound for the workgroup size (0 = module default)
- *   use_chunk_mode    0 plain, 1 chunked inner reduction, 2 final chunks
+ *   use_chunk_mode    0 plain, 1 chunked inner reduction, 2 final chunks, 3 matrix-core K-nearest neighbours
+ *                     (informative: the scheme is a property of the compiled module)
  *   indsi/j/p, dims*  argument indices and dimensions of the i, j and parameter variables
  *   ranges            7 pointers: ranges_i, slices_i, redranges_j, ranges_j, slices_j, redranges_i
  *                     (int64, on the data's device) and a HOST int64[6] with their row counts;

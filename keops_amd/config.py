@@ -26,6 +26,13 @@ lds_tile_bytes = 16384     # LDS bytes of one staged column tile
 # matrix-core chunked scheme (csrc/kernels/keops_chunk_mfma.h): wavefronts (32 output rows each) per workgroup
 chunk_waves = int(os.environ.get("KEOPS_AMD_CHUNK_WAVES", 8))
 
+# matrix-core final-product scheme (csrc/kernels/keops_final_mfma.h): Sum_j f(x_i,y_j) * v_j with dim(v) large
+final_chunk_min_dim = int(os.environ.get("KEOPS_AMD_FINAL_MIN_DIM", 64))   # smallest dim(v) that selects the scheme
+final_max_blocks = int(os.environ.get("KEOPS_AMD_FINAL_NB", 8))            # 32-column accumulator tiles per wavefront
+final_waves = int(os.environ.get("KEOPS_AMD_FINAL_WAVES", 8))              # wavefronts (32 output rows each) per workgroup
+final_tile_j = int(os.environ.get("KEOPS_AMD_FINAL_TJ", 32))               # reduced rows per staged tile (even)
+final_period = int(os.environ.get("KEOPS_AMD_FINAL_PERIOD", 4096))         # block-sum period in reduced rows
+
 # matrix-core KNN kernel (csrc/kernels/keops_knn_mfma.h)
 knn_tile_j = int(os.environ.get("KEOPS_AMD_KNN_TJ", 128))          # reference rows per LDS tile (<= 256)
 knn_max_waves = int(os.environ.get("KEOPS_AMD_KNN_WAVES", 8))     # wavefronts per workgroup sharing one staged tile

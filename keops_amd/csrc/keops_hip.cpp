@@ -257,14 +257,19 @@ struct LaunchHeader {
   const int64_t* offsets;
 };
 
-int launch_raw(Module& m, const char* kernel, unsigned gx, unsigned gy, unsigned block, void* params, size_t size,
-               hipStream_t stream) {
+int launch_raw3(Module& m, const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsigned block, void* params,
+                size_t size, hipStream_t stream) {
   hipFunction_t f;
   if (int rc = m.fn(kernel, &f)) return rc;
   void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, params, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
-  if (gx == 0 || gy == 0) return 0;
-  HIP_TRY(hipModuleLaunchKernel(f, gx, gy, 1, block, 1, 1, 0, stream, nullptr, extra));
+  if (gx == 0 || gy == 0 || gz == 0) return 0;
+  HIP_TRY(hipModuleLaunchKernel(f, gx, gy, gz, block, 1, 1, 0, stream, nullptr, extra));
   return 0;
+}
+
+int launch_raw(Module& m, const char* kernel, unsigned gx, unsigned gy, unsigned block, void* params, size_t size,
+               hipStream_t stream) {
+  return launch_raw3(m, kernel, gx, gy, 1, block, params, size, stream);
 }
 
 int launch(Module& m, const char* kernel, unsigned gx, unsigned gy, const LaunchHeader& h, void* const* args,
@@ -320,6 +325,20 @@ int64_t pick_slabs(int64_t qblocks, int64_t nr, int64_t tile, int64_t cus, int64
   return std::max<int64_t>(1, std::min<int64_t>(n, 1024));
 }
 
+// Workgroups that all take the same time run in rounds over the compute units: among the slab counts
+// n0 .. nmax pick the one whose grid (blocks * n) fills its last round best (a larger count must win
+// by 1.5 % to be preferred).
+int64_t balance_slabs(int64_t blocks, int64_t n0, int64_t nmax, int64_t slots) {
+  int64_t best = n0;
+  double best_eff = 0.0;
+  for (int64_t n = n0; n <= std::max(n0, nmax); n++) {
+    const int64_t g = blocks * n, rounds = (g + slots - 1) / slots;
+    const double eff = (double)g / (double)(rounds * slots);
+    if (eff > best_eff + 0.015) { best_eff = eff; best = n; }
+  }
+  return best;
+}
+
 int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr, void* out, int tag1D2D,
                hipStream_t stream) {
   const int64_t D = m.meta_int("knn_d", 0), DP = m.meta_int("knn_dpad", 0), K = m.meta_int("knn_k", 0);
@@ -340,19 +359,8 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   // filter pass
   const int64_t f_qblocks = (nq + FQB - 1) / FQB;
   int64_t f_slabs = pick_slabs(f_qblocks, nr, TJ, m.cu_count, 2, 1);
-  {
-    // one filter workgroup fills a CU and all of them take the same time: prefer a slab count whose
-    // grid is close to a whole number of rounds over the CUs
-    const int64_t cap = std::max<int64_t>(1, nr / (16 * TJ));
-    int64_t best = f_slabs;
-    double best_eff = 0.0;
-    for (int64_t n = f_slabs; n <= std::min<int64_t>(4 * f_slabs, cap); n++) {
-      const int64_t blocks = f_qblocks * n, rounds = (blocks + m.cu_count - 1) / m.cu_count;
-      const double eff = (double)blocks / (double)(rounds * m.cu_count);
-      if (eff > best_eff + 0.015) { best_eff = eff; best = n; }
-    }
-    f_slabs = best;
-  }
+  // one filter workgroup fills a CU and all of them take the same time
+  f_slabs = balance_slabs(f_qblocks, f_slabs, std::min<int64_t>(4 * f_slabs, std::max<int64_t>(1, nr / (16 * TJ))), m.cu_count);
   int64_t f_len = ((nr + f_slabs - 1) / f_slabs + TJ - 1) / TJ * TJ;
   f_slabs = std::max<int64_t>(1, (nr + f_len - 1) / f_len);
   const int64_t nlogs = f_qblocks * f_slabs * FW;
@@ -478,6 +486,54 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
   if (int rc = launch_raw(m, "keops_chk_main", (unsigned)((nx + QB - 1) / QB), 1, (unsigned)m.block, buf.data(), psize, stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
+  return 0;
+}
+
+// ---- matrix-core final-product scheme (kernels/keops_final_mfma.h) ----------------------------------
+
+// must match struct FinParams of kernels/keops_final_mfma.h (argument pointers follow)
+struct FinHeader {
+  int64_t nx, ny;
+  void* out;
+  void* partial;
+  int64_t slab_len;
+  int32_t nslabs;
+  int32_t pad_;
+};
+
+int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, int tag1D2D, hipStream_t stream) {
+  const int64_t DV = m.meta_int("fin_dv", 0), NZ = m.meta_int("fin_nz", 1), QB = m.meta_int("fin_qb", 256), TJ = m.tile_j;
+  if (DV <= 0 || NZ <= 0 || QB <= 0 || TJ <= 0) return fail(-1, "corrupt final-product module metadata");
+  const int64_t row_blocks = (nx + QB - 1) / QB;
+  // enough workgroups for the chip: cut the reduced axis in slabs when there are few output rows
+  int64_t nslabs = 1;
+  const int64_t target = 2 * (int64_t)m.cu_count;
+  if (tag1D2D == 1 || row_blocks * NZ < target) {
+    const int64_t max_slabs = std::max<int64_t>(1, ny / (8 * TJ));
+    nslabs = std::min<int64_t>(max_slabs, (target + row_blocks * NZ - 1) / (row_blocks * NZ));
+    if (tag1D2D == 1) nslabs = std::max<int64_t>(nslabs, std::min<int64_t>(max_slabs, 2));
+    nslabs = std::max<int64_t>(1, std::min<int64_t>(nslabs, 65535));
+  }
+  // one workgroup (8 wavefronts of ~230 VGPRs) fills a CU and all of them take the same time
+  nslabs = balance_slabs(row_blocks * NZ, nslabs, std::min<int64_t>(std::max<int64_t>(nslabs, 8), std::max<int64_t>(1, ny / (8 * TJ))), m.cu_count);
+  int64_t len = std::max<int64_t>(TJ, ((ny + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ);
+  nslabs = std::max<int64_t>(1, (ny + len - 1) / len);
+  FinHeader h{};
+  h.nx = nx; h.ny = ny; h.out = out; h.slab_len = len; h.nslabs = (int32_t)nslabs;
+  if (nslabs > 1) {
+    if (int rc = m.partial.reserve((size_t)nslabs * nx * DV * 4)) return rc;
+    h.partial = m.partial.ptr;
+  }
+  std::vector<char> buf(sizeof(FinHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs));
+  std::memcpy(buf.data(), &h, sizeof(h));
+  for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
+  if (int rc = launch_raw3(m, "keops_fin_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)NZ, (unsigned)m.block, buf.data(), buf.size(), stream)) return rc;
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
+  if (nslabs > 1) {
+    const int64_t gb = (nx * DV + 255) / 256;
+    if (int rc = launch_raw(m, "keops_fin_reduce", (unsigned)gb, 1, 256, buf.data(), buf.size(), stream)) return rc;
+  }
   return 0;
 }
 
@@ -701,6 +757,9 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
     if (use_ranges) return fail(-1, "the matrix-core KNN module does not handle ranges or batch dimensions");
     const int rowarg = m.meta_int("rowarg", 0), colarg = m.meta_int("colarg", 1);
     if (int rc = launch_knn(m, rows_total, cols_total, args[rowarg], args[colarg], out, tag1D2D, stream)) return rc;
+  } else if (m.scheme == "final") {
+    if (use_ranges) return fail(-1, "the matrix-core final-product module does not handle ranges or batch dimensions");
+    if (int rc = launch_final(m, rows_total, cols_total, out, args, tag1D2D, stream)) return rc;
   } else if (m.scheme == "chunk") {
     if (use_ranges) return fail(-1, "the matrix-core chunked module does not handle ranges or batch dimensions");
     if (int rc = launch_chunk(m, rows_total, cols_total, out, args, stream)) return rc;

@@ -1,0 +1,193 @@
+// Sum reductions whose formula is a scalar kernel times a high-dimensional reduced-index variable,
+//     out_i[0..DV) = sum_j f(x_i, y_j, p) * v_j[0..DV),
+// i.e. a dense (M x N) by (N x DV) product whose left factor is generated on the fly.
+//
+// Counterpart of the reference's "final chunk" schemes
+//   keopscore/keopscore/mapreduce/gpu/GpuReduc1D_finalchunks.py:19-69,72-225
+// which evaluate f once per pair into shared memory and then stream 64-wide chunks of v_j through
+// per-thread accumulators.  Here the product runs on the matrix cores in full float32:
+//   * a wavefront owns 32 output rows; at every step lane l evaluates the scalar
+//     f(x_{l%32}, y_{j0 + l/32}) -- this *is* the A operand layout of v_mfma_f32_32x32x2_f32 (row
+//     l%32, k = l/32), so the 64 pair values of a step never leave their registers;
+//   * the B operand of the same instruction is v[j0 + l/32][32 b + l%32], one conflict-free 4-byte
+//     LDS read per lane and 32-column block b of the staged v tile;
+//   * the 32 x 32 float32 accumulator tiles (one per column block, FIN_NB of them) stay in VGPRs
+//     for the whole sweep; column blocks beyond FIN_NB are handled by further workgroups
+//     (blockIdx.z), which re-evaluate f: it is cheap next to 2*DV flop per pair;
+//   * block summation: every FIN_PERIOD reduced rows the register tiles are folded into the
+//     output rows (owned by this workgroup, plain read-modify-write) and cleared, so rounding
+//     errors do not grow with the number of reduced rows;
+//   * few output rows: the reduced axis is cut in slabs (blockIdx.y) with one partial output per
+//     slab, summed in slab order by keops_fin_reduce (deterministic).
+//
+// The plug-in defines: T (float), KEOPS_NARGS, FIN_DV, FIN_VARG, FIN_NB, FIN_WAVES, FIN_TJ,
+// FIN_PERIOD, FIN_BLOCKSUM, the KEOPS_DIM* macros and row/col/par variable tables of the scalar
+// kernel f, and KeopsFormula::eval(xi, yj, p, fout[1]).
+#pragma once
+#include "keops_common.h"
+
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float fin_f32x16;
+
+#define FIN_BLOCK (64 * FIN_WAVES)
+#define FIN_QB (32 * FIN_WAVES)                    // output rows per workgroup
+#define FIN_NBTOT ((FIN_DV + 31) / 32)             // 32-column blocks of v
+#define FIN_VS (FIN_NB * 32)                       // floats per staged v row
+#define FIN_DY (KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1)
+
+struct FinParams {
+  i64 nx, ny;
+  T* out;          // [nx][FIN_DV]
+  T* partial;      // [nslabs][nx][FIN_DV] when nslabs > 1
+  i64 slab_len;    // reduced rows per slab (multiple of FIN_TJ)
+  int nslabs;
+  int pad_;
+  const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
+};
+
+extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const FinParams P) {
+  __shared__ __attribute__((aligned(16))) T vt[FIN_TJ * FIN_VS];   // v tile, this workgroup's column blocks
+  __shared__ __attribute__((aligned(16))) T ys[FIN_TJ * FIN_DY];   // reduced-index variables of f
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const i64 row0 = (i64)blockIdx.x * FIN_QB + wave * 32;  // first output row of this wavefront
+  i64 q = row0 + col;
+  if (q >= P.nx) q = P.nx - 1;  // clamped rows compute, never store
+  const int cb0 = blockIdx.z * FIN_NB;                      // first column block of this workgroup
+  const int c0 = cb0 * 32;                                  // first column
+  const int ncols = (int)keops_min((i64)FIN_VS, (i64)FIN_DV - c0);
+
+  T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
+#pragma unroll
+  for (int v = 0; v < KEOPS_NROWVARS; v++) {
+    const T* src = P.arg[keops_row_arg[v]] + q * keops_row_dim[v];
+#pragma unroll
+    for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
+  }
+  T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+#pragma unroll
+  for (int v = 0; v < KEOPS_NPARVARS; v++) {
+    const T* src = P.arg[keops_par_arg[v]];
+#pragma unroll
+    for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
+  }
+
+  fin_f32x16 acc[FIN_NB];
+#pragma unroll
+  for (int b = 0; b < FIN_NB; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[b][r] = 0.f;
+
+  T* dst = P.nslabs > 1 ? P.partial + (i64)blockIdx.y * P.nx * FIN_DV : P.out;
+  bool first = true;
+  // folds the register tiles into the output rows of this wavefront and clears them
+  auto fold = [&]() {
+    const i64 ibase = row0 + 4 * half;
+    T* o = dst + ibase * FIN_DV + c0 + col;
+    // folds are rare: keep their address arithmetic here instead of in registers across the sweep
+    asm volatile("" : "+v"(o));
+#pragma unroll
+    for (int b = 0; b < FIN_NB; b++) {
+      const int d = c0 + 32 * b + col;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int ir = 8 * (r >> 2) + (r & 3);
+        if (ibase + ir < P.nx && d < FIN_DV) {
+          T* oo = o + (i64)ir * FIN_DV + 32 * b;
+          *oo = first ? acc[b][r] : *oo + acc[b][r];
+        }
+        acc[b][r] = 0.f;
+      }
+    }
+    first = false;
+  };
+
+  const i64 jbeg = (i64)blockIdx.y * P.slab_len;
+  const i64 jend = keops_min(P.ny, jbeg + P.slab_len);
+  const T* vsrc = P.arg[FIN_VARG];
+
+  // software pipeline: the v rows of tile t+1 travel to registers while tile t is consumed
+  constexpr int NPF = (FIN_TJ * FIN_VS + FIN_BLOCK - 1) / FIN_BLOCK;
+  T pf[NPF];
+  auto prefetch = [&](i64 j0) {
+    const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * FIN_BLOCK;
+      const int row = e / FIN_VS, c = e - row * FIN_VS;
+      pf[u] = (row < n && c < ncols) ? vsrc[(j0 + row) * FIN_DV + c0 + c] : (T)0;  // zero rows/columns past the end
+    }
+  };
+  if (jbeg < jend) prefetch(jbeg);
+  int since_fold = 0;
+  for (i64 j0 = jbeg; j0 < jend; j0 += FIN_TJ) {
+    const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
+    __syncthreads();  // the previous tile has been consumed by every wavefront
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * FIN_BLOCK;
+      if (e < FIN_TJ * FIN_VS) vt[e] = pf[u];
+    }
+#pragma unroll
+    for (int v = 0; v < KEOPS_NCOLVARS; v++) {
+      const int dim = keops_col_dim[v];
+      const T* src = P.arg[keops_col_arg[v]] + j0 * dim;
+      for (int e = tid; e < n * dim; e += FIN_BLOCK) {
+        const int row = e / dim, c = e - row * dim;
+        ys[row * FIN_DY + keops_col_off[v] + c] = src[e];
+      }
+    }
+    __syncthreads();
+    if (j0 + FIN_TJ < jend) prefetch(j0 + FIN_TJ);
+
+    // operands of step s+1 (pair value and v entries) are fetched while the MFMAs of step s execute
+    auto operands = [&](int s, float& fv, float (&bv)[FIN_NB]) {
+      const int jr = 2 * s + half;  // reduced row of this lane's pair
+      const T* vrow = vt + jr * FIN_VS + col;
+#pragma unroll
+      for (int b = 0; b < FIN_NB; b++) bv[b] = vrow[32 * b];
+      T yj[FIN_DY];
+      constexpr int VEC = 4;
+      typedef T vecT __attribute__((ext_vector_type(VEC)));
+#pragma unroll
+      for (int c4 = 0; c4 < KEOPS_DIMY_PAD / VEC; c4++) {
+        const vecT w = *reinterpret_cast<const vecT*>(ys + jr * FIN_DY + c4 * VEC);
+#pragma unroll
+        for (int c = 0; c < VEC; c++) yj[c4 * VEC + c] = w[c];
+      }
+      T fout[1];
+      KeopsFormula::eval(xi, yj, p, fout);
+      fv = jr < n ? fout[0] : 0.f;  // select, never multiply: rows past the end hold garbage
+    };
+    float fcur, bcur[FIN_NB];
+    operands(0, fcur, bcur);
+#pragma unroll 2
+    for (int s = 0; s < FIN_TJ / 2; s++) {
+      float fnext = 0.f, bnext[FIN_NB];
+      if (s + 1 < FIN_TJ / 2) operands(s + 1, fnext, bnext);
+#pragma unroll
+      for (int b = 0; b < FIN_NB; b++) acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fcur, bcur[b], acc[b], 0, 0, 0);
+      fcur = fnext;
+#pragma unroll
+      for (int b = 0; b < FIN_NB; b++) bcur[b] = bnext[b];
+    }
+#if FIN_BLOCKSUM
+    since_fold += FIN_TJ;
+    if (since_fold >= FIN_PERIOD) {
+      fold();
+      since_fold = 0;
+    }
+#endif
+  }
+  fold();
+}
+
+// sums the per-slab partial outputs in slab order
+extern "C" __global__ void __launch_bounds__(256) keops_fin_reduce(const FinParams P) {
+  const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
+  const i64 total = P.nx * FIN_DV;
+  if (e >= total) return;
+  T s = P.partial[e];
+  for (int k = 1; k < P.nslabs; k++) s += P.partial[(i64)k * total + e];
+  P.out[e] = s;
+}

@@ -257,6 +257,72 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
     return "\n".join(src) + "\n", meta
 
 
+def match_final(red, dtype, dtypeacc, sum_scheme, map_reduce_id):
+    """(scalar kernel f, variable v) when ``red`` is Sum_Reduction(f * v) with f of dimension 1 and v a
+    plain reduced-index variable of dimension >= config.final_chunk_min_dim, in float32 on the dense
+    scheme (the shape GpuReduc1D_finalchunks.py:100-106 expects); None otherwise."""
+    from .formulas import ops as O
+    from .formulas.reductions import KIND_SUM
+
+    if red.kind != KIND_SUM or dtype != "float" or dtypeacc != "float" or "_ranges" in map_reduce_id:
+        return None
+    if sum_scheme not in ("block_sum", "direct_sum"):
+        return None
+    F = red.formula
+    if F.name != "Mult" or len(F.children) != 2:
+        return None
+    for f, v in (F.children, F.children[::-1]):
+        if f.dim == 1 and isinstance(v, O.Var) and v.cat == 1 - red.tagI and v.dim == F.dim and v.dim >= config.final_chunk_min_dim:
+            return f, v
+    return None
+
+
+def generate_final_plugin(red, match, sum_scheme, nargs):
+    """Module source for the matrix-core final-product scheme (kernels/keops_final_mfma.h)."""
+    f, vvar = match
+
+    class _Inner:  # what VarLayout needs: the scalar kernel with the reduction's orientation
+        formula, tagI = f, red.tagI
+
+    layout = VarLayout(_Inner)
+    L = Lir(row_cat=red.tagI, fast_math=True, dtype="float")
+    outs = lower(f, L)
+    lines, exprs = L.emit(outs, layout.names, indent="    ")
+    dimy_pad = 0 if layout.dimy == 0 else -(-layout.dimy // 4) * 4
+    nbtot = -(-vvar.dim // 32)
+    nb = min(nbtot, config.final_max_blocks)
+    # balance the column blocks over the workgroups that share a row block
+    nz = -(-nbtot // nb)
+    nb = -(-nbtot // nz)
+    waves, tj = config.final_waves, config.final_tile_j
+    ra, rd, ro = VarLayout.table(layout.rowvars)
+    ca, cd, co = VarLayout.table(layout.colvars)
+    pa, pd, po = VarLayout.table(layout.parvars)
+    meta = dict(scheme="final", block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
+                sizeof_acc=4, nrowvars=len(layout.rowvars), ncolvars=len(layout.colvars) + (0 if vvar in layout.colvars else 1),
+                nparvars=len(layout.parvars), fin_dv=vvar.dim, fin_nb=nb, fin_nz=nz, fin_qb=32 * waves, nops=L.count_ops(outs))
+    src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
+           "typedef float T;\ntypedef float TACC;", '#include "keops_common.h"']
+    defs = dict(
+        KEOPS_NARGS=nargs, FIN_DV=vvar.dim, FIN_VARG=vvar.ind, FIN_NB=nb, FIN_WAVES=waves, FIN_TJ=tj,
+        FIN_PERIOD=config.final_period, FIN_BLOCKSUM=int(sum_scheme == "block_sum"),
+        KEOPS_DIMX=layout.dimx, KEOPS_DIMY=layout.dimy, KEOPS_DIMY_PAD=dimy_pad, KEOPS_DIMP=layout.dimp,
+        KEOPS_NROWVARS=len(layout.rowvars), KEOPS_NCOLVARS=len(layout.colvars), KEOPS_NPARVARS=len(layout.parvars),
+    )
+    src += [f"#define {k} {v}" for k, v in defs.items()]
+    for name, vals in (("row_arg", ra), ("row_dim", rd), ("row_off", ro), ("col_arg", ca), ("col_dim", cd),
+                       ("col_off", co), ("par_arg", pa), ("par_dim", pd), ("par_off", po)):
+        src.append(f"static __device__ constexpr int keops_{name}[] = {_c_list(vals)};")
+    dx, dy, dp = max(1, layout.dimx), max(1, dimy_pad), max(1, layout.dimp)
+    src.append("struct KeopsFormula {")
+    src.append(f"  static __device__ __forceinline__ void eval(const T (&xi)[{dx}], const T (&yj)[{dy}], "
+               f"const T (&p)[{dp}], T (&fout)[1]) {{")
+    src += lines + [f"    fout[{k}] = {e};" for k, e in enumerate(exprs)]
+    src.append("  }\n};")
+    src.append('#include "keops_final_mfma.h"')
+    return "\n".join(src) + "\n", meta
+
+
 def get_keops_dll(
     map_reduce_id, red_formula_string, enable_chunks, enable_finalchunks, mul_var_highdim, aliases, nargs, dtype,
     dtypeacc, sum_scheme_string, tagHostDevice, tagCPUGPU, tag1D2D, use_half, use_fast_math, device_id, nx=None,
@@ -276,7 +342,7 @@ def get_keops_dll(
         # only the bucket matters for the cache key
         rows_hint = nx if nx < 8 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
-           use_fast_math, _rows_bucket(rows_hint), bool(enable_chunks), binder.templates_digest())
+           use_fast_math, _rows_bucket(rows_hint), bool(enable_chunks), bool(enable_finalchunks), binder.templates_digest())
     with _lock:
         hit = _cache.get(key)
     if hit is not None:
@@ -289,9 +355,15 @@ def get_keops_dll(
     else:
         knn = match_knn_sqdist(red, dtype, map_reduce_id) if enable_chunks else None
         chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
+        fin = None
+        if enable_finalchunks and knn is None and chk is None:
+            fin = match_final(red, dtype, dtypeacc, sum_scheme_string, map_reduce_id)
         if knn is not None:
             source, meta = generate_knn_plugin(red, knn[0], knn[1], nargs)
             use_chunk_mode = 3  # matrix-core filter scheme (no counterpart among the reference's chunk modes)
+        elif fin is not None:
+            source, meta = generate_final_plugin(red, fin, sum_scheme_string, nargs)
+            use_chunk_mode = 2  # as the reference's final-chunk mode (get_keops_dll.py:101-108)
         elif chk is not None:
             source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs)
             use_chunk_mode = 1

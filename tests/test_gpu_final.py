@@ -1,0 +1,120 @@
+"""GPU parity of the matrix-core final-product scheme (keops_final_mfma.h): Sum_j f(x_i,y_j) * v_j with
+a high-dimensional v.  The scheme is only a schedule, so the result must equal the plain reduction, cf.
+the reference's pykeops/test/test_finalchunks.py (Gaussian kernel times a 500-dimensional variable,
+compared with the dense torch formula)."""
+import numpy as np
+import pytest
+import torch
+
+from common import assert_sum_parity, to_dev
+from oracle.cpu_oracle import cpu_reduc
+
+pytestmark = pytest.mark.gpu
+
+FORMULA = "Exp(-g*SqDist(x,y))*b"
+
+
+def _inputs(M, N, Dv, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((M, 3)).astype(np.float32)
+    y = rng.standard_normal((N, 3)).astype(np.float32)
+    b = rng.standard_normal((N, Dv)).astype(np.float32)
+    g = np.array([0.75], np.float32)
+    return x, y, b, g
+
+
+def _scheme_used(name):
+    from keops_amd import keops_io
+
+    return any(m.meta("scheme") == name for m in keops_io._modules.values())
+
+
+def _aliases(Dv):
+    return ["x=Vi(3)", "y=Vj(3)", f"b=Vj({Dv})", "g=Pm(1)"]
+
+
+@pytest.mark.parametrize("M,N,Dv,scheme", [
+    (1000, 3000, 256, "block_sum"),     # few output rows: slabs over the reduced axis + ordered sum
+    (777, 1001, 200, "block_sum"),      # ragged last column block, ragged last tile
+    (333, 2500, 300, "direct_sum"),     # more column blocks than one wavefront keeps: two workgroups per row block
+    (70, 50, 64, "block_sum"),          # smallest dimension that selects the scheme, less than one tile pair
+    (256, 20000, 96, "block_sum"),      # several block-sum periods
+])
+def test_gaussian_times_highdim_vs_oracle(M, N, Dv, scheme):
+    from keops_amd.torch import Genred
+
+    x, y, b, g = _inputs(M, N, Dv, 11)
+    conv = Genred(FORMULA, _aliases(Dv), reduction_op="Sum", axis=1, sum_scheme=scheme)
+    got = conv(*to_dev(x, y, b, g)).cpu().numpy()
+    assert _scheme_used("final")
+    assert got.shape == (M, Dv)
+    ref = cpu_reduc("gauss", [x, y, b, g], M, N, Dv)
+    scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, Dv)
+    assert_sum_parity(got, ref, scale)
+    # independent pin: float64 closed form
+    x64, y64, b64 = (torch.from_numpy(t).double() for t in (x, y, b))
+    K = torch.exp(-0.75 * torch.cdist(x64, y64) ** 2)
+    assert_sum_parity(got, (K @ b64).numpy(), (K @ b64.abs()).numpy())
+
+
+def test_large_rows_subset_and_exact_linearity():
+    # enough rows for one slab; rows are independent, so a random subset is compared with the oracle
+    from keops_amd.torch import Genred
+
+    M, N, Dv = 60_000, 4_000, 128
+    x, y, b, g = _inputs(M, N, Dv, 12)
+    conv = Genred(FORMULA, _aliases(Dv), reduction_op="Sum", axis=1)
+    xd, yd, bd, gd = to_dev(x, y, b, g)
+    got = conv(xd, yd, bd, gd)
+    rows = np.sort(np.random.default_rng(3).choice(M, 256, replace=False)).astype(np.int64)
+    ref = cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
+    scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, Dv, rows=rows)
+    assert_sum_parity(got[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
+    assert torch.equal(conv(xd, yd, 2 * bd, gd), 2 * got)  # scaling v by a power of two is exact
+    assert torch.equal(conv(xd, yd, bd, gd), got)          # and the result is reproducible bit for bit
+
+
+def test_axis0_gpu2d_and_gradient():
+    from keops_amd.torch import Genred
+
+    M, N, Dv = 500, 640, 160
+    rng = np.random.default_rng(13)
+    x = rng.standard_normal((M, 3)).astype(np.float32)
+    y = rng.standard_normal((N, 3)).astype(np.float32)
+    a = rng.standard_normal((M, Dv)).astype(np.float32)
+    g = np.array([0.5], np.float32)
+    x64, y64, a64 = (torch.from_numpy(t).double() for t in (x, y, a))
+    K = torch.exp(-0.5 * torch.cdist(x64, y64) ** 2)
+    # reduction over i: the high-dimensional variable is indexed by i, the output by j
+    conv = Genred("a*Exp(-g*SqDist(x,y))", ["x=Vi(3)", "y=Vj(3)", f"a=Vi({Dv})", "g=Pm(1)"], reduction_op="Sum", axis=0)
+    xd, yd, ad, gd = to_dev(x, y, a, g)
+    got = conv(xd, yd, ad, gd, backend="GPU_2D").cpu().numpy()
+    assert_sum_parity(got, (K.T @ a64).numpy(), (K.T @ a64.abs()).numpy())
+    # gradient with respect to the high-dimensional variable is again a final product (over the other index)
+    b = rng.standard_normal((N, Dv)).astype(np.float32)
+    bd = torch.from_numpy(b).cuda().requires_grad_(True)
+    conv1 = Genred(FORMULA, _aliases(Dv), reduction_op="Sum", axis=1)
+    out = conv1(xd, yd, bd, gd)
+    e = torch.from_numpy(rng.standard_normal((M, Dv)).astype(np.float32)).cuda()
+    (gb,) = torch.autograd.grad(out, [bd], e)
+    e64 = e.cpu().double()
+    assert_sum_parity(gb.cpu().numpy(), (K.T @ e64).numpy(), (K.T @ e64.abs()).numpy())
+
+
+def test_lazytensor_front_end_and_fallbacks():
+    from keops_amd.torch import Genred, LazyTensor
+
+    M, N, Dv = 300, 400, 192
+    x, y, b, g = _inputs(M, N, Dv, 14)
+    xd, yd, bd, gd = to_dev(x, y, b, g)
+    x_i, y_j, b_j = LazyTensor(xd[:, None, :]), LazyTensor(yd[None, :, :]), LazyTensor(bd[None, :, :])
+    got = ((-0.75 * ((x_i - y_j) ** 2).sum(-1)).exp() * b_j).sum(dim=1)
+    x64, y64, b64 = (torch.from_numpy(t).double() for t in (x, y, b))
+    K = torch.exp(-0.75 * torch.cdist(x64, y64) ** 2)
+    assert_sum_parity(got.cpu().numpy(), (K @ b64).numpy(), (K @ b64.abs()).numpy())
+    # float64 data and Kahan summation are served by the generic kernel: same function
+    conv64 = Genred(FORMULA, _aliases(Dv), reduction_op="Sum", axis=1)
+    got64 = conv64(xd.double(), yd.double(), bd.double(), gd.double()).cpu().numpy()
+    assert np.max(np.abs(got64 - (torch.exp(-0.75 * torch.cdist(xd.double().cpu(), yd.double().cpu()) ** 2) @ b64).numpy())) < 1e-10
+    kahan = Genred(FORMULA, _aliases(Dv), reduction_op="Sum", axis=1, sum_scheme="kahan_scheme")(xd, yd, bd, gd)
+    assert_sum_parity(kahan.cpu().numpy(), (K @ b64).numpy(), (K @ b64.abs()).numpy())
