@@ -34,6 +34,15 @@ PUBLISHED_PAIRS_PER_S = 1e12 / 1.39
 MEASURED_TRAFFIC_BYTES = {
     # profiles/keops_conv_dense__gauss_1m_dv1.md: FETCH_SIZE 230808 KiB x 2.0 (copy calibration) + WRITE_SIZE 3906.25 KiB
     "gauss_1m_dv1": int((230808 * 2.0 + 3906.25) * 1024),
+    # profiles/keops_knn_filter__knn_d64.md: dominant kernel keops_knn_filter
+    "knn_d64": int((822401 * 2.0 + 163406) * 1024),
+    # profiles/keops_chk_main__laplace_d256.md
+    "laplace_d256": int((3534300 * 2.0 + 29700) * 1024),
+    # profiles/keops_fin_main__gauss_dv256.md
+    "gauss_dv256": int((8043160 * 2.0 + 10795000) * 1024),
+    # profiles/keops_conv_ranges__sparse_100x10k.md, keops_conv_ranges__lse_b16.md
+    "sparse_100x10k": int((85442 * 2.0 + 3906.25) * 1024),
+    "lse_b16": int((55633 * 2.0 + 6250) * 1024),
 }
 
 WORKLOADS = {
