@@ -36,8 +36,8 @@ MEASURED_TRAFFIC_BYTES = {
     "gauss_1m_dv1": int((230808 * 2.0 + 3906.25) * 1024),
     # profiles/keops_knn_filter__knn_d64.md: dominant kernel keops_knn_filter
     "knn_d64": int((822401 * 2.0 + 163406) * 1024),
-    # profiles/keops_chk_main__laplace_d256.md
-    "laplace_d256": int((3534300 * 2.0 + 29700) * 1024),
+    # profiles/keops_chk_final__laplace_d256.md
+    "laplace_d256": int((4292480 * 2.0 + 650811) * 1024),
     # profiles/keops_fin_main__gauss_dv256.md
     "gauss_dv256": int((8043160 * 2.0 + 10795000) * 1024),
     # profiles/keops_conv_ranges__sparse_100x10k.md, keops_conv_ranges__lse_b16.md

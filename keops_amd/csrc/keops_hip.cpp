@@ -450,9 +450,13 @@ struct ChkHeader {
   void* colsum;
   void* colpart;
   void* out;
+  void* partial;
+  int64_t slab_len;
+  int32_t nslabs;
+  int32_t pad_;
 };
 
-int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, hipStream_t stream) {
+int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, int tag1D2D, hipStream_t stream) {
   const int64_t D = m.meta_int("chk_d", 0), DP = m.meta_int("chk_dpad", 0), QB = m.meta_int("chk_qb", 128);
   const int mode = m.meta_int("chk_mode", 0);
   if (D <= 0 || DP <= 0) return fail(-1, "corrupt chunk module metadata");
@@ -462,12 +466,30 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
   const size_t o_xs = take((size_t)nx * DP * 4), o_ys = take((size_t)ny * DP * 4);
   const size_t o_xn = take((size_t)nx * 4), o_yn = take((size_t)ny * 4);
+  // final-product variant: slabs over the reduced axis fill the chip and round the grid to whole
+  // rounds of workgroups (one 8-wavefront workgroup per CU, all taking the same time)
+  const bool final = m.meta_int("chk_final", 0) != 0;
+  const int64_t row_blocks = (nx + QB - 1) / QB, TJ = m.tile_j;
+  int64_t nslabs = 1, slab_len = std::max<int64_t>(TJ, (ny + TJ - 1) / TJ * TJ);
+  if (final) {
+    const int64_t cap = std::max<int64_t>(1, ny / (8 * TJ));
+    const int64_t target = 2 * (int64_t)m.cu_count;
+    if (tag1D2D == 1 || row_blocks < target) {
+      nslabs = std::min<int64_t>(cap, (target + row_blocks - 1) / row_blocks);
+      if (tag1D2D == 1) nslabs = std::max<int64_t>(nslabs, std::min<int64_t>(cap, 2));
+      nslabs = std::max<int64_t>(1, std::min<int64_t>(nslabs, 65535));
+    }
+    nslabs = balance_slabs(row_blocks, nslabs, std::min<int64_t>(std::max<int64_t>(nslabs, 8), cap), m.cu_count);
+    slab_len = std::max<int64_t>(TJ, ((ny + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ);
+    nslabs = std::max<int64_t>(1, (ny + slab_len - 1) / slab_len);
+  }
+  const size_t o_part = take(final && nslabs > 1 ? (size_t)nslabs * nx * m.dimout * 4 : 0);
   if (int rc = m.partial.reserve(off)) return rc;
   char* ws = (char*)m.partial.ptr;
   std::vector<char> buf(sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 8);
   ChkHeader h{};
   h.nx = nx; h.ny = ny; h.xs = ws + o_xs; h.ys = ws + o_ys; h.xn = ws + o_xn; h.yn = ws + o_yn; h.colsum = ws + o_colsum;
-  h.colpart = ws + o_colpart; h.out = out;
+  h.colpart = ws + o_colpart; h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs;
   std::memcpy(buf.data(), &h, sizeof(h));
   for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
   const size_t psize = sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs);
@@ -484,8 +506,16 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   sz = with_which(1);
   if (int rc = launch_raw(m, "keops_chk_prep", (unsigned)((ny * lpr + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
-  if (int rc = launch_raw(m, "keops_chk_main", (unsigned)((nx + QB - 1) / QB), 1, (unsigned)m.block, buf.data(), psize, stream)) return rc;
+  if (final) {
+    if (int rc = launch_raw(m, "keops_chk_final", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)m.block, buf.data(), psize, stream)) return rc;
+  } else {
+    if (int rc = launch_raw(m, "keops_chk_main", (unsigned)row_blocks, 1, (unsigned)m.block, buf.data(), psize, stream)) return rc;
+  }
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
+  if (final && nslabs > 1) {
+    const int64_t gb = (nx * m.dimout + 255) / 256;
+    if (int rc = launch_raw(m, "keops_chk_reduce", (unsigned)gb, 1, 256, buf.data(), psize, stream)) return rc;
+  }
   return 0;
 }
 
@@ -762,7 +792,7 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
     if (int rc = launch_final(m, rows_total, cols_total, out, args, tag1D2D, stream)) return rc;
   } else if (m.scheme == "chunk") {
     if (use_ranges) return fail(-1, "the matrix-core chunked module does not handle ranges or batch dimensions");
-    if (int rc = launch_chunk(m, rows_total, cols_total, out, args, stream)) return rc;
+    if (int rc = launch_chunk(m, rows_total, cols_total, out, args, tag1D2D, stream)) return rc;
   } else if (!use_ranges) {
     // ---- dense scheme, optionally cut in column slabs ----
     const int64_t row_blocks = (rows_total + rows_per_block - 1) / rows_per_block;

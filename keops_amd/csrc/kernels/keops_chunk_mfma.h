@@ -26,9 +26,21 @@
 // folds them in its private accumulator; the two lanes of a row merge their accumulators at the end
 // (ReducePair), so sums are deterministic.
 //
+// When the post-chunk formula of a Sum reduction is itself "scalar times reduced-index variable",
+//     F'(s, ...) = g(s, ...) * v_j,
+// (CHK_FINAL, kernel keops_chk_final) the weighted accumulation also runs on the matrix cores, in
+// float32: register v of the s tile, once mapped through g, is the A operand of
+// v_mfma_f32_32x32x2_f32 (output row l % 32, k = l / 32 <-> reduced rows r_v and r_v + 4) and
+// v_j[r][32 b + l % 32] its B operand, one 4-byte LDS read per lane instead of dim(v) wave-wide
+// broadcast reads.  The 32 x 32 float32 output tiles stay in registers, are folded into the output
+// rows every CHK_PERIOD reduced rows (block summation) and the reduced axis can be cut in slabs
+// summed in order by keops_chk_reduce.
+//
 // The plug-in defines: T (float), TACC, KEOPS_NARGS, CHK_D, CHK_DPAD, CHK_MODE, CHK_XARG, CHK_YARG,
 // CHK_WAVES, the KEOPS_DIM* / KEOPS_RED_* / KEOPS_SUM_SCHEME macros, the row/col/par variable
-// tables of the *other* variables, and KeopsFormula::eval(xi, yj, p, s, fout).
+// tables of the *other* variables, and KeopsFormula::eval(xi, yj, p, s, fout); with CHK_FINAL also
+// CHK_FV_ARG, CHK_FV_DIM (argument index and dimension of v), CHK_FNB (32-column blocks),
+// CHK_PERIOD, CHK_BLOCKSUM, and eval returns the scalar g in fout[0].
 #pragma once
 #include "keops_reductions.h"
 
@@ -54,6 +66,10 @@ struct ChkParams {
   float* colsum;        // [CHK_DPAD]
   float* colpart;       // [nparts][CHK_DPAD] partial column sums
   T* out;               // [nx][KEOPS_DIMOUT]
+  T* partial;           // keops_chk_final: [nslabs][nx][KEOPS_DIMOUT] when nslabs > 1
+  i64 slab_len;         // keops_chk_final: reduced rows per slab (multiple of CHK_TJ)
+  int nslabs;
+  int pad_;
   const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
 };
 
@@ -156,6 +172,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
 
 // ---- main kernel --------------------------------------------------------------------------------
 
+#if !(defined(CHK_FINAL) && CHK_FINAL)
 extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const ChkParams P) {
   __shared__ __attribute__((aligned(16))) unsigned char as[CHK_TJ * CHK_STRIDE];  // A tile (hi|lo)
   __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
@@ -300,3 +317,192 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
     if (valid) acc.finalize(P.out + q * KEOPS_DIMOUT);
   }
 }
+#endif
+
+// ---- variant with the final product on the matrix cores -------------------------------------------
+
+#if defined(CHK_FINAL) && CHK_FINAL
+#define CHK_FVS (CHK_FNB * 32)  // floats per staged v row (columns past CHK_FV_DIM are zero)
+
+extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const ChkParams P) {
+  __shared__ __attribute__((aligned(16))) unsigned char as[CHK_TJ * CHK_STRIDE];  // A tile (hi|lo)
+  __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
+  __shared__ __attribute__((aligned(16))) T yo_s[CHK_TJ * CHK_DY];                // other column variables of g
+  __shared__ __attribute__((aligned(16))) T bt[CHK_TJ * CHK_FVS];                 // v tile
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const i64 row0 = (i64)blockIdx.x * CHK_QB + wave * 32;
+  i64 q = row0 + col;
+  if (q >= P.nx) q = P.nx - 1;  // clamped rows compute, never store
+
+  chk_bf16x8 bh[CHK_KB], bl[CHK_KB];
+#pragma unroll
+  for (int kb = 0; kb < CHK_KB; kb++) {
+    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + kb * 16 + 8 * half);
+    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+  }
+  const float xnq = CHK_MODE == 0 ? P.xn[q] : 0.f;
+  T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
+#pragma unroll
+  for (int v = 0; v < KEOPS_NROWVARS; v++) {
+    const T* src = P.arg[keops_row_arg[v]] + q * keops_row_dim[v];
+#pragma unroll
+    for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
+  }
+  T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+#pragma unroll
+  for (int v = 0; v < KEOPS_NPARVARS; v++) {
+    const T* src = P.arg[keops_par_arg[v]];
+#pragma unroll
+    for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
+  }
+
+  chk_f32x16 acc[CHK_FNB];
+#pragma unroll
+  for (int b = 0; b < CHK_FNB; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[b][r] = 0.f;
+
+  T* dst = P.nslabs > 1 ? P.partial + (i64)blockIdx.y * P.nx * CHK_FV_DIM : P.out;
+  bool first = true;
+  // folds the register tiles into the output rows of this wavefront and clears them
+  auto fold = [&]() {
+    const i64 ibase = row0 + 4 * half;
+    T* o = dst + ibase * CHK_FV_DIM + col;
+    asm volatile("" : "+v"(o));  // folds are rare: keep their address arithmetic out of the sweep's registers
+#pragma unroll
+    for (int b = 0; b < CHK_FNB; b++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int ir = 8 * (r >> 2) + (r & 3);
+        if (ibase + ir < P.nx && 32 * b + col < CHK_FV_DIM) {
+          T* oo = o + (i64)ir * CHK_FV_DIM + 32 * b;
+          *oo = first ? acc[b][r] : *oo + acc[b][r];
+        }
+        acc[b][r] = 0.f;
+      }
+    }
+    first = false;
+  };
+
+  const i64 jbeg = (i64)blockIdx.y * P.slab_len;
+  const i64 jend = keops_min(P.ny, jbeg + P.slab_len);
+  const T* vsrc = P.arg[CHK_FV_ARG];
+
+  constexpr int CH = CHK_ROWBYTES / 16;
+  constexpr int NPF = (CHK_TJ * CH + CHK_BLOCK - 1) / CHK_BLOCK;
+  constexpr int NPV = (CHK_TJ * CHK_FVS + CHK_BLOCK - 1) / CHK_BLOCK;
+  uint4 pf[NPF];
+  T pfv[NPV];
+  float pfn = 0.f;
+  auto prefetch = [&](i64 j0) {
+    const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
+    const uint4* src = reinterpret_cast<const uint4*>(P.ys + j0 * 2 * CHK_DPAD);
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * CHK_BLOCK;
+      pf[u] = (e < n * CH) ? src[e] : make_uint4(0u, 0u, 0u, 0u);
+    }
+    if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[j0 + tid] : 0.f;
+    // v tile, zero past the last row / column (the matrix product must not see stale values)
+#pragma unroll
+    for (int u = 0; u < NPV; u++) {
+      const int e = tid + u * CHK_BLOCK;
+      const int row = e / CHK_FVS, c = e - row * CHK_FVS;
+      pfv[u] = (row < n && c < CHK_FV_DIM) ? vsrc[(j0 + row) * CHK_FV_DIM + c] : (T)0;
+    }
+  };
+  if (jbeg < jend) prefetch(jbeg);
+  int since_fold = 0;
+  for (i64 j0 = jbeg; j0 < jend; j0 += CHK_TJ) {
+    const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * CHK_BLOCK;
+      if (e < CHK_TJ * CH) {
+        const int row = e / CH, c = e - row * CH;
+        *reinterpret_cast<uint4*>(as + row * CHK_STRIDE + c * 16) = pf[u];
+      }
+    }
+    if (CHK_MODE == 0 && tid < CHK_TJ) yn_s[tid] = pfn;
+#pragma unroll
+    for (int v = 0; v < KEOPS_NCOLVARS; v++) {
+      const int dim = keops_col_dim[v];
+      const T* src = P.arg[keops_col_arg[v]] + j0 * dim;
+      for (int e = tid; e < n * dim; e += CHK_BLOCK) {
+        const int row = e / dim, c = e - row * dim;
+        yo_s[row * CHK_DY + keops_col_off[v] + c] = src[e];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NPV; u++) {
+      const int e = tid + u * CHK_BLOCK;
+      if (e < CHK_TJ * CHK_FVS) bt[e] = pfv[u];
+    }
+    __syncthreads();
+    if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ);
+
+    chk_f32x16 s;
+    if (CHK_MODE == 0) {
+      chk_f32x4 kk[4];
+#pragma unroll
+      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const chk_f32x4*>(yn_s + 8 * b + 4 * half);
+#pragma unroll
+      for (int v = 0; v < 16; v++) s[v] = kk[v >> 2][v & 3];
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; v++) s[v] = 0.f;
+    }
+    const unsigned char* arow = as + col * CHK_STRIDE + 16 * half;
+#pragma unroll
+    for (int kb = 0; kb < CHK_KB; kb++) {
+      const chk_bf16x8 ah = *reinterpret_cast<const chk_bf16x8*>(arow + kb * 32);
+      const chk_bf16x8 al = *reinterpret_cast<const chk_bf16x8*>(arow + CHK_DPAD * 2 + kb * 32);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int r = 8 * (v >> 2) + 4 * half + (v & 3);
+      T sv = s[v];
+      if (CHK_MODE == 0) sv = __builtin_fmaxf(sv + xnq, 0.f);
+      T yj[CHK_DY];
+      constexpr int VEC = 16 / sizeof(T);
+      typedef T vecT __attribute__((ext_vector_type(VEC)));
+#pragma unroll
+      for (int c4 = 0; c4 < KEOPS_DIMY_PAD / VEC; c4++) {
+        const vecT w = *reinterpret_cast<const vecT*>(yo_s + r * CHK_DY + c4 * VEC);
+#pragma unroll
+        for (int c = 0; c < VEC; c++) yj[c4 * VEC + c] = w[c];
+      }
+      T fout[1];
+      KeopsFormula::eval(xi, yj, p, sv, fout);
+      const float g = r < n ? fout[0] : 0.f;  // select, never multiply: rows past the end hold garbage
+#pragma unroll
+      for (int b = 0; b < CHK_FNB; b++)
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(g, bt[r * CHK_FVS + 32 * b + col], acc[b], 0, 0, 0);
+    }
+#if CHK_BLOCKSUM
+    since_fold += CHK_TJ;
+    if (since_fold >= CHK_PERIOD) {
+      fold();
+      since_fold = 0;
+    }
+#endif
+  }
+  fold();
+}
+
+// sums the per-slab partial outputs in slab order
+extern "C" __global__ void __launch_bounds__(256) keops_chk_reduce(const ChkParams P) {
+  const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
+  const i64 total = P.nx * CHK_FV_DIM;
+  if (e >= total) return;
+  T s = P.partial[e];
+  for (int k = 1; k < P.nslabs; k++) s += P.partial[(i64)k * total + e];
+  P.out[e] = s;
+}
+#endif

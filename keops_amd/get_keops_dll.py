@@ -211,9 +211,22 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
     from .formulas import ops as O
     from .formulas.reductions import Reduction
 
+    from .formulas.reductions import KIND_SUM
+
     mode, node, xvar, yvar = match
     svar = O.Var(1 << 30, 1, 3)
     post = red.formula.replace(node, svar)
+    # post-chunk formula g(s, ...) * v_j of a float32 Sum: the product with v also runs on the matrix cores
+    final = None
+    if (red.kind == KIND_SUM and dtypeacc == "float" and sum_scheme in ("block_sum", "direct_sum")
+            and post.name == "Mult" and len(post.children) == 2):
+        for g, v in (post.children, post.children[::-1]):
+            if g.dim == 1 and isinstance(v, O.Var) and v.cat == 1 - red.tagI and v.dim == post.dim and v.dim <= 64:
+                final = (g, v)
+                break
+    full_post = post
+    if final is not None:
+        post = final[0]
 
     class _Post:  # what VarLayout needs: the post-chunk formula with the reduction's orientation
         formula, tagI = post, red.tagI
@@ -230,10 +243,11 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
     ra, rd, ro = VarLayout.table(layout.rowvars)
     ca, cd, co = VarLayout.table(layout.colvars)
     pa, pd, po = VarLayout.table(layout.parvars)
+    ncol_extra = 1 + (1 if final is not None and final[1] not in layout.colvars else 0)
     meta = dict(scheme="chunk", block=64 * waves, rows=1, tile_j=32, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
                 sizeof_acc=8 if dtypeacc == "double" else 4, nrowvars=len(layout.rowvars) + 1,
-                ncolvars=len(layout.colvars) + 1, nparvars=len(layout.parvars), chk_d=D, chk_dpad=dpad, chk_mode=mode,
-                chk_qb=32 * waves, nops=L.count_ops(outs))
+                ncolvars=len(layout.colvars) + ncol_extra, nparvars=len(layout.parvars), chk_d=D, chk_dpad=dpad,
+                chk_mode=mode, chk_qb=32 * waves, chk_final=int(final is not None), nops=L.count_ops(outs))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
            f"typedef float T;\ntypedef {dtypeacc} TACC;", '#include "keops_common.h"']
     defs = dict(
@@ -243,6 +257,10 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
         KEOPS_RED_KEEP=red.keep, KEOPS_RED_K=red.K, KEOPS_SUM_SCHEME=SUM_SCHEMES[sum_scheme],
         KEOPS_NROWVARS=len(layout.rowvars), KEOPS_NCOLVARS=len(layout.colvars), KEOPS_NPARVARS=len(layout.parvars),
     )
+    if final is not None:
+        defs.update(KEOPS_DIMFOUT=full_post.dim, CHK_FINAL=1, CHK_FV_ARG=final[1].ind, CHK_FV_DIM=final[1].dim,
+                    CHK_FNB=-(-final[1].dim // 32), CHK_PERIOD=config.final_period,
+                    CHK_BLOCKSUM=int(sum_scheme == "block_sum"))
     src += [f"#define {k} {v}" for k, v in defs.items()]
     for name, vals in (("row_arg", ra), ("row_dim", rd), ("row_off", ro), ("col_arg", ca), ("col_dim", cd),
                        ("col_off", co), ("par_arg", pa), ("par_dim", pd), ("par_off", po)):

@@ -102,3 +102,28 @@ def test_gradient_through_chunked_formula():
     ref = (torch.exp(-torch.cdist(xt, y.double()) ** 2) @ b.double()).sum()
     (rx,) = torch.autograd.grad(ref, [xt])
     assert rel_l2(gx.cpu().numpy(), rx.cpu().numpy()) < 1e-5
+
+
+def test_final_product_variant_and_generic_variant():
+    """Post-chunk formulas g(s)*b run their weighted sum on the matrix cores too (two 32-column blocks
+    here, forced column slabs); other post-chunk formulas keep the per-lane accumulation."""
+    from keops_amd import keops_io
+    from keops_amd.torch import Genred
+
+    M, N, D, Dv = 300, 2100, 64, 40
+    x, y, b = _laplace_inputs(M, N, D, Dv, 21)
+    xd, yd, bd = to_dev(x, y, b)
+    x64, y64, b64 = (torch.from_numpy(t).double() for t in (x, y, b))
+    K = torch.exp(-torch.cdist(x64, y64))
+    conv = Genred("Exp(-Norm2(x-y))*b", [f"x=Vi({D})", f"y=Vj({D})", f"b=Vj({Dv})"], reduction_op="Sum", axis=1)
+    for backend in ("GPU_1D", "GPU_2D"):
+        got = conv(xd, yd, bd, backend=backend).cpu().numpy()
+        assert_sum_parity(got, (K @ b64).numpy(), (K @ b64.abs()).numpy())
+    assert any(m.meta("chk_final") == "1" for m in keops_io._modules.values())
+    # not a plain product: generic accumulation in the formula's output dimension
+    conv2 = Genred("Exp(-Norm2(x-y))*b+b", [f"x=Vi({D})", f"y=Vj({D})", f"b=Vj({Dv})"], reduction_op="Sum", axis=1)
+    got2 = conv2(xd, yd, bd).cpu().numpy()
+    ref2 = (K @ b64 + b64.sum(0, keepdim=True)).numpy()
+    scale2 = (K @ b64.abs() + b64.abs().sum(0, keepdim=True)).numpy()
+    assert_sum_parity(got2, ref2, scale2)
+    assert any(m.meta("scheme") == "chunk" and m.meta("chk_final") == "0" for m in keops_io._modules.values())
