@@ -64,9 +64,19 @@ def compile_module(target_file, source, use_fast_math=True, device_id=0):
         raise KeOpsHipError(f"kernel compilation failed (code {rc}): {last_error()}")
 
 
+_iarr_cache = {}
+
+
 def _iarr(ctype, values):
-    values = list(values)
-    return (ctype * max(1, len(values)))(*values)
+    """ctypes array of ``values``; the small constant tuples of a call (variable indices, dimensions,
+    shapes) recur on every launch, so the arrays are kept."""
+    key = (ctype, tuple(values))
+    arr = _iarr_cache.get(key)
+    if arr is None:
+        if len(_iarr_cache) > 4096:
+            _iarr_cache.clear()
+        arr = _iarr_cache[key] = (ctype * max(1, len(key[1])))(*key[1])
+    return arr
 
 
 class Module:

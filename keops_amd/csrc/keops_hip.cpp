@@ -797,16 +797,18 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
     // ---- dense scheme, optionally cut in column slabs ----
     const int64_t row_blocks = (rows_total + rows_per_block - 1) / rows_per_block;
     int64_t nslabs = 1;
-    const int64_t target_blocks = 4 * (int64_t)m.cu_count;
+    // few rows: many short slabs, so that every SIMD holds several wavefronts and hides the latency
+    // of the dependent per-pair chain (one workgroup per CU would run at a fraction of the issue rate)
+    const int64_t target_blocks = 8 * (int64_t)m.cu_count;
     if (tag1D2D == 1 || row_blocks * 2 <= target_blocks) {
-      const int64_t max_slabs = std::max<int64_t>(1, cols_total / (4 * (int64_t)m.tile_j));
+      const int64_t max_slabs = std::max<int64_t>(1, cols_total / 256);
       nslabs = std::min<int64_t>(max_slabs, (target_blocks + row_blocks - 1) / row_blocks);
       if (tag1D2D == 1) nslabs = std::max<int64_t>(nslabs, std::min<int64_t>(max_slabs, 2));
       nslabs = std::min<int64_t>(nslabs, 65535);
     }
     if (nslabs > 1) {
       int64_t len = (cols_total + nslabs - 1) / nslabs;
-      len = ((len + m.tile_j - 1) / m.tile_j) * m.tile_j;
+      len = ((len + 63) / 64) * 64;
       nslabs = (cols_total + len - 1) / len;
       h.slab_len = len;
     }

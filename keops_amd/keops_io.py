@@ -108,4 +108,25 @@ class LoadKeOps_hip:
         return self
 
 
-keops_binder = {"hip": LoadKeOps_hip}
+_loaders = {}
+
+
+def load_keops_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula, aliases, nargs, dtype,
+                   lang, optional_flags, nx=None):
+    """Cached constructor (the reference keeps one LoadKeOps object per parameter set as well,
+    pykeops/pykeops/common/keops_io/LoadKeOps.py:23-31): parsing the formula and resolving the
+    module happen once, later calls only launch."""
+    from .get_keops_dll import _rows_bucket
+    from . import config
+
+    rows_hint = nx if (nx is not None and nx < 8 * 256 * config.block_size) else None
+    key = (tagCPUGPU, tag1D2D, tagHostDevice, bool(use_ranges), device_id_request, formula, tuple(aliases), nargs,
+           dtype, lang, tuple(sorted(optional_flags.items())), _rows_bucket(rows_hint))
+    obj = _loaders.get(key)
+    if obj is None:
+        obj = _loaders[key] = LoadKeOps_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula,
+                                            aliases, nargs, dtype, lang, optional_flags, nx=nx)
+    return obj
+
+
+keops_binder = {"hip": load_keops_hip}
