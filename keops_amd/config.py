@@ -20,8 +20,9 @@ dimfinalchunk = 64
 
 # workgroup geometry of the tiled kernels
 block_size = 256           # threads per workgroup (4 wavefronts)
-max_rows_per_lane = 4      # output rows held in the registers of one lane
+max_rows_per_lane = int(os.environ.get("KEOPS_AMD_MAX_ROWS", 4))      # output rows held in the registers of one lane
 lds_tile_bytes = 16384     # LDS bytes of one staged column tile
+lse_group = int(os.environ.get("KEOPS_AMD_LSE_GROUP", 8))  # log-sum-exp: columns folded per running-maximum update
 
 # matrix-core chunked scheme (csrc/kernels/keops_chunk_mfma.h): wavefronts (32 output rows each) per workgroup
 chunk_waves = int(os.environ.get("KEOPS_AMD_CHUNK_WAVES", 8))

@@ -55,6 +55,9 @@ __device__ __forceinline__ float keops_red_exp(float x) {
 }
 __device__ __forceinline__ double keops_red_exp(double x) { return __ocml_exp_f64(x); }
 
+__device__ __forceinline__ float keops_fmax(float a, float b) { return __builtin_fmaxf(a, b); }
+__device__ __forceinline__ double keops_fmax(double a, double b) { return __builtin_fmax(a, b); }
+
 template <typename A> __device__ __forceinline__ A keops_inf() { return (A)__builtin_huge_valf(); }
 
 __device__ __forceinline__ i64 keops_min(i64 a, i64 b) { return a < b ? a : b; }

@@ -18,7 +18,7 @@
 // The plug-in that precedes this header defines:  T, TACC, KEOPS_NARGS, KEOPS_DIMX, KEOPS_DIMY,
 // KEOPS_DIMY_PAD, KEOPS_DIMP, KEOPS_DIMFOUT, KEOPS_DIMRED, KEOPS_DIMOUT, KEOPS_RED_KIND,
 // KEOPS_RED_KEEP, KEOPS_RED_K, KEOPS_SUM_SCHEME, KEOPS_FAST_MATH, KEOPS_BLOCK, KEOPS_ROWS,
-// KEOPS_TILE_J, KEOPS_UNROLL_J, the tables keops_{row,col,par}_{arg,dim,off}[] with their counts
+// KEOPS_TILE_J, KEOPS_UNROLL_J, KEOPS_LSE_GROUP, the tables keops_{row,col,par}_{arg,dim,off}[] with their counts
 // KEOPS_NROWVARS / KEOPS_NCOLVARS / KEOPS_NPARVARS, and struct KeopsFormula.
 #pragma once
 #include "keops_reductions.h"
@@ -108,6 +108,42 @@ __device__ __forceinline__ void keops_sweep(const KeopsParams& P, const i64* col
 #pragma unroll
     for (int r = 0; r < KEOPS_ROWS; r++) tmp[r].init();
 #endif
+#if KEOPS_RED_KIND == 1 && KEOPS_SUM_SCHEME != 2
+    // log-sum-exp: columns are folded KEOPS_LSE_GROUP at a time (one maximum update per group);
+    // the last n % KEOPS_LSE_GROUP columns of a tile go one by one
+    constexpr int G = KEOPS_LSE_GROUP;
+    int jj0 = 0;
+    for (; jj0 + G <= n; jj0 += G) {
+      T yj[G][KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1];
+#pragma unroll
+      for (int g = 0; g < G; g++) keops_read_col(ys, jj0 + g, yj[g]);
+#pragma unroll
+      for (int r = 0; r < KEOPS_ROWS; r++) {
+        T f[G][KEOPS_DIMFOUT];
+#pragma unroll
+        for (int g = 0; g < G; g++) KeopsFormula::eval(xi[r], yj[g], p, f[g]);
+#if KEOPS_USE_TILE_TMP
+        tmp[r].template push_group<G>(f);
+#else
+        acc[r].template push_group<G>(f);
+#endif
+      }
+    }
+    for (int jj = jj0; jj < n; jj++) {
+      T yj[KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1];
+      keops_read_col(ys, jj, yj);
+#pragma unroll
+      for (int r = 0; r < KEOPS_ROWS; r++) {
+        T fout[KEOPS_DIMFOUT];
+        KeopsFormula::eval(xi[r], yj, p, fout);
+#if KEOPS_USE_TILE_TMP
+        tmp[r].push(fout, 0);
+#else
+        acc[r].push(fout, 0);
+#endif
+      }
+    }
+#else
 #pragma unroll KEOPS_UNROLL_J
     for (int jj = 0; jj < n; jj++) {
       T yj[KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1];
@@ -124,6 +160,7 @@ __device__ __forceinline__ void keops_sweep(const KeopsParams& P, const i64* col
 #endif
       }
     }
+#endif
 #if KEOPS_USE_TILE_TMP
 #pragma unroll
     for (int r = 0; r < KEOPS_ROWS; r++) acc[r].merge(tmp[r]);

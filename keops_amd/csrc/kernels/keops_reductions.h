@@ -115,6 +115,29 @@ template <typename A> struct KeopsAcc {
   }
   __device__ __forceinline__ void push(const T (&f)[KEOPS_FD], i64) { absorb<T>(f[0], &f[1]); }
   template <typename B> __device__ __forceinline__ void merge(const KeopsAcc<B>& o) { absorb<B>(o.m, o.s); }
+#if KEOPS_SUM_SCHEME != 2
+  // G pairs at once: one running-maximum update and one rescaling of s per group, then per pair a
+  // single exponential of (f - max) and one accumulation (the difference is formed first, as in the
+  // reference: folding the shift into a multiply-add would lose accuracy when |max| is large).  Same function as G calls of push (the
+  // running maximum only moves up, sums are shifted consistently); entries with f = -inf add nothing.
+  template <int G> __device__ __forceinline__ void push_group(const T (&f)[G][KEOPS_FD]) {
+    T mx = f[0][0];
+#pragma unroll
+    for (int g = 1; g < G; g++) mx = keops_fmax(mx, f[g][0]);
+    // the lower bound keeps (f - mnew) and (m - mnew) well defined when everything seen so far is -inf
+    const A mnew = keops_fmax(keops_fmax(m, (A)mx), (A)(-3.0e38f));
+    const A scale = (A)keops_red_exp((T)(m - mnew));
+#pragma unroll
+    for (int k = 0; k < KEOPS_FD - 1; k++) s[k] *= scale;
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+      const A e = (A)keops_red_exp((T)((A)f[g][0] - mnew));
+#pragma unroll
+      for (int k = 0; k < KEOPS_FD - 1; k++) s[k] += (A)f[g][1 + k] * e;
+    }
+    m = mnew;
+  }
+#endif
   __device__ __forceinline__ void store_partial(TACC* dst) const {
     dst[0] = (TACC)m;
 #pragma unroll

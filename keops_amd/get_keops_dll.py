@@ -60,8 +60,10 @@ def _c_list(xs):
     return "{" + ", ".join(str(int(x)) for x in xs) + "}"
 
 
-def choose_geometry(red, layout, nops, sizeof_t, nx=None):
-    """Rows per lane / tile length: register budget first, then enough workgroups for the chip."""
+def choose_geometry(red, layout, nops, sizeof_t, nx=None, irregular=False):
+    """Rows per lane / tile length: register budget first, then enough workgroups for the chip
+    (``irregular``: block-sparse / batched launches, whose workgroups do unequal amounts of work and
+    need many more of them to balance over the compute units)."""
     block = config.block_size
     dimy_pad = 0 if layout.dimy == 0 else -(-layout.dimy // (16 // sizeof_t)) * (16 // sizeof_t)
     per_row = layout.dimx + 2 * red.dimred * (2 if sizeof_t == 8 else 1) + min(nops, 32)
@@ -70,7 +72,7 @@ def choose_geometry(red, layout, nops, sizeof_t, nx=None):
         rows //= 2
     if nx is not None:
         # keep at least ~2 workgroups per compute unit when the row count allows it
-        while rows > 1 and nx < 2 * 256 * block * rows:
+        while rows > 1 and nx < (16 if irregular else 2) * 256 * block * rows:
             rows //= 2
     tile_j = config.lds_tile_bytes // max(1, dimy_pad * sizeof_t)
     tile_j = max(64, min(1024, 1 << (tile_j.bit_length() - 1)))
@@ -78,7 +80,7 @@ def choose_geometry(red, layout, nops, sizeof_t, nx=None):
     return dict(block=block, rows=rows, tile_j=tile_j, dimy_pad=dimy_pad, unroll=unroll)
 
 
-def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=None, geometry=None):
+def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=None, geometry=None, irregular=False):
     """HIP source of the kernel module for a reduction; returns (source, meta dict)."""
     sizeof_t = 8 if dtype == "double" else 4
     layout = VarLayout(red)
@@ -91,7 +93,7 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
     if exact:
         lines = ["    #pragma clang fp contract(off)"] + lines
     nops = L.count_ops(outs)
-    geo = choose_geometry(red, layout, nops, sizeof_t, nx)
+    geo = choose_geometry(red, layout, nops, sizeof_t, nx, irregular)
     if geometry:
         geo.update(geometry)
     ra, rd, ro = VarLayout.table(layout.rowvars)
@@ -112,6 +114,7 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
         KEOPS_DIMP=layout.dimp, KEOPS_DIMFOUT=red.formula.dim, KEOPS_DIMRED=red.dimred, KEOPS_DIMOUT=red.dim,
         KEOPS_RED_KIND=red.kind, KEOPS_RED_KEEP=red.keep, KEOPS_RED_K=red.K, KEOPS_SUM_SCHEME=SUM_SCHEMES[sum_scheme],
         KEOPS_BLOCK=geo["block"], KEOPS_ROWS=geo["rows"], KEOPS_TILE_J=geo["tile_j"], KEOPS_UNROLL_J=geo["unroll"],
+        KEOPS_LSE_GROUP=config.lse_group if (red.formula.dim <= 2 and geo["rows"] <= 2) else min(4, config.lse_group),
         KEOPS_NROWVARS=len(layout.rowvars), KEOPS_NCOLVARS=len(layout.colvars), KEOPS_NPARVARS=len(layout.parvars),
     )
     src += [f"#define {k} {v}" for k, v in defs.items()]
@@ -358,7 +361,7 @@ def get_keops_dll(
     rows_hint = None
     if nx is not None:
         # only the bucket matters for the cache key
-        rows_hint = nx if nx < 8 * 256 * config.block_size else None
+        rows_hint = nx if nx < 64 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
            use_fast_math, _rows_bucket(rows_hint), bool(enable_chunks), bool(enable_finalchunks), binder.templates_digest())
     with _lock:
@@ -386,7 +389,8 @@ def get_keops_dll(
             source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs)
             use_chunk_mode = 1
         else:
-            source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint)
+            source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint,
+                                           irregular="_ranges" in map_reduce_id)
         tag = hashlib.sha256((source + binder.templates_digest() + str(use_fast_math)).encode()).hexdigest()[:16]
         folder = config.get_build_folder()
         target = os.path.join(folder, f"hsaco_{tag}")

@@ -119,7 +119,7 @@ def load_keops_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_requ
     from .get_keops_dll import _rows_bucket
     from . import config
 
-    rows_hint = nx if (nx is not None and nx < 8 * 256 * config.block_size) else None
+    rows_hint = nx if (nx is not None and nx < 64 * 256 * config.block_size) else None
     key = (tagCPUGPU, tag1D2D, tagHostDevice, bool(use_ranges), device_id_request, formula, tuple(aliases), nargs,
            dtype, lang, tuple(sorted(optional_flags.items())), _rows_bucket(rows_hint))
     obj = _loaders.get(key)
