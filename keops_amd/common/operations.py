@@ -44,3 +44,27 @@ def postprocess(out, binding, reduction_op, nout, opt_arg, dtype):
             return (out[..., 0] + torch.log(out[..., 1]))[..., None]
         return out[..., 0][..., None] + torch.log(out[..., 1:])
     return out
+
+
+def ConjugateGradientSolver(linop, b, eps=1e-6):
+    """Conjugate gradient solution of ``linop(a) = b`` for a symmetric positive definite ``linop``
+    (pykeops/pykeops/common/operations.py:90-115: same iteration, same stopping rule
+    ``|r|^2 < numel(b) * eps^2``)."""
+    delta = b.numel() * eps ** 2
+    a = 0
+    r = b.clone()
+    nr2 = (r ** 2).sum()
+    if nr2 < delta:
+        return 0 * r
+    p = r.clone()
+    while True:
+        Mp = linop(p)
+        alp = nr2 / (p * Mp).sum()
+        a = a + alp * p
+        r = r - alp * Mp
+        nr2new = (r ** 2).sum()
+        if nr2new < delta:
+            break
+        p = r + (nr2new / nr2) * p
+        nr2 = nr2new
+    return a

@@ -413,7 +413,7 @@ class LazyTensor:
         axis -= self.nbatchdims
         return axis
 
-    def reduction(self, reduction_op, other=None, opt_arg=None, axis=None, dim=None, call=True, **kwargs):
+    def reduction(self, reduction_op, other=None, opt_arg=None, axis=None, dim=None, call=True, _solve_pid=None, **kwargs):
         """Apply a reduction over axis 0 (i) or 1 (j) (lazy_tensor.py:648-777)."""
         axis = self._axis(axis, dim)
         if axis not in (0, 1):
@@ -446,8 +446,18 @@ class LazyTensor:
             raise ValueError("the variables of the formula must occupy positions 0..n-1 without gaps")
         init_kw = {k: kwargs.pop(k) for k in list(kwargs) if k in
                    ("dtype_acc", "use_double_acc", "sum_scheme", "enable_chunks", "use_fast_math", "rec_multVar_highdim")}
-        fn = Genred(repr(formula), aliases, reduction_op=reduction_op, axis=axis, opt_arg=opt_arg,
-                    formula2=None if formula2 is None else repr(formula2), **init_kw)
+        if reduction_op == "Solve":
+            from .operations import KernelSolve
+
+            solve_kw = {k: kwargs.pop(k) for k in list(kwargs) if k in ("alpha", "eps")}
+            svar = next(v for v in formula.variables if v.ind == pos[_solve_pid])
+            solver = KernelSolve(repr(formula), aliases, f"Var({svar.ind},{svar.dim},{svar.cat})", axis=axis, **init_kw)
+
+            def fn(*args, **kw):
+                return solver(*args, **solve_kw, **kw)
+        else:
+            fn = Genred(repr(formula), aliases, reduction_op=reduction_op, axis=axis, opt_arg=opt_arg,
+                        formula2=None if formula2 is None else repr(formula2), **init_kw)
         data = [None] * nvars
         cats = {v.ind: v.cat for f in (formula,) + (() if formula2 is None else (formula2,)) for v in f.variables}
         dev = next((t.device for t in whole.variables.values() if isinstance(t, torch.Tensor)), None)
@@ -478,6 +488,30 @@ class LazyTensor:
         if call and all(d is not None for d in data):
             return run()
         return run
+
+    def solve(self, other, var=None, call=True, **kwargs):
+        """Solution ``a`` of ``sum_j self_ij a_j = other_i`` (plus ``alpha * a``) by conjugate gradient, for a
+        symmetric positive definite ``self`` (lazy_tensor.py:779-897; keyword arguments alpha, eps, backend,
+        ranges and the Genred options).  ``other`` is a 2D tensor (one row per index i) or an i-indexed
+        LazyTensor holding one."""
+        if var is not None:
+            raise NotImplementedError("solve(var=...) with a symbolic unknown is not available")
+        if isinstance(other, LazyTensor):
+            if len(other.variables) != 1 or not isinstance(other.formula, O.Var) or other.formula.cat != 0:
+                raise ValueError("'other' must be a plain i-indexed variable")
+            other = next(iter(other.variables.values()))
+        if not isinstance(other, torch.Tensor) or other.dim() < 2:
+            raise ValueError("'other' must be a 2D tensor, one row per index i")
+        unknown = LazyTensor(other, axis=1)  # the unknown is indexed like the reduced axis; 'other' is its start value
+        pid = next(iter(unknown.variables))
+        return (self * unknown).reduction("Solve", axis=self.nbatchdims + 1, call=call, _solve_pid=pid, **kwargs)
+
+    def matvec(self, v):
+        """Matrix-vector product with a 1D tensor, for scipy-style linear operator code (lazy_tensor.py matvec)."""
+        return self @ v
+
+    def rmatvec(self, v):
+        return self.T @ v
 
     def sum(self, axis=None, dim=None, **kwargs):
         ax = axis if axis is not None else dim
@@ -537,6 +571,12 @@ class LazyTensor:
 
     def Kmin_argKmin(self, K, axis=None, dim=None, **kwargs):
         return self.reduction("KMin_ArgKMin", opt_arg=K, axis=axis, dim=dim, **kwargs)
+
+
+# the reference also exposes every reduction under a "<name>_reduction" alias (lazy_tensor.py)
+for _name in ("min", "argmin", "min_argmin", "max", "argmax", "max_argmax", "Kmin", "argKmin", "Kmin_argKmin",
+              "sumsoftmaxweight"):
+    setattr(LazyTensor, _name + "_reduction", getattr(LazyTensor, _name))
 
 
 def Vi(x_or_ind, dim=None):
