@@ -1,0 +1,107 @@
+"""NumPy front end: the same Genred / KernelSolve call signatures on host arrays.
+
+Counterpart of pykeops/pykeops/numpy (generic/generic_red.py, operations.py).  The reference's NumPy
+binding hands host pointers to the GPU engine, which stages them itself (tagHostDevice = 0,
+keops_nvrtc.cpp load_args_FromHost).  The HIP library only takes device pointers, so the staging is
+done here: arrays are copied to the current HIP device as torch tensors, the torch binding runs the
+reduction, and the result comes back as a NumPy array.  There is no CPU computation path.
+"""
+import numpy as np
+import torch
+
+from ..torch import Genred as _TorchGenred
+from ..torch import KernelSolve as _TorchKernelSolve
+
+
+def _device(device_id):
+    if not torch.cuda.is_available():
+        raise RuntimeError("[KeOps] the HIP backend needs a GPU; there is no CPU computation path")
+    return torch.device("cuda", torch.cuda.current_device() if device_id in (-1, None) else device_id)
+
+
+def _to_device(args, dev):
+    out = []
+    for a in args:
+        a = np.ascontiguousarray(a)
+        if a.dtype not in (np.float32, np.float64):
+            raise ValueError("[KeOps] only float32 and float64 arrays are supported")
+        out.append(torch.from_numpy(a).to(dev))
+    return out
+
+
+def _ranges_to_device(ranges, dev):
+    if ranges is None:
+        return None
+    return tuple(torch.from_numpy(np.ascontiguousarray(r).astype(np.int64)).to(dev) for r in ranges)
+
+
+class Genred:
+    """``Genred(formula, aliases, reduction_op, axis, ...)(*numpy_arrays) -> numpy array``
+    (pykeops/pykeops/numpy/generic/generic_red.py)."""
+
+    def __init__(self, formula, aliases, reduction_op="Sum", axis=0, dtype=None, opt_arg=None, formula2=None,
+                 cuda_type=None, dtype_acc="auto", use_double_acc=False, sum_scheme="auto", enable_chunks=True,
+                 rec_multVar_highdim=False, use_fast_math=True):
+        self._fn = _TorchGenred(formula, aliases, reduction_op=reduction_op, axis=axis, opt_arg=opt_arg,
+                                formula2=formula2, dtype_acc=dtype_acc, use_double_acc=use_double_acc,
+                                sum_scheme=sum_scheme, enable_chunks=enable_chunks,
+                                rec_multVar_highdim=rec_multVar_highdim, use_fast_math=use_fast_math)
+
+    def __call__(self, *args, backend="auto", device_id=-1, ranges=None, out=None):
+        if backend == "CPU":
+            raise ValueError("[KeOps] backend 'CPU' is not available in the HIP build")
+        dev = _device(device_id)
+        res = self._fn(*_to_device(args, dev), backend=backend.replace("_Host", "").replace("_Device", ""),
+                       ranges=_ranges_to_device(ranges, dev))
+        res = res.cpu().numpy()
+        if out is not None:
+            out[...] = res
+            return out
+        return res
+
+
+class KernelSolve:
+    """``KernelSolve(formula, aliases, varinvalias, axis)(*numpy_arrays, alpha=..., eps=...)``
+    (pykeops/pykeops/numpy/operations.py)."""
+
+    def __init__(self, formula, aliases, varinvalias, axis=0, dtype=None, opt_arg=None, dtype_acc="auto",
+                 use_double_acc=False, sum_scheme="auto", enable_chunks=True, rec_multVar_highdim=None,
+                 use_fast_math=True):
+        self._fn = _TorchKernelSolve(formula, aliases, varinvalias, axis=axis, dtype_acc=dtype_acc,
+                                     use_double_acc=use_double_acc, sum_scheme=sum_scheme, enable_chunks=enable_chunks,
+                                     rec_multVar_highdim=rec_multVar_highdim, use_fast_math=use_fast_math)
+
+    def __call__(self, *args, backend="auto", device_id=-1, alpha=1e-10, eps=1e-6, ranges=None):
+        dev = _device(device_id)
+        res = self._fn(*_to_device(args, dev), backend=backend, alpha=alpha, eps=eps,
+                       ranges=_ranges_to_device(ranges, dev))
+        return res.cpu().numpy()
+
+
+def _split(output, aliases):
+    from ..common.parse_type import get_type
+
+    _, cat, dim, _ = get_type(output)
+    return list(aliases), (cat + 1) % 2, dim  # reduce over the other index
+
+
+def generic_sum(formula, output, *aliases, **kwargs):
+    """The first alias names the output and fixes the reduction axis
+    (pykeops/pykeops/numpy/generic/generic_ops.py)."""
+    al, axis, _ = _split(output, aliases)
+    return Genred(formula, al, reduction_op="Sum", axis=axis, **kwargs)
+
+
+def generic_logsumexp(formula, output, *aliases, **kwargs):
+    al, axis, _ = _split(output, aliases)
+    return Genred(formula, al, reduction_op="LogSumExp", axis=axis, **kwargs)
+
+
+def generic_argmin(formula, output, *aliases, **kwargs):
+    al, axis, _ = _split(output, aliases)
+    return Genred(formula, al, reduction_op="ArgMin", axis=axis, **kwargs)
+
+
+def generic_argkmin(formula, output, *aliases, **kwargs):
+    al, axis, dim = _split(output, aliases)
+    return Genred(formula, al, reduction_op="ArgKMin", axis=axis, opt_arg=dim, **kwargs)

@@ -54,3 +54,24 @@ def test_lazytensor_solve_float32():
     d = ((x_i - x_j) ** 2).sum(-1)
     assert torch.equal(d.argKmin_reduction(3, dim=1), d.argKmin(3, dim=1))
     assert torch.equal(d.min_reduction(dim=1), d.min(dim=1))
+
+
+def test_numpy_front_end():
+    import numpy as np
+
+    from keops_amd.numpy import Genred, KernelSolve, generic_argkmin
+
+    rng = np.random.default_rng(0)
+    x, y, b = rng.standard_normal((300, 3)), rng.standard_normal((500, 3)), rng.standard_normal((500, 2))
+    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)"], reduction_op="Sum", axis=1)
+    got = conv(x, y, b)
+    assert isinstance(got, np.ndarray) and got.dtype == np.float64
+    ref = np.exp(-((x[:, None, :] - y[None, :, :]) ** 2).sum(-1)) @ b
+    assert np.max(np.abs(got - ref)) < 1e-12
+    knn = generic_argkmin("SqDist(x,y)", "a = Vi(4)", "x = Vi(3)", "y = Vj(3)")
+    idx = knn(x.astype(np.float32), y.astype(np.float32))
+    d2 = ((x.astype(np.float32)[:, None, :] - y.astype(np.float32)[None, :, :]) ** 2).sum(-1)
+    assert np.array_equal(np.sort(idx, 1), np.sort(np.argsort(d2, 1, kind="stable")[:, :4], 1))
+    a = KernelSolve("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)"], "b", axis=1)(x, x, b[:300], alpha=0.3, eps=1e-12)
+    K = np.exp(-((x[:, None, :] - x[None, :, :]) ** 2).sum(-1))
+    assert np.max(np.abs(a - np.linalg.solve(0.3 * np.eye(300) + K, b[:300]))) < 1e-8
