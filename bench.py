@@ -32,8 +32,8 @@ PUBLISHED_PAIRS_PER_S = 1e12 / 1.39
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/);
 # None until measured for a workload
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/keops_conv_dense__gauss_1m_dv1.md: FETCH_SIZE 230808 KiB x 2.0 (copy calibration) + WRITE_SIZE 3906.25 KiB
-    "gauss_1m_dv1": int((230808 * 2.0 + 3906.25) * 1024),
+    # profiles/keops_conv_dense__gauss_1m_dv1.md: FETCH_SIZE 162134 KiB x 2.0 (copy calibration) + WRITE_SIZE 66406 KiB
+    "gauss_1m_dv1": int((162134 * 2.0 + 66406) * 1024),
     # profiles/keops_knn_filter__knn_d64.md: dominant kernel keops_knn_filter
     "knn_d64": int((822401 * 2.0 + 163406) * 1024),
     # profiles/keops_chk_final__laplace_d256.md
