@@ -28,7 +28,7 @@ lse_group = int(os.environ.get("KEOPS_AMD_LSE_GROUP", 8))  # log-sum-exp: column
 chunk_waves = int(os.environ.get("KEOPS_AMD_CHUNK_WAVES", 8))
 
 # matrix-core final-product scheme (csrc/kernels/keops_final_mfma.h): Sum_j f(x_i,y_j) * v_j with dim(v) large
-final_chunk_min_dim = int(os.environ.get("KEOPS_AMD_FINAL_MIN_DIM", 64))   # smallest dim(v) that selects the scheme
+final_chunk_min_dim = int(os.environ.get("KEOPS_AMD_FINAL_MIN_DIM", 24))   # smallest dim(v) that selects the scheme
 final_max_blocks = int(os.environ.get("KEOPS_AMD_FINAL_NB", 8))            # 32-column accumulator tiles per wavefront
 final_waves = int(os.environ.get("KEOPS_AMD_FINAL_WAVES", 8))              # wavefronts (32 output rows each) per workgroup
 final_tile_j = int(os.environ.get("KEOPS_AMD_FINAL_TJ", 32))               # reduced rows per staged tile (even)

@@ -280,7 +280,7 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
 
 def match_final(red, dtype, dtypeacc, sum_scheme, map_reduce_id):
     """(scalar kernel f, variable v) when ``red`` is Sum_Reduction(f * v) with f of dimension 1 and v a
-    plain reduced-index variable of dimension >= config.final_chunk_min_dim, in float32 on the dense
+    plain reduced-index variable of dimension >= config.final_chunk_min_dim (24), in float32 on the dense
     scheme (the shape GpuReduc1D_finalchunks.py:100-106 expects); None otherwise."""
     from .formulas import ops as O
     from .formulas.reductions import KIND_SUM
@@ -294,6 +294,10 @@ def match_final(red, dtype, dtypeacc, sum_scheme, map_reduce_id):
         return None
     for f, v in (F.children, F.children[::-1]):
         if f.dim == 1 and isinstance(v, O.Var) and v.cat == 1 - red.tagI and v.dim == F.dim and v.dim >= config.final_chunk_min_dim:
+            # a 32-column matrix tile costs as much as ~22 vector multiply-adds per pair: just above a
+            # multiple of 32 the vector kernel is still the faster one
+            if v.dim > 32 and v.dim % 32 != 0 and v.dim % 32 < 8 and v.dim < 128:
+                return None
             return f, v
     return None
 

@@ -37,7 +37,7 @@ def _aliases(Dv):
     (1000, 3000, 256, "block_sum"),     # few output rows: slabs over the reduced axis + ordered sum
     (777, 1001, 200, "block_sum"),      # ragged last column block, ragged last tile
     (333, 2500, 300, "direct_sum"),     # more column blocks than one wavefront keeps: two workgroups per row block
-    (70, 50, 64, "block_sum"),          # smallest dimension that selects the scheme, less than one tile pair
+    (70, 50, 24, "block_sum"),          # smallest dimension that selects the scheme, less than one tile pair
     (256, 20000, 96, "block_sum"),      # several block-sum periods
 ])
 def test_gaussian_times_highdim_vs_oracle(M, N, Dv, scheme):
