@@ -313,6 +313,7 @@ struct KnnHeader {
   void* logcount;
   void* overflow;
   int64_t logcap;
+  int32_t stage, pad_;
 };
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -359,10 +360,28 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   // filter pass
   const int64_t f_qblocks = (nq + FQB - 1) / FQB;
   int64_t f_slabs = pick_slabs(f_qblocks, nr, TJ, m.cu_count, 2, 1);
-  // one filter workgroup fills a CU and all of them take the same time
-  f_slabs = balance_slabs(f_qblocks, f_slabs, std::min<int64_t>(4 * f_slabs, std::max<int64_t>(1, nr / (16 * TJ))), m.cu_count);
+  // one filter workgroup fills a CU and all of them take the same time.  With at least 8 slabs the filter runs
+  // in two stages (every 4th slab, then the others, with thresholds refined in between): both grids should
+  // be close to whole rounds over the CUs
+  {
+    const int64_t cap = std::max<int64_t>(1, nr / (16 * TJ));
+    int64_t best = f_slabs;
+    double best_eff = 0.0;
+    for (int64_t n = f_slabs; n <= std::max(f_slabs, std::min<int64_t>(std::max<int64_t>(4 * f_slabs, 24), cap)); n++) {
+      auto eff = [&](int64_t blocks) {
+        const int64_t rounds = (blocks + m.cu_count - 1) / m.cu_count;
+        return (double)blocks / (double)(rounds * m.cu_count);
+      };
+      const int64_t na = n >= 8 ? (n + 3) / 4 : n;
+      const double e = n >= 8 ? (eff(f_qblocks * na) + 3.0 * eff(f_qblocks * (n - na))) / 4.0 : eff(f_qblocks * n);
+      if (e > best_eff + 0.015) { best_eff = e; best = n; }
+    }
+    f_slabs = best;
+  }
   int64_t f_len = ((nr + f_slabs - 1) / f_slabs + TJ - 1) / TJ * TJ;
   f_slabs = std::max<int64_t>(1, (nr + f_len - 1) / f_len);
+  const bool staged = two_phase && f_slabs >= 8;
+  const int64_t fa_slabs = staged ? (f_slabs + 3) / 4 : f_slabs, fb_slabs = f_slabs - fa_slabs;
   const int64_t nlogs = f_qblocks * f_slabs * FW;
   // expected survivors per query: SAMPLE * K (the sample's K-th neighbour is about the (SAMPLE*K)-th overall)
   const int64_t logcap = two_phase ? align_up((size_t)(4 * FQW * SAMPLE * K / f_slabs + 512), 64) : 0;
@@ -373,10 +392,11 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
   const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(512, nr / 64));
   const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
-  const size_t o_xh = take((size_t)nq * DP * 2), o_yh = take((size_t)nr * DP * 2);
+  const int64_t RW = DP * (m.meta_int("knn_split", 0) ? 2 : 1);  // bf16 elements per stored row ([hi] or [hi | lo])
+  const size_t o_xh = take((size_t)nq * RW * 2), o_yh = take((size_t)nr * RW * 2);
   const size_t o_xkey = take((size_t)nq * 4), o_ykey = take((size_t)nr * 4);
   const size_t o_pd = take((size_t)list_slabs * nq * K * 4), o_pi = take((size_t)list_slabs * nq * K * 4);
-  const size_t o_yhs = take((size_t)nsample * DP * 2), o_ykeys = take((size_t)nsample * 4);
+  const size_t o_yhs = take((size_t)nsample * RW * 2), o_ykeys = take((size_t)nsample * 4);
   const size_t o_thr = take((size_t)nq * 4), o_flag = take(256);
   const size_t o_logcount = take((size_t)(two_phase ? nlogs : 0) * 4), o_log = take((size_t)(two_phase ? nlogs : 0) * logcap * 8);
   if (int rc = m.partial.reserve(off)) return rc;
@@ -412,15 +432,24 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
     std::memcpy(&p.extra[0], &gargs[0], 8);
     std::memcpy(&p.extra[1], &gargs[1], 8);
     p.extra[2] = nsample;
-    const int64_t chunks = nsample * (DP / 8);
+    const int64_t chunks = nsample * (RW / 8);
     if (int rc = run("keops_knn_gather_sample", (unsigned)((chunks + 255) / 256), 1, 256, HS + 24)) return rc;
     if (int rc = adaptive(nsample, ws + o_yhs, ws + o_ykeys, (int)SAMPLE, a_slabs, a_len)) return rc;
-    if (int rc = run("keops_knn_thresholds", (unsigned)((nq + 255) / 256), 1, 256, HS)) return rc;
-    // (b) fixed-threshold filter over all references, survivors logged per wavefront
+    auto with_2int = [&](int a, int b) { int v[2] = {a, b}; std::memcpy(p.extra, v, 8); return HS + 8; };
+    if (int rc = run("keops_knn_thresholds", (unsigned)((nq + 255) / 256), 1, 256, with_2int(0, 0))) return rc;
+    // (b) fixed-threshold filter, survivors logged per wavefront; (c) exact replay of the logs.
+    // Staged: every 4th slab first, thresholds refined from its replay, then the other slabs.
     h.nr = nr; h.yh = ws + o_yh; h.ykey = ws + o_ykey; h.ref_step = 1; h.nslabs = (int32_t)f_slabs; h.slab_len = f_len;
-    if (int rc = run("keops_knn_filter", (unsigned)f_qblocks, (unsigned)f_slabs, (unsigned)(64 * FW), HS)) return rc;
-    // (c) exact replay of the logs
-    if (int rc = run("keops_knn_rerank", (unsigned)nlogs, 1, 64, with_int((int)f_qblocks))) return rc;
+    h.stage = staged ? 1 : 0;
+    if (int rc = run("keops_knn_filter", (unsigned)f_qblocks, (unsigned)fa_slabs, (unsigned)(64 * FW), HS)) return rc;
+    if (int rc = run("keops_knn_rerank", (unsigned)(f_qblocks * fa_slabs * FW), 1, 64, with_int((int)f_qblocks))) return rc;
+    if (staged) {
+      if (int rc = run("keops_knn_thresholds", (unsigned)((nq + 255) / 256), 1, 256, with_2int(1, (int)fa_slabs))) return rc;
+      h.stage = 2;
+      if (int rc = run("keops_knn_filter", (unsigned)f_qblocks, (unsigned)fb_slabs, (unsigned)(64 * FW), HS)) return rc;
+      if (int rc = run("keops_knn_rerank", (unsigned)(f_qblocks * fb_slabs * FW), 1, 64, with_int((int)f_qblocks))) return rc;
+      h.stage = 0;
+    }
     if (int rc = ensure_pinned(m, 64)) return rc;
     HIP_TRY(hipMemcpyAsync(m.pinned, h.overflow, 4, hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipStreamSynchronize(stream));

@@ -1,5 +1,7 @@
-// K-nearest-neighbour search (KMin / ArgKMin / KMin_ArgKMin of SqDist(x_i, y_j)) for D >= 32:
-// matrix-core filter + exact re-rank.
+// K-nearest-neighbour search (KMin / ArgKMin / KMin_ArgKMin of SqDist(x_i, y_j)): matrix-core filter +
+// exact re-rank.  One bf16 per component for D >= 32; for lower dimensions (dense point clouds, where
+// neighbours are close compared with the norms) every component is split as hi + lo (KNN_SPLIT) and the
+// inner product takes three MFMAs per k-block, which tightens the filter slack from 8e-3 to 5e-5.
 //
 // Replaces, for this formula, the generic kernel the reference would generate from
 //   keopscore/keopscore/mapreduce/gpu/GpuReduc1D.py:43-96 with
@@ -33,11 +35,14 @@
 //      (b) keops_knn_filter sweeps all references against the fixed thresholds and only logs the
 //      surviving (query, reference) pairs, each wavefront in a private region of global memory (no
 //      atomics, no list updates); (c) keops_knn_rerank replays every log with the exact distance and
-//      the same K-list insertion.  If a log overflows (pathological ties) the host falls back to the
-//      adaptive kernel over all references.
+//      the same K-list insertion.  With enough slabs, (b)-(c) run twice: first on every 4th slab, whose
+//      replayed lists tighten the thresholds (K-th distance among a quarter of the references instead of
+//      among the sample), then on the other slabs, which then log about four times fewer survivors.
+//      If a log overflows (pathological ties) the host falls back to the adaptive kernel over all
+//      references.
 //
 // The plug-in defines: T (float), KEOPS_NARGS, KNN_D, KNN_DPAD (D rounded up to 16), KNN_K,
-// KEOPS_RED_KEEP, KEOPS_DIMOUT, KNN_QSETS, KNN_WAVES (wavefronts per workgroup), KNN_TJ.
+// KEOPS_RED_KEEP, KEOPS_DIMOUT, KNN_QSETS, KNN_WAVES (wavefronts per workgroup), KNN_TJ, KNN_SPLIT.
 #pragma once
 #include "keops_common.h"
 
@@ -46,10 +51,21 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 knn_bf16x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float knn_f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float knn_f32x4;
 
+#ifndef KNN_SPLIT
+#define KNN_SPLIT 0
+#endif
 #define KNN_KB (KNN_DPAD / 16)         // 16-wide k blocks
-#define KNN_STRIDE (KNN_DPAD * 2 + 16) // bytes per staged reference row (16 B pad: conflict-free b128 reads)
-// filter slack: 4u(1+3u) + 2(D+1) 2^-24 with u = 2^-9, rounded up (see header comment)
+#define KNN_RW (KNN_DPAD * (1 + KNN_SPLIT))  // bf16 elements per stored row: [hi] or [hi | lo]
+#define KNN_STRIDE (KNN_RW * 2 + 16)   // bytes per staged reference row (16 B pad: conflict-free b128 reads)
+// Filter slack c.  One bf16 per component (D >= 32): 4u(1+3u) + 2(D+1) 2^-24 with u = 2^-9, rounded up.
+// Split operands x^ = hi + lo (KNN_SPLIT, low dimensions, where neighbours are close compared with the
+// norms): representation error 2^-18 per vector, the dropped lo*lo product 2^-18 |x^||y^|, fp32
+// accumulation of at most 100 exact bf16 products: 5 2^-18 + 200 2^-24 = 3.1e-5, rounded up.
+#if KNN_SPLIT
+#define KNN_C 5.0e-5f
+#else
 #define KNN_C 0.0082f
+#endif
 #define KNN_DELTA 2e-5f
 #define KNN_FLT_MAX 3.402823466e38f
 
@@ -57,8 +73,8 @@ struct KnnParams {
   i64 nq, nr;            // queries (output rows), references (reduced rows)
   const float* xq;       // [nq][KNN_D] original queries
   const float* yr;       // [nr][KNN_D] original references
-  __bf16* xh;            // [nq][KNN_DPAD] centred bf16 queries
-  __bf16* yh;            // [nr][KNN_DPAD]
+  __bf16* xh;            // [nq][KNN_RW] centred bf16 queries (times -2)
+  __bf16* yh;            // [nr][KNN_RW]
   float* xkey;           // [nq]  (1-c)|x^|^2
   float* ykey;           // [nr]
   float* colsum;         // [KNN_DPAD] column sums of the references
@@ -74,7 +90,13 @@ struct KnnParams {
   int* logcount;         // [nlogs] entries written (clamped to logcap)
   int* overflow;         // set to 1 when a log was too small
   i64 logcap;
+  int stage;             // filter / replay: which slabs this launch covers (knn_stage_slab)
+  int pad_;
 };
+
+// Slab handled by workgroup row y of a filter (or replay) launch.  stage 0: all slabs in order;
+// stage 1: every 4th slab (0, 4, 8, ...), whose exact replay tightens the thresholds; stage 2: the others.
+__device__ __forceinline__ int knn_stage_slab(int stage, int y) { return stage == 0 ? y : (stage == 1 ? 4 * y : y + y / 3 + 1); }
 
 // ---- pre-pass ---------------------------------------------------------------------------------
 
@@ -147,20 +169,28 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_prep(const KnnParams
   float nrm = 0.f;
   const bool live = row < n && sub * 4 < KNN_DPAD;
   if (live) {
-    knn_bf16x4 h;
+    knn_bf16x4 h, l;
 #pragma unroll
     for (int e = 0; e < 4; e++) {
       const int c = sub * 4 + e;
       float v = 0.f;
       if (c < KNN_D) v = src[row * KNN_D + c] - P.colsum[c] * inv;
       h[e] = (__bf16)v;
-      const float r = (float)h[e];
+      float r = (float)h[e];
+      if (KNN_SPLIT) {
+        l[e] = (__bf16)(v - r);
+        r += (float)l[e];  // exact: the two parts do not overlap
+      }
       nrm += r * r;
       // queries are stored as -2 x^ (exact in bf16) so that the MFMA accumulator, initialised with
       // the reference keys, directly holds (1-c)|y^|^2 - 2 <y^, x^>
-      if (!which) h[e] = (__bf16)(-2.0f * r);
+      if (!which) {
+        h[e] = (__bf16)(-2.0f * (float)h[e]);
+        if (KNN_SPLIT) l[e] = (__bf16)(-2.0f * (float)l[e]);
+      }
     }
-    *reinterpret_cast<knn_bf16x4*>(dst + row * KNN_DPAD + sub * 4) = h;
+    *reinterpret_cast<knn_bf16x4*>(dst + row * KNN_RW + sub * 4) = h;
+    if (KNN_SPLIT) *reinterpret_cast<knn_bf16x4*>(dst + row * KNN_RW + KNN_DPAD + sub * 4) = l;
   }
 #pragma unroll
   for (int o = KNN_LPR / 2; o > 0; o >>= 1) nrm += __shfl_xor(nrm, o, KNN_LPR);
@@ -225,6 +255,7 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
 
   // queries of this wavefront as MFMA B operands
   knn_bf16x8 bq[QSETS][KNN_KB];
+  knn_bf16x8 bql[QSETS][KNN_SPLIT ? KNN_KB : 1];  // low parts (split operands)
   float xk[QSETS], t[QSETS];
   bool valid[QSETS];
 #pragma unroll
@@ -233,8 +264,10 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
     valid[h] = q < P.nq;
     if (!valid[h]) q = P.nq - 1;
 #pragma unroll
-    for (int kb = 0; kb < KNN_KB; kb++)
-      bq[h][kb] = *reinterpret_cast<const knn_bf16x8*>(P.xh + q * KNN_DPAD + kb * 16 + 8 * half);
+    for (int kb = 0; kb < KNN_KB; kb++) {
+      bq[h][kb] = *reinterpret_cast<const knn_bf16x8*>(P.xh + q * KNN_RW + kb * 16 + 8 * half);
+      if (KNN_SPLIT) bql[h][kb] = *reinterpret_cast<const knn_bf16x8*>(P.xh + q * KNN_RW + KNN_DPAD + kb * 16 + 8 * half);
+    }
     xk[h] = P.xkey[q];
     // finite start value: padded rows carry an infinite key and never pass
     if (MODE == 0) t[h] = valid[h] ? KNN_FLT_MAX : -inf;
@@ -248,7 +281,8 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
   }
   int qcount = 0;    // wave-uniform number of queued candidates
   i64 logged = 0;    // wave-uniform number of entries already in this wavefront's log
-  const i64 logid = ((i64)blockIdx.y * gridDim.x + blockIdx.x) * WAVES + wave;
+  const int slab = MODE == 1 ? knn_stage_slab(P.stage, blockIdx.y) : (int)blockIdx.y;
+  const i64 logid = ((i64)slab * gridDim.x + blockIdx.x) * WAVES + wave;
   int2* mylog = MODE == 1 ? P.log + logid * P.logcap : nullptr;
 
   // MODE 0: re-examine the queued candidates (one per lane) and refresh the thresholds
@@ -290,16 +324,16 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
     }
   };
 
-  const i64 jbeg = (i64)blockIdx.y * P.slab_len;
+  const i64 jbeg = (i64)slab * P.slab_len;
   const i64 jend = keops_min(P.nr, jbeg + P.slab_len);
   // software pipeline: the rows of tile t+1 travel from HBM/L2 to registers while tile t is consumed
-  constexpr int CH = KNN_DPAD / 8;                          // 16-byte chunks per staged row
+  constexpr int CH = KNN_RW / 8;                            // 16-byte chunks per staged row
   constexpr int NPF = (KNN_TJ * CH + BLOCK - 1) / BLOCK;    // chunks per thread and tile
   uint4 pf[NPF];
   float pfkey = inf;
   auto prefetch = [&](i64 j0) {
     const int n = (int)keops_min((i64)KNN_TJ, jend - j0);
-    const uint4* src = reinterpret_cast<const uint4*>(P.yh + j0 * KNN_DPAD);
+    const uint4* src = reinterpret_cast<const uint4*>(P.yh + j0 * KNN_RW);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * BLOCK;
@@ -339,6 +373,15 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
 #pragma unroll
       for (int kb = 0; kb < KNN_KB; kb++) {
         const knn_bf16x8 a = *reinterpret_cast<const knn_bf16x8*>(arow + kb * 32);
+        if (KNN_SPLIT) {
+          // <hi + lo, hi + lo> without the lo * lo term, smallest products first
+          const knn_bf16x8 al = *reinterpret_cast<const knn_bf16x8*>(arow + KNN_DPAD * 2 + kb * 32);
+#pragma unroll
+          for (int h = 0; h < QSETS; h++) {
+            acc[h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bq[h][kb], acc[h], 0, 0, 0);
+            acc[h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bql[h][kb], acc[h], 0, 0, 0);
+          }
+        }
 #pragma unroll
         for (int h = 0; h < QSETS; h++) acc[h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bq[h][kb], acc[h], 0, 0, 0);
       }
@@ -428,7 +471,7 @@ extern "C" __global__ void __launch_bounds__(64 * KNN_FWAVES) keops_knn_filter(c
 // every KNN_SAMPLE-th reference row (bf16 row + key) gathered in a compact array for the sampling pass
 extern "C" __global__ void __launch_bounds__(256) keops_knn_gather_sample(const KnnParams P, __bf16* yh_s, float* ykey_sm,
                                                                            i64 nsample) {
-  constexpr int CH = KNN_DPAD / 8;
+  constexpr int CH = KNN_RW / 8;
   const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
   const i64 row = e / CH;
   const int c = (int)(e - row * CH);
@@ -439,13 +482,16 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_gather_sample(const 
 
 // ---- merge of the per-slab lists ----------------------------------------------------------------
 
-__device__ __forceinline__ void knn_merge_lists(const KnnParams& P, i64 q, float (&bv)[KNN_K], int (&bi)[KNN_K]) {
+// merges the sorted lists of slabs first, first + stride, ... (count of them) of query q
+__device__ __forceinline__ void knn_merge_lists(const KnnParams& P, i64 q, float (&bv)[KNN_K], int (&bi)[KNN_K],
+                                                int first, int stride, int count) {
 #pragma unroll
   for (int l = 0; l < KNN_K; l++) {
-    bv[l] = P.plist_d[q * KNN_K + l];
-    bi[l] = P.plist_i[q * KNN_K + l];
+    bv[l] = P.plist_d[((i64)first * P.nq + q) * KNN_K + l];
+    bi[l] = P.plist_i[((i64)first * P.nq + q) * KNN_K + l];
   }
-  for (int s = 1; s < P.nslabs; s++) {
+  for (int t = 1; t < count; t++) {
+    const int s = first + t * stride;
     for (int l = 0; l < KNN_K; l++) {
       const float d = P.plist_d[((i64)s * P.nq + q) * KNN_K + l];
       const int j = P.plist_i[((i64)s * P.nq + q) * KNN_K + l];
@@ -472,7 +518,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParam
   if (q >= P.nq) return;
   float bv[KNN_K];
   int bi[KNN_K];
-  knn_merge_lists(P, q, bv, bi);
+  knn_merge_lists(P, q, bv, bi, 0, 1, P.nslabs);
   T* out = P.out + q * KEOPS_DIMOUT;
 #pragma unroll
   for (int l = 0; l < KNN_K; l++) {
@@ -487,16 +533,22 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParam
   }
 }
 
-// thresholds of the filter pass from the K-lists of the sampling pass
-extern "C" __global__ void __launch_bounds__(256) keops_knn_thresholds(const KnnParams P) {
+// Thresholds of a filter pass from K-lists of a subset of the references (any such K-th distance is
+// an upper bound of the final one).  refine = 0: lists of the sampling pass (slabs 0 .. nslabs-1);
+// refine = 1: lists replayed from the stage-1 slabs (0, 4, 8, ...: `count` of them), kept only where
+// tighter than the current threshold.
+extern "C" __global__ void __launch_bounds__(256) keops_knn_thresholds(const KnnParams P, int refine, int count) {
   const i64 q = (i64)blockIdx.x * 256 + threadIdx.x;
-  if (q == 0) *P.overflow = 0;  // reset before the filter pass (a fill kernel would be one more launch)
+  if (q == 0 && !refine) *P.overflow = 0;  // reset before the filter passes (a fill kernel would be one more launch)
   if (q >= P.nq) return;
   float bv[KNN_K];
   int bi[KNN_K];
-  knn_merge_lists(P, q, bv, bi);
+  if (refine) knn_merge_lists(P, q, bv, bi, 0, 4, count);
+  else knn_merge_lists(P, q, bv, bi, 0, 1, P.nslabs);
   const float tau = bv[KNN_K - 1];
-  P.thr[q] = __builtin_fminf((tau + tau * KNN_DELTA) - P.xkey[q], KNN_FLT_MAX);
+  float t = __builtin_fminf((tau + tau * KNN_DELTA) - P.xkey[q], KNN_FLT_MAX);
+  if (refine) t = __builtin_fminf(t, P.thr[q]);
+  P.thr[q] = t;
 }
 
 // ---- replay of the candidate logs ---------------------------------------------------------------
@@ -509,10 +561,10 @@ extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParam
   __shared__ int li[QW][KNN_K];
   __shared__ int owner[QW];
   const int lane = threadIdx.x;
-  const i64 logid = blockIdx.x;
-  const int wave = (int)(logid % KNN_FWAVES);
-  const i64 rest = logid / KNN_FWAVES;
-  const i64 bx = rest % fgrid_x, slab = rest / fgrid_x;
+  const int wave = (int)(blockIdx.x % KNN_FWAVES);
+  const i64 rest = blockIdx.x / KNN_FWAVES;
+  const i64 bx = rest % fgrid_x, slab = knn_stage_slab(P.stage, (int)(rest / fgrid_x));
+  const i64 logid = (slab * fgrid_x + bx) * KNN_FWAVES + wave;
   const i64 qw0 = bx * (KNN_FWAVES * QW) + (i64)wave * QW;
   const float inf = __builtin_huge_valf();
   for (int e = lane; e < QW * KNN_K; e += 64) {

@@ -136,7 +136,7 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
 
 def match_knn_sqdist(red, dtype, map_reduce_id):
     """(row variable, column variable) when ``red`` is a K-min family reduction of SqDist between an
-    output-indexed and a reduced-index variable of dimension 32..256 in float32, on the dense
+    output-indexed and a reduced-index variable of dimension config.knn_min_dim..256 in float32, on the dense
     scheme; None otherwise.  Such reductions run on the matrix-core filter + exact re-rank kernels."""
     from .formulas import ops as O
 
@@ -146,7 +146,7 @@ def match_knn_sqdist(red, dtype, map_reduce_id):
     if f.name != "Sum" or f.children[0].name != "Square" or f.children[0].children[0].name != "Subtract":
         return None
     a, b = f.children[0].children[0].children
-    if not (isinstance(a, O.Var) and isinstance(b, O.Var)) or a.dim != b.dim or not 32 <= a.dim <= 256:
+    if not (isinstance(a, O.Var) and isinstance(b, O.Var)) or a.dim != b.dim or not config.knn_min_dim <= a.dim <= 256:
         return None
     if {a.cat, b.cat} != {0, 1}:
         return None
@@ -156,21 +156,23 @@ def match_knn_sqdist(red, dtype, map_reduce_id):
 def generate_knn_plugin(red, rowvar, colvar, nargs):
     D = rowvar.dim
     dpad = -(-D // 16) * 16
+    # low dimensions: neighbours are close compared with the norms, the operands are split as hi + lo
+    split = int(D < 32)
     qsets, tj = config.knn_qsets, config.knn_tile_j
     # as many wavefronts as the LDS budget allows share one staged reference tile: the K-lists of the
     # 32*qsets queries of every wavefront live in LDS (8 bytes per entry)
-    fixed = tj * (dpad * 2 + 16) + tj * 4
+    fixed = tj * (dpad * 2 * (1 + split) + 16) + tj * 4
     waves = config.knn_max_waves
     while waves > 1 and fixed + waves * (32 * qsets * (red.K * 8 + 4) + 512) > config.knn_lds_budget:
         waves //= 2
     meta = dict(scheme="knn", block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
                 sizeof_acc=4, nrowvars=1, ncolvars=1, nparvars=0, knn_d=D, knn_dpad=dpad, knn_k=red.K,
                 knn_qb=waves * 32 * qsets, knn_fwaves=config.knn_filter_waves, knn_fqsets=config.knn_filter_qsets,
-                knn_sample=config.knn_sample, rowarg=rowvar.ind, colarg=colvar.ind)
+                knn_sample=config.knn_sample, knn_split=split, rowarg=rowvar.ind, colarg=colvar.ind)
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}", "typedef float T;"]
     defs = dict(KEOPS_NARGS=nargs, KNN_D=D, KNN_DPAD=dpad, KNN_K=red.K, KEOPS_RED_KEEP=red.keep, KEOPS_DIMOUT=red.dim,
                 KNN_QSETS=qsets, KNN_TJ=tj, KNN_WAVES=waves, KNN_FWAVES=config.knn_filter_waves,
-                KNN_FQSETS=config.knn_filter_qsets, KNN_SAMPLE=config.knn_sample)
+                KNN_FQSETS=config.knn_filter_qsets, KNN_SAMPLE=config.knn_sample, KNN_SPLIT=split)
     src += [f"#define {k} {v}" for k, v in defs.items()]
     src.append('#include "keops_knn_mfma.h"')
     return "\n".join(src) + "\n", meta

@@ -83,3 +83,40 @@ def test_knn_config3_query_subset():
     xq, yq = torch.from_numpy(x).cuda()[q], torch.from_numpy(y).cuda()[idx[q, 0]]
     d0 = ((xq.double() - yq.double()) ** 2).sum(1)
     assert torch.allclose(vals[q, 0].double(), d0, rtol=1e-5)
+
+
+@pytest.mark.parametrize("M,N,D,K", [(3000, 70000, 3, 10), (1500, 40000, 2, 4), (2000, 50000, 16, 50), (500, 900, 3, 10),
+                                     (1200, 33000, 7, 1)])
+def test_knn_low_dimension_split_operands(M, N, D, K):
+    """Dense point clouds (D < 32): the filter uses hi + lo bf16 operands; results stay bit-identical
+    to the CPU oracle, in the two-phase schedule (N >= 32768, M >= 1024) and in the adaptive one."""
+    rng = np.random.default_rng(11)
+    x = rng.random((M, D)).astype(np.float32)
+    y = rng.random((N, D)).astype(np.float32)
+    y[40] = y[5]
+    y[N - 1] = y[5]
+    x[1] = y[5]
+    x[2] = x[2] + 100.0  # an outlier query far from every reference
+    vals, idx = _knn(D, K)(*to_dev(x, y))
+    from keops_amd import keops_io
+
+    assert any(m.meta("scheme") == "knn" and m.meta("knn_split") == "1" for m in keops_io._modules.values())
+    ref = cpu_reduc("sqdist", [x, y], M, N, 1, reduction="KMin_ArgKMin", K=K, scheme="direct_sum")
+    assert np.array_equal(idx.cpu().numpy().reshape(M, K), ref[:, 1::2].astype(np.int64))
+    assert np.array_equal(vals.cpu().numpy().reshape(M, K), ref[:, 0::2])
+    if K >= 3:
+        assert idx[1, :3].tolist() == [5, 40, N - 1]
+
+
+def test_knn_low_dimension_clustered_far_from_origin():
+    """Tight clusters far from the origin: centring on the global mean leaves large norms compared
+    with the neighbour distances; the filter must stay complete (no missed neighbour)."""
+    rng = np.random.default_rng(12)
+    C, per, D, K = 40, 1000, 3, 8
+    centres = 100.0 * rng.random((C, D))
+    y = (np.repeat(centres, per, 0) + 0.01 * rng.standard_normal((C * per, D))).astype(np.float32)
+    x = (np.repeat(centres, 50, 0) + 0.01 * rng.standard_normal((C * 50, D))).astype(np.float32)
+    vals, idx = _knn(D, K)(*to_dev(x, y))
+    ref = cpu_reduc("sqdist", [x, y], x.shape[0], y.shape[0], 1, reduction="KMin_ArgKMin", K=K, scheme="direct_sum")
+    assert np.array_equal(idx.cpu().numpy(), ref[:, 1::2].astype(np.int64))
+    assert np.array_equal(vals.cpu().numpy(), ref[:, 0::2])
