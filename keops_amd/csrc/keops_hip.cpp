@@ -834,7 +834,9 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
       const int64_t v = e ? std::atoll(e) : 0;
       return v > 0 ? v : (int64_t)64;
     }();
-    const int64_t target_blocks = per_cu * (int64_t)m.cu_count;
+    // K-smallest lists restart empty in every slab (more insertions, 2K values per row and slab to merge):
+    // fewer, longer slabs for that family
+    const int64_t target_blocks = (m.meta_int("red_kind", 0) == 4 ? std::min<int64_t>(per_cu, 8) : per_cu) * (int64_t)m.cu_count;
     if (tag1D2D == 1 || row_blocks * 2 <= target_blocks) {
       const int64_t max_slabs = std::max<int64_t>(1, cols_total / 256);
       nslabs = std::min<int64_t>(max_slabs, (target_blocks + row_blocks - 1) / row_blocks);

@@ -102,7 +102,7 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
     meta = dict(
         scheme="conv", block=geo["block"], rows=geo["rows"], tile_j=geo["tile_j"], dimred=red.dimred, dimout=red.dim,
         sizeof_t=sizeof_t, sizeof_acc=8 if dtypeacc == "double" else 4, nrowvars=len(layout.rowvars),
-        ncolvars=len(layout.colvars), nparvars=len(layout.parvars), nops=nops,
+        ncolvars=len(layout.colvars), nparvars=len(layout.parvars), nops=nops, red_kind=red.kind,
     )
     src = []
     src.append("//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()))
