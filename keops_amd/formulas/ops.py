@@ -1283,6 +1283,140 @@ def TensorProd(a, b):
     return TensorProdNode(as_op(a), as_op(b))
 
 
+def _ints(t, what):
+    try:
+        return tuple(int(x) for x in t)
+    except TypeError:
+        raise FormulaError(f"TensorDot: {what} must be a list of integers") from None
+
+
+class TensorDotNode(Op):
+    """TensorDot(a, b, dimsfa, dimsfb, contfa, contfb[, permute]) (maths/TensorDot.py:51-140): a and b are
+    row-major tensors of shapes dimsfa / dimsfb; axes contfa of a are contracted with axes contfb of b
+    (paired in order); the result carries the kept axes of a, then those of b, and source axis k of
+    that result ends at position permute[k]."""
+
+    name = "TensorDot"
+    __slots__ = ()
+
+    def __init__(self, a, b, dimsfa, dimsfb, contfa, contfb, permute=None):
+        dimsfa, dimsfb = _ints(dimsfa, "dimsfa"), _ints(dimsfb, "dimsfb")
+        contfa, contfb = _ints(contfa, "contfa"), _ints(contfb, "contfb")
+        if math.prod(dimsfa) != a.dim or math.prod(dimsfb) != b.dim:
+            raise FormulaError("TensorDot: tensor shapes do not match the operand dimensions")
+        if len(contfa) != len(contfb) or [dimsfa[k] for k in contfa] != [dimsfb[k] for k in contfb]:
+            raise FormulaError("TensorDot: contracted axes do not match")
+        if len(set(contfa)) != len(contfa) or len(set(contfb)) != len(contfb):
+            raise FormulaError("TensorDot: repeated contraction axis")
+        keep_a = [k for k in range(len(dimsfa)) if k not in contfa]
+        keep_b = [k for k in range(len(dimsfb)) if k not in contfb]
+        nkeep = len(keep_a) + len(keep_b)
+        permute = tuple(range(nkeep)) if permute is None else _ints(permute, "permute")
+        if sorted(permute) != list(range(nkeep)):
+            raise FormulaError("TensorDot: permute must be a permutation of the kept axes")
+        dim = math.prod([dimsfa[k] for k in keep_a]) * math.prod([dimsfb[k] for k in keep_b])
+        super().__init__((a, b), (dimsfa, dimsfb, contfa, contfb, permute), dim)
+
+    def _layout(self):
+        dimsfa, dimsfb, contfa, contfb, permute = self.params
+        keep_a = [k for k in range(len(dimsfa)) if k not in contfa]
+        keep_b = [k for k in range(len(dimsfb)) if k not in contfb]
+        return dimsfa, dimsfb, list(contfa), list(contfb), list(permute), keep_a, keep_b
+
+    def out_shape(self):
+        dimsfa, dimsfb, _, _, permute, keep_a, keep_b = self._layout()
+        keep = [dimsfa[k] for k in keep_a] + [dimsfb[k] for k in keep_b]
+        shape = [0] * len(keep)
+        for k, dst in enumerate(permute):
+            shape[dst] = keep[k]
+        return tuple(shape)
+
+    def lower(self, L, kids):
+        import numpy as np
+
+        a, b = kids
+        dimsfa, dimsfb, contfa, contfb, permute, keep_a, keep_b = self._layout()
+        C = math.prod([dimsfa[k] for k in contfa])
+        ia = np.arange(len(a)).reshape(dimsfa or (1,)).transpose(keep_a + contfa).reshape(-1, C) if dimsfa else np.zeros((1, 1), int)
+        ib = np.arange(len(b)).reshape(dimsfb or (1,)).transpose(keep_b + contfb).reshape(-1, C) if dimsfb else np.zeros((1, 1), int)
+        res = np.empty((ia.shape[0], ib.shape[0]), dtype=object)
+        for r in range(ia.shape[0]):
+            for c in range(ib.shape[0]):
+                acc = None
+                for k in range(C):
+                    t = L.mul(a[int(ia[r, k])], b[int(ib[c, k])])
+                    acc = t if acc is None else L.add(acc, t)
+                res[r, c] = acc
+        keep = [dimsfa[k] for k in keep_a] + [dimsfb[k] for k in keep_b]
+        if keep:
+            axes = sorted(range(len(permute)), key=permute.__getitem__)  # destination axis i <- source axis axes[i]
+            res = res.reshape(keep).transpose(axes)
+        return [x for x in res.ravel()]
+
+    def diff_t(self, v, gradin):
+        a, b = self.children
+        dimsfa, dimsfb, contfa, contfb, permute, keep_a, keep_b = self._layout()
+        gshape = self.out_shape()
+        na = len(keep_a)
+
+        def part(wrt_a):
+            # d(first operand) = TensorDot(gradin, other): contract the gradient axes that came from the
+            # other operand with that operand's kept axes, then order the result like the operand itself
+            if wrt_a:
+                other, odims, okeep, ocont = b, dimsfb, keep_b, contfb
+                gcont = [permute[na + t] for t in range(len(keep_b))]
+                mine_keep, mine_cont, src0 = keep_a, contfa, 0
+            else:
+                other, odims, okeep, ocont = a, dimsfa, keep_a, contfa
+                gcont = [permute[t] for t in range(na)]
+                mine_keep, mine_cont, src0 = keep_b, contfb, na
+            gkeep = [p for p in range(len(gshape)) if p not in gcont]   # ascending positions of the gradient
+            orest = [k for k in range(len(odims)) if k not in okeep]     # = sorted(ocont)
+            perm = []
+            for p in gkeep:
+                s = permute.index(p) - src0    # which kept axis of my operand sits at gradient position p
+                perm.append(mine_keep[s])
+            for beta in orest:
+                perm.append(mine_cont[ocont.index(beta)])
+            return TensorDot(gradin, other, gshape, odims, gcont, okeep, perm)
+
+        return Add(a.diff_t(v, part(True)), b.diff_t(v, part(False)))
+
+
+def TensorDot(a, b, dimsfa, dimsfb, contfa, contfb, permute=None):
+    return TensorDotNode(as_op(a), as_op(b), dimsfa, dimsfb, contfa, contfb, permute)
+
+
+def Kron(a, b, dimsfa, dimsfb):
+    """Kronecker product as np.kron (maths/Kron.py): einsum('ij..,lm..->iljm..')."""
+    dimsfa, dimsfb = _ints(dimsfa, "dimsfa"), _ints(dimsfb, "dimsfb")
+    if len(dimsfa) != len(dimsfb):
+        raise FormulaError("Kron: both tensors must have the same number of axes")
+    n = len(dimsfa)
+    return TensorDot(a, b, dimsfa, dimsfb, (), (), tuple(range(0, 2 * n, 2)) + tuple(range(1, 2 * n, 2)))
+
+
+def SqNormIso(s, x):
+    """s |x|^2 (maths/SqNormIso.py)."""
+    return Mult(as_op(s), SqNorm2(x))
+
+
+def SqNormDiag(s, x):
+    """sum_k s_k x_k^2 (maths/SqNormDiag.py)."""
+    return Sum(Mult(as_op(s), Square(x)))
+
+
+def SymSqNorm(a, x):
+    """sum_ij a_ij x_i x_j (maths/SymSqNorm.py)."""
+    x = as_op(x)
+    return Sum(Mult(as_op(a), TensorProd(x, x)))
+
+
+def Ind(*k):
+    """Index list literal of the formula grammar, e.g. TensorDot(a, b, Ind(2,3), Ind(3,2), Ind(1), Ind(0))."""
+    return tuple(int(x) for x in k)
+
+
 # ----------------------------------------------------------------------------- registry
 
 BUILDERS = dict(
@@ -1294,6 +1428,7 @@ BUILDERS = dict(
     IfElse=IfElse, Clamp=Clamp, ClampInt=ClampInt, DiffClampInt=DiffClampInt, Mod=Mod, Sum=Sum, SumT=SumT,
     Scalprod=Scalprod, Concat=Concat, Extract=Extract, ExtractT=ExtractT, OneHot=OneHot, Max=Max, Min=Min,
     ArgMax=ArgMax, ArgMin=ArgMin, MatVecMult=MatVecMult, VecMatMult=VecMatMult, TensorProd=TensorProd,
+    TensorDot=TensorDot,
 )
 
 # names that only exist as constructors (they expand into the nodes above)
@@ -1301,6 +1436,7 @@ FUNCTIONS = dict(
     BUILDERS,
     Vi=Vi, Vj=Vj, Pm=Pm, IntInv=IntInv, SqNorm2=SqNorm2, Norm2=Norm2, SqDist=SqDist, Normalize=Normalize,
     WeightedSqNorm=WeightedSqNorm, WeightedSqDist=WeightedSqDist, Elem=Elem, ElemT=ElemT,
+    Kron=Kron, SqNormIso=SqNormIso, SqNormDiag=SqNormDiag, SymSqNorm=SymSqNorm, Ind=Ind,
 )
 
 

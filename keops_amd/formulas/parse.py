@@ -53,6 +53,12 @@ class _Builder(ast.NodeVisitor):
             return node.value
         raise FormulaError(f"unsupported literal {node.value!r}")
 
+    def visit_Tuple(self, node):
+        # index lists of TensorDot / Kron, e.g. (2, 3)
+        return tuple(self.visit(e) for e in node.elts)
+
+    visit_List = visit_Tuple
+
     def visit_Name(self, node):
         if node.id in self.names:
             return self.names[node.id]

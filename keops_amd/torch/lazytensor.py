@@ -372,6 +372,16 @@ class LazyTensor:
     def tensorprod(self, other):
         return self.binary(other, O.TensorProd)
 
+    def keops_tensordot(self, other, dimfa, dimfb, contfa, contfb, *args):
+        """Tensor contraction of the vectors of self and other viewed as tensors of shapes dimfa / dimfb,
+        like np.tensordot, with an optional final axis permutation (lazy_tensor.py "keops_tensordot")."""
+        permute = tuple(args[0]) if args else None
+        return self.binary(other, lambda a, b: O.TensorDot(a, b, tuple(dimfa), tuple(dimfb), tuple(contfa), tuple(contfb), permute))
+
+    def keops_kron(self, other, dimfself, dimfother):
+        """Kronecker product, as np.kron on tensors of shapes dimfself / dimfother (lazy_tensor.py "keops_kron")."""
+        return self.binary(other, lambda a, b: O.Kron(a, b, tuple(dimfself), tuple(dimfother)))
+
     def grad(self, other, gradin):
         """Symbolic gradient [d_other self]^T gradin (lazy_tensor.py "grad")."""
         other, gradin = self._lift(other), self._lift(gradin)

@@ -204,3 +204,38 @@ def test_parser_errors_and_aliases():
     assert (r.dim, r.dimred) == (2, 2)
     r = parse_reduction("Max_SumShiftExpWeight_Reduction(SqDist(x,y),1,Concat(IntCst(1),x))", ["x=Vi(3)", "y=Vj(3)"])
     assert (r.dim, r.tagI) == (5, 1)
+
+
+def test_tensordot_kron_and_quadratic_forms():
+    """TensorDot against torch.tensordot / einsum (values and gradients with respect to both operands,
+    cf. the reference's pykeops/test/test_lazytensor_tensordot.py cases), Kron against torch.kron."""
+    al = ["a=Vi(0,12)", "b=Vj(1,24)", "c=Vj(2,6)", "s=Vj(3,9)", "u=Vi(4,3)"]
+    t = [_t(M, 12), _t(N, 24), _t(N, 6), _t(N, 9), _t(M, 3)]
+
+    def A(a):
+        return a.expand(M, N, 12).reshape(M, N, 2, 2, 3)
+
+    def B(b):
+        return b.expand(M, N, 24).reshape(M, N, 2, 3, 4)
+
+    # contract the last two axes of a (2,2,3) with the first two of b (2,3,4): result (2,4)
+    _check("TensorDot(a, b, Ind(2,2,3), Ind(2,3,4), Ind(1,2), Ind(0,1))", al, t,
+           lambda a, b, c, s, u: torch.einsum("mnijk,mnjkl->mnil", A(a), B(b)).reshape(M, N, 8), (0, 1))
+    # crossed pairing (axis 0 of a with axis 0 of b, axis 2 with axis 1) and a permuted result (4,2) instead of (2,4)
+    _check("TensorDot(a, b, Ind(2,2,3), Ind(2,3,4), Ind(0,2), Ind(0,1), Ind(1,0))", al, t,
+           lambda a, b, c, s, u: torch.einsum("mnijk,mnikl->mnlj", A(a), B(b)).reshape(M, N, 8), (0, 1))
+    # no contraction: outer product with interleaved axes = Kronecker product of a (2,6) and c (2,3) matrix
+    _check("Kron(a, c, Ind(2,6), Ind(2,3))", al, t,
+           lambda a, b, c, s, u: torch.einsum("mnij,mnkl->mnikjl", a.expand(M, N, 12).reshape(M, N, 2, 6),
+                                              c.expand(M, N, 6).reshape(M, N, 2, 3)).reshape(M, N, 72), (0, 2))
+    # repr -> parse round trip (the LazyTensor front end passes repr(formula) to Genred)
+    op = parse("TensorDot(a, b, Ind(2,2,3), Ind(2,3,4), Ind(0,2), Ind(0,1), Ind(1,0))", al)
+    assert parse(repr(op)) == op
+    # quadratic forms
+    _check("SymSqNorm(s, u)", al, t,
+           lambda a, b, c, s, u: torch.einsum("mnij,mni,mnj->mn", s.expand(M, N, 9).reshape(M, N, 3, 3),
+                                              u.expand(M, N, 3), u.expand(M, N, 3))[..., None], (3, 4))
+    _check("SqNormDiag(Extract(s,0,3), u)+SqNormIso(Elem(s,4), u)", al, t,
+           lambda a, b, c, s, u: (s[..., :3] * u * u).sum(-1, keepdim=True) + s[..., 4:5] * (u * u).sum(-1, keepdim=True), (3, 4))
+    with pytest.raises(Exception):
+        parse("TensorDot(a, b, Ind(2,2,3), Ind(2,3,4), Ind(1), Ind(2))", al)

@@ -84,3 +84,24 @@ def test_lazytensor_ranges_and_symbolic_variables():
         (-(LazyTensor((0, 2, 0)) - LazyTensor((1, 2, 1))).sqnorm2()).exp().reduction("Sum", axis=1))
     out = f(x, x)
     assert torch.allclose(out[:, 0], torch.exp(-torch.cdist(x, x) ** 2).sum(1), rtol=1e-4)
+
+
+def test_tensordot_and_kron_lazytensors():
+    """Matrix-valued variables contracted per pair (cf. the reference's test_lazytensor_tensordot.py)."""
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(3)
+    M, N = 70, 90
+    a = torch.randn(M, 2 * 3, dtype=torch.float64, device="cuda", requires_grad=True)
+    b = torch.randn(N, 3 * 4, dtype=torch.float64, device="cuda")
+    A, B = LazyTensor(a[:, None, :]), LazyTensor(b[None, :, :])
+    out = A.keops_tensordot(B, (2, 3), (3, 4), (1,), (0,)).sum_reduction(dim=1)     # sum_j A_i @ B_j, (M, 8)
+    ref = torch.einsum("mik,nkl->mil", a.reshape(M, 2, 3), b.reshape(N, 3, 4)).reshape(M, 8)
+    assert torch.allclose(out, ref, rtol=1e-10, atol=1e-10)
+    e = torch.randn(M, 8, dtype=torch.float64, device="cuda")
+    (g,) = torch.autograd.grad((out * e).sum(), [a])
+    (gr,) = torch.autograd.grad((ref * e).sum(), [a])
+    assert torch.allclose(g, gr, rtol=1e-10, atol=1e-10)
+    k = A.keops_kron(B, (2, 3), (3, 4)).sum_reduction(dim=1)                           # (M, 6*12)
+    kref = torch.stack([torch.kron(a[i].reshape(2, 3), b.reshape(N, 3, 4).sum(0)) for i in range(M)]).reshape(M, 72)
+    assert torch.allclose(k, kref, rtol=1e-10, atol=1e-10)
