@@ -1451,3 +1451,46 @@ def Grad(formula, v, gradin=None):
 
 
 FUNCTIONS["Grad"] = Grad
+
+
+def _fresh_probe(dim, *formulas):
+    """A variable no formula contains, used as a symbolic cotangent that must vanish from the result."""
+    inds = [w.ind for f in formulas for w in f.variables]
+    return Var(1 + (max(inds) if inds else 0) + (1 << 20), dim, 3)
+
+
+def Diff(formula, v, u):
+    """Forward-mode differential D_v F . u (autodiff/Diff.py:14-34: the adjoint of the gradient map).
+    The gradient G(g) = [d_v F]^T g is linear in its cotangent g, so its adjoint applied to u is the gradient
+    of <G(g), u> with respect to g: reverse mode twice, and g drops out."""
+    formula, v, u = as_op(formula), as_op(v), as_op(u)
+    if not isinstance(v, Var) or u.dim != v.dim:
+        raise FormulaError("Diff(F, v, u): v must be a variable and u must have its dimension")
+    g = _fresh_probe(formula.dim, formula, v, u)
+    inner = Scalprod(formula.diff_t(v, g), u) if v.dim > 1 else Mult(formula.diff_t(v, g), u)
+    res = inner.diff_t(g, IntCst(1))
+    if g in res.variables:
+        raise FormulaError("Diff: the formula contains an operation whose gradient is not linear in its cotangent")
+    return res
+
+
+def Divergence(formula, v):
+    """Trace of the Jacobian of F with respect to v (autodiff/Divergence.py:15-37); dim(F) = dim(v)."""
+    formula, v = as_op(formula), as_op(v)
+    if formula.dim != v.dim:
+        raise FormulaError("Divergence requires formula and variable to have the same dimension.")
+    acc = Zero(1)
+    for k in range(v.dim):
+        acc = Add(acc, Elem(Diff(formula, v, ElemT(IntCst(1), v.dim, k)), k))
+    return acc
+
+
+def Laplacian(formula, v):
+    """Divergence of the gradient of a scalar formula (autodiff/Laplacian.py:16-23)."""
+    formula, v = as_op(formula), as_op(v)
+    if formula.dim != 1:
+        raise FormulaError("Laplacian is only implemented for scalar formula.")
+    return Divergence(formula.diff_t(v, IntCst(1)), v)
+
+
+FUNCTIONS.update(Diff=Diff, Divergence=Divergence, Laplacian=Laplacian)

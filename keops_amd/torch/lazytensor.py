@@ -372,6 +372,23 @@ class LazyTensor:
     def tensorprod(self, other):
         return self.binary(other, O.TensorProd)
 
+    def diff(self, other, diffin):
+        """Symbolic forward-mode differential [d_other self] . diffin (lazy_tensor.py "diff")."""
+        other, diffin = self._lift(other), self._lift(diffin)
+        if not isinstance(other.formula, O.Var):
+            raise ValueError("LazyTensor.diff expects a variable as its first argument")
+        return self._like(O.Diff(self.formula, other.formula, diffin.formula), other, diffin)
+
+    def divergence(self, other):
+        """Symbolic divergence with respect to the variable ``other`` (lazy_tensor.py "divergence")."""
+        other = self._lift(other)
+        return self._like(O.Divergence(self.formula, other.formula), other)
+
+    def laplacian(self, other):
+        """Symbolic Laplacian of a scalar formula with respect to ``other`` (lazy_tensor.py "laplacian")."""
+        other = self._lift(other)
+        return self._like(O.Laplacian(self.formula, other.formula), other)
+
     def keops_tensordot(self, other, dimfa, dimfb, contfa, contfb, *args):
         """Tensor contraction of the vectors of self and other viewed as tensors of shapes dimfa / dimfb,
         like np.tensordot, with an optional final axis permutation (lazy_tensor.py "keops_tensordot")."""

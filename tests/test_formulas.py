@@ -239,3 +239,31 @@ def test_tensordot_kron_and_quadratic_forms():
            lambda a, b, c, s, u: (s[..., :3] * u * u).sum(-1, keepdim=True) + s[..., 4:5] * (u * u).sum(-1, keepdim=True), (3, 4))
     with pytest.raises(Exception):
         parse("TensorDot(a, b, Ind(2,2,3), Ind(2,3,4), Ind(1), Ind(2))", al)
+
+
+def test_forward_mode_diff_divergence_laplacian():
+    """Diff (forward mode), Divergence and Laplacian against torch.func / closed forms."""
+    al = ["x=Vi(0,3)", "y=Vj(1,3)", "u=Vi(2,3)", "g=Pm(3,1)"]
+    a = [_t(M, 3), _t(N, 3), _t(M, 3), _t(1, lo=0.5, hi=1.5)]
+
+    def F(x, y, g):
+        return torch.exp(-g * ((x - y) ** 2).sum(-1, keepdim=True)) * (x + y)
+
+    def jvp(x, y, u, g):
+        xb, yb, ub = (t.expand(M, N, 3) for t in (x, y, u))
+        return torch.func.jvp(lambda z: F(z, yb, g), (xb,), (ub,))[1]
+
+    _check("Diff(Exp(-g*SqDist(x,y))*(x+y), x, u)", al, a, jvp)
+    # divergence of the vector field z -> exp(-g|z-y|^2)(z+y) at z = x
+    def div(x, y, u, g):
+        xb, yb = x.expand(M, N, 3).reshape(-1, 3), y.expand(M, N, 3).reshape(-1, 3)
+        J = torch.func.vmap(torch.func.jacrev(lambda z, w: F(z, w, g)))(xb, yb)
+        return torch.diagonal(J, dim1=-2, dim2=-1).sum(-1).reshape(M, N, 1)
+
+    _check("Divergence(Exp(-g*SqDist(x,y))*(x+y), x)", al, a, div)
+    # Laplacian of a Gaussian: (4 g^2 r^2 - 2 g D) exp(-g r^2)
+    def lap(x, y, u, g):
+        r2 = ((x - y) ** 2).sum(-1, keepdim=True)
+        return (4 * g * g * r2 - 6 * g) * torch.exp(-g * r2)
+
+    _check("Laplacian(Exp(-g*SqDist(x,y)), x)", al, a, lap)

@@ -105,3 +105,21 @@ def test_tensordot_and_kron_lazytensors():
     k = A.keops_kron(B, (2, 3), (3, 4)).sum_reduction(dim=1)                           # (M, 6*12)
     kref = torch.stack([torch.kron(a[i].reshape(2, 3), b.reshape(N, 3, 4).sum(0)) for i in range(M)]).reshape(M, 72)
     assert torch.allclose(k, kref, rtol=1e-10, atol=1e-10)
+
+
+def test_laplacian_and_diff_lazytensors():
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(4)
+    M, N = 60, 80
+    x = torch.randn(M, 3, dtype=torch.float64, device="cuda")
+    y = torch.randn(N, 3, dtype=torch.float64, device="cuda")
+    u = torch.randn(M, 3, dtype=torch.float64, device="cuda")
+    X, Y, U = LazyTensor(x[:, None, :]), LazyTensor(y[None, :, :]), LazyTensor(u[:, None, :])
+    K = (-((X - Y) ** 2).sum(-1)).exp()
+    lap = K.laplacian(X).sum_reduction(dim=1)
+    r2 = torch.cdist(x, y) ** 2
+    assert torch.allclose(lap, ((4 * r2 - 6) * torch.exp(-r2)).sum(1, keepdim=True), rtol=1e-10, atol=1e-10)
+    d = K.diff(X, U).sum_reduction(dim=1)      # sum_j <grad_x K(x_i, y_j), u_i>
+    ref = (torch.exp(-r2)[:, :, None] * (-2 * (x[:, None, :] - y[None, :, :])) * u[:, None, :]).sum((1, 2))
+    assert torch.allclose(d[:, 0], ref, rtol=1e-10, atol=1e-10)
