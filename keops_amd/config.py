@@ -45,10 +45,20 @@ knn_lds_budget = 150 * 1024                                        # LDS bytes a
 knn_qsets = int(os.environ.get("KEOPS_AMD_KNN_QSETS", 1))          # 32-query operand sets per wavefront (<= 2)
 
 
+_build_folder = None
+
+
 def get_build_folder():
-    folder = os.environ.get("KEOPS_AMD_CACHE") or os.path.join(_PKG, "build")
+    folder = _build_folder or os.environ.get("KEOPS_AMD_CACHE") or os.path.join(_PKG, "build")
     os.makedirs(folder, exist_ok=True)
     return folder
+
+
+def set_build_folder(path=None):
+    """Folder of the on-disk cache of compiled kernel modules; None restores the default."""
+    global _build_folder
+    _build_folder = None if path is None else os.path.abspath(path)
+    return get_build_folder()
 
 
 def message(*args, **kwargs):

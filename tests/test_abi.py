@@ -100,3 +100,26 @@ def test_genred_front_end_host_logic():
             self.shape = s
 
     assert get_sizes(["x=Vi(3)", "y=Vj(3)", "p=Pm(1)"], T(5, 3), T(7, 3), T(1)) == (5, 7)
+
+
+def test_cache_folder_controls(tmp_path):
+    """set_build_folder / clean_keops_amd (pykeops.set_build_folder, clean_pykeops): modules are compiled
+    into the chosen folder (cross-compilation needs no GPU) and removed again."""
+    import os
+
+    import keops_amd
+    from keops_amd.get_keops_dll import get_keops_dll
+
+    os.environ.setdefault("KEOPS_HIP_ARCH", "gfx950")
+    default = keops_amd.get_build_folder()
+    try:
+        folder = keops_amd.set_build_folder(str(tmp_path / "cache"))
+        assert folder == keops_amd.get_build_folder() and os.path.isdir(folder)
+        al = ["x=Var(0,2,0)", "y=Var(1,2,1)"]
+        r = get_keops_dll("GpuReduc1D", "Sum_Reduction(SqDist(x,y),0)", 1, -1, 0, al, 2, "float", "float", "block_sum",
+                          1, 1, 0, False, True, 0)
+        assert r[2].startswith(folder) and os.path.exists(r[2])
+        assert keops_amd.clean_keops_amd() >= 1
+        assert not os.path.exists(r[2])
+    finally:
+        assert keops_amd.set_build_folder(None) == default
