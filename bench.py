@@ -168,12 +168,13 @@ def cpu_baseline(name, inp):
     except Exception:
         threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     lib()
-    # calibrate on 64 rows, then size the sample for about 10 s of CPU work
-    rows = np.arange(64, dtype=np.int64)
+    # calibrate on 64 rows per thread, then size the sample for about 12 s of CPU work
+    ncal = int(min(M, 64 * max(1, threads)))
+    rows = np.arange(ncal, dtype=np.int64)
     t0 = time.perf_counter()
     cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
-    rate = 64 * N / (time.perf_counter() - t0)
-    nrows = int(min(M, max(256, (10.0 * rate / N) // 256 * 256)))
+    rate = ncal * N / (time.perf_counter() - t0)
+    nrows = int(min(M, max(256, (12.0 * rate / N) // 256 * 256)))
     rows = np.sort(np.random.default_rng(0).choice(M, nrows, replace=False)).astype(np.int64)
     t0 = time.perf_counter()
     cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
