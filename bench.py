@@ -51,6 +51,7 @@ WORKLOADS = {
     "gauss_1m_dv8": ("Gaussian kernel sum 1e6 x 1e6, D=3, Dv=8, float32 (BASELINE config 2)", 28, "valu"),
     "gauss_1m_grad": ("gradient wrt x of the Gaussian kernel sum 1e6 x 1e6, D=3, Dv=1 (BASELINE config 2)", 21, "valu"),
     "gauss_10k": ("Gaussian kernel sum 1e4 x 1e4, D=3, Dv=1, float32 (BASELINE config 1)", 14, "valu"),
+    "gauss_100k": ("Gaussian kernel sum 1e5 x 1e5, D=3, Dv=1, float32 (reference benchmarks/README.md:13)", 14, "valu"),
     # 2*D flop of the <x,y> contraction per pair (the matrix-core work); filter and re-rank are not counted
     "knn_d64": ("KMin_ArgKMin K=10, 1e5 queries x 1e6 references, D=64 (BASELINE config 3)", 128, "mfma"),
     "sparse_100x10k": ("block-sparse Gaussian sum, 100 clusters x 10,000 points (BASELINE config 4)", 14, "valu"),
@@ -65,8 +66,8 @@ WORKLOADS = {
 def _np_inputs(name):
     import numpy as np
 
-    if name.startswith("gauss_1m") or name in ("gauss_10k", "gauss_dv256"):
-        M = N = 10_000 if name == "gauss_10k" else (200_000 if name == "gauss_dv256" else 1_000_000)
+    if name.startswith("gauss_1m") or name in ("gauss_10k", "gauss_100k", "gauss_dv256"):
+        M = N = {"gauss_10k": 10_000, "gauss_100k": 100_000, "gauss_dv256": 200_000}.get(name, 1_000_000)
         Dv = 8 if name.endswith("dv8") else (256 if name == "gauss_dv256" else 1)
         rng = np.random.default_rng(0 if name == "gauss_10k" else 1)
         x = rng.standard_normal((M, 3)).astype(np.float32)
