@@ -59,7 +59,7 @@ def test_cross_compilation_and_module_file_format(formula, aliases, expected_sch
 
 
 def test_metadata_tuple_matches_reference_conventions():
-    """dimx/dimy/indices as get_keops_dll.py:139-159 returns them (worked values of SURVEY 8a)."""
+    """dimx/dimy/indices as get_keops_dll.py:139-159 returns them."""
     al = ["x=Var(0,3,0)", "y=Var(1,3,1)", "b=Var(2,8,1)", "g=Var(3,1,2)"]
     r = get_keops_dll("GpuReduc1D", "Sum_Reduction(Exp(-g*SqDist(x,y))*b,0)", 1, -1, 0, al, 4, "float", "float",
                       "block_sum", 1, 1, 0, False, True, 0)

@@ -43,7 +43,7 @@ def test_laplace_chunked_vs_oracle(M, N, D, Dv):
 
 
 def test_config5b_laplace_d256_row_subset():
-    # BASELINE config 5b: M=N=200,000, D=256, Dv=16, x,y ~ N(0,1/D), seed 5
+    # headline configuration 5b: M=N=200,000, D=256, Dv=16, x,y ~ N(0,1/D), seed 5
     M = N = 200_000
     from keops_amd.torch import Genred
 

@@ -28,7 +28,7 @@ def _genred_gauss(Dv, **kw):
 
 
 def test_config1_gaussian_10k_full_parity():
-    # BASELINE config 1: M=N=10,000, D=3, float32, seed 0
+    # headline configuration 1: M=N=10,000, D=3, float32, seed 0
     M = N = 10000
     x, y, b, g = _gauss_inputs(M, N, 1, 0)
     got = _genred_gauss(1)(*to_dev(x, y, b, g)).cpu().numpy()
@@ -49,7 +49,7 @@ def test_ragged_sizes(M, N, Dv):
 
 @pytest.mark.parametrize("Dv", [1, 8])
 def test_config2_gaussian_1M_row_subset(Dv):
-    # BASELINE config 2: M=N=1,000,000, seed 1; oracle on 2048 random rows (rows are independent)
+    # headline configuration 2: M=N=1,000,000, seed 1; oracle on 2048 random rows (rows are independent)
     M = N = 1_000_000
     x, y, b, g = _gauss_inputs(M, N, Dv, 1)
     got = _genred_gauss(Dv)(*to_dev(x, y, b, g))

@@ -62,7 +62,7 @@ def test_knn_gaussian_uncentred_data_and_axis0():
 
 
 def test_knn_config3_query_subset():
-    # BASELINE config 3: M=100,000 queries, N=1,000,000 references, D=64, K=10, U[0,1), seed 2
+    # headline configuration 3: M=100,000 queries, N=1,000,000 references, D=64, K=10, U[0,1), seed 2
     M, N, D, K = 100_000, 1_000_000, 64, 10
     rng = np.random.default_rng(2)
     x = rng.random((M, D), dtype=np.float32)
