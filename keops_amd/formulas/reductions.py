@@ -156,6 +156,19 @@ def Grad_WithSavedForward(red, v, gradin, f0):
     return red.diff_t(v, gradin, f0)
 
 
+def Diff_WithSavedForward(red, v, u, f0):
+    """Forward-mode differential of a reduction (autodiff/Diff_WithSavedForward.py): the differential
+    of a sum is the sum of the differentials, indexed like the original output."""
+    if isinstance(red, Zero_Reduction):
+        return Zero_Reduction(red.dim, red.tagI)
+    if not isinstance(red, Sum_Reduction):
+        raise NotImplementedError(f"forward-mode differentiation through {red.string_id} is not supported")
+    d = ops.Diff(red.formula, v, u)
+    if isinstance(d, Zero):
+        return Zero_Reduction(red.dim, red.tagI)
+    return Sum_Reduction(d, red.tagI)
+
+
 REDUCTIONS = dict(
     Sum_Reduction=Sum_Reduction, Zero_Reduction=Zero_Reduction,
     Max_SumShiftExp_Reduction=Max_SumShiftExp_Reduction,
@@ -164,4 +177,5 @@ REDUCTIONS = dict(
     Max_ArgMax_Reduction=Max_ArgMax_Reduction, Max_Reduction=Max_Reduction, ArgMax_Reduction=ArgMax_Reduction,
     KMin_ArgKMin_Reduction=KMin_ArgKMin_Reduction, KMin_Reduction=KMin_Reduction,
     ArgKMin_Reduction=ArgKMin_Reduction, Grad_WithSavedForward=Grad_WithSavedForward,
+    Diff_WithSavedForward=Diff_WithSavedForward,
 )

@@ -87,6 +87,7 @@ class GenredAutograd_base:
         ctx.params = params
         ctx.dimout, ctx.tagIJ = int(info[0]), int(info[1])
         ctx.save_for_backward(*args, result)
+        ctx.save_for_forward(*args, result)
 
     @staticmethod
     def _backward(ctx, G, _):
@@ -131,8 +132,46 @@ class GenredAutograd_base:
         return (None, *grads)
 
 
+def _jvp(ctx, *tangents):
+    """Forward-mode rule (generic_red.py:318-380): the output tangent is the sum over the inputs that carry
+    a tangent of Genred("Diff_WithSavedForward(F, v, eta, result)") evaluated at (args, tangent, result)."""
+    params, dimout, tagIJ = ctx.params, ctx.dimout, ctx.tagIJ
+    args = ctx.saved_tensors[:-1]
+    nargs = len(args)
+    result = ctx.saved_tensors[-1].detach()
+    check_AD_supported(params.formula)
+    resvar = f"Var({nargs + 1},{dimout},{tagIJ})"
+    out = 0
+    for var_ind, sig in enumerate(params.aliases):
+        u = tangents[var_ind + 1]
+        if u is None:
+            continue
+        _, cat, dim, pos = get_type(sig, position_in_list=var_ind)
+        eta = f"Var({nargs},{dim},{cat})"
+        params_d = copy.copy(params)
+        params_d.formula = f"Diff_WithSavedForward({params.formula},Var({pos},{dim},{cat}),{eta},{resvar})"
+        params_d.aliases = params.aliases + [eta, resvar]
+        params_d.out = None
+        params_d.rec_multVar_highdim = None
+        out = out + GenredAutograd_fun(params_d, *args, u.contiguous(), result)
+    return out, None
+
+
 class GenredAutograd(torch.autograd.Function):
     """Entry point to the torch autograd engine (generic_red.py:262-302)."""
+
+    @staticmethod
+    def jvp(ctx, *tangents):
+        return _jvp(ctx, *tangents)
+
+    @staticmethod
+    def vmap(info, in_dims, params, *args):
+        # the vmapped axis becomes a leading batch dimension (generic_red.py:304-316); arguments that are
+        # not vmapped get a batch dimension of size 1, which broadcasts
+        args = [a[None, ...] if d is None else a.movedim(d, 0).contiguous() for a, d in zip(args, in_dims[1:])]
+        p = copy.copy(params)
+        p.out = None
+        return GenredAutograd.apply(p, *args), (0, None)
 
     @staticmethod
     def forward(*inputs):

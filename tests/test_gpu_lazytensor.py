@@ -123,3 +123,38 @@ def test_laplacian_and_diff_lazytensors():
     d = K.diff(X, U).sum_reduction(dim=1)      # sum_j <grad_x K(x_i, y_j), u_i>
     ref = (torch.exp(-r2)[:, :, None] * (-2 * (x[:, None, :] - y[None, :, :])) * u[:, None, :]).sum((1, 2))
     assert torch.allclose(d[:, 0], ref, rtol=1e-10, atol=1e-10)
+
+
+def test_forward_mode_jvp_through_genred():
+    """torch.func.jvp through a Sum reduction (cf. the reference's pykeops/test/test_torch_func.py)."""
+    from keops_amd.torch import Genred
+
+    torch.manual_seed(5)
+    M, N = 50, 70
+    x = torch.randn(M, 3, dtype=torch.float64, device="cuda")
+    y = torch.randn(N, 3, dtype=torch.float64, device="cuda")
+    b = torch.randn(N, 2, dtype=torch.float64, device="cuda")
+    ux, ub = torch.randn_like(x), torch.randn_like(b)
+    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)"], reduction_op="Sum", axis=1)
+
+    def dense(x_, b_):
+        return torch.exp(-((x_[:, None, :] - y[None, :, :]) ** 2).sum(-1)) @ b_
+
+    out, tan = torch.func.jvp(lambda x_, b_: conv(x_, y, b_), (x, b), (ux, ub))
+    ref, rtan = torch.func.jvp(dense, (x, b), (ux, ub))
+    assert torch.allclose(out, ref, rtol=1e-10, atol=1e-10)
+    assert torch.allclose(tan, rtan, rtol=1e-10, atol=1e-10)
+
+
+def test_vmap_through_genred():
+    from keops_amd.torch import Genred
+
+    torch.manual_seed(6)
+    B, M, N = 5, 40, 60
+    xs = torch.randn(B, M, 3, dtype=torch.float64, device="cuda")
+    y = torch.randn(N, 3, dtype=torch.float64, device="cuda")
+    b = torch.randn(N, 2, dtype=torch.float64, device="cuda")
+    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)"], reduction_op="Sum", axis=1)
+    out = torch.func.vmap(lambda x_: conv(x_, y, b))(xs)
+    ref = torch.exp(-((xs[:, :, None, :] - y[None, None, :, :]) ** 2).sum(-1)) @ b
+    assert out.shape == (B, M, 2) and torch.allclose(out, ref, rtol=1e-10, atol=1e-10)
