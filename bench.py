@@ -58,6 +58,9 @@ WORKLOADS = {
     "lse_b16": ("batched LogSumExp softmin B=16, 50,000 x 50,000, D=3 (BASELINE config 5a)", 17, "valu"),
     # 2*D flop of the contraction + sqrt, neg, exp + 2*Dv of the weighted accumulation
     "laplace_d256": ("Laplace kernel sum 2e5 x 2e5, D=256, Dv=16 (BASELINE config 5b)", 547, "mfma"),
+    # softmax-weighted sum of an inner product (attention-like).  Counted: exp + 2*Dv of the weighted sum, which runs
+    # on the float32 matrix cores and dominates; the 2*D*3 bf16 flop of the scores are not counted
+    "softmax_d64": ("SumSoftMaxWeight of <q,k> with 64-dimensional weights, 65536 x 65536, D=64", 130, "mfma32"),
     # 12 flop of the Gaussian kernel + 2*Dv of the product with the 256-dimensional variable (float32 matrix cores)
     "gauss_dv256": ("Gaussian kernel times a 256-dimensional variable, 2e5 x 2e5, D=3 (final-product scheme)", 524, "mfma32"),
 }
@@ -78,6 +81,12 @@ def _np_inputs(name):
         M, N, D = 100_000, 1_000_000, 64
         rng = np.random.default_rng(2)
         return dict(M=M, N=N, Dv=0, D=D, arrays=[rng.random((M, D), dtype=np.float32), rng.random((N, D), dtype=np.float32)])
+    if name == "softmax_d64":
+        M = N = 65_536
+        rng = np.random.default_rng(6)
+        q = (rng.standard_normal((M, 64)) / 64 ** 0.25).astype(np.float32)
+        k = (rng.standard_normal((N, 64)) / 64 ** 0.25).astype(np.float32)
+        return dict(M=M, N=N, Dv=64, D=64, arrays=[q, k, rng.standard_normal((N, 64)).astype(np.float32)])
     if name == "laplace_d256":
         M = N = 200_000
         rng = np.random.default_rng(5)
@@ -115,6 +124,9 @@ def build_step(name):
     if name == "knn_d64":
         knn = Genred("SqDist(x,y)", ["x=Vi(64)", "y=Vj(64)"], reduction_op="KMin_ArgKMin", axis=1, opt_arg=10)
         return (lambda: knn(*dev)), M * N, inp
+    if name == "softmax_d64":
+        att = Genred("(q|k)", ["q=Vi(64)", "k=Vj(64)", "v=Vj(64)"], reduction_op="SumSoftMaxWeight", axis=1, formula2="v")
+        return (lambda: att(*dev)), M * N, inp
     if name == "laplace_d256":
         lap = Genred("Exp(-Norm2(x-y))*b", ["x=Vi(256)", "y=Vj(256)", "b=Vj(16)"], reduction_op="Sum", axis=1)
         return (lambda: lap(*dev)), M * N, inp

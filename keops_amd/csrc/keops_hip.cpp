@@ -497,7 +497,8 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   const size_t o_xn = take((size_t)nx * 4), o_yn = take((size_t)ny * 4);
   // final-product variant: slabs over the reduced axis fill the chip and round the grid to whole
   // rounds of workgroups (one 8-wavefront workgroup per CU, all taking the same time)
-  const bool final = m.meta_int("chk_final", 0) != 0;
+  const bool softmax = m.meta_int("chk_softmax", 0) != 0;
+  const bool final = m.meta_int("chk_final", 0) != 0 || softmax;
   const int64_t row_blocks = (nx + QB - 1) / QB, TJ = m.tile_j;
   int64_t nslabs = 1, slab_len = std::max<int64_t>(TJ, (ny + TJ - 1) / TJ * TJ);
   if (final) {
@@ -512,7 +513,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
     slab_len = std::max<int64_t>(TJ, ((ny + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ);
     nslabs = std::max<int64_t>(1, (ny + slab_len - 1) / slab_len);
   }
-  const size_t o_part = take(final && nslabs > 1 ? (size_t)nslabs * nx * m.dimout * 4 : 0);
+  const size_t o_part = take(final && nslabs > 1 ? (size_t)nslabs * nx * m.dimred * 4 : 0);
   if (int rc = m.partial.reserve(off)) return rc;
   char* ws = (char*)m.partial.ptr;
   std::vector<char> buf(sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 8);
@@ -536,14 +537,14 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (int rc = launch_raw(m, "keops_chk_prep", (unsigned)((ny * lpr + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
   if (final) {
-    if (int rc = launch_raw(m, "keops_chk_final", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)m.block, buf.data(), psize, stream)) return rc;
+    if (int rc = launch_raw(m, softmax ? "keops_chk_softmax" : "keops_chk_final", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)m.block, buf.data(), psize, stream)) return rc;
   } else {
     if (int rc = launch_raw(m, "keops_chk_main", (unsigned)row_blocks, 1, (unsigned)m.block, buf.data(), psize, stream)) return rc;
   }
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
   if (final && nslabs > 1) {
-    const int64_t gb = (nx * m.dimout + 255) / 256;
-    if (int rc = launch_raw(m, "keops_chk_reduce", (unsigned)gb, 1, 256, buf.data(), psize, stream)) return rc;
+    const int64_t gb = (nx * m.dimred + 255) / 256;
+    if (int rc = launch_raw(m, softmax ? "keops_chk_softmax_reduce" : "keops_chk_reduce", (unsigned)gb, 1, 256, buf.data(), psize, stream)) return rc;
   }
   return 0;
 }

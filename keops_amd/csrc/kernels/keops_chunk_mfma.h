@@ -172,7 +172,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
 
 // ---- main kernel --------------------------------------------------------------------------------
 
-#if !(defined(CHK_FINAL) && CHK_FINAL)
+#if !(defined(CHK_FINAL) && CHK_FINAL) && !(defined(CHK_SOFTMAX) && CHK_SOFTMAX)
 extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const ChkParams P) {
   __shared__ __attribute__((aligned(16))) unsigned char as[CHK_TJ * CHK_STRIDE];  // A tile (hi|lo)
   __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
@@ -503,6 +503,234 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_reduce(const ChkPara
   if (e >= total) return;
   T s = P.partial[e];
   for (int k = 1; k < P.nslabs; k++) s += P.partial[(i64)k * total + e];
+  P.out[e] = s;
+}
+#endif
+
+// ---- variant for softmax-weighted sums (online log-sum-exp with the weighted sum on the matrix cores) ----
+//
+// Max_SumShiftExpWeight reduction whose post-chunk formulas are F'(s, ...) (scalar) and a weight that is
+// a plain reduced-index variable v_j, optionally preceded by a constant 1 (the SumSoftMaxWeight layout
+// [1, v_j] of the Python layer):   m_i = max_j F'_ij,   l_i = sum_j exp(F'_ij - m_i),
+// O_i = sum_j exp(F'_ij - m_i) v_j.  Per 32-row tile and wavefront: the running maximum of every output
+// row moves up (tile maximum over the lane's 16 values and its partner lane), the 32 x 32 float32 output
+// tiles and l are rescaled by exp(m_old - m_new) when any maximum of the wavefront moved (the factors
+// travel through LDS to the accumulator layout), then p = exp(F' - m_new) is the A operand of
+// v_mfma_f32_32x32x2_f32 against the staged v tile, exactly as in keops_chk_final.
+#if defined(CHK_SOFTMAX) && CHK_SOFTMAX
+#define CHK_SVS (CHK_FNB * 32)
+
+extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const ChkParams P) {
+  __shared__ __attribute__((aligned(16))) unsigned char as[CHK_TJ * CHK_STRIDE];
+  __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
+  __shared__ __attribute__((aligned(16))) T yo_s[CHK_TJ * CHK_DY];
+  __shared__ __attribute__((aligned(16))) T bt[CHK_TJ * CHK_SVS];
+  __shared__ __attribute__((aligned(16))) float al_s[CHK_WAVES][32];  // rescaling factors of a wavefront's rows
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const i64 row0 = (i64)blockIdx.x * CHK_QB + wave * 32;
+  i64 q = row0 + col;
+  if (q >= P.nx) q = P.nx - 1;
+
+  chk_bf16x8 bh[CHK_KB], bl[CHK_KB];
+#pragma unroll
+  for (int kb = 0; kb < CHK_KB; kb++) {
+    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + kb * 16 + 8 * half);
+    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+  }
+  const float xnq = CHK_MODE == 0 ? P.xn[q] : 0.f;
+  T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
+#pragma unroll
+  for (int v = 0; v < KEOPS_NROWVARS; v++) {
+    const T* src = P.arg[keops_row_arg[v]] + q * keops_row_dim[v];
+#pragma unroll
+    for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
+  }
+  T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+#pragma unroll
+  for (int v = 0; v < KEOPS_NPARVARS; v++) {
+    const T* src = P.arg[keops_par_arg[v]];
+#pragma unroll
+    for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
+  }
+
+  chk_f32x16 acc[CHK_FNB];
+#pragma unroll
+  for (int b = 0; b < CHK_FNB; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[b][r] = 0.f;
+  const float ninf = -__builtin_huge_valf();
+  float m_run = ninf;   // running maximum of output row `col` (identical in both halves)
+  float l_run = 0.f;    // this lane's share of sum_j exp(F' - m_run)
+
+  const i64 jbeg = (i64)blockIdx.y * P.slab_len;
+  const i64 jend = keops_min(P.ny, jbeg + P.slab_len);
+  const T* vsrc = P.arg[CHK_FV_ARG];
+
+  constexpr int CH = CHK_ROWBYTES / 16;
+  constexpr int NPF = (CHK_TJ * CH + CHK_BLOCK - 1) / CHK_BLOCK;
+  constexpr int NPV = (CHK_TJ * CHK_SVS + CHK_BLOCK - 1) / CHK_BLOCK;
+  uint4 pf[NPF];
+  T pfv[NPV];
+  float pfn = 0.f;
+  auto prefetch = [&](i64 j0) {
+    const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
+    const uint4* src = reinterpret_cast<const uint4*>(P.ys + j0 * 2 * CHK_DPAD);
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * CHK_BLOCK;
+      pf[u] = (e < n * CH) ? src[e] : make_uint4(0u, 0u, 0u, 0u);
+    }
+    if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[j0 + tid] : 0.f;
+#pragma unroll
+    for (int u = 0; u < NPV; u++) {
+      const int e = tid + u * CHK_BLOCK;
+      const int row = e / CHK_SVS, c = e - row * CHK_SVS;
+      pfv[u] = (row < n && c < CHK_FV_DIM) ? vsrc[(j0 + row) * CHK_FV_DIM + c] : (T)0;
+    }
+  };
+  if (jbeg < jend) prefetch(jbeg);
+  for (i64 j0 = jbeg; j0 < jend; j0 += CHK_TJ) {
+    const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * CHK_BLOCK;
+      if (e < CHK_TJ * CH) {
+        const int row = e / CH, c = e - row * CH;
+        *reinterpret_cast<uint4*>(as + row * CHK_STRIDE + c * 16) = pf[u];
+      }
+    }
+    if (CHK_MODE == 0 && tid < CHK_TJ) yn_s[tid] = pfn;
+#pragma unroll
+    for (int v = 0; v < KEOPS_NCOLVARS; v++) {
+      const int dim = keops_col_dim[v];
+      const T* src = P.arg[keops_col_arg[v]] + j0 * dim;
+      for (int e = tid; e < n * dim; e += CHK_BLOCK) {
+        const int row = e / dim, c = e - row * dim;
+        yo_s[row * CHK_DY + keops_col_off[v] + c] = src[e];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NPV; u++) {
+      const int e = tid + u * CHK_BLOCK;
+      if (e < CHK_TJ * CHK_SVS) bt[e] = pfv[u];
+    }
+    __syncthreads();
+    if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ);
+
+    chk_f32x16 s;
+    if (CHK_MODE == 0) {
+      chk_f32x4 kk[4];
+#pragma unroll
+      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const chk_f32x4*>(yn_s + 8 * b + 4 * half);
+#pragma unroll
+      for (int v = 0; v < 16; v++) s[v] = kk[v >> 2][v & 3];
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; v++) s[v] = 0.f;
+    }
+    const unsigned char* arow = as + col * CHK_STRIDE + 16 * half;
+#pragma unroll
+    for (int kb = 0; kb < CHK_KB; kb++) {
+      const chk_bf16x8 ah = *reinterpret_cast<const chk_bf16x8*>(arow + kb * 32);
+      const chk_bf16x8 al = *reinterpret_cast<const chk_bf16x8*>(arow + CHK_DPAD * 2 + kb * 32);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
+    }
+    // F' for the lane's 16 pairs (rows past the end: -inf, they weigh nothing) and the tile maximum
+    float mx = ninf;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int r = 8 * (v >> 2) + 4 * half + (v & 3);
+      T sv = s[v];
+      if (CHK_MODE == 0) sv = __builtin_fmaxf(sv + xnq, 0.f);
+      T yj[CHK_DY];
+      constexpr int VEC = 16 / sizeof(T);
+      typedef T vecT __attribute__((ext_vector_type(VEC)));
+#pragma unroll
+      for (int c4 = 0; c4 < KEOPS_DIMY_PAD / VEC; c4++) {
+        const vecT w = *reinterpret_cast<const vecT*>(yo_s + r * CHK_DY + c4 * VEC);
+#pragma unroll
+        for (int c = 0; c < VEC; c++) yj[c4 * VEC + c] = w[c];
+      }
+      T fout[1];
+      KeopsFormula::eval(xi, yj, p, sv, fout);
+      s[v] = r < n ? fout[0] : ninf;
+      mx = __builtin_fmaxf(mx, s[v]);
+    }
+    mx = __builtin_fmaxf(mx, __shfl_xor(mx, 32));  // the partner lane holds the other 16 reduced rows of this output row
+    const float m_new = __builtin_fmaxf(__builtin_fmaxf(m_run, mx), -3.0e38f);
+    if (__any(m_new != m_run)) {
+      // rescale: alpha_i = exp(m_old - m_new) for the rows of this wavefront, moved to the accumulator layout
+      const float alpha = keops_red_exp(m_run - m_new);
+      l_run *= alpha;
+      volatile float* aw = al_s[wave];
+      if (half == 0) aw[col] = alpha;
+      __threadfence_block();
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const float a = aw[8 * (r >> 2) + 4 * half + (r & 3)];
+#pragma unroll
+        for (int b = 0; b < CHK_FNB; b++) acc[b][r] *= a;
+      }
+      __threadfence_block();
+      m_run = m_new;
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int r = 8 * (v >> 2) + 4 * half + (v & 3);
+      const float pv = keops_red_exp(s[v] - m_run);
+      l_run += pv;
+#pragma unroll
+      for (int b = 0; b < CHK_FNB; b++)
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(pv, bt[r * CHK_SVS + 32 * b + col], acc[b], 0, 0, 0);
+    }
+  }
+
+  // results of this slab: [m, (l,) O_0 .. O_{dv-1}] per output row
+  l_run += __shfl_xor(l_run, 32);
+  T* dst = P.nslabs > 1 ? P.partial + (i64)blockIdx.y * P.nx * KEOPS_DIMRED : P.out;
+  if (half == 0 && row0 + col < P.nx) {
+    T* o = dst + (row0 + col) * KEOPS_DIMRED;
+    o[0] = m_run;
+    if (CHK_SM_ONE) o[1] = l_run;
+  }
+  {
+    const i64 ibase = row0 + 4 * half;
+    T* o = dst + ibase * KEOPS_DIMRED + 1 + CHK_SM_ONE + col;
+#pragma unroll
+    for (int b = 0; b < CHK_FNB; b++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int ir = 8 * (r >> 2) + (r & 3);
+        if (ibase + ir < P.nx && 32 * b + col < CHK_FV_DIM) o[(i64)ir * KEOPS_DIMRED + 32 * b] = acc[b][r];
+      }
+    }
+  }
+}
+
+// merges the per-slab (m, s) results in slab order: m = max_k m_k, s = sum_k exp(m_k - m) s_k
+extern "C" __global__ void __launch_bounds__(256) keops_chk_softmax_reduce(const ChkParams P) {
+  const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
+  const i64 total = P.nx * KEOPS_DIMRED;
+  if (e >= total) return;
+  const i64 i = e / KEOPS_DIMRED;
+  const int c = (int)(e - i * KEOPS_DIMRED);
+  float m = -__builtin_huge_valf();
+  for (int k = 0; k < P.nslabs; k++) m = __builtin_fmaxf(m, P.partial[(i64)k * total + i * KEOPS_DIMRED]);
+  if (c == 0) {
+    P.out[e] = m;
+    return;
+  }
+  const float mm = __builtin_fmaxf(m, -3.0e38f);
+  float s = 0.f;
+  for (int k = 0; k < P.nslabs; k++) {
+    const float mk = P.partial[(i64)k * total + i * KEOPS_DIMRED];
+    s += keops_red_exp(mk - mm) * P.partial[(i64)k * total + e];
+  }
   P.out[e] = s;
 }
 #endif

@@ -229,9 +229,24 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
             if g.dim == 1 and isinstance(v, O.Var) and v.cat == 1 - red.tagI and v.dim == post.dim and v.dim <= 64:
                 final = (g, v)
                 break
+    # post-chunk formulas [F'(s, ...), v_j] or [F', 1, v_j] of a float32 log-sum-exp family reduction: online softmax
+    # with the weighted sum on the matrix cores
+    from .formulas.reductions import KIND_LSE
+
+    softmax = None
+    if red.kind == KIND_LSE and dtypeacc == "float" and sum_scheme != "kahan_scheme" and post.name == "Concat":
+        Fp, G = post.children
+        one = 0
+        if G.name == "Concat" and isinstance(G.children[0], O.IntCst) and G.children[0].val == 1:
+            one, G = 1, G.children[1]
+        if Fp.dim == 1 and isinstance(G, O.Var) and G.cat == 1 - red.tagI and G.dim <= (64 if xvar.dim > 128 else 128):
+            softmax = (Fp, G, one)
     full_post = post
     if final is not None:
         post = final[0]
+    elif softmax is not None:
+        post = softmax[0]
+    wvar = final[1] if final is not None else (softmax[1] if softmax is not None else None)
 
     class _Post:  # what VarLayout needs: the post-chunk formula with the reduction's orientation
         formula, tagI = post, red.tagI
@@ -245,14 +260,26 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
     dpad = -(-D // 16) * 16
     dimy_pad = 0 if layout.dimy == 0 else -(-layout.dimy // 4) * 4
     waves = config.chunk_waves
+    # LDS of the kernel: staged tile (hi|lo rows), the other reduced-index variables, and either the v tile
+    # (final-product variant) or the accumulator exchange of the two lanes of a row
+    def lds_bytes(w):
+        fixed = 32 * (dpad * 4 + 16) + 128 + 32 * max(1, dimy_pad) * 4
+        if wvar is not None:
+            return fixed + 32 * (-(-wvar.dim // 32)) * 32 * 4 + 128 * w
+        return fixed + 32 * w * red.dimred * (8 if dtypeacc == "double" else 4)
+    while waves > 1 and lds_bytes(waves) > config.knn_lds_budget:
+        waves //= 2
+    if lds_bytes(waves) > config.knn_lds_budget:
+        return None, None
     ra, rd, ro = VarLayout.table(layout.rowvars)
     ca, cd, co = VarLayout.table(layout.colvars)
     pa, pd, po = VarLayout.table(layout.parvars)
-    ncol_extra = 1 + (1 if final is not None and final[1] not in layout.colvars else 0)
+    ncol_extra = 1 + (1 if wvar is not None and wvar not in layout.colvars else 0)
     meta = dict(scheme="chunk", block=64 * waves, rows=1, tile_j=32, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
                 sizeof_acc=8 if dtypeacc == "double" else 4, nrowvars=len(layout.rowvars) + 1,
                 ncolvars=len(layout.colvars) + ncol_extra, nparvars=len(layout.parvars), chk_d=D, chk_dpad=dpad,
-                chk_mode=mode, chk_qb=32 * waves, chk_final=int(final is not None), nops=L.count_ops(outs))
+                chk_mode=mode, chk_qb=32 * waves, chk_final=int(final is not None), chk_softmax=int(softmax is not None),
+                nops=L.count_ops(outs))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
            f"typedef float T;\ntypedef {dtypeacc} TACC;", '#include "keops_common.h"']
     defs = dict(
@@ -266,6 +293,9 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
         defs.update(KEOPS_DIMFOUT=full_post.dim, CHK_FINAL=1, CHK_FV_ARG=final[1].ind, CHK_FV_DIM=final[1].dim,
                     CHK_FNB=-(-final[1].dim // 32), CHK_PERIOD=config.final_period,
                     CHK_BLOCKSUM=int(sum_scheme == "block_sum"))
+    elif softmax is not None:
+        defs.update(KEOPS_DIMFOUT=full_post.dim, CHK_SOFTMAX=1, CHK_SM_ONE=softmax[2], CHK_FV_ARG=softmax[1].ind,
+                    CHK_FV_DIM=softmax[1].dim, CHK_FNB=-(-softmax[1].dim // 32))
     src += [f"#define {k} {v}" for k, v in defs.items()]
     for name, vals in (("row_arg", ra), ("row_dim", rd), ("row_off", ro), ("col_arg", ca), ("col_dim", cd),
                        ("col_off", co), ("par_arg", pa), ("par_dim", pd), ("par_off", po)):
@@ -393,8 +423,10 @@ def get_keops_dll(
             use_chunk_mode = 2  # as the reference's final-chunk mode (get_keops_dll.py:101-108)
         elif chk is not None:
             source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs)
-            use_chunk_mode = 1
+            use_chunk_mode = 1 if source is not None else 0
         else:
+            source = None
+        if source is None:
             source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint,
                                            irregular="_ranges" in map_reduce_id)
         tag = hashlib.sha256((source + binder.templates_digest() + str(use_fast_math)).encode()).hexdigest()[:16]

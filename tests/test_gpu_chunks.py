@@ -127,3 +127,40 @@ def test_final_product_variant_and_generic_variant():
     scale2 = (K @ b64.abs() + b64.abs().sum(0, keepdim=True)).numpy()
     assert_sum_parity(got2, ref2, scale2)
     assert any(m.meta("scheme") == "chunk" and m.meta("chk_final") == "0" for m in keops_io._modules.values())
+
+
+@pytest.mark.parametrize("M,N,D,Dv,axis", [(700, 900, 64, 64, 1), (333, 2100, 128, 40, 1), (500, 47, 32, 3, 1), (640, 500, 64, 16, 0),
+                                          (300, 5000, 256, 64, 1)])
+def test_softmax_weighted_sum_on_matrix_cores(M, N, D, Dv, axis):
+    """SumSoftMaxWeight of a scaled inner product (attention-like): online softmax with the weighted sum on
+    the matrix cores (keops_chk_softmax), against torch.softmax in float64; also the plain weighted
+    log-sum-exp layout (no leading 1) and forced column slabs."""
+    from keops_amd import keops_io
+    from keops_amd.torch import Genred
+
+    rng = np.random.default_rng(31)
+    q = (rng.standard_normal((M, D)) / D ** 0.25).astype(np.float32)
+    k = (rng.standard_normal((N, D)) / D ** 0.25).astype(np.float32)
+    nv = N if axis == 1 else M
+    v = rng.standard_normal((nv, Dv)).astype(np.float32)
+    qd, kd, vd = to_dev(q, k, v)
+    vcat = "Vj" if axis == 1 else "Vi"
+    att = Genred("p*(q|k)", [f"q=Vi({D})", f"k=Vj({D})", f"v={vcat}({Dv})", "p=Pm(1)"], reduction_op="SumSoftMaxWeight",
+                 axis=axis, formula2="v")
+    scale = torch.tensor([0.7], device="cuda")
+    S = 0.7 * torch.from_numpy(q).double() @ torch.from_numpy(k).double().T
+    if axis == 0:
+        S = S.T
+    ref = torch.softmax(S, dim=1) @ torch.from_numpy(v).double()
+    for backend in ("GPU_1D", "GPU_2D"):
+        got = att(qd, kd, vd, scale, backend=backend).cpu().double()
+        assert got.shape == ref.shape
+        assert float((got - ref).abs().max()) <= 2e-5 * float(ref.abs().max()), backend
+    assert any(m.meta("chk_softmax") == "1" for m in keops_io._modules.values())
+    # weighted log-sum-exp: log sum_j exp(S_ij) v_j with positive weights
+    w = np.abs(v[:, :min(Dv, 5)]) + 0.1
+    lse = Genred("p*(q|k)", [f"q=Vi({D})", f"k=Vj({D})", f"w={vcat}({w.shape[1]})", "p=Pm(1)"], reduction_op="LogSumExp",
+                 axis=axis, formula2="w")
+    gl = lse(qd, kd, to_dev(w)[0], scale).cpu().double()
+    refl = torch.logsumexp(S[:, :, None] + torch.log(torch.from_numpy(w).double())[None, :, :], dim=1)
+    assert float((gl - refl).abs().max()) <= 2e-5 * max(1.0, float(refl.abs().max()))
