@@ -93,6 +93,7 @@ struct ShapeTable {
   std::vector<int64_t> shapes;  // (nargs+1) x (nbatchdims+3): [batch.., M, N, D]
 
   int64_t* row(int k) { return shapes.data() + (size_t)k * (nbatchdims + 3); }
+  const int64_t* row(int k) const { return shapes.data() + (size_t)k * (nbatchdims + 3); }
 
   // Mirrors Sizes<TYPE>::Sizes / fill_shape / check_ranges (Sizes.h:86-150,176-330) with the
   // checks enabled: a mismatch is an error instead of undefined behaviour.
@@ -243,6 +244,168 @@ struct Module {
     return 0;
   }
 };
+
+// Device tables of a block-sparse or batched launch (Ranges.h:40-86, keops_nvrtc.cpp:152-248): one
+// (range id, first row, end row) entry per workgroup of rows_per_block rows, the reduced-index ranges and,
+// with batch dimensions, the first-row offsets of the variables for every workgroup -- in the order
+// [row variables | reduced variables | parameters], or one entry per argument when by_arg is set.
+struct RangeTables {
+  const int64_t *lookup = nullptr, *slices_x = nullptr, *ranges_y = nullptr, *offsets = nullptr;
+  int64_t nblocks = 0;
+};
+
+int ensure_pinned(Module& m, size_t bytes);
+
+// must match struct KeopsRangeTables of kernels/keops_common.h
+struct RangeHeader {
+  const int64_t *lookup = nullptr, *slices_x = nullptr, *ranges_y = nullptr, *offsets = nullptr;
+  int32_t nbatchdims = 0, nargs = 0;
+};
+
+// a block-sparse / batched launch of one of the matrix-core schemes
+struct RangeLaunch {
+  RangeTables tables;
+  int nbatchdims = 0;
+  bool user_ranges = false;
+  RangeHeader header(int nargs) const {
+    RangeHeader h;
+    h.lookup = tables.lookup; h.slices_x = tables.slices_x; h.ranges_y = tables.ranges_y; h.offsets = tables.offsets;
+    h.nbatchdims = nbatchdims; h.nargs = nargs;
+    return h;
+  }
+};
+
+int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ranges, int64_t* const* ranges,
+                         int64_t rows_total, int64_t rows_per_block, bool by_arg, const std::vector<int>& rowvars,
+                         const std::vector<int>& colvars, const std::vector<int>& vP, hipStream_t stream, RangeTables& rt) {
+  const int64_t* rx_dev = nullptr;  // row ranges, device (user ranges only)
+  std::vector<int64_t> rx_host;     // row ranges on the host
+  int64_t nranges = 0;
+  const int64_t *slices_dev = nullptr, *ry_dev = nullptr;
+  const int nb = S.nbatchdims;
+  const int nvars = by_arg ? m.nargs : m.nrowvars + m.ncolvars + m.nparvars;
+  std::vector<int64_t> synth;  // batch mode: [slices (nbatches)] [ranges_y (2*nbatches)]
+
+  if (user_ranges) {
+    const int sel = tagI == 0 ? 0 : 3;
+    nranges = ranges[6][sel];
+    rx_dev = ranges[sel];
+    slices_dev = ranges[sel + 1];
+    ry_dev = ranges[sel + 2];
+    rx_host.resize((size_t)2 * nranges);
+    // same synchronous read-back as the reference (keops_nvrtc.cpp:195-197)
+    if (nranges) HIP_TRY(hipMemcpyAsync(rx_host.data(), rx_dev, sizeof(int64_t) * 2 * nranges, hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipStreamSynchronize(stream));
+  } else {
+    // block-diagonal pattern, one range per batch (Ranges.h:40-86)
+    nranges = S.nbatches;
+    const int64_t R = tagI == 0 ? S.M : S.N, C = tagI == 0 ? S.N : S.M;
+    rx_host.resize((size_t)2 * nranges);
+    synth.resize((size_t)3 * nranges);
+    for (int64_t b = 0; b < nranges; b++) {
+      rx_host[2 * b] = b * R;
+      rx_host[2 * b + 1] = (b + 1) * R;
+      synth[b] = b + 1;
+      synth[nranges + 2 * b] = b * C;
+      synth[nranges + 2 * b + 1] = (b + 1) * C;
+    }
+  }
+
+  // lookup table: one entry per workgroup (keops_nvrtc.cpp:210-231)
+  int64_t nblocks = 0;
+  for (int64_t r = 0; r < nranges; r++) {
+    const int64_t len = rx_host[2 * r + 1] - rx_host[2 * r];
+    if (len < 0 || rx_host[2 * r] < 0 || rx_host[2 * r + 1] > rows_total)
+      return fail(-1, "row range " + std::to_string(r) + " is out of bounds");
+    nblocks += (len + rows_per_block - 1) / rows_per_block;
+  }
+
+  // batch mode tables only depend on the shapes: reuse them across calls
+  std::vector<int64_t> key;
+  bool reuse = false;
+  if (!user_ranges) {
+    key.push_back(tagI);
+    key.push_back(by_arg ? 1 : 0);
+    key.push_back(rows_per_block);
+    key.insert(key.end(), S.shapes.begin(), S.shapes.end());
+    reuse = key == m.tables_key && m.tables.ptr != nullptr;
+  }
+  const size_t n_lookup = (size_t)3 * nblocks, n_off = nb > 0 ? (size_t)nblocks * nvars : 0, n_syn = synth.size();
+  const size_t total = n_lookup + n_off + n_syn;
+  if (!reuse && total > 0) {
+    if (m.tables_in_flight) {
+      HIP_TRY(hipEventSynchronize(m.tables_copied));
+      m.tables_in_flight = false;
+    }
+    if (int rc = ensure_pinned(m, total * sizeof(int64_t))) return rc;
+    int64_t* lk = (int64_t*)m.pinned;
+    int64_t* off = lk + n_lookup;
+    int64_t* syn = off + n_off;
+    int64_t idx = 0;
+    for (int64_t r = 0; r < nranges; r++) {
+      const int64_t s = rx_host[2 * r], len = rx_host[2 * r + 1] - s;
+      for (int64_t j = 0; j < len; j += rows_per_block) {
+        lk[3 * idx] = r;
+        lk[3 * idx + 1] = s + j;
+        lk[3 * idx + 2] = s + j + std::min(rows_per_block, len - j);
+        idx++;
+      }
+    }
+    if (nb > 0) {
+      // per-block first-row offsets of every variable (keops_nvrtc.cpp:75-149, ranges_utils.h:27-91)
+      const int W = nb + 3;
+      const int64_t R = tagI == 0 ? S.M : S.N, C = tagI == 0 ? S.N : S.M;
+      const int rpos = tagI == 0 ? nb : nb + 1, cpos = tagI == 0 ? nb + 1 : nb;
+      std::vector<int64_t> shp(nb + 1);
+      for (int64_t k = 0; k < nblocks; k++) {
+        const int64_t rid = lk[3 * k];
+        const int64_t patch = lk[3 * k + 1] - rid * R;
+        int64_t* o = off + k * nvars;
+        int c = 0;
+        if (by_arg) std::fill(o, o + nvars, (int64_t)0);
+        for (int v : rowvars) {
+          const int64_t* r = S.row(v + 1);
+          for (int b = 0; b < nb; b++) shp[b] = r[b];
+          shp[nb] = r[rpos];
+          o[by_arg ? v : c++] = patch + broadcast_index(rid * R, nb, S.shapes.data(), shp.data());
+        }
+        for (int v : colvars) {
+          const int64_t* r = S.row(v + 1);
+          for (int b = 0; b < nb; b++) shp[b] = r[b];
+          shp[nb] = r[cpos];
+          o[by_arg ? v : c++] = broadcast_index(rid * C, nb, S.shapes.data(), shp.data());
+        }
+        for (int v : vP) {
+          const int64_t* r = S.row(v + 1);
+          for (int b = 0; b < nb; b++) shp[b] = r[b];
+          shp[nb] = 1;
+          o[by_arg ? v : c++] = broadcast_index(rid, nb, S.shapes.data(), shp.data());
+        }
+        (void)W;
+      }
+    }
+    if (n_syn) std::memcpy(syn, synth.data(), n_syn * sizeof(int64_t));
+    if (int rc = m.tables.reserve(total * sizeof(int64_t))) return rc;
+    HIP_TRY(hipMemcpyAsync(m.tables.ptr, m.pinned, total * sizeof(int64_t), hipMemcpyHostToDevice, stream));
+    if (!m.tables_copied) HIP_TRY(hipEventCreateWithFlags(&m.tables_copied, hipEventDisableTiming));
+    HIP_TRY(hipEventRecord(m.tables_copied, stream));
+    m.tables_in_flight = true;
+    m.tables_key = key;
+    m.cached_nblocks = nblocks;
+  }
+  const int64_t* tab = (const int64_t*)m.tables.ptr;
+  rt.nblocks = nblocks;
+  rt.lookup = tab;
+  rt.offsets = nb > 0 ? tab + n_lookup : nullptr;
+  if (user_ranges) {
+    rt.slices_x = slices_dev;
+    rt.ranges_y = ry_dev;
+  } else {
+    rt.slices_x = tab + n_lookup + n_off;
+    rt.ranges_y = tab + n_lookup + n_off + nranges;
+  }
+  return 0;
+}
 
 // Kernel argument block: must match struct KeopsParams of kernels/keops_conv.h.
 struct LaunchHeader {
@@ -483,25 +646,29 @@ struct ChkHeader {
   int64_t slab_len;
   int32_t nslabs;
   int32_t pad_;
+  int64_t nxs, nys;
+  RangeHeader rt;
 };
 
-int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, int tag1D2D, hipStream_t stream) {
+// rg: block-sparse / batched launch (module built with ranges=1), else null; nxs, nys: rows of the chunked arguments
+int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, int tag1D2D, hipStream_t stream,
+                 const RangeLaunch* rg, int64_t nxs, int64_t nys) {
   const int64_t D = m.meta_int("chk_d", 0), DP = m.meta_int("chk_dpad", 0), QB = m.meta_int("chk_qb", 128);
   const int mode = m.meta_int("chk_mode", 0);
   if (D <= 0 || DP <= 0) return fail(-1, "corrupt chunk module metadata");
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
-  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(512, ny / 64));
+  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(512, nys / 64));
   const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
-  const size_t o_xs = take((size_t)nx * DP * 4), o_ys = take((size_t)ny * DP * 4);
-  const size_t o_xn = take((size_t)nx * 4), o_yn = take((size_t)ny * 4);
+  const size_t o_xs = take((size_t)nxs * DP * 4), o_ys = take((size_t)nys * DP * 4);
+  const size_t o_xn = take((size_t)nxs * 4), o_yn = take((size_t)nys * 4);
   // final-product variant: slabs over the reduced axis fill the chip and round the grid to whole
   // rounds of workgroups (one 8-wavefront workgroup per CU, all taking the same time)
   const bool softmax = m.meta_int("chk_softmax", 0) != 0;
   const bool final = m.meta_int("chk_final", 0) != 0 || softmax;
-  const int64_t row_blocks = (nx + QB - 1) / QB, TJ = m.tile_j;
+  const int64_t row_blocks = rg ? rg->tables.nblocks : (nx + QB - 1) / QB, TJ = m.tile_j;
   int64_t nslabs = 1, slab_len = std::max<int64_t>(TJ, (ny + TJ - 1) / TJ * TJ);
-  if (final) {
+  if (final && !rg) {
     const int64_t cap = std::max<int64_t>(1, ny / (8 * TJ));
     const int64_t target = 2 * (int64_t)m.cu_count;
     if (tag1D2D == 1 || row_blocks < target) {
@@ -520,6 +687,8 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   ChkHeader h{};
   h.nx = nx; h.ny = ny; h.xs = ws + o_xs; h.ys = ws + o_ys; h.xn = ws + o_xn; h.yn = ws + o_yn; h.colsum = ws + o_colsum;
   h.colpart = ws + o_colpart; h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs;
+  h.nxs = nxs; h.nys = nys;
+  if (rg) h.rt = rg->header(m.nargs);
   std::memcpy(buf.data(), &h, sizeof(h));
   for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
   const size_t psize = sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs);
@@ -532,9 +701,11 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   }
   const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
   size_t sz = with_which(0);
-  if (int rc = launch_raw(m, "keops_chk_prep", (unsigned)((nx * lpr + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_chk_prep", (unsigned)((nxs * lpr + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
   sz = with_which(1);
-  if (int rc = launch_raw(m, "keops_chk_prep", (unsigned)((ny * lpr + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_chk_prep", (unsigned)((nys * lpr + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  if (rg && rg->user_ranges)
+    if (int rc = launch_raw(m, "keops_chk_fill_neutral", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), psize, stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
   if (final) {
     if (int rc = launch_raw(m, softmax ? "keops_chk_softmax" : "keops_chk_final", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)m.block, buf.data(), psize, stream)) return rc;
@@ -559,27 +730,30 @@ struct FinHeader {
   int64_t slab_len;
   int32_t nslabs;
   int32_t pad_;
+  RangeHeader rt;
 };
 
-int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, int tag1D2D, hipStream_t stream) {
+int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, int tag1D2D, hipStream_t stream,
+                 const RangeLaunch* rg) {
   const int64_t DV = m.meta_int("fin_dv", 0), NZ = m.meta_int("fin_nz", 1), QB = m.meta_int("fin_qb", 256), TJ = m.tile_j;
   if (DV <= 0 || NZ <= 0 || QB <= 0 || TJ <= 0) return fail(-1, "corrupt final-product module metadata");
-  const int64_t row_blocks = (nx + QB - 1) / QB;
+  const int64_t row_blocks = rg ? rg->tables.nblocks : (nx + QB - 1) / QB;
   // enough workgroups for the chip: cut the reduced axis in slabs when there are few output rows
   int64_t nslabs = 1;
   const int64_t target = 2 * (int64_t)m.cu_count;
-  if (tag1D2D == 1 || row_blocks * NZ < target) {
+  if (!rg && (tag1D2D == 1 || row_blocks * NZ < target)) {
     const int64_t max_slabs = std::max<int64_t>(1, ny / (8 * TJ));
     nslabs = std::min<int64_t>(max_slabs, (target + row_blocks * NZ - 1) / (row_blocks * NZ));
     if (tag1D2D == 1) nslabs = std::max<int64_t>(nslabs, std::min<int64_t>(max_slabs, 2));
     nslabs = std::max<int64_t>(1, std::min<int64_t>(nslabs, 65535));
   }
   // one workgroup (8 wavefronts of ~230 VGPRs) fills a CU and all of them take the same time
-  nslabs = balance_slabs(row_blocks * NZ, nslabs, std::min<int64_t>(std::max<int64_t>(nslabs, 8), std::max<int64_t>(1, ny / (8 * TJ))), m.cu_count);
+  if (!rg) nslabs = balance_slabs(row_blocks * NZ, nslabs, std::min<int64_t>(std::max<int64_t>(nslabs, 8), std::max<int64_t>(1, ny / (8 * TJ))), m.cu_count);
   int64_t len = std::max<int64_t>(TJ, ((ny + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ);
   nslabs = std::max<int64_t>(1, (ny + len - 1) / len);
   FinHeader h{};
   h.nx = nx; h.ny = ny; h.out = out; h.slab_len = len; h.nslabs = (int32_t)nslabs;
+  if (rg) h.rt = rg->header(m.nargs);
   if (nslabs > 1) {
     if (int rc = m.partial.reserve((size_t)nslabs * nx * DV * 4)) return rc;
     h.partial = m.partial.ptr;
@@ -587,6 +761,8 @@ int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   std::vector<char> buf(sizeof(FinHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs));
   std::memcpy(buf.data(), &h, sizeof(h));
   for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
+  if (rg && rg->user_ranges)
+    if (int rc = launch_raw(m, "keops_fin_fill_neutral", (unsigned)((nx * DV + 255) / 256), 1, 256, buf.data(), buf.size(), stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
   if (int rc = launch_raw3(m, "keops_fin_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)NZ, (unsigned)m.block, buf.data(), buf.size(), stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
@@ -817,12 +993,37 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
     if (use_ranges) return fail(-1, "the matrix-core KNN module does not handle ranges or batch dimensions");
     const int rowarg = m.meta_int("rowarg", 0), colarg = m.meta_int("colarg", 1);
     if (int rc = launch_knn(m, rows_total, cols_total, args[rowarg], args[colarg], out, tag1D2D, stream)) return rc;
-  } else if (m.scheme == "final") {
-    if (use_ranges) return fail(-1, "the matrix-core final-product module does not handle ranges or batch dimensions");
-    if (int rc = launch_final(m, rows_total, cols_total, out, args, tag1D2D, stream)) return rc;
-  } else if (m.scheme == "chunk") {
-    if (use_ranges) return fail(-1, "the matrix-core chunked module does not handle ranges or batch dimensions");
-    if (int rc = launch_chunk(m, rows_total, cols_total, out, args, tag1D2D, stream)) return rc;
+  } else if (m.scheme == "final" || m.scheme == "chunk") {
+    const bool built_for_ranges = m.meta_int("ranges", 0) != 0;
+    if (use_ranges != built_for_ranges)
+      return fail(-1, built_for_ranges ? "this module was built for block-sparse or batched reductions"
+                                       : "this module was built for dense reductions without batch dimensions");
+    RangeLaunch rg;
+    if (use_ranges) {
+      rg.nbatchdims = nb;
+      rg.user_ranges = user_ranges;
+      const int64_t qb = m.meta_int(m.scheme == "final" ? "fin_qb" : "chk_qb", 256);
+      if (int rc = prepare_range_tables(m, S, tagI, user_ranges, ranges, rows_total, qb, true, rowvars, colvars, vP, stream,
+                                        rg.tables))
+        return rc;
+    }
+    // rows of an argument: a batch dimension of size 1 is broadcast, not stored
+    auto arg_rows = [&](int arg, int64_t len) {
+      const int64_t* r = S.row(arg + 1);
+      int64_t n = len;
+      for (int b = 0; b < nb; b++) n *= r[b];
+      return n;
+    };
+    if (m.scheme == "final") {
+      if (int rc = launch_final(m, rows_total, cols_total, out, args, tag1D2D, stream, use_ranges ? &rg : nullptr)) return rc;
+    } else {
+      const int xarg = m.meta_int("chk_xarg", -1), yarg = m.meta_int("chk_yarg", -1);
+      if (xarg < 0 || yarg < 0 || xarg >= m.nargs || yarg >= m.nargs) return fail(-1, "corrupt chunk module metadata");
+      const int64_t nxs = nb > 0 ? arg_rows(xarg, tagI == 0 ? S.M : S.N) : rows_total;
+      const int64_t nys = nb > 0 ? arg_rows(yarg, tagI == 0 ? S.N : S.M) : cols_total;
+      if (int rc = launch_chunk(m, rows_total, cols_total, out, args, tag1D2D, stream, use_ranges ? &rg : nullptr, nxs, nys))
+        return rc;
+    }
   } else if (!use_ranges) {
     // ---- dense scheme, optionally cut in column slabs ----
     const int64_t row_blocks = (rows_total + rows_per_block - 1) / rows_per_block;
@@ -867,128 +1068,15 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
     }
   } else {
     // ---- block-sparse / batched scheme (Ranges.h, keops_nvrtc.cpp:152-248) ----
-    const int64_t* rx_dev = nullptr;  // row ranges, device (user ranges only)
-    std::vector<int64_t> rx_host;     // row ranges on the host
-    int64_t nranges = 0;
-    const int64_t *slices_dev = nullptr, *ry_dev = nullptr;
-    const int nvars = m.nrowvars + m.ncolvars + m.nparvars;
-    std::vector<int64_t> synth;  // batch mode: [slices (nbatches)] [ranges_y (2*nbatches)]
-
-    if (user_ranges) {
-      const int sel = tagI == 0 ? 0 : 3;
-      nranges = ranges[6][sel];
-      rx_dev = ranges[sel];
-      slices_dev = ranges[sel + 1];
-      ry_dev = ranges[sel + 2];
-      rx_host.resize((size_t)2 * nranges);
-      // same synchronous read-back as the reference (keops_nvrtc.cpp:195-197)
-      if (nranges) HIP_TRY(hipMemcpyAsync(rx_host.data(), rx_dev, sizeof(int64_t) * 2 * nranges, hipMemcpyDeviceToHost, stream));
-      HIP_TRY(hipStreamSynchronize(stream));
-    } else {
-      // block-diagonal pattern, one range per batch (Ranges.h:40-86)
-      nranges = S.nbatches;
-      const int64_t R = tagI == 0 ? S.M : S.N, C = tagI == 0 ? S.N : S.M;
-      rx_host.resize((size_t)2 * nranges);
-      synth.resize((size_t)3 * nranges);
-      for (int64_t b = 0; b < nranges; b++) {
-        rx_host[2 * b] = b * R;
-        rx_host[2 * b + 1] = (b + 1) * R;
-        synth[b] = b + 1;
-        synth[nranges + 2 * b] = b * C;
-        synth[nranges + 2 * b + 1] = (b + 1) * C;
-      }
-    }
-
-    // lookup table: one entry per workgroup (keops_nvrtc.cpp:210-231)
-    int64_t nblocks = 0;
-    for (int64_t r = 0; r < nranges; r++) {
-      const int64_t len = rx_host[2 * r + 1] - rx_host[2 * r];
-      if (len < 0 || rx_host[2 * r] < 0 || rx_host[2 * r + 1] > rows_total)
-        return fail(-1, "row range " + std::to_string(r) + " is out of bounds");
-      nblocks += (len + rows_per_block - 1) / rows_per_block;
-    }
-
-    // batch mode tables only depend on the shapes: reuse them across calls
-    std::vector<int64_t> key;
-    bool reuse = false;
-    if (!user_ranges) {
-      key.push_back(tagI);
-      key.push_back(rows_per_block);
-      key.insert(key.end(), S.shapes.begin(), S.shapes.end());
-      reuse = key == m.tables_key && m.tables.ptr != nullptr;
-    }
-    const size_t n_lookup = (size_t)3 * nblocks, n_off = nb > 0 ? (size_t)nblocks * nvars : 0, n_syn = synth.size();
-    const size_t total = n_lookup + n_off + n_syn;
-    if (!reuse && total > 0) {
-      if (m.tables_in_flight) {
-        HIP_TRY(hipEventSynchronize(m.tables_copied));
-        m.tables_in_flight = false;
-      }
-      if (int rc = ensure_pinned(m, total * sizeof(int64_t))) return rc;
-      int64_t* lk = (int64_t*)m.pinned;
-      int64_t* off = lk + n_lookup;
-      int64_t* syn = off + n_off;
-      int64_t idx = 0;
-      for (int64_t r = 0; r < nranges; r++) {
-        const int64_t s = rx_host[2 * r], len = rx_host[2 * r + 1] - s;
-        for (int64_t j = 0; j < len; j += rows_per_block) {
-          lk[3 * idx] = r;
-          lk[3 * idx + 1] = s + j;
-          lk[3 * idx + 2] = s + j + std::min(rows_per_block, len - j);
-          idx++;
-        }
-      }
-      if (nb > 0) {
-        // per-block first-row offsets of every variable (keops_nvrtc.cpp:75-149, ranges_utils.h:27-91)
-        const int W = nb + 3;
-        const int64_t R = tagI == 0 ? S.M : S.N, C = tagI == 0 ? S.N : S.M;
-        const int rpos = tagI == 0 ? nb : nb + 1, cpos = tagI == 0 ? nb + 1 : nb;
-        std::vector<int64_t> shp(nb + 1);
-        for (int64_t k = 0; k < nblocks; k++) {
-          const int64_t rid = lk[3 * k];
-          const int64_t patch = lk[3 * k + 1] - rid * R;
-          int64_t* o = off + k * nvars;
-          int c = 0;
-          for (int v : rowvars) {
-            const int64_t* r = S.row(v + 1);
-            for (int b = 0; b < nb; b++) shp[b] = r[b];
-            shp[nb] = r[rpos];
-            o[c++] = patch + broadcast_index(rid * R, nb, S.shapes.data(), shp.data());
-          }
-          for (int v : colvars) {
-            const int64_t* r = S.row(v + 1);
-            for (int b = 0; b < nb; b++) shp[b] = r[b];
-            shp[nb] = r[cpos];
-            o[c++] = broadcast_index(rid * C, nb, S.shapes.data(), shp.data());
-          }
-          for (int v : vP) {
-            const int64_t* r = S.row(v + 1);
-            for (int b = 0; b < nb; b++) shp[b] = r[b];
-            shp[nb] = 1;
-            o[c++] = broadcast_index(rid, nb, S.shapes.data(), shp.data());
-          }
-          (void)W;
-        }
-      }
-      if (n_syn) std::memcpy(syn, synth.data(), n_syn * sizeof(int64_t));
-      if (int rc = m.tables.reserve(total * sizeof(int64_t))) return rc;
-      HIP_TRY(hipMemcpyAsync(m.tables.ptr, m.pinned, total * sizeof(int64_t), hipMemcpyHostToDevice, stream));
-      if (!m.tables_copied) HIP_TRY(hipEventCreateWithFlags(&m.tables_copied, hipEventDisableTiming));
-      HIP_TRY(hipEventRecord(m.tables_copied, stream));
-      m.tables_in_flight = true;
-      m.tables_key = key;
-      m.cached_nblocks = nblocks;
-    }
-    const int64_t* tab = (const int64_t*)m.tables.ptr;
-    h.lookup = tab;
-    h.offsets = nb > 0 ? tab + n_lookup : nullptr;
-    if (user_ranges) {
-      h.slices_x = slices_dev;
-      h.ranges_y = ry_dev;
-    } else {
-      h.slices_x = tab + n_lookup + n_off;
-      h.ranges_y = tab + n_lookup + n_off + nranges;
-    }
+    RangeTables rt;
+    if (int rc = prepare_range_tables(m, S, tagI, user_ranges, ranges, rows_total, rows_per_block, false, rowvars, colvars,
+                                      vP, stream, rt))
+      return rc;
+    const int64_t nblocks = rt.nblocks;
+    h.lookup = rt.lookup;
+    h.offsets = rt.offsets;
+    h.slices_x = rt.slices_x;
+    h.ranges_y = rt.ranges_y;
     if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
     if (user_ranges) {
       const int64_t gb = (rows_total + m.block - 1) / m.block;

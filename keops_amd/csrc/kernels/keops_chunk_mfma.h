@@ -70,6 +70,8 @@ struct ChkParams {
   i64 slab_len;         // keops_chk_final: reduced rows per slab (multiple of CHK_TJ)
   int nslabs;
   int pad_;
+  i64 nxs, nys;         // rows of the chunked row / column arguments (fewer than nx, ny when a batch dimension is broadcast)
+  KeopsRangeTables rt;  // block-sparse / batch geometry (KEOPS_MC_RANGES)
   const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
 };
 
@@ -84,8 +86,8 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum(const ChkPara
   __shared__ float part[256];
   constexpr int RG = 256 / CHK_CW;
   const int cw = threadIdx.x % CHK_CW, rg = threadIdx.x / CHK_CW;
-  const i64 rows_per_block = (P.ny + gridDim.x - 1) / gridDim.x;
-  const i64 r0 = (i64)blockIdx.x * rows_per_block, r1 = keops_min(P.ny, r0 + rows_per_block);
+  const i64 rows_per_block = (P.nys + gridDim.x - 1) / gridDim.x;
+  const i64 r0 = (i64)blockIdx.x * rows_per_block, r1 = keops_min(P.nys, r0 + rows_per_block);
   const T* y = P.arg[CHK_YARG];
   for (int c0 = 0; c0 < CHK_DPAD; c0 += CHK_CW) {
     const int c = c0 + cw;
@@ -138,13 +140,13 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum_final(const C
 // (deterministic).
 #define CHK_LPR (CHK_DPAD / 4 <= 4 ? 4 : (CHK_DPAD / 4 <= 8 ? 8 : (CHK_DPAD / 4 <= 16 ? 16 : (CHK_DPAD / 4 <= 32 ? 32 : 64))))
 extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams P, int which) {
-  const i64 n = which ? P.ny : P.nx;
+  const i64 n = which ? P.nys : P.nxs;
   const T* src = P.arg[which ? CHK_YARG : CHK_XARG];
   __bf16* dst = which ? P.ys : P.xs;
   const int q = threadIdx.x % CHK_LPR;
   const i64 row = ((i64)blockIdx.x * 256 + threadIdx.x) / CHK_LPR;
   const bool live = row < n && q * 4 < CHK_DPAD;
-  const float inv = 1.0f / (float)P.ny;
+  const float inv = 1.0f / (float)P.nys;
   const float scale = (CHK_MODE == 0 && !which) ? -2.0f : 1.0f;
   float nrm = 0.f;
   if (live) {
@@ -181,30 +183,35 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
-  i64 q = (i64)blockIdx.x * CHK_QB + wave * 32 + col;
-  const bool valid = q < P.nx;
-  if (!valid) q = P.nx - 1;
+  KeopsTileGeom G;
+  G.init(P.rt, P.nx, CHK_QB);
+  const i64 row0 = G.row_first + wave * 32;  // first output row of this wavefront
+  const bool wave_live = row0 < G.row_end;   // a wavefront without rows only helps staging the tiles
+  i64 q = row0 + col;
+  const bool valid = q < G.row_end;
+  if (!valid) q = G.row_end - 1;
+  const i64 qx = G.row(CHK_XARG, q);
 
   // B operands: split rows of the chunked row variable
   chk_bf16x8 bh[CHK_KB], bl[CHK_KB];
 #pragma unroll
   for (int kb = 0; kb < CHK_KB; kb++) {
-    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + kb * 16 + 8 * half);
-    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + kb * 16 + 8 * half);
+    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
   }
-  const float xnq = CHK_MODE == 0 ? P.xn[q] : 0.f;
+  const float xnq = CHK_MODE == 0 ? P.xn[qx] : 0.f;
   // other row variables and parameters of the post-chunk formula
   T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NROWVARS; v++) {
-    const T* src = P.arg[keops_row_arg[v]] + q * keops_row_dim[v];
+    const T* src = P.arg[keops_row_arg[v]] + G.row(keops_row_arg[v], q) * keops_row_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
   }
   T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NPARVARS; v++) {
-    const T* src = P.arg[keops_par_arg[v]];
+    const T* src = P.arg[keops_par_arg[v]] + G.par(keops_par_arg[v]) * keops_par_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
   }
@@ -216,19 +223,22 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
   constexpr int NPF = (CHK_TJ * CH + CHK_BLOCK - 1) / CHK_BLOCK;
   uint4 pf[NPF];
   float pfn = 0.f;
-  auto prefetch = [&](i64 j0) {
-    const int n = (int)keops_min((i64)CHK_TJ, P.ny - j0);
-    const uint4* src = reinterpret_cast<const uint4*>(P.ys + j0 * 2 * CHK_DPAD);
+  auto prefetch = [&](i64 j0, i64 jend) {
+    const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
+    const i64 jy = G.col(CHK_YARG, j0);
+    const uint4* src = reinterpret_cast<const uint4*>(P.ys + jy * 2 * CHK_DPAD);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * CHK_BLOCK;
       pf[u] = (e < n * CH) ? src[e] : make_uint4(0u, 0u, 0u, 0u);
     }
-    if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[j0 + tid] : 0.f;
+    if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[jy + tid] : 0.f;
   };
-  if (P.ny > 0) prefetch(0);
-  for (i64 j0 = 0; j0 < P.ny; j0 += CHK_TJ) {
-    const int n = (int)keops_min((i64)CHK_TJ, P.ny - j0);
+  // folds the reduced rows [jbeg, jend) into the accumulators
+  auto sweep = [&](i64 jbeg, i64 jend) {
+  if (jbeg < jend) prefetch(jbeg, jend);
+  for (i64 j0 = jbeg; j0 < jend; j0 += CHK_TJ) {
+    const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
     __syncthreads();
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
@@ -243,14 +253,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
 #pragma unroll
     for (int v = 0; v < KEOPS_NCOLVARS; v++) {
       const int dim = keops_col_dim[v];
-      const T* src = P.arg[keops_col_arg[v]] + j0 * dim;
+      const T* src = P.arg[keops_col_arg[v]] + G.col(keops_col_arg[v], j0) * dim;
       for (int e = tid; e < n * dim; e += CHK_BLOCK) {
         const int row = e / dim, c = e - row * dim;
         yo_s[row * CHK_DY + keops_col_off[v] + c] = src[e];
       }
     }
     __syncthreads();
-    if (j0 + CHK_TJ < P.ny) prefetch(j0 + CHK_TJ);
+    if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ, jend);
+    if (!wave_live) continue;
 
     // s tile: accumulator register v of this lane is reduced row 8*(v/4) + 4*half + v%4
     chk_f32x16 s;
@@ -305,6 +316,12 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
     acc.merge(tmp);
 #endif
   }
+  };
+#if KEOPS_MC_RANGES
+  G.for_each_range(P.rt, sweep);
+#else
+  sweep(0, P.ny);
+#endif
 
   // the two lanes of an output row merge their accumulators (lower reduced rows first)
   __syncthreads();
@@ -332,28 +349,32 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
-  const i64 row0 = (i64)blockIdx.x * CHK_QB + wave * 32;
+  KeopsTileGeom G;
+  G.init(P.rt, P.nx, CHK_QB);
+  const i64 row0 = G.row_first + wave * 32;  // first output row of this wavefront
+  const bool wave_live = row0 < G.row_end;   // a wavefront without rows only helps staging the tiles
   i64 q = row0 + col;
-  if (q >= P.nx) q = P.nx - 1;  // clamped rows compute, never store
+  if (q >= G.row_end) q = G.row_end - 1;
+  const i64 qx = G.row(CHK_XARG, q);  // clamped rows compute, never store
 
   chk_bf16x8 bh[CHK_KB], bl[CHK_KB];
 #pragma unroll
   for (int kb = 0; kb < CHK_KB; kb++) {
-    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + kb * 16 + 8 * half);
-    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + kb * 16 + 8 * half);
+    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
   }
-  const float xnq = CHK_MODE == 0 ? P.xn[q] : 0.f;
+  const float xnq = CHK_MODE == 0 ? P.xn[qx] : 0.f;
   T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NROWVARS; v++) {
-    const T* src = P.arg[keops_row_arg[v]] + q * keops_row_dim[v];
+    const T* src = P.arg[keops_row_arg[v]] + G.row(keops_row_arg[v], q) * keops_row_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
   }
   T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NPARVARS; v++) {
-    const T* src = P.arg[keops_par_arg[v]];
+    const T* src = P.arg[keops_par_arg[v]] + G.par(keops_par_arg[v]) * keops_par_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
   }
@@ -376,7 +397,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int ir = 8 * (r >> 2) + (r & 3);
-        if (ibase + ir < P.nx && 32 * b + col < CHK_FV_DIM) {
+        if (ibase + ir < G.row_end && 32 * b + col < CHK_FV_DIM) {
           T* oo = o + (i64)ir * CHK_FV_DIM + 32 * b;
           *oo = first ? acc[b][r] : *oo + acc[b][r];
         }
@@ -386,8 +407,6 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
     first = false;
   };
 
-  const i64 jbeg = (i64)blockIdx.y * P.slab_len;
-  const i64 jend = keops_min(P.ny, jbeg + P.slab_len);
   const T* vsrc = P.arg[CHK_FV_ARG];
 
   constexpr int CH = CHK_ROWBYTES / 16;
@@ -396,25 +415,28 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
   uint4 pf[NPF];
   T pfv[NPV];
   float pfn = 0.f;
-  auto prefetch = [&](i64 j0) {
+  auto prefetch = [&](i64 j0, i64 jend) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
-    const uint4* src = reinterpret_cast<const uint4*>(P.ys + j0 * 2 * CHK_DPAD);
+    const i64 jy = G.col(CHK_YARG, j0), jv = G.col(CHK_FV_ARG, j0);
+    const uint4* src = reinterpret_cast<const uint4*>(P.ys + jy * 2 * CHK_DPAD);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * CHK_BLOCK;
       pf[u] = (e < n * CH) ? src[e] : make_uint4(0u, 0u, 0u, 0u);
     }
-    if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[j0 + tid] : 0.f;
+    if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[jy + tid] : 0.f;
     // v tile, zero past the last row / column (the matrix product must not see stale values)
 #pragma unroll
     for (int u = 0; u < NPV; u++) {
       const int e = tid + u * CHK_BLOCK;
       const int row = e / CHK_FVS, c = e - row * CHK_FVS;
-      pfv[u] = (row < n && c < CHK_FV_DIM) ? vsrc[(j0 + row) * CHK_FV_DIM + c] : (T)0;
+      pfv[u] = (row < n && c < CHK_FV_DIM) ? vsrc[(jv + row) * CHK_FV_DIM + c] : (T)0;
     }
   };
-  if (jbeg < jend) prefetch(jbeg);
   int since_fold = 0;
+  // folds the reduced rows [jbeg, jend) into the register tiles
+  auto sweep = [&](i64 jbeg, i64 jend) {
+  if (jbeg < jend) prefetch(jbeg, jend);
   for (i64 j0 = jbeg; j0 < jend; j0 += CHK_TJ) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
     __syncthreads();
@@ -430,7 +452,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
 #pragma unroll
     for (int v = 0; v < KEOPS_NCOLVARS; v++) {
       const int dim = keops_col_dim[v];
-      const T* src = P.arg[keops_col_arg[v]] + j0 * dim;
+      const T* src = P.arg[keops_col_arg[v]] + G.col(keops_col_arg[v], j0) * dim;
       for (int e = tid; e < n * dim; e += CHK_BLOCK) {
         const int row = e / dim, c = e - row * dim;
         yo_s[row * CHK_DY + keops_col_off[v] + c] = src[e];
@@ -442,7 +464,8 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
       if (e < CHK_TJ * CHK_FVS) bt[e] = pfv[u];
     }
     __syncthreads();
-    if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ);
+    if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ, jend);
+    if (!wave_live) continue;
 
     chk_f32x16 s;
     if (CHK_MODE == 0) {
@@ -493,6 +516,12 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
     }
 #endif
   }
+  };
+#if KEOPS_MC_RANGES
+  G.for_each_range(P.rt, sweep);
+#else
+  sweep((i64)blockIdx.y * P.slab_len, keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len));
+#endif
   fold();
 }
 
@@ -529,28 +558,32 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
-  const i64 row0 = (i64)blockIdx.x * CHK_QB + wave * 32;
+  KeopsTileGeom G;
+  G.init(P.rt, P.nx, CHK_QB);
+  const i64 row0 = G.row_first + wave * 32;  // first output row of this wavefront
+  const bool wave_live = row0 < G.row_end;   // a wavefront without rows only helps staging the tiles
   i64 q = row0 + col;
-  if (q >= P.nx) q = P.nx - 1;
+  if (q >= G.row_end) q = G.row_end - 1;
+  const i64 qx = G.row(CHK_XARG, q);
 
   chk_bf16x8 bh[CHK_KB], bl[CHK_KB];
 #pragma unroll
   for (int kb = 0; kb < CHK_KB; kb++) {
-    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + kb * 16 + 8 * half);
-    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + q * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + kb * 16 + 8 * half);
+    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
   }
-  const float xnq = CHK_MODE == 0 ? P.xn[q] : 0.f;
+  const float xnq = CHK_MODE == 0 ? P.xn[qx] : 0.f;
   T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NROWVARS; v++) {
-    const T* src = P.arg[keops_row_arg[v]] + q * keops_row_dim[v];
+    const T* src = P.arg[keops_row_arg[v]] + G.row(keops_row_arg[v], q) * keops_row_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
   }
   T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NPARVARS; v++) {
-    const T* src = P.arg[keops_par_arg[v]];
+    const T* src = P.arg[keops_par_arg[v]] + G.par(keops_par_arg[v]) * keops_par_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
   }
@@ -564,8 +597,6 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
   float m_run = ninf;   // running maximum of output row `col` (identical in both halves)
   float l_run = 0.f;    // this lane's share of sum_j exp(F' - m_run)
 
-  const i64 jbeg = (i64)blockIdx.y * P.slab_len;
-  const i64 jend = keops_min(P.ny, jbeg + P.slab_len);
   const T* vsrc = P.arg[CHK_FV_ARG];
 
   constexpr int CH = CHK_ROWBYTES / 16;
@@ -574,23 +605,26 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
   uint4 pf[NPF];
   T pfv[NPV];
   float pfn = 0.f;
-  auto prefetch = [&](i64 j0) {
+  auto prefetch = [&](i64 j0, i64 jend) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
-    const uint4* src = reinterpret_cast<const uint4*>(P.ys + j0 * 2 * CHK_DPAD);
+    const i64 jy = G.col(CHK_YARG, j0), jv = G.col(CHK_FV_ARG, j0);
+    const uint4* src = reinterpret_cast<const uint4*>(P.ys + jy * 2 * CHK_DPAD);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * CHK_BLOCK;
       pf[u] = (e < n * CH) ? src[e] : make_uint4(0u, 0u, 0u, 0u);
     }
-    if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[j0 + tid] : 0.f;
+    if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[jy + tid] : 0.f;
 #pragma unroll
     for (int u = 0; u < NPV; u++) {
       const int e = tid + u * CHK_BLOCK;
       const int row = e / CHK_SVS, c = e - row * CHK_SVS;
-      pfv[u] = (row < n && c < CHK_FV_DIM) ? vsrc[(j0 + row) * CHK_FV_DIM + c] : (T)0;
+      pfv[u] = (row < n && c < CHK_FV_DIM) ? vsrc[(jv + row) * CHK_FV_DIM + c] : (T)0;
     }
   };
-  if (jbeg < jend) prefetch(jbeg);
+  // folds the reduced rows [jbeg, jend) into the running maxima, sums and register tiles
+  auto sweep = [&](i64 jbeg, i64 jend) {
+  if (jbeg < jend) prefetch(jbeg, jend);
   for (i64 j0 = jbeg; j0 < jend; j0 += CHK_TJ) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
     __syncthreads();
@@ -606,7 +640,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
 #pragma unroll
     for (int v = 0; v < KEOPS_NCOLVARS; v++) {
       const int dim = keops_col_dim[v];
-      const T* src = P.arg[keops_col_arg[v]] + j0 * dim;
+      const T* src = P.arg[keops_col_arg[v]] + G.col(keops_col_arg[v], j0) * dim;
       for (int e = tid; e < n * dim; e += CHK_BLOCK) {
         const int row = e / dim, c = e - row * dim;
         yo_s[row * CHK_DY + keops_col_off[v] + c] = src[e];
@@ -618,7 +652,8 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
       if (e < CHK_TJ * CHK_SVS) bt[e] = pfv[u];
     }
     __syncthreads();
-    if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ);
+    if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ, jend);
+    if (!wave_live) continue;
 
     chk_f32x16 s;
     if (CHK_MODE == 0) {
@@ -689,11 +724,17 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
         acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(pv, bt[r * CHK_SVS + 32 * b + col], acc[b], 0, 0, 0);
     }
   }
+  };
+#if KEOPS_MC_RANGES
+  G.for_each_range(P.rt, sweep);
+#else
+  sweep((i64)blockIdx.y * P.slab_len, keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len));
+#endif
 
   // results of this slab: [m, (l,) O_0 .. O_{dv-1}] per output row
   l_run += __shfl_xor(l_run, 32);
   T* dst = P.nslabs > 1 ? P.partial + (i64)blockIdx.y * P.nx * KEOPS_DIMRED : P.out;
-  if (half == 0 && row0 + col < P.nx) {
+  if (half == 0 && row0 + col < G.row_end) {
     T* o = dst + (row0 + col) * KEOPS_DIMRED;
     o[0] = m_run;
     if (CHK_SM_ONE) o[1] = l_run;
@@ -706,7 +747,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int ir = 8 * (r >> 2) + (r & 3);
-        if (ibase + ir < P.nx && 32 * b + col < CHK_FV_DIM) o[(i64)ir * KEOPS_DIMRED + 32 * b] = acc[b][r];
+        if (ibase + ir < G.row_end && 32 * b + col < CHK_FV_DIM) o[(i64)ir * KEOPS_DIMRED + 32 * b] = acc[b][r];
       }
     }
   }
@@ -732,5 +773,23 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_softmax_reduce(const
     s += keops_red_exp(mk - mm) * P.partial[(i64)k * total + e];
   }
   P.out[e] = s;
+}
+#endif
+
+#if KEOPS_MC_RANGES
+// block-sparse mode: output rows that belong to no row range keep the neutral element of the reduction
+extern "C" __global__ void __launch_bounds__(256) keops_chk_fill_neutral(const ChkParams P) {
+  const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (i >= P.nx) return;
+#if defined(CHK_FINAL) && CHK_FINAL
+  for (int d = 0; d < CHK_FV_DIM; d++) P.out[i * CHK_FV_DIM + d] = (T)0;
+#elif defined(CHK_SOFTMAX) && CHK_SOFTMAX
+  P.out[i * KEOPS_DIMRED] = -__builtin_huge_valf();
+  for (int d = 1; d < KEOPS_DIMRED; d++) P.out[i * KEOPS_DIMRED + d] = (T)0;
+#else
+  KeopsAcc<TACC> acc;
+  acc.init();
+  acc.finalize(P.out + i * KEOPS_DIMOUT);
+#endif
 }
 #endif

@@ -61,3 +61,86 @@ __device__ __forceinline__ double keops_fmax(double a, double b) { return __buil
 template <typename A> __device__ __forceinline__ A keops_inf() { return (A)__builtin_huge_valf(); }
 
 __device__ __forceinline__ i64 keops_min(i64 a, i64 b) { return a < b ? a : b; }
+
+// ---- block-sparse / batched geometry of the matrix-core schemes ------------------------------------
+//
+// Same tables as the generic block-sparse kernel (keopscore/keopscore/mapreduce/gpu/GpuReduc1D_ranges.py:74-173,
+// keopscore/keopscore/binders/nvrtc/keops_nvrtc.cpp:152-248): one lookup entry (range id, first row,
+// end row) per workgroup, the reduced-index ranges of every row range, and, with batch dimensions, the
+// first-row offset of every argument for every workgroup (here indexed by argument number).
+// A module built with KEOPS_MC_RANGES = 0 ignores the tables: every helper folds to the dense case.
+#ifndef KEOPS_MC_RANGES
+#define KEOPS_MC_RANGES 0
+#endif
+
+struct KeopsRangeTables {
+  const i64* lookup;    // [nblocks][3] = (range id, first row, end row)
+  const i64* slices_x;  // end slice of every row range
+  const i64* ranges_y;  // [*][2] reduced-index ranges
+  const i64* offsets;   // batch mode: [nblocks][nargs] first-row offsets by argument
+  int nbatchdims;
+  int nargs;
+};
+
+// rows owned by a workgroup and the index arithmetic of its arguments
+struct KeopsTileGeom {
+  i64 row_first, row_end;  // global output rows [row_first, row_end) of this workgroup
+  i64 slice_first, slice_end;
+  const i64* offs;         // batch mode: this workgroup's per-argument offsets, else null
+
+  __device__ __forceinline__ void init(const KeopsRangeTables& R, i64 nx, int rows_per_block) {
+#if KEOPS_MC_RANGES
+    const i64 bid = blockIdx.x;
+    const i64 range_id = R.lookup[3 * bid];
+    row_first = R.lookup[3 * bid + 1];
+    row_end = R.lookup[3 * bid + 2];
+    slice_first = range_id < 1 ? 0 : R.slices_x[range_id - 1];
+    slice_end = R.slices_x[range_id];
+    offs = R.nbatchdims > 0 ? R.offsets + (i64)R.nargs * bid : nullptr;
+#else
+    row_first = (i64)blockIdx.x * rows_per_block;
+    row_end = keops_min(nx, row_first + rows_per_block);
+    slice_first = slice_end = 0;
+    offs = nullptr;
+#endif
+  }
+  // row of argument `arg` that holds global output row q / reduced row j / the parameter
+  __device__ __forceinline__ i64 row(int arg, i64 q) const {
+#if KEOPS_MC_RANGES
+    return offs ? offs[arg] + (q - row_first) : q;
+#else
+    return q;
+#endif
+  }
+  __device__ __forceinline__ i64 col(int arg, i64 j) const {
+#if KEOPS_MC_RANGES
+    return offs ? offs[arg] + j : j;
+#else
+    return j;
+#endif
+  }
+  __device__ __forceinline__ i64 par(int arg) const {
+#if KEOPS_MC_RANGES
+    return offs ? offs[arg] : 0;
+#else
+    return 0;
+#endif
+  }
+  // calls sweep(jbeg, jend) for every maximal run of contiguous reduced-index ranges of this workgroup;
+  // with batch dimensions the single range of the batch is swept as [0, length) (batch-relative indices,
+  // the offsets move the arguments)
+  template <typename F> __device__ __forceinline__ void for_each_range(const KeopsRangeTables& R, F&& sweep) const {
+#if KEOPS_MC_RANGES
+    if (slice_first >= slice_end) return;
+    i64 start_y = R.ranges_y[2 * slice_first];
+    for (i64 index = slice_first; index < slice_end; index++) {
+      if (index + 1 >= slice_end || R.ranges_y[2 * index + 2] != R.ranges_y[2 * index + 1]) {
+        const i64 end_y = R.ranges_y[2 * index + 1];
+        if (offs) sweep((i64)0, end_y - start_y);
+        else sweep(start_y, end_y);
+        if (index + 1 < slice_end) start_y = R.ranges_y[2 * index + 2];
+      }
+    }
+#endif
+  }
+};

@@ -41,6 +41,7 @@ struct FinParams {
   i64 slab_len;    // reduced rows per slab (multiple of FIN_TJ)
   int nslabs;
   int pad_;
+  KeopsRangeTables rt;  // block-sparse / batch geometry (KEOPS_MC_RANGES)
   const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
 };
 
@@ -50,9 +51,12 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
-  const i64 row0 = (i64)blockIdx.x * FIN_QB + wave * 32;  // first output row of this wavefront
+  KeopsTileGeom G;
+  G.init(P.rt, P.nx, FIN_QB);
+  const i64 row0 = G.row_first + wave * 32;  // first output row of this wavefront
+  const bool wave_live = row0 < G.row_end;   // a wavefront without rows only helps staging the tiles
   i64 q = row0 + col;
-  if (q >= P.nx) q = P.nx - 1;  // clamped rows compute, never store
+  if (q >= G.row_end) q = G.row_end - 1;  // clamped rows compute, never store
   const int cb0 = blockIdx.z * FIN_NB;                      // first column block of this workgroup
   const int c0 = cb0 * 32;                                  // first column
   const int ncols = (int)keops_min((i64)FIN_VS, (i64)FIN_DV - c0);
@@ -60,14 +64,14 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
   T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NROWVARS; v++) {
-    const T* src = P.arg[keops_row_arg[v]] + q * keops_row_dim[v];
+    const T* src = P.arg[keops_row_arg[v]] + G.row(keops_row_arg[v], q) * keops_row_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
   }
   T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NPARVARS; v++) {
-    const T* src = P.arg[keops_par_arg[v]];
+    const T* src = P.arg[keops_par_arg[v]] + G.par(keops_par_arg[v]) * keops_par_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
   }
@@ -92,7 +96,7 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int ir = 8 * (r >> 2) + (r & 3);
-        if (ibase + ir < P.nx && d < FIN_DV) {
+        if (ibase + ir < G.row_end && d < FIN_DV) {
           T* oo = o + (i64)ir * FIN_DV + 32 * b;
           *oo = first ? acc[b][r] : *oo + acc[b][r];
         }
@@ -102,24 +106,25 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
     first = false;
   };
 
-  const i64 jbeg = (i64)blockIdx.y * P.slab_len;
-  const i64 jend = keops_min(P.ny, jbeg + P.slab_len);
   const T* vsrc = P.arg[FIN_VARG];
 
   // software pipeline: the v rows of tile t+1 travel to registers while tile t is consumed
   constexpr int NPF = (FIN_TJ * FIN_VS + FIN_BLOCK - 1) / FIN_BLOCK;
   T pf[NPF];
-  auto prefetch = [&](i64 j0) {
+  auto prefetch = [&](i64 j0, i64 jend) {
     const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
+    const i64 jv = G.col(FIN_VARG, j0);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * FIN_BLOCK;
       const int row = e / FIN_VS, c = e - row * FIN_VS;
-      pf[u] = (row < n && c < ncols) ? vsrc[(j0 + row) * FIN_DV + c0 + c] : (T)0;  // zero rows/columns past the end
+      pf[u] = (row < n && c < ncols) ? vsrc[(jv + row) * FIN_DV + c0 + c] : (T)0;  // zero rows/columns past the end
     }
   };
-  if (jbeg < jend) prefetch(jbeg);
   int since_fold = 0;
+  // folds the reduced rows [jbeg, jend) into the register tiles
+  auto sweep = [&](i64 jbeg, i64 jend) {
+  if (jbeg < jend) prefetch(jbeg, jend);
   for (i64 j0 = jbeg; j0 < jend; j0 += FIN_TJ) {
     const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
     __syncthreads();  // the previous tile has been consumed by every wavefront
@@ -131,14 +136,15 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
 #pragma unroll
     for (int v = 0; v < KEOPS_NCOLVARS; v++) {
       const int dim = keops_col_dim[v];
-      const T* src = P.arg[keops_col_arg[v]] + j0 * dim;
+      const T* src = P.arg[keops_col_arg[v]] + G.col(keops_col_arg[v], j0) * dim;
       for (int e = tid; e < n * dim; e += FIN_BLOCK) {
         const int row = e / dim, c = e - row * dim;
         ys[row * FIN_DY + keops_col_off[v] + c] = src[e];
       }
     }
     __syncthreads();
-    if (j0 + FIN_TJ < jend) prefetch(j0 + FIN_TJ);
+    if (j0 + FIN_TJ < jend) prefetch(j0 + FIN_TJ, jend);
+    if (!wave_live) continue;
 
     // operands of step s+1 (pair value and v entries) are fetched while the MFMAs of step s execute
     auto operands = [&](int s, float& fv, float (&bv)[FIN_NB]) {
@@ -179,6 +185,12 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
     }
 #endif
   }
+  };
+#if KEOPS_MC_RANGES
+  G.for_each_range(P.rt, sweep);
+#else
+  sweep((i64)blockIdx.y * P.slab_len, keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len));
+#endif
   fold();
 }
 
@@ -191,3 +203,11 @@ extern "C" __global__ void __launch_bounds__(256) keops_fin_reduce(const FinPara
   for (int k = 1; k < P.nslabs; k++) s += P.partial[(i64)k * total + e];
   P.out[e] = s;
 }
+
+#if KEOPS_MC_RANGES
+// block-sparse mode: output rows that belong to no row range are zero
+extern "C" __global__ void __launch_bounds__(256) keops_fin_fill_neutral(const FinParams P) {
+  const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (e < P.nx * FIN_DV) P.out[e] = (T)0;
+}
+#endif

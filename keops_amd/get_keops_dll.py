@@ -187,7 +187,7 @@ def match_chunk(red, dtype, map_reduce_id, use_fast_math):
     from .formulas import ops as O
     from .formulas.reductions import KIND_LSE, KIND_SUM
 
-    if red.kind not in (KIND_SUM, KIND_LSE) or dtype != "float" or not use_fast_math or "_ranges" in map_reduce_id:
+    if red.kind not in (KIND_SUM, KIND_LSE) or dtype != "float" or not use_fast_math:
         return None
     found = []
     for node in red.formula.walk():
@@ -211,8 +211,9 @@ def match_chunk(red, dtype, map_reduce_id, use_fast_math):
     return (mode, node) + ((a, b) if a.cat == red.tagI else (b, a))
 
 
-def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
-    """Module source for the matrix-core chunked scheme (kernels/keops_chunk_mfma.h)."""
+def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=False):
+    """Module source for the matrix-core chunked scheme (kernels/keops_chunk_mfma.h); ``irregular``: the
+    block-sparse / batched variant (GpuReduc1D_ranges_chunks.py:21-183)."""
     from .formulas import ops as O
     from .formulas.reductions import Reduction
 
@@ -226,7 +227,8 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
     if (red.kind == KIND_SUM and dtypeacc == "float" and sum_scheme in ("block_sum", "direct_sum")
             and post.name == "Mult" and len(post.children) == 2):
         for g, v in (post.children, post.children[::-1]):
-            if g.dim == 1 and isinstance(v, O.Var) and v.cat == 1 - red.tagI and v.dim == post.dim and v.dim <= 64:
+            if (g.dim == 1 and isinstance(v, O.Var) and v.cat == 1 - red.tagI and v.dim == post.dim
+                    and v.dim <= (64 if xvar.dim > 128 else 128)):
                 final = (g, v)
                 break
     # post-chunk formulas [F'(s, ...), v_j] or [F', 1, v_j] of a float32 log-sum-exp family reduction: online softmax
@@ -279,9 +281,10 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs):
                 sizeof_acc=8 if dtypeacc == "double" else 4, nrowvars=len(layout.rowvars) + 1,
                 ncolvars=len(layout.colvars) + ncol_extra, nparvars=len(layout.parvars), chk_d=D, chk_dpad=dpad,
                 chk_mode=mode, chk_qb=32 * waves, chk_final=int(final is not None), chk_softmax=int(softmax is not None),
-                nops=L.count_ops(outs))
+                chk_xarg=xvar.ind, chk_yarg=yvar.ind, ranges=int(irregular), nops=L.count_ops(outs))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
-           f"typedef float T;\ntypedef {dtypeacc} TACC;", '#include "keops_common.h"']
+           f"typedef float T;\ntypedef {dtypeacc} TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
+           '#include "keops_common.h"']
     defs = dict(
         KEOPS_NARGS=nargs, CHK_D=D, CHK_DPAD=dpad, CHK_MODE=mode, CHK_XARG=xvar.ind, CHK_YARG=yvar.ind, CHK_WAVES=waves,
         KEOPS_DIMX=layout.dimx, KEOPS_DIMY=layout.dimy, KEOPS_DIMY_PAD=dimy_pad, KEOPS_DIMP=layout.dimp,
@@ -317,7 +320,7 @@ def match_final(red, dtype, dtypeacc, sum_scheme, map_reduce_id):
     from .formulas import ops as O
     from .formulas.reductions import KIND_SUM
 
-    if red.kind != KIND_SUM or dtype != "float" or dtypeacc != "float" or "_ranges" in map_reduce_id:
+    if red.kind != KIND_SUM or dtype != "float" or dtypeacc != "float":
         return None
     if sum_scheme not in ("block_sum", "direct_sum"):
         return None
@@ -334,8 +337,9 @@ def match_final(red, dtype, dtypeacc, sum_scheme, map_reduce_id):
     return None
 
 
-def generate_final_plugin(red, match, sum_scheme, nargs):
-    """Module source for the matrix-core final-product scheme (kernels/keops_final_mfma.h)."""
+def generate_final_plugin(red, match, sum_scheme, nargs, irregular=False):
+    """Module source for the matrix-core final-product scheme (kernels/keops_final_mfma.h); ``irregular``: the
+    block-sparse / batched variant (GpuReduc1D_ranges_finalchunks.py:20-91)."""
     f, vvar = match
 
     class _Inner:  # what VarLayout needs: the scalar kernel with the reduction's orientation
@@ -357,9 +361,11 @@ def generate_final_plugin(red, match, sum_scheme, nargs):
     pa, pd, po = VarLayout.table(layout.parvars)
     meta = dict(scheme="final", block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
                 sizeof_acc=4, nrowvars=len(layout.rowvars), ncolvars=len(layout.colvars) + (0 if vvar in layout.colvars else 1),
-                nparvars=len(layout.parvars), fin_dv=vvar.dim, fin_nb=nb, fin_nz=nz, fin_qb=32 * waves, nops=L.count_ops(outs))
+                nparvars=len(layout.parvars), fin_dv=vvar.dim, fin_nb=nb, fin_nz=nz, fin_qb=32 * waves, ranges=int(irregular),
+                nops=L.count_ops(outs))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
-           "typedef float T;\ntypedef float TACC;", '#include "keops_common.h"']
+           "typedef float T;\ntypedef float TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
+           '#include "keops_common.h"']
     defs = dict(
         KEOPS_NARGS=nargs, FIN_DV=vvar.dim, FIN_VARG=vvar.ind, FIN_NB=nb, FIN_WAVES=waves, FIN_TJ=tj,
         FIN_PERIOD=config.final_period, FIN_BLOCKSUM=int(sum_scheme == "block_sum"),
@@ -410,6 +416,7 @@ def get_keops_dll(
     if tagZero:
         target, tag, src_file = "", "zero", ""
     else:
+        irregular = "_ranges" in map_reduce_id
         knn = match_knn_sqdist(red, dtype, map_reduce_id) if enable_chunks else None
         chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
         fin = None
@@ -419,16 +426,16 @@ def get_keops_dll(
             source, meta = generate_knn_plugin(red, knn[0], knn[1], nargs)
             use_chunk_mode = 3  # matrix-core filter scheme (no counterpart among the reference's chunk modes)
         elif fin is not None:
-            source, meta = generate_final_plugin(red, fin, sum_scheme_string, nargs)
+            source, meta = generate_final_plugin(red, fin, sum_scheme_string, nargs, irregular=irregular)
             use_chunk_mode = 2  # as the reference's final-chunk mode (get_keops_dll.py:101-108)
         elif chk is not None:
-            source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs)
+            source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs, irregular=irregular)
             use_chunk_mode = 1 if source is not None else 0
         else:
             source = None
         if source is None:
             source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint,
-                                           irregular="_ranges" in map_reduce_id)
+                                           irregular=irregular)
         tag = hashlib.sha256((source + binder.templates_digest() + str(use_fast_math)).encode()).hexdigest()[:16]
         folder = config.get_build_folder()
         target = os.path.join(folder, f"hsaco_{tag}")
