@@ -35,7 +35,7 @@ MEASURED_TRAFFIC_BYTES = {
     # profiles/keops_conv_dense__gauss_1m_dv1.md: FETCH_SIZE 162134 KiB x 2.0 (copy calibration) + WRITE_SIZE 66406 KiB
     "gauss_1m_dv1": int((162134 * 2.0 + 66406) * 1024),
     # profiles/keops_knn_filter__knn_d64.md: dominant kernel keops_knn_filter
-    "knn_d64": int(2 * (390498 * 2.0 + 36649) * 1024),
+    "knn_d64": int(2 * (391283 * 2.0 + 43486) * 1024),
     # profiles/keops_chk_final__laplace_d256.md
     "laplace_d256": int((4292480 * 2.0 + 650811) * 1024),
     # profiles/keops_fin_main__gauss_dv256.md

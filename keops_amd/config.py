@@ -41,6 +41,8 @@ knn_max_waves = int(os.environ.get("KEOPS_AMD_KNN_WAVES", 8))     # wavefronts p
 knn_filter_waves = int(os.environ.get("KEOPS_AMD_KNN_FWAVES", 16))  # fixed-threshold filter: wavefronts per workgroup
 knn_filter_qsets = int(os.environ.get("KEOPS_AMD_KNN_FQSETS", 2))   # and 32-query operand sets per wavefront
 knn_sample = int(os.environ.get("KEOPS_AMD_KNN_SAMPLE", 16))            # sampling pass: every 16th reference
+knn_sample_waves = int(os.environ.get("KEOPS_AMD_KNN_SWAVES", 8))  # sampling pass: wavefronts per workgroup
+knn_sample_qsets = int(os.environ.get("KEOPS_AMD_KNN_SQSETS", 1))   # and 32-query operand sets per wavefront
 knn_lds_budget = 150 * 1024                                        # LDS bytes a KNN workgroup may use (160 KB per CU)
 knn_qsets = int(os.environ.get("KEOPS_AMD_KNN_QSETS", 1))          # 32-query operand sets per wavefront (<= 2)
 

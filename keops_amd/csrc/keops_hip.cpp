@@ -481,11 +481,12 @@ struct KnnHeader {
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
-// number of reference slabs that gives about `per_cu` workgroups per compute unit
-int64_t pick_slabs(int64_t qblocks, int64_t nr, int64_t tile, int64_t cus, int64_t per_cu, int forced_min) {
+// number of reference slabs that gives about `per_cu` workgroups per compute unit; a slab holds at least
+// min_tiles staged tiles (adaptive lists restart in every slab: longer slabs; fixed thresholds: short ones are fine)
+int64_t pick_slabs(int64_t qblocks, int64_t nr, int64_t tile, int64_t cus, int64_t per_cu, int forced_min, int64_t min_tiles = 16) {
   int64_t n = std::max<int64_t>(1, (per_cu * cus) / std::max<int64_t>(1, qblocks));
   n = std::max<int64_t>(n, forced_min);
-  n = std::min<int64_t>(n, std::max<int64_t>(1, nr / (16 * tile)));
+  n = std::min<int64_t>(n, std::max<int64_t>(1, nr / (min_tiles * tile)));
   return std::max<int64_t>(1, std::min<int64_t>(n, 1024));
 }
 
@@ -503,31 +504,44 @@ int64_t balance_slabs(int64_t blocks, int64_t n0, int64_t nmax, int64_t slots) {
   return best;
 }
 
+// smallest sample of the threshold estimate and smallest reference set handled in two phases (tuning knobs)
+int64_t knn_min_sample() {
+  static const int64_t v = [] { const char* e = getenv("KEOPS_HIP_KNN_MIN_SAMPLE"); return e ? std::max<int64_t>(64, atoll(e)) : 4096; }();
+  return v;
+}
+int64_t knn_two_phase_min_refs() {
+  static const int64_t v = [] { const char* e = getenv("KEOPS_HIP_KNN_TWO_PHASE_MIN"); return e ? std::max<int64_t>(1024, atoll(e)) : 32768; }();
+  return v;
+}
+
 int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr, void* out, int tag1D2D,
                hipStream_t stream) {
   const int64_t D = m.meta_int("knn_d", 0), DP = m.meta_int("knn_dpad", 0), K = m.meta_int("knn_k", 0);
   const int64_t QB = m.meta_int("knn_qb", 256), TJ = m.tile_j;
-  const int64_t FW = m.meta_int("knn_fwaves", 16), FQW = 32 * m.meta_int("knn_fqsets", 2), SAMPLE = m.meta_int("knn_sample", 16);
+  const int64_t FW = m.meta_int("knn_fwaves", 16), FQW = 32 * m.meta_int("knn_fqsets", 2);
   const int64_t FQB = FW * FQW;
   if (D <= 0 || DP <= 0 || K <= 0) return fail(-1, "corrupt knn module metadata");
   if (nr > 2147483647LL) return fail(-1, "too many reference rows for 32-bit indices");
-  const bool two_phase = nr >= 32768 && nr / SAMPLE >= 8 * K && nq >= 1024;
+  // sampling step of the threshold estimate: every 16th reference for large sets, a sample of >= ~4096 rows otherwise
+  const int64_t SAMPLE = std::max<int64_t>(2, std::min<int64_t>(m.meta_int("knn_sample", 16), nr / knn_min_sample()));
+  const bool two_phase = nr >= knn_two_phase_min_refs() && nr / SAMPLE >= 8 * K && nq >= 1024;
   const int64_t nsample = two_phase ? (nr + SAMPLE - 1) / SAMPLE : 0;
 
   // adaptive pass: over the sample (two-phase) or over everything
   const int64_t a_nr = two_phase ? nsample : nr;
-  const int64_t a_qblocks = (nq + QB - 1) / QB;
-  int64_t a_slabs = pick_slabs(a_qblocks, a_nr, TJ, m.cu_count, 2, tag1D2D == 1 && !two_phase ? 2 : 1);
+  const int64_t SQB = m.meta_int("knn_sqb", QB), SBLOCK = m.meta_int("knn_sblock", m.block);
+  const int64_t a_qblocks = (nq + (two_phase ? SQB : QB) - 1) / (two_phase ? SQB : QB);
+  int64_t a_slabs = pick_slabs(a_qblocks, a_nr, TJ, m.cu_count, 2, tag1D2D == 1 && !two_phase ? 2 : 1, 16);
   int64_t a_len = ((a_nr + a_slabs - 1) / a_slabs + TJ - 1) / TJ * TJ;
   a_slabs = std::max<int64_t>(1, (a_nr + a_len - 1) / a_len);
   // filter pass
   const int64_t f_qblocks = (nq + FQB - 1) / FQB;
-  int64_t f_slabs = pick_slabs(f_qblocks, nr, TJ, m.cu_count, 2, 1);
+  int64_t f_slabs = pick_slabs(f_qblocks, nr, TJ, m.cu_count, 2, 1, 4);
   // one filter workgroup fills a CU and all of them take the same time.  With at least 8 slabs the filter runs
   // in two stages (every 4th slab, then the others, with thresholds refined in between): both grids should
   // be close to whole rounds over the CUs
   {
-    const int64_t cap = std::max<int64_t>(1, nr / (16 * TJ));
+    const int64_t cap = std::max<int64_t>(1, nr / (4 * TJ));
     int64_t best = f_slabs;
     double best_eff = 0.0;
     for (int64_t n = f_slabs; n <= std::max(f_slabs, std::min<int64_t>(std::max<int64_t>(4 * f_slabs, 24), cap)); n++) {
@@ -547,7 +561,7 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   const int64_t fa_slabs = staged ? (f_slabs + 3) / 4 : f_slabs, fb_slabs = f_slabs - fa_slabs;
   const int64_t nlogs = f_qblocks * f_slabs * FW;
   // expected survivors per query: SAMPLE * K (the sample's K-th neighbour is about the (SAMPLE*K)-th overall)
-  const int64_t logcap = two_phase ? align_up((size_t)(4 * FQW * SAMPLE * K / f_slabs + 512), 64) : 0;
+  const int64_t logcap = two_phase ? align_up((size_t)(5 * FQW * SAMPLE * K / f_slabs + 512), 64) : 0;
   const int64_t list_slabs = std::max<int64_t>(a_slabs, two_phase ? f_slabs : 1);
 
   // workspace layout
@@ -564,7 +578,7 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   const size_t o_logcount = take((size_t)(two_phase ? nlogs : 0) * 4), o_log = take((size_t)(two_phase ? nlogs : 0) * logcap * 8);
   if (int rc = m.partial.reserve(off)) return rc;
   char* ws = (char*)m.partial.ptr;
-  struct Packed { KnnHeader h; int64_t extra[3]; } p{};
+  struct Packed { KnnHeader h; int64_t extra[4]; } p{};
   KnnHeader& h = p.h;
   h.nq = nq; h.nr = nr; h.xq = xq; h.yr = yr;
   h.xh = ws + o_xh; h.yh = ws + o_yh; h.xkey = ws + o_xkey; h.ykey = ws + o_ykey; h.colsum = ws + o_colsum; h.colpart = ws + o_colpart;
@@ -584,9 +598,11 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   if (int rc = run("keops_knn_prep", (unsigned)((nr * lpr + 255) / 256), 1, 256, with_int(1))) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
 
-  auto adaptive = [&](int64_t refs, void* yh, void* ykey, int step, int64_t slabs, int64_t len) -> int {
+  auto adaptive = [&](const char* kernel, int64_t refs, void* yh, void* ykey, int step, int64_t slabs, int64_t len) -> int {
     h.nr = refs; h.yh = yh; h.ykey = ykey; h.ref_step = step; h.nslabs = (int32_t)slabs; h.slab_len = len;
-    return run("keops_knn_main", (unsigned)a_qblocks, (unsigned)slabs, (unsigned)m.block, HS);
+    const bool sampling = step > 1;
+    const int64_t qb = sampling ? SQB : QB;
+    return run(kernel, (unsigned)((nq + qb - 1) / qb), (unsigned)slabs, (unsigned)(sampling ? SBLOCK : m.block), HS);
   };
   bool done = false;
   if (two_phase) {
@@ -595,9 +611,10 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
     std::memcpy(&p.extra[0], &gargs[0], 8);
     std::memcpy(&p.extra[1], &gargs[1], 8);
     p.extra[2] = nsample;
+    p.extra[3] = SAMPLE;  // read as a 32-bit integer (little endian)
     const int64_t chunks = nsample * (RW / 8);
-    if (int rc = run("keops_knn_gather_sample", (unsigned)((chunks + 255) / 256), 1, 256, HS + 24)) return rc;
-    if (int rc = adaptive(nsample, ws + o_yhs, ws + o_ykeys, (int)SAMPLE, a_slabs, a_len)) return rc;
+    if (int rc = run("keops_knn_gather_sample", (unsigned)((chunks + 255) / 256), 1, 256, HS + 32)) return rc;
+    if (int rc = adaptive("keops_knn_sample", nsample, ws + o_yhs, ws + o_ykeys, (int)SAMPLE, a_slabs, a_len)) return rc;
     auto with_2int = [&](int a, int b) { int v[2] = {a, b}; std::memcpy(p.extra, v, 8); return HS + 8; };
     if (int rc = run("keops_knn_thresholds", (unsigned)((nq + 255) / 256), 1, 256, with_2int(0, 0))) return rc;
     // (b) fixed-threshold filter, survivors logged per wavefront; (c) exact replay of the logs.
@@ -619,11 +636,11 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
     done = *(volatile int*)m.pinned == 0;  // a log overflowed (pathological ties): redo adaptively
   }
   if (!done) {
-    int64_t slabs = pick_slabs(a_qblocks, nr, TJ, m.cu_count, 2, tag1D2D == 1 ? 2 : 1);
+    int64_t slabs = pick_slabs((nq + QB - 1) / QB, nr, TJ, m.cu_count, 2, tag1D2D == 1 ? 2 : 1);
     slabs = std::min<int64_t>(slabs, list_slabs);
     int64_t len = ((nr + slabs - 1) / slabs + TJ - 1) / TJ * TJ;
     slabs = std::max<int64_t>(1, (nr + len - 1) / len);
-    if (int rc = adaptive(nr, ws + o_yh, ws + o_ykey, 1, slabs, len)) return rc;
+    if (int rc = adaptive("keops_knn_main", nr, ws + o_yh, ws + o_ykey, 1, slabs, len)) return rc;
   }
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
   if (int rc = run("keops_knn_merge", (unsigned)((nq + 255) / 256), 1, 256, HS)) return rc;

@@ -30,8 +30,10 @@
 //   4. The reference axis can be cut in slabs (blockIdx.y); keops_knn_merge merges the per-slab
 //      lists under the same key and writes the output in the reference's layout.
 //   5. Large problems run in two phases so that the matrix-core sweep never waits for a re-rank:
-//      (a) the adaptive kernel of steps 2-3 runs on every KNN_SAMPLE-th reference only; the K-th
-//      distance it finds is an upper bound of the final one and becomes a *fixed* threshold;
+//      (a) keops_knn_sample sweeps every step-th reference (step <= KNN_SAMPLE) and keeps, per query, the K
+//      smallest *upper bounds* U = L + 2c(|x^|^2 + |y^|^2) of the pair distances, straight from the
+//      matrix-core values (no exact distance, no memory access per candidate); the K-th of them bounds the
+//      final K-th distance from above and becomes a *fixed* threshold;
 //      (b) keops_knn_filter sweeps all references against the fixed thresholds and only logs the
 //      surviving (query, reference) pairs, each wavefront in a private region of global memory (no
 //      atomics, no list updates); (c) keops_knn_rerank replays every log with the exact distance and
@@ -42,7 +44,8 @@
 //      references.
 //
 // The plug-in defines: T (float), KEOPS_NARGS, KNN_D, KNN_DPAD (D rounded up to 16), KNN_K,
-// KEOPS_RED_KEEP, KEOPS_DIMOUT, KNN_QSETS, KNN_WAVES (wavefronts per workgroup), KNN_TJ, KNN_SPLIT.
+// KEOPS_RED_KEEP, KEOPS_DIMOUT, KNN_QSETS, KNN_WAVES (wavefronts per workgroup), KNN_TJ, KNN_SPLIT,
+// KNN_FWAVES / KNN_FQSETS (filter geometry), KNN_SWAVES / KNN_SQSETS (sampling pass geometry).
 #pragma once
 #include "keops_common.h"
 
@@ -67,6 +70,8 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float knn_f32x4;
 #define KNN_C 0.0082f
 #endif
 #define KNN_DELTA 2e-5f
+// distance of the upper bound U to the lower bound L of a pair: U - L = 2c (|x^|^2 + |y^|^2) = KNN_E (xkey + ykey)
+#define KNN_E (2.0f * KNN_C / (1.0f - KNN_C))
 #define KNN_FLT_MAX 3.402823466e38f
 
 struct KnnParams {
@@ -244,9 +249,18 @@ __device__ __forceinline__ void knn_insert(float* lv, int* li, float d, int j) {
 
 // MODE 0 (adaptive): thresholds follow the K-lists, full queues are re-examined at once.
 // MODE 1 (fixed thresholds): full queues are appended to the wavefront's log in global memory.
+// MODE 2 (threshold estimate): adaptive, but nothing is re-examined: the K-lists hold the upper bounds
+//   U = L + KNN_E (xkey + ykey) of the pair distances, computed from the matrix-core values alone (no memory
+//   access per candidate); their K-th smallest bounds the K-th exact distance from above.  Lane l of a
+//   wavefront owns the sorted list of query l in registers (one v_med3_f32 per entry and insertion).
+//   Candidates wait in the wavefront's queue; when 64 are waiting they are dealt to small per-query bins in
+//   LDS (`cand`, counters in `owner`; one LDS atomic per candidate, all 64 in flight together) and every
+//   owner folds its bin into its list.
+#define KNN_BIN 8  // candidates per query bin
 template <int MODE, int WAVES, int QSETS>
 __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys, float* ykey_s, float (*lv)[KNN_K],
-                                          int (*li)[KNN_K], int* owner, int (*qq)[64], int (*qj)[64]) {
+                                          int (*li)[KNN_K], int* owner, int (*qq)[64], int (*qj)[64],
+                                          float* cand = nullptr) {
   constexpr int BLOCK = 64 * WAVES, QW = 32 * QSETS, QB = WAVES * QW;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
@@ -270,7 +284,7 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
     }
     xk[h] = P.xkey[q];
     // finite start value: padded rows carry an infinite key and never pass
-    if (MODE == 0) t[h] = valid[h] ? KNN_FLT_MAX : -inf;
+    if (MODE != 1) t[h] = valid[h] ? KNN_FLT_MAX : -inf;
     else t[h] = valid[h] ? P.thr[q] : -inf;
   }
   if (MODE == 0) {
@@ -279,6 +293,57 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
       (&li[0][0])[e] = 0;
     }
   }
+  // MODE 2: sorted list of upper bounds of query `lane` of this wavefront (lanes < QW), bins empty
+  float lst[MODE == 2 ? KNN_K : 1];
+  volatile int* bin_n = MODE == 2 ? owner + wave * QW : nullptr;
+  volatile float* bin_v = MODE == 2 ? cand + wave * QW * KNN_BIN : nullptr;
+  if (MODE == 2) {
+#pragma unroll
+    for (int k = 0; k < KNN_K; k++) lst[k] = inf;
+    if (lane < QW) bin_n[lane] = 0;
+    __threadfence_block();
+  }
+  // MODE 2: the nb queued upper bounds are dealt to the bins of their queries, every owner lane folds its bin
+  // into its list (a bin that overflows is emptied and refilled), then all lanes get the new thresholds
+  auto drain = [&](int nb) {
+    __threadfence_block();
+    bool pending = lane < nb;
+    int ql = 0;
+    float u = inf;
+    if (pending) {
+      ql = qq[wave][lane];
+      u = __int_as_float(qj[wave][lane]);
+    }
+    while (__any(pending)) {
+      if (pending) {
+        const int pos = atomicAdd(const_cast<int*>(&bin_n[ql]), 1);
+        if (pos < KNN_BIN) {
+          bin_v[ql * KNN_BIN + pos] = u;
+          pending = false;
+        }
+      }
+      __threadfence_block();
+      if (lane < QW) {
+        const int n = min(bin_n[lane], KNN_BIN);
+        bin_n[lane] = 0;
+        for (int i = 0; i < n; i++) {
+          const float c = bin_v[lane * KNN_BIN + i];
+          // sorted insertion: new[k] = median(c, old[k-1], old[k]), new[0] = min(c, old[0])
+#pragma unroll
+          for (int k = (MODE == 2 ? KNN_K : 1) - 1; k > 0; k--) lst[k] = __builtin_amdgcn_fmed3f(c, lst[k - 1], lst[k]);
+          lst[0] = __builtin_fminf(c, lst[0]);
+        }
+      }
+      __threadfence_block();
+    }
+    const float tau = lst[(MODE == 2 ? KNN_K : 1) - 1];
+#pragma unroll
+    for (int h = 0; h < QSETS; h++) {
+      const float tq = __shfl(tau, h * 32 + col);
+      // a pair can only enter the list of upper bounds when its lower bound is below the K-th of them
+      t[h] = valid[h] ? __builtin_fminf(tq - xk[h], KNN_FLT_MAX) : -inf;
+    }
+  };
   int qcount = 0;    // wave-uniform number of queued candidates
   i64 logged = 0;    // wave-uniform number of entries already in this wavefront's log
   const int slab = MODE == 1 ? knn_stage_slab(P.stage, blockIdx.y) : (int)blockIdx.y;
@@ -395,6 +460,34 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
         for (int v = 1; v < 16; v += 2)
           m = __builtin_fminf(__builtin_fminf(m, acc[h][v]), v + 1 < 16 ? acc[h][v + 1] : acc[h][v]);
         if (__builtin_expect(!__any(m <= t[h]), 1)) continue;
+        if (MODE == 2) {
+          // A threshold estimate may ignore candidates (the bound only gets looser): every lane offers the
+          // smallest of its 16 pairs of this sub-tile, which is nearly every candidate once they are sparse.
+          float yk = 0.f;  // key of the row that holds the minimum
+#pragma unroll
+          for (int v = 0; v < 16; v++) yk = acc[h][v] == m ? kk[v >> 2][v & 3] : yk;
+          const float u = (m + xk[h]) + KNN_E * (xk[h] + yk);
+          bool mine = m <= t[h];
+          unsigned long long bal = __ballot(mine);
+          while (bal != 0ull) {
+            const int slot = qcount + __popcll(bal & ((1ull << lane) - 1ull));
+            if (mine && slot < 64) {
+              qq[wave][slot] = h * 32 + col;
+              qj[wave][slot] = __float_as_int(u);
+              mine = false;
+            }
+            qcount += __popcll(bal);
+            if (qcount >= 64) {
+              drain(64);
+              qcount = 0;
+              mine = mine && (m <= t[h]);  // lanes that found the queue full retry unless excluded now
+              bal = __ballot(mine);
+            } else {
+              bal = 0ull;
+            }
+          }
+          continue;
+        }
         // all 16 compares first (independent, pipelined), then scalar tests of their wave-wide masks
         unsigned long long bals[16];
 #pragma unroll
@@ -425,6 +518,20 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
         }
       }
     }
+  }
+  if (MODE == 2) {
+    // lists of this slab straight from the owners' registers
+    drain(qcount);
+    const i64 q = qw0 + lane;
+    if (lane < QW && q < P.nq) {
+#pragma unroll
+      for (int l = 0; l < (MODE == 2 ? KNN_K : 1); l++) {
+        const i64 o = ((i64)blockIdx.y * P.nq + q) * KNN_K + l;
+        P.plist_d[o] = lst[l];
+        P.plist_i[o] = 0;
+      }
+    }
+    return;
   }
   if (qcount > 0) {
     if (MODE == 0) process(qcount);
@@ -459,6 +566,17 @@ extern "C" __global__ void __launch_bounds__(64 * KNN_WAVES) keops_knn_main(cons
   knn_sweep<0, KNN_WAVES, KNN_QSETS>(P, ys, ykey_s, lv, li, owner, qq, qj);
 }
 
+// threshold estimate from a subset of the references: K-lists of upper bounds, no memory access per candidate
+extern "C" __global__ void __launch_bounds__(64 * KNN_SWAVES) keops_knn_sample(const KnnParams P) {
+  __shared__ __attribute__((aligned(16))) unsigned char ys[KNN_TJ * KNN_STRIDE];
+  __shared__ __attribute__((aligned(16))) float ykey_s[KNN_TJ];
+  __shared__ int qq[KNN_SWAVES][64];                              // queued candidates: local query
+  __shared__ int qj[KNN_SWAVES][64];                              //                    upper bound (float bits)
+  __shared__ int bin_n[KNN_SWAVES * 32 * KNN_SQSETS];             // candidates dealt to every query
+  __shared__ float bin_v[KNN_SWAVES * 32 * KNN_SQSETS * KNN_BIN];  // their upper bounds
+  knn_sweep<2, KNN_SWAVES, KNN_SQSETS>(P, ys, ykey_s, nullptr, nullptr, bin_n, qq, qj, bin_v);
+}
+
 // fixed-threshold filter: KNN_FWAVES wavefronts of 32*KNN_FQSETS queries share every staged tile
 extern "C" __global__ void __launch_bounds__(64 * KNN_FWAVES) keops_knn_filter(const KnnParams P) {
   __shared__ __attribute__((aligned(16))) unsigned char ys[KNN_TJ * KNN_STRIDE];
@@ -468,16 +586,16 @@ extern "C" __global__ void __launch_bounds__(64 * KNN_FWAVES) keops_knn_filter(c
   knn_sweep<1, KNN_FWAVES, KNN_FQSETS>(P, ys, ykey_s, nullptr, nullptr, nullptr, qq, qj);
 }
 
-// every KNN_SAMPLE-th reference row (bf16 row + key) gathered in a compact array for the sampling pass
+// every step-th reference row (bf16 row + key) gathered in a compact array for the sampling pass
 extern "C" __global__ void __launch_bounds__(256) keops_knn_gather_sample(const KnnParams P, __bf16* yh_s, float* ykey_sm,
-                                                                           i64 nsample) {
+                                                                           i64 nsample, int step) {
   constexpr int CH = KNN_RW / 8;
   const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
   const i64 row = e / CH;
   const int c = (int)(e - row * CH);
   if (row >= nsample) return;
-  reinterpret_cast<uint4*>(yh_s)[e] = reinterpret_cast<const uint4*>(P.yh)[row * KNN_SAMPLE * CH + c];
-  if (c == 0) ykey_sm[row] = P.ykey[row * KNN_SAMPLE];
+  reinterpret_cast<uint4*>(yh_s)[e] = reinterpret_cast<const uint4*>(P.yh)[row * step * CH + c];
+  if (c == 0) ykey_sm[row] = P.ykey[row * step];
 }
 
 // ---- merge of the per-slab lists ----------------------------------------------------------------
@@ -534,9 +652,10 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParam
 }
 
 // Thresholds of a filter pass from K-lists of a subset of the references (any such K-th distance is
-// an upper bound of the final one).  refine = 0: lists of the sampling pass (slabs 0 .. nslabs-1);
-// refine = 1: lists replayed from the stage-1 slabs (0, 4, 8, ...: `count` of them), kept only where
-// tighter than the current threshold.
+// an upper bound of the final one).  refine = 0: lists of upper bounds U of the sampling pass (slabs
+// 0 .. nslabs-1): K references have an exact float32 distance <= U_K (1 + delta), so every final neighbour has a
+// lower bound L <= U_K (1 + delta)^2; refine = 1: exact lists replayed from the stage-1 slabs (0, 4, 8, ...:
+// `count` of them), kept only where tighter than the current threshold.
 extern "C" __global__ void __launch_bounds__(256) keops_knn_thresholds(const KnnParams P, int refine, int count) {
   const i64 q = (i64)blockIdx.x * 256 + threadIdx.x;
   if (q == 0 && !refine) *P.overflow = 0;  // reset before the filter passes (a fill kernel would be one more launch)
@@ -546,7 +665,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_thresholds(const Knn
   if (refine) knn_merge_lists(P, q, bv, bi, 0, 4, count);
   else knn_merge_lists(P, q, bv, bi, 0, 1, P.nslabs);
   const float tau = bv[KNN_K - 1];
-  float t = __builtin_fminf((tau + tau * KNN_DELTA) - P.xkey[q], KNN_FLT_MAX);
+  float t = __builtin_fminf((tau + tau * (refine ? KNN_DELTA : 3.0f * KNN_DELTA)) - P.xkey[q], KNN_FLT_MAX);
   if (refine) t = __builtin_fminf(t, P.thr[q]);
   P.thr[q] = t;
 }

@@ -165,14 +165,20 @@ def generate_knn_plugin(red, rowvar, colvar, nargs):
     waves = config.knn_max_waves
     while waves > 1 and fixed + waves * (32 * qsets * (red.K * 8 + 4) + 512) > config.knn_lds_budget:
         waves //= 2
+    # sampling pass (threshold estimate): the K-list of a query lives in the registers of one lane, so the
+    # geometry of the filter (four wavefronts per SIMD, 128 registers each) holds for small K only
+    swaves, sqsets = config.knn_sample_waves, config.knn_sample_qsets
+    if red.K > 16 or dpad * (1 + split) > 64:
+        swaves = min(swaves, 8)
     meta = dict(scheme="knn", block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
                 sizeof_acc=4, nrowvars=1, ncolvars=1, nparvars=0, knn_d=D, knn_dpad=dpad, knn_k=red.K,
                 knn_qb=waves * 32 * qsets, knn_fwaves=config.knn_filter_waves, knn_fqsets=config.knn_filter_qsets,
-                knn_sample=config.knn_sample, knn_split=split, rowarg=rowvar.ind, colarg=colvar.ind)
+                knn_sample=config.knn_sample, knn_split=split, knn_sqb=swaves * 32 * sqsets, knn_sblock=64 * swaves,
+                rowarg=rowvar.ind, colarg=colvar.ind)
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}", "typedef float T;"]
     defs = dict(KEOPS_NARGS=nargs, KNN_D=D, KNN_DPAD=dpad, KNN_K=red.K, KEOPS_RED_KEEP=red.keep, KEOPS_DIMOUT=red.dim,
                 KNN_QSETS=qsets, KNN_TJ=tj, KNN_WAVES=waves, KNN_FWAVES=config.knn_filter_waves,
-                KNN_FQSETS=config.knn_filter_qsets, KNN_SAMPLE=config.knn_sample, KNN_SPLIT=split)
+                KNN_FQSETS=config.knn_filter_qsets, KNN_SWAVES=swaves, KNN_SQSETS=sqsets, KNN_SPLIT=split)
     src += [f"#define {k} {v}" for k, v in defs.items()]
     src.append('#include "keops_knn_mfma.h"')
     return "\n".join(src) + "\n", meta
