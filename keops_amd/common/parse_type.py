@@ -4,6 +4,7 @@ Same behaviour as pykeops/pykeops/common/parse_type.py (get_type :71-131, get_si
 complete_aliases :9-45, get_optional_flags :134-207, parse_dtype_acc :210-240) and
 pykeops/pykeops/common/utils.py:11-35 (axis2cat / cat2axis).
 """
+import functools
 import re
 
 from ..formulas.parse import parse_alias
@@ -24,8 +25,10 @@ def cat2axis(cat):
     raise ValueError("Category should be Vi or Vj.")
 
 
+@functools.lru_cache(maxsize=4096)
 def get_type(type_str, position_in_list=None):
-    """'x = Vi(3)' -> ('x', 0, 3, position); 'Var(2,5,1)' -> (None, 1, 5, 2)."""
+    """'x = Vi(3)' -> ('x', 0, 3, position); 'Var(2,5,1)' -> (None, 1, 5, 2).  Pure function of its arguments,
+    called for every alias of every reduction call: memoised."""
     s = type_str.replace("Vx", "Vi").replace("Vy", "Vj")
     name, var = parse_alias(s, position_in_list if position_in_list is not None else 0)
     pos = var.ind

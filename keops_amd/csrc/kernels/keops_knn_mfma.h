@@ -672,13 +672,18 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_thresholds(const Knn
 
 // ---- replay of the candidate logs ---------------------------------------------------------------
 
-// One wavefront per log (= per filter wavefront and slab): exact distances and K-list insertion for
-// its 32*KNN_FQSETS queries, then the partial lists of that slab.
+// One wavefront per log (= per filter wavefront and slab): exact distances for its candidates, 64 at a time,
+// and the K best of each of its 32*KNN_FQSETS queries under the key (distance, index).  Lane l owns the sorted
+// list of query l in registers; a candidate is first compared with the current K-th entry of its query (kept
+// in LDS: most candidates of a fixed-threshold filter lose there), the others are dealt to small per-query
+// bins (one LDS atomic each) that the owners fold into their lists.
 extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParams P, int fgrid_x) {
   constexpr int QW = 32 * KNN_FQSETS;
-  __shared__ float lv[QW][KNN_K];
-  __shared__ int li[QW][KNN_K];
-  __shared__ int owner[QW];
+  __shared__ int bin_n[QW];
+  __shared__ float bin_d[QW * KNN_BIN];
+  __shared__ int bin_j[QW * KNN_BIN];
+  __shared__ float kth_d[QW];  // current K-th entry of every query
+  __shared__ int kth_j[QW];
   const int lane = threadIdx.x;
   const int wave = (int)(blockIdx.x % KNN_FWAVES);
   const i64 rest = blockIdx.x / KNN_FWAVES;
@@ -686,14 +691,26 @@ extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParam
   const i64 logid = (slab * fgrid_x + bx) * KNN_FWAVES + wave;
   const i64 qw0 = bx * (KNN_FWAVES * QW) + (i64)wave * QW;
   const float inf = __builtin_huge_valf();
-  for (int e = lane; e < QW * KNN_K; e += 64) {
-    (&lv[0][0])[e] = inf;
-    (&li[0][0])[e] = 0;
+  float ld[KNN_K];
+  int lj[KNN_K];
+#pragma unroll
+  for (int k = 0; k < KNN_K; k++) {
+    ld[k] = inf;
+    lj[k] = 0;
   }
-  __syncthreads();
+  volatile int* bn = bin_n;
+  volatile float* bd = bin_d;
+  volatile int* bj = bin_j;
+  volatile float* kd = kth_d;
+  volatile int* kj = kth_j;
+  if (lane < QW) {
+    bn[lane] = 0;
+    kd[lane] = inf;
+    kj[lane] = 0x7fffffff;
+  }
+  __threadfence_block();
   const int count = P.logcount[logid];
   const int2* mylog = P.log + logid * P.logcap;
-  volatile int* ow = owner;
   for (int base = 0; base < count; base += 64) {
     const bool act = base + lane < count;
     int ql = 0, j = 0;
@@ -704,25 +721,53 @@ extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParam
       j = e.y;
       d = knn_exact_sqdist(P.xq + (qw0 + ql) * KNN_D, P.yr + (i64)j * KNN_D);
     }
-    bool done = !act;
-    while (__any(!done)) {
-      if (!done) ow[ql] = lane;
-      __threadfence_block();
-      if (!done && ow[ql] == lane) {
-        knn_insert(lv[ql], li[ql], d, j);
-        done = true;
+    bool pending = act && knn_better(d, j, kd[ql], kj[ql]);
+    while (__any(pending)) {
+      if (pending) {
+        const int pos = atomicAdd(&bin_n[ql], 1);
+        if (pos < KNN_BIN) {
+          bd[ql * KNN_BIN + pos] = d;
+          bj[ql * KNN_BIN + pos] = j;
+          pending = false;
+        }
       }
       __threadfence_block();
+      if (lane < QW) {
+        const int n = min(bn[lane], KNN_BIN);
+        if (n > 0) {
+          bn[lane] = 0;
+          for (int i = 0; i < n; i++) {
+            const float cd = bd[lane * KNN_BIN + i];
+            const int cj = bj[lane * KNN_BIN + i];
+            // sorted insertion in registers: entry k becomes old[k-1] when the candidate goes before old[k-1],
+            // the candidate when it goes before old[k] only, and stays otherwise
+            bool before_cur = knn_better(cd, cj, ld[KNN_K - 1], lj[KNN_K - 1]);
+#pragma unroll
+            for (int k = KNN_K - 1; k > 0; k--) {
+              const bool before_prev = knn_better(cd, cj, ld[k - 1], lj[k - 1]);
+              ld[k] = before_prev ? ld[k - 1] : (before_cur ? cd : ld[k]);
+              lj[k] = before_prev ? lj[k - 1] : (before_cur ? cj : lj[k]);
+              before_cur = before_prev;
+            }
+            ld[0] = before_cur ? cd : ld[0];
+            lj[0] = before_cur ? cj : lj[0];
+          }
+          kd[lane] = ld[KNN_K - 1];
+          kj[lane] = lj[KNN_K - 1];
+        }
+      }
+      __threadfence_block();
+      // candidates that found their bin full try again unless the list has moved past them
+      pending = pending && knn_better(d, j, kd[ql], kj[ql]);
     }
   }
-  __syncthreads();
-  for (int e = lane; e < QW * KNN_K; e += 64) {
-    const int ql = e / KNN_K, l = e - ql * KNN_K;
-    const i64 q = qw0 + ql;
-    if (q < P.nq) {
+  const i64 q = qw0 + lane;
+  if (lane < QW && q < P.nq) {
+#pragma unroll
+    for (int l = 0; l < KNN_K; l++) {
       const i64 o = (slab * P.nq + q) * KNN_K + l;
-      P.plist_d[o] = lv[ql][l];
-      P.plist_i[o] = li[ql][l];
+      P.plist_d[o] = ld[l];
+      P.plist_i[o] = lj[l];
     }
   }
 }
