@@ -41,8 +41,8 @@ MEASURED_TRAFFIC_BYTES = {
     # profiles/keops_fin_main__gauss_dv256.md
     "gauss_dv256": int((8043160 * 2.0 + 10795000) * 1024),
     # profiles/keops_conv_ranges__sparse_100x10k.md, keops_conv_ranges__lse_b16.md
-    "sparse_100x10k": int((85442 * 2.0 + 3906.25) * 1024),
-    "lse_b16": int((55633 * 2.0 + 6250) * 1024),
+    "sparse_100x10k": int((109492 * 2.0 + 3906.25) * 1024),
+    "lse_b16": int((55625 * 2.0 + 6250) * 1024),
 }
 
 WORKLOADS = {
