@@ -49,9 +49,14 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 chk_bf16x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float chk_f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float chk_f32x4;
 
+#ifndef CHK_NC
+#define CHK_NC 1                             // wavefronts that share 32 output rows and split the contraction
+#endif
 #define CHK_BLOCK (64 * CHK_WAVES)
-#define CHK_QB (32 * CHK_WAVES)              // output rows per workgroup
+#define CHK_QB (32 * CHK_WAVES / CHK_NC)     // output rows per workgroup
 #define CHK_KB (CHK_DPAD / 16)
+#define CHK_KBC (CHK_KB / CHK_NC)            // 16-wide k blocks per wavefront
+#define CHK_VS (16 / CHK_NC)                 // values of a 32 x 32 tile each lane evaluates
 #define CHK_ROWBYTES (CHK_DPAD * 4)          // hi part then lo part, bf16 each
 #define CHK_STRIDE (CHK_ROWBYTES + 16)       // padded LDS row
 #define CHK_TJ 32                            // reduced rows per staged tile
@@ -135,7 +140,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum_final(const C
   }
 }
 
-// One row per group of CHK_LPR lanes, 4 columns per lane; which = 0: row variable (stored times -2
+// One row per group of CHK_LPR lanes, 4 columns per lane and pass; which = 0: row variable (stored times -2
 // in CHK_MODE 0), 1: column variable.  The squared norm is reduced inside the lane group
 // (deterministic).
 #define CHK_LPR (CHK_DPAD / 4 <= 4 ? 4 : (CHK_DPAD / 4 <= 8 ? 8 : (CHK_DPAD / 4 <= 16 ? 16 : (CHK_DPAD / 4 <= 32 ? 32 : 64))))
@@ -145,15 +150,15 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
   __bf16* dst = which ? P.ys : P.xs;
   const int q = threadIdx.x % CHK_LPR;
   const i64 row = ((i64)blockIdx.x * 256 + threadIdx.x) / CHK_LPR;
-  const bool live = row < n && q * 4 < CHK_DPAD;
+  const bool live = row < n;
   const float inv = 1.0f / (float)P.nys;
   const float scale = (CHK_MODE == 0 && !which) ? -2.0f : 1.0f;
   float nrm = 0.f;
-  if (live) {
+  for (int c0 = q * 4; c0 < CHK_DPAD && live; c0 += CHK_LPR * 4) {
     chk_bf16x4 hi, lo;
 #pragma unroll
     for (int e = 0; e < 4; e++) {
-      const int c = q * 4 + e;
+      const int c = c0 + e;
       float v = 0.f;
       if (c < CHK_D) {
         v = src[row * CHK_D + c];
@@ -164,8 +169,8 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
       hi[e] = (__bf16)v;
       lo[e] = (__bf16)(v - (float)hi[e]);
     }
-    *reinterpret_cast<chk_bf16x4*>(dst + row * 2 * CHK_DPAD + q * 4) = hi;
-    *reinterpret_cast<chk_bf16x4*>(dst + row * 2 * CHK_DPAD + CHK_DPAD + q * 4) = lo;
+    *reinterpret_cast<chk_bf16x4*>(dst + row * 2 * CHK_DPAD + c0) = hi;
+    *reinterpret_cast<chk_bf16x4*>(dst + row * 2 * CHK_DPAD + CHK_DPAD + c0) = lo;
   }
 #pragma unroll
   for (int o = CHK_LPR / 2; o > 0; o >>= 1) nrm += __shfl_xor(nrm, o, CHK_LPR);
@@ -176,16 +181,25 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
 
 #if !(defined(CHK_FINAL) && CHK_FINAL) && !(defined(CHK_SOFTMAX) && CHK_SOFTMAX)
 extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const ChkParams P) {
-  __shared__ __attribute__((aligned(16))) unsigned char as[CHK_TJ * CHK_STRIDE];  // A tile (hi|lo)
+  // A tile (hi|lo); after the sweep the same memory holds the accumulators that the lanes of a row merge
+  constexpr int TILE_BYTES = CHK_TJ * CHK_STRIDE;
+  constexpr int MERGE_BYTES = (int)sizeof(TACC) * CHK_QB * (2 * CHK_NC - 1) * KEOPS_DIMRED;
+  __shared__ __attribute__((aligned(16))) unsigned char as[TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES];
   __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
   __shared__ __attribute__((aligned(16))) T yo_s[CHK_TJ * CHK_DY];                // other column variables
-  __shared__ TACC merge_s[CHK_QB][KEOPS_DIMRED];
+  TACC (*merge_s)[2 * CHK_NC - 1][KEOPS_DIMRED] = reinterpret_cast<TACC (*)[2 * CHK_NC - 1][KEOPS_DIMRED]>(as);
+#if CHK_NC > 1
+  __shared__ float xch[CHK_WAVES * 16 * 64];  // partial 32 x 32 tiles of the wavefronts that split the contraction
+#endif
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
   KeopsTileGeom G;
   G.init(P.rt, P.nx, CHK_QB);
-  const i64 row0 = G.row_first + wave * 32;  // first output row of this wavefront
+  // CHK_NC wavefronts share 32 output rows: wavefront `chunk` of group `grp` contracts k blocks
+  // [chunk * CHK_KBC, (chunk + 1) * CHK_KBC) and evaluates values [chunk * CHK_VS, (chunk + 1) * CHK_VS) of each tile
+  const int grp = wave / CHK_NC, chunk = wave % CHK_NC;
+  const i64 row0 = G.row_first + grp * 32;   // first output row of this wavefront
   const bool wave_live = row0 < G.row_end;   // a wavefront without rows only helps staging the tiles
   i64 q = row0 + col;
   const bool valid = q < G.row_end;
@@ -193,11 +207,12 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
   const i64 qx = G.row(CHK_XARG, q);
 
   // B operands: split rows of the chunked row variable
-  chk_bf16x8 bh[CHK_KB], bl[CHK_KB];
+  chk_bf16x8 bh[CHK_KBC], bl[CHK_KBC];
 #pragma unroll
-  for (int kb = 0; kb < CHK_KB; kb++) {
-    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + kb * 16 + 8 * half);
-    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+  for (int kb = 0; kb < CHK_KBC; kb++) {
+    const int k0 = (chunk * CHK_KBC + kb) * 16 + 8 * half;
+    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + k0);
+    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + k0);
   }
   const float xnq = CHK_MODE == 0 ? P.xn[qx] : 0.f;
   // other row variables and parameters of the post-chunk formula
@@ -261,6 +276,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
     }
     __syncthreads();
     if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ, jend);
+#if CHK_NC == 1
     if (!wave_live) continue;
 
     // s tile: accumulator register v of this lane is reduced row 8*(v/4) + 4*half + v%4
@@ -284,15 +300,47 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
     }
+#else
+    // partial tile of this wavefront's k blocks, handed to the group through LDS
+    if (wave_live) {
+      chk_f32x16 s;
+#pragma unroll
+      for (int v = 0; v < 16; v++) s[v] = 0.f;
+      const unsigned char* arow = as + col * CHK_STRIDE + 16 * half + chunk * CHK_KBC * 32;
+#pragma unroll
+      for (int kb = 0; kb < CHK_KBC; kb++) {
+        const chk_bf16x8 ah = *reinterpret_cast<const chk_bf16x8*>(arow + kb * 32);
+        const chk_bf16x8 al = *reinterpret_cast<const chk_bf16x8*>(arow + CHK_DPAD * 2 + kb * 32);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[kb], s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
+      }
+#pragma unroll
+      for (int v = 0; v < 16; v++) xch[(wave * 16 + v) * 64 + lane] = s[v];
+    }
+    __syncthreads();
+    if (!wave_live) continue;
+    // this wavefront's share of the tile: partial sums added in chunk order (deterministic)
+    float s[CHK_VS];
+#pragma unroll
+    for (int vv = 0; vv < CHK_VS; vv++) {
+      const int v = chunk * CHK_VS + vv;
+      float t = CHK_MODE == 0 ? yn_s[8 * (v >> 2) + 4 * half + (v & 3)] : 0.f;
+#pragma unroll
+      for (int c = 0; c < CHK_NC; c++) t += xch[((grp * CHK_NC + c) * 16 + v) * 64 + lane];
+      s[vv] = t;
+    }
+#endif
 #if KEOPS_USE_TILE_TMP
     KeopsAcc<T> tmp;
     tmp.init();
 #endif
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
+    for (int vv = 0; vv < CHK_VS; vv++) {
+      const int v = chunk * CHK_VS + vv;
       const int r = 8 * (v >> 2) + 4 * half + (v & 3);
       if (r < n) {
-        T sv = s[v];
+        T sv = s[vv];
         if (CHK_MODE == 0) sv = __builtin_fmaxf(sv + xnq, 0.f);
         T yj[CHK_DY];
         constexpr int VEC = 16 / sizeof(T);
@@ -323,14 +371,18 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
   sweep(0, P.ny);
 #endif
 
-  // the two lanes of an output row merge their accumulators (lower reduced rows first)
+  // the 2 * CHK_NC lanes of an output row merge their accumulators in a fixed order
   __syncthreads();
-  if (half == 1) acc.store_partial(merge_s[wave * 32 + col]);
+  const int part = chunk * 2 + half;
+  if (part > 0) acc.store_partial(merge_s[grp * 32 + col][part - 1]);
   __syncthreads();
-  if (half == 0) {
-    KeopsAcc<TACC> other;
-    other.load_partial(merge_s[wave * 32 + col]);
-    acc.merge(other);
+  if (part == 0) {
+#pragma unroll
+    for (int k = 0; k < 2 * CHK_NC - 1; k++) {
+      KeopsAcc<TACC> other;
+      other.load_partial(merge_s[grp * 32 + col][k]);
+      acc.merge(other);
+    }
     if (valid) acc.finalize(P.out + q * KEOPS_DIMOUT);
   }
 }

@@ -76,6 +76,9 @@ def choose_geometry(red, layout, nops, sizeof_t, nx=None, irregular=False):
             rows //= 2
     tile_j = config.lds_tile_bytes // max(1, dimy_pad * sizeof_t)
     tile_j = max(64, min(1024, 1 << (tile_j.bit_length() - 1)))
+    # very wide reduced-index rows: shorter tiles so that the staged tile still fits the LDS of a compute unit
+    while tile_j > 16 and tile_j * dimy_pad * sizeof_t > 96 * 1024:
+        tile_j //= 2
     unroll = 2 if nops * rows <= 128 else 1
     return dict(block=block, rows=rows, tile_j=tile_j, dimy_pad=dimy_pad, unroll=unroll)
 
@@ -187,7 +190,7 @@ def generate_knn_plugin(red, rowvar, colvar, nargs):
 def match_chunk(red, dtype, map_reduce_id, use_fast_math):
     """(mode, node, row variable, column variable) when the formula of a Sum / log-sum-exp reduction
     contains exactly one high-dimensional contraction SqDist(x_i, y_j) (mode 0) or <x_i, y_j> (mode 1)
-    between plain variables of dimension 32..256 that appear nowhere else in the formula (the
+    between plain variables of dimension 32..1024 that appear nowhere else in the formula (the
     reference's conditions, Chunkable_Op.py:20-41 and Chunk_Mode_Constants.py:56-60, with the
     matrix-core dimension range instead of its >= 146 threshold).  None otherwise."""
     from .formulas import ops as O
@@ -205,7 +208,7 @@ def match_chunk(red, dtype, map_reduce_id, use_fast_math):
         if mode is None:
             continue
         a, b = pair
-        if isinstance(a, O.Var) and isinstance(b, O.Var) and a.dim == b.dim and 32 <= a.dim <= 256 and {a.cat, b.cat} == {0, 1}:
+        if isinstance(a, O.Var) and isinstance(b, O.Var) and a.dim == b.dim and 32 <= a.dim <= config.chunk_max_dim and {a.cat, b.cat} == {0, 1}:
             if node not in [f[1] for f in found]:
                 found.append((mode, node, a, b))
     if len(found) != 1:
@@ -228,9 +231,12 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
     mode, node, xvar, yvar = match
     svar = O.Var(1 << 30, 1, 3)
     post = red.formula.replace(node, svar)
+    # beyond 256 components the split operands of 32 output rows no longer fit the registers of one wavefront:
+    # nc wavefronts share the rows, each contracts 1/nc of the components, partial tiles meet in LDS
+    nc = 1 if xvar.dim <= 256 else (2 if xvar.dim <= 512 else 4)
     # post-chunk formula g(s, ...) * v_j of a float32 Sum: the product with v also runs on the matrix cores
     final = None
-    if (red.kind == KIND_SUM and dtypeacc == "float" and sum_scheme in ("block_sum", "direct_sum")
+    if (nc == 1 and red.kind == KIND_SUM and dtypeacc == "float" and sum_scheme in ("block_sum", "direct_sum")
             and post.name == "Mult" and len(post.children) == 2):
         for g, v in (post.children, post.children[::-1]):
             if (g.dim == 1 and isinstance(v, O.Var) and v.cat == 1 - red.tagI and v.dim == post.dim
@@ -242,7 +248,7 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
     from .formulas.reductions import KIND_LSE
 
     softmax = None
-    if red.kind == KIND_LSE and dtypeacc == "float" and sum_scheme != "kahan_scheme" and post.name == "Concat":
+    if nc == 1 and red.kind == KIND_LSE and dtypeacc == "float" and sum_scheme != "kahan_scheme" and post.name == "Concat":
         Fp, G = post.children
         one = 0
         if G.name == "Concat" and isinstance(G.children[0], O.IntCst) and G.children[0].val == 1:
@@ -265,19 +271,22 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
     outs = lower(post, L)
     lines, exprs = L.emit(outs, layout.names, indent="    ")
     D = xvar.dim
-    dpad = -(-D // 16) * 16
+    dpad = -(-D // (16 * nc)) * 16 * nc
     dimy_pad = 0 if layout.dimy == 0 else -(-layout.dimy // 4) * 4
     waves = config.chunk_waves
     # LDS of the kernel: staged tile (hi|lo rows), the other reduced-index variables, and either the v tile
     # (final-product variant) or the accumulator exchange of the two lanes of a row
     def lds_bytes(w):
-        fixed = 32 * (dpad * 4 + 16) + 128 + 32 * max(1, dimy_pad) * 4
+        tile = 32 * (dpad * 4 + 16)
+        fixed = 128 + 32 * max(1, dimy_pad) * 4
         if wvar is not None:
-            return fixed + 32 * (-(-wvar.dim // 32)) * 32 * 4 + 128 * w
-        return fixed + 32 * w * red.dimred * (8 if dtypeacc == "double" else 4)
-    while waves > 1 and lds_bytes(waves) > config.knn_lds_budget:
+            return tile + fixed + 32 * (-(-wvar.dim // 32)) * 32 * 4 + 128 * w
+        # the accumulator exchange reuses the memory of the staged tile
+        merge = (32 * w // nc) * (2 * nc - 1) * red.dimred * (8 if dtypeacc == "double" else 4)
+        return max(tile, merge) + fixed + (w * 16 * 64 * 4 if nc > 1 else 0)
+    while waves > nc and lds_bytes(waves) > config.knn_lds_budget:
         waves //= 2
-    if lds_bytes(waves) > config.knn_lds_budget:
+    if waves < nc or lds_bytes(waves) > config.knn_lds_budget:
         return None, None
     ra, rd, ro = VarLayout.table(layout.rowvars)
     ca, cd, co = VarLayout.table(layout.colvars)
@@ -286,13 +295,13 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
     meta = dict(scheme="chunk", block=64 * waves, rows=1, tile_j=32, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
                 sizeof_acc=8 if dtypeacc == "double" else 4, nrowvars=len(layout.rowvars) + 1,
                 ncolvars=len(layout.colvars) + ncol_extra, nparvars=len(layout.parvars), chk_d=D, chk_dpad=dpad,
-                chk_mode=mode, chk_qb=32 * waves, chk_final=int(final is not None), chk_softmax=int(softmax is not None),
+                chk_mode=mode, chk_qb=32 * waves // nc, chk_final=int(final is not None), chk_softmax=int(softmax is not None),
                 chk_xarg=xvar.ind, chk_yarg=yvar.ind, ranges=int(irregular), nops=L.count_ops(outs))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
            f"typedef float T;\ntypedef {dtypeacc} TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
            '#include "keops_common.h"']
     defs = dict(
-        KEOPS_NARGS=nargs, CHK_D=D, CHK_DPAD=dpad, CHK_MODE=mode, CHK_XARG=xvar.ind, CHK_YARG=yvar.ind, CHK_WAVES=waves,
+        KEOPS_NARGS=nargs, CHK_D=D, CHK_DPAD=dpad, CHK_MODE=mode, CHK_XARG=xvar.ind, CHK_YARG=yvar.ind, CHK_WAVES=waves, CHK_NC=nc,
         KEOPS_DIMX=layout.dimx, KEOPS_DIMY=layout.dimy, KEOPS_DIMY_PAD=dimy_pad, KEOPS_DIMP=layout.dimp,
         KEOPS_DIMFOUT=post.dim, KEOPS_DIMRED=red.dimred, KEOPS_DIMOUT=red.dim, KEOPS_RED_KIND=red.kind,
         KEOPS_RED_KEEP=red.keep, KEOPS_RED_K=red.K, KEOPS_SUM_SCHEME=SUM_SCHEMES[sum_scheme],

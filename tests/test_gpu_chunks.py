@@ -164,3 +164,41 @@ def test_softmax_weighted_sum_on_matrix_cores(M, N, D, Dv, axis):
     gl = lse(qd, kd, to_dev(w)[0], scale).cpu().double()
     refl = torch.logsumexp(S[:, :, None] + torch.log(torch.from_numpy(w).double())[None, :, :], dim=1)
     assert float((gl - refl).abs().max()) <= 2e-5 * max(1.0, float(refl.abs().max()))
+
+
+@pytest.mark.parametrize("M,N,D,Dv", [(200, 300, 300, 1), (700, 1000, 512, 16), (333, 777, 700, 3), (150, 260, 1024, 2)])
+def test_contraction_beyond_256_components(M, N, D, Dv):
+    """Several wavefronts share 32 output rows and split the contraction (D = 300 is the size of the reference's
+    pykeops/test/test_chunks.py); Sum and log-sum-exp against dense float64."""
+    from keops_amd import keops_io
+    from keops_amd.torch import Genred
+
+    x, y, b = _laplace_inputs(M, N, D, Dv, 51)
+    xd, yd, bd = to_dev(x, y, b)
+    x64, y64, b64 = (torch.from_numpy(t).double() for t in (x, y, b))
+    K = torch.exp(-torch.cdist(x64, y64))
+    conv = Genred("Exp(-Norm2(x-y))*b", [f"x=Vi({D})", f"y=Vj({D})", f"b=Vj({Dv})"], reduction_op="Sum", axis=1)
+    got = conv(xd, yd, bd).cpu().numpy()
+    assert any(m.meta("scheme") == "chunk" and m.meta("chk_d") == str(D) for m in keops_io._modules.values())
+    assert_sum_parity(got, (K @ b64).numpy(), (K @ b64.abs()).numpy())
+    # reduction over i, inner-product mode, log-sum-exp
+    lse = Genred("p*(x|y)", [f"x=Vi({D})", f"y=Vj({D})", "p=Pm(1)"], reduction_op="LogSumExp", axis=0)
+    gl = lse(xd, yd, torch.tensor([0.5], device="cuda")).cpu().double()[:, 0]
+    refl = torch.logsumexp(0.5 * x64 @ y64.T, dim=0)
+    assert float((gl - refl).abs().max()) <= 2e-5 * max(1.0, float(refl.abs().max()))
+
+
+def test_contraction_beyond_256_components_batched():
+    """Shapes of the reference's pykeops/test/test_chunks_ranges.py: two batch dimensions, D = 300."""
+    from keops_amd.torch import LazyTensor
+
+    B1, B2, M, N, D, Dv = 2, 3, 200, 300, 300, 1
+    gen = torch.Generator().manual_seed(52)
+    x = torch.randn(B1, B2, M, 1, D, generator=gen) / 8
+    y = torch.randn(B1, 1, 1, N, D, generator=gen) / 8
+    b = torch.randn(B1, B2, 1, N, Dv, generator=gen)
+    got = ((-((LazyTensor(x.cuda()) - LazyTensor(y.cuda())) ** 2).sum(-1)).exp() * LazyTensor(b.cuda())).sum(dim=3).cpu()
+    K = torch.exp(-((x.double() - y.double()) ** 2).sum(-1))          # (B1, B2, M, N)
+    ref = K @ b.double()[:, :, 0]
+    scale = K @ b.double()[:, :, 0].abs()
+    assert_sum_parity(got.numpy(), ref.numpy(), scale.numpy())
