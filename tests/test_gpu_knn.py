@@ -120,3 +120,33 @@ def test_knn_low_dimension_clustered_far_from_origin():
     ref = cpu_reduc("sqdist", [x, y], x.shape[0], y.shape[0], 1, reduction="KMin_ArgKMin", K=K, scheme="direct_sum")
     assert np.array_equal(idx.cpu().numpy(), ref[:, 1::2].astype(np.int64))
     assert np.array_equal(vals.cpu().numpy(), ref[:, 0::2])
+
+
+@pytest.mark.parametrize("D", [64, 3])
+def test_knn_two_phase_with_massive_ties(D):
+    """Sizes that take the sampled-threshold schedule, on data full of exact ties: integer grid coordinates with
+    every reference stored four times (the strict-'<' rule keeps the lower index), and queries that coincide with
+    references."""
+    M, N, K = 2048, 40000, 10
+    rng = np.random.default_rng(61)
+    base = rng.integers(0, 4, size=(N // 4, D)).astype(np.float32)
+    y = np.concatenate([base, base, base, base], 0)
+    x = rng.integers(0, 4, size=(M, D)).astype(np.float32)
+    x[:100] = y[:100]
+    ref = cpu_reduc("sqdist", [x, y], M, N, 1, reduction="KMin_ArgKMin", K=K, scheme="direct_sum")
+    vals, idx = _knn(D, K)(*to_dev(x, y))
+    assert np.array_equal(idx.cpu().numpy().reshape(M, K), ref[:, 1::2].astype(np.int64))
+    assert np.array_equal(vals.cpu().numpy().reshape(M, K), ref[:, 0::2])
+
+
+def test_knn_two_phase_log_overflow_falls_back():
+    """All references identical: every pair passes any threshold, the candidate logs overflow and the launch
+    falls back to the adaptive schedule; the K lowest indices win the ties."""
+    M, N, D, K = 1100, 33000, 32, 6
+    rng = np.random.default_rng(62)
+    x = rng.random((M, D)).astype(np.float32)
+    y = np.tile(rng.random((1, D)).astype(np.float32), (N, 1))
+    vals, idx = _knn(D, K)(*to_dev(x, y))
+    assert np.array_equal(idx.cpu().numpy().reshape(M, K), np.tile(np.arange(K), (M, 1)))
+    ref = cpu_reduc("sqdist", [x, y[:K]], M, K, 1, reduction="KMin", K=K, scheme="direct_sum")
+    assert np.array_equal(vals.cpu().numpy().reshape(M, K), ref)
