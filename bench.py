@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
-HBM.  The default workload is BASELINE.json's headline configuration: the Gaussian kernel sum
+HBM.  The default workload is the headline configuration of the reference's benchmarks: the Gaussian kernel sum
 a_i = sum_j exp(-|x_i-y_j|^2/sigma^2) b_j at M = N = 1,000,000, D = 3, Dv = 1, float32.
 The last line printed is ONE JSON object with the throughput (pair interactions per second), the
 roofline of the dominant kernel (algorithmic flops / kernel time measured with HIP events on the
@@ -47,17 +47,17 @@ MEASURED_TRAFFIC_BYTES = {
 
 WORKLOADS = {
     # name: (description, algorithmic flop per pair, roofline bound)
-    "gauss_1m_dv1": ("Gaussian kernel sum 1e6 x 1e6, D=3, Dv=1, float32 (BASELINE config 2)", 14, "valu"),
-    "gauss_1m_dv8": ("Gaussian kernel sum 1e6 x 1e6, D=3, Dv=8, float32 (BASELINE config 2)", 28, "valu"),
-    "gauss_1m_grad": ("gradient wrt x of the Gaussian kernel sum 1e6 x 1e6, D=3, Dv=1 (BASELINE config 2)", 21, "valu"),
-    "gauss_10k": ("Gaussian kernel sum 1e4 x 1e4, D=3, Dv=1, float32 (BASELINE config 1)", 14, "valu"),
+    "gauss_1m_dv1": ("Gaussian kernel sum 1e6 x 1e6, D=3, Dv=1, float32 (benchmark configuration 2)", 14, "valu"),
+    "gauss_1m_dv8": ("Gaussian kernel sum 1e6 x 1e6, D=3, Dv=8, float32 (benchmark configuration 2)", 28, "valu"),
+    "gauss_1m_grad": ("gradient wrt x of the Gaussian kernel sum 1e6 x 1e6, D=3, Dv=1 (benchmark configuration 2)", 21, "valu"),
+    "gauss_10k": ("Gaussian kernel sum 1e4 x 1e4, D=3, Dv=1, float32 (benchmark configuration 1)", 14, "valu"),
     "gauss_100k": ("Gaussian kernel sum 1e5 x 1e5, D=3, Dv=1, float32 (reference benchmarks/README.md:13)", 14, "valu"),
     # 2*D flop of the <x,y> contraction per pair (the matrix-core work); filter and re-rank are not counted
-    "knn_d64": ("KMin_ArgKMin K=10, 1e5 queries x 1e6 references, D=64 (BASELINE config 3)", 128, "mfma"),
-    "sparse_100x10k": ("block-sparse Gaussian sum, 100 clusters x 10,000 points (BASELINE config 4)", 14, "valu"),
-    "lse_b16": ("batched LogSumExp softmin B=16, 50,000 x 50,000, D=3 (BASELINE config 5a)", 17, "valu"),
+    "knn_d64": ("KMin_ArgKMin K=10, 1e5 queries x 1e6 references, D=64 (benchmark configuration 3)", 128, "mfma"),
+    "sparse_100x10k": ("block-sparse Gaussian sum, 100 clusters x 10,000 points (benchmark configuration 4)", 14, "valu"),
+    "lse_b16": ("batched LogSumExp softmin B=16, 50,000 x 50,000, D=3 (benchmark configuration 5a)", 17, "valu"),
     # 2*D flop of the contraction + sqrt, neg, exp + 2*Dv of the weighted accumulation
-    "laplace_d256": ("Laplace kernel sum 2e5 x 2e5, D=256, Dv=16 (BASELINE config 5b)", 547, "mfma"),
+    "laplace_d256": ("Laplace kernel sum 2e5 x 2e5, D=256, Dv=16 (benchmark configuration 5b)", 547, "mfma"),
     # softmax-weighted sum of an inner product (attention-like).  Counted: exp + 2*Dv of the weighted sum, which runs
     # on the float32 matrix cores and dominates; the 2*D*3 bf16 flop of the scores are not counted
     "softmax_d64": ("SumSoftMaxWeight of <q,k> with 64-dimensional weights, 65536 x 65536, D=64", 130, "mfma32"),

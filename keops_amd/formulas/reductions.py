@@ -161,6 +161,16 @@ def Diff_WithSavedForward(red, v, u, f0):
     of a sum is the sum of the differentials, indexed like the original output."""
     if isinstance(red, Zero_Reduction):
         return Zero_Reduction(red.dim, red.tagI)
+    if isinstance(red, Max_SumShiftExpWeight_Reduction):
+        # Valid once (m, s) is flattened to m + log(s) or a weighted softmax by the Python layer: the tangent of
+        # the output is [0, d(sum_j exp(F - m) G)] with the saved maximum m held fixed, whose image through the
+        # flattening is the tangent of the flattened result (Max_SumShiftExpWeight_Reduction.py:105-121).
+        F, G = red.formulaF, red.formulaG
+        M = Extract(f0, 0, F.dim)
+        d = ops.Diff(ops.Mult(Exp(Subtract(F, M)), G), v, u)
+        if isinstance(d, Zero):
+            return Zero_Reduction(red.dim, red.tagI)
+        return Sum_Reduction(Concat(Zero(F.dim), d), red.tagI)
     if not isinstance(red, Sum_Reduction):
         raise NotImplementedError(f"forward-mode differentiation through {red.string_id} is not supported")
     d = ops.Diff(red.formula, v, u)

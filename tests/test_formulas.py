@@ -267,3 +267,30 @@ def test_forward_mode_diff_divergence_laplacian():
         return (4 * g * g * r2 - 6 * g) * torch.exp(-g * r2)
 
     _check("Laplacian(Exp(-g*SqDist(x,y)), x)", al, a, lap)
+
+
+def test_forward_mode_through_log_sum_exp_reduction():
+    """Diff_WithSavedForward of a Max_SumShiftExpWeight reduction: [0, d(sum_j exp(F - m) G)] with the saved
+    maximum m; flattened as the Python layer does (tangent of m + log s is ds / s) it must equal the jvp of a
+    dense weighted log-sum-exp (cf. the reference's pykeops/test/test_torch_func_logsumexp.py)."""
+    x, y, w, u = _t(M, 3), _t(N, 3), _t(N, 1, lo=0.2, hi=1.0), _t(M, 3)
+    al = ["x=Var(0,3,0)", "y=Var(1,3,1)", "w=Var(2,1,1)", "u=Var(3,3,0)", "ms=Var(4,2,0)"]
+    red = parse_reduction("Diff_WithSavedForward(Max_SumShiftExpWeight_Reduction(-SqDist(x,y),0,w),x,u,ms)", al)
+    assert red.string_id == "Sum_Reduction" and red.dim == 2 and red.tagI == 0
+
+    def lse(x_):
+        F = -((x_[:, None, :] - y[None, :, :]) ** 2).sum(-1)
+        return torch.log((torch.exp(F) * w[None, :, 0]).sum(1))
+
+    F = -((x[:, None, :] - y[None, :, :]) ** 2).sum(-1)
+    m = F.max(1, keepdim=True).values
+    s = (torch.exp(F - m) * w[None, :, 0]).sum(1, keepdim=True)
+    ms = torch.cat([m, s], 1)
+    dense = dense_eval(red.formula, None, [t.numpy() for t in (x, y, w, u, ms)], M, N)   # (M, N, 2)
+    dms = dense.sum(1)
+    assert np.all(dms[:, 0] == 0)
+    _, ref = torch.func.jvp(lse, (x,), (u,))
+    assert np.allclose(dms[:, 1] / s[:, 0].numpy(), ref.numpy(), rtol=1e-10, atol=1e-10)
+    # a tangent that the formula does not depend on gives the zero reduction
+    z = parse_reduction("Diff_WithSavedForward(Max_SumShiftExpWeight_Reduction(-SqDist(x,y),0,w),Var(5,1,2),Var(6,1,2),ms)", al)
+    assert z.string_id == "Zero_Reduction"

@@ -158,3 +158,60 @@ def test_vmap_through_genred():
     out = torch.func.vmap(lambda x_: conv(x_, y, b))(xs)
     ref = torch.exp(-((xs[:, :, None, :] - y[None, None, :, :]) ** 2).sum(-1)) @ b
     assert out.shape == (B, M, 2) and torch.allclose(out, ref, rtol=1e-10, atol=1e-10)
+
+
+def _func_cases():
+    """Shapes and functions of the reference's pykeops/test/test_torch_func.py (Gaussian sum with a batched
+    parameter) and test_torch_func_logsumexp.py (weighted log-sum-exp), in float64 on the device."""
+    torch.manual_seed(0)
+    B1, B2, M, N, D = 5, 4, 10, 20, 2
+    kw = dict(dtype=torch.float64, device="cuda")
+    x_i, y_j = torch.randn(B1, B2, M, 1, D, **kw), torch.randn(B1, 1, 1, N, D, **kw)
+    b_j, p = torch.randn(B1, B2, 1, N, 1, **kw), torch.rand(B1, 1, 1, 1, 1, **kw)
+    w_j = torch.rand(B1, B2, 1, N, 1, **kw) + 0.1
+
+    def sum_torch(x_i, y_j, b_j, p):
+        K_ij = (-p[..., 0] * ((x_i - y_j) ** 2).sum(-1)).exp()[..., None]
+        return ((K_ij * b_j).sum(-3)).norm()
+
+    def sum_keops(x_i, y_j, b_j, p):
+        from keops_amd.torch import LazyTensor
+
+        nb = x_i.dim() - 3
+        K_ij = (-LazyTensor(p) * ((LazyTensor(x_i) - LazyTensor(y_j)) ** 2).sum(-1)).exp()
+        return ((K_ij * LazyTensor(b_j)).sum(nb)).norm()
+
+    def lse_torch(x_i, y_j, w_j):
+        D2_ij = (0.3 * ((x_i - y_j) ** 2).sum(-1))[..., None]
+        return ((D2_ij.exp() * w_j).sum(-3)).log().norm()
+
+    def lse_keops(x_i, y_j, w_j):
+        from keops_amd.torch import LazyTensor
+
+        nb = x_i.dim() - 3
+        D2_ij = 0.3 * ((LazyTensor(x_i) - LazyTensor(y_j)) ** 2).sum(-1)
+        return D2_ij.logsumexp(axis=nb, other=LazyTensor(w_j)).norm()
+
+    tangents = tuple(torch.randn_like(t) for t in (x_i, y_j, b_j, p))
+    return (sum_torch, sum_keops, (x_i, y_j, b_j, p), tangents), (lse_torch, lse_keops, (x_i, y_j, w_j), tangents[:3])
+
+
+@pytest.mark.parametrize("which", [0, 1])
+def test_torch_func_transforms(which):
+    """grad, vjp, jvp, jacrev, jacfwd, hessian and vmap of a scalar function of a reduction agree with dense torch,
+    for a Sum and for a weighted log-sum-exp reduction (forward mode through the (max, sum) pair)."""
+    f_torch, f_keops, args, tans = _func_cases()[which]
+    idx = tuple(range(len(args)))
+    close = lambda a, b: torch.allclose(a, b, rtol=1e-8, atol=1e-8)
+    assert close(f_keops(*args), f_torch(*args))
+    for a, b in zip(torch.func.grad(f_keops, idx)(*args), torch.func.grad(f_torch, idx)(*args)):
+        assert close(a, b)
+    one = torch.tensor(1.0, dtype=torch.float64, device="cuda")
+    for a, b in zip(torch.func.vjp(f_keops, *args)[1](one), torch.func.vjp(f_torch, *args)[1](one)):
+        assert close(a, b)
+    assert close(torch.func.jvp(f_keops, args, tans)[1], torch.func.jvp(f_torch, args, tans)[1])
+    for a, b in zip(torch.func.jacrev(f_keops, idx)(*args), torch.func.jacrev(f_torch, idx)(*args)):
+        assert close(a, b)
+    assert close(torch.func.jacfwd(f_keops)(*args), torch.func.jacfwd(f_torch)(*args))
+    assert close(torch.func.hessian(f_keops)(*args), torch.func.hessian(f_torch)(*args))
+    assert close(torch.func.vmap(f_keops)(*args), torch.func.vmap(f_torch)(*args))
