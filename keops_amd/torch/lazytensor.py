@@ -13,6 +13,7 @@ position (Var(k,dim,cat)) when a reduction is requested.
 from __future__ import annotations
 
 import itertools
+import math
 
 import torch
 
@@ -129,6 +130,13 @@ class LazyTensor:
     def dim(self):
         return len(self.shape)
 
+    def __str__(self):
+        """Verbose identifier: formula, symbolic variables and shape (lazy_tensor.py:959-996)."""
+        out = f"KeOps LazyTensor\n    formula: {self.formula!r}"
+        if self.symbolic:
+            out += "\n    symbolic variables: " + ", ".join(f"Var{v}" for v in sorted(self.symbolic))
+        return out + f"\n    shape: {self.shape}"
+
     @property
     def dtype(self):
         return self._dtype
@@ -235,11 +243,17 @@ class LazyTensor:
 
     __hash__ = object.__hash__
 
-    def __matmul__(self, v):
-        """K @ v with v a (..,N,D) tensor: sum_j K_ij v_j (lazy_tensor.py:2490-2527)."""
+    def __matmul__(self, v, **kwargs):
+        """K @ v: sum_j K_ij v_j with v a (N,) vector or a (..,N,D) tensor, K of trailing dimension 1; keyword
+        arguments (sum_scheme, out, backend, ...) go to the reduction (lazy_tensor.py:2490-2527)."""
         if isinstance(v, LazyTensor):
-            return (self * v).sum(self.nbatchdims + 1)
-        return (self * LazyTensor(v, axis=1) if v.dim() == 2 else self * LazyTensor(v.unsqueeze(-3))).sum(self.nbatchdims + 1)
+            return (self * v).sum(self.nbatchdims + 1, **kwargs)
+        if self.ndim != 1:
+            raise ValueError("The 'K @ v' syntax is only supported for LazyTensors 'K' whose trailing dimension "
+                             f"is equal to 1. Here, K.shape = {self.shape}.")
+        if v.dim() == 1:
+            return (self * LazyTensor(v.view(1, -1, 1))).sum(self.nbatchdims + 1, **kwargs).view(-1)
+        return (self * LazyTensor(v.unsqueeze(-3))).sum(self.nbatchdims + 1, **kwargs)
 
     def __getitem__(self, key):
         if isinstance(key, int):
@@ -308,6 +322,13 @@ class LazyTensor:
     def sinxdivx(self):
         return self.unary(O.SinXDivX)
 
+    def sinc(self):
+        """sin(pi x) / (pi x), as torch.sinc (lazy_tensor.py:1267-1274)."""
+        return (math.pi * self).sinxdivx()
+
+    def power(self, other):
+        return self ** other
+
     def mod(self, modulus, offset=0):
         return self.ternary(modulus, offset, O.Mod)
 
@@ -354,11 +375,23 @@ class LazyTensor:
     def concat(self, other):
         return self.binary(other, O.Concat)
 
-    def concatenate(self, others, axis=-1):
-        res = self
-        for o in others:
+    @staticmethod
+    def concatenate(tuple_of_lt, axis=-1):
+        """``LazyTensor.concatenate((x_1, ..., x_n), -1)``: concatenation along the last dimension, the only
+        one that supports it (lazy_tensor.py:1728-1760)."""
+        if not isinstance(tuple_of_lt, tuple) or len(tuple_of_lt) == 0 or not isinstance(tuple_of_lt[0], LazyTensor):
+            raise ValueError("LazyTensor.concatenate is implemented on non-empty tuples of LazyTensors.")
+        if axis not in (-1, len(tuple_of_lt[0].shape) - 1):
+            raise ValueError("LazyTensor only supports concatenation along the last axis.")
+        res = tuple_of_lt[0]
+        for o in tuple_of_lt[1:]:
             res = res.concat(o)
         return res
+
+    @staticmethod
+    def cat(tuple_of_lt, dim):
+        """torch-style alias of :meth:`concatenate`."""
+        return LazyTensor.concatenate(tuple_of_lt, dim)
 
     def one_hot(self, D):
         return self.unary(O.OneHot, D)

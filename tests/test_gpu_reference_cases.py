@@ -1,0 +1,106 @@
+"""Cases of the reference's own LazyTensor test files, run on the HIP backend with device tensors and compared
+with dense torch: pykeops/test/test_transpose.py, test_lazytensor_clamp.py, test_sinc.py,
+test_contiguous_torch.py, test_lazytensor_gaussian_inplace.py, test_lazytensor_grad.py (same shapes, seeds and
+tolerances)."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def test_transpose():
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(0)
+    x, y = torch.randn(1000, 3, device="cuda"), torch.randn(2000, 3, device="cuda")
+    K_keops = (-((LazyTensor(x[:, None, :]) - LazyTensor(y[None, :, :])) ** 2).sum(2)).exp()
+    K_torch = (-((x[:, None, :] - y[None, :, :]) ** 2).sum(2)).exp()
+    w = torch.rand(1000, 2, device="cuda")
+    assert torch.allclose(K_keops.t() @ w, K_torch.t() @ w, rtol=1e-5, atol=1e-4)
+
+
+def test_clamp_forward_and_backward():
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(0)
+    M, N, D = 1000, 1000, 3
+    x = torch.randn(M, 1, D, requires_grad=True, device="cuda")
+    y = torch.randn(1, N, D, device="cuda")
+    a, b = -1.23, 1.54
+
+    def fun(x, y, keops):
+        if keops:
+            x, y = LazyTensor(x), LazyTensor(y)
+        Dxy = ((x * y).clamp(a, b)).sum(dim=2)
+        return (-(Dxy ** 2)).exp().sum(dim=1)
+
+    out = [fun(x, y, k).squeeze() for k in (False, True)]
+    assert torch.allclose(out[0], out[1], rtol=1e-5, atol=1e-4)
+    g = [torch.autograd.grad((o ** 2).sum(), [x])[0] for o in out]
+    assert torch.allclose(g[0], g[1], atol=0.01, rtol=0.001)
+
+
+def test_sinc_and_its_gradient():
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(0)
+    x = (torch.rand(5, 1, dtype=torch.float64) * 2 * math.pi).cuda().requires_grad_(True)
+    y = x.detach().clone().requires_grad_(True)
+    s1 = LazyTensor(x[:, None]).sinc().sum(0)
+    s1.backward()
+    s2 = torch.sum(torch.sinc(y))
+    s2.backward()
+    assert torch.allclose(s1, s2) and torch.allclose(x.grad, y.grad)
+
+
+def test_non_contiguous_input_gives_the_same_result():
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(0)
+    a1 = torch.rand(2, 1000, 5, device="cuda")
+    a2 = a1.permute(2, 0, 1).contiguous().permute(1, 2, 0)   # same values, other strides
+    b, c = torch.rand(2, 1000, 5, device="cuda"), torch.rand(2, 1000, 5, device="cuda")
+    b_j = LazyTensor(b[:, None])
+    d1 = LazyTensor(a1[:, :, None]).sqdist(b_j).exp() @ c
+    with pytest.warns(UserWarning, match="not contiguous"):
+        d2 = LazyTensor(a2[:, :, None]).sqdist(b_j).exp() @ c
+    assert not a2.is_contiguous() and torch.equal(d2, d1)
+
+
+def test_matmul_into_a_preallocated_output():
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(0)
+    M, N, D, DV = 20, 30, 3, 1
+    x = torch.rand(M, 1, D, device="cuda") / math.sqrt(D)
+    y = torch.rand(1, N, D, device="cuda") / math.sqrt(D)
+    b = torch.randn(N, DV, device="cuda")
+    a = torch.empty(M, DV, device="cuda")
+    Kxy = (-((LazyTensor(x) - LazyTensor(y)).square()).sum(dim=2)).exp()
+    ret = Kxy.__matmul__(b, sum_scheme="block_sum", out=a)
+    ref = (-((x - y).square()).sum(dim=2)).exp() @ b
+    assert ret.data_ptr() == a.data_ptr() and torch.allclose(a, ref)
+
+
+def test_first_and_second_order_gradients():
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(0)
+    M, N, DV = 100, 100, 1
+    x = torch.rand(M, 1, 3, requires_grad=True, device="cuda")
+    y = torch.rand(1, N, 1, device="cuda")
+    b = torch.randn(N, DV, device="cuda")
+
+    def fun(x, y, keops):
+        if keops:
+            x, y = LazyTensor(x), LazyTensor(y)
+        return ((x.cos() - y).sum(dim=2) @ b).squeeze()
+
+    out = [fun(x, y, k) for k in (True, False)]
+    assert torch.allclose(out[0], out[1], rtol=1e-4)
+    g = [torch.autograd.grad((o ** 2).sum(), [x], create_graph=True)[0] for o in out]
+    assert torch.allclose(g[0], g[1], rtol=1e-4, atol=1e-4)
+    g2 = [torch.autograd.grad((gk ** 2).sum(), [x])[0] for gk in g]
+    assert torch.allclose(g2[0], g2[1], rtol=1e-3, atol=1e-2)
