@@ -22,6 +22,9 @@ dimfinalchunk = 64
 block_size = 256           # threads per workgroup (4 wavefronts)
 max_rows_per_lane = int(os.environ.get("KEOPS_AMD_MAX_ROWS", 4))      # output rows held in the registers of one lane
 lds_tile_bytes = 16384     # LDS bytes of one staged column tile
+# formula bodies of more than segment_threshold statements are cut into functions of segment_statements each
+segment_threshold = int(os.environ.get("KEOPS_AMD_SEGMENT_MIN", 1024))
+segment_statements = int(os.environ.get("KEOPS_AMD_SEGMENT", 512))
 lse_group = int(os.environ.get("KEOPS_AMD_LSE_GROUP", 8))  # log-sum-exp: columns folded per running-maximum update
 
 # matrix-core chunked scheme (csrc/kernels/keops_chunk_mfma.h): wavefronts (32 output rows each) per workgroup

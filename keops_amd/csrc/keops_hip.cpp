@@ -822,7 +822,10 @@ int keops_hip_compile(const char* target_file, const char* hip_src, int use_fast
   hiprtcResult r = hiprtcCreateProgram(&prog, hip_src, "keops_module.hip", (int)hdr_name.size(), hdr_text.data(), hdr_name.data());
   if (r != HIPRTC_SUCCESS) return fail((int)r, std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r));
   const std::string arch = "--offload-arch=" + target_arch(device_id);
-  std::vector<const char*> opts = {arch.c_str(), "-O3", "-std=c++17", "-fno-math-errno", "-ffp-contract=fast-honor-pragmas",
+  // optimisation level: -O3 unless KEOPS_HIP_OPT_LEVEL names another one (very long straight-line kernels)
+  const char* lvl = getenv("KEOPS_HIP_OPT_LEVEL");
+  const std::string olevel = std::string("-O") + (lvl && *lvl ? lvl : "3");
+  std::vector<const char*> opts = {arch.c_str(), olevel.c_str(), "-std=c++17", "-fno-math-errno", "-ffp-contract=fast-honor-pragmas",
                                    // packed FP32 instructions are kept out of every kernel of this library
                                    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
   const std::string fm = std::string("-DKEOPS_FAST_MATH=") + (use_fast_math ? "1" : "0");

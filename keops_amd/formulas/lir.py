@@ -262,16 +262,25 @@ class Lir:
             return "(T)INFINITY" if v > 0 else "-(T)INFINITY"
         return f"(T){v!r}" if self.dtype == "double" else f"{float(v)!r}f".replace("e+", "e")
 
-    def emit(self, outputs, names, indent="    "):
+    def emit(self, outputs, names, indent="    ", segment=0, segment_prefix=(), segment_min=0):
         """C++ statements computing ``outputs`` (value ids).
 
         ``names`` maps a load key (cat, ind, k) to the C++ expression that reads it.
         Returns (lines, exprs) where exprs[k] is the C++ expression of outputs[k].
+
+        ``segment`` > 0: a body of more than ``segment_min`` statements (formulas on vectors of hundreds of components)
+        is cut into non-inlined device functions ``keops_seg_<k>(xi, yj, p, keops_live)`` of at most that many
+        statements each, whose definitions are left in ``self.prelude`` (to be placed before the caller); values
+        that cross a cut travel through the array ``keops_live``.  The compiler's time grows much faster than
+        linearly with the length of one straight-line function; that of a sequence of bounded functions does not.
+        ``segment_prefix``: lines repeated at the top of every such function (pragmas).
         """
+        self.prelude = []
         live = self.live(outputs)
         f32 = self.dtype == "float"
         ref = {}
         lines = []
+        stmts = []  # (value id, is boolean, expression, ids of the operands)
         for i in sorted(live):
             n = self.nodes[i]
             op = n[0]
@@ -319,7 +328,43 @@ class Lir:
                 raise AssertionError(op)
             ref[i] = f"t{i}"
             lines.append(f"{indent}const {'bool' if boolean else 'T'} t{i} = {e};")
-        return lines, [ref[o] if self.nodes[o][0] not in ("const",) else ref[o] for o in outputs]
+            stmts.append((i, boolean, e, [j for j in (n[2:] if op == "call" else n[1:])]))
+        if not segment or len(stmts) <= max(segment, segment_min):
+            return lines, [ref[o] for o in outputs]
+
+        # ---- long bodies: bounded, non-inlined functions ----
+        seg_of = {st[0]: k // segment for k, st in enumerate(stmts)}
+        nseg = (len(stmts) + segment - 1) // segment
+        is_bool = {st[0]: st[1] for st in stmts}
+        crossing = {}  # value id -> slot of keops_live
+        for i, _, _, deps in stmts:
+            for j in deps:
+                if j in seg_of and seg_of[j] != seg_of[i] and j not in crossing:
+                    crossing[j] = len(crossing)
+        for o in outputs:
+            if o in seg_of and o not in crossing:
+                crossing[o] = len(crossing)
+        for k in range(nseg):
+            body = [st for st in stmts if seg_of[st[0]] == k]
+            fn = [f"static __device__ __attribute__((noinline)) void keops_seg_{k}(const T* __restrict__ xi, "
+                  f"const T* __restrict__ yj, const T* __restrict__ p, T* __restrict__ keops_live) {{"]
+            fn += list(segment_prefix)
+            ins = sorted({j for st in body for j in st[3] if j in seg_of and seg_of[j] != k})
+            for j in ins:
+                if is_bool[j]:
+                    fn.append(f"  const bool t{j} = keops_live[{crossing[j]}] != (T)0;")
+                else:
+                    fn.append(f"  const T t{j} = keops_live[{crossing[j]}];")
+            for i, boolean, e, _ in body:
+                fn.append(f"  const {'bool' if boolean else 'T'} t{i} = {e};")
+                if i in crossing:
+                    fn.append(f"  keops_live[{crossing[i]}] = {'(T)' if boolean else ''}t{i};")
+            fn.append("}")
+            self.prelude += fn
+        calls = [f"{indent}T keops_live[{max(1, len(crossing))}];"]
+        calls += [f"{indent}keops_seg_{k}(xi, yj, p, keops_live);" for k in range(nseg)]
+        exprs = [f"keops_live[{crossing[o]}]" if o in crossing else ref[o] for o in outputs]
+        return calls, exprs
 
 
 def lower(formula, L: Lir):

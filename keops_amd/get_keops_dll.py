@@ -92,9 +92,10 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
     exact = red.kind in (KIND_MIN, KIND_MAX, KIND_KMIN)
     L = Lir(row_cat=red.tagI, fast_math=use_fast_math, dtype=dtype, exact_order=exact)
     outs = lower(red.formula, L)
-    lines, exprs = L.emit(outs, layout.names, indent="    ")
-    if exact:
-        lines = ["    #pragma clang fp contract(off)"] + lines
+    pragma = ["    #pragma clang fp contract(off)"] if exact else []
+    lines, exprs = L.emit(outs, layout.names, indent="    ", segment=config.segment_statements, segment_prefix=pragma,
+                          segment_min=config.segment_threshold)
+    lines = pragma + lines
     nops = L.count_ops(outs)
     geo = choose_geometry(red, layout, nops, sizeof_t, nx, irregular)
     if geometry:
@@ -125,6 +126,7 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
                        ("col_off", co), ("par_arg", pa), ("par_dim", pd), ("par_off", po)):
         src.append(f"static __device__ constexpr int keops_{name}[] = {_c_list(vals)};")
     dx, dy, dp = max(1, layout.dimx), max(1, geo["dimy_pad"]), max(1, layout.dimp)
+    src += L.prelude
     src.append("struct KeopsFormula {")
     src.append(
         f"  static __device__ __forceinline__ void eval(const T (&xi)[{dx}], const T (&yj)[{dy}], "

@@ -104,3 +104,19 @@ def test_first_and_second_order_gradients():
     assert torch.allclose(g[0], g[1], rtol=1e-4, atol=1e-4)
     g2 = [torch.autograd.grad((gk ** 2).sum(), [x])[0] for gk in g]
     assert torch.allclose(g2[0], g2[1], rtol=1e-3, atol=1e-2)
+
+
+def test_min_argmin_of_a_formula_on_990_components():
+    """pykeops/test/test_torch.py::test_LazyTensor_min_chunked: vectors of 990 components, a formula that is not a
+    contraction (its long straight-line body is compiled as a chain of bounded functions)."""
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(0)
+    M, N, D = 120, 150, 990
+    x, y = torch.rand(M, D, device="cuda"), torch.rand(N, D, device="cuda")
+    K_ij = ((-((LazyTensor(x.unsqueeze(-2)) + LazyTensor(y.unsqueeze(-3))) ** 2)).exp()).sum(-1)
+    m, am = K_ij.min_argmin(dim=0)
+    dense = (-((x.unsqueeze(-2) + y.unsqueeze(-3)) ** 2)).exp().sum(-1, keepdim=True)
+    rm, ram = dense.min(dim=0)
+    assert m.shape == rm.shape and torch.allclose(m, rm, atol=1e-5, rtol=1e-5)
+    assert torch.equal(am.long(), ram)
