@@ -42,24 +42,40 @@ static inline float __builtin_amdgcn_rsqf(float x) { return 1.0f / std::sqrt(x);
 _cache = {}
 
 
-def dense_eval(formula, aliases, args, M, N, dtype=np.float64, fast_math=False):
+def dense_eval(formula, aliases, args, M, N, dtype=np.float64, fast_math=False, segment=0):
     """Evaluate a formula string (or Op) on all pairs.  args[k] is (M,d) | (N,d) | (d,) following the
-    category of variable k.  Returns an array (M, N, dim)."""
+    category of variable k.  Returns an array (M, N, dim).  ``segment`` > 0: the body is emitted as a chain of
+    functions of that many statements (the form used for very long formulas), on the concatenated xi / yj / p
+    arrays of the kernels."""
     op = parse(formula, aliases) if isinstance(formula, str) else formula
     ctype = "double" if np.dtype(dtype) == np.float64 else "float"
     L = Lir(row_cat=0, fast_math=fast_math, dtype=ctype)
     outs = lower(op, L)
-    names = {}
-    for v in op.variables:
-        for k in range(v.dim):
-            names[(v.cat, v.ind, k)] = f"a{v.ind}[{k}]"
-    lines, exprs = L.emit(outs, names)
-    decl = []
-    for v in op.variables:
-        idx = {0: "i", 1: "j", 2: "0"}[v.cat]
-        decl.append(f"    const T* a{v.ind} = (const T*)args[{v.ind}] + (int64_t){idx} * {v.dim};")
+    names, decl = {}, []
+    if segment:
+        off = {0: 0, 1: 0, 2: 0}
+        arr = {0: "xi", 1: "yj", 2: "p"}
+        copies = []
+        for v in op.variables:
+            idx = {0: "i", 1: "j", 2: "0"}[v.cat]
+            for k in range(v.dim):
+                names[(v.cat, v.ind, k)] = f"{arr[v.cat]}[{off[v.cat] + k}]"
+            copies.append(f"    for (int k = 0; k < {v.dim}; k++) {arr[v.cat]}[{off[v.cat]} + k] = "
+                          f"((const T*)args[{v.ind}] + (int64_t){idx} * {v.dim})[k];")
+            off[v.cat] += v.dim
+        decl = [f"    T xi[{max(1, off[0])}], yj[{max(1, off[1])}], p[{max(1, off[2])}];"] + copies
+        lines, exprs = L.emit(outs, names, segment=segment, segment_min=0)
+    else:
+        for v in op.variables:
+            for k in range(v.dim):
+                names[(v.cat, v.ind, k)] = f"a{v.ind}[{k}]"
+        lines, exprs = L.emit(outs, names)
+        for v in op.variables:
+            idx = {0: "i", 1: "j", 2: "0"}[v.cat]
+            decl.append(f"    const T* a{v.ind} = (const T*)args[{v.ind}] + (int64_t){idx} * {v.dim};")
     body = "\n".join(decl + lines + [f"    o[{k}] = {e};" for k, e in enumerate(exprs)])
-    src = _PREAMBLE % dict(T=ctype) + f"""
+    prelude = "#define __device__\n" + "\n".join(L.prelude) + "\n"
+    src = _PREAMBLE % dict(T=ctype) + prelude + f"""
 extern "C" void dense(int64_t M, int64_t N, const void* const* args, T* out) {{
   for (int64_t i = 0; i < M; i++) for (int64_t j = 0; j < N; j++) {{
     T* o = out + (i * N + j) * {op.dim};

@@ -294,3 +294,18 @@ def test_forward_mode_through_log_sum_exp_reduction():
     # a tangent that the formula does not depend on gives the zero reduction
     z = parse_reduction("Diff_WithSavedForward(Max_SumShiftExpWeight_Reduction(-SqDist(x,y),0,w),Var(5,1,2),Var(6,1,2),ms)", al)
     assert z.string_id == "Zero_Reduction"
+
+
+def test_long_bodies_as_chains_of_functions():
+    """The segmented emission (functions of a few statements chained through a value array) computes what the
+    single straight-line body computes, including boolean values that cross a cut and outputs that are loads or
+    constants."""
+    al = ["x=Vi(0,6)", "y=Vj(1,6)", "g=Pm(2,1)"]
+    a = [_t(M, 6).numpy(), _t(N, 6).numpy(), _t(1, lo=0.5, hi=1.5).numpy()]
+    for formula in (
+        "Concat(Exp(-g*SqDist(x,y))*(x+y), IfElse(x-y, Abs(x)*Step(y), Sin(x*y)+Square(y)))",
+        "Concat(Concat(x, IntCst(2)), Sum(Sqrt(Abs(x-y)))*Extract(y,1,2))",
+    ):
+        whole = dense_eval(formula, al, a, M, N)
+        for seg in (1, 3, 7):
+            assert np.array_equal(dense_eval(formula, al, a, M, N, segment=seg), whole), (formula, seg)
