@@ -120,3 +120,35 @@ def test_min_argmin_of_a_formula_on_990_components():
     rm, ram = dense.min(dim=0)
     assert m.shape == rm.shape and torch.allclose(m, rm, atol=1e-5, rtol=1e-5)
     assert torch.equal(am.long(), ram)
+
+
+@pytest.mark.parametrize("shapes,in_dims,out_dims", [
+    (((5, 10, 1, 2), (5, 1, 20, 2), (5, 1, 20, 1)), 0, 0),
+    (((10, 5, 1, 2), (1, 5, 20, 2), (1, 5, 20, 1)), 1, 1),
+    (((10, 5, 1, 2), (5, 1, 20, 2), (1, 5, 20, 1)), (1, 0, 1), 2),
+])
+def test_vmap_with_in_and_out_dims_and_gradient(shapes, in_dims, out_dims):
+    """pykeops/test/test_vmap.py: torch.vmap over different positions of the mapped dimension, and a gradient
+    taken through the mapped function."""
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(0)
+    kw = dict(dtype=torch.float64, device="cuda")
+    x_i = torch.randn(*shapes[0], requires_grad=True, **kw)
+    x_j, y_j = torch.randn(*shapes[1], **kw), torch.randn(*shapes[2], **kw)
+
+    def fn(x_i, x_j, y_j, use_keops=True):
+        if use_keops:
+            x_i, x_j, y_j = LazyTensor(x_i), LazyTensor(x_j), LazyTensor(y_j)
+        K_ij = (-((x_i - x_j) ** 2).sum(-1)).exp()
+        if not use_keops:
+            K_ij = K_ij[..., None]
+        return (K_ij * y_j).sum(1)
+
+    res_keops = torch.vmap(fn, in_dims=in_dims, out_dims=out_dims)(x_i, x_j, y_j, use_keops=True)
+    res_torch = torch.vmap(fn, in_dims=in_dims, out_dims=out_dims)(x_i, x_j, y_j, use_keops=False)
+    assert torch.allclose(res_keops, res_torch)
+    u = torch.rand(res_torch.shape, **kw)
+    (g_torch,) = torch.autograd.grad(res_torch, x_i, u)
+    (g_keops,) = torch.autograd.grad(res_keops, x_i, u)
+    assert torch.allclose(g_keops, g_torch)
