@@ -63,6 +63,21 @@ class GenredAutograd_base:
         nbatchdims = max(len(a.shape) for a in args) - 2
         use_ranges = nbatchdims > 0 or params.ranges is not None
         device_id, device_args = set_device(tagCPUGPU, tagHostDevice, params.device_id_request, *args)
+        host_out, staged = None, False
+        if tagCPUGPU == 1 and tagHostDevice == 0:
+            # host-resident tensors with a GPU backend: staged through device memory, as the reference's binder
+            # does in load_args_FromHost (keops_nvrtc.cpp:46-73); the library itself only takes device pointers
+            if not torch.cuda.is_available():
+                raise ValueError("[KeOps] the HIP backend needs a GPU: none is visible to torch")
+            dev = torch.device("cuda", device_id)
+            args = tuple(a.to(dev) for a in args)
+            if params.ranges:
+                params = copy.copy(params)
+                params.ranges = tuple(r.to(dev) for r in params.ranges)
+            if params.out is not None:
+                params = copy.copy(params)
+                host_out, params.out = params.out, None
+            tagHostDevice, device_args, staged = 1, dev, True
         nout = params.nx if params.axis == 1 else params.ny
         myconv = keops_binder["hip"](
             tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id, params.formula, params.aliases, len(args),
@@ -77,6 +92,11 @@ class GenredAutograd_base:
         if params.ranges:
             params.ranges = tuple(r.to(memory_format=torch.contiguous_format, dtype=torch.int64) for r in params.ranges)
         result = myconv.genred_pytorch(device_args, params.ranges, params.nx, params.ny, nbatchdims, params.out, *args)
+        if host_out is not None:
+            host_out.copy_(result.view(host_out.shape))
+            result = host_out
+        elif staged:
+            result = result.cpu()
         return result, torch.tensor([myconv.dimout, myconv.tagIJ])
 
     @staticmethod

@@ -152,3 +152,28 @@ def test_vmap_with_in_and_out_dims_and_gradient(shapes, in_dims, out_dims):
     (g_torch,) = torch.autograd.grad(res_torch, x_i, u)
     (g_keops,) = torch.autograd.grad(res_keops, x_i, u)
     assert torch.allclose(g_keops, g_torch)
+
+
+def test_host_resident_tensors_are_staged_through_the_device():
+    """pykeops/test/test_lazytensor_gaussian_fromhost.py: tensors in host memory with the GPU backend, result
+    back in host memory; gradient and a preallocated host output as well."""
+    from keops_amd.torch import Genred, LazyTensor
+
+    torch.manual_seed(0)
+    M, N, D, DV = 2500, 2000, 3, 1
+    x = (torch.rand(M, 1, D, dtype=torch.float64) / math.sqrt(D)).requires_grad_(True)
+    y = torch.rand(1, N, D, dtype=torch.float64) / math.sqrt(D)
+    b = torch.randn(N, DV, dtype=torch.float64)
+    Kxy = (-((LazyTensor(x) - LazyTensor(y)).square()).sum(dim=2)).exp()
+    out = Kxy.__matmul__(b, sum_scheme="block_sum", device_id=0)
+    ref = (-((x - y).square()).sum(dim=2)).exp() @ b
+    assert out.device.type == "cpu" and torch.allclose(out, ref)
+    (g,) = torch.autograd.grad(out.sum(), [x])
+    (gr,) = torch.autograd.grad(ref.sum(), [x])
+    assert g.device.type == "cpu" and torch.allclose(g, gr)
+    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(1)"], reduction_op="Sum", axis=1)
+    a = torch.empty(M, DV, dtype=torch.float64)
+    ret = conv(x.detach()[:, 0], y[0], b, out=a)
+    assert ret.data_ptr() == a.data_ptr() and torch.allclose(a, ref.detach())
+    with pytest.raises(ValueError):
+        conv(x.detach()[:, 0], y[0], b, backend="CPU")   # no CPU implementation behind this API
