@@ -1150,6 +1150,155 @@ def OneHot(f, dim):
     return OneHotNode(as_op(f), dim)
 
 
+class BSplineImplNode(Op):
+    """All B-spline functions of order ``order`` on the knot vector ``knots``, sampled at the scalar ``x``, by
+    De Boor's recursion in place (maths/BSpline.py:19-95): n_knots - 1 values, of which the first
+    n_knots - order - 1 are the splines (the others are intermediate storage)."""
+
+    name = "BSpline_Impl"
+    __slots__ = ()
+
+    def __init__(self, knots, x, order):
+        order = int(order)
+        if order < 0:
+            raise FormulaError(f"The order of a BSpline must be >= 0, but received {order}.")
+        if x.dim != 1:
+            raise FormulaError(f"BSplines must be sampled at scalar values, but received a vector of size {x.dim}.")
+        if knots.dim < order + 2:
+            raise FormulaError(f"BSplines of order {order} require at least {order + 2} knots, but only received "
+                               f"a vector of size {knots.dim}.")
+        super().__init__((knots, x), (order,), knots.dim - 1)
+
+    def lower(self, L, kids):
+        t, (x,) = kids
+        one, zero = L.const(1.0), L.const(0.0)
+        # order 0: indicator of t[j] <= x < t[j+1]
+        out = [L.select(L.le(t[j], x), L.select(L.lt(x, t[j + 1]), one, zero), zero) for j in range(self.dim)]
+
+        def ratio(lo, hi):  # (x - t_lo) / (t_hi - t_lo), 0 on an empty knot span
+            return L.select(L.lt(t[lo], t[hi]), L.div(L.sub(x, t[lo]), L.sub(t[hi], t[lo])), zero)
+
+        for k in range(1, self.params[0] + 1):
+            r1 = ratio(0, k)
+            for i in range(self.dim - k):
+                r2 = ratio(i + 1, i + 1 + k)
+                out[i] = L.add(L.mul(r1, out[i]), L.mul(L.sub(one, r2), out[i + 1]))
+                r1 = r2
+        return out
+
+    def diff_t(self, v, gradin):
+        raise NotImplementedError("KeOps BSplines are not yet differentiable. Please consider disabling autograd "
+                                  "for the relevant variables with 'x.detach()'.")
+
+
+def BSpline(knots, x, order):
+    """Vector of the n_knots - order - 1 B-spline functions of order ``order`` at x (maths/BSpline.py:112-115)."""
+    knots, x = as_op(knots), as_op(x)
+    return Extract(BSplineImplNode(knots, x, order), 0, knots.dim - int(order) - 1)
+
+
+def _softdtw_table(L, x, y, gamma):
+    """r[j][i] of the soft dynamic time warping recursion on squared differences (maths/SoftDTW_SqDist.py:31-69):
+    r = (x_i - y_j)^2 + softmin_gamma(r[j-1][i-1], r[j-1][i], r[j][i-1])."""
+    n, m = len(x), len(y)
+    r = [[None] * n for _ in range(m)]
+
+    def d2(i, j):
+        d = L.sub(x[i], y[j])
+        return L.mul(d, d)
+
+    def fmin(a, b):
+        return L.select(L.lt(b, a), b, a)
+
+    r[0][0] = d2(0, 0)
+    for i in range(1, n):
+        r[0][i] = L.add(d2(i, 0), r[0][i - 1])
+    for j in range(1, m):
+        r[j][0] = L.add(d2(0, j), r[j - 1][0])
+        for i in range(1, n):
+            a, b, c = r[j - 1][i - 1], r[j - 1][i], r[j][i - 1]
+            mn = fmin(fmin(a, b), c)
+            e = L.add(L.add(L.exp(L.div(L.sub(mn, a), gamma)), L.exp(L.div(L.sub(mn, c), gamma))),
+                      L.exp(L.div(L.sub(mn, b), gamma)))
+            r[j][i] = L.add(d2(i, j), L.sub(mn, L.mul(gamma, L.log(e))))
+    return r
+
+
+class SoftDTWSqDistNode(Op):
+    """Soft-DTW discrepancy between the series x (size n) and y (size m) with smoothing gamma, on squared
+    differences (maths/SoftDTW_SqDist.py:21-83)."""
+
+    name = "SoftDTW_SqDist"
+    __slots__ = ()
+
+    def __init__(self, x, y, gamma):
+        if gamma.dim != 1:
+            raise FormulaError("input gamma should be scalar")
+        super().__init__((x, y, gamma), (), 1)
+
+    def lower(self, L, kids):
+        x, y, (gamma,) = kids
+        return [_softdtw_table(L, x, y, gamma)[-1][-1]]
+
+    def diff_t(self, v, gradin):
+        x, y, gamma = self.children
+        if v in gamma.variables:
+            raise FormulaError("autograd wrt gamma in SoftDTW_SqDist operation not implemented.")
+        grad = Mult(GradSoftDTWSqDistNode(x, y, gamma), gradin)
+        return Add(x.diff_t(v, Extract(grad, 0, x.dim)), y.diff_t(v, Extract(grad, x.dim, y.dim)))
+
+
+class GradSoftDTWSqDistNode(Op):
+    """Gradient of SoftDTW_SqDist with respect to (x, y), size n + m: forward table, then the backward recursion
+    on the alignment weights e[j][i] (maths/SoftDTW_SqDist.py:86-213)."""
+
+    name = "GradSoftDTW_SqDist"
+    __slots__ = ()
+
+    def __init__(self, x, y, gamma):
+        if gamma.dim != 1:
+            raise FormulaError("input gamma should be scalar")
+        super().__init__((x, y, gamma), (), x.dim + y.dim)
+
+    def lower(self, L, kids):
+        x, y, (gamma,) = kids
+        n, m = len(x), len(y)
+        r = _softdtw_table(L, x, y, gamma)
+        two = L.const(2.0)
+
+        def diff(i, j):
+            return L.sub(x[i], y[j])
+
+        def w(r_to, r_from, d):  # exp((r_to - r_from - d^2) / gamma): share of cell `to` that came through `from`
+            return L.exp(L.div(L.sub(L.sub(r_to, r_from), L.mul(d, d)), gamma))
+
+        e = [[None] * n for _ in range(m)]
+        e[m - 1][n - 1] = L.const(1.0)
+        for i in range(n - 2, -1, -1):
+            e[m - 1][i] = L.mul(w(r[m - 1][i + 1], r[m - 1][i], diff(i + 1, m - 1)), e[m - 1][i + 1])
+        for j in range(m - 2, -1, -1):
+            e[j][n - 1] = L.mul(w(r[j + 1][n - 1], r[j][n - 1], diff(n - 1, j + 1)), e[j + 1][n - 1])
+            for i in range(n - 2, -1, -1):
+                a = w(r[j][i + 1], r[j][i], diff(i + 1, j))
+                b = w(r[j + 1][i], r[j][i], diff(i, j + 1))
+                c = w(r[j + 1][i + 1], r[j][i], diff(i + 1, j + 1))
+                e[j][i] = L.add(L.add(L.mul(a, e[j][i + 1]), L.mul(b, e[j + 1][i])), L.mul(c, e[j + 1][i + 1]))
+        gx, gy = [L.const(0.0)] * n, [L.const(0.0)] * m
+        for j in range(m):
+            for i in range(n):
+                t = L.mul(L.mul(two, diff(i, j)), e[j][i])
+                gx[i] = L.add(gx[i], t)
+                gy[j] = L.sub(gy[j], t)
+        return gx + gy
+
+    def diff_t(self, v, gradin):
+        raise FormulaError("autograd for GradSoftDTW_SqDist operation not implemented.")
+
+
+def SoftDTW_SqDist(x, y, gamma):
+    return SoftDTWSqDistNode(as_op(x), as_op(y), as_op(gamma))
+
+
 class VecReduceNode(Op):
     """Max / Min / ArgMax / ArgMin over the components of a vector formula."""
 
@@ -1428,7 +1577,9 @@ BUILDERS = dict(
     IfElse=IfElse, Clamp=Clamp, ClampInt=ClampInt, DiffClampInt=DiffClampInt, Mod=Mod, Sum=Sum, SumT=SumT,
     Scalprod=Scalprod, Concat=Concat, Extract=Extract, ExtractT=ExtractT, OneHot=OneHot, Max=Max, Min=Min,
     ArgMax=ArgMax, ArgMin=ArgMin, MatVecMult=MatVecMult, VecMatMult=VecMatMult, TensorProd=TensorProd,
-    TensorDot=TensorDot,
+    TensorDot=TensorDot, SoftDTW_SqDist=SoftDTW_SqDist,
+    GradSoftDTW_SqDist=lambda x, y, g: GradSoftDTWSqDistNode(as_op(x), as_op(y), as_op(g)),
+    BSpline_Impl=lambda knots, x, order: BSplineImplNode(as_op(knots), as_op(x), order),
 )
 
 # names that only exist as constructors (they expand into the nodes above)
@@ -1436,7 +1587,7 @@ FUNCTIONS = dict(
     BUILDERS,
     Vi=Vi, Vj=Vj, Pm=Pm, IntInv=IntInv, SqNorm2=SqNorm2, Norm2=Norm2, SqDist=SqDist, Normalize=Normalize,
     WeightedSqNorm=WeightedSqNorm, WeightedSqDist=WeightedSqDist, Elem=Elem, ElemT=ElemT,
-    Kron=Kron, SqNormIso=SqNormIso, SqNormDiag=SqNormDiag, SymSqNorm=SymSqNorm, Ind=Ind,
+    Kron=Kron, SqNormIso=SqNormIso, SqNormDiag=SqNormDiag, SymSqNorm=SymSqNorm, Ind=Ind, BSpline=BSpline,
 )
 
 
@@ -1451,6 +1602,22 @@ def Grad(formula, v, gradin=None):
 
 
 FUNCTIONS["Grad"] = Grad
+
+
+def GradMatrix(f, v):
+    """Matrix of the gradient operator of f with respect to v (transpose of the Jacobian), row by row: the
+    concatenation over the standard basis e_k of the output space of [d_v f]^T e_k (maths/GradMatrix.py:22-34)."""
+    f, v = as_op(f), as_op(v)
+    if not isinstance(v, Var):
+        raise FormulaError("GradMatrix(F, v): v must be a variable")
+    res = None
+    for k in range(f.dim):
+        g = f.diff_t(v, ElemT(IntCst(1), f.dim, k))
+        res = g if res is None else Concat(res, g)
+    return res
+
+
+FUNCTIONS["GradMatrix"] = GradMatrix
 
 
 def _fresh_probe(dim, *formulas):

@@ -393,6 +393,19 @@ class LazyTensor:
         """torch-style alias of :meth:`concatenate`."""
         return LazyTensor.concatenate(tuple_of_lt, dim)
 
+    def softdtw_sqdist(self, other, gamma):
+        """Soft-DTW discrepancy (squared differences) between the series self and other, smoothing gamma."""
+        return self.ternary(other, gamma, O.SoftDTW_SqDist)
+
+    def grad_matrix(self, other):
+        """Matrix of the gradient operator of self with respect to the variable other, flattened row by row."""
+        other = self._lift(other)
+        return self._like(O.GradMatrix(self.formula, other.formula), other)
+
+    def bspline(self, x, k=0):
+        """Vector of B-spline functions of order k for the knots ``self``, evaluated at the scalar x."""
+        return self.binary(x, lambda knots, t: O.BSpline(knots, t, k))
+
     def one_hot(self, D):
         return self.unary(O.OneHot, D)
 

@@ -309,3 +309,68 @@ def test_long_bodies_as_chains_of_functions():
         whole = dense_eval(formula, al, a, M, N)
         for seg in (1, 3, 7):
             assert np.array_equal(dense_eval(formula, al, a, M, N, segment=seg), whole), (formula, seg)
+
+
+@pytest.mark.parametrize("order", [0, 1, 3])
+def test_bspline_against_scipy(order):
+    """BSpline(knots, x, order): the n_knots - order - 1 basis functions of De Boor's recursion, against
+    scipy.interpolate.BSpline.basis_element on a non-uniform knot vector with a repeated knot."""
+    from scipy.interpolate import BSpline as SciBSpline
+
+    knots = np.array([[0.0, 0.5, 0.5, 1.2, 2.0, 2.7, 3.1, 4.0]])
+    nk = knots.shape[1]
+    P = 57
+    x = np.linspace(-0.313, 4.237, P)[:, None]  # no sample on a knot: scipy closes the last span on the right
+    al = [f"t=Pm(0,{nk})", "x=Vi(1,1)"]
+    got = dense_eval(f"BSpline(t,x,{order})", al, [knots[0], x], P, 1)[:, 0, :]
+    assert got.shape == (P, nk - order - 1)
+    ref = np.zeros_like(got)
+    for i in range(nk - order - 1):
+        if knots[0, i] < knots[0, i + order + 1]:
+            b = SciBSpline.basis_element(knots[0, i:i + order + 2], extrapolate=False)(x[:, 0])
+            ref[:, i] = np.nan_to_num(b)
+    inside = (x[:, 0] >= 0.0) & (x[:, 0] < 4.0)
+    assert np.allclose(got[inside], ref[inside], atol=1e-12)
+    assert np.all(got[~inside] == 0)
+    assert np.allclose(got[(x[:, 0] >= knots[0, order]) & (x[:, 0] < knots[0, nk - order - 1])].sum(1), 1.0)  # partition of unity
+    with pytest.raises(FormulaError):
+        parse("BSpline(t,x,7)", al)
+    with pytest.raises(NotImplementedError):
+        O.Grad(parse(f"BSpline(t,x,{order})", al), O.Var(1, 1, 0), O.Var(2, nk - order - 1, 0))
+
+
+def test_softdtw_and_grad_matrix():
+    """SoftDTW_SqDist against a plain torch dynamic program (value and gradients through autograd), and
+    GradMatrix against torch.func.jacrev."""
+    n, m = 5, 4
+    x, y, g = _t(M, n), _t(N, m), _t(1, lo=0.3, hi=0.9)
+
+    def softdtw(xv, yv, gam):
+        r = [[None] * n for _ in range(m)]
+        for j in range(m):
+            for i in range(n):
+                d2 = (xv[..., i] - yv[..., j]) ** 2
+                if i == 0 and j == 0:
+                    r[j][i] = d2
+                elif j == 0:
+                    r[j][i] = d2 + r[j][i - 1]
+                elif i == 0:
+                    r[j][i] = d2 + r[j - 1][i]
+                else:
+                    prev = torch.stack([r[j - 1][i - 1], r[j - 1][i], r[j][i - 1]], -1)
+                    r[j][i] = d2 - gam * torch.logsumexp(-prev / gam, -1)
+        return r[m - 1][n - 1][..., None]
+
+    al = [f"x=Vi(0,{n})", f"y=Vj(1,{m})", "g=Pm(2,1)"]
+    _check("SoftDTW_SqDist(x,y,g)", al, [x, y, g], lambda xv, yv, gv: softdtw(xv, yv, gv[..., 0]), grad_wrt=(0, 1), tol=1e-9)
+
+    al2 = ["x=Vi(0,3)", "y=Vj(1,3)"]
+    x3, y3 = _t(M, 3), _t(N, 3)
+
+    def F(xv, yv):
+        return torch.cat([torch.exp(-((xv - yv) ** 2).sum(-1, keepdim=True)) * yv[..., :1], (xv * yv)[..., 1:]], -1)
+
+    got = dense_eval("GradMatrix(Concat(Exp(-SqDist(x,y))*Elem(y,0), Extract(x*y,1,2)), x)", al2, [x3.numpy(), y3.numpy()], M, N)
+    xb, yb = x3[:, None, :].expand(M, N, 3), y3[None, :, :].expand(M, N, 3)
+    jac = torch.func.vmap(torch.func.vmap(torch.func.jacrev(F)))(xb, yb)      # (M, N, out 3, in 3)
+    assert np.allclose(got, jac.reshape(M, N, 9).numpy(), rtol=1e-10, atol=1e-10)

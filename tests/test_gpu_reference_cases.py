@@ -177,3 +177,40 @@ def test_host_resident_tensors_are_staged_through_the_device():
     assert ret.data_ptr() == a.data_ptr() and torch.allclose(a, ref.detach())
     with pytest.raises(ValueError):
         conv(x.detach()[:, 0], y[0], b, backend="CPU")   # no CPU implementation behind this API
+
+
+def test_softdtw_bspline_and_grad_matrix_on_the_device():
+    """The three operations of keopscore/formulas/maths that are dynamic programs or operators on formulas
+    (SoftDTW_SqDist.py, BSpline.py, GradMatrix.py), reduced on the device and compared with the host evaluation of
+    the same formulas."""
+    import numpy as np
+
+    from host_eval import dense_eval
+    from keops_amd.torch import LazyTensor
+
+    torch.manual_seed(3)
+    M, N = 60, 70
+    x = torch.rand(M, 6, dtype=torch.float64, device="cuda")
+    y = torch.rand(N, 5, dtype=torch.float64, device="cuda")
+    x_i, y_j = LazyTensor(x[:, None, :]), LazyTensor(y[None, :, :])
+    got = x_i.softdtw_sqdist(y_j, 0.5).sum(dim=1)
+    al = ["x=Vi(0,6)", "y=Vj(1,5)"]
+    ref = dense_eval("SoftDTW_SqDist(x,y,0.5)", al, [x.cpu().numpy(), y.cpu().numpy()], M, N).sum(1)
+    assert np.allclose(got.cpu().numpy(), ref, rtol=1e-10)
+    xg = x.clone().requires_grad_(True)
+    (g,) = torch.autograd.grad(LazyTensor(xg[:, None, :]).softdtw_sqdist(y_j, 0.5).sum(dim=1).sum(), [xg])
+    refg = dense_eval("Grad(SoftDTW_SqDist(x,y,0.5),x,Var(2,1,1))", al, [x.cpu().numpy(), y.cpu().numpy(), np.ones((N, 1))], M, N).sum(1)
+    assert np.allclose(g.cpu().numpy(), refg, rtol=1e-9, atol=1e-12)
+
+    knots = torch.tensor([0.0, 0.2, 0.35, 0.6, 0.8, 1.0, 1.3], dtype=torch.float64, device="cuda")
+    t_i = LazyTensor(x[:, None, :1])
+    spl = LazyTensor(knots.view(1, 1, -1)).bspline(t_i * y_j[0], 2).sum(dim=1)
+    refs = dense_eval("BSpline(k,Elem(x,0)*Elem(y,0),2)", al + ["k=Pm(2,7)"], [x.cpu().numpy(), y.cpu().numpy(), knots.cpu().numpy()], M, N).sum(1)
+    assert spl.shape == (M, 4) and np.allclose(spl.cpu().numpy(), refs, rtol=1e-10, atol=1e-12)
+
+    u_i, v_j = LazyTensor(x[:, None, :3].contiguous()), LazyTensor(y[None, :, :3].contiguous())
+    gm = (-(u_i - v_j) ** 2).exp().grad_matrix(u_i)
+    assert gm.shape == (M, N, 9)
+    refm = dense_eval("GradMatrix(Exp(-Square(u-v)),u)", ["u=Vi(0,3)", "v=Vj(1,3)"],
+                      [x[:, :3].cpu().numpy(), y[:, :3].cpu().numpy()], M, N).sum(1)
+    assert np.allclose(gm.sum(dim=1).cpu().numpy(), refm, rtol=1e-10, atol=1e-12)
