@@ -36,6 +36,7 @@ final_chunk_min_dim = int(os.environ.get("KEOPS_AMD_FINAL_MIN_DIM", 24))   # sma
 final_max_blocks = int(os.environ.get("KEOPS_AMD_FINAL_NB", 8))            # 32-column accumulator tiles per wavefront
 final_waves = int(os.environ.get("KEOPS_AMD_FINAL_WAVES", 8))              # wavefronts (32 output rows each) per workgroup
 final_tile_j = int(os.environ.get("KEOPS_AMD_FINAL_TJ", 32))               # reduced rows per staged tile (even)
+final_split3 = os.environ.get("KEOPS_AMD_FINAL_SPLIT3", "1") != "0"          # product in three bfloat16 terms per operand
 final_period = int(os.environ.get("KEOPS_AMD_FINAL_PERIOD", 4096))         # block-sum period in reduced rows
 
 # matrix-core KNN kernel (csrc/kernels/keops_knn_mfma.h)

@@ -747,6 +747,7 @@ struct FinHeader {
   int64_t slab_len;
   int32_t nslabs;
   int32_t pad_;
+  void* vsplit;
   RangeHeader rt;
 };
 
@@ -771,17 +772,25 @@ int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   FinHeader h{};
   h.nx = nx; h.ny = ny; h.out = out; h.slab_len = len; h.nslabs = (int32_t)nslabs;
   if (rg) h.rt = rg->header(m.nargs);
-  if (nslabs > 1) {
-    if (int rc = m.partial.reserve((size_t)nslabs * nx * DV * 4)) return rc;
-    h.partial = m.partial.ptr;
+  // split-operand variant (dense launches): v rewritten once as three bfloat16 terms, tile by tile
+  const bool split3 = !rg && m.meta_int("fin_split3", 0) != 0;
+  const int64_t DVP = (DV + 31) / 32 * 32, ntiles = (ny + TJ - 1) / TJ;
+  const size_t part_bytes = nslabs > 1 ? align_up((size_t)nslabs * nx * DV * 4, 256) : 0;
+  const size_t split_bytes = split3 ? (size_t)ntiles * 3 * DVP * TJ * 2 : 0;
+  if (part_bytes + split_bytes > 0) {
+    if (int rc = m.partial.reserve(part_bytes + split_bytes)) return rc;
+    if (nslabs > 1) h.partial = m.partial.ptr;
+    if (split3) h.vsplit = (char*)m.partial.ptr + part_bytes;
   }
   std::vector<char> buf(sizeof(FinHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs));
   std::memcpy(buf.data(), &h, sizeof(h));
   for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
   if (rg && rg->user_ranges)
     if (int rc = launch_raw(m, "keops_fin_fill_neutral", (unsigned)((nx * DV + 255) / 256), 1, 256, buf.data(), buf.size(), stream)) return rc;
+  if (split3)
+    if (int rc = launch_raw(m, "keops_fin_split", (unsigned)((ntiles * DVP * TJ + 255) / 256), 1, 256, buf.data(), buf.size(), stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
-  if (int rc = launch_raw3(m, "keops_fin_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)NZ, (unsigned)m.block, buf.data(), buf.size(), stream)) return rc;
+  if (int rc = launch_raw3(m, split3 ? "keops_fin_main3" : "keops_fin_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)NZ, (unsigned)m.block, buf.data(), buf.size(), stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
   if (nslabs > 1) {
     const int64_t gb = (nx * DV + 255) / 256;

@@ -41,6 +41,7 @@ struct FinParams {
   i64 slab_len;    // reduced rows per slab (multiple of FIN_TJ)
   int nslabs;
   int pad_;
+  __bf16* vsplit;       // keops_fin_split: v as three bfloat16 terms, [tile][term][column][row in tile]
   KeopsRangeTables rt;  // block-sparse / batch geometry (KEOPS_MC_RANGES)
   const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
 };
@@ -209,5 +210,211 @@ extern "C" __global__ void __launch_bounds__(256) keops_fin_reduce(const FinPara
 extern "C" __global__ void __launch_bounds__(256) keops_fin_fill_neutral(const FinParams P) {
   const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
   if (e < P.nx * FIN_DV) P.out[e] = (T)0;
+}
+#endif
+
+// ---- the same product with every operand written as three bfloat16 terms ------------------------------
+//
+// x = h + m + l with h = bf16(x), m = bf16(x - h), l = bf16(x - h - m) carries the 24 significant bits of a
+// float32, and f * v ~ hh + (hm + mh) + (hl + lh + mm) drops terms below 2^-24 |f v| only: float32 accuracy
+// from six v_mfma_f32_32x32x16_bf16 (6 x 32 cycles per 32 x 32 x 16 block) where the float32 instruction
+// v_mfma_f32_32x32x2_f32 needs 8 x 64 cycles.  Dense launches only (the pre-split copy of v is laid out tile by
+// tile from reduced row 0):
+//   * keops_fin_split writes v once as [tile][term][column][row in tile] bfloat16, zero past the last row and
+//     column, so that a workgroup stages a tile with straight 16-byte copies and a lane reads the 8 consecutive
+//     reduced rows of its B operand (column l % 32, rows 8 (l / 32) ..) with one ds_read_b128 (rows padded to
+//     FIN_TS elements: conflict-free);
+//   * lane l evaluates f for output row l % 32 and the 8 reduced rows 8 (l / 32) .. of a 16-row block -- the A
+//     operand layout -- and splits the 8 values in registers.
+#if defined(FIN_SPLIT3) && FIN_SPLIT3 && !KEOPS_MC_RANGES
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 fin_bf16x8;
+#define FIN_TS (FIN_TJ + 8)            // bfloat16 elements per staged column (padded)
+#define FIN_DVP (FIN_NBTOT * 32)       // columns of the split copy
+
+extern "C" __global__ void __launch_bounds__(256) keops_fin_split(const FinParams P) {
+  const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;   // one (tile, column, row in tile)
+  const i64 ntiles = (P.ny + FIN_TJ - 1) / FIN_TJ;
+  if (e >= ntiles * FIN_DVP * FIN_TJ) return;
+  const int r = (int)(e % FIN_TJ);
+  const int c = (int)((e / FIN_TJ) % FIN_DVP);
+  const i64 tile = e / ((i64)FIN_TJ * FIN_DVP);
+  const i64 j = tile * FIN_TJ + r;
+  const float x = (j < P.ny && c < FIN_DV) ? P.arg[FIN_VARG][j * FIN_DV + c] : 0.f;
+  const __bf16 h = (__bf16)x;
+  const float r1 = x - (float)h;
+  const __bf16 m = (__bf16)r1;
+  const __bf16 l = (__bf16)(r1 - (float)m);
+  __bf16* dst = P.vsplit + (tile * 3 * FIN_DVP + c) * FIN_TJ + r;
+  dst[0] = h;
+  dst[(i64)FIN_DVP * FIN_TJ] = m;
+  dst[(i64)2 * FIN_DVP * FIN_TJ] = l;
+}
+
+extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const FinParams P) {
+  __shared__ __attribute__((aligned(16))) __bf16 vt[3 * FIN_VS * FIN_TS];  // [term][column][row], this workgroup's column blocks
+  __shared__ __attribute__((aligned(16))) T ys[2][FIN_TJ * FIN_DY];         // reduced-index variables of f: this tile and the next
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const i64 row0 = (i64)blockIdx.x * FIN_QB + wave * 32;  // first output row of this wavefront
+  const bool wave_live = row0 < P.nx;
+  i64 q = row0 + col;
+  if (q >= P.nx) q = P.nx - 1;  // clamped rows compute, never store
+  const int cb0 = blockIdx.z * FIN_NB;
+  const int c0 = cb0 * 32;
+
+  T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
+#pragma unroll
+  for (int v = 0; v < KEOPS_NROWVARS; v++) {
+    const T* src = P.arg[keops_row_arg[v]] + q * keops_row_dim[v];
+#pragma unroll
+    for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
+  }
+  T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+#pragma unroll
+  for (int v = 0; v < KEOPS_NPARVARS; v++) {
+    const T* src = P.arg[keops_par_arg[v]];
+#pragma unroll
+    for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
+  }
+
+  fin_f32x16 acc[FIN_NB];
+#pragma unroll
+  for (int b = 0; b < FIN_NB; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[b][r] = 0.f;
+
+  T* dst = P.nslabs > 1 ? P.partial + (i64)blockIdx.y * P.nx * FIN_DV : P.out;
+  bool first = true;
+  // folds the register tiles into the output rows of this wavefront and clears them
+  auto fold = [&]() {
+    const i64 ibase = row0 + 4 * half;
+    T* o = dst + ibase * FIN_DV + c0 + col;
+    asm volatile("" : "+v"(o));
+#pragma unroll
+    for (int b = 0; b < FIN_NB; b++) {
+      const int d = c0 + 32 * b + col;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int ir = 8 * (r >> 2) + (r & 3);
+        if (ibase + ir < P.nx && d < FIN_DV) {
+          T* oo = o + (i64)ir * FIN_DV + 32 * b;
+          *oo = first ? acc[b][r] : *oo + acc[b][r];
+        }
+        acc[b][r] = 0.f;
+      }
+    }
+    first = false;
+  };
+
+  const i64 jbeg = (i64)blockIdx.y * P.slab_len;   // multiple of FIN_TJ
+  const i64 jend = keops_min(P.ny, jbeg + P.slab_len);
+
+  // a staged tile: per term FIN_VS columns of FIN_TJ rows, 16-byte chunks
+  constexpr int CPC = FIN_TJ / 8;                         // chunks per column
+  constexpr int NCH = 3 * FIN_VS * CPC;                   // chunks per tile
+  constexpr int NPF = (NCH + FIN_BLOCK - 1) / FIN_BLOCK;
+  uint4 pf[NPF];
+  auto prefetch = [&](i64 j0) {
+    const uint4* base = reinterpret_cast<const uint4*>(P.vsplit + (j0 / FIN_TJ) * 3 * FIN_DVP * FIN_TJ);
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * FIN_BLOCK;
+      const int term = e / (FIN_VS * CPC), rest = e - term * (FIN_VS * CPC);
+      const int c = rest / CPC, part = rest - c * CPC;
+      // columns past the padded width of the split copy belong to no block of v
+      pf[u] = (e < NCH && c0 + c < FIN_DVP) ? base[((i64)term * FIN_DVP + c0 + c) * CPC + part] : make_uint4(0u, 0u, 0u, 0u);
+    }
+  };
+  // A operand of a 16-row block: the pair values of output row `col` and the 8 reduced rows jb + 8 half + e, in
+  // three terms.  The reduced-index variables of f are staged one tile ahead of their use.
+  auto stage_y = [&](i64 j0) {
+    T* dsty = ys[(j0 / FIN_TJ) & 1];
+    const int n = (int)keops_min((i64)FIN_TJ, P.ny - j0);
+#pragma unroll
+    for (int v = 0; v < KEOPS_NCOLVARS; v++) {
+      const int dim = keops_col_dim[v];
+      const T* src = P.arg[keops_col_arg[v]] + j0 * dim;
+      for (int e = tid; e < n * dim; e += FIN_BLOCK) {
+        const int row = e / dim, c = e - row * dim;
+        dsty[row * FIN_DY + keops_col_off[v] + c] = src[e];
+      }
+    }
+  };
+  auto operands = [&](i64 jb, fin_bf16x8& oh, fin_bf16x8& om, fin_bf16x8& ol) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const i64 j = jb + 8 * half + e;
+      const T* yrow = ys[(jb / FIN_TJ) & 1] + (int)(j % FIN_TJ) * FIN_DY;
+      T yj[FIN_DY];
+      constexpr int VEC = 4;
+      typedef T vecT __attribute__((ext_vector_type(VEC)));
+#pragma unroll
+      for (int c4 = 0; c4 < KEOPS_DIMY_PAD / VEC; c4++) {
+        const vecT w = *reinterpret_cast<const vecT*>(yrow + c4 * VEC);
+#pragma unroll
+        for (int c = 0; c < VEC; c++) yj[c4 * VEC + c] = w[c];
+      }
+      T fout[1];
+      KeopsFormula::eval(xi, yj, p, fout);
+      const float f = j < jend ? fout[0] : 0.f;  // select, never multiply: rows past the end hold garbage
+      const __bf16 h = (__bf16)f;
+      const float r1 = f - (float)h;
+      const __bf16 m = (__bf16)r1;
+      oh[e] = h;
+      om[e] = m;
+      ol[e] = (__bf16)(r1 - (float)m);
+    }
+  };
+  if (jbeg < jend) {
+    prefetch(jbeg);
+    stage_y(jbeg);
+  }
+  int since_fold = 0;
+  for (i64 j0 = jbeg; j0 < jend; j0 += FIN_TJ) {
+    const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
+    __syncthreads();  // the previous tile has been consumed by every wavefront
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * FIN_BLOCK;
+      if (e < NCH) {
+        const int term = e / (FIN_VS * CPC), rest = e - term * (FIN_VS * CPC);
+        const int c = rest / CPC, part = rest - c * CPC;
+        *reinterpret_cast<uint4*>(vt + ((term * FIN_VS + c) * FIN_TS + part * 8)) = pf[u];
+      }
+    }
+    if (j0 + FIN_TJ < jend) stage_y(j0 + FIN_TJ);
+    __syncthreads();
+    if (j0 + FIN_TJ < jend) prefetch(j0 + FIN_TJ);
+    if (!wave_live) continue;
+
+#pragma unroll
+    for (int kb = 0; kb < FIN_TJ / 16; kb++) {
+      fin_bf16x8 ah, am, al;
+      operands(j0 + 16 * kb, ah, am, al);
+      const __bf16* brow = vt + col * FIN_TS + 16 * kb + 8 * half;
+#pragma unroll
+      for (int b = 0; b < FIN_NB; b++) {
+        const fin_bf16x8 bh = *reinterpret_cast<const fin_bf16x8*>(brow + (0 * FIN_VS + 32 * b) * FIN_TS);
+        const fin_bf16x8 bm = *reinterpret_cast<const fin_bf16x8*>(brow + (1 * FIN_VS + 32 * b) * FIN_TS);
+        const fin_bf16x8 bl = *reinterpret_cast<const fin_bf16x8*>(brow + (2 * FIN_VS + 32 * b) * FIN_TS);
+        // smallest terms first
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am, bm, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am, bh, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bm, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh, acc[b], 0, 0, 0);
+      }
+    }
+#if FIN_BLOCKSUM
+    since_fold += FIN_TJ;
+    if (since_fold >= FIN_PERIOD) {
+      fold();
+      since_fold = 0;
+    }
+#endif
+  }
+  fold();
 }
 #endif
