@@ -37,7 +37,9 @@ MEASURED_TRAFFIC_BYTES = {
     # profiles/keops_knn_filter__knn_d64.md: dominant kernel keops_knn_filter
     "knn_d64": int(2 * (391283 * 2.0 + 43486) * 1024),
     # profiles/keops_chk_final__laplace_d256.md
-    "laplace_d256": int((4292480 * 2.0 + 650811) * 1024),
+    "laplace_d256": int((5070320 * 2.0 + 666150) * 1024),
+    # profiles/keops_chk_softmax__softmax_d64.md
+    "softmax_d64": int((204925 * 2.0 + 33804) * 1024),
     # profiles/keops_fin_main3__gauss_dv256.md
     "gauss_dv256": int((10715900 * 2.0 + 10797000) * 1024),
     # profiles/keops_conv_ranges__sparse_100x10k.md, keops_conv_ranges__lse_b16.md
@@ -58,9 +60,10 @@ WORKLOADS = {
     "lse_b16": ("batched LogSumExp softmin B=16, 50,000 x 50,000, D=3 (benchmark configuration 5a)", 17, "valu"),
     # 2*D flop of the contraction + sqrt, neg, exp + 2*Dv of the weighted accumulation
     "laplace_d256": ("Laplace kernel sum 2e5 x 2e5, D=256, Dv=16 (benchmark configuration 5b)", 547, "mfma"),
-    # softmax-weighted sum of an inner product (attention-like).  Counted: exp + 2*Dv of the weighted sum, which runs
-    # on the float32 matrix cores and dominates; the 2*D*3 bf16 flop of the scores are not counted
-    "softmax_d64": ("SumSoftMaxWeight of <q,k> with 64-dimensional weights, 65536 x 65536, D=64", 130, "mfma32"),
+    # softmax-weighted sum of an inner product (attention-like): 2*D flop of the scores, exp, 2*Dv of the weighted
+    # sum.  Both products run on the bf16 matrix cores with float32-class accuracy (operands in two resp. three
+    # bf16 terms, three resp. six instructions per block); the algorithmic flop are counted once
+    "softmax_d64": ("SumSoftMaxWeight of <q,k> with 64-dimensional weights, 65536 x 65536, D=64", 258, "mfma"),
     # 12 flop of the Gaussian kernel + 2*Dv of the product with the 256-dimensional variable; the product runs on
     # the bf16 matrix cores with every operand in three bf16 terms (six instructions per block, float32 accuracy):
     # the algorithmic flop are counted once

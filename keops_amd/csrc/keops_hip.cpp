@@ -664,6 +664,7 @@ struct ChkHeader {
   int32_t nslabs;
   int32_t pad_;
   int64_t nxs, nys;
+  void* vsplit;
   RangeHeader rt;
 };
 
@@ -698,6 +699,10 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
     nslabs = std::max<int64_t>(1, (ny + slab_len - 1) / slab_len);
   }
   const size_t o_part = take(final && nslabs > 1 ? (size_t)nslabs * nx * m.dimred * 4 : 0);
+  // weighted sums with three-term bfloat16 operands (dense launches): pre-split copy of v, tile by tile
+  const bool split3 = final && !rg && m.meta_int("chk_split3", 0) != 0;
+  const int64_t vcols = m.meta_int("chk_vcols", 0), ntiles = (ny + TJ - 1) / TJ;
+  const size_t o_vsplit = take(split3 ? (size_t)ntiles * 3 * vcols * 40 * 2 : 0);
   if (int rc = m.partial.reserve(off)) return rc;
   char* ws = (char*)m.partial.ptr;
   std::vector<char> buf(sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 8);
@@ -705,6 +710,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   h.nx = nx; h.ny = ny; h.xs = ws + o_xs; h.ys = ws + o_ys; h.xn = ws + o_xn; h.yn = ws + o_yn; h.colsum = ws + o_colsum;
   h.colpart = ws + o_colpart; h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs;
   h.nxs = nxs; h.nys = nys;
+  if (split3) h.vsplit = ws + o_vsplit;
   if (rg) h.rt = rg->header(m.nargs);
   std::memcpy(buf.data(), &h, sizeof(h));
   for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
@@ -721,6 +727,8 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (int rc = launch_raw(m, "keops_chk_prep", (unsigned)((nxs * lpr + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
   sz = with_which(1);
   if (int rc = launch_raw(m, "keops_chk_prep", (unsigned)((nys * lpr + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  if (split3)
+    if (int rc = launch_raw(m, "keops_chk_split", (unsigned)((ntiles * vcols * TJ + 255) / 256), 1, 256, buf.data(), psize, stream)) return rc;
   if (rg && rg->user_ranges)
     if (int rc = launch_raw(m, "keops_chk_fill_neutral", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), psize, stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));

@@ -76,6 +76,7 @@ struct ChkParams {
   int nslabs;
   int pad_;
   i64 nxs, nys;         // rows of the chunked row / column arguments (fewer than nx, ny when a batch dimension is broadcast)
+  __bf16* vsplit;       // CHK_SPLIT3: v as three bfloat16 terms, [tile][term][column][CHK_TS positions]
   KeopsRangeTables rt;  // block-sparse / batch geometry (KEOPS_MC_RANGES)
   const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
 };
@@ -388,6 +389,151 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
 }
 #endif
 
+// ---- weighted sums with every operand in three bfloat16 terms ----------------------------------------
+//
+// Dense launches of the two variants below (CHK_SPLIT3).  x = h + m + l with h = bf16(x), m = bf16(x - h),
+// l = bf16(x - h - m) carries the 24 significant bits of a float32 and w * v ~ hh + (hm + mh) + (hl + lh + mm)
+// drops terms below 2^-24 |w v| only: float32 accuracy from six v_mfma_f32_32x32x16_bf16 (6 x 32 cycles per
+// 32 x 32 x 16 block) where v_mfma_f32_32x32x2_f32 needs 8 x 64.  The pair weights sit in the accumulator layout
+// of the s tile (register v of lane l: reduced row 8 (v/4) + 4 (l/32) + v%4 of output row l % 32); registers
+// 8 kb .. 8 kb + 7 are the A operand of k block kb when the contraction index runs over the reduced rows in the
+// order 16 kb + {0,1,2,3,8,9,10,11} for lanes 0-31 and 16 kb + {4,..,7,12,..,15} for lanes 32-63, so
+// keops_chk_split stores v with its rows in that order: row r of a 32-row tile at position
+// 16 (r/16) + 8 ((r>>2)&1) + 4 ((r>>3)&1) + r%4 of [tile][term][column][CHK_TS], and a lane reads the 8 rows of
+// its B operand with one ds_read_b128 (CHK_TS = 40 elements per column: conflict-free).
+#if defined(CHK_SPLIT3) && CHK_SPLIT3
+#define CHK_V3 1
+#ifndef CHK_PRESPLIT
+#define CHK_PRESPLIT 1
+#endif
+#define CHK_V3_PRESPLIT (CHK_PRESPLIT && !KEOPS_MC_RANGES)  // block-sparse / batched launches split the tile while staging it
+#define CHK_TS 40
+#define CHK_VCOLS (CHK_FNB * 32)
+
+#if CHK_V3_PRESPLIT
+extern "C" __global__ void __launch_bounds__(256) keops_chk_split(const ChkParams P) {
+  const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;   // one (tile, column, row in tile)
+  const i64 ntiles = (P.ny + CHK_TJ - 1) / CHK_TJ;
+  if (e >= ntiles * CHK_VCOLS * CHK_TJ) return;
+  const int r = (int)(e % CHK_TJ);
+  const int c = (int)((e / CHK_TJ) % CHK_VCOLS);
+  const i64 tile = e / ((i64)CHK_TJ * CHK_VCOLS);
+  const i64 j = tile * CHK_TJ + r;
+  const float x = (j < P.ny && c < CHK_FV_DIM) ? P.arg[CHK_FV_ARG][j * CHK_FV_DIM + c] : 0.f;
+  const __bf16 h = (__bf16)x;
+  const float r1 = x - (float)h;
+  const __bf16 m = (__bf16)r1;
+  const __bf16 l = (__bf16)(r1 - (float)m);
+  const int pos = 16 * (r >> 4) + 8 * ((r >> 2) & 1) + 4 * ((r >> 3) & 1) + (r & 3);
+  __bf16* dst = P.vsplit + (tile * 3 * CHK_VCOLS + c) * CHK_TS + pos;
+  dst[0] = h;
+  dst[(i64)CHK_VCOLS * CHK_TS] = m;
+  dst[(i64)2 * CHK_VCOLS * CHK_TS] = l;
+}
+
+// 16-byte chunks of one staged tile and their prefetch registers
+#define CHK_V3_CHUNKS (3 * CHK_VCOLS * CHK_TS / 8)
+#define CHK_V3_NPF ((CHK_V3_CHUNKS + CHK_BLOCK - 1) / CHK_BLOCK)
+
+__device__ __forceinline__ void chk_v3_prefetch(const ChkParams& P, i64 j0, int tid, uint4 (&pf)[CHK_V3_NPF]) {
+  const uint4* base = reinterpret_cast<const uint4*>(P.vsplit + (j0 / CHK_TJ) * 3 * CHK_VCOLS * CHK_TS);
+#pragma unroll
+  for (int u = 0; u < CHK_V3_NPF; u++) {
+    const int e = tid + u * CHK_BLOCK;
+    pf[u] = e < CHK_V3_CHUNKS ? base[e] : make_uint4(0u, 0u, 0u, 0u);
+  }
+}
+
+__device__ __forceinline__ void chk_v3_store(__bf16* bt3, int tid, const uint4 (&pf)[CHK_V3_NPF]) {
+#pragma unroll
+  for (int u = 0; u < CHK_V3_NPF; u++) {
+    const int e = tid + u * CHK_BLOCK;
+    if (e < CHK_V3_CHUNKS) reinterpret_cast<uint4*>(bt3)[e] = pf[u];
+  }
+}
+#endif
+
+// Block-sparse and batched launches (reduced-index ranges start anywhere, no pre-split copy): the tile is split
+// while it is staged.  A task is one column and the 8 reduced rows of one (k block, lane half) group, i.e. 8
+// consecutive positions of the LDS layout: 8 coalesced float32 loads (prefetched one tile ahead), one
+// ds_write_b128 per term.
+#define CHK_V3_TASKS (CHK_VCOLS * 4)
+#define CHK_V3_NT ((CHK_V3_TASKS + CHK_BLOCK - 1) / CHK_BLOCK)
+
+__device__ __forceinline__ void chk_v3_gather(const T* vsrc, i64 jv, int n, int tid, float (&pfv)[CHK_V3_NT * 8]) {
+#pragma unroll
+  for (int u = 0; u < CHK_V3_NT; u++) {
+    const int t = tid + u * CHK_BLOCK;
+    const int c = t % CHK_VCOLS, g = t / CHK_VCOLS;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const int r = 16 * (g >> 1) + 4 * (g & 1) + (e < 4 ? e : e + 4);
+      pfv[u * 8 + e] = (t < CHK_V3_TASKS && r < n && c < CHK_FV_DIM) ? vsrc[(jv + r) * CHK_FV_DIM + c] : 0.f;
+    }
+  }
+}
+
+__device__ __forceinline__ void chk_v3_scatter(__bf16* bt3, int tid, const float (&pfv)[CHK_V3_NT * 8]) {
+#pragma unroll
+  for (int u = 0; u < CHK_V3_NT; u++) {
+    const int t = tid + u * CHK_BLOCK;
+    if (t < CHK_V3_TASKS) {
+      const int c = t % CHK_VCOLS, g = t / CHK_VCOLS;
+      chk_bf16x8 h8, m8, l8;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float x = pfv[u * 8 + e];
+        const __bf16 h = (__bf16)x;
+        const float r1 = x - (float)h;
+        const __bf16 m = (__bf16)r1;
+        h8[e] = h;
+        m8[e] = m;
+        l8[e] = (__bf16)(r1 - (float)m);
+      }
+      __bf16* dst = bt3 + c * CHK_TS + 8 * g;
+      *reinterpret_cast<chk_bf16x8*>(dst) = h8;
+      *reinterpret_cast<chk_bf16x8*>(dst + CHK_VCOLS * CHK_TS) = m8;
+      *reinterpret_cast<chk_bf16x8*>(dst + 2 * CHK_VCOLS * CHK_TS) = l8;
+    }
+  }
+}
+
+// acc[b] += W (32 output rows x 32 reduced rows, the 16 weights w of this lane) * v (staged terms bt3)
+__device__ __forceinline__ void chk_v3_product(const float (&w)[16], const __bf16* bt3, int col, int half,
+                                               chk_f32x16 (&acc)[CHK_FNB]) {
+#pragma unroll
+  for (int kb = 0; kb < 2; kb++) {
+    chk_bf16x8 ah, am, al;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float x = w[8 * kb + e];
+      const __bf16 h = (__bf16)x;
+      const float r1 = x - (float)h;
+      const __bf16 m = (__bf16)r1;
+      ah[e] = h;
+      am[e] = m;
+      al[e] = (__bf16)(r1 - (float)m);
+    }
+    const __bf16* brow = bt3 + col * CHK_TS + 16 * kb + 8 * half;
+#pragma unroll
+    for (int b = 0; b < CHK_FNB; b++) {
+      const chk_bf16x8 bh = *reinterpret_cast<const chk_bf16x8*>(brow + (0 * CHK_VCOLS + 32 * b) * CHK_TS);
+      const chk_bf16x8 bm = *reinterpret_cast<const chk_bf16x8*>(brow + (1 * CHK_VCOLS + 32 * b) * CHK_TS);
+      const chk_bf16x8 bl = *reinterpret_cast<const chk_bf16x8*>(brow + (2 * CHK_VCOLS + 32 * b) * CHK_TS);
+      // smallest terms first
+      acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am, bm, acc[b], 0, 0, 0);
+      acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh, acc[b], 0, 0, 0);
+      acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl, acc[b], 0, 0, 0);
+      acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am, bh, acc[b], 0, 0, 0);
+      acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bm, acc[b], 0, 0, 0);
+      acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh, acc[b], 0, 0, 0);
+    }
+  }
+}
+#else
+#define CHK_V3 0
+#endif
+
 // ---- variant with the final product on the matrix cores -------------------------------------------
 
 #if defined(CHK_FINAL) && CHK_FINAL
@@ -397,7 +543,11 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
   __shared__ __attribute__((aligned(16))) unsigned char as[CHK_TJ * CHK_STRIDE];  // A tile (hi|lo)
   __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
   __shared__ __attribute__((aligned(16))) T yo_s[CHK_TJ * CHK_DY];                // other column variables of g
+#if CHK_V3
+  __shared__ __attribute__((aligned(16))) __bf16 bt3[3 * CHK_VCOLS * CHK_TS];       // v tile in three terms
+#else
   __shared__ __attribute__((aligned(16))) T bt[CHK_TJ * CHK_FVS];                 // v tile
+#endif
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
@@ -463,9 +613,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
 
   constexpr int CH = CHK_ROWBYTES / 16;
   constexpr int NPF = (CHK_TJ * CH + CHK_BLOCK - 1) / CHK_BLOCK;
-  constexpr int NPV = (CHK_TJ * CHK_FVS + CHK_BLOCK - 1) / CHK_BLOCK;
   uint4 pf[NPF];
+#if CHK_V3 && CHK_V3_PRESPLIT
+  uint4 pf3[CHK_V3_NPF];
+#elif CHK_V3
+  float pfv[CHK_V3_NT * 8];
+#else
+  constexpr int NPV = (CHK_TJ * CHK_FVS + CHK_BLOCK - 1) / CHK_BLOCK;
   T pfv[NPV];
+#endif
   float pfn = 0.f;
   auto prefetch = [&](i64 j0, i64 jend) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
@@ -478,12 +634,18 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
     }
     if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[jy + tid] : 0.f;
     // v tile, zero past the last row / column (the matrix product must not see stale values)
+#if CHK_V3 && CHK_V3_PRESPLIT
+    chk_v3_prefetch(P, j0, tid, pf3);
+#elif CHK_V3
+    chk_v3_gather(vsrc, jv, n, tid, pfv);
+#else
 #pragma unroll
     for (int u = 0; u < NPV; u++) {
       const int e = tid + u * CHK_BLOCK;
       const int row = e / CHK_FVS, c = e - row * CHK_FVS;
       pfv[u] = (row < n && c < CHK_FV_DIM) ? vsrc[(jv + row) * CHK_FV_DIM + c] : (T)0;
     }
+#endif
   };
   int since_fold = 0;
   // folds the reduced rows [jbeg, jend) into the register tiles
@@ -510,11 +672,17 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
         yo_s[row * CHK_DY + keops_col_off[v] + c] = src[e];
       }
     }
+#if CHK_V3 && CHK_V3_PRESPLIT
+    chk_v3_store(bt3, tid, pf3);
+#elif CHK_V3
+    chk_v3_scatter(bt3, tid, pfv);
+#else
 #pragma unroll
     for (int u = 0; u < NPV; u++) {
       const int e = tid + u * CHK_BLOCK;
       if (e < CHK_TJ * CHK_FVS) bt[e] = pfv[u];
     }
+#endif
     __syncthreads();
     if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ, jend);
     if (!wave_live) continue;
@@ -539,6 +707,9 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
     }
+#if CHK_V3
+    float gw[16];
+#endif
 #pragma unroll
     for (int v = 0; v < 16; v++) {
       const int r = 8 * (v >> 2) + 4 * half + (v & 3);
@@ -556,10 +727,17 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
       T fout[1];
       KeopsFormula::eval(xi, yj, p, sv, fout);
       const float g = r < n ? fout[0] : 0.f;  // select, never multiply: rows past the end hold garbage
+#if CHK_V3
+      gw[v] = g;
+#else
 #pragma unroll
       for (int b = 0; b < CHK_FNB; b++)
         acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(g, bt[r * CHK_FVS + 32 * b + col], acc[b], 0, 0, 0);
+#endif
     }
+#if CHK_V3
+    chk_v3_product(gw, bt3, col, half, acc);
+#endif
 #if CHK_BLOCKSUM
     since_fold += CHK_TJ;
     if (since_fold >= CHK_PERIOD) {
@@ -605,7 +783,11 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
   __shared__ __attribute__((aligned(16))) unsigned char as[CHK_TJ * CHK_STRIDE];
   __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
   __shared__ __attribute__((aligned(16))) T yo_s[CHK_TJ * CHK_DY];
+#if CHK_V3
+  __shared__ __attribute__((aligned(16))) __bf16 bt3[3 * CHK_VCOLS * CHK_TS];       // v tile in three terms
+#else
   __shared__ __attribute__((aligned(16))) T bt[CHK_TJ * CHK_SVS];
+#endif
   __shared__ __attribute__((aligned(16))) float al_s[CHK_WAVES][32];  // rescaling factors of a wavefront's rows
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -653,9 +835,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
 
   constexpr int CH = CHK_ROWBYTES / 16;
   constexpr int NPF = (CHK_TJ * CH + CHK_BLOCK - 1) / CHK_BLOCK;
-  constexpr int NPV = (CHK_TJ * CHK_SVS + CHK_BLOCK - 1) / CHK_BLOCK;
   uint4 pf[NPF];
+#if CHK_V3 && CHK_V3_PRESPLIT
+  uint4 pf3[CHK_V3_NPF];
+#elif CHK_V3
+  float pfv[CHK_V3_NT * 8];
+#else
+  constexpr int NPV = (CHK_TJ * CHK_SVS + CHK_BLOCK - 1) / CHK_BLOCK;
   T pfv[NPV];
+#endif
   float pfn = 0.f;
   auto prefetch = [&](i64 j0, i64 jend) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
@@ -667,12 +855,18 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
       pf[u] = (e < n * CH) ? src[e] : make_uint4(0u, 0u, 0u, 0u);
     }
     if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[jy + tid] : 0.f;
+#if CHK_V3 && CHK_V3_PRESPLIT
+    chk_v3_prefetch(P, j0, tid, pf3);
+#elif CHK_V3
+    chk_v3_gather(vsrc, jv, n, tid, pfv);
+#else
 #pragma unroll
     for (int u = 0; u < NPV; u++) {
       const int e = tid + u * CHK_BLOCK;
       const int row = e / CHK_SVS, c = e - row * CHK_SVS;
       pfv[u] = (row < n && c < CHK_FV_DIM) ? vsrc[(jv + row) * CHK_FV_DIM + c] : (T)0;
     }
+#endif
   };
   // folds the reduced rows [jbeg, jend) into the running maxima, sums and register tiles
   auto sweep = [&](i64 jbeg, i64 jend) {
@@ -698,11 +892,17 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
         yo_s[row * CHK_DY + keops_col_off[v] + c] = src[e];
       }
     }
+#if CHK_V3 && CHK_V3_PRESPLIT
+    chk_v3_store(bt3, tid, pf3);
+#elif CHK_V3
+    chk_v3_scatter(bt3, tid, pfv);
+#else
 #pragma unroll
     for (int u = 0; u < NPV; u++) {
       const int e = tid + u * CHK_BLOCK;
       if (e < CHK_TJ * CHK_SVS) bt[e] = pfv[u];
     }
+#endif
     __syncthreads();
     if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ, jend);
     if (!wave_live) continue;
@@ -766,15 +966,25 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
       __threadfence_block();
       m_run = m_new;
     }
+#if CHK_V3
+    float pw[16];
+#endif
 #pragma unroll
     for (int v = 0; v < 16; v++) {
       const int r = 8 * (v >> 2) + 4 * half + (v & 3);
       const float pv = keops_red_exp(s[v] - m_run);
       l_run += pv;
+#if CHK_V3
+      pw[v] = pv;
+#else
 #pragma unroll
       for (int b = 0; b < CHK_FNB; b++)
         acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(pv, bt[r * CHK_SVS + 32 * b + col], acc[b], 0, 0, 0);
+#endif
     }
+#if CHK_V3
+    chk_v3_product(pw, bt3, col, half, acc);
+#endif
   }
   };
 #if KEOPS_MC_RANGES

@@ -276,13 +276,15 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
     dpad = -(-D // (16 * nc)) * 16 * nc
     dimy_pad = 0 if layout.dimy == 0 else -(-layout.dimy // 4) * 4
     waves = config.chunk_waves
+    split3 = int(wvar is not None and config.final_split3)
     # LDS of the kernel: staged tile (hi|lo rows), the other reduced-index variables, and either the v tile
     # (final-product variant) or the accumulator exchange of the two lanes of a row
     def lds_bytes(w):
         tile = 32 * (dpad * 4 + 16)
         fixed = 128 + 32 * max(1, dimy_pad) * 4
         if wvar is not None:
-            return tile + fixed + 32 * (-(-wvar.dim // 32)) * 32 * 4 + 128 * w
+            vtile = 3 * (-(-wvar.dim // 32)) * 32 * 40 * 2 if split3 else 32 * (-(-wvar.dim // 32)) * 32 * 4
+            return tile + fixed + vtile + 128 * w
         # the accumulator exchange reuses the memory of the staged tile
         merge = (32 * w // nc) * (2 * nc - 1) * red.dimred * (8 if dtypeacc == "double" else 4)
         return max(tile, merge) + fixed + (w * 16 * 64 * 4 if nc > 1 else 0)
@@ -298,7 +300,8 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
                 sizeof_acc=8 if dtypeacc == "double" else 4, nrowvars=len(layout.rowvars) + 1,
                 ncolvars=len(layout.colvars) + ncol_extra, nparvars=len(layout.parvars), chk_d=D, chk_dpad=dpad,
                 chk_mode=mode, chk_qb=32 * waves // nc, chk_final=int(final is not None), chk_softmax=int(softmax is not None),
-                chk_xarg=xvar.ind, chk_yarg=yvar.ind, ranges=int(irregular), nops=L.count_ops(outs))
+                chk_xarg=xvar.ind, chk_yarg=yvar.ind, ranges=int(irregular), chk_split3=int(split3 and config.chunk_presplit),
+                chk_vcols=0 if wvar is None else -(-wvar.dim // 32) * 32, nops=L.count_ops(outs))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
            f"typedef float T;\ntypedef {dtypeacc} TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
            '#include "keops_common.h"']
@@ -316,6 +319,8 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
     elif softmax is not None:
         defs.update(KEOPS_DIMFOUT=full_post.dim, CHK_SOFTMAX=1, CHK_SM_ONE=softmax[2], CHK_FV_ARG=softmax[1].ind,
                     CHK_FV_DIM=softmax[1].dim, CHK_FNB=-(-softmax[1].dim // 32))
+    defs["CHK_SPLIT3"] = split3
+    defs["CHK_PRESPLIT"] = int(config.chunk_presplit)
     src += [f"#define {k} {v}" for k, v in defs.items()]
     for name, vals in (("row_arg", ra), ("row_dim", rd), ("row_off", ro), ("col_arg", ca), ("col_dim", cd),
                        ("col_off", co), ("par_arg", pa), ("par_dim", pd), ("par_off", po)):
