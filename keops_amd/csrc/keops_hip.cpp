@@ -781,7 +781,8 @@ int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   h.nx = nx; h.ny = ny; h.out = out; h.slab_len = len; h.nslabs = (int32_t)nslabs;
   if (rg) h.rt = rg->header(m.nargs);
   // split-operand variant (dense launches): v rewritten once as three bfloat16 terms, tile by tile
-  const bool split3 = !rg && m.meta_int("fin_split3", 0) != 0;
+  const bool split3_kernel = m.meta_int("fin_split3", 0) != 0;  // three-term kernel; dense launches pre-split v
+  const bool split3 = !rg && split3_kernel;
   const int64_t DVP = (DV + 31) / 32 * 32, ntiles = (ny + TJ - 1) / TJ;
   const size_t part_bytes = nslabs > 1 ? align_up((size_t)nslabs * nx * DV * 4, 256) : 0;
   const size_t split_bytes = split3 ? (size_t)ntiles * 3 * DVP * TJ * 2 : 0;
@@ -798,7 +799,7 @@ int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (split3)
     if (int rc = launch_raw(m, "keops_fin_split", (unsigned)((ntiles * DVP * TJ + 255) / 256), 1, 256, buf.data(), buf.size(), stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
-  if (int rc = launch_raw3(m, split3 ? "keops_fin_main3" : "keops_fin_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)NZ, (unsigned)m.block, buf.data(), buf.size(), stream)) return rc;
+  if (int rc = launch_raw3(m, split3_kernel ? "keops_fin_main3" : "keops_fin_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)NZ, (unsigned)m.block, buf.data(), buf.size(), stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
   if (nslabs > 1) {
     const int64_t gb = (nx * DV + 255) / 256;

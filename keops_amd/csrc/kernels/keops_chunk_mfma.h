@@ -251,7 +251,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
     if (CHK_MODE == 0) pfn = (tid < n) ? P.yn[jy + tid] : 0.f;
   };
   // folds the reduced rows [jbeg, jend) into the accumulators
-  auto sweep = [&](i64 jbeg, i64 jend) {
+  i64 jbeg, jend;
+#if KEOPS_MC_RANGES
+  G.rewind(P.rt);
+  while (G.next(P.rt, jbeg, jend)) {
+#else
+  jbeg = 0;
+  jend = P.ny;
+  {
+#endif
   if (jbeg < jend) prefetch(jbeg, jend);
   for (i64 j0 = jbeg; j0 < jend; j0 += CHK_TJ) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
@@ -365,12 +373,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
     acc.merge(tmp);
 #endif
   }
-  };
-#if KEOPS_MC_RANGES
-  G.for_each_range(P.rt, sweep);
-#else
-  sweep(0, P.ny);
-#endif
+  }
 
   // the 2 * CHK_NC lanes of an output row merge their accumulators in a fixed order
   __syncthreads();
@@ -649,7 +652,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
   };
   int since_fold = 0;
   // folds the reduced rows [jbeg, jend) into the register tiles
-  auto sweep = [&](i64 jbeg, i64 jend) {
+  i64 jbeg, jend;
+#if KEOPS_MC_RANGES
+  G.rewind(P.rt);
+  while (G.next(P.rt, jbeg, jend)) {
+#else
+  jbeg = (i64)blockIdx.y * P.slab_len;
+  jend = keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len);
+  {
+#endif
   if (jbeg < jend) prefetch(jbeg, jend);
   for (i64 j0 = jbeg; j0 < jend; j0 += CHK_TJ) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
@@ -746,12 +757,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
     }
 #endif
   }
-  };
-#if KEOPS_MC_RANGES
-  G.for_each_range(P.rt, sweep);
-#else
-  sweep((i64)blockIdx.y * P.slab_len, keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len));
-#endif
+  }
   fold();
 }
 
@@ -869,7 +875,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
 #endif
   };
   // folds the reduced rows [jbeg, jend) into the running maxima, sums and register tiles
-  auto sweep = [&](i64 jbeg, i64 jend) {
+  i64 jbeg, jend;
+#if KEOPS_MC_RANGES
+  G.rewind(P.rt);
+  while (G.next(P.rt, jbeg, jend)) {
+#else
+  jbeg = (i64)blockIdx.y * P.slab_len;
+  jend = keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len);
+  {
+#endif
   if (jbeg < jend) prefetch(jbeg, jend);
   for (i64 j0 = jbeg; j0 < jend; j0 += CHK_TJ) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
@@ -986,12 +1000,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
     chk_v3_product(pw, bt3, col, half, acc);
 #endif
   }
-  };
-#if KEOPS_MC_RANGES
-  G.for_each_range(P.rt, sweep);
-#else
-  sweep((i64)blockIdx.y * P.slab_len, keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len));
-#endif
+  }
 
   // results of this slab: [m, (l,) O_0 .. O_{dv-1}] per output row
   l_run += __shfl_xor(l_run, 32);

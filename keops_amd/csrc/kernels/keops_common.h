@@ -126,21 +126,33 @@ struct KeopsTileGeom {
     return 0;
 #endif
   }
-  // calls sweep(jbeg, jend) for every maximal run of contiguous reduced-index ranges of this workgroup;
-  // with batch dimensions the single range of the batch is swept as [0, length) (batch-relative indices,
-  // the offsets move the arguments)
-  template <typename F> __device__ __forceinline__ void for_each_range(const KeopsRangeTables& R, F&& sweep) const {
+  // Cursor over the maximal runs of contiguous reduced-index ranges of this workgroup: next() yields [jbeg, jend)
+  // until the ranges are exhausted.  With batch dimensions the single range of the batch is swept as [0, length)
+  // (batch-relative indices, the offsets move the arguments).  A dense module yields its one interval once.
+  // (A loop around the sweep instead of a callback: the sweep must be inlined, or the register tiles it updates
+  // would live in scratch memory.)
+  i64 cur_index, cur_start;
+  __device__ __forceinline__ void rewind(const KeopsRangeTables& R) {
+    cur_index = slice_first;
 #if KEOPS_MC_RANGES
-    if (slice_first >= slice_end) return;
-    i64 start_y = R.ranges_y[2 * slice_first];
-    for (i64 index = slice_first; index < slice_end; index++) {
-      if (index + 1 >= slice_end || R.ranges_y[2 * index + 2] != R.ranges_y[2 * index + 1]) {
-        const i64 end_y = R.ranges_y[2 * index + 1];
-        if (offs) sweep((i64)0, end_y - start_y);
-        else sweep(start_y, end_y);
-        if (index + 1 < slice_end) start_y = R.ranges_y[2 * index + 2];
+    cur_start = slice_first < slice_end ? R.ranges_y[2 * slice_first] : 0;
+#else
+    cur_start = 0;
+#endif
+  }
+  __device__ __forceinline__ bool next(const KeopsRangeTables& R, i64& jbeg, i64& jend) {
+#if KEOPS_MC_RANGES
+    for (; cur_index < slice_end; cur_index++) {
+      if (cur_index + 1 >= slice_end || R.ranges_y[2 * cur_index + 2] != R.ranges_y[2 * cur_index + 1]) {
+        const i64 end_y = R.ranges_y[2 * cur_index + 1];
+        jbeg = offs ? (i64)0 : cur_start;
+        jend = offs ? end_y - cur_start : end_y;
+        if (cur_index + 1 < slice_end) cur_start = R.ranges_y[2 * cur_index + 2];
+        cur_index++;
+        return true;
       }
     }
 #endif
+    return false;
   }
 };

@@ -124,7 +124,15 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
   };
   int since_fold = 0;
   // folds the reduced rows [jbeg, jend) into the register tiles
-  auto sweep = [&](i64 jbeg, i64 jend) {
+  i64 jbeg, jend;
+#if KEOPS_MC_RANGES
+  G.rewind(P.rt);
+  while (G.next(P.rt, jbeg, jend)) {
+#else
+  jbeg = (i64)blockIdx.y * P.slab_len;
+  jend = keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len);
+  {
+#endif
   if (jbeg < jend) prefetch(jbeg, jend);
   for (i64 j0 = jbeg; j0 < jend; j0 += FIN_TJ) {
     const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
@@ -186,12 +194,7 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
     }
 #endif
   }
-  };
-#if KEOPS_MC_RANGES
-  G.for_each_range(P.rt, sweep);
-#else
-  sweep((i64)blockIdx.y * P.slab_len, keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len));
-#endif
+  }
   fold();
 }
 
@@ -218,19 +221,22 @@ extern "C" __global__ void __launch_bounds__(256) keops_fin_fill_neutral(const F
 // x = h + m + l with h = bf16(x), m = bf16(x - h), l = bf16(x - h - m) carries the 24 significant bits of a
 // float32, and f * v ~ hh + (hm + mh) + (hl + lh + mm) drops terms below 2^-24 |f v| only: float32 accuracy
 // from six v_mfma_f32_32x32x16_bf16 (6 x 32 cycles per 32 x 32 x 16 block) where the float32 instruction
-// v_mfma_f32_32x32x2_f32 needs 8 x 64 cycles.  Dense launches only (the pre-split copy of v is laid out tile by
-// tile from reduced row 0):
-//   * keops_fin_split writes v once as [tile][term][column][row in tile] bfloat16, zero past the last row and
-//     column, so that a workgroup stages a tile with straight 16-byte copies and a lane reads the 8 consecutive
-//     reduced rows of its B operand (column l % 32, rows 8 (l / 32) ..) with one ds_read_b128 (rows padded to
-//     FIN_TS elements: conflict-free);
+// v_mfma_f32_32x32x2_f32 needs 8 x 64 cycles.
+//   * Dense launches: keops_fin_split writes v once as [tile][term][column][row in tile] bfloat16, zero past the
+//     last row and column, so that a workgroup stages a tile with straight 16-byte copies.  Block-sparse and
+//     batched launches (ranges start anywhere) split the float32 tile while staging it, one column and 8 rows per
+//     task.  Either way a lane reads the 8 consecutive reduced rows of its B operand (column l % 32, rows
+//     8 (l / 32) ..) with one ds_read_b128 (columns padded to FIN_TS elements: conflict-free);
 //   * lane l evaluates f for output row l % 32 and the 8 reduced rows 8 (l / 32) .. of a 16-row block -- the A
 //     operand layout -- and splits the 8 values in registers.
-#if defined(FIN_SPLIT3) && FIN_SPLIT3 && !KEOPS_MC_RANGES
+// keops_fin_main above (float32 instruction) remains for modules built without FIN_SPLIT3.
+#if defined(FIN_SPLIT3) && FIN_SPLIT3
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 fin_bf16x8;
 #define FIN_TS (FIN_TJ + 8)            // bfloat16 elements per staged column (padded)
 #define FIN_DVP (FIN_NBTOT * 32)       // columns of the split copy
+#define FIN_PRESPLIT (!KEOPS_MC_RANGES)  // block-sparse / batched launches split the tile while staging it
 
+#if FIN_PRESPLIT
 extern "C" __global__ void __launch_bounds__(256) keops_fin_split(const FinParams P) {
   const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;   // one (tile, column, row in tile)
   const i64 ntiles = (P.ny + FIN_TJ - 1) / FIN_TJ;
@@ -249,31 +255,34 @@ extern "C" __global__ void __launch_bounds__(256) keops_fin_split(const FinParam
   dst[(i64)FIN_DVP * FIN_TJ] = m;
   dst[(i64)2 * FIN_DVP * FIN_TJ] = l;
 }
+#endif
 
 extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const FinParams P) {
   __shared__ __attribute__((aligned(16))) __bf16 vt[3 * FIN_VS * FIN_TS];  // [term][column][row], this workgroup's column blocks
-  __shared__ __attribute__((aligned(16))) T ys[2][FIN_TJ * FIN_DY];         // reduced-index variables of f: this tile and the next
+  __shared__ __attribute__((aligned(16))) T ys[FIN_TJ * FIN_DY];            // reduced-index variables of f
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
-  const i64 row0 = (i64)blockIdx.x * FIN_QB + wave * 32;  // first output row of this wavefront
-  const bool wave_live = row0 < P.nx;
+  KeopsTileGeom G;
+  G.init(P.rt, P.nx, FIN_QB);
+  const i64 row0 = G.row_first + wave * 32;  // first output row of this wavefront
+  const bool wave_live = row0 < G.row_end;   // a wavefront without rows only helps staging the tiles
   i64 q = row0 + col;
-  if (q >= P.nx) q = P.nx - 1;  // clamped rows compute, never store
+  if (q >= G.row_end) q = G.row_end - 1;     // clamped rows compute, never store
   const int cb0 = blockIdx.z * FIN_NB;
   const int c0 = cb0 * 32;
 
   T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NROWVARS; v++) {
-    const T* src = P.arg[keops_row_arg[v]] + q * keops_row_dim[v];
+    const T* src = P.arg[keops_row_arg[v]] + G.row(keops_row_arg[v], q) * keops_row_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
   }
   T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NPARVARS; v++) {
-    const T* src = P.arg[keops_par_arg[v]];
+    const T* src = P.arg[keops_par_arg[v]] + G.par(keops_par_arg[v]) * keops_par_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
   }
@@ -297,7 +306,7 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int ir = 8 * (r >> 2) + (r & 3);
-        if (ibase + ir < P.nx && d < FIN_DV) {
+        if (ibase + ir < G.row_end && d < FIN_DV) {
           T* oo = o + (i64)ir * FIN_DV + 32 * b;
           *oo = first ? acc[b][r] : *oo + acc[b][r];
         }
@@ -307,15 +316,13 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
     first = false;
   };
 
-  const i64 jbeg = (i64)blockIdx.y * P.slab_len;   // multiple of FIN_TJ
-  const i64 jend = keops_min(P.ny, jbeg + P.slab_len);
-
-  // a staged tile: per term FIN_VS columns of FIN_TJ rows, 16-byte chunks
+#if FIN_PRESPLIT
+  // a staged tile: per term FIN_VS columns of FIN_TJ rows, 16-byte chunks of the pre-split copy
   constexpr int CPC = FIN_TJ / 8;                         // chunks per column
   constexpr int NCH = 3 * FIN_VS * CPC;                   // chunks per tile
   constexpr int NPF = (NCH + FIN_BLOCK - 1) / FIN_BLOCK;
   uint4 pf[NPF];
-  auto prefetch = [&](i64 j0) {
+  auto prefetch = [&](i64 j0, i64 jend) {
     const uint4* base = reinterpret_cast<const uint4*>(P.vsplit + (j0 / FIN_TJ) * 3 * FIN_DVP * FIN_TJ);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
@@ -326,54 +333,7 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
       pf[u] = (e < NCH && c0 + c < FIN_DVP) ? base[((i64)term * FIN_DVP + c0 + c) * CPC + part] : make_uint4(0u, 0u, 0u, 0u);
     }
   };
-  // A operand of a 16-row block: the pair values of output row `col` and the 8 reduced rows jb + 8 half + e, in
-  // three terms.  The reduced-index variables of f are staged one tile ahead of their use.
-  auto stage_y = [&](i64 j0) {
-    T* dsty = ys[(j0 / FIN_TJ) & 1];
-    const int n = (int)keops_min((i64)FIN_TJ, P.ny - j0);
-#pragma unroll
-    for (int v = 0; v < KEOPS_NCOLVARS; v++) {
-      const int dim = keops_col_dim[v];
-      const T* src = P.arg[keops_col_arg[v]] + j0 * dim;
-      for (int e = tid; e < n * dim; e += FIN_BLOCK) {
-        const int row = e / dim, c = e - row * dim;
-        dsty[row * FIN_DY + keops_col_off[v] + c] = src[e];
-      }
-    }
-  };
-  auto operands = [&](i64 jb, fin_bf16x8& oh, fin_bf16x8& om, fin_bf16x8& ol) {
-#pragma unroll
-    for (int e = 0; e < 8; e++) {
-      const i64 j = jb + 8 * half + e;
-      const T* yrow = ys[(jb / FIN_TJ) & 1] + (int)(j % FIN_TJ) * FIN_DY;
-      T yj[FIN_DY];
-      constexpr int VEC = 4;
-      typedef T vecT __attribute__((ext_vector_type(VEC)));
-#pragma unroll
-      for (int c4 = 0; c4 < KEOPS_DIMY_PAD / VEC; c4++) {
-        const vecT w = *reinterpret_cast<const vecT*>(yrow + c4 * VEC);
-#pragma unroll
-        for (int c = 0; c < VEC; c++) yj[c4 * VEC + c] = w[c];
-      }
-      T fout[1];
-      KeopsFormula::eval(xi, yj, p, fout);
-      const float f = j < jend ? fout[0] : 0.f;  // select, never multiply: rows past the end hold garbage
-      const __bf16 h = (__bf16)f;
-      const float r1 = f - (float)h;
-      const __bf16 m = (__bf16)r1;
-      oh[e] = h;
-      om[e] = m;
-      ol[e] = (__bf16)(r1 - (float)m);
-    }
-  };
-  if (jbeg < jend) {
-    prefetch(jbeg);
-    stage_y(jbeg);
-  }
-  int since_fold = 0;
-  for (i64 j0 = jbeg; j0 < jend; j0 += FIN_TJ) {
-    const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
-    __syncthreads();  // the previous tile has been consumed by every wavefront
+  auto store_tile = [&]() {
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * FIN_BLOCK;
@@ -383,15 +343,109 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
         *reinterpret_cast<uint4*>(vt + ((term * FIN_VS + c) * FIN_TS + part * 8)) = pf[u];
       }
     }
-    if (j0 + FIN_TJ < jend) stage_y(j0 + FIN_TJ);
+  };
+#else
+  // no pre-split copy (reduced-index ranges start anywhere): a task is one column and 8 consecutive reduced rows,
+  // 8 coalesced float32 loads prefetched one tile ahead, split and written with one ds_write_b128 per term
+  constexpr int NTASK = FIN_VS * (FIN_TJ / 8);
+  constexpr int NT = (NTASK + FIN_BLOCK - 1) / FIN_BLOCK;
+  float pf[NT * 8];
+  const T* vsrc = P.arg[FIN_VARG];
+  auto prefetch = [&](i64 j0, i64 jend) {
+    const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
+    const i64 jv = G.col(FIN_VARG, j0);
+#pragma unroll
+    for (int u = 0; u < NT; u++) {
+      const int t = tid + u * FIN_BLOCK;
+      const int c = t % FIN_VS, g = t / FIN_VS;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const int r = 8 * g + e;
+        pf[u * 8 + e] = (t < NTASK && r < n && c0 + c < FIN_DV) ? vsrc[(jv + r) * FIN_DV + c0 + c] : 0.f;
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int u = 0; u < NT; u++) {
+      const int t = tid + u * FIN_BLOCK;
+      if (t < NTASK) {
+        const int c = t % FIN_VS, g = t / FIN_VS;
+        fin_bf16x8 h8, m8, l8;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const float x = pf[u * 8 + e];
+          const __bf16 h = (__bf16)x;
+          const float r1 = x - (float)h;
+          const __bf16 m = (__bf16)r1;
+          h8[e] = h;
+          m8[e] = m;
+          l8[e] = (__bf16)(r1 - (float)m);
+        }
+        __bf16* d = vt + c * FIN_TS + 8 * g;
+        *reinterpret_cast<fin_bf16x8*>(d) = h8;
+        *reinterpret_cast<fin_bf16x8*>(d + FIN_VS * FIN_TS) = m8;
+        *reinterpret_cast<fin_bf16x8*>(d + 2 * FIN_VS * FIN_TS) = l8;
+      }
+    }
+  };
+#endif
+
+  int since_fold = 0;
+  // folds the reduced rows [jbeg, jend) into the register tiles
+  i64 jbeg, jend;
+#if KEOPS_MC_RANGES
+  G.rewind(P.rt);
+  while (G.next(P.rt, jbeg, jend)) {
+#else
+  jbeg = (i64)blockIdx.y * P.slab_len;
+  jend = keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len);
+  {
+#endif
+  if (jbeg < jend) prefetch(jbeg, jend);
+  for (i64 j0 = jbeg; j0 < jend; j0 += FIN_TJ) {
+    const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
+    __syncthreads();  // the previous tile has been consumed by every wavefront
+    store_tile();
+#pragma unroll
+    for (int v = 0; v < KEOPS_NCOLVARS; v++) {
+      const int dim = keops_col_dim[v];
+      const T* src = P.arg[keops_col_arg[v]] + G.col(keops_col_arg[v], j0) * dim;
+      for (int e = tid; e < n * dim; e += FIN_BLOCK) {
+        const int row = e / dim, c = e - row * dim;
+        ys[row * FIN_DY + keops_col_off[v] + c] = src[e];
+      }
+    }
     __syncthreads();
-    if (j0 + FIN_TJ < jend) prefetch(j0 + FIN_TJ);
+    if (j0 + FIN_TJ < jend) prefetch(j0 + FIN_TJ, jend);
     if (!wave_live) continue;
 
 #pragma unroll
     for (int kb = 0; kb < FIN_TJ / 16; kb++) {
+      // A operand: the pair values of output row `col` and the 8 reduced rows 16 kb + 8 half + e, in three terms
       fin_bf16x8 ah, am, al;
-      operands(j0 + 16 * kb, ah, am, al);
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const int jr = 16 * kb + 8 * half + e;
+        T yj[FIN_DY];
+        constexpr int VEC = 4;
+        typedef T vecT __attribute__((ext_vector_type(VEC)));
+#pragma unroll
+        for (int c4 = 0; c4 < KEOPS_DIMY_PAD / VEC; c4++) {
+          const vecT w = *reinterpret_cast<const vecT*>(ys + jr * FIN_DY + c4 * VEC);
+#pragma unroll
+          for (int c = 0; c < VEC; c++) yj[c4 * VEC + c] = w[c];
+        }
+        T fout[1];
+        KeopsFormula::eval(xi, yj, p, fout);
+        const float f = jr < n ? fout[0] : 0.f;  // select, never multiply: rows past the end hold garbage
+        const __bf16 h = (__bf16)f;
+        const float r1 = f - (float)h;
+        const __bf16 m = (__bf16)r1;
+        ah[e] = h;
+        am[e] = m;
+        al[e] = (__bf16)(r1 - (float)m);
+      }
       const __bf16* brow = vt + col * FIN_TS + 16 * kb + 8 * half;
 #pragma unroll
       for (int b = 0; b < FIN_NB; b++) {
@@ -414,6 +468,7 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
       since_fold = 0;
     }
 #endif
+  }
   }
   fold();
 }

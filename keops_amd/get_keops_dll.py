@@ -384,7 +384,7 @@ def generate_final_plugin(red, match, sum_scheme, nargs, irregular=False):
     meta = dict(scheme="final", block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
                 sizeof_acc=4, nrowvars=len(layout.rowvars), ncolvars=len(layout.colvars) + (0 if vvar in layout.colvars else 1),
                 nparvars=len(layout.parvars), fin_dv=vvar.dim, fin_nb=nb, fin_nz=nz, fin_qb=32 * waves, ranges=int(irregular),
-                fin_split3=int(config.final_split3 and not irregular and tj % 16 == 0),
+                fin_split3=int(config.final_split3 and tj % 16 == 0),
                 nops=L.count_ops(outs))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
            "typedef float T;\ntypedef float TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
@@ -392,7 +392,7 @@ def generate_final_plugin(red, match, sum_scheme, nargs, irregular=False):
     defs = dict(
         KEOPS_NARGS=nargs, FIN_DV=vvar.dim, FIN_VARG=vvar.ind, FIN_NB=nb, FIN_WAVES=waves, FIN_TJ=tj,
         FIN_PERIOD=config.final_period, FIN_BLOCKSUM=int(sum_scheme == "block_sum"),
-        FIN_SPLIT3=int(config.final_split3 and not irregular and tj % 16 == 0),
+        FIN_SPLIT3=int(config.final_split3 and tj % 16 == 0),
         KEOPS_DIMX=layout.dimx, KEOPS_DIMY=layout.dimy, KEOPS_DIMY_PAD=dimy_pad, KEOPS_DIMP=layout.dimp,
         KEOPS_NROWVARS=len(layout.rowvars), KEOPS_NCOLVARS=len(layout.colvars), KEOPS_NPARVARS=len(layout.parvars),
     )
