@@ -73,6 +73,14 @@ __device__ __forceinline__ i64 keops_min(i64 a, i64 b) { return a < b ? a : b; }
 #define KEOPS_MC_RANGES 0
 #endif
 
+// A value that is the same in every lane of a wavefront (loaded from a table at a wave-uniform address): kept in
+// scalar registers
+__device__ __forceinline__ i64 keops_uniform(i64 v) {
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)(v & 0xffffffffll));
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)((unsigned long long)v >> 32));
+  return (i64)(((unsigned long long)hi << 32) | lo);
+}
+
 struct KeopsRangeTables {
   const i64* lookup;    // [nblocks][3] = (range id, first row, end row)
   const i64* slices_x;  // end slice of every row range
@@ -91,11 +99,11 @@ struct KeopsTileGeom {
   __device__ __forceinline__ void init(const KeopsRangeTables& R, i64 nx, int rows_per_block) {
 #if KEOPS_MC_RANGES
     const i64 bid = blockIdx.x;
-    const i64 range_id = R.lookup[3 * bid];
-    row_first = R.lookup[3 * bid + 1];
-    row_end = R.lookup[3 * bid + 2];
-    slice_first = range_id < 1 ? 0 : R.slices_x[range_id - 1];
-    slice_end = R.slices_x[range_id];
+    const i64 range_id = keops_uniform(R.lookup[3 * bid]);
+    row_first = keops_uniform(R.lookup[3 * bid + 1]);
+    row_end = keops_uniform(R.lookup[3 * bid + 2]);
+    slice_first = range_id < 1 ? 0 : keops_uniform(R.slices_x[range_id - 1]);
+    slice_end = keops_uniform(R.slices_x[range_id]);
     offs = R.nbatchdims > 0 ? R.offsets + (i64)R.nargs * bid : nullptr;
 #else
     row_first = (i64)blockIdx.x * rows_per_block;
@@ -107,21 +115,21 @@ struct KeopsTileGeom {
   // row of argument `arg` that holds global output row q / reduced row j / the parameter
   __device__ __forceinline__ i64 row(int arg, i64 q) const {
 #if KEOPS_MC_RANGES
-    return offs ? offs[arg] + (q - row_first) : q;
+    return offs ? keops_uniform(offs[arg]) + (q - row_first) : q;
 #else
     return q;
 #endif
   }
   __device__ __forceinline__ i64 col(int arg, i64 j) const {
 #if KEOPS_MC_RANGES
-    return offs ? offs[arg] + j : j;
+    return offs ? keops_uniform(offs[arg]) + j : j;
 #else
     return j;
 #endif
   }
   __device__ __forceinline__ i64 par(int arg) const {
 #if KEOPS_MC_RANGES
-    return offs ? offs[arg] : 0;
+    return offs ? keops_uniform(offs[arg]) : 0;
 #else
     return 0;
 #endif
@@ -135,7 +143,7 @@ struct KeopsTileGeom {
   __device__ __forceinline__ void rewind(const KeopsRangeTables& R) {
     cur_index = slice_first;
 #if KEOPS_MC_RANGES
-    cur_start = slice_first < slice_end ? R.ranges_y[2 * slice_first] : 0;
+    cur_start = slice_first < slice_end ? keops_uniform(R.ranges_y[2 * slice_first]) : 0;
 #else
     cur_start = 0;
 #endif
@@ -144,10 +152,10 @@ struct KeopsTileGeom {
 #if KEOPS_MC_RANGES
     for (; cur_index < slice_end; cur_index++) {
       if (cur_index + 1 >= slice_end || R.ranges_y[2 * cur_index + 2] != R.ranges_y[2 * cur_index + 1]) {
-        const i64 end_y = R.ranges_y[2 * cur_index + 1];
+        const i64 end_y = keops_uniform(R.ranges_y[2 * cur_index + 1]);
         jbeg = offs ? (i64)0 : cur_start;
         jend = offs ? end_y - cur_start : end_y;
-        if (cur_index + 1 < slice_end) cur_start = R.ranges_y[2 * cur_index + 2];
+        if (cur_index + 1 < slice_end) cur_start = keops_uniform(R.ranges_y[2 * cur_index + 2]);
         cur_index++;
         return true;
       }
