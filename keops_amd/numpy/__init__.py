@@ -105,3 +105,51 @@ def generic_argmin(formula, output, *aliases, **kwargs):
 def generic_argkmin(formula, output, *aliases, **kwargs):
     al, axis, dim = _split(output, aliases)
     return Genred(formula, al, reduction_op="ArgKMin", axis=axis, opt_arg=dim, **kwargs)
+
+
+# ---- LazyTensor on NumPy arrays (pykeops/pykeops/numpy/lazytensor/LazyTensor.py) ---------------------------
+
+from ..torch.lazytensor import LazyTensor as _TorchLazyTensor  # noqa: E402
+
+
+def _np_out(res):
+    if isinstance(res, torch.Tensor):
+        return res.cpu().numpy()
+    if isinstance(res, tuple):
+        return tuple(_np_out(r) for r in res)
+    return res
+
+
+class LazyTensor(_TorchLazyTensor):
+    """The symbolic LazyTensor of the torch layer on NumPy arrays: arrays are moved to the current device when the
+    LazyTensor is built and reductions return NumPy arrays."""
+
+    def __init__(self, x=None, axis=None):
+        if isinstance(x, np.ndarray):
+            if x.dtype not in (np.float32, np.float64):
+                raise ValueError("[KeOps] only float32 and float64 arrays are supported")
+            x = torch.from_numpy(np.ascontiguousarray(x)).to(_device(-1))
+        elif isinstance(x, (np.floating, np.integer)):
+            x = x.item()
+        super().__init__(x, axis)
+
+    def reduction(self, *args, call=True, **kwargs):
+        if isinstance(kwargs.get("ranges"), tuple) and isinstance(kwargs["ranges"][0], np.ndarray):
+            kwargs["ranges"] = _ranges_to_device(kwargs["ranges"], _device(-1))
+        res = super().reduction(*args, call=call, **kwargs)
+        if callable(res) and not isinstance(res, torch.Tensor):
+            return lambda *a, **k: _np_out(res(*[torch.from_numpy(np.ascontiguousarray(t)).to(_device(-1))
+                                                 if isinstance(t, np.ndarray) else t for t in a], **k))
+        return _np_out(res)
+
+
+def Vi(x_or_ind, dim=None):
+    return LazyTensor(x_or_ind, axis=0) if dim is None else LazyTensor((x_or_ind, dim, 0))
+
+
+def Vj(x_or_ind, dim=None):
+    return LazyTensor(x_or_ind, axis=1) if dim is None else LazyTensor((x_or_ind, dim, 1))
+
+
+def Pm(x_or_ind, dim=None):
+    return LazyTensor(x_or_ind, axis=2) if dim is None else LazyTensor((x_or_ind, dim, 2))

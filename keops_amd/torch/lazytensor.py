@@ -142,7 +142,7 @@ class LazyTensor:
         return self._dtype
 
     def _like(self, formula, *others):
-        res = LazyTensor()
+        res = type(self)()
         res.formula = formula
         srcs = (self,) + others
         for s in srcs:
@@ -164,7 +164,7 @@ class LazyTensor:
         return res
 
     def _lift(self, other):
-        return other if isinstance(other, LazyTensor) else LazyTensor(other)
+        return other if isinstance(other, LazyTensor) else type(self)(other)
 
     def unary(self, fn, *params):
         return self._like(fn(self.formula, *params))
@@ -251,9 +251,9 @@ class LazyTensor:
         if self.ndim != 1:
             raise ValueError("The 'K @ v' syntax is only supported for LazyTensors 'K' whose trailing dimension "
                              f"is equal to 1. Here, K.shape = {self.shape}.")
-        if v.dim() == 1:
-            return (self * LazyTensor(v.view(1, -1, 1))).sum(self.nbatchdims + 1, **kwargs).view(-1)
-        return (self * LazyTensor(v.unsqueeze(-3))).sum(self.nbatchdims + 1, **kwargs)
+        if v.ndim == 1:
+            return (self * type(self)(v.reshape(1, -1, 1))).sum(self.nbatchdims + 1, **kwargs).reshape(-1)
+        return (self * type(self)(v.reshape(v.shape[:-2] + (1,) + v.shape[-2:]))).sum(self.nbatchdims + 1, **kwargs)
 
     def __getitem__(self, key):
         if isinstance(key, int):

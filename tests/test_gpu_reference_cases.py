@@ -214,3 +214,27 @@ def test_softdtw_bspline_and_grad_matrix_on_the_device():
     refm = dense_eval("GradMatrix(Exp(-Square(u-v)),u)", ["u=Vi(0,3)", "v=Vj(1,3)"],
                       [x[:, :3].cpu().numpy(), y[:, :3].cpu().numpy()], M, N).sum(1)
     assert np.allclose(gm.sum(dim=1).cpu().numpy(), refm, rtol=1e-10, atol=1e-12)
+
+
+def test_numpy_lazytensor_and_generic_ops():
+    """The NumPy front end (pykeops.numpy: LazyTensor, Vi / Vj / Pm, generic_argkmin) on host arrays, cf.
+    pykeops/test/test_numpy.py: arrays are staged through the device, results come back as NumPy arrays."""
+    import numpy as np
+
+    from keops_amd.numpy import LazyTensor, Pm, Vi, Vj, generic_argkmin
+
+    rng = np.random.default_rng(0)
+    x, y, b = rng.random((300, 3)), rng.random((500, 3)), rng.standard_normal((500, 2))
+    K = (-((LazyTensor(x[:, None, :]) - LazyTensor(y[None, :, :])) ** 2).sum(-1) / 0.25).exp()
+    a = K @ b
+    ref = np.exp(-((x[:, None, :] - y[None, :, :]) ** 2).sum(-1) / 0.25) @ b
+    assert isinstance(a, np.ndarray) and a.dtype == np.float64 and np.allclose(a, ref, rtol=1e-10)
+    s = (Vi(x) - Vj(y)).sqnorm2()
+    idx = s.argKmin(5, dim=1)
+    refi = np.argsort(((x[:, None, :] - y[None, :, :]) ** 2).sum(-1), axis=1, kind="stable")[:, :5]
+    assert isinstance(idx, np.ndarray) and np.array_equal(idx.astype(np.int64), refi)
+    knn = generic_argkmin("SqDist(x,y)", "a = Vi(5)", "x = Vi(3)", "y = Vj(3)")
+    assert np.array_equal(knn(x, y).astype(np.int64), refi)
+    lse = ((Vi(x) * Vj(y)).sum(-1) * Pm(np.array([2.0]))).logsumexp(dim=1)
+    refl = np.log(np.exp(2.0 * x @ y.T).sum(1))
+    assert np.allclose(lse[:, 0], refl, rtol=1e-10)
