@@ -531,7 +531,10 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   const int64_t a_nr = two_phase ? nsample : nr;
   const int64_t SQB = m.meta_int("knn_sqb", QB), SBLOCK = m.meta_int("knn_sblock", m.block);
   const int64_t a_qblocks = (nq + (two_phase ? SQB : QB) - 1) / (two_phase ? SQB : QB);
-  int64_t a_slabs = pick_slabs(a_qblocks, a_nr, TJ, m.cu_count, 2, tag1D2D == 1 && !two_phase ? 2 : 1, 16);
+  static const int64_t main_per_cu = [] { const char* e = getenv("KEOPS_HIP_KNN_MAIN_PER_CU"); return e ? std::max<int64_t>(1, atoll(e)) : 2; }();
+  static const int64_t main_min_tiles = [] { const char* e = getenv("KEOPS_HIP_KNN_MAIN_MIN_TILES"); return e ? std::max<int64_t>(1, atoll(e)) : 16; }();
+  int64_t a_slabs = pick_slabs(a_qblocks, a_nr, TJ, m.cu_count, two_phase ? 2 : main_per_cu, tag1D2D == 1 && !two_phase ? 2 : 1,
+                               two_phase ? 16 : main_min_tiles);
   int64_t a_len = ((a_nr + a_slabs - 1) / a_slabs + TJ - 1) / TJ * TJ;
   a_slabs = std::max<int64_t>(1, (a_nr + a_len - 1) / a_len);
   // filter pass
@@ -636,7 +639,7 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
     done = *(volatile int*)m.pinned == 0;  // a log overflowed (pathological ties): redo adaptively
   }
   if (!done) {
-    int64_t slabs = pick_slabs((nq + QB - 1) / QB, nr, TJ, m.cu_count, 2, tag1D2D == 1 ? 2 : 1);
+    int64_t slabs = pick_slabs((nq + QB - 1) / QB, nr, TJ, m.cu_count, main_per_cu, tag1D2D == 1 ? 2 : 1, main_min_tiles);
     slabs = std::min<int64_t>(slabs, list_slabs);
     int64_t len = ((nr + slabs - 1) / slabs + TJ - 1) / TJ * TJ;
     slabs = std::max<int64_t>(1, (nr + len - 1) / len);
@@ -1028,9 +1031,36 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
   h.slab_len = cols_total;
 
   if (m.scheme == "knn") {
-    if (use_ranges) return fail(-1, "the matrix-core KNN module does not handle ranges or batch dimensions");
+    if (user_ranges) return fail(-1, "the matrix-core KNN module does not handle block-sparse ranges");
     const int rowarg = m.meta_int("rowarg", 0), colarg = m.meta_int("colarg", 1);
-    if (int rc = launch_knn(m, rows_total, cols_total, args[rowarg], args[colarg], out, tag1D2D, stream)) return rc;
+    if (rowarg < 0 || colarg < 0 || rowarg >= m.nargs || colarg >= m.nargs) return fail(-1, "corrupt knn module metadata");
+    if (nb == 0) {
+      if (int rc = launch_knn(m, rows_total, cols_total, args[rowarg], args[colarg], out, tag1D2D, stream)) return rc;
+    } else {
+      // batch dimensions: one pass of the dense pipeline per batch on the same stream (indices are relative to
+      // the batch, as in GpuReduc1D_ranges.py:151-158); a batch dimension of size 1 is broadcast
+      const int64_t R = tagI == 0 ? S.M : S.N, C = tagI == 0 ? S.N : S.M;
+      const int64_t D = m.meta_int("knn_d", 0);
+      std::vector<int64_t> shp(nb + 1);
+      auto first_row = [&](int arg, int64_t b, int64_t len) {
+        const int64_t* r = S.row(arg + 1);
+        for (int k = 0; k < nb; k++) shp[k] = r[k];
+        shp[nb] = len;
+        return broadcast_index(b * len, nb, S.shapes.data(), shp.data());
+      };
+      const bool timing = m.timing;
+      if (timing) HIP_TRY(hipEventRecord(m.ev0, stream));
+      m.timing = false;
+      int rc = 0;
+      for (int64_t b = 0; b < S.nbatches && rc == 0; b++) {
+        const char* xq = (const char*)args[rowarg] + first_row(rowarg, b, R) * D * m.sizeof_t;
+        const char* yr = (const char*)args[colarg] + first_row(colarg, b, C) * D * m.sizeof_t;
+        rc = launch_knn(m, R, C, xq, yr, (char*)out + b * R * dimout * m.sizeof_t, tag1D2D, stream);
+      }
+      m.timing = timing;
+      if (rc) return rc;
+      if (timing) HIP_TRY(hipEventRecord(m.ev1, stream));
+    }
   } else if (m.scheme == "final" || m.scheme == "chunk") {
     const bool built_for_ranges = m.meta_int("ranges", 0) != 0;
     if (use_ranges != built_for_ranges)

@@ -139,13 +139,15 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
     return "\n".join(src) + "\n", meta
 
 
-def match_knn_sqdist(red, dtype, map_reduce_id):
+def match_knn_sqdist(red, dtype, map_reduce_id, batch_loop=0, pairs=0):
     """(row variable, column variable) when ``red`` is a K-min family reduction of SqDist between an
     output-indexed and a reduced-index variable of dimension config.knn_min_dim..256 in float32, on the dense
-    scheme; None otherwise.  Such reductions run on the matrix-core filter + exact re-rank kernels."""
+    scheme or (``batch_loop``) on batch dimensions served one batch at a time; None otherwise.  Such reductions
+    run on the matrix-core filter + exact re-rank kernels.  ``pairs``: when not 0, the call holds less than
+    2**pairs pairs; small problems stay on the general-purpose kernel, whose fixed cost is lower."""
     from .formulas import ops as O
 
-    if red.kind != KIND_KMIN or dtype != "float" or "_ranges" in map_reduce_id or red.K > 64:
+    if red.kind != KIND_KMIN or dtype != "float" or ("_ranges" in map_reduce_id and not batch_loop) or red.K > 64:
         return None
     f = red.formula
     if f.name != "Sum" or f.children[0].name != "Square" or f.children[0].children[0].name != "Subtract":
@@ -154,6 +156,12 @@ def match_knn_sqdist(red, dtype, map_reduce_id):
     if not (isinstance(a, O.Var) and isinstance(b, O.Var)) or a.dim != b.dim or not config.knn_min_dim <= a.dim <= 256:
         return None
     if {a.cat, b.cat} != {0, 1}:
+        return None
+    if pairs and (1 << (int(pairs) - 1)) * max(a.dim, 16) < config.knn_min_work:
+        # the pre-pass, the warm-up of the adaptive lists and the merge cost about 0.3 ms whatever the size
+        return None
+    if "_ranges" in map_reduce_id and (1 << (int(batch_loop) - 1)) * max(a.dim, 8) < config.knn_batch_min_work:
+        # one pass per batch costs about 0.3 ms of launches: below this the batched general-purpose kernel wins
         return None
     return (a, b) if a.cat == red.tagI else (b, a)
 
@@ -413,10 +421,14 @@ def generate_final_plugin(red, match, sum_scheme, nargs, irregular=False):
 def get_keops_dll(
     map_reduce_id, red_formula_string, enable_chunks, enable_finalchunks, mul_var_highdim, aliases, nargs, dtype,
     dtypeacc, sum_scheme_string, tagHostDevice, tagCPUGPU, tag1D2D, use_half, use_fast_math, device_id, nx=None,
+    batch_loop=0, pairs=0,
 ):
     """Same arguments and same 19-tuple as the reference's get_keops_dll (get_keops_dll.py:78-159),
     plus ``nx``: the number of output rows of the call being prepared, used to pick the number of
-    rows per lane.  ``dtype`` / ``dtypeacc`` are C type names ("float" | "double")."""
+    rows per lane, and ``batch_loop``: when not 0, the "_ranges" of the scheme id stand for a few batches
+    of less than 2**batch_loop pairs each without block-sparse ranges, which a dense module may serve one batch
+    at a time; ``pairs``: when not 0, the call (each batch of it) holds less than 2**pairs pairs.  ``dtype`` / ``dtypeacc`` are C
+    type names ("float" | "double")."""
     if use_half or dtype not in ("float", "double"):
         raise ValueError("[KeOps] only float32 and float64 data are supported by the HIP backend")
     if "Gpu" not in map_reduce_id:
@@ -429,7 +441,8 @@ def get_keops_dll(
         # only the bucket matters for the cache key
         rows_hint = nx if nx < 64 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
-           use_fast_math, _rows_bucket(rows_hint), bool(enable_chunks), bool(enable_finalchunks), binder.templates_digest())
+           use_fast_math, _rows_bucket(rows_hint), bool(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs),
+           binder.templates_digest())
     with _lock:
         hit = _cache.get(key)
     if hit is not None:
@@ -441,7 +454,7 @@ def get_keops_dll(
         target, tag, src_file = "", "zero", ""
     else:
         irregular = "_ranges" in map_reduce_id
-        knn = match_knn_sqdist(red, dtype, map_reduce_id) if enable_chunks else None
+        knn = match_knn_sqdist(red, dtype, map_reduce_id, batch_loop, pairs) if enable_chunks else None
         chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
         fin = None
         if enable_finalchunks and knn is None and chk is None:

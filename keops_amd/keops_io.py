@@ -22,7 +22,7 @@ class LoadKeOps_hip:
     empty_ranges = tuple([_NULL_RANGE.ctypes.data] * 7)
 
     def __init__(self, tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula, aliases, nargs,
-                 dtype, lang, optional_flags, nx=None):
+                 dtype, lang, optional_flags, nx=None, batch_loop=0, pairs=0):
         if lang not in ("torch", "pytorch"):
             raise ValueError("[KeOps] the HIP backend binds torch tensors only")
         if tagCPUGPU != 1 or tagHostDevice != 1:
@@ -53,7 +53,7 @@ class LoadKeOps_hip:
          dimsy, dimsp) = get_keops_dll(
             map_reduce_id, formula, p.enable_chunks, -1, p.mult_var_highdim, p.aliases, nargs, p.c_dtype,
             p.c_dtype_acc, p.sum_scheme, tagHostDevice, tagCPUGPU, tag1D2D, False, optional_flags["use_fast_math"],
-            device_id_request, nx=nx,
+            device_id_request, nx=nx, batch_loop=batch_loop, pairs=pairs,
         )
         # the engine reports (output-indexed, reduced) variable lists; the ABI takes (i, j) lists
         if p.tagI == 1:
@@ -112,20 +112,28 @@ _loaders = {}
 
 
 def load_keops_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula, aliases, nargs, dtype,
-                   lang, optional_flags, nx=None):
+                   lang, optional_flags, nx=None, ny=None, batch=None):
     """Cached constructor (the reference keeps one LoadKeOps object per parameter set as well,
     pykeops/pykeops/common/keops_io/LoadKeOps.py:23-31): parsing the formula and resolving the
-    module happen once, later calls only launch."""
+    module happen once, later calls only launch.  ``nx`` / ``ny``: output and reduced rows of the call (of each
+    batch); ``batch``: (number of batches, M, N) of a call with batch dimensions and no block-sparse ranges: a few
+    large batches may be served one at a time by a dense module."""
     from .get_keops_dll import _rows_bucket
     from . import config
 
     rows_hint = nx if (nx is not None and nx < 64 * 256 * config.block_size) else None
+    # log2 bucket of the pairs per batch when there are few batches: the engine weighs it against the formula
+    batch_loop = int(batch[1] * batch[2]).bit_length() if (batch and batch[0] <= config.knn_batch_max) else 0
+    # log2 bucket of the pairs of the call (of each batch), 0: unknown or beyond every threshold of the engine
+    pairs = int(nx * ny).bit_length() if (nx is not None and ny is not None) else 0
+    if pairs > 40:
+        pairs = 0
     key = (tagCPUGPU, tag1D2D, tagHostDevice, bool(use_ranges), device_id_request, formula, tuple(aliases), nargs,
-           dtype, lang, tuple(sorted(optional_flags.items())), _rows_bucket(rows_hint))
+           dtype, lang, tuple(sorted(optional_flags.items())), _rows_bucket(rows_hint), batch_loop, pairs)
     obj = _loaders.get(key)
     if obj is None:
         obj = _loaders[key] = LoadKeOps_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula,
-                                            aliases, nargs, dtype, lang, optional_flags, nx=nx)
+                                            aliases, nargs, dtype, lang, optional_flags, nx=nx, batch_loop=batch_loop, pairs=pairs)
     return obj
 
 

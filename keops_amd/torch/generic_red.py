@@ -79,9 +79,15 @@ class GenredAutograd_base:
                 host_out, params.out = params.out, None
             tagHostDevice, device_args, staged = 1, dev, True
         nout = params.nx if params.axis == 1 else params.ny
+        batch = None
+        if nbatchdims > 0 and params.ranges is None:
+            nbatches = 1
+            for d in range(nbatchdims):
+                nbatches *= max(a.shape[d] if a.dim() == nbatchdims + 2 else 1 for a in args)
+            batch = (nbatches, params.nx, params.ny)
         myconv = keops_binder["hip"](
             tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id, params.formula, params.aliases, len(args),
-            params.dtype, "torch", params.optional_flags, nx=nout,
+            params.dtype, "torch", params.optional_flags, nx=nout, ny=params.nx + params.ny - nout, batch=batch,
         ).import_module()
         if not all(a.is_contiguous() for a in args):
             warnings.warn(

@@ -10,6 +10,20 @@ from oracle.cpu_oracle import cpu_reduc
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _matrix_core_scheme_at_every_size(monkeypatch):
+    """Small problems normally stay on the general-purpose kernel: these tests are about the other one."""
+    import keops_amd.get_keops_dll as engine
+    from keops_amd import config, keops_io
+
+    monkeypatch.setattr(config, "knn_min_work", 0)
+    engine._cache.clear()
+    keops_io._loaders.clear()
+    yield
+    engine._cache.clear()
+    keops_io._loaders.clear()
+
+
 def _knn(D, K, op="KMin_ArgKMin", axis=1):
     from keops_amd.torch import Genred
 
@@ -19,7 +33,7 @@ def _knn(D, K, op="KMin_ArgKMin", axis=1):
 def _uses_mfma_module():
     from keops_amd import keops_io
 
-    return any(m.meta("scheme") == "knn" for m in keops_io._modules.values())
+    return any(ld.module is not None and ld.module.meta("scheme") == "knn" for ld in keops_io._loaders.values())
 
 
 @pytest.mark.parametrize("M,N,D,K", [(1000, 20000, 64, 10), (777, 5001, 40, 3), (300, 3000, 128, 1), (5000, 9999, 32, 16),
@@ -150,3 +164,58 @@ def test_knn_two_phase_log_overflow_falls_back():
     assert np.array_equal(idx.cpu().numpy().reshape(M, K), np.tile(np.arange(K), (M, 1)))
     ref = cpu_reduc("sqdist", [x, y[:K]], M, K, 1, reduction="KMin", K=K, scheme="direct_sum")
     assert np.array_equal(vals.cpu().numpy().reshape(M, K), ref)
+
+
+def test_batched_knn_one_dense_pass_per_batch(monkeypatch):
+    """A few large batches (here: the size limits lowered) run the matrix-core pipeline once per batch, with
+    a broadcast batch dimension on the queries; indices are relative to the batch (GpuReduc1D_ranges.py:151-158)
+    and must equal a stable argsort of the float32 distances computed in the reference's operation order."""
+    from keops_amd import config, keops_io
+    from keops_amd.torch import LazyTensor
+
+    import keops_amd.get_keops_dll as engine
+
+    monkeypatch.setattr(config, "knn_batch_min_work", 1)
+    engine._cache.clear()
+    keops_io._loaders.clear()
+    B, M, N, D, K = 3, 700, 1500, 8, 5
+    gen = torch.Generator().manual_seed(12)
+    x = torch.rand(1, M, D, generator=gen)
+    y = torch.rand(B, N, D, generator=gen)
+    xd, yd = x.cuda(), y.cuda()
+    D_ij = ((LazyTensor(xd[:, :, None, :]) - LazyTensor(yd[:, None, :, :])) ** 2).sum(-1)
+    idx = D_ij.argKmin(K, dim=2).cpu()
+    used = [ld for key, ld in keops_io._loaders.items() if key[3]]
+    assert used and all(ld.module.meta("scheme") == "knn" for ld in used)
+    assert idx.shape == (B, M, K)
+    for b in range(B):
+        d = np.zeros((M, N), np.float32)
+        for k in range(D):
+            d += (x[0, :, k, None].numpy() - y[b, None, :, k].numpy()) ** 2
+        ref = np.argsort(d, axis=1, kind="stable")[:, :K]
+        assert np.array_equal(idx[b].numpy(), ref), b
+    # values and indices together, reduction over the other axis
+    vals, idj = D_ij.Kmin_argKmin(K, dim=1)
+    assert vals.shape == (B, N, K) and idj.shape == (B, N, K)
+    for b in range(B):
+        d = np.zeros((N, M), np.float32)
+        for k in range(D):
+            d += (x[0, None, :, k].numpy() - y[b, :, None, k].numpy()) ** 2
+        ref = np.argsort(d, axis=1, kind="stable")[:, :K]
+        assert np.array_equal(idj[b].cpu().numpy(), ref), b
+        assert np.array_equal(vals[b].cpu().numpy(), np.take_along_axis(d, ref, 1)), b
+
+
+def test_small_problem_stays_on_the_general_purpose_kernel(monkeypatch):
+    """Below config.knn_min_work the fixed cost of the matrix-core pipeline does not pay: same results from the
+    general-purpose kernel."""
+    from keops_amd import config, keops_io
+
+    monkeypatch.setattr(config, "knn_min_work", 1 << 31)
+    x, y = np.random.default_rng(3).random((2, 900, 64), dtype=np.float32)
+    idx = _knn(64, 10, "ArgKMin")(*to_dev(x, y)).cpu().numpy()
+    assert not _uses_mfma_module() and len(keops_io._loaders) == 1
+    d = np.zeros((900, 900), np.float32)
+    for k in range(64):
+        d += (x[:, None, k] - y[None, :, k]) ** 2
+    assert np.array_equal(idx, np.argsort(d, axis=1, kind="stable")[:, :10])
