@@ -193,11 +193,19 @@ struct DeviceBuffer {
   size_t bytes = 0;
   int reserve(size_t n) {
     if (n <= bytes) return 0;
-    if (ptr) (void)hipFree(ptr);
+    // (while a stream records into a HIP graph both calls are refused: a launch has to run once, with the same
+    // shapes, before it is captured)
+    if (ptr) {
+      hipError_t e = hipFree(ptr);
+      if (e != hipSuccess) return fail((int)e, std::string("hipFree of workspace failed: ") + hipGetErrorString(e));
+    }
     ptr = nullptr;
     bytes = 0;
     hipError_t e = hipMalloc(&ptr, n);
-    if (e != hipSuccess) return fail((int)e, std::string("hipMalloc of workspace failed: ") + hipGetErrorString(e));
+    if (e != hipSuccess) {
+      ptr = nullptr;
+      return fail((int)e, std::string("hipMalloc of workspace failed: ") + hipGetErrorString(e));
+    }
     bytes = n;
     return 0;
   }
@@ -275,6 +283,16 @@ struct RangeLaunch {
   }
 };
 
+// true while `stream` records into a HIP graph: launches that wait for the device cannot take part
+bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st != hipStreamCaptureStatusNone;
+}
+
 int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ranges, int64_t* const* ranges,
                          int64_t rows_total, int64_t rows_per_block, bool by_arg, const std::vector<int>& rowvars,
                          const std::vector<int>& colvars, const std::vector<int>& vP, hipStream_t stream, RangeTables& rt) {
@@ -293,6 +311,9 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
     slices_dev = ranges[sel + 1];
     ry_dev = ranges[sel + 2];
     rx_host.resize((size_t)2 * nranges);
+    if (stream_is_capturing(stream))
+      return fail(-1, "block-sparse ranges are read back from the device at every call: such a launch cannot be "
+                      "captured in a HIP graph");
     // same synchronous read-back as the reference (keops_nvrtc.cpp:195-197)
     if (nranges) HIP_TRY(hipMemcpyAsync(rx_host.data(), rx_dev, sizeof(int64_t) * 2 * nranges, hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipStreamSynchronize(stream));
@@ -524,7 +545,8 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   if (nr > 2147483647LL) return fail(-1, "too many reference rows for 32-bit indices");
   // sampling step of the threshold estimate: every 16th reference for large sets, a sample of >= ~4096 rows otherwise
   const int64_t SAMPLE = std::max<int64_t>(2, std::min<int64_t>(m.meta_int("knn_sample", 16), nr / knn_min_sample()));
-  const bool two_phase = nr >= knn_two_phase_min_refs() && nr / SAMPLE >= 8 * K && nq >= 1024;
+  // the two-phase schedule reads a flag back from the device: not while the stream records into a HIP graph
+  const bool two_phase = nr >= knn_two_phase_min_refs() && nr / SAMPLE >= 8 * K && nq >= 1024 && !stream_is_capturing(stream);
   const int64_t nsample = two_phase ? (nr + SAMPLE - 1) / SAMPLE : 0;
 
   // adaptive pass: over the sample (two-phase) or over everything

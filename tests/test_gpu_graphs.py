@@ -1,0 +1,103 @@
+"""HIP graph capture of launches (torch.cuda.graph): after one eager call with the same shapes, which sizes the
+workspaces, a launch records kernels and copies only, so the replayed graph must reproduce the eager result bit for
+bit on new input values.  Launches that have to wait for the device adapt (the KNN scheme takes its adaptive
+schedule) or refuse with a clear error (block-sparse ranges)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _replays_like_eager(fn, inputs, replays=3):
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            fn(*inputs)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = fn(*inputs)
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    for _ in range(replays):
+        for t in inputs:
+            if t.numel() > 1:
+                t.copy_(torch.randn(t.shape, device="cuda", generator=gen) * t.std())
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        ref = fn(*inputs)           # eager work between the replays
+        torch.cuda.synchronize()
+        if not torch.equal(got, ref):
+            return False
+    return True
+
+
+def _scheme_of_last_module():
+    from keops_amd import keops_io
+
+    return list(keops_io._loaders.values())[-1].module.meta("scheme")
+
+
+def test_dense_schemes_under_graph_capture():
+    from keops_amd.torch import Genred
+
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    r = lambda *s: torch.randn(*s, device="cuda", generator=gen)
+    x, y, b, g = r(5000, 3), r(7000, 3), r(7000, 2), torch.tensor([0.5], device="cuda")
+    conv = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)", "g=Pm(1)"], reduction_op="Sum", axis=1)
+    assert _replays_like_eager(conv, [x, y, b, g])
+    assert _replays_like_eager(conv, [r(300, 3), y, b, g])          # few rows: column slabs + merge kernel
+    lse = Genred("-g*SqDist(x,y)", ["x=Vi(3)", "y=Vj(3)", "g=Pm(1)"], reduction_op="LogSumExp", axis=1)
+    assert _replays_like_eager(lse, [x, y, g])
+    lap = Genred("Exp(-Norm2(x-y))*b", ["x=Vi(128)", "y=Vj(128)", "b=Vj(8)"], reduction_op="Sum", axis=1)
+    assert _replays_like_eager(lap, [r(3000, 128) / 3, r(4000, 128) / 3, r(4000, 8)])
+    assert _scheme_of_last_module() == "chunk"
+    fin = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(200)", "g=Pm(1)"], reduction_op="Sum", axis=1)
+    assert _replays_like_eager(fin, [x, y, r(7000, 200), g])
+    assert _scheme_of_last_module() == "final"
+
+
+def test_batched_reduction_under_graph_capture():
+    from keops_amd.torch import LazyTensor
+
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    xb, yb, bb = (torch.randn(*s, device="cuda", generator=gen) for s in ((4, 2000, 3), (4, 3000, 3), (4, 3000, 1)))
+
+    def batched(xb, yb, bb):
+        d = ((LazyTensor(xb[:, :, None, :]) - LazyTensor(yb[:, None, :, :])) ** 2).sum(-1)
+        return ((-d).exp() * LazyTensor(bb[:, None, :, :])).sum(2)
+
+    assert _replays_like_eager(batched, [xb, yb, bb])
+
+
+def test_knn_scheme_takes_its_adaptive_schedule_under_capture():
+    """20000 x 40000 references would run the sampled two-phase schedule, which reads a flag back from the device;
+    under capture the launch uses the adaptive one: same neighbours, no wait."""
+    from keops_amd.torch import Genred
+
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    x, y = torch.rand(20000, 16, device="cuda", generator=gen), torch.rand(40000, 16, device="cuda", generator=gen)
+    knn = Genred("SqDist(x,y)", ["x=Vi(16)", "y=Vj(16)"], reduction_op="ArgKMin", axis=1, opt_arg=8)
+    assert _replays_like_eager(knn, [x, y], replays=2)
+    assert _scheme_of_last_module() == "knn"
+
+
+def test_block_sparse_ranges_refuse_capture_with_a_clear_error():
+    from keops_amd.torch import Genred
+
+    x, y, b = (torch.randn(n, d, device="cuda") for n, d in ((1000, 3), (1200, 3), (1200, 1)))
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device="cuda")
+    ranges = (i64([[0, 500], [500, 1000]]), i64([1, 2]), i64([[0, 600], [600, 1200]]),
+              i64([[0, 600], [600, 1200]]), i64([1, 2]), i64([[0, 500], [500, 1000]]))
+    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(1)"], reduction_op="Sum", axis=1)
+    ref = conv(x, y, b, ranges=ranges)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="cannot be captured"):
+        with torch.cuda.graph(graph):
+            conv(x, y, b, ranges=ranges)
+    torch.cuda.synchronize()
+    assert torch.equal(conv(x, y, b, ranges=ranges), ref)             # the stream is usable again
