@@ -43,6 +43,7 @@ final_period = int(os.environ.get("KEOPS_AMD_FINAL_PERIOD", 4096))         # blo
 # matrix-core KNN kernel (csrc/kernels/keops_knn_mfma.h)
 knn_min_dim = int(os.environ.get("KEOPS_AMD_KNN_MIN_DIM", 2))         # smallest vector dimension served by the matrix-core KNN scheme
 knn_tile_j = int(os.environ.get("KEOPS_AMD_KNN_TJ", 128))          # reference rows per LDS tile (<= 256)
+knn_filter_tile_j = int(os.environ.get("KEOPS_AMD_KNN_FTJ", 256))  # reference rows per LDS tile of the fixed-threshold filter
 knn_max_waves = int(os.environ.get("KEOPS_AMD_KNN_WAVES", 8))     # wavefronts per workgroup sharing one staged tile
 knn_filter_waves = int(os.environ.get("KEOPS_AMD_KNN_FWAVES", 16))  # fixed-threshold filter: wavefronts per workgroup
 knn_filter_qsets = int(os.environ.get("KEOPS_AMD_KNN_FQSETS", 2))   # and 32-query operand sets per wavefront

@@ -538,7 +538,7 @@ int64_t knn_two_phase_min_refs() {
 int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr, void* out, int tag1D2D,
                hipStream_t stream) {
   const int64_t D = m.meta_int("knn_d", 0), DP = m.meta_int("knn_dpad", 0), K = m.meta_int("knn_k", 0);
-  const int64_t QB = m.meta_int("knn_qb", 256), TJ = m.tile_j;
+  const int64_t QB = m.meta_int("knn_qb", 256), TJ = m.tile_j, FTJ = m.meta_int("knn_ftj", m.tile_j);
   const int64_t FW = m.meta_int("knn_fwaves", 16), FQW = 32 * m.meta_int("knn_fqsets", 2);
   const int64_t FQB = FW * FQW;
   if (D <= 0 || DP <= 0 || K <= 0) return fail(-1, "corrupt knn module metadata");
@@ -561,12 +561,12 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   a_slabs = std::max<int64_t>(1, (a_nr + a_len - 1) / a_len);
   // filter pass
   const int64_t f_qblocks = (nq + FQB - 1) / FQB;
-  int64_t f_slabs = pick_slabs(f_qblocks, nr, TJ, m.cu_count, 2, 1, 4);
+  int64_t f_slabs = pick_slabs(f_qblocks, nr, FTJ, m.cu_count, 2, 1, 4);
   // one filter workgroup fills a CU and all of them take the same time.  With at least 8 slabs the filter runs
   // in two stages (every 4th slab, then the others, with thresholds refined in between): both grids should
   // be close to whole rounds over the CUs
   {
-    const int64_t cap = std::max<int64_t>(1, nr / (4 * TJ));
+    const int64_t cap = std::max<int64_t>(1, nr / (4 * FTJ));
     int64_t best = f_slabs;
     double best_eff = 0.0;
     for (int64_t n = f_slabs; n <= std::max(f_slabs, std::min<int64_t>(std::max<int64_t>(4 * f_slabs, 24), cap)); n++) {
@@ -580,7 +580,7 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
     }
     f_slabs = best;
   }
-  int64_t f_len = ((nr + f_slabs - 1) / f_slabs + TJ - 1) / TJ * TJ;
+  int64_t f_len = ((nr + f_slabs - 1) / f_slabs + FTJ - 1) / FTJ * FTJ;
   f_slabs = std::max<int64_t>(1, (nr + f_len - 1) / f_len);
   const bool staged = two_phase && f_slabs >= 8;
   const int64_t fa_slabs = staged ? (f_slabs + 3) / 4 : f_slabs, fb_slabs = f_slabs - fa_slabs;

@@ -44,7 +44,7 @@
 //      references.
 //
 // The plug-in defines: T (float), KEOPS_NARGS, KNN_D, KNN_DPAD (D rounded up to 16), KNN_K,
-// KEOPS_RED_KEEP, KEOPS_DIMOUT, KNN_QSETS, KNN_WAVES (wavefronts per workgroup), KNN_TJ, KNN_SPLIT,
+// KEOPS_RED_KEEP, KEOPS_DIMOUT, KNN_QSETS, KNN_WAVES (wavefronts per workgroup), KNN_TJ, KNN_FTJ, KNN_SPLIT,
 // KNN_FWAVES / KNN_FQSETS (filter geometry), KNN_SWAVES / KNN_SQSETS (sampling pass geometry).
 #pragma once
 #include "keops_common.h"
@@ -56,6 +56,10 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float knn_f32x4;
 
 #ifndef KNN_SPLIT
 #define KNN_SPLIT 0
+#endif
+static_assert(KNN_FQSETS <= 2 && KNN_SQSETS <= 2, "one lane per query owns its list in the replay and sampling kernels");
+#ifndef KNN_FTJ
+#define KNN_FTJ KNN_TJ                 // reference rows per staged tile of the fixed-threshold filter
 #endif
 #define KNN_KB (KNN_DPAD / 16)         // 16-wide k blocks
 #define KNN_RW (KNN_DPAD * (1 + KNN_SPLIT))  // bf16 elements per stored row: [hi] or [hi | lo]
@@ -257,7 +261,7 @@ __device__ __forceinline__ void knn_insert(float* lv, int* li, float d, int j) {
 //   LDS (`cand`, counters in `owner`; one LDS atomic per candidate, all 64 in flight together) and every
 //   owner folds its bin into its list.
 #define KNN_BIN 8  // candidates per query bin
-template <int MODE, int WAVES, int QSETS>
+template <int MODE, int WAVES, int QSETS, int TJ = KNN_TJ>
 __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys, float* ykey_s, float (*lv)[KNN_K],
                                           int (*li)[KNN_K], int* owner, int (*qq)[64], int (*qj)[64],
                                           float* cand = nullptr) {
@@ -393,11 +397,11 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
   const i64 jend = keops_min(P.nr, jbeg + P.slab_len);
   // software pipeline: the rows of tile t+1 travel from HBM/L2 to registers while tile t is consumed
   constexpr int CH = KNN_RW / 8;                            // 16-byte chunks per staged row
-  constexpr int NPF = (KNN_TJ * CH + BLOCK - 1) / BLOCK;    // chunks per thread and tile
+  constexpr int NPF = (TJ * CH + BLOCK - 1) / BLOCK;    // chunks per thread and tile
   uint4 pf[NPF];
   float pfkey = inf;
   auto prefetch = [&](i64 j0) {
-    const int n = (int)keops_min((i64)KNN_TJ, jend - j0);
+    const int n = (int)keops_min((i64)TJ, jend - j0);
     const uint4* src = reinterpret_cast<const uint4*>(P.yh + j0 * KNN_RW);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
@@ -406,35 +410,38 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
     }
     pfkey = (tid < n) ? P.ykey[j0 + tid] : inf;
   };
-  static_assert(KNN_TJ <= BLOCK, "one key per thread");
+  static_assert(TJ <= BLOCK, "one key per thread");
+  // this lane's operand row and keys inside a sub-tile of 32 staged rows
+  const unsigned char* const abase = ys + col * KNN_STRIDE + 16 * half;
+  const float* const kbase = ykey_s + 4 * half;
   if (jbeg < jend) prefetch(jbeg);
-  for (i64 j0 = jbeg; j0 < jend; j0 += KNN_TJ) {
-    const int n = (int)keops_min((i64)KNN_TJ, jend - j0);
+  for (i64 j0 = jbeg; j0 < jend; j0 += TJ) {
+    const int n = (int)keops_min((i64)TJ, jend - j0);
     __syncthreads();  // every wavefront is done with the previous tile
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * BLOCK;
-      if (e < KNN_TJ * CH) {
+      if (e < TJ * CH) {
         const int row = e / CH, c = e - row * CH;
         *reinterpret_cast<uint4*>(ys + row * KNN_STRIDE + c * 16) = pf[u];
       }
     }
-    if (tid < KNN_TJ) ykey_s[tid] = pfkey;
+    if (tid < TJ) ykey_s[tid] = pfkey;
     __syncthreads();
-    if (j0 + KNN_TJ < jend) prefetch(j0 + KNN_TJ);
+    if (j0 + TJ < jend) prefetch(j0 + TJ);
     const int nsub = (n + 31) / 32;
     for (int sub = 0; sub < nsub; sub++) {
       // accumulator register v of this lane is reference row 8*(v/4) + 4*half + v%4 of the sub-tile:
       // start from the keys of those rows
       knn_f32x4 kk[4];
 #pragma unroll
-      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const knn_f32x4*>(ykey_s + sub * 32 + 8 * b + 4 * half);
+      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const knn_f32x4*>(kbase + sub * 32 + 8 * b);
       knn_f32x16 acc[QSETS];
 #pragma unroll
       for (int h = 0; h < QSETS; h++)
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[h][v] = kk[v >> 2][v & 3];
-      const unsigned char* arow = ys + (sub * 32 + col) * KNN_STRIDE + 16 * half;
+      const unsigned char* arow = abase + sub * (32 * KNN_STRIDE);
 #pragma unroll
       for (int kb = 0; kb < KNN_KB; kb++) {
         const knn_bf16x8 a = *reinterpret_cast<const knn_bf16x8*>(arow + kb * 32);
@@ -455,10 +462,12 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
 #pragma unroll
       for (int h = 0; h < QSETS; h++) {
         // cheap screen first: the smallest of the lane's 16 values against the threshold (min3 tree)
-        float m = acc[h][0];
+        // (three-operand minima only: a two-operand v_min_f32 of matrix-core results costs two more instructions
+        // that quiet its inputs)
+        float m = __builtin_fminf(__builtin_fminf(acc[h][0], acc[h][1]), acc[h][2]);
 #pragma unroll
-        for (int v = 1; v < 16; v += 2)
-          m = __builtin_fminf(__builtin_fminf(m, acc[h][v]), v + 1 < 16 ? acc[h][v + 1] : acc[h][v]);
+        for (int v = 3; v < 15; v += 2) m = __builtin_fminf(__builtin_fminf(m, acc[h][v]), acc[h][v + 1]);
+        m = __builtin_fminf(__builtin_fminf(m, acc[h][15]), KNN_FLT_MAX);
         if (__builtin_expect(!__any(m <= t[h]), 1)) continue;
         if (MODE == 2) {
           // A threshold estimate may ignore candidates (the bound only gets looser): every lane offers the
@@ -579,11 +588,11 @@ extern "C" __global__ void __launch_bounds__(64 * KNN_SWAVES) keops_knn_sample(c
 
 // fixed-threshold filter: KNN_FWAVES wavefronts of 32*KNN_FQSETS queries share every staged tile
 extern "C" __global__ void __launch_bounds__(64 * KNN_FWAVES) keops_knn_filter(const KnnParams P) {
-  __shared__ __attribute__((aligned(16))) unsigned char ys[KNN_TJ * KNN_STRIDE];
-  __shared__ __attribute__((aligned(16))) float ykey_s[KNN_TJ];
+  __shared__ __attribute__((aligned(16))) unsigned char ys[KNN_FTJ * KNN_STRIDE];
+  __shared__ __attribute__((aligned(16))) float ykey_s[KNN_FTJ];
   __shared__ int qq[KNN_FWAVES][64];
   __shared__ int qj[KNN_FWAVES][64];
-  knn_sweep<1, KNN_FWAVES, KNN_FQSETS>(P, ys, ykey_s, nullptr, nullptr, nullptr, qq, qj);
+  knn_sweep<1, KNN_FWAVES, KNN_FQSETS, KNN_FTJ>(P, ys, ykey_s, nullptr, nullptr, nullptr, qq, qj);
 }
 
 // every step-th reference row (bf16 row + key) gathered in a compact array for the sampling pass

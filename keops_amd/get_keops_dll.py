@@ -172,6 +172,8 @@ def generate_knn_plugin(red, rowvar, colvar, nargs):
     # low dimensions: neighbours are close compared with the norms, the operands are split as hi + lo
     split = int(D < 32)
     qsets, tj = config.knn_qsets, config.knn_tile_j
+    if not (1 <= config.knn_filter_qsets <= 2 and 1 <= config.knn_sample_qsets <= 2 and 1 <= qsets <= 2):
+        raise ValueError("[KeOps] the KNN kernels take one or two 32-query operand sets per wavefront")
     # as many wavefronts as the LDS budget allows share one staged reference tile: the K-lists of the
     # 32*qsets queries of every wavefront live in LDS (8 bytes per entry)
     fixed = tj * (dpad * 2 * (1 + split) + 16) + tj * 4
@@ -183,15 +185,19 @@ def generate_knn_plugin(red, rowvar, colvar, nargs):
     swaves, sqsets = config.knn_sample_waves, config.knn_sample_qsets
     if red.K > 16 or dpad * (1 + split) > 64:
         swaves = min(swaves, 8)
+    # the filter's workgroup is a whole compute unit that drains at every tile change: longer tiles there
+    ftj = max(tj, min(config.knn_filter_tile_j, 64 * config.knn_filter_waves))
+    while ftj > tj and ftj * (dpad * 2 * (1 + split) + 16) > 96 * 1024:
+        ftj //= 2
     meta = dict(scheme="knn", block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
                 sizeof_acc=4, nrowvars=1, ncolvars=1, nparvars=0, knn_d=D, knn_dpad=dpad, knn_k=red.K,
                 knn_qb=waves * 32 * qsets, knn_fwaves=config.knn_filter_waves, knn_fqsets=config.knn_filter_qsets,
-                knn_sample=config.knn_sample, knn_split=split, knn_sqb=swaves * 32 * sqsets, knn_sblock=64 * swaves,
+                knn_sample=config.knn_sample, knn_split=split, knn_ftj=ftj, knn_sqb=swaves * 32 * sqsets, knn_sblock=64 * swaves,
                 rowarg=rowvar.ind, colarg=colvar.ind)
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}", "typedef float T;"]
     defs = dict(KEOPS_NARGS=nargs, KNN_D=D, KNN_DPAD=dpad, KNN_K=red.K, KEOPS_RED_KEEP=red.keep, KEOPS_DIMOUT=red.dim,
                 KNN_QSETS=qsets, KNN_TJ=tj, KNN_WAVES=waves, KNN_FWAVES=config.knn_filter_waves,
-                KNN_FQSETS=config.knn_filter_qsets, KNN_SWAVES=swaves, KNN_SQSETS=sqsets, KNN_SPLIT=split)
+                KNN_FQSETS=config.knn_filter_qsets, KNN_FTJ=ftj, KNN_SWAVES=swaves, KNN_SQSETS=sqsets, KNN_SPLIT=split)
     src += [f"#define {k} {v}" for k, v in defs.items()]
     src.append('#include "keops_knn_mfma.h"')
     return "\n".join(src) + "\n", meta
