@@ -123,3 +123,15 @@ def test_cache_folder_controls(tmp_path):
         assert not os.path.exists(r[2])
     finally:
         assert keops_amd.set_build_folder(None) == default
+
+
+def test_reference_named_helpers_exist_and_health_check_runs(capsys):
+    """pykeops' top-level helpers (pykeops/__init__.py:20-104) under their own names."""
+    import keops_amd
+
+    for name in ("set_verbose", "get_build_folder", "set_build_folder", "clean_pykeops", "check_health",
+                 "test_torch_bindings", "test_numpy_bindings"):
+        assert callable(getattr(keops_amd, name)), name
+    assert keops_amd.check_health() is True
+    out = capsys.readouterr().out
+    assert "libkeops_hip.so" in out and "cache folder" in out
