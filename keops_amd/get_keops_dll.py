@@ -236,6 +236,49 @@ def match_chunk(red, dtype, map_reduce_id, use_fast_math):
     return (mode, node) + ((a, b) if a.cat == red.tagI else (b, a))
 
 
+def plan_row_col_product(red, dtype, use_fast_math, enable_chunks):
+    """Sum reductions of g_ij * w_ij where g is a scalar function of one high-dimensional contraction between an
+    output-indexed variable x_i and a reduced-index variable y_j, and w is x_i, y_j, x_i - y_j or y_j - x_i: the
+    gradients of radial and scalar-product kernels with respect to their points (Grad of Exp(-g*SqDist(x,y))*b with
+    respect to x is -2 g <e_i, b_j> K_ij (x_i - y_j)).  The long vectors outside the contraction keep such formulas
+    off the chunked scheme (Chunk_Mode_Constants.py:56-60) and on a kernel that holds whole rows per lane, but
+
+        sum_j g_ij (a x_i + c y_j) = a x_i sum_j g_ij + c sum_j g_ij y_j
+
+    is one scalar chunked reduction and matrix-core weighted sums of column slices of y.  Returns None or a dict
+    with sign, G (the scalar formula), row / col (the variables) and their coefficients a, c."""
+    from .formulas import ops as O
+
+    if not enable_chunks or not isinstance(red, Sum_Reduction) or dtype != "float" or not use_fast_math:
+        return None
+    F, sign = red.formula, 1
+    while F.name == "Minus":
+        F, sign = F.children[0], -sign
+    if F.name != "Mult" or len(F.children) != 2:
+        return None
+    for G, W in (F.children, F.children[::-1]):
+        if G.dim != 1 or W.dim < 32:
+            continue
+        wsign = 1
+        while W.name == "Minus":
+            W, wsign = W.children[0], -wsign
+        if isinstance(W, O.Var):
+            terms = [(1, W)]
+        elif W.name in ("Subtract", "Add") and all(isinstance(c, O.Var) for c in W.children):
+            terms = [(1, W.children[0]), (-1 if W.name == "Subtract" else 1, W.children[1])]
+        else:
+            continue
+        m = match_chunk(Sum_Reduction(G, red.tagI), dtype, "GpuReduc1D", use_fast_math)
+        if m is None:
+            continue
+        _, _, row, col = m
+        if any(v != row and v != col for _, v in terms) or len({v for _, v in terms}) != len(terms):
+            continue
+        coef = {v: c for c, v in terms}
+        return dict(sign=sign * wsign, G=G, row=row, col=col, a=coef.get(row, 0), c=coef.get(col, 0))
+    return None
+
+
 def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=False):
     """Module source for the matrix-core chunked scheme (kernels/keops_chunk_mfma.h); ``irregular``: the
     block-sparse / batched variant (GpuReduc1D_ranges_chunks.py:21-183)."""

@@ -11,8 +11,8 @@ import torch
 
 from . import binder
 from .common.parse_type import parse_dtype_acc
-from .formulas.parse import parse_alias
-from .get_keops_dll import get_keops_dll
+from .formulas.parse import parse_alias, parse_reduction
+from .get_keops_dll import get_keops_dll, plan_row_col_product
 
 _NULL_RANGE = np.array([-1], dtype=np.int64)
 _modules = {}
@@ -47,6 +47,31 @@ class LoadKeOps_hip:
         p.enable_chunks = optional_flags["enable_chunks"]
         p.mult_var_highdim = optional_flags.get("multVar_highdim", 0)
         p.tagHostDevice, p.tagCPUGPU = tagHostDevice, tagCPUGPU
+        self.plan = None
+        if tag1D2D == 0 and p.c_dtype == "float" and p.c_dtype_acc == "float":
+            red = parse_reduction(formula, p.aliases)
+            self.plan = plan_row_col_product(red, p.c_dtype, optional_flags["use_fast_math"], p.enable_chunks)
+        if self.plan is not None:
+            # sum_j g_ij (a x_i + c y_j) as a x_i sum_j g_ij + c sum_j g_ij y_j: one scalar reduction and weighted
+            # sums of column slices of y, each a module of the chunked scheme (get_keops_dll.plan_row_col_product)
+            plan, tagI = self.plan, red.tagI
+            D = plan["row"].dim
+            width = 64 if D > 128 else 128
+            sub = lambda f, extra: LoadKeOps_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, f,
+                                                 list(aliases) + extra, nargs + len(extra), dtype, lang, optional_flags,
+                                                 nx=nx, batch_loop=batch_loop, pairs=pairs)
+            self.sub_scalar = sub(f"Sum_Reduction({plan['G']!r},{tagI})", []) if plan["a"] else None
+            self.sub_slices = []
+            if plan["c"]:
+                for c0 in range(0, D, width):
+                    w = min(width, D - c0)
+                    v = f"Var({nargs},{w},{plan['col'].cat})"
+                    self.sub_slices.append((c0, c0 + w, sub(f"Sum_Reduction(Mult({plan['G']!r},{v}),{tagI})", [v])))
+            p.tagI, p.tagZero, p.dim, p.dimred = tagI, 0, D, D
+            p.device_id_request, p.nargs = device_id_request, nargs
+            p.reduction_op, p.axis = "Sum_Reduction", 1 - tagI
+            self.dimout, self.tagIJ, self.module = D, tagI, None
+            return
         map_reduce_id = "GpuReduc" + ("1D" if tag1D2D == 0 else "2D") + ("_ranges" if use_ranges else "")
         (p.tag, p.source_name, p.low_level_code_file, p.tagI, p.tagZero, p.use_half, p.use_fast_math,
          p.cuda_block_size, p.use_chunk_mode, p.tag1D2D, p.dimred, p.dim, p.dimy, indsi, indsj, indsp, dimsx,
@@ -70,7 +95,30 @@ class LoadKeOps_hip:
             if self.module is None:
                 self.module = _modules[key] = binder.Module(max(0, device_id_request), nargs, p.low_level_code_file)
 
+    def _row_col_product(self, device_args, ranges, nx, ny, nbatchdims, out, *args):
+        plan = self.plan
+        row, col = args[plan["row"].ind], args[plan["col"].ind]
+        res = None
+        if self.sub_slices:
+            parts = [ld.genred_pytorch(device_args, ranges, nx, ny, nbatchdims, None, *args, col[..., c0:c1].contiguous())
+                     for c0, c1, ld in self.sub_slices]
+            res = parts[0] if len(parts) == 1 else torch.cat(parts, dim=-1)
+            if plan["sign"] * plan["c"] < 0:
+                res = res.neg_()
+        if self.sub_scalar is not None:
+            total = self.sub_scalar.genred_pytorch(device_args, ranges, nx, ny, nbatchdims, None, *args)
+            if plan["sign"] * plan["a"] < 0:
+                total = total.neg_()
+            res = row * total if res is None else torch.addcmul(res, row, total)
+        if out is None:
+            return res
+        if tuple(out.shape) != tuple(res.shape) or not out.is_contiguous():
+            raise ValueError(f"[KeOps] 'out' must be a contiguous tensor of shape {tuple(res.shape)}")
+        return out.copy_(res)
+
     def genred_pytorch(self, device_args, ranges, nx, ny, nbatchdims, out, *args):
+        if self.plan is not None:
+            return self._row_col_product(device_args, ranges, nx, ny, nbatchdims, out, *args)
         p = self.params
         if not ranges:
             ranges_ptr, keep = self.empty_ranges, None

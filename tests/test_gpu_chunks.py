@@ -202,3 +202,56 @@ def test_contraction_beyond_256_components_batched():
     ref = K @ b.double()[:, :, 0]
     scale = K @ b.double()[:, :, 0].abs()
     assert_sum_parity(got.numpy(), ref.numpy(), scale.numpy())
+
+
+@pytest.mark.parametrize("D,kernel", [(64, "gauss"), (256, "laplace"), (200, "expdot"), (640, "gauss")])
+def test_gradients_wrt_points_as_scalar_and_weighted_sums(D, kernel):
+    """d/dx and d/dy of sum_ij e_i . K(x_i, y_j) b_j for radial and scalar-product kernels in high dimension:
+    g_ij (x_i - y_j) (or g_ij y_j) is computed as x_i sum_j g_ij - sum_j g_ij y_j, chunked reductions only
+    (get_keops_dll.plan_row_col_product).  Reference: torch.autograd on the dense float64 formula."""
+    from keops_amd import keops_io
+    from keops_amd.torch import Genred
+
+    M, N, Dv = 333, 450, 3
+    gen = torch.Generator().manual_seed(D)
+    x, y, b, e = (torch.randn(*s, generator=gen) for s in ((M, D), (N, D), (N, Dv), (M, Dv)))
+    x, y = x / D ** 0.5, y / D ** 0.5 + 0.1
+    formula = {"gauss": "Exp(-g*SqDist(x,y))*b", "laplace": "Exp(-g*Norm2(x-y))*b", "expdot": "Exp(g*(x|y))*b"}[kernel]
+    conv = Genred(formula, [f"x=Vi({D})", f"y=Vj({D})", f"b=Vj({Dv})", "g=Pm(1)"], reduction_op="Sum", axis=1)
+    xd, yd = x.cuda().requires_grad_(True), y.cuda().requires_grad_(True)
+    g = torch.tensor([0.7])
+    keops_io._loaders.clear()
+    out = conv(xd, yd, b.cuda(), g.cuda())
+    gx, gy = torch.autograd.grad(out, [xd, yd], e.cuda())
+    planned = [ld for ld in keops_io._loaders.values() if ld.plan is not None]
+    assert len(planned) == 2 and all(ld.module is None for ld in planned)
+    subs = [s for ld in planned for s in ([ld.sub_scalar] if ld.sub_scalar else []) + [t[2] for t in ld.sub_slices]]
+    assert subs and all(s.module.meta("scheme") == "chunk" for s in subs)
+    x64, y64 = x.double().requires_grad_(True), y.double().requires_grad_(True)
+    if kernel == "gauss":
+        K = torch.exp(-0.7 * torch.cdist(x64, y64) ** 2)
+    elif kernel == "laplace":
+        K = torch.exp(-0.7 * torch.cdist(x64, y64))
+    else:
+        K = torch.exp(0.7 * x64 @ y64.T)
+    rx, ry = torch.autograd.grad(((K @ b.double()) * e.double()).sum(), [x64, y64])
+    assert rel_l2(gx.cpu().numpy(), rx.numpy()) < 2e-5, rel_l2(gx.cpu().numpy(), rx.numpy())
+    assert rel_l2(gy.cpu().numpy(), ry.numpy()) < 2e-5, rel_l2(gy.cpu().numpy(), ry.numpy())
+
+
+def test_gradient_wrt_points_with_batch_dimensions_and_out():
+    from keops_amd.torch import LazyTensor
+
+    B, M, N, D = 3, 200, 260, 96
+    gen = torch.Generator().manual_seed(77)
+    x, y, b = torch.randn(B, M, D, generator=gen) / D ** 0.5, torch.randn(1, N, D, generator=gen) / D ** 0.5, torch.randn(B, N, 2, generator=gen)
+    xd, yd, bd = x.cuda().requires_grad_(True), y.cuda().requires_grad_(True), b.cuda()
+    K_ij = (-((LazyTensor(xd[:, :, None, :]) - LazyTensor(yd[:, None, :, :])) ** 2).sum(-1)).exp()
+    out = (K_ij * LazyTensor(bd[:, None, :, :])).sum(dim=2)
+    gx, gy = torch.autograd.grad(out.sum(), [xd, yd])
+    x64, y64 = x.double().requires_grad_(True), y.double().requires_grad_(True)
+    K = torch.exp(-torch.cdist(x64, y64.expand(B, N, D)) ** 2)
+    rx, ry = torch.autograd.grad((K @ b.double()).sum(), [x64, y64])
+    assert gx.shape == rx.shape and gy.shape == ry.shape
+    assert rel_l2(gx.cpu().numpy(), rx.numpy()) < 2e-5
+    assert rel_l2(gy.cpu().numpy(), ry.numpy()) < 2e-5
