@@ -255,3 +255,28 @@ def test_gradient_wrt_points_with_batch_dimensions_and_out():
     assert gx.shape == rx.shape and gy.shape == ry.shape
     assert rel_l2(gx.cpu().numpy(), rx.numpy()) < 2e-5
     assert rel_l2(gy.cpu().numpy(), ry.numpy()) < 2e-5
+
+
+def test_attention_backward_uses_chunked_reductions():
+    """Gradients of softmax(q k^T) v and of a log-sum-exp with respect to queries and keys (D = 64): every
+    reduction of the backward pass runs on the chunked scheme."""
+    from keops_amd import keops_io
+    from keops_amd.torch import LazyTensor
+
+    M, N, D, Dv = 500, 700, 64, 32
+    gen = torch.Generator().manual_seed(9)
+    q, k, v = torch.randn(M, D, generator=gen) / D ** 0.25, torch.randn(N, D, generator=gen) / D ** 0.25, torch.randn(N, Dv, generator=gen)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    keops_io._loaders.clear()
+    S_ij = (LazyTensor(qd[:, None, :]) * LazyTensor(kd[None, :, :])).sum(-1)
+    out = S_ij.sumsoftmaxweight(LazyTensor(vd[None, :, :]), dim=1)
+    lse = S_ij.logsumexp(dim=1)
+    e = torch.randn(M, Dv, generator=gen)
+    gq, gk, gv = torch.autograd.grad([out, lse], [qd, kd, vd], [e.cuda(), torch.ones(M, 1, device="cuda")])
+    assert all(ld.plan is not None or ld.module.meta("scheme") == "chunk" for ld in keops_io._loaders.values())
+    q64, k64, v64 = (t.double().requires_grad_(True) for t in (q, k, v))
+    S = q64 @ k64.T
+    rq, rk, rv = torch.autograd.grad([torch.softmax(S, 1) @ v64, torch.logsumexp(S, 1, keepdim=True)], [q64, k64, v64],
+                                     [e.double(), torch.ones(M, 1, dtype=torch.float64)])
+    for got, ref in ((gq, rq), (gk, rk), (gv, rv)):
+        assert rel_l2(got.cpu().numpy(), ref.numpy()) < 3e-5, rel_l2(got.cpu().numpy(), ref.numpy())
