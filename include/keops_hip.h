@@ -77,8 +77,14 @@ void keops_hip_module_destroy(void* module);
  *                     argndims[k] entries each
  *   hip_stream        hipStream_t to launch on (NULL = default stream)
  *   sync              non-zero: wait for completion before returning (the reference always does)
- * Returns 0 or a hipError_t / negative library code.
+ * Returns 0 or a hipError_t / negative library code.  KEOPS_HIP_NOT_CERTIFIED: a K-nearest-neighbour module for
+ * vectors of more than 256 components ranks candidates found with reduced-precision products; when ties or
+ * near-ties at the K-th distance keep it from proving that no reference was left out, it returns this code, `out`
+ * is not valid and the caller runs the same call on a module compiled without the chunked schemes
+ * (enable_chunks = 0), as keops_amd/keops_io.py does.  No counterpart in the reference, whose chunked kernels
+ * (GpuReduc1D_chunks.py) accumulate in float32.
  */
+#define KEOPS_HIP_NOT_CERTIFIED (-7)
 int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, int64_t ny, int tagI,
                      int tagZero, int tag1D2D, int64_t dimred, int64_t block_size, int use_chunk_mode,
                      const int* indsi, int ni, const int* indsj, int nj, const int* indsp, int np,

@@ -17,6 +17,13 @@ class KeOpsHipError(RuntimeError):
     pass
 
 
+NOT_CERTIFIED = -7  # KEOPS_HIP_NOT_CERTIFIED of include/keops_hip.h
+
+
+class KeOpsNotCertified(KeOpsHipError):
+    """A high-dimensional K-nearest-neighbour launch could not prove its result exact: run the exact kernel."""
+
+
 def lib():
     global _lib
     if _lib is None:
@@ -124,6 +131,8 @@ class Module:
             int(dimout), dx, dy, dp, rp, so, len(shapeout), ctypes.c_void_p(out_ptr), ap, sh, nd,
             ctypes.c_void_p(stream), int(bool(sync)),
         )
+        if rc == NOT_CERTIFIED:
+            raise KeOpsNotCertified(last_error())
         if rc != 0:
             raise KeOpsHipError(f"kernel launch failed (code {rc}): {last_error()}")
         return 0

@@ -728,15 +728,23 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   const bool split3 = final && !rg && m.meta_int("chk_split3", 0) != 0;
   const int64_t vcols = m.meta_int("chk_vcols", 0), ntiles = (ny + TJ - 1) / TJ;
   const size_t o_vsplit = take(split3 ? (size_t)ntiles * 3 * vcols * 40 * 2 : 0);
+  // K nearest neighbours in high dimension: the sweep keeps knn_inner > K approximate candidates per row in the
+  // workspace, a second kernel re-ranks them exactly into `out` and counts the rows it cannot certify
+  const int64_t knn_inner = m.meta_int("chk_knn_inner", 0);
+  if (knn_inner > 0 && (rg || final)) return fail(-1, "corrupt chunk module metadata");
+  const size_t o_lists = take(knn_inner > 0 ? (size_t)nx * 2 * knn_inner * 4 : 0), o_flag = take(knn_inner > 0 ? 256 : 0);
+  if (knn_inner > 0 && stream_is_capturing(stream))
+    return fail(-1, "this K-nearest-neighbour launch reads a flag back from the device: it cannot be captured in a HIP graph");
   if (int rc = m.partial.reserve(off)) return rc;
   char* ws = (char*)m.partial.ptr;
-  std::vector<char> buf(sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 8);
+  std::vector<char> buf(sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 32);
   ChkHeader h{};
   h.nx = nx; h.ny = ny; h.xs = ws + o_xs; h.ys = ws + o_ys; h.xn = ws + o_xn; h.yn = ws + o_yn; h.colsum = ws + o_colsum;
   h.colpart = ws + o_colpart; h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs;
   h.nxs = nxs; h.nys = nys;
   if (split3) h.vsplit = ws + o_vsplit;
   if (rg) h.rt = rg->header(m.nargs);
+  if (knn_inner > 0) h.out = ws + o_lists;
   std::memcpy(buf.data(), &h, sizeof(h));
   for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
   const size_t psize = sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs);
@@ -766,6 +774,19 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (final && nslabs > 1) {
     const int64_t gb = (nx * m.dimred + 255) / 256;
     if (int rc = launch_raw(m, softmax ? "keops_chk_softmax_reduce" : "keops_chk_reduce", (unsigned)gb, 1, 256, buf.data(), psize, stream)) return rc;
+  }
+  if (knn_inner > 0) {
+    void* extra[3] = {ws + o_lists, out, ws + o_flag};  // struct ChkKnnExtra of kernels/keops_chunk_mfma.h
+    std::memcpy(buf.data() + psize, extra, sizeof(extra));
+    if (int rc = launch_raw(m, "keops_chk_knn_ymax", 1, 1, 256, buf.data(), psize + sizeof(extra), stream)) return rc;
+    if (int rc = launch_raw(m, "keops_chk_knn_rerank", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), psize + sizeof(extra), stream)) return rc;
+    if (int rc = ensure_pinned(m, 64)) return rc;
+    HIP_TRY(hipMemcpyAsync(m.pinned, ws + o_flag, 4, hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipStreamSynchronize(stream));
+    const int bad = *(volatile int*)m.pinned;
+    if (bad != 0)
+      return fail(KEOPS_HIP_NOT_CERTIFIED, std::to_string(bad) + " rows have neighbours that the matrix-core pass cannot separate "
+                                           "(ties or near-ties at the K-th distance): recompute this call on the exact kernel");
   }
   return 0;
 }

@@ -392,6 +392,97 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
 }
 #endif
 
+// ---- K nearest neighbours in high dimension: exact re-rank of the lists of the sweep -----------------
+//
+// CHK_KNN_K: the module serves a KMin-family reduction of SqDist(x, y) with K = CHK_KNN_K.  keops_chk_main keeps the
+// KEOPS_RED_K > K smallest *approximate* squared distances per row (split bfloat16 operands: |approx - d| <=
+// CHK_KNN_C (|x^|^2 + |y^|^2) for the centred rows x^, y^) in the reference's (value, index) list layout.  Here
+// one lane per row computes the float32 distances of its candidates in the reference's operation order (sequential
+// sum of squared differences, no fused multiply-add), sorts them under (distance, index) and writes the K best.
+// The result is certified when every reference left out of the list is provably farther than the K-th neighbour:
+// (a_last - eps) (1 - 1e-4) > d_K with a_last the largest approximate distance kept and eps the bound above at the
+// largest |y^|^2; rows that fail the test are counted and the caller recomputes the call on the exact kernel.
+#if defined(CHK_KNN_K)
+#define CHK_KNN_C 2.0e-4f
+struct ChkKnnExtra {
+  const float* lists;  // [nx][2 * KEOPS_RED_K] approximate (value, index) pairs of the sweep
+  T* out;              // [nx][CHK_KNN_DIMOUT]
+  int* flag;           // flag[0]: rows that are not certified; flag[1] (as float): max_j |y^_j|^2
+};
+
+extern "C" __global__ void __launch_bounds__(256) keops_chk_knn_ymax(const ChkParams P, const ChkKnnExtra E) {
+  __shared__ float red[256];
+  float m = 0.f;
+  for (i64 j = threadIdx.x; j < P.ny; j += 256) m = __builtin_fmaxf(m, P.yn[j]);
+  red[threadIdx.x] = m;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) red[threadIdx.x] = __builtin_fmaxf(red[threadIdx.x], red[threadIdx.x + o]);
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    E.flag[0] = 0;
+    reinterpret_cast<float*>(E.flag)[1] = red[0];
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(256) keops_chk_knn_rerank(const ChkParams P, const ChkKnnExtra E) {
+  const i64 q = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (q >= P.nx) return;
+  const float inf = __builtin_huge_valf();
+  const float* L = E.lists + q * 2 * KEOPS_RED_K;
+  const T* xq = P.arg[CHK_XARG] + q * CHK_D;
+  float bd[CHK_KNN_K];
+  int bj[CHK_KNN_K];
+#pragma unroll
+  for (int l = 0; l < CHK_KNN_K; l++) {
+    bd[l] = inf;
+    bj[l] = 0;
+  }
+  float a_last = inf;
+  for (int c = 0; c < KEOPS_RED_K; c++) {
+    const float a = L[2 * c];
+    a_last = a;
+    if (!(a < inf)) break;  // fewer references than list entries: nothing was left out
+    const int j = (int)L[2 * c + 1];
+    const T* yr = P.arg[CHK_YARG] + (i64)j * CHK_D;
+    float d = 0.f;
+    {
+#pragma clang fp contract(off)
+      for (int k = 0; k < CHK_D; k++) {
+        const float t = xq[k] - yr[k];
+        d = d + t * t;
+      }
+    }
+    // sorted insertion under (distance, index)
+    bool before_cur = d < bd[CHK_KNN_K - 1] || (d == bd[CHK_KNN_K - 1] && j < bj[CHK_KNN_K - 1]);
+#pragma unroll
+    for (int l = CHK_KNN_K - 1; l > 0; l--) {
+      const bool before_prev = d < bd[l - 1] || (d == bd[l - 1] && j < bj[l - 1]);
+      bd[l] = before_prev ? bd[l - 1] : (before_cur ? d : bd[l]);
+      bj[l] = before_prev ? bj[l - 1] : (before_cur ? j : bj[l]);
+      before_cur = before_prev;
+    }
+    bd[0] = before_cur ? d : bd[0];
+    bj[0] = before_cur ? j : bj[0];
+  }
+  T* o = E.out + q * CHK_KNN_DIMOUT;
+#pragma unroll
+  for (int l = 0; l < CHK_KNN_K; l++) {
+    if (CHK_KNN_KEEP == 0) {
+      o[2 * l] = bd[l];
+      o[2 * l + 1] = (T)bj[l];
+    } else {
+      o[l] = CHK_KNN_KEEP == 1 ? bd[l] : (T)bj[l];
+    }
+  }
+  if (a_last < inf) {
+    const float eps = CHK_KNN_C * (P.xn[q] + reinterpret_cast<const float*>(E.flag)[1]);
+    if (!((a_last - eps) * (1.0f - 1.0e-4f) > bd[CHK_KNN_K - 1])) atomicAdd(E.flag, 1);
+  }
+}
+#endif
+
 // ---- weighted sums with every operand in three bfloat16 terms ----------------------------------------
 //
 // Dense launches of the two variants below (CHK_SPLIT3).  x = h + m + l with h = bf16(x), m = bf16(x - h),

@@ -203,6 +203,45 @@ def generate_knn_plugin(red, rowvar, colvar, nargs):
     return "\n".join(src) + "\n", meta
 
 
+def match_knn_highdim(red, dtype, map_reduce_id, use_fast_math):
+    """(mode, node, row variable, column variable) in match_chunk's format when ``red`` is a K-min family reduction
+    of SqDist between an output-indexed and a reduced-index variable of more than 256 (the limit of the KNN
+    scheme) and at most config.chunk_max_dim components, float32, dense: the chunked sweep keeps K +
+    config.knn_highdim_margin approximate candidates per row and a second kernel re-ranks them exactly."""
+    from .formulas import ops as O
+
+    if (red.kind != KIND_KMIN or dtype != "float" or not use_fast_math or "_ranges" in map_reduce_id
+            or red.K + config.knn_highdim_margin > 40 or red.formula.dim != 1):
+        return None
+    f = red.formula
+    if f.name != "Sum" or f.children[0].name != "Square" or f.children[0].children[0].name != "Subtract":
+        return None
+    a, b = f.children[0].children[0].children
+    if not (isinstance(a, O.Var) and isinstance(b, O.Var)) or a.dim != b.dim or not 256 < a.dim <= config.chunk_max_dim:
+        return None
+    if {a.cat, b.cat} != {0, 1}:
+        return None
+    return (0, f) + ((a, b) if a.cat == red.tagI else (b, a))
+
+
+def generate_knn_highdim_plugin(red, match, nargs):
+    """Chunked module whose sweep runs a KMin_ArgKMin reduction with K + margin entries on the approximate
+    distances, plus the exact re-rank kernels (kernels/keops_chunk_mfma.h, CHK_KNN_K)."""
+    from .formulas.reductions import KMin_ArgKMin_Reduction
+
+    inner = KMin_ArgKMin_Reduction(red.formula, red.K + config.knn_highdim_margin, red.tagI)
+    source, meta = generate_chunk_plugin(inner, match, "float", "direct_sum", nargs)
+    if source is None:
+        return None, None
+    meta.update(dimred=red.dimred, dimout=red.dim, chk_knn=red.K, chk_knn_inner=inner.K)
+    head, body = source.split("\n", 1)
+    head = "//@keops " + " ".join(f"{k}={v}" for k, v in meta.items())
+    defs = f"#define CHK_KNN_K {red.K}\n#define CHK_KNN_KEEP {red.keep}\n#define CHK_KNN_DIMOUT {red.dim}\n"
+    marker = '#include "keops_common.h"\n'
+    assert marker in body
+    return head + "\n" + body.replace(marker, marker + defs, 1), meta
+
+
 def match_chunk(red, dtype, map_reduce_id, use_fast_math):
     """(mode, node, row variable, column variable) when the formula of a Sum / log-sum-exp reduction
     contains exactly one high-dimensional contraction SqDist(x_i, y_j) (mode 0) or <x_i, y_j> (mode 1)
@@ -504,6 +543,7 @@ def get_keops_dll(
     else:
         irregular = "_ranges" in map_reduce_id
         knn = match_knn_sqdist(red, dtype, map_reduce_id, batch_loop, pairs) if enable_chunks else None
+        knn_hd = match_knn_highdim(red, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
         chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
         fin = None
         if enable_finalchunks and knn is None and chk is None:
@@ -516,6 +556,9 @@ def get_keops_dll(
             use_chunk_mode = 2  # as the reference's final-chunk mode (get_keops_dll.py:101-108)
         elif chk is not None:
             source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs, irregular=irregular)
+            use_chunk_mode = 1 if source is not None else 0
+        elif knn_hd is not None:
+            source, meta = generate_knn_highdim_plugin(red, knn_hd, nargs)
             use_chunk_mode = 1 if source is not None else 0
         else:
             source = None

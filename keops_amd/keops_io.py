@@ -47,6 +47,10 @@ class LoadKeOps_hip:
         p.enable_chunks = optional_flags["enable_chunks"]
         p.mult_var_highdim = optional_flags.get("multVar_highdim", 0)
         p.tagHostDevice, p.tagCPUGPU = tagHostDevice, tagCPUGPU
+        # what a twin of this object without the matrix-core schemes is built from (see genred_pytorch)
+        self._ctor = (tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula, list(aliases), nargs,
+                      dtype, lang, dict(optional_flags), nx)
+        self._exact = None
         self.plan = None
         if tag1D2D == 0 and p.c_dtype == "float" and p.c_dtype_acc == "float":
             red = parse_reduction(formula, p.aliases)
@@ -142,11 +146,18 @@ class LoadKeOps_hip:
             out.zero_()
             return out
         stream = torch.cuda.current_stream(out.device).cuda_stream
-        self.module(
-            p.tagHostDevice, p.dimy, nx, ny, p.tagI, p.tagZero, p.use_half, p.tag1D2D, p.dimred, p.cuda_block_size,
-            p.use_chunk_mode, p.indsi, p.indsj, p.indsp, p.dim, p.dimsx, p.dimsy, p.dimsp, ranges_ptr, tuple(out.shape),
-            int(out.data_ptr()), args_ptr, argshapes, stream=stream, sync=False,
-        )
+        try:
+            self.module(
+                p.tagHostDevice, p.dimy, nx, ny, p.tagI, p.tagZero, p.use_half, p.tag1D2D, p.dimred, p.cuda_block_size,
+                p.use_chunk_mode, p.indsi, p.indsj, p.indsp, p.dim, p.dimsx, p.dimsy, p.dimsp, ranges_ptr,
+                tuple(out.shape), int(out.data_ptr()), args_ptr, argshapes, stream=stream, sync=False,
+            )
+        except binder.KeOpsNotCertified:
+            # high-dimensional K nearest neighbours with ties at the K-th distance: same call on the exact kernel
+            if self._exact is None:
+                c = self._ctor
+                self._exact = LoadKeOps_hip(*c[:10], dict(c[10], enable_chunks=0), nx=c[11])
+            return self._exact.genred_pytorch(device_args, ranges, nx, ny, nbatchdims, out, *args)
         del keep
         return out
 

@@ -219,3 +219,55 @@ def test_small_problem_stays_on_the_general_purpose_kernel(monkeypatch):
     for k in range(64):
         d += (x[:, None, k] - y[None, :, k]) ** 2
     assert np.array_equal(idx, np.argsort(d, axis=1, kind="stable")[:, :10])
+
+
+def _sequential_sqdist(x, y):
+    """Float32 squared distances in the reference's operation order (sum of squared differences, component by
+    component, no fused multiply-add)."""
+    d = np.zeros((x.shape[0], y.shape[0]), np.float32)
+    for k in range(x.shape[1]):
+        d += (x[:, None, k] - y[None, :, k]) ** 2
+    return d
+
+
+@pytest.mark.parametrize("M,N,D,K,op", [(700, 5000, 300, 10, "ArgKMin"), (300, 3000, 784, 5, "KMin_ArgKMin"),
+                                        (100, 2500, 1000, 3, "KMin"), (50, 7, 400, 10, "KMin_ArgKMin")])
+def test_knn_beyond_256_components_chunked_sweep_and_exact_rerank(M, N, D, K, op):
+    """More than 256 components: the chunked matrix-core sweep keeps K + 6 approximate candidates, the re-rank
+    kernel orders them by exact float32 distance and certifies that nothing was left out: bit-exact indices and
+    values against a stable argsort of the reference-order distances (N < K: the tail stays (inf, 0))."""
+    from keops_amd import keops_io
+
+    rng = np.random.default_rng(D + K)
+    x, y = rng.random((M, D), dtype=np.float32), rng.random((N, D), dtype=np.float32)
+    out = _knn(D, K, op)(*to_dev(x, y))
+    (ld,) = keops_io._loaders.values()
+    assert ld.module.meta("scheme") == "chunk" and ld.module.meta("chk_knn") == str(K) and ld._exact is None
+    d = _sequential_sqdist(x, y)
+    order = np.argsort(d, axis=1, kind="stable")[:, :K]
+    vals = np.take_along_axis(d, order, 1)
+    if N < K:
+        order = np.concatenate([order, np.zeros((M, K - N), order.dtype)], 1)
+        vals = np.concatenate([vals, np.full((M, K - N), np.inf, np.float32)], 1)
+    if op == "ArgKMin":
+        assert np.array_equal(out.cpu().numpy().astype(np.int64), order)
+    elif op == "KMin":
+        assert np.array_equal(out.cpu().numpy(), vals)
+    else:
+        assert np.array_equal(out[0].cpu().numpy(), vals) and np.array_equal(out[1].cpu().numpy().astype(np.int64), order)
+
+
+def test_knn_beyond_256_components_ties_fall_back_to_the_exact_kernel():
+    """Every reference row appears 20 times: the K-th distance is tied with rows outside any list of K + 6
+    candidates, the launch reports that it cannot certify its result and the call is redone on the exact kernel
+    (lowest index first among equal distances)."""
+    from keops_amd import keops_io
+
+    M, D, K = 200, 320, 10
+    rng = np.random.default_rng(1)
+    x = rng.random((M, D), dtype=np.float32)
+    y = np.tile(rng.random((60, D), dtype=np.float32), (20, 1))
+    idx = _knn(D, K, "ArgKMin")(*to_dev(x, y)).cpu().numpy()
+    (ld,) = keops_io._loaders.values()
+    assert ld.module.meta("chk_knn") == str(K) and ld._exact is not None and ld._exact.module.meta("scheme") == "conv"
+    assert np.array_equal(idx.astype(np.int64), np.argsort(_sequential_sqdist(x, y), axis=1, kind="stable")[:, :K])
