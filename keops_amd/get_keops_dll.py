@@ -542,14 +542,22 @@ def get_keops_dll(
         target, tag, src_file = "", "zero", ""
     else:
         irregular = "_ranges" in map_reduce_id
-        knn = match_knn_sqdist(red, dtype, map_reduce_id, batch_loop, pairs) if enable_chunks else None
-        knn_hd = match_knn_highdim(red, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
+        # Min / ArgMin / Min_ArgMin of a scalar formula are the K = 1 members of the K-min family (same accumulator
+        # and output layout, same "first index wins" rule): they share its matrix-core schemes
+        red_k = red
+        if red.kind == KIND_MIN and red.formula.dim == 1 and config.min_as_kmin:
+            from .formulas.reductions import KEEP_BOTH, KEEP_VAL, ArgKMin_Reduction, KMin_ArgKMin_Reduction, KMin_Reduction
+
+            cls = KMin_ArgKMin_Reduction if red.keep == KEEP_BOTH else (KMin_Reduction if red.keep == KEEP_VAL else ArgKMin_Reduction)
+            red_k = cls(red.formula, 1, red.tagI)
+        knn = match_knn_sqdist(red_k, dtype, map_reduce_id, batch_loop, pairs) if enable_chunks else None
+        knn_hd = match_knn_highdim(red_k, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
         chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
         fin = None
         if enable_finalchunks and knn is None and chk is None:
             fin = match_final(red, dtype, dtypeacc, sum_scheme_string, map_reduce_id)
         if knn is not None:
-            source, meta = generate_knn_plugin(red, knn[0], knn[1], nargs)
+            source, meta = generate_knn_plugin(red_k, knn[0], knn[1], nargs)
             use_chunk_mode = 3  # matrix-core filter scheme (no counterpart among the reference's chunk modes)
         elif fin is not None:
             source, meta = generate_final_plugin(red, fin, sum_scheme_string, nargs, irregular=irregular)
@@ -558,7 +566,7 @@ def get_keops_dll(
             source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs, irregular=irregular)
             use_chunk_mode = 1 if source is not None else 0
         elif knn_hd is not None:
-            source, meta = generate_knn_highdim_plugin(red, knn_hd, nargs)
+            source, meta = generate_knn_highdim_plugin(red_k, knn_hd, nargs)
             use_chunk_mode = 1 if source is not None else 0
         else:
             source = None

@@ -271,3 +271,31 @@ def test_knn_beyond_256_components_ties_fall_back_to_the_exact_kernel():
     (ld,) = keops_io._loaders.values()
     assert ld.module.meta("chk_knn") == str(K) and ld._exact is not None and ld._exact.module.meta("scheme") == "conv"
     assert np.array_equal(idx.astype(np.int64), np.argsort(_sequential_sqdist(x, y), axis=1, kind="stable")[:, :K])
+
+
+@pytest.mark.parametrize("D,scheme", [(64, "knn"), (400, "chunk")])
+def test_min_family_of_sqdist_runs_as_k_equal_one(D, scheme):
+    """Min, ArgMin and Min_ArgMin of SqDist share the K-min schemes with K = 1 (same layout, first index wins):
+    bit-exact against the reference-order distances, duplicated references included."""
+    from keops_amd import keops_io
+    from keops_amd.torch import Genred
+
+    M, N = 600, 4000
+    rng = np.random.default_rng(D)
+    x, y = rng.random((M, D), dtype=np.float32), rng.random((N, D), dtype=np.float32)
+    if scheme == "knn":
+        y[N // 2:] = y[:N // 2]          # exact ties: the lower index must win
+    d = _sequential_sqdist(x, y)
+    ref_i, ref_v = d.argmin(1), d.min(1)
+    for op in ("ArgMin", "Min", "Min_ArgMin"):
+        keops_io._loaders.clear()
+        out = Genred("SqDist(x,y)", [f"x=Vi({D})", f"y=Vj({D})"], reduction_op=op, axis=1)(*to_dev(x, y))
+        (ld,) = keops_io._loaders.values()
+        assert ld.module.meta("scheme") == scheme, op
+        if op == "ArgMin":
+            assert np.array_equal(out.cpu().numpy()[:, 0].astype(np.int64), ref_i)
+        elif op == "Min":
+            assert np.array_equal(out.cpu().numpy()[:, 0], ref_v)
+        else:
+            assert np.array_equal(out[0].cpu().numpy()[:, 0], ref_v)
+            assert np.array_equal(out[1].cpu().numpy()[:, 0].astype(np.int64), ref_i)
