@@ -50,6 +50,7 @@ knn_filter_qsets = int(os.environ.get("KEOPS_AMD_KNN_FQSETS", 2))   # and 32-que
 knn_sample = int(os.environ.get("KEOPS_AMD_KNN_SAMPLE", 16))            # sampling pass: every 16th reference
 knn_sample_waves = int(os.environ.get("KEOPS_AMD_KNN_SWAVES", 8))  # sampling pass: wavefronts per workgroup
 knn_sample_qsets = int(os.environ.get("KEOPS_AMD_KNN_SQSETS", 1))   # and 32-query operand sets per wavefront
+vchunk_min_dim = int(os.environ.get("KEOPS_AMD_VCHUNK_MIN_DIM", 100))   # long elementwise sums beyond this many components keep their rows in memory
 min_as_kmin = int(os.environ.get("KEOPS_AMD_MIN_AS_KMIN", 1))        # Min / ArgMin of SqDist on the KNN schemes (K = 1)
 knn_highdim_margin = int(os.environ.get("KEOPS_AMD_KNN_HD_MARGIN", 6))   # extra approximate candidates kept per row by the high-dimensional KNN sweep
 knn_min_work = int(os.environ.get("KEOPS_AMD_KNN_MIN_WORK", 1 << 31))      # smallest pairs x max(D, 16) served by the matrix-core KNN scheme

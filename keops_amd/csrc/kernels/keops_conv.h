@@ -20,8 +20,19 @@
 // KEOPS_RED_KEEP, KEOPS_RED_K, KEOPS_SUM_SCHEME, KEOPS_FAST_MATH, KEOPS_BLOCK, KEOPS_ROWS,
 // KEOPS_TILE_J, KEOPS_UNROLL_J, KEOPS_LSE_GROUP, the tables keops_{row,col,par}_{arg,dim,off}[] with their counts
 // KEOPS_NROWVARS / KEOPS_NCOLVARS / KEOPS_NPARVARS, and struct KeopsFormula.
+//
+// KEOPS_VCHUNK (formulas with one long elementwise sum, the vector-ALU counterpart of GpuReduc1D_chunks.py:19-118):
+// the plug-in also defines VCH_D (components), VCH_DPAD, VCH_NROW / VCH_NCOL (long output-indexed / reduced-index
+// variables), the flags keops_{row,col}_long[] and positions keops_vch_{row,col}[] of those variables in the
+// tables, VCH_USES_YJ, and struct KeopsChunkFormula (one component of the sum).  Long variables are not copied to
+// x_i / y_j: the reduced-index ones are staged whole in LDS for a short tile of columns, the output-indexed ones are
+// read from memory 16 bytes at a time (one cache line serves four such reads), each read feeding KEOPS_TILE_J
+// running sums held in registers; KeopsFormula::eval takes the finished sum as an extra argument.
 #pragma once
 #include "keops_reductions.h"
+#ifndef KEOPS_VCHUNK
+#define KEOPS_VCHUNK 0
+#endif
 
 // Kernel argument block; the host library fills the same layout (keops_hip.cpp: LaunchParams).
 struct KeopsParams {
@@ -47,6 +58,9 @@ struct KeopsParams {
 __device__ __forceinline__ void keops_load_row(const KeopsParams& P, const i64* rowoff, i64 i, T (&xi)[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1]) {
 #pragma unroll
   for (int v = 0; v < KEOPS_NROWVARS; v++) {
+#if KEOPS_VCHUNK
+    if (keops_row_long[v]) continue;
+#endif
     const T* src = P.arg[keops_row_arg[v]] + (rowoff[v] + i) * keops_row_dim[v];
 #pragma unroll
     for (int d = 0; d < keops_row_dim[v]; d++) xi[keops_row_off[v] + d] = src[d];
@@ -68,6 +82,9 @@ __device__ __forceinline__ void keops_load_params(const KeopsParams& P, const i6
 __device__ __forceinline__ void keops_stage_tile(const KeopsParams& P, const i64* coloff, i64 j0, int n, T* ys) {
 #pragma unroll
   for (int v = 0; v < KEOPS_NCOLVARS; v++) {
+#if KEOPS_VCHUNK
+    if (keops_col_long[v]) continue;
+#endif
     const int dim = keops_col_dim[v];
     const T* src = P.arg[keops_col_arg[v]] + (coloff[v] + j0) * dim;
     const int total = n * dim;
@@ -90,6 +107,122 @@ __device__ __forceinline__ void keops_read_col(const T* ys, int jj, T (&yj)[KEOP
   }
 }
 
+#if KEOPS_VCHUNK
+// ---- the pair loop of formulas with one long elementwise sum -----------------------------------
+
+static_assert(KEOPS_ROWS == 1, "one output row per lane");
+constexpr int VCH_VEC = 16 / sizeof(T);
+typedef T vch_vec __attribute__((ext_vector_type(VCH_VEC)));
+
+// Folds columns [jbeg, jend) into acc[0].  xlong[v]: this lane's row of the v-th long output-indexed variable.
+__device__ __forceinline__ void keops_sweep(const KeopsParams& P, const i64* coloff, i64 jbeg, i64 jend, i64 jshift,
+                                            const T (&xi)[KEOPS_ROWS][KEOPS_DIMX > 0 ? KEOPS_DIMX : 1],
+                                            const T (&p)[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1],
+                                            KeopsAcc<TACC> (&acc)[KEOPS_ROWS], T* ys, T* yl,
+                                            const T* const (&xlong)[VCH_NROW > 0 ? VCH_NROW : 1]) {
+#if KEOPS_RED_KIND >= 2
+#pragma clang fp contract(off)  // index-carrying reductions: the running sum keeps the reference's roundings
+#endif
+  constexpr int NR = VCH_NROW > 0 ? VCH_NROW : 1, NC = VCH_NCOL > 0 ? VCH_NCOL : 1;
+  for (i64 j0 = jbeg; j0 < jend; j0 += KEOPS_TILE_J) {
+    const int n = (int)keops_min((i64)KEOPS_TILE_J, jend - j0);
+    __syncthreads();  // the previous tile has been consumed by every wave
+    keops_stage_tile(P, coloff, j0, n, ys);
+    // long reduced-index variables: row jj of variable v at yl + (jj * VCH_NCOL + v) * VCH_DPAD
+#pragma unroll
+    for (int v = 0; v < VCH_NCOL; v++) {
+      const T* src = P.arg[keops_col_arg[keops_vch_col[v]]] + (coloff[keops_vch_col[v]] + j0) * VCH_D;
+      for (int e = threadIdx.x; e < n * VCH_D; e += KEOPS_BLOCK) {
+        const int row = e / VCH_D, c = e - row * VCH_D;
+        yl[(row * VCH_NCOL + v) * VCH_DPAD + c] = src[e];
+      }
+    }
+    __syncthreads();
+    T s[KEOPS_TILE_J];
+#pragma unroll
+    for (int jj = 0; jj < KEOPS_TILE_J; jj++) s[jj] = (T)0;
+    T yj0[KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1] = {};
+    // whole groups of VCH_VEC components, in order (a sequential sum, as the reference's)
+    for (int k0 = 0; k0 + VCH_VEC <= VCH_D; k0 += VCH_VEC) {
+      T xk[NR][VCH_VEC];
+#pragma unroll
+      for (int v = 0; v < VCH_NROW; v++)
+#pragma unroll
+        for (int c = 0; c < VCH_VEC; c++) xk[v][c] = xlong[v][k0 + c];
+#pragma unroll
+      for (int jj = 0; jj < KEOPS_TILE_J; jj++) {
+        T yk[NC][VCH_VEC];
+#pragma unroll
+        for (int v = 0; v < VCH_NCOL; v++) {
+          const vch_vec w = *reinterpret_cast<const vch_vec*>(yl + (jj * VCH_NCOL + v) * VCH_DPAD + k0);
+#pragma unroll
+          for (int c = 0; c < VCH_VEC; c++) yk[v][c] = w[c];
+        }
+#if VCH_USES_YJ
+        T yj[KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1];
+        keops_read_col(ys, jj, yj);
+#else
+        const T (&yj)[KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1] = yj0;
+#endif
+#pragma unroll
+        for (int c = 0; c < VCH_VEC; c++) {
+          T xc[NR], yc[NC];
+#pragma unroll
+          for (int v = 0; v < NR; v++) xc[v] = xk[v][c];
+#pragma unroll
+          for (int v = 0; v < NC; v++) yc[v] = yk[v][c];
+          s[jj] = s[jj] + KeopsChunkFormula::eval(xc, yc, xi[0], yj, p);
+        }
+      }
+    }
+    // the last VCH_D % VCH_VEC components
+    if (VCH_D % VCH_VEC != 0) {
+      constexpr int k0 = VCH_D / VCH_VEC * VCH_VEC;
+#pragma unroll
+      for (int jj = 0; jj < KEOPS_TILE_J; jj++) {
+#if VCH_USES_YJ
+        T yj[KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1];
+        keops_read_col(ys, jj, yj);
+#else
+        const T (&yj)[KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1] = yj0;
+#endif
+#pragma unroll
+        for (int c = 0; c < VCH_D % VCH_VEC; c++) {
+          T xc[NR] = {}, yc[NC] = {};
+#pragma unroll
+          for (int v = 0; v < VCH_NROW; v++) xc[v] = xlong[v][k0 + c];
+#pragma unroll
+          for (int v = 0; v < VCH_NCOL; v++) yc[v] = yl[(jj * VCH_NCOL + v) * VCH_DPAD + k0 + c];
+          s[jj] = s[jj] + KeopsChunkFormula::eval(xc, yc, xi[0], yj, p);
+        }
+      }
+    }
+#if KEOPS_USE_TILE_TMP
+    KeopsAcc<T> tmp;
+    tmp.init();
+#endif
+#pragma unroll
+    for (int jj = 0; jj < KEOPS_TILE_J; jj++) {
+      if (jj < n) {
+        T yj[KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1];
+        keops_read_col(ys, jj, yj);
+        T fout[KEOPS_DIMFOUT];
+        KeopsFormula::eval(xi[0], yj, p, s[jj], fout);
+#if KEOPS_USE_TILE_TMP
+        tmp.push(fout, j0 + jj - jshift);
+#else
+        acc[0].push(fout, j0 + jj - jshift);
+#endif
+      }
+    }
+#if KEOPS_USE_TILE_TMP
+    acc[0].merge(tmp);
+#endif
+  }
+}
+#define KEOPS_SWEEP_EXTRA , yl, xlong
+#else
+#define KEOPS_SWEEP_EXTRA
 // ---- the pair loop over one contiguous column range ----------------------------------------
 
 // Folds columns [jbeg, jend) into acc[].  jshift is subtracted from the column index handed to
@@ -168,6 +301,8 @@ __device__ __forceinline__ void keops_sweep(const KeopsParams& P, const i64* col
   }
 }
 
+#endif  // KEOPS_VCHUNK
+
 // ---- dense scheme ---------------------------------------------------------------------------
 
 extern "C" __global__ void __launch_bounds__(KEOPS_BLOCK) keops_conv_dense(const KeopsParams P) {
@@ -188,7 +323,14 @@ extern "C" __global__ void __launch_bounds__(KEOPS_BLOCK) keops_conv_dense(const
 
   const i64 jbeg = (i64)blockIdx.y * P.slab_len;
   const i64 jend = keops_min(P.ny, jbeg + P.slab_len);
-  keops_sweep(P, zero_off, jbeg, jend, 0, xi, p, acc, ys);
+#if KEOPS_VCHUNK
+  __shared__ __attribute__((aligned(16))) T yl[KEOPS_TILE_J * (VCH_NCOL > 0 ? VCH_NCOL : 1) * VCH_DPAD];
+  const T* xlong[VCH_NROW > 0 ? VCH_NROW : 1] = {};
+#pragma unroll
+  for (int v = 0; v < VCH_NROW; v++)
+    xlong[v] = P.arg[keops_row_arg[keops_vch_row[v]]] + (row0 < P.nx ? row0 : P.nx - 1) * VCH_D;
+#endif
+  keops_sweep(P, zero_off, jbeg, jend, 0, xi, p, acc, ys KEOPS_SWEEP_EXTRA);
 
 #pragma unroll
   for (int r = 0; r < KEOPS_ROWS; r++) {
@@ -263,6 +405,17 @@ extern "C" __global__ void __launch_bounds__(KEOPS_BLOCK) keops_conv_ranges(cons
     acc[r].init();
   }
 
+#if KEOPS_VCHUNK
+  __shared__ __attribute__((aligned(16))) T yl[KEOPS_TILE_J * (VCH_NCOL > 0 ? VCH_NCOL : 1) * VCH_DPAD];
+  const T* xlong[VCH_NROW > 0 ? VCH_NROW : 1] = {};
+  {
+    i64 rel = (i64)threadIdx.x;
+    if (start_x + rel >= end_x) rel = end_x - start_x - 1;
+#pragma unroll
+    for (int v = 0; v < VCH_NROW; v++)
+      xlong[v] = P.arg[keops_row_arg[keops_vch_row[v]]] + (rowoff[keops_vch_row[v]] + (batched ? rel : start_x + rel)) * VCH_D;
+  }
+#endif
   if (start_slice < end_slice) {
     i64 start_y = P.ranges_y[2 * start_slice];
     for (i64 index = start_slice; index < end_slice; index++) {
@@ -270,9 +423,9 @@ extern "C" __global__ void __launch_bounds__(KEOPS_BLOCK) keops_conv_ranges(cons
         const i64 end_y = P.ranges_y[2 * index + 1];
         // batch mode: variables are read at (offset + j - start_y) and indices are batch-relative
         if (batched)
-          keops_sweep(P, coloff, 0, end_y - start_y, 0, xi, p, acc, ys);
+          keops_sweep(P, coloff, 0, end_y - start_y, 0, xi, p, acc, ys KEOPS_SWEEP_EXTRA);
         else
-          keops_sweep(P, coloff, start_y, end_y, 0, xi, p, acc, ys);
+          keops_sweep(P, coloff, start_y, end_y, 0, xi, p, acc, ys KEOPS_SWEEP_EXTRA);
         if (index + 1 < end_slice) start_y = P.ranges_y[2 * index + 2];
       }
     }

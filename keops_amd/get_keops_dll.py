@@ -203,6 +203,161 @@ def generate_knn_plugin(red, rowvar, colvar, nargs):
     return "\n".join(src) + "\n", meta
 
 
+def match_vchunk(red):
+    """(node, E, long variables) when the formula contains exactly one Sum(E) over an elementwise expression E of
+    more than config.vchunk_min_dim components whose long operands are plain i- or j-indexed variables that appear
+    nowhere else (the reference's chunkable operations and its rule against mixing chunked and post-chunk
+    variables, Chunkable_Op.py:20-41, Chunk_Mode_Constants.py:56-60); None otherwise."""
+    from .formulas import ops as O
+
+    def elementwise(node, D):
+        if isinstance(node, O.Var):
+            return node.dim == 1 or (node.dim == D and node.cat in (0, 1))
+        if not node.children:
+            return node.dim == 1  # constants
+        return isinstance(node, O.Elementwise) and node.dim in (1, D) and all(elementwise(c, D) for c in node.children)
+
+    found = []
+    for node in red.formula.walk():
+        if node.name == "Sum" and node.children[0].dim > config.vchunk_min_dim and node not in [f[0] for f in found]:
+            E = node.children[0]
+            if elementwise(E, E.dim):
+                found.append((node, E))
+    if len(found) != 1:
+        return None
+    node, E = found[0]
+    longs = [v for v in E.variables if v.dim == E.dim and v.dim > 1]
+    if not longs or any(v.cat not in (0, 1) for v in longs):
+        return None
+    post = red.formula.replace(node, O.Var(1 << 30, 1, 3))
+    if any(v in longs for v in post.variables) or any(v.dim > config.vchunk_min_dim for v in post.variables):
+        return None
+    return node, E, longs
+
+
+def generate_vchunk_plugin(red, match, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, irregular=False):
+    """Module source for formulas with one long elementwise sum (GpuReduc1D_chunks.py:19-118 without matrix-core
+    form: L1 distances, weighted or transformed sums, float64 contractions): the general-purpose kernels of
+    kernels/keops_conv.h built with KEOPS_VCHUNK, where the long rows stay in memory (the reduced-index ones staged in
+    LDS tile by tile, the output-indexed ones streamed through the cache) and only the running sums of a tile of
+    columns live in registers."""
+    from .formulas import ops as O
+
+    node, E, longs = match
+    D = E.dim
+    sizeof_t = 8 if dtype == "double" else 4
+    vec = 16 // sizeof_t
+    dpad = -(-D // vec) * vec
+    svar = O.Var(1 << 30, 1, 3)
+    post = red.formula.replace(node, svar)
+    exact = red.kind in (KIND_MIN, KIND_MAX, KIND_KMIN)
+    full = VarLayout(red)
+    row_long = [v for v in full.rowvars if v in longs]
+    col_long = [v for v in full.colvars if v in longs]
+
+    # short variables of E: collect them through a copy of E whose long variables are replaced by scalars
+    Es, stand_in = E, {}
+    for n, v in enumerate(longs):
+        stand_in[v] = O.Var((1 << 20) + n, 1, v.cat)
+        Es = Es.replace(v, stand_in[v])
+    if Es.dim != 1:
+        return None, None
+
+    class _All:
+        tagI = red.tagI
+        formula = O.Concat(post, Es)
+
+    small = VarLayout(_All)
+    small_rows = [v for v in small.rowvars if v not in stand_in.values()]
+    small_cols = [v for v in small.colvars if v not in stand_in.values()]
+    names, dimx, dimy = {}, 0, 0
+    for group, arr in ((small_rows, "xi"), (small_cols, "yj"), (small.parvars, "p")):
+        off = 0
+        for v in group:
+            for k in range(v.dim):
+                names[(v.cat, v.ind, k)] = f"{arr}[{off + k}]"
+            off += v.dim
+        if arr == "xi":
+            dimx = off
+        elif arr == "yj":
+            dimy = off
+    dimp = small.dimp
+    for n, v in enumerate(row_long):
+        names[(v.cat, stand_in[v].ind, 0)] = f"xl[{n}]"
+    for n, v in enumerate(col_long):
+        names[(v.cat, stand_in[v].ind, 0)] = f"yl[{n}]"
+    names[(3, svar.ind, 0)] = "s"
+    pragma = ["    #pragma clang fp contract(off)"] if exact else []
+    Le = Lir(row_cat=red.tagI, fast_math=use_fast_math, dtype=dtype, exact_order=exact)
+    e_lines, e_exprs = Le.emit(lower(Es, Le), names, indent="    ")
+    Lp = Lir(row_cat=red.tagI, fast_math=use_fast_math, dtype=dtype, exact_order=exact)
+    p_outs = lower(post, Lp)
+    p_lines, p_exprs = Lp.emit(p_outs, names, indent="    ")
+    uses_yj = any(v.cat == 1 - red.tagI for v in Es.variables if v not in stand_in.values())
+    dimy_pad = 0 if dimy == 0 else -(-dimy // vec) * vec
+    # columns per tile: their running sums live in registers, their long rows in LDS
+    per_col = (len(col_long) * dpad + dimy_pad) * sizeof_t
+    tile_j = 32
+    while tile_j > 4 and tile_j * per_col > 64 * 1024:
+        tile_j //= 2
+    if tile_j * per_col > 96 * 1024:
+        return None, None
+    # tables in the order of the full variable lists (the launcher's offsets follow it); long variables are flagged
+    def table(group, shorts):
+        args, dims, offs, flag, o = [], [], [], [], 0
+        for v in group:
+            args.append(v.ind)
+            dims.append(v.dim)
+            flag.append(int(v not in shorts))
+            offs.append(0 if v not in shorts else o)
+            o += v.dim if v in shorts else 0
+        return (args or [0]), (dims or [0]), (offs or [0]), (flag or [0])
+
+    ra, rd, ro, rl = table(full.rowvars, small_rows)
+    ca, cd, co, cl = table(full.colvars, small_cols)
+    pa, pd, po = VarLayout.table(full.parvars)
+    if [v for v in full.parvars] != [v for v in small.parvars]:
+        return None, None
+    meta = dict(scheme="conv", block=config.block_size, rows=1, tile_j=tile_j, dimred=red.dimred, dimout=red.dim,
+                sizeof_t=sizeof_t, sizeof_acc=8 if dtypeacc == "double" else 4, nrowvars=len(full.rowvars),
+                ncolvars=len(full.colvars), nparvars=len(full.parvars), nops=Lp.count_ops(p_outs), red_kind=red.kind,
+                vchunk=D)
+    src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
+           f"typedef {dtype} T;\ntypedef {dtypeacc} TACC;", '#include "keops_common.h"']
+    defs = dict(
+        KEOPS_NARGS=nargs, KEOPS_DIMX=dimx, KEOPS_DIMY=dimy, KEOPS_DIMY_PAD=dimy_pad, KEOPS_DIMP=dimp,
+        KEOPS_DIMFOUT=post.dim, KEOPS_DIMRED=red.dimred, KEOPS_DIMOUT=red.dim, KEOPS_RED_KIND=red.kind,
+        KEOPS_RED_KEEP=red.keep, KEOPS_RED_K=red.K, KEOPS_SUM_SCHEME=SUM_SCHEMES[sum_scheme],
+        KEOPS_BLOCK=config.block_size, KEOPS_ROWS=1, KEOPS_TILE_J=tile_j, KEOPS_UNROLL_J=1, KEOPS_LSE_GROUP=1,
+        KEOPS_NROWVARS=len(full.rowvars), KEOPS_NCOLVARS=len(full.colvars), KEOPS_NPARVARS=len(full.parvars),
+        KEOPS_VCHUNK=1, VCH_D=D, VCH_DPAD=dpad, VCH_NROW=len(row_long), VCH_NCOL=len(col_long), VCH_USES_YJ=int(uses_yj),
+    )
+    src += [f"#define {k} {v}" for k, v in defs.items()]
+    for name, vals in (("row_arg", ra), ("row_dim", rd), ("row_off", ro), ("row_long", rl), ("col_arg", ca), ("col_dim", cd),
+                       ("col_off", co), ("col_long", cl), ("par_arg", pa), ("par_dim", pd), ("par_off", po),
+                       ("vch_row", [full.rowvars.index(v) for v in row_long] or [0]),
+                       ("vch_col", [full.colvars.index(v) for v in col_long] or [0])):
+        src.append(f"static __device__ constexpr int keops_{name}[] = {_c_list(vals)};")
+    dx, dy, dp = max(1, dimx), max(1, dimy_pad), max(1, dimp)
+    nr, nc = max(1, len(row_long)), max(1, len(col_long))
+    src.append("// one component of the long sum: xl / yl hold that component of the long variables")
+    src.append("struct KeopsChunkFormula {")
+    src.append(f"  static __device__ __forceinline__ T eval(const T (&xl)[{nr}], const T (&yl)[{nc}], const T (&xi)[{dx}], "
+               f"const T (&yj)[{dy}], const T (&p)[{dp}]) {{")
+    src += pragma + e_lines
+    src.append(f"    return {e_exprs[0]};")
+    src.append("  }\n};")
+    src.append("// post-chunk formula: s is the value of the long sum")
+    src.append("struct KeopsFormula {")
+    src.append(f"  static __device__ __forceinline__ void eval(const T (&xi)[{dx}], const T (&yj)[{dy}], "
+               f"const T (&p)[{dp}], const T s, T (&fout)[{post.dim}]) {{")
+    src += pragma + p_lines
+    src += [f"    fout[{k}] = {e};" for k, e in enumerate(p_exprs)]
+    src.append("  }\n};")
+    src.append('#include "keops_conv.h"')
+    return "\n".join(src) + "\n", meta
+
+
 def match_knn_highdim(red, dtype, map_reduce_id, use_fast_math):
     """(mode, node, row variable, column variable) in match_chunk's format when ``red`` is a K-min family reduction
     of SqDist between an output-indexed and a reduced-index variable of more than 256 (the limit of the KNN
@@ -570,6 +725,12 @@ def get_keops_dll(
             use_chunk_mode = 1 if source is not None else 0
         else:
             source = None
+        if source is None and enable_chunks:
+            vch = match_vchunk(red)
+            if vch is not None:
+                source, meta = generate_vchunk_plugin(red, vch, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs,
+                                                      irregular=irregular)
+                use_chunk_mode = 1 if source is not None else 0
         if source is None:
             source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint,
                                            irregular=irregular)
