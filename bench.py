@@ -56,6 +56,11 @@ WORKLOADS = {
     "gauss_100k": ("Gaussian kernel sum 1e5 x 1e5, D=3, Dv=1, float32 (reference benchmarks/README.md:13)", 14, "valu"),
     # 2*D flop of the <x,y> contraction per pair (the matrix-core work); filter and re-rank are not counted
     "knn_d64": ("KMin_ArgKMin K=10, 1e5 queries x 1e6 references, D=64 (benchmark configuration 3)", 128, "mfma"),
+    # nearest neighbours among MNIST-sized rows (784 components): squared distances on the chunked matrix-core
+    # sweep + exact re-rank (2*D flop of the contraction per pair), Manhattan distances on the vector-ALU chunked
+    # variant of the general-purpose kernel (subtract, absolute value, add per component)
+    "knn_d784": ("ArgKMin K=10 of SqDist, 1e4 queries x 6e4 references, D=784", 1568, "mfma"),
+    "knn_l1_d784": ("ArgKMin K=10 of the L1 distance, 1e4 queries x 6e4 references, D=784", 2352, "valu"),
     "sparse_100x10k": ("block-sparse Gaussian sum, 100 clusters x 10,000 points (benchmark configuration 4)", 14, "valu"),
     "lse_b16": ("batched LogSumExp softmin B=16, 50,000 x 50,000, D=3 (benchmark configuration 5a)", 17, "valu"),
     # 2*D flop of the contraction + sqrt, neg, exp + 2*Dv of the weighted accumulation
@@ -85,6 +90,10 @@ def _np_inputs(name):
     if name == "knn_d64":
         M, N, D = 100_000, 1_000_000, 64
         rng = np.random.default_rng(2)
+        return dict(M=M, N=N, Dv=0, D=D, arrays=[rng.random((M, D), dtype=np.float32), rng.random((N, D), dtype=np.float32)])
+    if name in ("knn_d784", "knn_l1_d784"):
+        M, N, D = 10_000, 60_000, 784
+        rng = np.random.default_rng(7)
         return dict(M=M, N=N, Dv=0, D=D, arrays=[rng.random((M, D), dtype=np.float32), rng.random((N, D), dtype=np.float32)])
     if name == "softmax_d64":
         M = N = 65_536
@@ -128,6 +137,10 @@ def build_step(name):
     M, N, Dv = inp["M"], inp["N"], inp["Dv"]
     if name == "knn_d64":
         knn = Genred("SqDist(x,y)", ["x=Vi(64)", "y=Vj(64)"], reduction_op="KMin_ArgKMin", axis=1, opt_arg=10)
+        return (lambda: knn(*dev)), M * N, inp
+    if name in ("knn_d784", "knn_l1_d784"):
+        dist = "SqDist(x,y)" if name == "knn_d784" else "Sum(Abs(x-y))"
+        knn = Genred(dist, ["x=Vi(784)", "y=Vj(784)"], reduction_op="ArgKMin", axis=1, opt_arg=10)
         return (lambda: knn(*dev)), M * N, inp
     if name == "softmax_d64":
         att = Genred("(q|k)", ["q=Vi(64)", "k=Vj(64)", "v=Vj(64)"], reduction_op="SumSoftMaxWeight", axis=1, formula2="v")
