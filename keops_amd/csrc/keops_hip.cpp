@@ -732,7 +732,16 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   // workspace, a second kernel re-ranks them exactly into `out` and counts the rows it cannot certify
   const int64_t knn_inner = m.meta_int("chk_knn_inner", 0);
   if (knn_inner > 0 && (rg || final)) return fail(-1, "corrupt chunk module metadata");
-  const size_t o_lists = take(knn_inner > 0 ? (size_t)nx * 2 * knn_inner * 4 : 0), o_flag = take(knn_inner > 0 ? 256 : 0);
+  if (knn_inner > 0) {
+    // column slabs fill the chip (one workgroup per CU at these operand sizes); the re-rank gives one lane to every
+    // candidate of a row: at most 64 / knn_inner slabs
+    const int64_t cap = std::max<int64_t>(1, std::min<int64_t>(64 / knn_inner, ny / (16 * TJ)));
+    const int64_t n0 = std::max<int64_t>(1, std::min<int64_t>(cap, (m.cu_count + row_blocks - 1) / row_blocks));
+    nslabs = balance_slabs(row_blocks, n0, cap, m.cu_count);
+    slab_len = std::max<int64_t>(TJ, ((ny + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ);
+    nslabs = std::max<int64_t>(1, (ny + slab_len - 1) / slab_len);
+  }
+  const size_t o_lists = take(knn_inner > 0 ? (size_t)nslabs * nx * 2 * knn_inner * 4 : 0), o_flag = take(knn_inner > 0 ? 256 : 0);
   if (knn_inner > 0 && stream_is_capturing(stream))
     return fail(-1, "this K-nearest-neighbour launch reads a flag back from the device: it cannot be captured in a HIP graph");
   if (int rc = m.partial.reserve(off)) return rc;
@@ -753,7 +762,8 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (mode == 0) {
     if (int rc = launch_raw(m, "keops_chk_colsum", (unsigned)nparts, 1, 256, buf.data(), psize, stream)) return rc;
     const size_t szp = with_which(nparts);
-    if (int rc = launch_raw(m, "keops_chk_colsum_final", 1, 1, 256, buf.data(), szp, stream)) return rc;
+    const int64_t cw = D > 128 ? 256 : (D > 64 ? 128 : (D > 32 ? 64 : 32));  // CHK_CW: columns per workgroup
+    if (int rc = launch_raw(m, "keops_chk_colsum_final", (unsigned)((DP + cw - 1) / cw), 1, 256, buf.data(), szp, stream)) return rc;
   }
   const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
   size_t sz = with_which(0);
@@ -768,7 +778,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (final) {
     if (int rc = launch_raw(m, softmax ? "keops_chk_softmax" : "keops_chk_final", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)m.block, buf.data(), psize, stream)) return rc;
   } else {
-    if (int rc = launch_raw(m, "keops_chk_main", (unsigned)row_blocks, 1, (unsigned)m.block, buf.data(), psize, stream)) return rc;
+    if (int rc = launch_raw(m, "keops_chk_main", (unsigned)row_blocks, (unsigned)(knn_inner > 0 ? nslabs : 1), (unsigned)m.block, buf.data(), psize, stream)) return rc;
   }
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
   if (final && nslabs > 1) {
@@ -779,7 +789,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
     void* extra[3] = {ws + o_lists, out, ws + o_flag};  // struct ChkKnnExtra of kernels/keops_chunk_mfma.h
     std::memcpy(buf.data() + psize, extra, sizeof(extra));
     if (int rc = launch_raw(m, "keops_chk_knn_ymax", 1, 1, 256, buf.data(), psize + sizeof(extra), stream)) return rc;
-    if (int rc = launch_raw(m, "keops_chk_knn_rerank", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), psize + sizeof(extra), stream)) return rc;
+    if (int rc = launch_raw(m, "keops_chk_knn_rerank", (unsigned)((nx + 3) / 4), 1, 256, buf.data(), psize + sizeof(extra), stream)) return rc;
     if (int rc = ensure_pinned(m, 64)) return rc;
     HIP_TRY(hipMemcpyAsync(m.pinned, ws + o_flag, 4, hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipStreamSynchronize(stream));

@@ -95,7 +95,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum(const ChkPara
   const i64 rows_per_block = (P.nys + gridDim.x - 1) / gridDim.x;
   const i64 r0 = (i64)blockIdx.x * rows_per_block, r1 = keops_min(P.nys, r0 + rows_per_block);
   const T* y = P.arg[CHK_YARG];
-  for (int c0 = 0; c0 < CHK_DPAD; c0 += CHK_CW) {
+  for (int c0 = blockIdx.x * CHK_CW; c0 < CHK_DPAD; c0 += gridDim.x * CHK_CW) {
     const int c = c0 + cw;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     if (c < CHK_D) {
@@ -126,9 +126,17 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum_final(const C
   const int cw = threadIdx.x % CHK_CW, rg = threadIdx.x / CHK_CW;
   for (int c0 = 0; c0 < CHK_DPAD; c0 += CHK_CW) {
     const int c = c0 + cw;
-    float s = 0.f;
-    if (c < CHK_DPAD)
-      for (int b = rg; b < nparts; b += RG) s += P.colpart[(i64)b * CHK_DPAD + c];
+    // eight interleaved partial sums, added in a fixed order: the loads of one thread do not wait for each other
+    float s8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (c < CHK_DPAD) {
+      int b = rg;
+      for (; b + 7 * RG < nparts; b += 8 * RG) {
+#pragma unroll
+        for (int u = 0; u < 8; u++) s8[u] += P.colpart[(i64)(b + u * RG) * CHK_DPAD + c];
+      }
+      for (; b < nparts; b += RG) s8[0] += P.colpart[(i64)b * CHK_DPAD + c];
+    }
+    const float s = ((s8[0] + s8[1]) + (s8[2] + s8[3])) + ((s8[4] + s8[5]) + (s8[6] + s8[7]));
     part[threadIdx.x] = s;
     __syncthreads();
     if (rg == 0 && c < CHK_DPAD) {
@@ -256,8 +264,9 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
   G.rewind(P.rt);
   while (G.next(P.rt, jbeg, jend)) {
 #else
-  jbeg = 0;
-  jend = P.ny;
+  // (the K-nearest-neighbour variant cuts the reduced axis in slabs, one list of candidates per slab)
+  jbeg = (i64)blockIdx.y * P.slab_len;
+  jend = keops_min(P.ny, jbeg + P.slab_len);
   {
 #endif
   if (jbeg < jend) prefetch(jbeg, jend);
@@ -387,7 +396,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
       other.load_partial(merge_s[grp * 32 + col][k]);
       acc.merge(other);
     }
-    if (valid) acc.finalize(P.out + q * KEOPS_DIMOUT);
+    if (valid) acc.finalize(P.out + ((i64)blockIdx.y * P.nx + q) * KEOPS_DIMOUT);
   }
 }
 #endif
@@ -395,7 +404,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
 // ---- K nearest neighbours in high dimension: exact re-rank of the lists of the sweep -----------------
 //
 // CHK_KNN_K: the module serves a KMin-family reduction of SqDist(x, y) with K = CHK_KNN_K.  keops_chk_main keeps the
-// KEOPS_RED_K > K smallest *approximate* squared distances per row (split bfloat16 operands: |approx - d| <=
+// KEOPS_RED_K > K smallest *approximate* squared distances per row and column slab (split bfloat16 operands: |approx - d| <=
 // CHK_KNN_C (|x^|^2 + |y^|^2) for the centred rows x^, y^) in the reference's (value, index) list layout.  Here
 // one lane per row computes the float32 distances of its candidates in the reference's operation order (sequential
 // sum of squared differences, no fused multiply-add), sorts them under (distance, index) and writes the K best.
@@ -405,7 +414,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
 #if defined(CHK_KNN_K)
 #define CHK_KNN_C 2.0e-4f
 struct ChkKnnExtra {
-  const float* lists;  // [nx][2 * KEOPS_RED_K] approximate (value, index) pairs of the sweep
+  const float* lists;  // [nslabs][nx][2 * KEOPS_RED_K] approximate (value, index) pairs of the sweep
   T* out;              // [nx][CHK_KNN_DIMOUT]
   int* flag;           // flag[0]: rows that are not certified; flag[1] (as float): max_j |y^_j|^2
 };
@@ -426,59 +435,62 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_knn_ymax(const ChkPa
   }
 }
 
+// One wavefront per row; lane c re-examines candidate c % KEOPS_RED_K of slab c / KEOPS_RED_K (the launcher keeps
+// nslabs * KEOPS_RED_K <= 64), ranks are counted across the lanes under (distance, index, lane).
 extern "C" __global__ void __launch_bounds__(256) keops_chk_knn_rerank(const ChkParams P, const ChkKnnExtra E) {
-  const i64 q = (i64)blockIdx.x * 256 + threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const i64 q = (i64)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (q >= P.nx) return;
   const float inf = __builtin_huge_valf();
-  const float* L = E.lists + q * 2 * KEOPS_RED_K;
+  const int ncand = P.nslabs * KEOPS_RED_K;
+  const int slab = lane / KEOPS_RED_K, entry = lane - slab * KEOPS_RED_K;
   const T* xq = P.arg[CHK_XARG] + q * CHK_D;
-  float bd[CHK_KNN_K];
-  int bj[CHK_KNN_K];
-#pragma unroll
-  for (int l = 0; l < CHK_KNN_K; l++) {
-    bd[l] = inf;
-    bj[l] = 0;
-  }
-  float a_last = inf;
-  for (int c = 0; c < KEOPS_RED_K; c++) {
-    const float a = L[2 * c];
-    a_last = a;
-    if (!(a < inf)) break;  // fewer references than list entries: nothing was left out
-    const int j = (int)L[2 * c + 1];
-    const T* yr = P.arg[CHK_YARG] + (i64)j * CHK_D;
-    float d = 0.f;
-    {
+  float a = inf, d = inf;
+  int j = 0x7fffffff;
+  if (lane < ncand) {
+    const float* L = E.lists + ((i64)slab * P.nx + q) * 2 * KEOPS_RED_K;
+    a = L[2 * entry];
+    if (a < inf) {
+      j = (int)L[2 * entry + 1];
+      const T* yr = P.arg[CHK_YARG] + (i64)j * CHK_D;
+      float t = 0.f;
+      {
 #pragma clang fp contract(off)
-      for (int k = 0; k < CHK_D; k++) {
-        const float t = xq[k] - yr[k];
-        d = d + t * t;
+        for (int k = 0; k < CHK_D; k++) {
+          const float u = xq[k] - yr[k];
+          t = t + u * u;
+        }
       }
+      d = t;
     }
-    // sorted insertion under (distance, index)
-    bool before_cur = d < bd[CHK_KNN_K - 1] || (d == bd[CHK_KNN_K - 1] && j < bj[CHK_KNN_K - 1]);
+  }
+  // what was left out of slab s has an approximate distance >= the last entry of its list (inf: nothing left out)
+  float a_last = (lane < ncand && entry == KEOPS_RED_K - 1) ? a : inf;
 #pragma unroll
-    for (int l = CHK_KNN_K - 1; l > 0; l--) {
-      const bool before_prev = d < bd[l - 1] || (d == bd[l - 1] && j < bj[l - 1]);
-      bd[l] = before_prev ? bd[l - 1] : (before_cur ? d : bd[l]);
-      bj[l] = before_prev ? bj[l - 1] : (before_cur ? j : bj[l]);
-      before_cur = before_prev;
-    }
-    bd[0] = before_cur ? d : bd[0];
-    bj[0] = before_cur ? j : bj[0];
+  for (int o = 32; o > 0; o >>= 1) a_last = __builtin_fminf(a_last, __shfl_xor(a_last, o));
+  int rank = 0;
+  for (int c = 0; c < ncand; c++) {
+    const float dc = __shfl(d, c);
+    const int jc = __shfl(j, c);
+    rank += (dc < d || (dc == d && (jc < j || (jc == j && c < lane)))) ? 1 : 0;
   }
   T* o = E.out + q * CHK_KNN_DIMOUT;
-#pragma unroll
-  for (int l = 0; l < CHK_KNN_K; l++) {
+  if (lane < ncand && rank < CHK_KNN_K) {
+    const T jv = d < inf ? (T)j : (T)0;
     if (CHK_KNN_KEEP == 0) {
-      o[2 * l] = bd[l];
-      o[2 * l + 1] = (T)bj[l];
+      o[2 * rank] = d;
+      o[2 * rank + 1] = jv;
     } else {
-      o[l] = CHK_KNN_KEEP == 1 ? bd[l] : (T)bj[l];
+      o[rank] = CHK_KNN_KEEP == 1 ? (T)d : jv;
     }
   }
-  if (a_last < inf) {
+  // K-th exact distance: held by the lane of rank K - 1
+  float dk = (lane < ncand && rank == CHK_KNN_K - 1) ? d : -inf;
+#pragma unroll
+  for (int o2 = 32; o2 > 0; o2 >>= 1) dk = __builtin_fmaxf(dk, __shfl_xor(dk, o2));
+  if (lane == 0 && a_last < inf) {
     const float eps = CHK_KNN_C * (P.xn[q] + reinterpret_cast<const float*>(E.flag)[1]);
-    if (!((a_last - eps) * (1.0f - 1.0e-4f) > bd[CHK_KNN_K - 1])) atomicAdd(E.flag, 1);
+    if (!((a_last - eps) * (1.0f - 1.0e-4f) > dk)) atomicAdd(E.flag, 1);
   }
 }
 #endif
