@@ -15,6 +15,8 @@ import math
 from .lir import Lir
 
 
+import copy as _copy
+
 class FormulaError(ValueError):
     """Raised for ill-formed formulas (mirrors KeOps_Error -> ValueError in the reference)."""
 
@@ -73,6 +75,42 @@ class Op:
             return self
         kids = [c.replace(old, new) for c in self.children]
         return self.rebuild(kids)
+
+    def substitute(self, mapping, memo=None):
+        """Replace several sub-formulas at once (``mapping``: old -> new) in one traversal; shared sub-trees are
+        rebuilt once."""
+        if memo is None:
+            memo = {}
+        r = mapping.get(self)
+        if r is not None:
+            return r
+        if not self.children:
+            return self
+        r = memo.get(id(self))
+        if r is None:
+            kids = [c.substitute(mapping, memo) for c in self.children]
+            r = self if all(k is c for k, c in zip(kids, self.children)) else self.rebuild(kids)
+            memo[id(self)] = r
+        return r
+
+    def rename_vars(self, mapping, memo=None):
+        """Copy of this tree with variables renamed (``mapping``: Var -> Var of the same dimension and category,
+        injective).  A pure renaming cannot enable or undo a simplification, so nodes are cloned without going
+        through the simplifying constructors."""
+        if memo is None:
+            memo = {}
+        if not self.children:
+            return mapping.get(self, self)
+        r = memo.get(id(self))
+        if r is None:
+            kids = tuple(c.rename_vars(mapping, memo) for c in self.children)
+            if all(k is c for k, c in zip(kids, self.children)):
+                r = self
+            else:
+                r = _copy.copy(self)
+                r.children, r._hash, r._vars = kids, None, None
+            memo[id(self)] = r
+        return r
 
     def rebuild(self, kids):
         """Re-create this node over new children through the simplifying constructor."""

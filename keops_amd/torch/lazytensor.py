@@ -38,6 +38,9 @@ def _broadcast_batch(a, b):
     return tuple(out)
 
 
+_genred_cache = {}
+
+
 class LazyTensor:
     """Symbolic wrapper for torch tensors (see the module docstring)."""
 
@@ -503,10 +506,8 @@ class LazyTensor:
             k += 1
 
         def settle(f):
-            for v in f.variables:
-                if v.ind in pos:
-                    f = f.replace(v, O.Var(pos[v.ind], v.dim, v.cat))
-            return f
+            moved = {v: O.Var(pos[v.ind], v.dim, v.cat) for v in f.variables if v.ind in pos and pos[v.ind] != v.ind}
+            return f.rename_vars(moved) if moved else f
 
         formula = settle(self.formula)
         formula2 = None if other is None else settle(other.formula)
@@ -529,8 +530,19 @@ class LazyTensor:
             def fn(*args, **kw):
                 return solver(*args, **solve_kw, **kw)
         else:
-            fn = Genred(repr(formula), aliases, reduction_op=reduction_op, axis=axis, opt_arg=opt_arg,
-                        formula2=None if formula2 is None else repr(formula2), **init_kw)
+            # one Genred object per (formula, options): iterative algorithms rebuild the same LazyTensor every pass
+            f1, f2 = repr(formula), None if formula2 is None else repr(formula2)
+            key = (f1, f2, tuple(aliases), reduction_op, axis, opt_arg, tuple(sorted(init_kw.items())))
+            try:
+                fn = _genred_cache.get(key)
+            except TypeError:  # unhashable option value
+                key, fn = None, None
+            if fn is None:
+                fn = Genred(f1, aliases, reduction_op=reduction_op, axis=axis, opt_arg=opt_arg, formula2=f2, **init_kw)
+                if key is not None:
+                    if len(_genred_cache) >= 512:
+                        _genred_cache.clear()
+                    _genred_cache[key] = fn
         data = [None] * nvars
         cats = {v.ind: v.cat for f in (formula,) + (() if formula2 is None else (formula2,)) for v in f.variables}
         dev = next((t.device for t in whole.variables.values() if isinstance(t, torch.Tensor)), None)
