@@ -280,3 +280,30 @@ def test_attention_backward_uses_chunked_reductions():
                                      [e.double(), torch.ones(M, 1, dtype=torch.float64)])
     for got, ref in ((gq, rq), (gk, rk), (gv, rv)):
         assert rel_l2(got.cpu().numpy(), ref.numpy()) < 3e-5, rel_l2(got.cpu().numpy(), ref.numpy())
+
+
+def test_point_gradient_formula_with_block_sparse_ranges_and_out():
+    """The formula g_ij (x_i - y_j) written by hand, with block-sparse ranges and a preallocated output: the
+    scalar and weighted chunked reductions both receive the ranges."""
+    from keops_amd import keops_io
+    from keops_amd.torch import Genred
+
+    M, N, D = 600, 800, 72
+    gen = torch.Generator().manual_seed(21)
+    x, y = torch.randn(M, D, generator=gen) / D ** 0.5, torch.randn(N, D, generator=gen) / D ** 0.5
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device="cuda")
+    ranges = (i64([[0, 250], [250, 600]]), i64([1, 3]), i64([[0, 300], [100, 500], [500, 800]]),
+              i64([[0, 300], [100, 500], [500, 800]]), i64([1, 2, 3]), i64([[0, 250], [250, 600], [250, 600]]))
+    keops_io._loaders.clear()
+    fn = Genred("Exp(-SqDist(x,y))*(x-y)", [f"x=Vi({D})", f"y=Vj({D})"], reduction_op="Sum", axis=1)
+    out = torch.empty(M, D, device="cuda")
+    res = fn(x.cuda(), y.cuda(), ranges=ranges, out=out)
+    assert res.data_ptr() == out.data_ptr()
+    assert any(ld.plan is not None for ld in keops_io._loaders.values())
+    mask = torch.zeros(M, N, dtype=torch.bool)
+    mask[:250, :300] = True
+    mask[250:, 100:] = True
+    x64, y64 = x.double(), y.double()
+    K = torch.exp(-torch.cdist(x64, y64) ** 2) * mask
+    ref = x64 * K.sum(1, keepdim=True) - K @ y64
+    assert rel_l2(out.cpu().numpy(), ref.numpy()) < 2e-5
