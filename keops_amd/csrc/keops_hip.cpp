@@ -303,6 +303,7 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
   const int nb = S.nbatchdims;
   const int nvars = by_arg ? m.nargs : m.nrowvars + m.ncolvars + m.nparvars;
   std::vector<int64_t> synth;  // batch mode: [slices (nbatches)] [ranges_y (2*nbatches)]
+  std::vector<int64_t> range_work;  // block-sparse mode: reduced rows per row range
 
   if (user_ranges) {
     const int sel = tagI == 0 ? 0 : 3;
@@ -316,7 +317,25 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
                       "captured in a HIP graph");
     // same synchronous read-back as the reference (keops_nvrtc.cpp:195-197)
     if (nranges) HIP_TRY(hipMemcpyAsync(rx_host.data(), rx_dev, sizeof(int64_t) * 2 * nranges, hipMemcpyDeviceToHost, stream));
+    // the slices and reduced ranges too: workgroups are issued longest first (below)
+    const int64_t nred = ranges[6][sel + 2];
+    std::vector<int64_t> sl_host((size_t)nranges), ry_host((size_t)2 * std::max<int64_t>(0, nred));
+    if (nranges && ranges[6][sel + 1] == nranges && nred > 0) {
+      HIP_TRY(hipMemcpyAsync(sl_host.data(), slices_dev, sizeof(int64_t) * nranges, hipMemcpyDeviceToHost, stream));
+      HIP_TRY(hipMemcpyAsync(ry_host.data(), ry_dev, sizeof(int64_t) * 2 * nred, hipMemcpyDeviceToHost, stream));
+    } else {
+      sl_host.clear();
+    }
     HIP_TRY(hipStreamSynchronize(stream));
+    if (!sl_host.empty()) {
+      // reduced rows swept by the workgroups of every row range
+      range_work.assign((size_t)nranges, 0);
+      for (int64_t r = 0; r < nranges; r++) {
+        const int64_t a = r == 0 ? 0 : sl_host[r - 1], b = sl_host[r];
+        if (a < 0 || b < a || b > nred) return fail(-1, "slices of row range " + std::to_string(r) + " are out of bounds");
+        for (int64_t k = a; k < b; k++) range_work[r] += std::max<int64_t>(0, ry_host[2 * k + 1] - ry_host[2 * k]);
+      }
+    }
   } else {
     // block-diagonal pattern, one range per batch (Ranges.h:40-86)
     nranges = S.nbatches;
@@ -362,8 +381,16 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
     int64_t* lk = (int64_t*)m.pinned;
     int64_t* off = lk + n_lookup;
     int64_t* syn = off + n_off;
+    // Workgroups start in table order.  Block-sparse patterns give them very different amounts of work: the row
+    // ranges with the longest sweeps go first, so that the last workgroups to start are the short ones and the
+    // chip does not idle behind a few long stragglers.
+    std::vector<int64_t> order((size_t)nranges);
+    for (int64_t r = 0; r < nranges; r++) order[r] = r;
+    if (!range_work.empty())
+      std::stable_sort(order.begin(), order.end(), [&](int64_t a, int64_t b) { return range_work[a] > range_work[b]; });
     int64_t idx = 0;
-    for (int64_t r = 0; r < nranges; r++) {
+    for (int64_t ro = 0; ro < nranges; ro++) {
+      const int64_t r = order[ro];
       const int64_t s = rx_host[2 * r], len = rx_host[2 * r + 1] - s;
       for (int64_t j = 0; j < len; j += rows_per_block) {
         lk[3 * idx] = r;
