@@ -80,8 +80,8 @@ void keops_hip_module_destroy(void* module);
  * Returns 0 or a hipError_t / negative library code.  KEOPS_HIP_NOT_CERTIFIED: a K-nearest-neighbour module for
  * vectors of more than 256 components ranks candidates found with reduced-precision products; when ties or
  * near-ties at the K-th distance keep it from proving that no reference was left out, it returns this code, `out`
- * is not valid and the caller runs the same call on a module compiled without the chunked schemes
- * (enable_chunks = 0), as keops_amd/keops_io.py does.  No counterpart in the reference, whose chunked kernels
+ * is not valid and the caller runs the same call on a module compiled without the matrix-core schemes,
+ * as keops_amd/keops_io.py does.  No counterpart in the reference, whose chunked kernels
  * (GpuReduc1D_chunks.py) accumulate in float32.
  */
 #define KEOPS_HIP_NOT_CERTIFIED (-7)

@@ -443,7 +443,7 @@ def plan_row_col_product(red, dtype, use_fast_math, enable_chunks):
     with sign, G (the scalar formula), row / col (the variables) and their coefficients a, c."""
     from .formulas import ops as O
 
-    if not enable_chunks or not isinstance(red, Sum_Reduction) or dtype != "float" or not use_fast_math:
+    if not enable_chunks or enable_chunks < 0 or not isinstance(red, Sum_Reduction) or dtype != "float" or not use_fast_math:
         return None
     F, sign = red.formula, 1
     while F.name == "Minus":
@@ -684,7 +684,7 @@ def get_keops_dll(
         # only the bucket matters for the cache key
         rows_hint = nx if nx < 64 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
-           use_fast_math, _rows_bucket(rows_hint), bool(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs),
+           use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs),
            binder.templates_digest())
     with _lock:
         hit = _cache.get(key)
@@ -705,11 +705,14 @@ def get_keops_dll(
 
             cls = KMin_ArgKMin_Reduction if red.keep == KEEP_BOTH else (KMin_Reduction if red.keep == KEEP_VAL else ArgKMin_Reduction)
             red_k = cls(red.formula, 1, red.tagI)
-        knn = match_knn_sqdist(red_k, dtype, map_reduce_id, batch_loop, pairs) if enable_chunks else None
-        knn_hd = match_knn_highdim(red_k, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
-        chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (enable_chunks and knn is None) else None
+        # enable_chunks: 1 every scheme, 0 the general-purpose kernel only, -1 no matrix-core scheme (exact float32
+        # arithmetic in the reference's order) but the vector-ALU chunked variant for long sums
+        mc = int(enable_chunks) > 0
+        knn = match_knn_sqdist(red_k, dtype, map_reduce_id, batch_loop, pairs) if mc else None
+        knn_hd = match_knn_highdim(red_k, dtype, map_reduce_id, use_fast_math) if (mc and knn is None) else None
+        chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (mc and knn is None) else None
         fin = None
-        if enable_finalchunks and knn is None and chk is None:
+        if enable_finalchunks and mc and knn is None and chk is None:
             fin = match_final(red, dtype, dtypeacc, sum_scheme_string, map_reduce_id)
         if knn is not None:
             source, meta = generate_knn_plugin(red_k, knn[0], knn[1], nargs)

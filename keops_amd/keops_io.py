@@ -156,7 +156,7 @@ class LoadKeOps_hip:
             # high-dimensional K nearest neighbours with ties at the K-th distance: same call on the exact kernel
             if self._exact is None:
                 c = self._ctor
-                self._exact = LoadKeOps_hip(*c[:10], dict(c[10], enable_chunks=0), nx=c[11])
+                self._exact = LoadKeOps_hip(*c[:10], dict(c[10], enable_chunks=-1), nx=c[11])
             return self._exact.genred_pytorch(device_args, ranges, nx, ny, nbatchdims, out, *args)
         del keep
         return out

@@ -269,7 +269,8 @@ def test_knn_beyond_256_components_ties_fall_back_to_the_exact_kernel():
     y = np.tile(rng.random((60, D), dtype=np.float32), (20, 1))
     idx = _knn(D, K, "ArgKMin")(*to_dev(x, y)).cpu().numpy()
     (ld,) = keops_io._loaders.values()
-    assert ld.module.meta("chk_knn") == str(K) and ld._exact is not None and ld._exact.module.meta("scheme") == "conv"
+    assert ld.module.meta("chk_knn") == str(K) and ld._exact is not None
+    assert ld._exact.module.meta("scheme") == "conv" and ld._exact.module.meta("vchunk") == str(D)
     assert np.array_equal(idx.astype(np.int64), np.argsort(_sequential_sqdist(x, y), axis=1, kind="stable")[:, :K])
 
 
