@@ -218,10 +218,17 @@ def match_vchunk(red):
         return isinstance(node, O.Elementwise) and node.dim in (1, D) and all(elementwise(c, D) for c in node.children)
 
     found = []
+    exact = red.kind in (KIND_MIN, KIND_MAX, KIND_KMIN)
     for node in red.formula.walk():
-        if node.name == "Sum" and node.children[0].dim > config.vchunk_min_dim and node not in [f[0] for f in found]:
-            E = node.children[0]
-            if elementwise(E, E.dim):
+        if node.children and node.children[0].dim > config.vchunk_min_dim and node not in [f[0] for f in found]:
+            E = None
+            if node.name == "Sum":
+                E = node.children[0]
+            elif node.name == "Scalprod" and not exact:
+                # (a|b) = Sum(a*b); index-carrying reductions keep the reference's fused multiply-add chain
+                # (Scalprod.py:32-36) on the general-purpose kernel
+                E = O.Mult(node.children[0], node.children[1])
+            if E is not None and E.dim == node.children[0].dim and elementwise(E, E.dim):
                 found.append((node, E))
     if len(found) != 1:
         return None

@@ -89,3 +89,25 @@ def test_weighted_long_sum_with_batch_dimensions_and_logsumexp():
     dense = -(((x.double()[:, :, None, :] - y.double()[:, None, :, :]).abs() * w.double()[:, :, None, :]).sum(-1)) * 0.3
     ref = torch.logsumexp(dense, dim=1)
     assert float((out - ref).abs().max()) < 2e-5 * float(ref.abs().max())
+
+
+def test_long_scalar_products_float64_and_transformed():
+    """(a|b) is Sum(a*b): a float64 linear kernel and Sum(Exp(x*y)*z), which the engine rewrites as a scalar
+    product with an elementwise operand."""
+    from keops_amd.torch import Genred
+
+    M, N, D = 260, 340, 300
+    gen = torch.Generator().manual_seed(8)
+    x, y, z = (torch.randn(n, D, generator=gen, dtype=torch.float64) / D ** 0.5 for n in (M, N, N))
+    b = torch.randn(N, 2, generator=gen, dtype=torch.float64)
+    lin = Genred("(x|y)*b", [f"x=Vi({D})", f"y=Vj({D})", "b=Vj(2)"], reduction_op="Sum", axis=1)
+    out = lin(x.cuda(), y.cuda(), b.cuda()).cpu()
+    assert _last_module().meta("vchunk") == str(D)
+    ref = (x @ y.T) @ b
+    assert float((out - ref).abs().max()) < 1e-12 * float(ref.abs().max())
+    f32 = lambda t: t.float().cuda()
+    tr = Genred("Sum(Exp(x*y)*z)", [f"x=Vi({D})", f"y=Vj({D})", f"z=Vj({D})"], reduction_op="Sum", axis=1)
+    out2 = tr(f32(x), f32(y), f32(z)).cpu().double()
+    assert _last_module().meta("vchunk") == str(D)
+    ref2 = (torch.exp(x[:, None, :] * y[None, :, :]) * z[None, :, :]).sum(-1).sum(1, keepdim=True)
+    assert float((out2 - ref2).abs().max()) < 1e-5 * float(ref2.abs().max())
