@@ -240,20 +240,25 @@ template <typename A> struct KeopsAcc {
         idx[k][l] = 0;
       }
   }
+  // entry l becomes old[l-1] when the candidate goes before old[l-1], the candidate when it goes before old[l]
+  // only, and stays otherwise: one compare per entry, shared by two neighbours, and for float32 values the new
+  // entry is the median of (candidate, old[l-1], old[l]) in one instruction
+  static __device__ __forceinline__ float mid(float x, float a, float b, bool, bool) { return __builtin_amdgcn_fmed3f(x, a, b); }
+  static __device__ __forceinline__ double mid(double x, double a, double b, bool before_a, bool before_b) {
+    return before_a ? a : (before_b ? x : b);
+  }
   __device__ __forceinline__ void insert(int k, A x, int j) {
     if (x < v[k][KEOPS_RED_K - 1]) {
-      v[k][KEOPS_RED_K - 1] = x;
-      idx[k][KEOPS_RED_K - 1] = j;
+      bool before_cur = true;
 #pragma unroll
       for (int l = KEOPS_RED_K - 1; l > 0; l--) {
-        const bool sw = v[k][l] < v[k][l - 1];
-        const A a = v[k][l], b = v[k][l - 1];
-        const int ia = idx[k][l], ib = idx[k][l - 1];
-        v[k][l - 1] = sw ? a : b;
-        v[k][l] = sw ? b : a;
-        idx[k][l - 1] = sw ? ia : ib;
-        idx[k][l] = sw ? ib : ia;
+        const bool before_prev = x < v[k][l - 1];
+        idx[k][l] = before_prev ? idx[k][l - 1] : (before_cur ? j : idx[k][l]);
+        v[k][l] = mid(x, v[k][l - 1], v[k][l], before_prev, before_cur);
+        before_cur = before_prev;
       }
+      idx[k][0] = before_cur ? j : idx[k][0];
+      v[k][0] = before_cur ? x : v[k][0];
     }
   }
   __device__ __forceinline__ void push(const T (&f)[KEOPS_FD], i64 j) {
