@@ -53,7 +53,7 @@ knn_sample_qsets = int(os.environ.get("KEOPS_AMD_KNN_SQSETS", 1))   # and 32-que
 vchunk_min_dim = int(os.environ.get("KEOPS_AMD_VCHUNK_MIN_DIM", 100))   # long elementwise sums beyond this many components keep their rows in memory
 min_as_kmin = int(os.environ.get("KEOPS_AMD_MIN_AS_KMIN", 1))        # Min / ArgMin of SqDist on the KNN schemes (K = 1)
 knn_highdim_margin = int(os.environ.get("KEOPS_AMD_KNN_HD_MARGIN", 6))   # extra approximate candidates kept per row by the high-dimensional KNN sweep
-knn_min_work = int(os.environ.get("KEOPS_AMD_KNN_MIN_WORK", 1 << 31))      # smallest pairs x max(D, 16) served by the matrix-core KNN scheme
+knn_min_work = int(os.environ.get("KEOPS_AMD_KNN_MIN_WORK", 1 << 32))      # smallest pairs x max(D, 16) served by the matrix-core KNN scheme
 knn_batch_max = int(os.environ.get("KEOPS_AMD_KNN_BATCH_MAX", 64))    # batched KNN: at most this many batches are served one by one
 knn_batch_min_work = int(os.environ.get("KEOPS_AMD_KNN_BATCH_MIN_WORK", 1 << 33))  # ... of at least this many pairs x max(D, 8) each
 knn_lds_budget = 150 * 1024                                        # LDS bytes a KNN workgroup may use (160 KB per CU)

@@ -211,7 +211,7 @@ def test_small_problem_stays_on_the_general_purpose_kernel(monkeypatch):
     general-purpose kernel."""
     from keops_amd import config, keops_io
 
-    monkeypatch.setattr(config, "knn_min_work", 1 << 31)
+    monkeypatch.setattr(config, "knn_min_work", 1 << 32)
     x, y = np.random.default_rng(3).random((2, 900, 64), dtype=np.float32)
     idx = _knn(64, 10, "ArgKMin")(*to_dev(x, y)).cpu().numpy()
     assert not _uses_mfma_module() and len(keops_io._loaders) == 1
