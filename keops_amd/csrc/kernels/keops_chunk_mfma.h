@@ -186,6 +186,53 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
   if (CHK_MODE == 0 && live && q == 0) (which ? P.yn : P.xn)[row] = nrm;
 }
 
+// Squared distances come out of the expansion |x^|^2 + |y^|^2 - 2 <x^, y^> with 16-bit operands: an absolute error
+// of about 2^-17 (|x^|^2 + |y^|^2), harmless unless the pair is close compared with the norms (identical or
+// neighbouring points, kernels much narrower than the cloud), where it would be a large relative error.  A value
+// below 1/8 of the sum of the squared norms is therefore recomputed from the float32 rows.  In high dimension
+// random pairs never come that close, so the branch costs one compare; clustered data pay for their accuracy.
+#ifndef CHK_NEAR
+#define CHK_NEAR 0.125f
+#endif
+// near_bound: CHK_NEAR (xn + largest yn of the staged tile), the only test on the common path.
+__device__ __forceinline__ float chk_near_bound(const float* yn_s, float xn, int col) {
+  float m = yn_s[col];
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) m = __builtin_fmaxf(m, __shfl_xor(m, o));
+  return CHK_NEAR * (xn + m);
+}
+// sv[u]: squared distance of this lane's output row to reduced row 8*(v/4) + 4*half + v%4 of the tile, v = v0 + u,
+// from the expansion; entries that are small compared with the norms are replaced by the float32 value.
+template <int NV>
+__device__ __forceinline__ void chk_fix_near(const ChkParams& P, float (&sv)[NV], int v0, int half, int n, float xn,
+                                             const float* yn_s, float near_bound, i64 ix, i64 jy0) {
+  float m = sv[0];
+#pragma unroll
+  for (int u = 1; u < NV; u++) m = __builtin_fminf(m, sv[u]);
+  if (__builtin_expect(!__any(m < near_bound), 1)) return;
+  unsigned mask = 0u;
+#pragma unroll
+  for (int u = 0; u < NV; u++) {
+    const int v = v0 + u, r = 8 * (v >> 2) + 4 * half + (v & 3);
+    if (r < n && sv[u] < CHK_NEAR * (xn + yn_s[r])) mask |= 1u << u;
+  }
+  const T* x = P.arg[CHK_XARG] + ix * CHK_D;
+  while (mask != 0u) {
+    const int u0 = __ffs(mask) - 1;
+    mask &= mask - 1u;
+    const int v = v0 + u0, r = 8 * (v >> 2) + 4 * half + (v & 3);
+    const T* y = P.arg[CHK_YARG] + (jy0 + r) * CHK_D;
+    float d = 0.f;
+#pragma nounroll
+    for (int k = 0; k < CHK_D; k++) {
+      const float t = x[k] - y[k];
+      d = __builtin_fmaf(t, t, d);
+    }
+#pragma unroll
+    for (int u = 0; u < NV; u++) sv[u] = (u == u0) ? d : sv[u];
+  }
+}
+
 // ---- main kernel --------------------------------------------------------------------------------
 
 #if !(defined(CHK_FINAL) && CHK_FINAL) && !(defined(CHK_SOFTMAX) && CHK_SOFTMAX)
@@ -294,6 +341,8 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
     }
     __syncthreads();
     if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ, jend);
+    const float near_bound = CHK_MODE == 0 ? chk_near_bound(yn_s, xnq, col) : 0.f;
+    const i64 jy0 = G.col(CHK_YARG, j0);
 #if CHK_NC == 1
     if (!wave_live) continue;
 
@@ -353,13 +402,16 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
     KeopsAcc<T> tmp;
     tmp.init();
 #endif
+    float sq[CHK_VS];
+#pragma unroll
+    for (int vv = 0; vv < CHK_VS; vv++) sq[vv] = CHK_MODE == 0 ? __builtin_fmaxf(s[vv] + xnq, 0.f) : s[vv];
+    if (CHK_MODE == 0) chk_fix_near<CHK_VS>(P, sq, chunk * CHK_VS, half, n, xnq, yn_s, near_bound, qx, jy0);
 #pragma unroll
     for (int vv = 0; vv < CHK_VS; vv++) {
       const int v = chunk * CHK_VS + vv;
       const int r = 8 * (v >> 2) + 4 * half + (v & 3);
       if (r < n) {
-        T sv = s[vv];
-        if (CHK_MODE == 0) sv = __builtin_fmaxf(sv + xnq, 0.f);
+        T sv = sq[vv];
         T yj[CHK_DY];
         constexpr int VEC = 16 / sizeof(T);
         typedef T vecT __attribute__((ext_vector_type(VEC)));
@@ -799,6 +851,8 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
 #endif
     __syncthreads();
     if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ, jend);
+    const float near_bound = CHK_MODE == 0 ? chk_near_bound(yn_s, xnq, col) : 0.f;
+    const i64 jy0 = G.col(CHK_YARG, j0);
     if (!wave_live) continue;
 
     chk_f32x16 s;
@@ -821,14 +875,17 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
     }
+    float sq[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) sq[v] = CHK_MODE == 0 ? __builtin_fmaxf(s[v] + xnq, 0.f) : s[v];
+    if (CHK_MODE == 0) chk_fix_near<16>(P, sq, 0, half, n, xnq, yn_s, near_bound, qx, jy0);
 #if CHK_V3
     float gw[16];
 #endif
 #pragma unroll
     for (int v = 0; v < 16; v++) {
       const int r = 8 * (v >> 2) + 4 * half + (v & 3);
-      T sv = s[v];
-      if (CHK_MODE == 0) sv = __builtin_fmaxf(sv + xnq, 0.f);
+      T sv = sq[v];
       T yj[CHK_DY];
       constexpr int VEC = 16 / sizeof(T);
       typedef T vecT __attribute__((ext_vector_type(VEC)));
@@ -1022,6 +1079,8 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
 #endif
     __syncthreads();
     if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ, jend);
+    const float near_bound = CHK_MODE == 0 ? chk_near_bound(yn_s, xnq, col) : 0.f;
+    const i64 jy0 = G.col(CHK_YARG, j0);
     if (!wave_live) continue;
 
     chk_f32x16 s;
@@ -1044,13 +1103,16 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
     }
+    float sq[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) sq[v] = CHK_MODE == 0 ? __builtin_fmaxf(s[v] + xnq, 0.f) : s[v];
+    if (CHK_MODE == 0) chk_fix_near<16>(P, sq, 0, half, n, xnq, yn_s, near_bound, qx, jy0);
     // F' for the lane's 16 pairs (rows past the end: -inf, they weigh nothing) and the tile maximum
     float mx = ninf;
 #pragma unroll
     for (int v = 0; v < 16; v++) {
       const int r = 8 * (v >> 2) + 4 * half + (v & 3);
-      T sv = s[v];
-      if (CHK_MODE == 0) sv = __builtin_fmaxf(sv + xnq, 0.f);
+      T sv = sq[v];
       T yj[CHK_DY];
       constexpr int VEC = 16 / sizeof(T);
       typedef T vecT __attribute__((ext_vector_type(VEC)));

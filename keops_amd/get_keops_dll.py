@@ -425,7 +425,7 @@ def match_chunk(red, dtype, map_reduce_id, use_fast_math):
         if mode is None:
             continue
         a, b = pair
-        if isinstance(a, O.Var) and isinstance(b, O.Var) and a.dim == b.dim and 32 <= a.dim <= config.chunk_max_dim and {a.cat, b.cat} == {0, 1}:
+        if isinstance(a, O.Var) and isinstance(b, O.Var) and a.dim == b.dim and config.chunk_min_dim <= a.dim <= config.chunk_max_dim and {a.cat, b.cat} == {0, 1}:
             if node not in [f[1] for f in found]:
                 found.append((mode, node, a, b))
     if len(found) != 1:

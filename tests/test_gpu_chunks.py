@@ -307,3 +307,36 @@ def test_point_gradient_formula_with_block_sparse_ranges_and_out():
     K = torch.exp(-torch.cdist(x64, y64) ** 2) * mask
     ref = x64 * K.sum(1, keepdim=True) - K @ y64
     assert rel_l2(out.cpu().numpy(), ref.numpy()) < 2e-5
+
+
+@pytest.mark.parametrize("reduction", ["Sum", "LogSumExp"])
+def test_narrow_kernel_on_clustered_points_and_self_interaction(reduction):
+    """Tight clusters far apart and a kernel as narrow as a cluster, x = y: every pair that matters is close compared
+    with the norms, where the 16-bit expansion of |x - y|^2 alone would be off by 2^-17 of the squared norms (10 %
+    of the kernel value here).  Such pairs are recomputed from the float32 rows: parity as everywhere else."""
+    from keops_amd.torch import Genred
+
+    D, C, per = 64, 20, 100
+    gen = torch.Generator().manual_seed(31)
+    centres = torch.randn(C, D, generator=gen)
+    x = (centres[:, None, :] + 0.01 * torch.randn(C, per, D, generator=gen)).reshape(C * per, D)
+    b = torch.randn(C * per, 5, generator=gen)
+    g = torch.tensor([1.0 / (2 * 0.01 ** 2 * D)])                 # exp(-g s) ~ exp(-1) inside a cluster
+    xd = x.cuda()
+    x64 = x.double()
+    S = torch.cdist(x64, x64) ** 2
+    if reduction == "Sum":
+        conv = Genred("Exp(-g*SqDist(x,y))*b", [f"x=Vi({D})", f"y=Vj({D})", "b=Vj(5)", "g=Pm(1)"], reduction_op="Sum", axis=1)
+        out = conv(xd, xd, b.cuda(), g.cuda()).cpu()
+        assert _scheme_used("chunk")
+        K = torch.exp(-g.double() * S)
+        assert_sum_parity(out.numpy(), (K @ b.double()).numpy(), (K @ b.double().abs()).numpy())
+        # the diagonal alone: a kernel so narrow that only the self-interaction is left
+        conv1 = Genred("Exp(-g*SqDist(x,y))", [f"x=Vi({D})", f"y=Vj({D})", "g=Pm(1)"], reduction_op="Sum", axis=1)
+        ones = conv1(xd, xd, (1e4 * g).cuda()).cpu()
+        assert float((ones - 1).abs().max()) < 1e-5
+    else:
+        lse = Genred("-g*SqDist(x,y)", [f"x=Vi({D})", f"y=Vj({D})", "g=Pm(1)"], reduction_op="LogSumExp", axis=1)
+        out = lse(xd, xd, g.cuda()).cpu().double()[:, 0]
+        ref = torch.logsumexp(-g.double() * S, dim=1)
+        assert float((out - ref).abs().max()) < 1e-5 * max(1.0, float(ref.abs().max()))
