@@ -102,6 +102,11 @@ class LoadKeOps_hip:
     def _row_col_product(self, device_args, ranges, nx, ny, nbatchdims, out, *args):
         plan = self.plan
         row, col = args[plan["row"].ind], args[plan["col"].ind]
+        if plan["a"] == -plan["c"]:
+            # g (x - y) = g ((x - m) - (y - m)): with m the mean of y the two sums that are subtracted are as small
+            # as the cloud allows, which limits the cancellation when the pairs that matter are close
+            m = col.mean(dim=-2, keepdim=True)
+            row, col = row - m, col - m
         res = None
         if self.sub_slices:
             parts = [ld.genred_pytorch(device_args, ranges, nx, ny, nbatchdims, None, *args, col[..., c0:c1].contiguous())
