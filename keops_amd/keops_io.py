@@ -64,13 +64,16 @@ class LoadKeOps_hip:
             sub = lambda f, extra: LoadKeOps_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, f,
                                                  list(aliases) + extra, nargs + len(extra), dtype, lang, optional_flags,
                                                  nx=nx, batch_loop=batch_loop, pairs=pairs)
-            self.sub_scalar = sub(f"Sum_Reduction({plan['G']!r},{tagI})", []) if plan["a"] else None
-            self.sub_slices = []
+            self.sub_slices, self.ones_column = [], False
             if plan["c"]:
                 for c0 in range(0, D, width):
                     w = min(width, D - c0)
+                    # when the last slice has room, a column of ones rides along: its sum is sum_j g_ij
+                    if plan["a"] and c0 + w == D and w < width:
+                        self.ones_column, w = True, w + 1
                     v = f"Var({nargs},{w},{plan['col'].cat})"
-                    self.sub_slices.append((c0, c0 + w, sub(f"Sum_Reduction(Mult({plan['G']!r},{v}),{tagI})", [v])))
+                    self.sub_slices.append((c0, min(D, c0 + w), sub(f"Sum_Reduction(Mult({plan['G']!r},{v}),{tagI})", [v])))
+            self.sub_scalar = sub(f"Sum_Reduction({plan['G']!r},{tagI})", []) if (plan["a"] and not self.ones_column) else None
             p.tagI, p.tagZero, p.dim, p.dimred = tagI, 0, D, D
             p.device_id_request, p.nargs = device_id_request, nargs
             p.reduction_op, p.axis = "Sum_Reduction", 1 - tagI
@@ -107,17 +110,24 @@ class LoadKeOps_hip:
             # as the cloud allows, which limits the cancellation when the pairs that matter are close
             m = col.mean(dim=-2, keepdim=True)
             row, col = row - m, col - m
-        res = None
+        res = total = None
         if self.sub_slices:
-            parts = [ld.genred_pytorch(device_args, ranges, nx, ny, nbatchdims, None, *args, col[..., c0:c1].contiguous())
-                     for c0, c1, ld in self.sub_slices]
+            parts = []
+            for k, (c0, c1, ld) in enumerate(self.sub_slices):
+                v = col[..., c0:c1]
+                if self.ones_column and k == len(self.sub_slices) - 1:
+                    v = torch.cat([v, torch.ones_like(v[..., :1])], dim=-1)
+                parts.append(ld.genred_pytorch(device_args, ranges, nx, ny, nbatchdims, None, *args, v.contiguous()))
+            if self.ones_column:
+                total, parts[-1] = parts[-1][..., -1:], parts[-1][..., :-1]
             res = parts[0] if len(parts) == 1 else torch.cat(parts, dim=-1)
             if plan["sign"] * plan["c"] < 0:
-                res = res.neg_()
+                res = -res
         if self.sub_scalar is not None:
             total = self.sub_scalar.genred_pytorch(device_args, ranges, nx, ny, nbatchdims, None, *args)
+        if total is not None:
             if plan["sign"] * plan["a"] < 0:
-                total = total.neg_()
+                total = -total
             res = row * total if res is None else torch.addcmul(res, row, total)
         if out is None:
             return res

@@ -226,6 +226,7 @@ def test_gradients_wrt_points_as_scalar_and_weighted_sums(D, kernel):
     planned = [ld for ld in keops_io._loaders.values() if ld.plan is not None]
     assert len(planned) == 2 and all(ld.module is None for ld in planned)
     subs = [s for ld in planned for s in ([ld.sub_scalar] if ld.sub_scalar else []) + [t[2] for t in ld.sub_slices]]
+    assert all((ld.sub_scalar is None) == (ld.ones_column or kernel == "expdot") for ld in planned)
     assert subs and all(s.module.meta("scheme") == "chunk" for s in subs)
     x64, y64 = x.double().requires_grad_(True), y.double().requires_grad_(True)
     if kernel == "gauss":
