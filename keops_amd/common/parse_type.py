@@ -86,7 +86,8 @@ def get_optional_flags(reduction_op_internal, dtype_acc, use_double_acc, sum_sch
         )
     return dict(
         dtype_acc=dtype_acc, sum_scheme=sum_scheme, use_fast_math=1 if use_fast_math else 0,
-        enable_chunks=1 if enable_chunks else 0,
+        # False: no matrix-core scheme (exact float32 / float64 arithmetic); long sums still keep their rows in memory
+        enable_chunks=1 if enable_chunks else -1,
     )
 
 

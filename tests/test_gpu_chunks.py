@@ -36,7 +36,7 @@ def test_laplace_chunked_vs_oracle(M, N, D, Dv):
     ref = cpu_reduc("laplace", [x, y, b], M, N, Dv)
     scale = cpu_reduc("laplace", [x, y, np.abs(b)], M, N, Dv)
     assert_sum_parity(got, ref, scale)
-    # the un-chunked generic kernel (enable_chunks=False) is the same function
+    # without the matrix-core schemes (enable_chunks=False: exact float32 arithmetic) it is the same function
     plain = Genred("Exp(-Norm2(x-y))*b", [f"x=Vi({D})", f"y=Vj({D})", f"b=Vj({Dv})"], reduction_op="Sum", axis=1,
                    enable_chunks=False)(*to_dev(x, y, b)).cpu().numpy()
     assert_sum_parity(plain, ref, scale)
