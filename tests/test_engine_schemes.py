@@ -91,3 +91,31 @@ def test_modules_of_the_new_schemes_compile(formula, dtype, mode, key):
     with open(exact[1]) as f:
         head = f.readline()
     assert "scheme=conv" in head
+
+
+def test_lazytensor_settles_variables_in_one_pass_and_reuses_the_reduction_object():
+    """Data tensors get positions 0..n-1 in order of appearance (a pure renaming of the symbolic tree) and two
+    LazyTensors with the same formula and options share one Genred object."""
+    import torch
+
+    from keops_amd.formulas.ops import Exp, Sum, Var
+    from keops_amd.torch import LazyTensor
+    from keops_amd.torch import lazytensor as lt
+
+    f = Exp(-Sum((Var(7, 3, 0) - Var(9, 3, 1)) ** 2)) * Var(12, 2, 1)
+    g = f.rename_vars({Var(7, 3, 0): Var(0, 3, 0), Var(9, 3, 1): Var(1, 3, 1), Var(12, 2, 1): Var(2, 2, 1)})
+    assert repr(g) == repr(f).replace("Var(7,", "Var(0,").replace("Var(9,", "Var(1,").replace("Var(12,", "Var(2,")
+    assert [v.ind for v in g.variables] == [0, 1, 2] and [v.ind for v in f.variables] == [7, 9, 12]
+    assert f.rename_vars({}) is f
+
+    def build(x, y, b):
+        K = (-((LazyTensor(x[:, None, :]) - LazyTensor(y[None, :, :])) ** 2).sum(-1)).exp() * LazyTensor(b[None, :, :])
+        return K.sum(1, call=False)
+
+    lt._genred_cache.clear()
+    r1 = build(torch.zeros(5, 3), torch.zeros(7, 3), torch.zeros(7, 2))
+    n = len(lt._genred_cache)
+    r2 = build(torch.ones(6, 3), torch.ones(4, 3), torch.ones(4, 2))
+    assert n == 1 and len(lt._genred_cache) == 1 and callable(r1) and callable(r2)
+    (key,) = lt._genred_cache
+    assert key[0] == "Mult(Exp(Minus(Sum(Square(Subtract(Var(0,3,0),Var(1,3,1)))))),Var(2,2,1))"
