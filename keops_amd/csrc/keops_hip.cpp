@@ -558,7 +558,7 @@ int64_t knn_min_sample() {
   return v;
 }
 int64_t knn_two_phase_min_refs() {
-  static const int64_t v = [] { const char* e = getenv("KEOPS_HIP_KNN_TWO_PHASE_MIN"); return e ? std::max<int64_t>(1024, atoll(e)) : 32768; }();
+  static const int64_t v = [] { const char* e = getenv("KEOPS_HIP_KNN_TWO_PHASE_MIN"); return e ? std::max<int64_t>(1024, atoll(e)) : 16384; }();
   return v;
 }
 

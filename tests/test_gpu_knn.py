@@ -103,7 +103,7 @@ def test_knn_config3_query_subset():
                                      (1200, 33000, 7, 1)])
 def test_knn_low_dimension_split_operands(M, N, D, K):
     """Dense point clouds (D < 32): the filter uses hi + lo bf16 operands; results stay bit-identical
-    to the CPU oracle, in the two-phase schedule (N >= 32768, M >= 1024) and in the adaptive one."""
+    to the CPU oracle, in the two-phase schedule (N >= 16384, M >= 1024) and in the adaptive one."""
     rng = np.random.default_rng(11)
     x = rng.random((M, D)).astype(np.float32)
     y = rng.random((N, D)).astype(np.float32)
