@@ -300,3 +300,17 @@ def test_min_family_of_sqdist_runs_as_k_equal_one(D, scheme):
         else:
             assert np.array_equal(out[0].cpu().numpy()[:, 0], ref_v)
             assert np.array_equal(out[1].cpu().numpy()[:, 0].astype(np.int64), ref_i)
+
+
+def test_nearest_row_over_the_first_index_beyond_256_components():
+    """ArgMin over i (axis=0) at D = 300: the K = 1 member of the family on the chunked sweep with exact re-rank."""
+    from keops_amd import keops_io
+    from keops_amd.torch import Genred
+
+    M, N, D = 1500, 400, 300
+    rng = np.random.default_rng(5)
+    x, y = rng.random((M, D), dtype=np.float32), rng.random((N, D), dtype=np.float32)
+    out = Genred("SqDist(x,y)", [f"x=Vi({D})", f"y=Vj({D})"], reduction_op="ArgMin", axis=0)(*to_dev(x, y))
+    (ld,) = keops_io._loaders.values()
+    assert ld.module.meta("chk_knn") == "1"
+    assert np.array_equal(out.cpu().numpy()[:, 0].astype(np.int64), _sequential_sqdist(y, x).argmin(1))

@@ -111,3 +111,25 @@ def test_long_scalar_products_float64_and_transformed():
     assert _last_module().meta("vchunk") == str(D)
     ref2 = (torch.exp(x[:, None, :] * y[None, :, :]) * z[None, :, :]).sum(-1).sum(1, keepdim=True)
     assert float((out2 - ref2).abs().max()) < 1e-5 * float(ref2.abs().max())
+
+
+def test_long_sum_over_the_first_index_with_block_sparse_ranges():
+    """Reduction over i (axis=0) of an L1 kernel with block-sparse ranges: rows that no range covers give 0."""
+    from keops_amd.torch import Genred
+
+    M, N, D = 500, 640, 150
+    gen = torch.Generator().manual_seed(12)
+    x, y, e = torch.randn(M, D, generator=gen) / D, torch.randn(N, D, generator=gen) / D, torch.randn(M, 2, generator=gen)
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device="cuda")
+    # ranges_i, slices_i, redranges_j (for axis=1) and ranges_j, slices_j, redranges_i (used here, axis=0)
+    ranges = (i64([[0, 200], [200, 500]]), i64([1, 2]), i64([[0, 300], [300, 600]]),
+              i64([[0, 300], [300, 600]]), i64([1, 2]), i64([[0, 200], [200, 500]]))
+    fn = Genred("Exp(-Sum(Abs(x-y)))*e", [f"x=Vi({D})", f"y=Vj({D})", "e=Vi(2)"], reduction_op="Sum", axis=0)
+    out = fn(x.cuda(), y.cuda(), e.cuda(), ranges=ranges).cpu()
+    assert _last_module().meta("vchunk") == str(D)
+    mask = torch.zeros(M, N, dtype=torch.bool)
+    mask[:200, :300] = True
+    mask[200:, 300:600] = True
+    K = torch.exp(-torch.cdist(x.double(), y.double(), p=1)) * mask
+    assert rel_l2(out.numpy(), (K.T @ e.double()).numpy()) < 1e-5
+    assert torch.all(out[600:] == 0)
