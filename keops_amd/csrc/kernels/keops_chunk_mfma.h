@@ -288,6 +288,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
   }
   KeopsAcc<TACC> acc;
   acc.init();
+#if defined(CHK_KNN_K)
+  // K-nearest-neighbour sweep: the 2 * CHK_NC lanes of an output row keep separate candidate lists.  The row's
+  // KEOPS_RED_K-th smallest value overall cannot exceed the last entry of any of them, so the smallest of those last
+  // entries (exchanged through tau_s once per tile; an older value is only looser) screens the candidates of all:
+  // far fewer wave-wide list insertions than with each lane's own last entry.
+  __shared__ float tau_s[CHK_WAVES][32];
+  if (half == 0) tau_s[wave][col] = __builtin_huge_valf();
+  float tau_row = __builtin_huge_valf();
+#endif
 
   // software pipeline: tile t+1 travels to registers while tile t is consumed
   constexpr int CH = CHK_ROWBYTES / 16;
@@ -343,6 +352,10 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
     if (j0 + CHK_TJ < jend) prefetch(j0 + CHK_TJ, jend);
     const float near_bound = CHK_MODE == 0 ? chk_near_bound(yn_s, xnq, col) : 0.f;
     const i64 jy0 = G.col(CHK_YARG, j0);
+#if defined(CHK_KNN_K)
+#pragma unroll
+    for (int c = 0; c < CHK_NC; c++) tau_row = __builtin_fminf(tau_row, tau_s[grp * CHK_NC + c][col]);
+#endif
 #if CHK_NC == 1
     if (!wave_live) continue;
 
@@ -423,15 +436,26 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
         }
         T fout[KEOPS_DIMFOUT];
         KeopsFormula::eval(xi, yj, p, sv, fout);
-#if KEOPS_USE_TILE_TMP
+#if defined(CHK_KNN_K)
+        if (fout[0] < tau_row) acc.push(fout, j0 + r);
+#elif KEOPS_USE_TILE_TMP
         tmp.push(fout, j0 + r);
 #else
         acc.push(fout, j0 + r);
 #endif
       }
     }
-#if KEOPS_USE_TILE_TMP
+#if KEOPS_USE_TILE_TMP && !defined(CHK_KNN_K)
     acc.merge(tmp);
+#endif
+#if defined(CHK_KNN_K)
+    {
+      // last entry of this lane's list and of the partner lane (the other 16 reduced rows of the tile)
+      float mine = (float)acc.v[0][KEOPS_RED_K - 1];
+      mine = __builtin_fminf(mine, __shfl_xor(mine, 32));
+      tau_row = __builtin_fminf(tau_row, mine);
+      if (half == 0) tau_s[wave][col] = mine;
+    }
 #endif
   }
   }
