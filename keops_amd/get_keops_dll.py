@@ -577,6 +577,7 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
     elif softmax is not None:
         defs.update(KEOPS_DIMFOUT=full_post.dim, CHK_SOFTMAX=1, CHK_SM_ONE=softmax[2], CHK_FV_ARG=softmax[1].ind,
                     CHK_FV_DIM=softmax[1].dim, CHK_FNB=-(-softmax[1].dim // 32))
+    defs["CHK_NEAR"] = f"{float(config.chunk_near)!r}f"
     defs["CHK_SPLIT3"] = split3
     defs["CHK_PRESPLIT"] = int(config.chunk_presplit)
     src += [f"#define {k} {v}" for k, v in defs.items()]
