@@ -30,7 +30,7 @@ lse_group = int(os.environ.get("KEOPS_AMD_LSE_GROUP", 8))  # log-sum-exp: column
 # matrix-core chunked scheme (csrc/kernels/keops_chunk_mfma.h): wavefronts (32 output rows each) per workgroup
 chunk_waves = int(os.environ.get("KEOPS_AMD_CHUNK_WAVES", 8))
 chunk_presplit = os.environ.get("KEOPS_AMD_CHUNK_PRESPLIT", "1") != "0"  # dense launches: pre-split copy of the weights
-chunk_min_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MIN_DIM", 32))    # smallest contraction served by the matrix-core chunked scheme
+chunk_min_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MIN_DIM", 24))    # smallest contraction served by the matrix-core chunked scheme
 chunk_near = float(os.environ.get("KEOPS_AMD_CHUNK_NEAR", 0.125))     # squared distances below this fraction of |x|^2+|y|^2 are recomputed in float32 (0: never)
 chunk_max_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MAX_DIM", 1024))  # largest contraction served by the matrix-core chunked scheme
 

@@ -407,7 +407,7 @@ def generate_knn_highdim_plugin(red, match, nargs):
 def match_chunk(red, dtype, map_reduce_id, use_fast_math):
     """(mode, node, row variable, column variable) when the formula of a Sum / log-sum-exp reduction
     contains exactly one high-dimensional contraction SqDist(x_i, y_j) (mode 0) or <x_i, y_j> (mode 1)
-    between plain variables of dimension 32..1024 that appear nowhere else in the formula (the
+    between plain variables of dimension config.chunk_min_dim..config.chunk_max_dim (24..1024) that appear nowhere else in the formula (the
     reference's conditions, Chunkable_Op.py:20-41 and Chunk_Mode_Constants.py:56-60, with the
     matrix-core dimension range instead of its >= 146 threshold).  None otherwise."""
     from .formulas import ops as O

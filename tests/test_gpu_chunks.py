@@ -25,7 +25,7 @@ def _scheme_used(name):
     return any(m.meta("scheme") == name for m in keops_io._modules.values())
 
 
-@pytest.mark.parametrize("M,N,D,Dv", [(1000, 1500, 256, 16), (333, 4097, 64, 3), (2049, 31, 100, 1), (50, 70, 32, 2)])
+@pytest.mark.parametrize("M,N,D,Dv", [(1000, 1500, 256, 16), (333, 4097, 64, 3), (2049, 31, 100, 1), (50, 70, 32, 2), (700, 1300, 24, 2)])
 def test_laplace_chunked_vs_oracle(M, N, D, Dv):
     from keops_amd.torch import Genred
 
