@@ -458,7 +458,7 @@ def plan_row_col_product(red, dtype, use_fast_math, enable_chunks):
     if F.name != "Mult" or len(F.children) != 2:
         return None
     for G, W in (F.children, F.children[::-1]):
-        if G.dim != 1 or W.dim < 32:
+        if G.dim != 1 or W.dim < config.chunk_min_dim:
             continue
         wsign = 1
         while W.name == "Minus":
