@@ -204,7 +204,7 @@ def test_contraction_beyond_256_components_batched():
     assert_sum_parity(got.numpy(), ref.numpy(), scale.numpy())
 
 
-@pytest.mark.parametrize("D,kernel", [(64, "gauss"), (256, "laplace"), (200, "expdot"), (640, "gauss")])
+@pytest.mark.parametrize("D,kernel", [(64, "gauss"), (256, "laplace"), (200, "expdot"), (640, "gauss"), (24, "laplace")])
 def test_gradients_wrt_points_as_scalar_and_weighted_sums(D, kernel):
     """d/dx and d/dy of sum_ij e_i . K(x_i, y_j) b_j for radial and scalar-product kernels in high dimension:
     g_ij (x_i - y_j) (or g_ij y_j) is computed as x_i sum_j g_ij - sum_j g_ij y_j, chunked reductions only
