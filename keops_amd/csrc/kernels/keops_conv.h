@@ -24,7 +24,8 @@
 // KEOPS_VCHUNK (formulas with one long elementwise sum, the vector-ALU counterpart of GpuReduc1D_chunks.py:19-118):
 // the plug-in also defines VCH_D (components), VCH_DPAD, VCH_NROW / VCH_NCOL (long output-indexed / reduced-index
 // variables), the flags keops_{row,col}_long[] and positions keops_vch_{row,col}[] of those variables in the
-// tables, VCH_USES_YJ, and struct KeopsChunkFormula (one component of the sum).  Long variables are not copied to
+// tables, VCH_USES_YJ, VCH_FMA (the sum is a scalar product folded with explicit fused multiply-adds, as the reference's
+// Scalprod: eval then returns the two factors), and struct KeopsChunkFormula (one component of the sum).  Long variables are not copied to
 // x_i / y_j: the reduced-index ones are staged whole in LDS for a short tile of columns, the output-indexed ones are
 // read from memory 16 bytes at a time (one cache line serves four such reads), each read feeding KEOPS_TILE_J
 // running sums held in registers; KeopsFormula::eval takes the finished sum as an extra argument.
@@ -171,7 +172,13 @@ __device__ __forceinline__ void keops_sweep(const KeopsParams& P, const i64* col
           for (int v = 0; v < NR; v++) xc[v] = xk[v][c];
 #pragma unroll
           for (int v = 0; v < NC; v++) yc[v] = yk[v][c];
+#if VCH_FMA
+          T fb;
+          const T fa = KeopsChunkFormula::eval(xc, yc, xi[0], yj, p, fb);
+          s[jj] = keops_fma(fa, fb, s[jj]);  // the reference's scalar-product chain (Scalprod.py:32-36)
+#else
           s[jj] = s[jj] + KeopsChunkFormula::eval(xc, yc, xi[0], yj, p);
+#endif
         }
       }
     }
@@ -193,7 +200,13 @@ __device__ __forceinline__ void keops_sweep(const KeopsParams& P, const i64* col
           for (int v = 0; v < VCH_NROW; v++) xc[v] = xlong[v][k0 + c];
 #pragma unroll
           for (int v = 0; v < VCH_NCOL; v++) yc[v] = yl[(jj * VCH_NCOL + v) * VCH_DPAD + k0 + c];
+#if VCH_FMA
+          T fb;
+          const T fa = KeopsChunkFormula::eval(xc, yc, xi[0], yj, p, fb);
+          s[jj] = keops_fma(fa, fb, s[jj]);  // the reference's scalar-product chain (Scalprod.py:32-36)
+#else
           s[jj] = s[jj] + KeopsChunkFormula::eval(xc, yc, xi[0], yj, p);
+#endif
         }
       }
     }

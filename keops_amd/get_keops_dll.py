@@ -221,25 +221,29 @@ def match_vchunk(red):
     exact = red.kind in (KIND_MIN, KIND_MAX, KIND_KMIN)
     for node in red.formula.walk():
         if node.children and node.children[0].dim > config.vchunk_min_dim and node not in [f[0] for f in found]:
-            E = None
+            E, pair = None, None
             if node.name == "Sum":
                 E = node.children[0]
-            elif node.name == "Scalprod" and not exact:
+            elif node.name == "Scalprod":
                 # (a|b) = Sum(a*b); index-carrying reductions keep the reference's fused multiply-add chain
-                # (Scalprod.py:32-36) on the general-purpose kernel
+                # (Scalprod.py:32-36): the two factors are then evaluated separately and folded with an explicit fma
                 E = O.Mult(node.children[0], node.children[1])
+                if exact:
+                    pair = (node.children[0], node.children[1])
+                    if not all(elementwise(c, c.dim) and c.dim == node.children[0].dim for c in pair):
+                        E = None
             if E is not None and E.dim == node.children[0].dim and elementwise(E, E.dim):
-                found.append((node, E))
+                found.append((node, E, pair))
     if len(found) != 1:
         return None
-    node, E = found[0]
+    node, E, pair = found[0]
     longs = [v for v in E.variables if v.dim == E.dim and v.dim > 1]
     if not longs or any(v.cat not in (0, 1) for v in longs):
         return None
     post = red.formula.replace(node, O.Var(1 << 30, 1, 3))
     if any(v in longs for v in post.variables) or any(v.dim > config.vchunk_min_dim for v in post.variables):
         return None
-    return node, E, longs
+    return node, E, longs, pair
 
 
 def generate_vchunk_plugin(red, match, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, irregular=False):
@@ -250,7 +254,7 @@ def generate_vchunk_plugin(red, match, dtype, dtypeacc, sum_scheme, use_fast_mat
     columns live in registers."""
     from .formulas import ops as O
 
-    node, E, longs = match
+    node, E, longs, pair = match
     D = E.dim
     sizeof_t = 8 if dtype == "double" else 4
     vec = 16 // sizeof_t
@@ -296,7 +300,16 @@ def generate_vchunk_plugin(red, match, dtype, dtypeacc, sum_scheme, use_fast_mat
     names[(3, svar.ind, 0)] = "s"
     pragma = ["    #pragma clang fp contract(off)"] if exact else []
     Le = Lir(row_cat=red.tagI, fast_math=use_fast_math, dtype=dtype, exact_order=exact)
-    e_lines, e_exprs = Le.emit(lower(Es, Le), names, indent="    ")
+    if pair is None:
+        e_lines, e_exprs = Le.emit(lower(Es, Le), names, indent="    ")
+    else:
+        # the two factors of the scalar product, one component each
+        factors = []
+        for f in pair:
+            for v in longs:
+                f = f.replace(v, stand_in[v])
+            factors.append(f)
+        e_lines, e_exprs = Le.emit(lower(factors[0], Le) + lower(factors[1], Le), names, indent="    ")
     Lp = Lir(row_cat=red.tagI, fast_math=use_fast_math, dtype=dtype, exact_order=exact)
     p_outs = lower(post, Lp)
     p_lines, p_exprs = Lp.emit(p_outs, names, indent="    ")
@@ -337,7 +350,7 @@ def generate_vchunk_plugin(red, match, dtype, dtypeacc, sum_scheme, use_fast_mat
         KEOPS_RED_KEEP=red.keep, KEOPS_RED_K=red.K, KEOPS_SUM_SCHEME=SUM_SCHEMES[sum_scheme],
         KEOPS_BLOCK=config.block_size, KEOPS_ROWS=1, KEOPS_TILE_J=tile_j, KEOPS_UNROLL_J=1, KEOPS_LSE_GROUP=1,
         KEOPS_NROWVARS=len(full.rowvars), KEOPS_NCOLVARS=len(full.colvars), KEOPS_NPARVARS=len(full.parvars),
-        KEOPS_VCHUNK=1, VCH_D=D, VCH_DPAD=dpad, VCH_NROW=len(row_long), VCH_NCOL=len(col_long), VCH_USES_YJ=int(uses_yj),
+        KEOPS_VCHUNK=1, VCH_D=D, VCH_DPAD=dpad, VCH_NROW=len(row_long), VCH_NCOL=len(col_long), VCH_USES_YJ=int(uses_yj), VCH_FMA=int(pair is not None),
     )
     src += [f"#define {k} {v}" for k, v in defs.items()]
     for name, vals in (("row_arg", ra), ("row_dim", rd), ("row_off", ro), ("row_long", rl), ("col_arg", ca), ("col_dim", cd),
@@ -350,9 +363,9 @@ def generate_vchunk_plugin(red, match, dtype, dtypeacc, sum_scheme, use_fast_mat
     src.append("// one component of the long sum: xl / yl hold that component of the long variables")
     src.append("struct KeopsChunkFormula {")
     src.append(f"  static __device__ __forceinline__ T eval(const T (&xl)[{nr}], const T (&yl)[{nc}], const T (&xi)[{dx}], "
-               f"const T (&yj)[{dy}], const T (&p)[{dp}]) {{")
+               f"const T (&yj)[{dy}], const T (&p)[{dp}]{'' if pair is None else ', T& fb'}) {{")
     src += pragma + e_lines
-    src.append(f"    return {e_exprs[0]};")
+    src.append(f"    return {e_exprs[0]};" if pair is None else f"    fb = {e_exprs[1]};\n    return {e_exprs[0]};")
     src.append("  }\n};")
     src.append("// post-chunk formula: s is the value of the long sum")
     src.append("struct KeopsFormula {")

@@ -133,3 +133,30 @@ def test_long_sum_over_the_first_index_with_block_sparse_ranges():
     K = torch.exp(-torch.cdist(x.double(), y.double(), p=1)) * mask
     assert rel_l2(out.numpy(), (K.T @ e.double()).numpy()) < 1e-5
     assert torch.all(out[600:] == 0)
+
+
+def test_scalar_product_neighbours_keep_the_fused_multiply_add_chain(monkeypatch):
+    """ArgKMin of 1 - (x|y) at D = 300 (angular neighbours of normalised rows): the chunked kernel folds the products
+    with the reference's fma chain, so values and indices are bit-identical to the general-purpose kernel."""
+    import keops_amd.get_keops_dll as engine
+    from keops_amd import config, keops_io
+    from keops_amd.torch import Genred
+
+    M, N, D, K = 300, 5000, 300, 6
+    rng = np.random.default_rng(17)
+    x, y = rng.standard_normal((M, D)).astype(np.float32), rng.standard_normal((N, D)).astype(np.float32)
+    x /= np.linalg.norm(x, axis=1, keepdims=True)
+    y /= np.linalg.norm(y, axis=1, keepdims=True)
+    knn = lambda: Genred("IntCst(1)-(x|y)", [f"x=Vi({D})", f"y=Vj({D})"], reduction_op="KMin_ArgKMin", axis=1, opt_arg=K)
+    vals, idx = knn()(*to_dev(x, y))
+    assert _last_module().meta("vchunk") == str(D)
+    monkeypatch.setattr(config, "vchunk_min_dim", 1 << 20)
+    engine._cache.clear()
+    keops_io._loaders.clear()
+    vals0, idx0 = knn()(*to_dev(x, y))
+    assert _last_module().meta("vchunk") is None
+    engine._cache.clear()
+    keops_io._loaders.clear()
+    assert torch.equal(vals, vals0) and torch.equal(idx, idx0)
+    ref = np.argsort(1 - x.astype(np.float64) @ y.astype(np.float64).T, axis=1)[:, :K]
+    assert (idx.cpu().numpy() == ref).mean() > 0.999
