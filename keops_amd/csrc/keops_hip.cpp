@@ -728,7 +728,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (D <= 0 || DP <= 0) return fail(-1, "corrupt chunk module metadata");
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
-  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(512, nys / 64));
+  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(128, nys / 64));
   const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
   const size_t o_xs = take((size_t)nxs * DP * 4), o_ys = take((size_t)nys * DP * 4);
   const size_t o_xn = take((size_t)nxs * 4), o_yn = take((size_t)nys * 4);
