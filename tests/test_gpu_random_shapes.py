@@ -1,0 +1,58 @@
+"""Seeded random shapes across the schemes (general-purpose, chunked matrix-core, chunked vector-ALU, nearest
+neighbours with exact re-rank): ragged sizes, dimensions around every threshold of the engine, vectors whose length
+is not a multiple of the load width.  References: dense float64 torch formulas; float32 sums in the reference's
+order for indices."""
+import numpy as np
+import pytest
+import torch
+
+from keops_amd.torch import Genred
+
+pytestmark = pytest.mark.gpu
+
+DIMS = [24, 25, 31, 32, 33, 47, 64, 100, 101, 129, 200, 257, 300, 511, 784, 1025, 1100]
+
+
+def _case(seed):
+    rng = np.random.default_rng(seed)
+    M, N = int(rng.integers(1, 1500)), int(rng.integers(200, 1500))
+    D = int(rng.choice(DIMS))
+    kind = ["sum_sq", "sum_l1", "lse_sq", "knn_sq", "knn_l1", "sum_dot64"][seed % 6]
+    x = torch.from_numpy(rng.standard_normal((M, D))).float() / D ** 0.5
+    y = torch.from_numpy(rng.standard_normal((N, D))).float() / D ** 0.5
+    b = torch.from_numpy(rng.standard_normal((N, 2))).float()
+    return kind, M, N, D, x, y, b, rng
+
+
+@pytest.mark.parametrize("seed", range(36))
+def test_random_shape(seed):
+    kind, M, N, D, x, y, b, rng = _case(seed)
+    xd, yd, bd = x.cuda(), y.cuda(), b.cuda()
+    x64, y64, b64 = x.double(), y.double(), b.double()
+    var = [f"x=Vi({D})", f"y=Vj({D})"]
+    if kind in ("sum_sq", "sum_l1"):
+        f = "Exp(-SqDist(x,y))*b" if kind == "sum_sq" else "Exp(-Sum(Abs(x-y)))*b"
+        out = Genred(f, var + ["b=Vj(2)"], reduction_op="Sum", axis=1)(xd, yd, bd).cpu().double()
+        K = torch.exp(-torch.cdist(x64, y64) ** 2) if kind == "sum_sq" else torch.exp(-torch.cdist(x64, y64, p=1))
+        ref, scale = K @ b64, K @ b64.abs()
+        # condition-aware bound; the float32 sum of D terms in the exponent adds about D * 2^-24 of its value
+        tol = 1e-5 + D * 6e-8 * float(torch.cdist(x64, y64, p=1 if kind == "sum_l1" else 2).max()) ** (1 if kind == "sum_l1" else 2)
+        assert float(((out - ref).abs() / scale.clamp_min(1e-300)).max()) < tol
+    elif kind == "lse_sq":
+        out = Genred("-SqDist(x,y)", var, reduction_op="LogSumExp", axis=1)(xd, yd).cpu().double()[:, 0]
+        ref = torch.logsumexp(-torch.cdist(x64, y64) ** 2, 1)
+        assert float((out - ref).abs().max()) < 2e-5 * max(1.0, float(ref.abs().max()))
+    elif kind in ("knn_sq", "knn_l1"):
+        K = int(rng.integers(1, 12))
+        f = "SqDist(x,y)" if kind == "knn_sq" else "Sum(Abs(x-y))"
+        idx = Genred(f, var, reduction_op="ArgKMin", axis=1, opt_arg=K)(xd, yd).cpu().numpy()
+        d = np.zeros((M, N), np.float32)
+        xn, yn = x.numpy(), y.numpy()
+        for k in range(D):
+            t = xn[:, None, k] - yn[None, :, k]
+            d += t * t if kind == "knn_sq" else np.abs(t)
+        assert np.array_equal(idx.astype(np.int64), np.argsort(d, axis=1, kind="stable")[:, :K])
+    else:
+        out = Genred("(x|y)*b", var + ["b=Vj(2)"], reduction_op="Sum", axis=1)(xd.double(), yd.double(), bd.double()).cpu()
+        ref = (x64 @ y64.T) @ b64
+        assert float((out - ref).abs().max()) < 1e-11 * max(1.0, float(ref.abs().max()))
