@@ -88,7 +88,9 @@ template <typename A> struct KeopsAcc {
   // Branch-free form of the same update: one exponential of -|fm - m| and selects.
   template <typename B> __device__ __forceinline__ void absorb(B fm, const B* g) {
     const bool keep = m > (A)fm;  // false when equal or when m is still -inf
-    const A e = (A)keops_red_exp(keep ? (T)((A)fm - m) : (T)(m - (A)fm));
+    // both sides still empty (-inf - -inf): the maximum with a finite bound drops the NaN, the factor is 0
+    const A d = keops_fmax(keep ? (A)fm - m : m - (A)fm, (A)(-3.0e38f));
+    const A e = (A)keops_red_exp((T)d);
 #pragma unroll
     for (int k = 0; k < KEOPS_FD - 1; k++) {
 #if KEOPS_SUM_SCHEME == 2

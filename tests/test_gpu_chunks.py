@@ -341,3 +341,19 @@ def test_narrow_kernel_on_clustered_points_and_self_interaction(reduction):
         out = lse(xd, xd, g.cuda()).cpu().double()[:, 0]
         ref = torch.logsumexp(-g.double() * S, dim=1)
         assert float((out - ref).abs().max()) < 1e-5 * max(1.0, float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("N,D", [(12, 257), (3, 64), (9, 300), (1, 40)])
+def test_log_sum_exp_with_fewer_columns_than_a_tile(N, D):
+    """Fewer reduced rows than the lanes that share an output row can take: some of their accumulators stay empty
+    (maximum -inf, sum 0) and merging two empty ones must stay empty, not NaN."""
+    from keops_amd.torch import LazyTensor
+
+    gen = torch.Generator().manual_seed(N * D)
+    x, y, v = torch.randn(1, 300, D, generator=gen) / D ** 0.5, torch.randn(1, N, D, generator=gen) / D ** 0.5, torch.randn(1, N, 3, generator=gen)
+    S_ij = (LazyTensor(x.cuda()[:, :, None, :]) * LazyTensor(y.cuda()[:, None, :, :])).sum(-1)
+    out = S_ij.sumsoftmaxweight(LazyTensor(v.cuda()[:, None, :, :]), dim=2).cpu().double()
+    lse = S_ij.logsumexp(dim=2).cpu().double()[..., 0]
+    S = x.double() @ y.double().transpose(1, 2)
+    assert float((out - torch.softmax(S, 2) @ v.double()).abs().max()) < 2e-5
+    assert float((lse - torch.logsumexp(S, 2)).abs().max()) < 2e-5
