@@ -196,11 +196,21 @@ def cpu_baseline(name, inp):
 
     M, N, Dv = inp["M"], inp["N"], inp["Dv"]
     x, y, b, g = inp["arrays"]
-    try:
-        threads = ctypes.CDLL(None).omp_get_max_threads()
-    except Exception:
-        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     lib()
+    try:
+        gomp = ctypes.CDLL("libgomp.so.1")
+        threads = gomp.omp_get_max_threads()
+    except Exception:
+        gomp, threads = None, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
     # calibrate on 64 rows per thread, then size the sample for about 12 s of CPU work
     ncal = int(min(M, 64 * max(1, threads)))
     rows = np.arange(ncal, dtype=np.int64)
@@ -212,8 +222,50 @@ def cpu_baseline(name, inp):
     t0 = time.perf_counter()
     cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
     dt = time.perf_counter() - t0
-    return dict(value=nrows * N / dt, unit="pairs/s", cores=int(threads), kind="port",
-                sample=f"{nrows} random output rows x {N} columns of the same inputs ({dt:.1f} s, OpenMP over rows)")
+    res = dict(value=nrows * N / dt, unit="pairs/s", cores=int(threads), kind="port", cpu_model=model,
+               sample=f"{nrows} random output rows x {N} columns of the same inputs ({dt:.1f} s, OpenMP over rows)")
+    if gomp is not None and threads > 1:
+        # the same loop on one thread (about 4 s)
+        n1 = int(max(16, (4.0 * rate / threads / N) // 16 * 16))
+        gomp.omp_set_num_threads(1)
+        t0 = time.perf_counter()
+        cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows[:n1])
+        dt1 = time.perf_counter() - t0
+        gomp.omp_set_num_threads(int(threads))
+        res["value_1_thread"] = min(n1, len(rows)) * N / dt1
+        res["sample_1_thread"] = f"{min(n1, len(rows))} of those rows on one thread ({dt1:.1f} s)"
+    return res
+
+
+def calibration(mfma):
+    """Issue rates of loop-only kernels (keops_hip_calibrate): wavefront instructions per cycle and SIMD at the
+    nominal 2.4 GHz clock, for 1, 2 and 4 wavefronts per SIMD (256 CUs x 4 SIMDs; a workgroup is 4 wavefronts)."""
+    import torch
+
+    from keops_amd import binder
+
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    simds, clock = 4 * cus, 2.4e9
+    rows = []
+    kinds = [(3, "v_mfma_f32_32x32x16_bf16", (1, 2, 4))] if mfma else [
+        (0, "v_fmac_f32 chains", (1, 2, 4, 8)), (1, "Gaussian pair mix with v_exp_f32 (9 instr)", (1, 2, 4, 8)),
+        (2, "Gaussian pair mix without v_exp_f32 (8 instr)", (1, 2, 4, 8))]
+    for kind, label, chain_set in kinds:
+        for chains in chain_set:
+            for waves in (1, 2, 4):
+                blocks = cus * waves  # one workgroup = 4 wavefronts = one per SIMD of a CU
+                iters = 200_000 // chains if kind != 3 else 100_000 // chains
+                ms, ipw = binder.calibrate(kind, chains, blocks, iters)
+                total = ipw * blocks * 4  # wavefront instructions
+                per_cycle = total / (ms * 1e-3) / simds / clock
+                row = dict(kind=label, chains=chains, waves_per_simd=waves, ms=round(ms, 3),
+                           wave_instr_per_cycle_per_simd_at_2p4GHz=round(per_cycle, 4))
+                if kind == 3:
+                    row["PFLOP_per_s"] = round(total * 32 * 32 * 16 * 2 / (ms * 1e-3) / 1e15, 3)
+                else:
+                    row["lane_instr_per_s"] = total * 64 / (ms * 1e-3)
+                rows.append(row)
+    return {"calibration": "mfma" if mfma else "valu", "cus": cus, "rows": rows}
 
 
 def main():
@@ -223,6 +275,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="gauss_1m_dv1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--valu-calibration", action="store_true",
+                    help="loop-only kernels: what the vector ALU sustains on chains of v_fmac_f32 and on the "
+                         "instruction mix of a Gaussian pair, with and without v_exp_f32, at 1/2/4 wavefronts per SIMD")
+    ap.add_argument("--mfma-calibration", action="store_true",
+                    help="loop-only kernels: what the matrix cores sustain on 1/2/4 dependent chains of "
+                         "v_mfma_f32_32x32x16_bf16 per wavefront")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run a plain 1 GiB device copy instead of a workload (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -234,6 +292,9 @@ def main():
 
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a HIP device")
+    if args.valu_calibration or args.mfma_calibration:
+        print(json.dumps(calibration(args.mfma_calibration)))
+        return
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
         dst = torch.empty_like(src)
@@ -291,7 +352,7 @@ def main():
         "roofline": {
             "bound": "mfma" if bound.startswith("mfma") else bound, "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-            "kernel_ms": kms, "flop_per_pair": flop_per_pair,
+            "kernel_ms": kms, "end_to_end_ms": dt * 1e3, "flop_per_pair": flop_per_pair,
             "note": note,
         },
     }

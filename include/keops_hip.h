@@ -18,6 +18,7 @@
 #ifndef KEOPS_HIP_H
 #define KEOPS_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -58,11 +59,18 @@ void keops_hip_module_destroy(void* module);
 /*
  * Run one map-reduce.  Replaces KeOps_module<TYPE>::launch_kernel (keops_nvrtc.cpp:390-643);
  * arguments keep the reference's meaning and order:
- *   tagHostDevice     must be 1 (all data pointers are device pointers)
+ *   tagHostDevice     1: out, args and ranges[0..5] are device pointers.  0: they are host pointers
+ *                     (load_args_FromHost / range_preprocess_from_host of the reference,
+ *                     keopscore/keopscore/include/utils_pe.h:66-99, keops_nvrtc.cpp:250-325): the library copies
+ *                     them into one pooled device allocation owned by the module, runs the same kernels, copies
+ *                     out back and returns once it is in host memory (whatever `sync` says)
  *   dimY              total dimension of the reduced-index variables
  *   nx, ny            sizes M and N of the i and j axes (per batch)
  *   tagI              0: output indexed by i (reduce over j); 1: output indexed by j
- *   tagZero           1: the formula is identically zero, out is filled with zeros
+ *   tagZero           1: the formula is identically zero: out is filled with zeros by a fill kernel on hip_stream and
+ *                     nothing else runs.  A module is still required (it gives the element size); the engine
+ *                     compiles none for a zero formula, so keops_amd/keops_io.py fills out itself and never
+ *                     passes 1 here
  *   tag1D2D           0: one pass over the reduced axis; 1: force the column-slab (2D) scheme
  *   dimred, dimout    accumulator and output dimensions per row
  *   block_size        upper bound for the workgroup size (0 = module default)
@@ -100,14 +108,26 @@ const char* keops_hip_last_error(void);
 const char* keops_hip_module_meta(void* module, const char* key);
 
 /*
- * Average duration in milliseconds of the kernels launched by the most recent
- * keops_hip_launch on this module, measured with HIP events on the launch stream when
- * timing has been enabled with keops_hip_module_set_timing(module, 1); -1 if unavailable.
+ * Time in milliseconds between two HIP events recorded on the launch stream around the main kernels of
+ * the most recent keops_hip_launch on this module (the sweep over the pairs; pre-passes that prepare
+ * operands and the final merge of slab partials lie outside), when timing has been enabled with
+ * keops_hip_module_set_timing(module, 1); -1 if unavailable.  With timing on, a launch waits for its second event.
  * No counterpart in the reference (it only has commented-out clock() stamps,
  * keops_nvrtc.cpp:402-412); used by the benchmark's roofline measurement.
  */
 void keops_hip_module_set_timing(void* module, int enabled);
 double keops_hip_module_last_kernel_ms(void* module);
+
+/*
+ * Loop-only calibration of the instruction issue rates the roofline fractions are held against: runs a grid of
+ * `blocks` workgroups of 4 wavefronts, each wavefront issuing `iters` rounds of `chains` independent dependency
+ * chains, and returns the elapsed time in ms and the counted instructions per wavefront.
+ *   kind 0: v_fmac_f32 only (8 per chain and round); kind 1: the 9-instruction mix of a Gaussian pair (3 sub,
+ *   mul, 2 fma, mul, v_exp_f32, fma); kind 2: the same without v_exp_f32; kind 3: v_mfma_f32_32x32x16_bf16
+ *   (4 per chain and round).  chains: 1, 2, 4, 8 (kinds 0-2) or 1, 2, 4 (kind 3).
+ * Measurement aid without counterpart in the reference; used by bench.py --valu-calibration / --mfma-calibration.
+ */
+int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave);
 
 #ifdef __cplusplus
 }

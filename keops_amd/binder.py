@@ -49,8 +49,19 @@ def lib():
             P, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, I64, P, P, P, P, P, ctypes.c_int, P, P, P, P, P,
             ctypes.c_int,
         ]
+        L.keops_hip_calibrate.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 2
         _lib = L
     return _lib
+
+
+def calibrate(kind, chains, blocks, iters, device_id=0):
+    """(milliseconds, counted instructions per wavefront) of one loop-only calibration kernel
+    (keops_hip_calibrate of include/keops_hip.h)."""
+    ms, ipw = ctypes.c_double(0), ctypes.c_double(0)
+    rc = lib().keops_hip_calibrate(int(device_id), int(kind), int(chains), int(blocks), int(iters), ctypes.byref(ms), ctypes.byref(ipw))
+    if rc != 0:
+        raise KeOpsHipError(f"calibration failed (code {rc}): {last_error()}")
+    return ms.value, ipw.value
 
 
 def last_error():
@@ -136,3 +147,4 @@ class Module:
         if rc != 0:
             raise KeOpsHipError(f"kernel launch failed (code {rc}): {last_error()}")
         return 0
+

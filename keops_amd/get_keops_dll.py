@@ -607,14 +607,16 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
     return "\n".join(src) + "\n", meta
 
 
-def match_final(red, dtype, dtypeacc, sum_scheme, map_reduce_id):
+def match_final(red, dtype, dtypeacc, sum_scheme, map_reduce_id, use_fast_math=True):
     """(scalar kernel f, variable v) when ``red`` is Sum_Reduction(f * v) with f of dimension 1 and v a
     plain reduced-index variable of dimension >= config.final_chunk_min_dim (24), in float32 on the dense
-    scheme (the shape GpuReduc1D_finalchunks.py:100-106 expects); None otherwise."""
+    scheme (the shape GpuReduc1D_finalchunks.py:100-106 expects); None otherwise.  The scheme evaluates f with the
+    hardware's fast exp / sqrt / reciprocal and forms the product from bfloat16 terms: use_fast_math=False keeps
+    such formulas on the exact vector kernel."""
     from .formulas import ops as O
     from .formulas.reductions import KIND_SUM
 
-    if red.kind != KIND_SUM or dtype != "float" or dtypeacc != "float":
+    if red.kind != KIND_SUM or dtype != "float" or dtypeacc != "float" or not use_fast_math:
         return None
     if sum_scheme not in ("block_sum", "direct_sum"):
         return None
@@ -734,7 +736,7 @@ def get_keops_dll(
         chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (mc and knn is None) else None
         fin = None
         if enable_finalchunks and mc and knn is None and chk is None:
-            fin = match_final(red, dtype, dtypeacc, sum_scheme_string, map_reduce_id)
+            fin = match_final(red, dtype, dtypeacc, sum_scheme_string, map_reduce_id, use_fast_math)
         if knn is not None:
             source, meta = generate_knn_plugin(red_k, knn[0], knn[1], nargs)
             use_chunk_mode = 3  # matrix-core filter scheme (no counterpart among the reference's chunk modes)

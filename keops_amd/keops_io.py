@@ -25,11 +25,8 @@ class LoadKeOps_hip:
                  dtype, lang, optional_flags, nx=None, batch_loop=0, pairs=0):
         if lang not in ("torch", "pytorch"):
             raise ValueError("[KeOps] the HIP backend binds torch tensors only")
-        if tagCPUGPU != 1 or tagHostDevice != 1:
-            raise ValueError(
-                "[KeOps] the HIP backend computes on device-resident tensors only "
-                "(backend 'CPU' and host-memory inputs are not available)"
-            )
+        if tagCPUGPU != 1 or tagHostDevice not in (0, 1):
+            raise ValueError("[KeOps] the HIP backend computes on the GPU only (backend 'CPU' is not available)")
         aliases_new = []
         for k, alias in enumerate(aliases):
             name, var = parse_alias(alias, k)
@@ -160,7 +157,9 @@ class LoadKeOps_hip:
         if p.tagZero:
             out.zero_()
             return out
-        stream = torch.cuda.current_stream(out.device).cuda_stream
+        # host tensors (tagHostDevice = 0): the library stages them itself and returns when out is back on the host
+        dev = out.device if out.is_cuda else torch.device("cuda", max(0, p.device_id_request))
+        stream = torch.cuda.current_stream(dev).cuda_stream
         try:
             self.module(
                 p.tagHostDevice, p.dimy, nx, ny, p.tagI, p.tagZero, p.use_half, p.tag1D2D, p.dimred, p.cuda_block_size,

@@ -1,10 +1,10 @@
 """NumPy front end: the same Genred / KernelSolve call signatures on host arrays.
 
-Counterpart of pykeops/pykeops/numpy (generic/generic_red.py, operations.py).  The reference's NumPy
-binding hands host pointers to the GPU engine, which stages them itself (tagHostDevice = 0,
-keops_nvrtc.cpp load_args_FromHost).  The HIP library only takes device pointers, so the staging is
-done here: arrays are copied to the current HIP device as torch tensors, the torch binding runs the
-reduction, and the result comes back as a NumPy array.  There is no CPU computation path.
+Counterpart of pykeops/pykeops/numpy (generic/generic_red.py, operations.py).  As in the reference, Genred hands
+host pointers to the GPU engine, which stages them itself (tagHostDevice = 0, keops_nvrtc.cpp load_args_FromHost):
+the arrays are wrapped as host torch tensors without a copy and the result comes back in host memory.  KernelSolve
+and LazyTensor, which launch many reductions on the same data, copy their arrays to the current HIP device once.
+There is no CPU computation path.
 """
 import numpy as np
 import torch
@@ -51,8 +51,16 @@ class Genred:
         if backend == "CPU":
             raise ValueError("[KeOps] backend 'CPU' is not available in the HIP build")
         dev = _device(device_id)
-        res = self._fn(*_to_device(args, dev), backend=backend.replace("_Host", "").replace("_Device", ""),
-                       ranges=_ranges_to_device(ranges, dev))
+        host = []
+        for a in args:
+            a = np.ascontiguousarray(a)
+            if a.dtype not in (np.float32, np.float64):
+                raise ValueError("[KeOps] only float32 and float64 arrays are supported")
+            host.append(torch.from_numpy(a))
+        if ranges is not None:
+            ranges = tuple(torch.from_numpy(np.ascontiguousarray(r).astype(np.int64)) for r in ranges)
+        res = self._fn(*host, backend=backend.replace("_Host", "").replace("_Device", "").replace("_host", "").replace("_device", ""),
+                       device_id=dev.index, ranges=ranges)
         res = res.cpu().numpy()
         if out is not None:
             out[...] = res

@@ -60,24 +60,11 @@ class GenredAutograd_base:
             or params.rec_multVar_highdim else 0
         )
         tagCPUGPU, tag1D2D, tagHostDevice = get_tag_backend(params.backend, args)
+        # where the data lives decides what kind of pointers the library receives, whatever the backend string says
+        tagHostDevice = 1 if all(a.is_cuda for a in args) else 0
         nbatchdims = max(len(a.shape) for a in args) - 2
         use_ranges = nbatchdims > 0 or params.ranges is not None
         device_id, device_args = set_device(tagCPUGPU, tagHostDevice, params.device_id_request, *args)
-        host_out, staged = None, False
-        if tagCPUGPU == 1 and tagHostDevice == 0:
-            # host-resident tensors with a GPU backend: staged through device memory, as the reference's binder
-            # does in load_args_FromHost (keops_nvrtc.cpp:46-73); the library itself only takes device pointers
-            if not torch.cuda.is_available():
-                raise ValueError("[KeOps] the HIP backend needs a GPU: none is visible to torch")
-            dev = torch.device("cuda", device_id)
-            args = tuple(a.to(dev) for a in args)
-            if params.ranges:
-                params = copy.copy(params)
-                params.ranges = tuple(r.to(dev) for r in params.ranges)
-            if params.out is not None:
-                params = copy.copy(params)
-                host_out, params.out = params.out, None
-            tagHostDevice, device_args, staged = 1, dev, True
         nout = params.nx if params.axis == 1 else params.ny
         batch = None
         if nbatchdims > 0 and params.ranges is None:
@@ -85,10 +72,37 @@ class GenredAutograd_base:
             for d in range(nbatchdims):
                 nbatches *= max(a.shape[d] if a.dim() == nbatchdims + 2 else 1 for a in args)
             batch = (nbatches, params.nx, params.ny)
-        myconv = keops_binder["hip"](
-            tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id, params.formula, params.aliases, len(args),
-            params.dtype, "torch", params.optional_flags, nx=nout, ny=params.nx + params.ny - nout, batch=batch,
-        ).import_module()
+
+        def binder_for(tag_hd):
+            return keops_binder["hip"](
+                tagCPUGPU, tag1D2D, tag_hd, use_ranges, device_id, params.formula, params.aliases, len(args),
+                params.dtype, "torch", params.optional_flags, nx=nout, ny=params.nx + params.ny - nout, batch=batch,
+            ).import_module()
+
+        host_out, staged, myconv = None, False, None
+        if tagCPUGPU == 1 and tagHostDevice == 0:
+            # host-resident tensors with a GPU backend: the library copies them to the device itself
+            # (tagHostDevice = 0, the reference's load_args_FromHost, keops_nvrtc.cpp:46-73) ...
+            if not torch.cuda.is_available():
+                raise ValueError("[KeOps] the HIP backend needs a GPU: none is visible to torch")
+            myconv = binder_for(0)
+            if myconv.plan is not None:
+                # ... except for reductions that the binding layer evaluates as several launches combined with
+                # torch operations on the device: those are staged here
+                dev = torch.device("cuda", device_id)
+                args = tuple(a.to(dev) for a in args)
+                if params.ranges:
+                    params = copy.copy(params)
+                    params.ranges = tuple(r.to(dev) for r in params.ranges)
+                if params.out is not None:
+                    params = copy.copy(params)
+                    host_out, params.out = params.out, None
+                tagHostDevice, device_args, staged, myconv = 1, dev, True, None
+            elif params.ranges:
+                params = copy.copy(params)
+                params.ranges = tuple(r.cpu() for r in params.ranges)
+        if myconv is None:
+            myconv = binder_for(tagHostDevice)
         if not all(a.is_contiguous() for a in args):
             warnings.warn(
                 "[KeOps] at least one of the input tensors is not contiguous. "

@@ -14,7 +14,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
-FORMULAS = dict(dense=0, gauss=1, gauss_gradx=2, sqdist=3, lse_gauss=4, laplace=5)
+FORMULAS = dict(dense=0, gauss=1, gauss_gradx=2, sqdist=3, lse_gauss=4, laplace=5, l1dist=6, exp_l1=7, scalprod=8,
+                gauss_gradx_abs=9)
 REDUCTIONS = dict(
     Sum=0, Max_SumShiftExpWeight=1, Max_SumShiftExp=1, Min_ArgMin=2, Max_ArgMax=3, KMin_ArgKMin=4,
     Min=5, ArgMin=6, Max=7, ArgMax=8, KMin=9, ArgKMin=10,
@@ -27,8 +28,13 @@ def build(force=False):
     target = os.path.join(_HERE, "liboracle_cpu.so")
     if force:
         subprocess.run(["make", "-C", _HERE, "clean"], check=True, stdout=subprocess.DEVNULL)
-    if force or not os.path.exists(target):
+    # make is incremental: a library older than cpu_reduc.c is rebuilt, an up-to-date one is left alone
+    # (no compiler on the machine: use the library that travelled with the tree)
+    try:
         subprocess.run(["make", "-C", _HERE], check=True, stdout=subprocess.DEVNULL)
+    except (OSError, subprocess.CalledProcessError):
+        if not os.path.exists(target):
+            raise
     return target
 
 

@@ -17,7 +17,8 @@
  *
  * The pair formula F(x_i, y_j, p) is either one of a few hand-written bodies that follow the
  * reference's per-op evaluation order (Subtract.py:21-24, Square.py:17-18, Sum.py:20-24,
- * Mult.py:25, Minus.py:20-23, Exp.py + math_functions.py:86, Sqrt.py:17), or a dense table
+ * Mult.py:25, Minus.py:20-23, Exp.py + math_functions.py:86, Sqrt.py:17, Abs.py, Scalprod.py:32-36
+ * with its fused multiply-add chain), or a dense table
  * F[i][j][:] computed by the caller (numpy / torch closed form), so that every reduction can be
  * exercised on any formula.
  *
@@ -58,7 +59,11 @@ enum {
   F_GAUSS_GRADX = 2,/* Grad of F_GAUSS wrt x, gradin G args: x y b g G[Dv]         -> D      */
   F_SQDIST = 3,     /* SqDist(x,y)                    args: x[D] y[D]              -> 1      */
   F_LSE_GAUSS = 4,  /* Concat(l - SqDist(x,y)*e, 1)   args: x[D] y[D] l[1] e[1]    -> 2      */
-  F_LAPLACE = 5     /* Exp(-Norm2(x-y))*b             args: x[D] y[D] b[Dv]        -> Dv     */
+  F_LAPLACE = 5,    /* Exp(-Norm2(x-y))*b             args: x[D] y[D] b[Dv]        -> Dv     */
+  F_L1DIST = 6,     /* Sum(Abs(x-y))                  args: x[D] y[D]              -> 1      */
+  F_EXP_L1 = 7,     /* Exp(-Sum(Abs(x-y)))*b          args: x[D] y[D] b[Dv]        -> Dv     */
+  F_SCALPROD = 8,   /* (x|y)*b                        args: x[D] y[D] b[Dv]        -> Dv     */
+  F_GAUSS_GRADX_ABS = 9 /* |F_GAUSS_GRADX| term by term: the condition scale sum_j |F_ij| of the tests */
 };
 
 typedef struct {
@@ -78,6 +83,25 @@ static inline real sqdist_seq(const real *x, const real *y, int D) {
     real q = d * d;
     s += q;
   }
+  return s;
+}
+
+/* Sum(Abs(Subtract(x,y))): out = 0; out += |x_k - y_k| in order (Subtract.py:21-24, Abs.py +
+   math_functions.py keops_abs, Sum.py:20-24) */
+static inline real l1dist_seq(const real *x, const real *y, int D) {
+  real s = (real)0;
+  for (int k = 0; k < D; k++) {
+    real d = x[k] - y[k];
+    real q = sizeof(real) == 4 ? (real)fabsf((float)d) : (real)fabs((double)d);
+    s += q;
+  }
+  return s;
+}
+
+/* Scalprod(x,y): out = 0; out = fma(x_k, y_k, out) in order (Scalprod.py:32-36, keops_fma) */
+static inline real scalprod_fma(const real *x, const real *y, int D) {
+  real s = (real)0;
+  for (int k = 0; k < D; k++) s = sizeof(real) == 4 ? (real)fmaf((float)x[k], (float)y[k], (float)s) : (real)fma((double)x[k], (double)y[k], (double)s);
   return s;
 }
 
@@ -109,6 +133,15 @@ static void eval_pair(const fctx *c, long i, long j, real *fout) {
     real coef = -((real)2 * (a[3][0] * (e * gb)));
     for (int k = 0; k < D; k++) fout[k] = coef * (x[k] - y[k]);
   } break;
+  case F_GAUSS_GRADX_ABS: {
+    int D = dm[0], Dv = dm[2];
+    const real *x = a[0] + i * D, *y = a[1] + j * D, *b = a[2] + j * Dv, *G = a[4] + i * Dv;
+    real e = r_exp(-(a[3][0] * sqdist_seq(x, y, D)));
+    real gb = (real)0;
+    for (int k = 0; k < Dv; k++) gb += (real)fabs((double)(G[k] * b[k]));
+    real coef = (real)2 * (real)fabs((double)a[3][0]) * (e * gb);
+    for (int k = 0; k < D; k++) fout[k] = coef * (real)fabs((double)(x[k] - y[k]));
+  } break;
   case F_SQDIST: {
     int D = dm[0];
     fout[0] = sqdist_seq(a[0] + i * D, a[1] + j * D, D);
@@ -125,6 +158,23 @@ static void eval_pair(const fctx *c, long i, long j, real *fout) {
     real e = r_exp(-r_sqrt(s));
     const real *b = a[2] + j * Dv;
     for (int k = 0; k < Dv; k++) fout[k] = e * b[k];
+  } break;
+  case F_L1DIST: {
+    int D = dm[0];
+    fout[0] = l1dist_seq(a[0] + i * D, a[1] + j * D, D);
+  } break;
+  case F_EXP_L1: {
+    int D = dm[0], Dv = dm[2];
+    real s = l1dist_seq(a[0] + i * D, a[1] + j * D, D);
+    real e = r_exp(-s);
+    const real *b = a[2] + j * Dv;
+    for (int k = 0; k < Dv; k++) fout[k] = e * b[k];
+  } break;
+  case F_SCALPROD: {
+    int D = dm[0], Dv = dm[2];
+    real s = scalprod_fma(a[0] + i * D, a[1] + j * D, D);
+    const real *b = a[2] + j * Dv;
+    for (int k = 0; k < Dv; k++) fout[k] = s * b[k];
   } break;
   }
 }

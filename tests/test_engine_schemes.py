@@ -119,3 +119,16 @@ def test_lazytensor_settles_variables_in_one_pass_and_reuses_the_reduction_objec
     assert n == 1 and len(lt._genred_cache) == 1 and callable(r1) and callable(r2)
     (key,) = lt._genred_cache
     assert key[0] == "Mult(Exp(Minus(Sum(Square(Subtract(Var(0,3,0),Var(1,3,1)))))),Var(2,2,1))"
+
+
+def test_no_fast_math_keeps_every_formula_off_the_matrix_core_schemes():
+    """use_fast_math=False means float32 arithmetic with library exp / sqrt on the vector kernel: neither the chunked
+    nor the final-product scheme (bfloat16-split products, hardware exp2 / rsq) may be chosen."""
+    al = ["x=Var(0,3,0)", "y=Var(1,3,1)", "b=Var(2,32,1)", "u=Var(3,64,0)", "v=Var(4,64,1)", "c=Var(5,2,1)"]
+    for formula in ("Sum_Reduction(Exp(-Sqrt(SqDist(x,y)))*b,0)", "Sum_Reduction(Exp(-SqDist(u,v))*c,0)"):
+        fast = get_keops_dll("GpuReduc1D", formula, 1, -1, 0, al, 6, "float", "float", "block_sum", 1, 1, 0, False, True, 0)
+        exact = get_keops_dll("GpuReduc1D", formula, 1, -1, 0, al, 6, "float", "float", "block_sum", 1, 1, 0, False, False, 0)
+        assert fast[8] in (1, 2) and exact[8] == 0
+        with open(exact[1]) as f:
+            src = f.read()
+        assert "scheme=conv" in src.splitlines()[0] and "__builtin_amdgcn_exp2f" not in src

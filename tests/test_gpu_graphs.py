@@ -101,3 +101,68 @@ def test_block_sparse_ranges_refuse_capture_with_a_clear_error():
             conv(x, y, b, ranges=ranges)
     torch.cuda.synchronize()
     assert torch.equal(conv(x, y, b, ranges=ranges), ref)             # the stream is usable again
+
+
+def test_captured_graph_survives_later_eager_calls_at_other_shapes():
+    """A captured graph holds raw pointers into the module's workspace.  A later eager call of the same formula that
+    needs a larger workspace must not free it under the graph: the library keeps the graph's buffer alive and gives the
+    eager calls a new one, so both keep producing the right results."""
+    from keops_amd.torch import Genred
+
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    r = lambda *s: torch.randn(*s, device="cuda", generator=gen)
+    conv = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)", "g=Pm(1)"], reduction_op="Sum", axis=1)
+    x, y, b, g = r(300, 3), r(60000, 3), r(60000, 2), torch.tensor([0.5], device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        conv(x, y, b, g)                      # sizes the slab workspace
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = conv(x, y, b, g)
+    graph.replay()
+    torch.cuda.synchronize()
+    ref = out.clone()
+    # a smaller call of the same module (same row bucket) fits the frozen workspace
+    small = conv(x[:200].contiguous(), y[:30000].contiguous(), b[:30000].contiguous(), g)
+    torch.cuda.synchronize()
+    assert torch.isfinite(small).all()
+    # a larger one outgrows it (1562 slabs of 400 rows against 234 of 300): new buffer, the old one stays with the graph
+    x2 = r(400, 3)
+    y2, b2 = r(400000, 3), r(400000, 2)
+    big = conv(x2, y2, b2, g)
+    torch.cuda.synchronize()
+    K = torch.exp(-0.5 * torch.cdist(x2.double(), y2.double()) ** 2)
+    assert float((big.double() - K @ b2.double()).norm() / (K @ b2.double()).norm()) < 1e-5
+    for _ in range(2):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref)
+    # batched launches: the graph reads lookup / offset tables; a call with other batch shapes builds its own
+    from keops_amd.torch import LazyTensor
+
+    def batched(xb, yb, bb):
+        d = ((LazyTensor(xb[:, :, None, :]) - LazyTensor(yb[:, None, :, :])) ** 2).sum(-1)
+        return ((-d).exp() * LazyTensor(bb[:, None, :, :])).sum(2)
+
+    xb, yb, bb = r(4, 700, 3), r(4, 900, 3), r(4, 900, 1)
+    with torch.cuda.stream(side):
+        batched(xb, yb, bb)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2):
+        outb = batched(xb, yb, bb)
+    g2.replay()
+    torch.cuda.synchronize()
+    refb = outb.clone()
+    other = batched(r(3, 1100, 3), r(3, 500, 3), r(3, 500, 1))      # other shapes, same module: new tables
+    torch.cuda.synchronize()
+    assert torch.isfinite(other).all()
+    outb.zero_()
+    g2.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(outb, refb)

@@ -56,6 +56,68 @@ def test_block_sparse_gaussian(nclusters, per):
     assert_sum_parity(got0[rows], ref0, scale0)
 
 
+def test_config4_block_sparse_100x10k_row_subset():
+    """Headline configuration 4 at its full size: 100 clusters x 10,000 points, seed 3, sigma = 0.1, cluster pairs
+    kept when their centres are closer than 1.0; the oracle evaluates 2048 random rows (CpuReduc_ranges.py:150-228)."""
+    from keops_amd.torch import Genred
+
+    nclusters, per = 100, 10_000
+    c, x, y, b = _clustered(nclusters, per, 3)
+    g = np.array([1 / 0.1**2], np.float32)
+    ranges, keep = _ranges(c, per)
+    M = N = nclusters * per
+    conv = Genred(GAUSS, AL, reduction_op="Sum", axis=1)
+    dev = to_dev(x, y, b, g)
+    rd = tuple(r.cuda() for r in ranges)
+    got = conv(*dev, ranges=rd)
+    rows = np.sort(np.random.default_rng(1).choice(M, 2048, replace=False)).astype(np.int64)
+    r3 = tuple(r.numpy() for r in ranges[:3])
+    ref = cpu_reduc("gauss", [x, y, b, g], M, N, 1, ranges=r3, rows=rows)
+    scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, 1, ranges=r3, rows=rows)
+    assert_sum_parity(got[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
+    # size-independent properties on the full output: exact linearity in b; dropping every range of one row
+    # cluster zeroes exactly its rows and leaves the others bit-identical
+    assert torch.equal(conv(dev[0], dev[1], 2 * dev[2], dev[3], ranges=rd), 2 * got)
+    keep2 = keep.clone()
+    keep2[7, :] = False
+    from keops_amd.torch.cluster import from_matrix
+
+    r = torch.tensor([[per * k, per * (k + 1)] for k in range(nclusters)], dtype=torch.int64)
+    got2 = conv(*dev, ranges=tuple(t.cuda() for t in from_matrix(r, r, keep2)))
+    assert torch.all(got2[7 * per:8 * per] == 0)
+    assert torch.equal(got2[:7 * per], got[:7 * per]) and torch.equal(got2[8 * per:], got[8 * per:])
+
+
+def test_config5a_lse_b16_50k_row_subset():
+    """Headline configuration 5a at its full size: B = 16 batches of 50,000 x 50,000, eps = 0.05, seed 4; the oracle
+    evaluates 128 random rows of every batch."""
+    from keops_amd.torch import Genred
+
+    B, M, N = 16, 50_000, 50_000
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((B, M, 3)).astype(np.float32)
+    y = rng.standard_normal((B, N, 3)).astype(np.float32)
+    l = rng.standard_normal((B, N, 1)).astype(np.float32)
+    e = np.array([1 / 0.05], np.float32)
+    lse = Genred("l-SqDist(x,y)*e", ["x=Vi(3)", "y=Vj(3)", "l=Vj(1)", "e=Pm(1)"], reduction_op="LogSumExp", axis=1)
+    xd, yd, ld, ed = to_dev(x, y, l, e)
+    got = lse(xd, yd, ld, ed)
+    assert tuple(got.shape) == (B, M, 1)
+    pick = np.random.default_rng(44)
+    for bidx in range(B):
+        rows = np.sort(pick.choice(M, 128, replace=False)).astype(np.int64)
+        ms = cpu_reduc("lse_gauss", [x[bidx], y[bidx], l[bidx], e], M, N, 2, reduction="Max_SumShiftExp", rows=rows)
+        ref = ms[:, 0].astype(np.float64) + np.log(ms[:, 1].astype(np.float64))
+        g = got[bidx, torch.from_numpy(rows).cuda(), 0].cpu().numpy()
+        assert np.max(np.abs(g - ref) / np.maximum(1, np.abs(ref))) <= 1e-5, bidx
+    # size-independent property on the full output: LSE(l + c) = LSE(l) + c (c = 4 is exact on these magnitudes up
+    # to one rounding of the sum), and batches are independent: batch 3 alone gives the same bits
+    shifted = lse(xd, yd, ld + 4.0, ed)
+    assert float((shifted - got - 4.0).abs().max()) <= 2e-5
+    alone = lse(xd[3], yd[3], ld[3], ed)
+    assert float((alone - got[3]).abs().max()) <= 2e-5
+
+
 def test_ranges_uncovered_rows_unsorted_and_adjacent_ranges():
     from keops_amd.torch import Genred
 

@@ -244,3 +244,77 @@ def test_row_subset_is_exact():
     full = cpu_reduc("gauss", [x, y, b, g], M, N, 1)
     rows = np.array([5, 17, 199, 0], np.int64)
     assert np.array_equal(cpu_reduc("gauss", [x, y, b, g], M, N, 1, rows=rows), full[rows])
+
+
+def test_kahan_and_double_accumulation_on_an_ill_conditioned_sum():
+    # 10^6 terms of 0.1f: the plain float32 running sum drifts by about 1 %, the compensated sum
+    # and the float64 accumulator must not (a Kahan update with a wrong sign or a dropped compensation fails)
+    N = 1_000_000
+    F = np.full((1, N, 1), 0.1, np.float32)
+    exact = float(np.float32(0.1)) * N  # every term is the same float32 value
+    direct = float(cpu_reduc("dense", [F], 1, N, 1, scheme="direct_sum")[0, 0])
+    kahan = float(cpu_reduc("dense", [F], 1, N, 1, scheme="kahan_scheme")[0, 0])
+    dacc = cpu_reduc("dense", [F], 1, N, 1, scheme="direct_sum", acc_double=True)[0, 0]
+    assert abs(direct - exact) / exact > 1e-4
+    assert abs(kahan - exact) / exact < 1e-7
+    # float64 accumulation of float32 terms, rounded once at the end
+    assert dacc == np.float32(np.sum(F.astype(np.float64)))
+    # block_sum with a float64 accumulator: float32 partial sums of sqrt(N) = 1000 terms, folded in float64
+    blocks = np.float32(0.0)
+    part = np.float32(0.0)
+    for _ in range(1000):
+        part = np.float32(part + np.float32(0.1))
+    want = np.float32(np.float64(part) * 1000)
+    assert cpu_reduc("dense", [F], 1, N, 1, scheme="block_sum", acc_double=True)[0, 0] == want
+    del blocks
+    # compensated log-sum-exp weights (Max_SumShiftExpWeight, kahan_scheme): f = 0 everywhere, weights 0.1f
+    FW = np.concatenate([np.zeros((1, N, 1), np.float32), F], -1)
+    ms_d = cpu_reduc("dense", [FW], 1, N, 2, reduction="Max_SumShiftExpWeight", scheme="direct_sum")[0]
+    ms_k = cpu_reduc("dense", [FW], 1, N, 2, reduction="Max_SumShiftExpWeight", scheme="kahan_scheme")[0]
+    assert ms_k[0] == 0 and abs(float(ms_k[1]) - exact) / exact < 1e-7 and abs(float(ms_d[1]) - exact) / exact > 1e-4
+
+
+def test_l1_bodies_closed_form_and_order():
+    M, N, D, Dv = 23, 41, 37, 2
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((M, D)).astype(np.float32)
+    y = rng.standard_normal((N, D)).astype(np.float32)
+    b = rng.standard_normal((N, Dv)).astype(np.float32)
+    d1 = np.abs(x.astype(np.float64)[:, None, :] - y.astype(np.float64)[None, :, :]).sum(-1)
+    got = cpu_reduc("l1dist", [x, y], M, N, 1, reduction="Min", scheme="direct_sum")
+    assert np.allclose(got[:, 0], d1.min(1), rtol=1e-5)
+    # sequential float32 sum in component order, bit for bit
+    seq = np.zeros((M, N), np.float32)
+    for k in range(D):
+        seq = seq + np.abs(x[:, None, k] - y[None, :, k])
+    assert np.array_equal(got[:, 0], seq.min(1))
+    ker = cpu_reduc("exp_l1", [x / 8, y / 8, b], M, N, Dv)
+    ref = np.exp(-d1 / 8) @ b.astype(np.float64)
+    assert np.linalg.norm(ker - ref) / np.linalg.norm(ref) < 2e-6
+    # transposed operands or a squared difference would change the answer
+    assert not np.allclose(ker, np.exp(-(d1 / 8) ** 2) @ b.astype(np.float64), rtol=1e-3)
+
+
+def test_scalprod_body_uses_a_fused_multiply_add_chain():
+    M, N, D, Dv = 9, 31, 50, 3
+    rng = np.random.default_rng(13)
+    x = rng.standard_normal((M, D)).astype(np.float32)
+    y = rng.standard_normal((N, D)).astype(np.float32)
+    b = rng.standard_normal((N, Dv)).astype(np.float32)
+    got = cpu_reduc("scalprod", [x, y, b], M, N, Dv)
+    ref = (x.astype(np.float64) @ y.astype(np.float64).T) @ b.astype(np.float64)
+    assert np.linalg.norm(got - ref) / np.linalg.norm(ref) < 2e-6
+    # one pair, two components [1, a].[-rn(a*a), a]: the chain fma(a, a, fma(1, -r, 0)) returns the exact
+    # residual a*a - rn(a*a); separate multiply and add would return 0, the reverse order too
+    a = np.float32(1.0 + 2.0 ** -12 + 2.0 ** -20)
+    r = np.float32(a * a)
+    resid = float(np.float64(a) * np.float64(a) - np.float64(r))
+    assert resid != 0.0
+    xx = np.array([[1.0, a]], np.float32)
+    yy = np.array([[-r, a]], np.float32)
+    one = np.ones((1, 1), np.float32)
+    assert float(cpu_reduc("scalprod", [xx, yy, one], 1, 1, 1)[0, 0]) == np.float32(resid)
+    # float64 twin
+    x64, y64, b64 = x.astype(np.float64), y.astype(np.float64), b.astype(np.float64)
+    got64 = cpu_reduc("scalprod", [x64, y64, b64], M, N, Dv, dtype=np.float64)
+    assert np.allclose(got64, ref, rtol=1e-13, atol=1e-13)
