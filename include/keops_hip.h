@@ -124,7 +124,7 @@ double keops_hip_module_last_kernel_ms(void* module);
  * chains, and returns the elapsed time in ms and the counted instructions per wavefront.
  *   kind 0: v_fmac_f32 only (8 per chain and round); kind 1: the 9-instruction mix of a Gaussian pair (3 sub,
  *   mul, 2 fma, mul, v_exp_f32, fma); kind 2: the same without v_exp_f32; kind 3: v_mfma_f32_32x32x16_bf16
- *   (4 per chain and round).  chains: 1, 2, 4, 8 (kinds 0-2) or 1, 2, 4 (kind 3).
+ *   (4 per chain and round); kind 4: v_mfma_f32_32x32x16_f16.  chains: 1, 2, 4, 8 (kinds 0-2) or 1, 2, 4 (kinds 3, 4).
  * Measurement aid without counterpart in the reference; used by bench.py --valu-calibration / --mfma-calibration.
  */
 int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave);

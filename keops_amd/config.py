@@ -31,7 +31,11 @@ lse_group = int(os.environ.get("KEOPS_AMD_LSE_GROUP", 8))  # log-sum-exp: column
 chunk_waves = int(os.environ.get("KEOPS_AMD_CHUNK_WAVES", 8))
 chunk_presplit = os.environ.get("KEOPS_AMD_CHUNK_PRESPLIT", "1") != "0"  # dense launches: pre-split copy of the weights
 chunk_min_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MIN_DIM", 24))    # smallest contraction served by the matrix-core chunked scheme
-chunk_near = float(os.environ.get("KEOPS_AMD_CHUNK_NEAR", 0.125))     # squared distances below this fraction of |x|^2+|y|^2 are recomputed in float32 (0: never)
+# squared distances below this fraction of |x|^2+|y|^2 are recomputed in float32 (0: never).  Default: 1/4, which
+# bounds the relative error of every squared distance by 4 * 1.4e-7 (the expansion is off by about 1.4e-7 of the
+# norms), the order of the rounding of the reference's own float32 sum; 1/8 below 32 components, where random pairs
+# come that close often enough for the recomputation to cost more than it is worth (+50 % at D = 24)
+chunk_near = os.environ.get("KEOPS_AMD_CHUNK_NEAR", "auto")
 chunk_max_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MAX_DIM", 1024))  # largest contraction served by the matrix-core chunked scheme
 
 # matrix-core final-product scheme (csrc/kernels/keops_final_mfma.h): Sum_j f(x_i,y_j) * v_j with dim(v) large

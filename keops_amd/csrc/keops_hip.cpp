@@ -773,6 +773,7 @@ struct ChkHeader {
   int32_t pad_;
   int64_t nxs, nys;
   void* vsplit;
+  void* scal;
   RangeHeader rt;
 };
 
@@ -787,7 +788,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(128, nys / 64));
   const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
   const size_t o_xs = take((size_t)nxs * DP * 4), o_ys = take((size_t)nys * DP * 4);
-  const size_t o_xn = take((size_t)nxs * 4), o_yn = take((size_t)nys * 4);
+  const size_t o_xn = take((size_t)nxs * 4), o_yn = take((size_t)nys * 4), o_scal = take(8);
   // final-product variant: slabs over the reduced axis fill the chip and round the grid to whole
   // rounds of workgroups (one 8-wavefront workgroup per CU, all taking the same time)
   const bool softmax = m.meta_int("chk_softmax", 0) != 0;
@@ -833,7 +834,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   ChkHeader h{};
   h.nx = nx; h.ny = ny; h.xs = ws + o_xs; h.ys = ws + o_ys; h.xn = ws + o_xn; h.yn = ws + o_yn; h.colsum = ws + o_colsum;
   h.colpart = ws + o_colpart; h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs;
-  h.nxs = nxs; h.nys = nys;
+  h.nxs = nxs; h.nys = nys; h.scal = ws + o_scal;
   if (split3) h.vsplit = ws + o_vsplit;
   if (rg) h.rt = rg->header(m.nargs);
   if (knn_inner > 0) h.out = ws + o_lists;
@@ -847,6 +848,13 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
     const size_t szp = with_which(nparts);
     const int64_t cw = D > 128 ? 256 : (D > 64 ? 128 : (D > 32 ? 64 : 32));  // CHK_CW: columns per workgroup
     if (int rc = launch_raw(m, "keops_chk_colsum_final", (unsigned)((DP + cw - 1) / cw), 1, 256, buf.data(), szp, stream)) return rc;
+  }
+  // power-of-two scales of the half-precision operands: largest |component| of both arguments
+  if (int e = keops_static_fill_zero(ws + o_scal, 8, stream)) return fail(e, std::string("zero fill failed: ") + hipGetErrorString((hipError_t)e));
+  {
+    const int64_t elems = std::max(nxs, nys) * D;
+    const unsigned gb = (unsigned)std::max<int64_t>(1, std::min<int64_t>(2048, (elems + 256 * 8 - 1) / (256 * 8)));
+    if (int rc = launch_raw(m, "keops_chk_absmax", gb, 1, 256, buf.data(), psize, stream)) return rc;
   }
   const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
   size_t sz = with_which(0);

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 #include "keops_static.h"
 
@@ -63,16 +64,24 @@ static __global__ void __launch_bounds__(256) keops_valu_loop(float* out, int it
 
 typedef float keops_f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 keops_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 keops_f16x8 __attribute__((ext_vector_type(8)));
 
-// `iters` rounds of CHAINS independent v_mfma_f32_32x32x16_bf16 accumulation chains per wavefront
-template <int CHAINS>
+// `iters` rounds of CHAINS independent v_mfma_f32_32x32x16_bf16 (HALF = 0) or _f16 (HALF = 1) accumulation chains per
+// wavefront; the operands carry full-width random significands (the power drawn, hence the sustained clock,
+// depends on the data)
+template <int CHAINS, int HALF>
 static __global__ void __launch_bounds__(256) keops_mfma_loop(float* out, int iters) {
   keops_f32x16 acc[CHAINS];
-  keops_bf16x8 a, b;
+  typedef typename std::conditional<HALF == 1, keops_f16x8, keops_bf16x8>::type vec8;
+  typedef typename std::conditional<HALF == 1, _Float16, __bf16>::type elem;
+  vec8 a, b;
+  unsigned h = 0x9e3779b9u * (threadIdx.x + 1u);
 #pragma unroll
   for (int e = 0; e < 8; e++) {
-    a[e] = (__bf16)(1.0f + (float)((threadIdx.x + e) & 3));
-    b[e] = (__bf16)(0.5f);
+    h = h * 1664525u + 1013904223u;
+    a[e] = (elem)(1.0f + (float)(h >> 8) * (1.0f / 16777216.0f));
+    h = h * 1664525u + 1013904223u;
+    b[e] = (elem)(((h & 1u) ? -1.0f : 1.0f) * (0.5f + (float)(h >> 8) * (0.5f / 16777216.0f)));
   }
 #pragma unroll
   for (int k = 0; k < CHAINS; k++)
@@ -82,7 +91,10 @@ static __global__ void __launch_bounds__(256) keops_mfma_loop(float* out, int it
 #pragma unroll
     for (int u = 0; u < 4; u++)
 #pragma unroll
-      for (int k = 0; k < CHAINS; k++) acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[k], 0, 0, 0);
+      for (int k = 0; k < CHAINS; k++) {
+        if constexpr (HALF == 1) acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[k], 0, 0, 0);
+        else acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[k], 0, 0, 0);
+      }
   }
   float r = 0.f;
 #pragma unroll
@@ -93,7 +105,7 @@ static __global__ void __launch_bounds__(256) keops_mfma_loop(float* out, int it
 }
 
 // Runs one calibration loop on `stream`: grid of `blocks` workgroups of 256 lanes (4 wavefronts), `iters` rounds.
-// kind 0/1/2: vector loop with MIX = kind; kind 3: matrix loop.  chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
+// kind 0/1/2: vector loop with MIX = kind; kind 3 / 4: matrix loop on bf16 / f16 operands.  chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
 // instr_per_lane receives the number of counted instructions one wavefront issues (vector: per lane = per wavefront
 // instruction count; matrix: v_mfma instructions).  out must hold blocks * 256 floats.
 int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* out, void* stream, double* instr_per_wave) {
@@ -113,12 +125,15 @@ int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* o
       if (chains == 1) VALU_CASE(1, 2); else if (chains == 2) VALU_CASE(2, 2); else if (chains == 4) VALU_CASE(4, 2);
       else if (chains == 8) VALU_CASE(8, 2); else return (int)hipErrorInvalidValue;
     }
-  } else if (kind == 3) {
+  } else if (kind == 3 || kind == 4) {
     *instr_per_wave = 4.0 * chains * (double)iters;
-    if (chains == 1) hipLaunchKernelGGL((keops_mfma_loop<1>), g, b, 0, s, out, iters);
-    else if (chains == 2) hipLaunchKernelGGL((keops_mfma_loop<2>), g, b, 0, s, out, iters);
-    else if (chains == 4) hipLaunchKernelGGL((keops_mfma_loop<4>), g, b, 0, s, out, iters);
+#define MFMA_CASE(C) do { if (kind == 3) hipLaunchKernelGGL((keops_mfma_loop<C, 0>), g, b, 0, s, out, iters); \
+                          else hipLaunchKernelGGL((keops_mfma_loop<C, 1>), g, b, 0, s, out, iters); } while (0)
+    if (chains == 1) MFMA_CASE(1);
+    else if (chains == 2) MFMA_CASE(2);
+    else if (chains == 4) MFMA_CASE(4);
     else return (int)hipErrorInvalidValue;
+#undef MFMA_CASE
   } else {
     return (int)hipErrorInvalidValue;
   }

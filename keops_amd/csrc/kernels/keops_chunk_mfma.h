@@ -9,15 +9,17 @@
 // become a scalar variable.  Here the chunked sub-formula
 //     s_ij = SqDist(x_i, y_j) = |x_i|^2 + |y_j|^2 - 2 <x_i, y_j>      (CHK_MODE 0)
 //     s_ij = <x_i, y_j>                                                (CHK_MODE 1)
-// is produced for a 32 x 32 tile of pairs by v_mfma_f32_32x32x16_bf16, and the post-chunk formula
+// is produced for a 32 x 32 tile of pairs by v_mfma_f32_32x32x16_f16, and the post-chunk formula
 // F'(s_ij, other variables) is the generated straight-line code of KeopsFormula::eval.
 //
-// Precision: every float32 operand is split once as x = hi + lo with hi = bf16(x), lo = bf16(x - hi)
-// (a 16-bit significand in total) and <x, y> is accumulated in float32 from the three products
-// hi*hi + hi*lo + lo*hi; the dropped lo*lo term and the split residuals are below 2^-16 |x||y|.
-// For SqDist the rows are first centred on the column mean of y, which keeps |x|^2 + |y|^2 - 2<x,y>
-// well conditioned.  This is the accuracy class of the fast-math build; with use_fast_math=False
-// the engine does not select this scheme.
+// Precision: every float32 operand is split once as x = hi + lo with hi = half(a x), lo = half(a x - hi)
+// (two 11-bit significands, 22 bits in total; a is a power of two chosen per launch from the largest
+// component so that the terms sit high in the half-precision range: keops_chk_absmax, chk_pow2_scale) and
+// <x, y> is accumulated in float32 from the three products hi*hi + hi*lo + lo*hi; the dropped lo*lo term and
+// the split residuals are below 3 * 2^-22 |x||y| = 7.2e-7 |x||y|.  For SqDist the rows are first centred on the
+// column mean of y, which keeps |x|^2 + |y|^2 - 2<x,y> well conditioned: the squared distance is off by at
+// most 7.2e-7 (|x^|^2 + |y^|^2), the order of what the float32 sum of D squared differences of the reference
+// itself carries (sqrt(D) 2^-24 s).  With use_fast_math=False the engine does not select this scheme.
 //
 // Work decomposition: a wavefront owns 32 output rows ("queries") whose split operands stay in
 // VGPRs as the MFMA B matrix; the workgroup stages 32 reduced rows at a time in LDS (A matrix plus
@@ -46,6 +48,9 @@
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 chk_bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 chk_bf16x4;
+typedef _Float16 chk_half;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 chk_h8;
+typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 chk_h4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float chk_f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float chk_f32x4;
 
@@ -57,15 +62,15 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float chk_f32x4;
 #define CHK_KB (CHK_DPAD / 16)
 #define CHK_KBC (CHK_KB / CHK_NC)            // 16-wide k blocks per wavefront
 #define CHK_VS (16 / CHK_NC)                 // values of a 32 x 32 tile each lane evaluates
-#define CHK_ROWBYTES (CHK_DPAD * 4)          // hi part then lo part, bf16 each
+#define CHK_ROWBYTES (CHK_DPAD * 4)          // hi part then lo part, half precision each
 #define CHK_STRIDE (CHK_ROWBYTES + 16)       // padded LDS row
 #define CHK_TJ 32                            // reduced rows per staged tile
 #define CHK_DY (KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1)
 
 struct ChkParams {
   i64 nx, ny;           // output rows, reduced rows
-  __bf16* xs;           // [nx][2*CHK_DPAD] split (and centred, scaled) rows of the chunked row variable
-  __bf16* ys;           // [ny][2*CHK_DPAD]
+  chk_half* xs;         // [nx][2*CHK_DPAD] split (and centred, scaled) rows of the chunked row variable
+  chk_half* ys;         // [ny][2*CHK_DPAD]
   float* xn;            // [nx] |x - mu|^2      (CHK_MODE 0)
   float* yn;            // [ny]
   float* colsum;        // [CHK_DPAD]
@@ -77,6 +82,7 @@ struct ChkParams {
   int pad_;
   i64 nxs, nys;         // rows of the chunked row / column arguments (fewer than nx, ny when a batch dimension is broadcast)
   __bf16* vsplit;       // CHK_SPLIT3: v as three bfloat16 terms, [tile][term][column][CHK_TS positions]
+  float* scal;          // [2] largest |component| of the chunked row / column arguments (bit patterns, keops_chk_absmax)
   KeopsRangeTables rt;  // block-sparse / batch geometry (KEOPS_MC_RANGES)
   const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
 };
@@ -95,7 +101,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum(const ChkPara
   const i64 rows_per_block = (P.nys + gridDim.x - 1) / gridDim.x;
   const i64 r0 = (i64)blockIdx.x * rows_per_block, r1 = keops_min(P.nys, r0 + rows_per_block);
   const T* y = P.arg[CHK_YARG];
-  for (int c0 = blockIdx.x * CHK_CW; c0 < CHK_DPAD; c0 += gridDim.x * CHK_CW) {
+  for (int c0 = 0; c0 < CHK_DPAD; c0 += CHK_CW) {  // every workgroup: all columns of its own rows
     const int c = c0 + cw;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     if (c < CHK_D) {
@@ -124,7 +130,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum_final(const C
   __shared__ float part[256];
   constexpr int RG = 256 / CHK_CW;
   const int cw = threadIdx.x % CHK_CW, rg = threadIdx.x / CHK_CW;
-  for (int c0 = 0; c0 < CHK_DPAD; c0 += CHK_CW) {
+  for (int c0 = blockIdx.x * CHK_CW; c0 < CHK_DPAD; c0 += gridDim.x * CHK_CW) {  // one group of columns per workgroup
     const int c = c0 + cw;
     // eight interleaved partial sums, added in a fixed order: the loads of one thread do not wait for each other
     float s8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -149,6 +155,45 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum_final(const C
   }
 }
 
+// Largest |component| of the two chunked arguments: atomic maximum on the bit patterns of non-negative floats
+// (order-independent, hence deterministic).  The host zeroes P.scal before the launch.
+extern "C" __global__ void __launch_bounds__(256) keops_chk_absmax(const ChkParams P) {
+  const T* x = P.arg[CHK_XARG];
+  const T* y = P.arg[CHK_YARG];
+  const i64 nxe = P.nxs * CHK_D, nye = P.nys * CHK_D, step = (i64)gridDim.x * 256;
+  float mx = 0.f, my = 0.f;
+  for (i64 e = (i64)blockIdx.x * 256 + threadIdx.x; e < nxe; e += step) mx = __builtin_fmaxf(mx, __builtin_fabsf((float)x[e]));
+  for (i64 e = (i64)blockIdx.x * 256 + threadIdx.x; e < nye; e += step) my = __builtin_fmaxf(my, __builtin_fabsf((float)y[e]));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mx = __builtin_fmaxf(mx, __shfl_xor(mx, o));
+    my = __builtin_fmaxf(my, __shfl_xor(my, o));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    atomicMax(reinterpret_cast<unsigned*>(P.scal), __float_as_uint(mx));
+    atomicMax(reinterpret_cast<unsigned*>(P.scal) + 1, __float_as_uint(my));
+  }
+}
+
+// Power of two that brings components bounded by B into [2^12, 2^13) (1 for B = 0, clamped to 2^+-60): the split
+// terms then sit high in the half-precision range (lo terms stay normal down to components 2^-15 of the largest,
+// below that they lose absolute accuracy 2^-25 against a largest component of 2^12) and nothing can overflow
+// (|-2 a x| < 2^14, products < 2^27 per component, accumulated in float32).
+__device__ __forceinline__ float chk_pow2_scale(float B) {
+  const int e = (int)((__float_as_uint(B) >> 23) & 0xffu);
+  if (e == 0 || e == 255) return 1.f;
+  int t = 266 - e;  // 127 + 12 - (e - 127)
+  t = t < 67 ? 67 : (t > 187 ? 187 : t);
+  return __uint_as_float((unsigned)t << 23);
+}
+// scales of the row (which = 0) and column (1) operands.  Centred rows (CHK_MODE 0) are bounded by
+// |x| + |mean y| <= max|x| + max|y| and |y| + |mean y| <= 2 max|y|.
+__device__ __forceinline__ float chk_operand_scale(const float* scal, int which) {
+  const float ax = scal[0], ay = scal[1];
+  if (CHK_MODE == 0) return chk_pow2_scale(which ? 2.f * ay : ax + ay);
+  return chk_pow2_scale(which ? ay : ax);
+}
+
 // One row per group of CHK_LPR lanes, 4 columns per lane and pass; which = 0: row variable (stored times -2
 // in CHK_MODE 0), 1: column variable.  The squared norm is reduced inside the lane group
 // (deterministic).
@@ -156,15 +201,15 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum_final(const C
 extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams P, int which) {
   const i64 n = which ? P.nys : P.nxs;
   const T* src = P.arg[which ? CHK_YARG : CHK_XARG];
-  __bf16* dst = which ? P.ys : P.xs;
+  chk_half* dst = which ? P.ys : P.xs;
   const int q = threadIdx.x % CHK_LPR;
   const i64 row = ((i64)blockIdx.x * 256 + threadIdx.x) / CHK_LPR;
   const bool live = row < n;
   const float inv = 1.0f / (float)P.nys;
-  const float scale = (CHK_MODE == 0 && !which) ? -2.0f : 1.0f;
+  const float scale = ((CHK_MODE == 0 && !which) ? -2.0f : 1.0f) * chk_operand_scale(P.scal, which);
   float nrm = 0.f;
   for (int c0 = q * 4; c0 < CHK_DPAD && live; c0 += CHK_LPR * 4) {
-    chk_bf16x4 hi, lo;
+    chk_h4 hi, lo;
 #pragma unroll
     for (int e = 0; e < 4; e++) {
       const int c = c0 + e;
@@ -175,22 +220,24 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
       }
       nrm += v * v;
       v *= scale;
-      hi[e] = (__bf16)v;
-      lo[e] = (__bf16)(v - (float)hi[e]);
+      hi[e] = (_Float16)v;
+      lo[e] = (_Float16)(v - (float)hi[e]);
     }
-    *reinterpret_cast<chk_bf16x4*>(dst + row * 2 * CHK_DPAD + c0) = hi;
-    *reinterpret_cast<chk_bf16x4*>(dst + row * 2 * CHK_DPAD + CHK_DPAD + c0) = lo;
+    *reinterpret_cast<chk_h4*>(dst + row * 2 * CHK_DPAD + c0) = hi;
+    *reinterpret_cast<chk_h4*>(dst + row * 2 * CHK_DPAD + CHK_DPAD + c0) = lo;
   }
 #pragma unroll
   for (int o = CHK_LPR / 2; o > 0; o >>= 1) nrm += __shfl_xor(nrm, o, CHK_LPR);
   if (CHK_MODE == 0 && live && q == 0) (which ? P.yn : P.xn)[row] = nrm;
 }
 
-// Squared distances come out of the expansion |x^|^2 + |y^|^2 - 2 <x^, y^> with 16-bit operands: an absolute error
-// of about 2^-17 (|x^|^2 + |y^|^2), harmless unless the pair is close compared with the norms (identical or
-// neighbouring points, kernels much narrower than the cloud), where it would be a large relative error.  A value
-// below 1/8 of the sum of the squared norms is therefore recomputed from the float32 rows.  In high dimension
-// random pairs never come that close, so the branch costs one compare; clustered data pay for their accuracy.
+// Squared distances come out of the expansion |x^|^2 + |y^|^2 - 2 <x^, y^> with 22-bit operands and float32
+// accumulation: an absolute error of about 1.4e-7 (|x^|^2 + |y^|^2) (bound: 7.2e-7), harmless unless the pair is
+// close compared with the norms (identical or neighbouring points, kernels narrower than the cloud), where it would
+// be a large relative error.  A value below CHK_NEAR (1/4; 1/8 below 32 components) of the sum of the squared
+// norms is therefore recomputed from the float32 rows: every squared distance is then good to a relative 6e-7, the
+// order of the rounding of the reference's own float32 sum of D squared differences.  In high dimension random
+// pairs never come that close, so the branch costs one compare; clustered data pay for their accuracy.
 #ifndef CHK_NEAR
 #define CHK_NEAR 0.125f
 #endif
@@ -242,6 +289,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
   constexpr int MERGE_BYTES = (int)sizeof(TACC) * CHK_QB * (2 * CHK_NC - 1) * KEOPS_DIMRED;
   __shared__ __attribute__((aligned(16))) unsigned char as[TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES];
   __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
+  __shared__ __attribute__((aligned(16))) float yns_s[CHK_TJ];  // the same norms times chk_sc: initial value of the s tile
   __shared__ __attribute__((aligned(16))) T yo_s[CHK_TJ * CHK_DY];                // other column variables
   TACC (*merge_s)[2 * CHK_NC - 1][KEOPS_DIMRED] = reinterpret_cast<TACC (*)[2 * CHK_NC - 1][KEOPS_DIMRED]>(as);
 #if CHK_NC > 1
@@ -263,14 +311,16 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
   const i64 qx = G.row(CHK_XARG, q);
 
   // B operands: split rows of the chunked row variable
-  chk_bf16x8 bh[CHK_KBC], bl[CHK_KBC];
+  chk_h8 bh[CHK_KBC], bl[CHK_KBC];
 #pragma unroll
   for (int kb = 0; kb < CHK_KBC; kb++) {
     const int k0 = (chunk * CHK_KBC + kb) * 16 + 8 * half;
-    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + k0);
-    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + k0);
+    bh[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + k0);
+    bl[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + k0);
   }
   const float xnq = CHK_MODE == 0 ? P.xn[qx] : 0.f;
+  // the tile comes out of the matrix cores times chk_sc (a power of two: the scales of the two operands)
+  const float chk_sc = chk_operand_scale(P.scal, 0) * chk_operand_scale(P.scal, 1), chk_inv = 1.0f / chk_sc;
   // other row variables and parameters of the post-chunk formula
   T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
 #pragma unroll
@@ -337,7 +387,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
         *reinterpret_cast<uint4*>(as + row * CHK_STRIDE + c * 16) = pf[u];
       }
     }
-    if (CHK_MODE == 0 && tid < CHK_TJ) yn_s[tid] = pfn;
+    if (CHK_MODE == 0 && tid < CHK_TJ) { yn_s[tid] = pfn; yns_s[tid] = pfn * chk_sc; }
     // the other reduced-index variables of this tile (small: loaded directly)
 #pragma unroll
     for (int v = 0; v < KEOPS_NCOLVARS; v++) {
@@ -364,7 +414,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
     if (CHK_MODE == 0) {
       chk_f32x4 kk[4];
 #pragma unroll
-      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const chk_f32x4*>(yn_s + 8 * b + 4 * half);
+      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const chk_f32x4*>(yns_s + 8 * b + 4 * half);
 #pragma unroll
       for (int v = 0; v < 16; v++) s[v] = kk[v >> 2][v & 3];
     } else {
@@ -374,11 +424,11 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
     const unsigned char* arow = as + col * CHK_STRIDE + 16 * half;
 #pragma unroll
     for (int kb = 0; kb < CHK_KB; kb++) {
-      const chk_bf16x8 ah = *reinterpret_cast<const chk_bf16x8*>(arow + kb * 32);
-      const chk_bf16x8 al = *reinterpret_cast<const chk_bf16x8*>(arow + CHK_DPAD * 2 + kb * 32);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[kb], s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
+      const chk_h8 ah = *reinterpret_cast<const chk_h8*>(arow + kb * 32);
+      const chk_h8 al = *reinterpret_cast<const chk_h8*>(arow + CHK_DPAD * 2 + kb * 32);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[kb], s, 0, 0, 0);
     }
 #else
     // partial tile of this wavefront's k blocks, handed to the group through LDS
@@ -389,11 +439,11 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
       const unsigned char* arow = as + col * CHK_STRIDE + 16 * half + chunk * CHK_KBC * 32;
 #pragma unroll
       for (int kb = 0; kb < CHK_KBC; kb++) {
-        const chk_bf16x8 ah = *reinterpret_cast<const chk_bf16x8*>(arow + kb * 32);
-        const chk_bf16x8 al = *reinterpret_cast<const chk_bf16x8*>(arow + CHK_DPAD * 2 + kb * 32);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[kb], s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
+        const chk_h8 ah = *reinterpret_cast<const chk_h8*>(arow + kb * 32);
+        const chk_h8 al = *reinterpret_cast<const chk_h8*>(arow + CHK_DPAD * 2 + kb * 32);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[kb], s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[kb], s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[kb], s, 0, 0, 0);
       }
 #pragma unroll
       for (int v = 0; v < 16; v++) xch[(wave * 16 + v) * 64 + lane] = s[v];
@@ -405,7 +455,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
 #pragma unroll
     for (int vv = 0; vv < CHK_VS; vv++) {
       const int v = chunk * CHK_VS + vv;
-      float t = CHK_MODE == 0 ? yn_s[8 * (v >> 2) + 4 * half + (v & 3)] : 0.f;
+      float t = CHK_MODE == 0 ? yns_s[8 * (v >> 2) + 4 * half + (v & 3)] : 0.f;
 #pragma unroll
       for (int c = 0; c < CHK_NC; c++) t += xch[((grp * CHK_NC + c) * 16 + v) * 64 + lane];
       s[vv] = t;
@@ -417,7 +467,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
 #endif
     float sq[CHK_VS];
 #pragma unroll
-    for (int vv = 0; vv < CHK_VS; vv++) sq[vv] = CHK_MODE == 0 ? __builtin_fmaxf(s[vv] + xnq, 0.f) : s[vv];
+    for (int vv = 0; vv < CHK_VS; vv++) sq[vv] = CHK_MODE == 0 ? __builtin_fmaxf(__builtin_fmaf(s[vv], chk_inv, xnq), 0.f) : s[vv] * chk_inv;
     if (CHK_MODE == 0) chk_fix_near<CHK_VS>(P, sq, chunk * CHK_VS, half, n, xnq, yn_s, near_bound, qx, jy0);
 #pragma unroll
     for (int vv = 0; vv < CHK_VS; vv++) {
@@ -724,6 +774,7 @@ __device__ __forceinline__ void chk_v3_product(const float (&w)[16], const __bf1
 extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const ChkParams P) {
   __shared__ __attribute__((aligned(16))) unsigned char as[CHK_TJ * CHK_STRIDE];  // A tile (hi|lo)
   __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
+  __shared__ __attribute__((aligned(16))) float yns_s[CHK_TJ];  // the same norms times chk_sc: initial value of the s tile
   __shared__ __attribute__((aligned(16))) T yo_s[CHK_TJ * CHK_DY];                // other column variables of g
 #if CHK_V3
   __shared__ __attribute__((aligned(16))) __bf16 bt3[3 * CHK_VCOLS * CHK_TS];       // v tile in three terms
@@ -741,13 +792,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
   if (q >= G.row_end) q = G.row_end - 1;
   const i64 qx = G.row(CHK_XARG, q);  // clamped rows compute, never store
 
-  chk_bf16x8 bh[CHK_KB], bl[CHK_KB];
+  chk_h8 bh[CHK_KB], bl[CHK_KB];
 #pragma unroll
   for (int kb = 0; kb < CHK_KB; kb++) {
-    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + kb * 16 + 8 * half);
-    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+    bh[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + kb * 16 + 8 * half);
+    bl[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
   }
   const float xnq = CHK_MODE == 0 ? P.xn[qx] : 0.f;
+  // the tile comes out of the matrix cores times chk_sc (a power of two: the scales of the two operands)
+  const float chk_sc = chk_operand_scale(P.scal, 0) * chk_operand_scale(P.scal, 1), chk_inv = 1.0f / chk_sc;
   T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NROWVARS; v++) {
@@ -852,7 +905,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
         *reinterpret_cast<uint4*>(as + row * CHK_STRIDE + c * 16) = pf[u];
       }
     }
-    if (CHK_MODE == 0 && tid < CHK_TJ) yn_s[tid] = pfn;
+    if (CHK_MODE == 0 && tid < CHK_TJ) { yn_s[tid] = pfn; yns_s[tid] = pfn * chk_sc; }
 #pragma unroll
     for (int v = 0; v < KEOPS_NCOLVARS; v++) {
       const int dim = keops_col_dim[v];
@@ -883,7 +936,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
     if (CHK_MODE == 0) {
       chk_f32x4 kk[4];
 #pragma unroll
-      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const chk_f32x4*>(yn_s + 8 * b + 4 * half);
+      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const chk_f32x4*>(yns_s + 8 * b + 4 * half);
 #pragma unroll
       for (int v = 0; v < 16; v++) s[v] = kk[v >> 2][v & 3];
     } else {
@@ -893,15 +946,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
     const unsigned char* arow = as + col * CHK_STRIDE + 16 * half;
 #pragma unroll
     for (int kb = 0; kb < CHK_KB; kb++) {
-      const chk_bf16x8 ah = *reinterpret_cast<const chk_bf16x8*>(arow + kb * 32);
-      const chk_bf16x8 al = *reinterpret_cast<const chk_bf16x8*>(arow + CHK_DPAD * 2 + kb * 32);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[kb], s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
+      const chk_h8 ah = *reinterpret_cast<const chk_h8*>(arow + kb * 32);
+      const chk_h8 al = *reinterpret_cast<const chk_h8*>(arow + CHK_DPAD * 2 + kb * 32);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[kb], s, 0, 0, 0);
     }
     float sq[16];
 #pragma unroll
-    for (int v = 0; v < 16; v++) sq[v] = CHK_MODE == 0 ? __builtin_fmaxf(s[v] + xnq, 0.f) : s[v];
+    for (int v = 0; v < 16; v++) sq[v] = CHK_MODE == 0 ? __builtin_fmaxf(__builtin_fmaf(s[v], chk_inv, xnq), 0.f) : s[v] * chk_inv;
     if (CHK_MODE == 0) chk_fix_near<16>(P, sq, 0, half, n, xnq, yn_s, near_bound, qx, jy0);
 #if CHK_V3
     float gw[16];
@@ -972,6 +1025,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_reduce(const ChkPara
 extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const ChkParams P) {
   __shared__ __attribute__((aligned(16))) unsigned char as[CHK_TJ * CHK_STRIDE];
   __shared__ __attribute__((aligned(16))) float yn_s[CHK_TJ];
+  __shared__ __attribute__((aligned(16))) float yns_s[CHK_TJ];  // the same norms times chk_sc: initial value of the s tile
   __shared__ __attribute__((aligned(16))) T yo_s[CHK_TJ * CHK_DY];
 #if CHK_V3
   __shared__ __attribute__((aligned(16))) __bf16 bt3[3 * CHK_VCOLS * CHK_TS];       // v tile in three terms
@@ -990,13 +1044,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
   if (q >= G.row_end) q = G.row_end - 1;
   const i64 qx = G.row(CHK_XARG, q);
 
-  chk_bf16x8 bh[CHK_KB], bl[CHK_KB];
+  chk_h8 bh[CHK_KB], bl[CHK_KB];
 #pragma unroll
   for (int kb = 0; kb < CHK_KB; kb++) {
-    bh[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + kb * 16 + 8 * half);
-    bl[kb] = *reinterpret_cast<const chk_bf16x8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+    bh[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + kb * 16 + 8 * half);
+    bl[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
   }
   const float xnq = CHK_MODE == 0 ? P.xn[qx] : 0.f;
+  // the tile comes out of the matrix cores times chk_sc (a power of two: the scales of the two operands)
+  const float chk_sc = chk_operand_scale(P.scal, 0) * chk_operand_scale(P.scal, 1), chk_inv = 1.0f / chk_sc;
   T xi[KEOPS_DIMX > 0 ? KEOPS_DIMX : 1];
 #pragma unroll
   for (int v = 0; v < KEOPS_NROWVARS; v++) {
@@ -1080,7 +1136,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
         *reinterpret_cast<uint4*>(as + row * CHK_STRIDE + c * 16) = pf[u];
       }
     }
-    if (CHK_MODE == 0 && tid < CHK_TJ) yn_s[tid] = pfn;
+    if (CHK_MODE == 0 && tid < CHK_TJ) { yn_s[tid] = pfn; yns_s[tid] = pfn * chk_sc; }
 #pragma unroll
     for (int v = 0; v < KEOPS_NCOLVARS; v++) {
       const int dim = keops_col_dim[v];
@@ -1111,7 +1167,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
     if (CHK_MODE == 0) {
       chk_f32x4 kk[4];
 #pragma unroll
-      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const chk_f32x4*>(yn_s + 8 * b + 4 * half);
+      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const chk_f32x4*>(yns_s + 8 * b + 4 * half);
 #pragma unroll
       for (int v = 0; v < 16; v++) s[v] = kk[v >> 2][v & 3];
     } else {
@@ -1121,15 +1177,15 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
     const unsigned char* arow = as + col * CHK_STRIDE + 16 * half;
 #pragma unroll
     for (int kb = 0; kb < CHK_KB; kb++) {
-      const chk_bf16x8 ah = *reinterpret_cast<const chk_bf16x8*>(arow + kb * 32);
-      const chk_bf16x8 al = *reinterpret_cast<const chk_bf16x8*>(arow + CHK_DPAD * 2 + kb * 32);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh[kb], s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl[kb], s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh[kb], s, 0, 0, 0);
+      const chk_h8 ah = *reinterpret_cast<const chk_h8*>(arow + kb * 32);
+      const chk_h8 al = *reinterpret_cast<const chk_h8*>(arow + CHK_DPAD * 2 + kb * 32);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[kb], s, 0, 0, 0);
     }
     float sq[16];
 #pragma unroll
-    for (int v = 0; v < 16; v++) sq[v] = CHK_MODE == 0 ? __builtin_fmaxf(s[v] + xnq, 0.f) : s[v];
+    for (int v = 0; v < 16; v++) sq[v] = CHK_MODE == 0 ? __builtin_fmaxf(__builtin_fmaf(s[v], chk_inv, xnq), 0.f) : s[v] * chk_inv;
     if (CHK_MODE == 0) chk_fix_near<16>(P, sq, 0, half, n, xnq, yn_s, near_bound, qx, jy0);
     // F' for the lane's 16 pairs (rows past the end: -inf, they weigh nothing) and the tile maximum
     float mx = ninf;

@@ -590,7 +590,8 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
     elif softmax is not None:
         defs.update(KEOPS_DIMFOUT=full_post.dim, CHK_SOFTMAX=1, CHK_SM_ONE=softmax[2], CHK_FV_ARG=softmax[1].ind,
                     CHK_FV_DIM=softmax[1].dim, CHK_FNB=-(-softmax[1].dim // 32))
-    defs["CHK_NEAR"] = f"{float(config.chunk_near)!r}f"
+    near = (0.125 if D < 32 else 0.25) if config.chunk_near == "auto" else float(config.chunk_near)
+    defs["CHK_NEAR"] = f"{near!r}f"
     defs["CHK_SPLIT3"] = split3
     defs["CHK_PRESPLIT"] = int(config.chunk_presplit)
     src += [f"#define {k} {v}" for k, v in defs.items()]

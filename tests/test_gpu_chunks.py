@@ -357,3 +357,89 @@ def test_log_sum_exp_with_fewer_columns_than_a_tile(N, D):
     S = x.double() @ y.double().transpose(1, 2)
     assert float((out - torch.softmax(S, 2) @ v.double()).abs().max()) < 2e-5
     assert float((lse - torch.logsumexp(S, 2)).abs().max()) < 2e-5
+
+
+@pytest.mark.parametrize("clustered", [False, True])
+@pytest.mark.parametrize("reduction", ["Sum", "LogSumExp"])
+@pytest.mark.parametrize("D", [24, 64, 256])
+@pytest.mark.parametrize("width", [3, 10, 30, 100])
+def test_narrow_but_not_local_kernels_meet_parity_on_the_default_path(width, D, reduction, clustered):
+    """Kernels that are narrow compared with the cloud without being local: g (|x^|^2 + |y^|^2) = width for the
+    centred points, where an error eps (|x^|^2 + |y^|^2) on the squared distance becomes width * eps on every
+    kernel value and the pairs that matter are too far apart (s > 1/8 of the norms) to be recomputed in float32.
+    Default flags (enable_chunks=True, use_fast_math=True): the matrix-core chunked scheme, against the CPU oracle
+    (float32, the reference's operation order) at 1e-5."""
+    from keops_amd.torch import Genred
+
+    M, N = 600, 3000
+    rng = np.random.default_rng(1000 * width + D + (7 if clustered else 0))
+    if clustered:
+        # 30 clusters of relative radius 1/2: inside a cluster s is about 1/5 of |x^|^2 + |y^|^2, above the 1/8 threshold
+        c = rng.standard_normal((30, D)) / np.sqrt(D)
+        x = (c[rng.integers(0, 30, M)] + 0.5 * rng.standard_normal((M, D)) / np.sqrt(D)).astype(np.float32)
+        y = (c[rng.integers(0, 30, N)] + 0.5 * rng.standard_normal((N, D)) / np.sqrt(D)).astype(np.float32)
+    else:
+        x = (rng.standard_normal((M, D)) / np.sqrt(D)).astype(np.float32)
+        y = (rng.standard_normal((N, D)) / np.sqrt(D)).astype(np.float32)
+    mu = y.mean(0)
+    norms = float(((x - mu) ** 2).sum(1).mean() + ((y - mu) ** 2).sum(1).mean())
+    g = np.array([width / norms], np.float32)
+    if reduction == "Sum":
+        b = rng.standard_normal((N, 2)).astype(np.float32)
+        conv = Genred("Exp(-g*SqDist(x,y))*b", [f"x=Vi({D})", f"y=Vj({D})", "b=Vj(2)", "g=Pm(1)"], reduction_op="Sum", axis=1)
+        got = conv(*to_dev(x, y, b, g)).cpu().numpy()
+        assert _scheme_used("chunk")
+        ref = cpu_reduc("gauss", [x, y, b, g], M, N, 2)
+        scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, 2)
+        if width <= 30:
+            assert_sum_parity(got, ref, scale)
+        else:
+            # exp(-g s) with g s ~ 100 amplifies any rounding of s a hundredfold: the float32 arithmetic of the
+            # reference itself (sum of D squared differences, about sqrt(D) 2^-24 s) is then 1e-5 .. 5e-5 away from
+            # the exact kernel sum, and no independent float32 evaluation can agree with it more closely than that.
+            # Measured here in float64: the chunked scheme must be as close to the exact value as the reference is.
+            x64, y64, b64 = x.astype(np.float64), y.astype(np.float64), b.astype(np.float64)
+            S = ((x64 ** 2).sum(1)[:, None] + (y64 ** 2).sum(1)[None, :] - 2 * x64 @ y64.T)
+            S = np.maximum(S, 0)
+            near = S < 1e-3 * S.mean()
+            if near.any():  # the expansion is inexact for near-coincident points: direct differences there
+                ii, jj = np.nonzero(near)
+                S[ii, jj] = ((x64[ii] - y64[jj]) ** 2).sum(1)
+            K = np.exp(-float(g[0]) * S)
+            truth, scale64 = K @ b64, K @ np.abs(b64)
+            # rows whose kernel values all lie below the float32 range (exp(-90) and less) are zero on the GPU, whose
+            # exp flushes denormal results, and denormal in the reference: they are compared in absolute terms
+            tiny = scale64 < 1e-30
+            assert np.all(np.abs(got[tiny]) <= 1e-30)
+            scale64 = np.where(tiny, np.inf, scale64)
+            err_ref = np.max(np.abs(ref - truth) / scale64)
+            err_got = np.max(np.abs(got - truth) / scale64)
+            nrm_ref, nrm_got = rel_l2(ref, truth), rel_l2(got, truth)
+            assert err_got <= max(1e-5, 2 * err_ref), f"chunked scheme {err_got:.2e} vs reference arithmetic {err_ref:.2e} from the exact sum"
+            assert nrm_got <= max(1e-5, 2 * nrm_ref), f"norm-wise: chunked scheme {nrm_got:.2e} vs reference arithmetic {nrm_ref:.2e}"
+            print(f"width {width} D {D} clustered {clustered}: element-wise {err_got:.2e} (reference {err_ref:.2e}), "
+                  f"norm-wise {nrm_got:.2e} (reference {nrm_ref:.2e}), vs oracle {np.max(np.abs(got - ref) / scale):.2e}")
+    else:
+        l = rng.standard_normal((N, 1)).astype(np.float32)
+        lse = Genred("l-SqDist(x,y)*g", [f"x=Vi({D})", f"y=Vj({D})", "l=Vj(1)", "g=Pm(1)"], reduction_op="LogSumExp", axis=1)
+        got = lse(*to_dev(x, y, l, g)).cpu().numpy()[:, 0]
+        assert _scheme_used("chunk")
+        ms = cpu_reduc("lse_gauss", [x, y, l, g], M, N, 2, reduction="Max_SumShiftExp")
+        ref = ms[:, 0].astype(np.float64) + np.log(ms[:, 1].astype(np.float64))
+        assert np.max(np.abs(got - ref) / np.maximum(1, np.abs(ref))) <= 1e-5
+
+
+def test_results_do_not_depend_on_what_the_workspace_held_before():
+    """The pre-pass (column sums, operand copies) lives in a workspace that is reused from call to call: a call must
+    give the same bits on a fresh workspace and after another call of the same module has left its data there."""
+    from keops_amd.torch import Genred
+
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    r = lambda *s: torch.randn(*s, device="cuda", generator=gen)
+    conv = Genred("Exp(-Norm2(x-y))*b", ["x=Vi(72)", "y=Vj(72)", "b=Vj(3)"], reduction_op="Sum", axis=1)
+    x, y, b = r(900, 72) / 8, r(20000, 72) / 8, r(20000, 3)
+    first = conv(x, y, b).clone()
+    conv(5 + r(2000, 72), 3 + r(60000, 72), r(60000, 3))   # other sizes, other data, same module and workspace
+    again = conv(x, y, b)
+    assert torch.equal(first, again)
+    assert _scheme_used("chunk")
