@@ -119,6 +119,26 @@ void keops_hip_module_set_timing(void* module, int enabled);
 double keops_hip_module_last_kernel_ms(void* module);
 
 /*
+ * keops_hip_launch for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose launch_kernel allocates and
+ * frees its tables inside every call (keops_nvrtc.cpp:468-481,632-640).  Same meaning of the arguments as
+ * keops_hip_launch with tagHostDevice = 1, no ranges and no batch dimensions; the launch is asynchronous on
+ * hip_stream.  Every workspace the kernels need (column-slab partial accumulators, the operand copies and
+ * partials of the matrix-core chunked and final-product schemes) is taken from a static device buffer of
+ * keops_hip_noalloc_scratch_bytes() = 128 MiB that each GPU holds from its first use until the process ends; the
+ * call performs no hipMalloc / hipFree / hipHostMalloc and creates no events.  A launch whose workspace exceeds the
+ * buffer, block-sparse or batched launches (they build device tables) and the K-nearest-neighbour schemes (they
+ * read flags back through pinned memory) are refused with an error.  All calls on one GPU share the buffer:
+ * calls that overlap on one GPU (two streams, two threads, or a captured graph replayed beside an eager call) race.
+ */
+int keops_hip_launch_noalloc(void* module, int64_t nx, int64_t ny, int tagI, int tag1D2D, int64_t dimred,
+                             const int* indsi, int ni, const int* indsj, int nj, const int* indsp, int np,
+                             int64_t dimout, const int64_t* dimsx, const int64_t* dimsy, const int64_t* dimsp,
+                             const int64_t* shapeout, int nshapeout, void* out, void* const* args,
+                             const int64_t* argshapes_flat, const int* argndims, void* hip_stream);
+size_t keops_hip_noalloc_scratch_bytes(void);
+
+/*
  * Loop-only calibration of the instruction issue rates the roofline fractions are held against: runs a grid of
  * `blocks` workgroups of 4 wavefronts, each wavefront issuing `iters` rounds of `chains` independent dependency
  * chains, and returns the elapsed time in ms and the counted instructions per wavefront.

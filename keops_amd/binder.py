@@ -49,9 +49,18 @@ def lib():
             P, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, I64, P, P, P, P, P, ctypes.c_int, P, P, P, P, P,
             ctypes.c_int,
         ]
+        L.keops_hip_launch_noalloc.argtypes = [
+            P, I64, I64, ctypes.c_int, ctypes.c_int, I64, P, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, I64, P, P, P,
+            P, ctypes.c_int, P, P, P, P, P,
+        ]
+        L.keops_hip_noalloc_scratch_bytes.restype = ctypes.c_size_t
         L.keops_hip_calibrate.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 2
         _lib = L
     return _lib
+
+
+def noalloc_scratch_bytes():
+    return int(lib().keops_hip_noalloc_scratch_bytes())
 
 
 def calibrate(kind, chains, blocks, iters, device_id=0):
@@ -148,3 +157,21 @@ class Module:
             raise KeOpsHipError(f"kernel launch failed (code {rc}): {last_error()}")
         return 0
 
+    def call_noalloc(self, nx, ny, tagI, tag1D2D, dimred, indsi, indsj, indsp, dimout, dimsx, dimsy, dimsp, shapeout,
+                     out_ptr, args_ptr, argshapes, stream=0):
+        """keops_hip_launch_noalloc: device pointers, no ranges, no batch dimensions; workspaces come from the
+        library's static scratch buffer and nothing is allocated."""
+        ci, cj, cp = _iarr(ctypes.c_int, indsi), _iarr(ctypes.c_int, indsj), _iarr(ctypes.c_int, indsp)
+        dx, dy, dp = _iarr(ctypes.c_int64, dimsx), _iarr(ctypes.c_int64, dimsy), _iarr(ctypes.c_int64, dimsp)
+        so = _iarr(ctypes.c_int64, shapeout)
+        ap = (ctypes.c_void_p * max(1, len(args_ptr)))(*args_ptr)
+        sh = _iarr(ctypes.c_int64, [int(d) for shp in argshapes for d in shp])
+        nd = _iarr(ctypes.c_int, [len(shp) for shp in argshapes])
+        rc = lib().keops_hip_launch_noalloc(
+            self.handle, int(nx), int(ny), int(tagI), int(tag1D2D), int(dimred), ci, len(indsi), cj, len(indsj), cp,
+            len(indsp), int(dimout), dx, dy, dp, so, len(shapeout), ctypes.c_void_p(out_ptr), ap, sh, nd,
+            ctypes.c_void_p(stream),
+        )
+        if rc != 0:
+            raise KeOpsHipError(f"kernel launch failed (code {rc}): {last_error()}")
+        return 0

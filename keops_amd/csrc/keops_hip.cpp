@@ -1412,6 +1412,42 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
                           ranges, shapeout, nshapeout, out, args, argshapes_flat, argndims, stream, sync);
 }
 
+int keops_hip_launch_noalloc(void* module, int64_t nx, int64_t ny, int tagI, int tag1D2D, int64_t dimred,
+                             const int* indsi, int ni, const int* indsj, int nj, const int* indsp, int np,
+                             int64_t dimout, const int64_t* dimsx, const int64_t* dimsy, const int64_t* dimsp,
+                             const int64_t* shapeout, int nshapeout, void* out, void* const* args,
+                             const int64_t* argshapes_flat, const int* argndims, void* hip_stream) {
+  Module* mp = (Module*)module;
+  if (!mp) return fail(-1, "keops_hip_launch_noalloc: null module");
+  Module& m = *mp;
+  if (m.scheme == "knn" || m.meta_int("chk_knn_inner", 0) > 0)
+    return fail(-1, "keops_hip_launch_noalloc: the K-nearest-neighbour schemes read flags back through pinned host memory; "
+                    "use keops_hip_launch");
+  if (m.timing) return fail(-1, "keops_hip_launch_noalloc: switch kernel timing off (it creates events)");
+  hipStream_t stream = (hipStream_t)hip_stream;
+  HIP_TRY(hipSetDevice(m.device));
+  void* sp = nullptr;
+  size_t sbytes = 0;
+  if (int e = keops_static_scratch(m.device, &sp, &sbytes))
+    return fail(e, std::string("address of the static scratch buffer: ") + hipGetErrorString((hipError_t)e));
+  // the module's workspace is, for this call, a view of the static scratch buffer; nothing else may be allocated
+  DeviceBuffer view;
+  view.ptr = sp;
+  view.bytes = sbytes;
+  view.borrowed = true;
+  std::swap(m.partial, view);
+  g_noalloc = true;
+  int64_t no_ranges[1] = {-1};
+  int64_t* rg[7] = {no_ranges, no_ranges, no_ranges, no_ranges, no_ranges, no_ranges, no_ranges};
+  int rc = launch_on_device(m, nx, ny, tagI, 0, tag1D2D, dimred, indsi, ni, indsj, nj, indsp, np, dimout, dimsx, dimsy, dimsp, rg,
+                            shapeout, nshapeout, out, args, argshapes_flat, argndims, stream, 0);
+  g_noalloc = false;
+  std::swap(m.partial, view);
+  return rc;
+}
+
+size_t keops_hip_noalloc_scratch_bytes(void) { return (size_t)KEOPS_STATIC_SCRATCH_BYTES; }
+
 int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave) {
   if (!ms || !instr_per_wave || blocks <= 0 || iters <= 0) return fail(-1, "keops_hip_calibrate: bad arguments");
   HIP_TRY(hipSetDevice(device_id < 0 ? 0 : device_id));

@@ -1,13 +1,44 @@
 // Device code that is compiled into libkeops_hip.so itself (everything else is JIT-compiled per formula):
+//   * the static scratch buffer of the entry point that allocates nothing (keops_hip_launch_noalloc),
 //   * a fill kernel (zero formulas: a kernel instead of hipMemsetAsync, which must stay out of captured graphs),
 //   * loop-only calibration kernels for the vector ALU and the matrix cores (keops_hip_calibrate): they measure
 //     what an instruction stream without memory traffic sustains, the ceiling the map-reduce kernels are held to.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <mutex>
 #include <type_traits>
 
 #include "keops_static.h"
+
+// ---- static scratch ---------------------------------------------------------------------------------------------
+
+static __device__ __align__(256) unsigned char scratch[KEOPS_STATIC_SCRATCH_BYTES];
+
+namespace {
+std::mutex g_scratch_mutex;
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+// Address of this device's copy of the scratch array (every GPU holds its own copy at its own address); looked up
+// once per device with that device current.  Returns a hipError_t.
+int keops_static_scratch(int device, void** ptr, size_t* bytes) {
+  if (device < 0 || device >= kMaxDevices) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return (int)e;
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[device] = p;
+  }
+  *ptr = g_scratch_ptr[device];
+  *bytes = (size_t)KEOPS_STATIC_SCRATCH_BYTES;
+  return 0;
+}
 
 // ---- fill -----------------------------------------------------------------------------------------------------------
 
