@@ -330,8 +330,10 @@ def main():
     kms = sum(kernel_ms) / len(kernel_ms)
     achieved = pairs * flop_per_pair / (kms * 1e-3) / 1e12
     peak = {"valu": PEAK_FP32_VECTOR_TFLOPS, "mfma": PEAK_BF16_MFMA_TFLOPS, "mfma32": PEAK_FP32_MFMA_TFLOPS}[bound]
-    note = {"valu": "peak is the packed-FP32 vector figure; kernels here issue scalar FP32 VALU ops only "
-                    "(packed FP32 is disabled), whose ceiling is 78.6 TFLOP/s",
+    note = {"valu": "peak is the packed-FP32 vector figure; packed FP32 instructions are disabled in this build. "
+                    "Gaussian sums take their exponents from the matrix cores when the device-side check allows it "
+                    "(kernels/keops_radial_mfma.h): the vector ALU then issues v_exp_f32 + one fma per pair and output "
+                    "component, and the algorithmic flop of the exponent are not vector-ALU work any more",
             "mfma": "peak is the dense bf16 matrix figure", "mfma32": "peak is the dense fp32 matrix figure"}[bound]
     out = {
         "metric": "pair interactions/sec (M*N/s), 1e6x1e6 D=3 Gauss sum" if args.workload == "gauss_1m_dv1"

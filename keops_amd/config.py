@@ -38,6 +38,15 @@ chunk_min_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MIN_DIM", 24))    # smallest
 chunk_near = os.environ.get("KEOPS_AMD_CHUNK_NEAR", "auto")
 chunk_max_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MAX_DIM", 1024))  # largest contraction served by the matrix-core chunked scheme
 
+# exponents of low-dimensional Gaussian kernel sums on the matrix cores (csrc/kernels/keops_radial_mfma.h)
+radial = os.environ.get("KEOPS_AMD_RADIAL", "1") != "0"
+radial_max_dim = 8                  # components of the points (7 D + 8 slots of the scalar product fit four instructions)
+radial_max_dv = 8                   # components of the weights (16 accumulators per component in every lane)
+# the path is taken when |c| log2(e) (max |x^|^2 + max |y^|^2) <= this bound for the centred points (checked on the
+# device): the exponent is then off by at most 8 * 2^-24 of it, a kernel value by 7e-5 at worst and 1e-6 typically
+radial_limit = float(os.environ.get("KEOPS_AMD_RADIAL_LIMIT", 128.0))
+radial_min_pairs_log2 = int(os.environ.get("KEOPS_AMD_RADIAL_MIN_PAIRS", 28))  # calls below 2**27 pairs: general-purpose kernel only
+
 # matrix-core final-product scheme (csrc/kernels/keops_final_mfma.h): Sum_j f(x_i,y_j) * v_j with dim(v) large
 final_chunk_min_dim = int(os.environ.get("KEOPS_AMD_FINAL_MIN_DIM", 24))   # smallest dim(v) that selects the scheme
 final_max_blocks = int(os.environ.get("KEOPS_AMD_FINAL_NB", 8))            # 32-column accumulator tiles per wavefront

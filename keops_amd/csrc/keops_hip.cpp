@@ -515,6 +515,7 @@ struct LaunchHeader {
   const int64_t* slices_x;
   const int64_t* ranges_y;
   const int64_t* offsets;
+  const unsigned* guard;
 };
 
 int launch_raw3(Module& m, const char* kernel, unsigned gx, unsigned gy, unsigned gz, unsigned block, void* params,
@@ -554,6 +555,70 @@ int ensure_pinned(Module& m, size_t bytes) {
   m.pinned_bytes = 0;
   HIP_TRY(hipHostMalloc(&m.pinned, bytes, hipHostMallocDefault));
   m.pinned_bytes = bytes;
+  return 0;
+}
+
+// ---- exponents of low-dimensional radial kernels on the matrix cores (kernels/keops_radial_mfma.h) ----
+
+size_t align_up(size_t x, size_t a);
+
+// must match struct RadParams of kernels/keops_radial_mfma.h (argument pointers follow)
+struct RadHeader {
+  int64_t nx, ny;
+  void* xa;
+  void* yb;
+  void* bw;
+  void* colsum;
+  void* colpart;
+  void* scal;
+  void* out;
+  void* partial;
+  int64_t slab_len;
+  int32_t nslabs, nparts;
+};
+
+// Launches the pre-pass, the decision kernel and the matrix-core sweep of a module built with radial=1, all
+// asynchronous; *guard receives the device address of the flag that the general-purpose kernels, launched by the
+// caller right after, test before doing anything.  Workspace: the first `reserved` bytes of m.partial stay free for
+// the caller (slab partials of the general-purpose kernel).
+int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, hipStream_t stream, size_t reserved,
+                  const unsigned** guard) {
+  const int64_t D = m.meta_int("rad_d", 0), DV = m.meta_int("rad_dv", 0), NKB = m.meta_int("rad_nkb", 0);
+  const int64_t RB = m.meta_int("rad_rb", 0), WAVES = m.meta_int("rad_waves", 0), TJ = 128;
+  if (D <= 0 || DV <= 0 || NKB <= 0 || RB <= 0 || WAVES <= 0) return fail(-1, "corrupt radial module metadata");
+  const int64_t ntiles = (ny + TJ - 1) / TJ, rows_per_wg = 32 * RB * WAVES, row_blocks = (nx + rows_per_wg - 1) / rows_per_wg;
+  // slabs over the reduced axis: about 16 workgroups per compute unit, whole tiles per slab
+  int64_t nslabs = std::max<int64_t>(1, (16 * (int64_t)m.cu_count + row_blocks - 1) / row_blocks);
+  nslabs = std::min<int64_t>(nslabs, std::max<int64_t>(1, ntiles / 8));
+  int64_t slab_len = ((ny + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ;
+  nslabs = std::max<int64_t>(1, (ny + slab_len - 1) / slab_len);
+  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(256, ny / 1024));
+  size_t off = align_up(reserved, 256);
+  auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+  const size_t o_scal = take(16), o_colsum = take((size_t)D * 4), o_colpart = take((size_t)nparts * D * 4);
+  const size_t o_xa = take((size_t)nx * NKB * 32), o_yb = take((size_t)ntiles * TJ * NKB * 32), o_bw = take((size_t)ntiles * TJ * DV * 4);
+  const size_t o_part = take((size_t)nslabs * nx * DV * 4);
+  if (int rc = m.partial.reserve(off)) return rc;
+  char* ws = (char*)m.partial.ptr;
+  std::vector<char> buf(sizeof(RadHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 16);
+  RadHeader h{};
+  h.nx = nx; h.ny = ny; h.xa = ws + o_xa; h.yb = ws + o_yb; h.bw = ws + o_bw; h.colsum = ws + o_colsum; h.colpart = ws + o_colpart;
+  h.scal = ws + o_scal; h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs; h.nparts = nparts;
+  std::memcpy(buf.data(), &h, sizeof(h));
+  for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
+  const size_t psize = sizeof(RadHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs);
+  auto with_which = [&](int w) { std::memcpy(buf.data() + psize, &w, 4); return psize + 4; };
+  if (int rc = launch_raw(m, "keops_rad_colsum", (unsigned)nparts, 1, 256, buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_colsum_final", 1, 1, 64, buf.data(), psize, stream)) return rc;
+  size_t sz = with_which(0);
+  if (int rc = launch_raw(m, "keops_rad_prep", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  sz = with_which(1);
+  if (int rc = launch_raw(m, "keops_rad_prep", (unsigned)((ntiles * TJ + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_decide", 1, 1, 64, buf.data(), psize, stream)) return rc;
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
+  if (int rc = launch_raw(m, "keops_rad_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)(64 * WAVES), buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_reduce", (unsigned)((nx * DV + 255) / 256), 1, 256, buf.data(), psize, stream)) return rc;
+  *guard = (const unsigned*)(ws + o_scal) + 2;
   return 0;
 }
 
@@ -1280,11 +1345,17 @@ static int launch_on_device(Module& m, int64_t nx, int64_t ny, int tagI, int tag
       h.slab_len = len;
     }
     h.nslabs = (int32_t)nslabs;
-    if (nslabs > 1) {
-      if (int rc = m.partial.reserve((size_t)nslabs * rows_total * m.dimred * m.sizeof_acc)) return rc;
-      h.partial = m.partial.ptr;
+    const size_t slab_bytes = nslabs > 1 ? (size_t)nslabs * rows_total * m.dimred * m.sizeof_acc : 0;
+    const bool radial = m.meta_int("radial", 0) != 0;
+    if (radial) {
+      // exponents on the matrix cores when the data allow it (decided on the device); the kernels below then return
+      // at once, and the other way round.  Both share the workspace: slab partials first.
+      if (int rc = launch_radial(m, rows_total, cols_total, out, args, stream, slab_bytes, &h.guard)) return rc;
+    } else if (slab_bytes) {
+      if (int rc = m.partial.reserve(slab_bytes)) return rc;
     }
-    if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
+    if (nslabs > 1) h.partial = m.partial.ptr;
+    if (m.timing && !radial) HIP_TRY(hipEventRecord(m.ev0, stream));
     if (int rc = launch(m, "keops_conv_dense", (unsigned)row_blocks, (unsigned)nslabs, h, args, stream)) return rc;
     if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
     if (nslabs > 1) {

@@ -48,6 +48,8 @@ struct KeopsParams {
   const i64* slices_x;  // ranges: end slice of every row range
   const i64* ranges_y;  // ranges: [*][2] column ranges
   const i64* offsets;   // batch mode: [nblocks][nvars] first-row offsets per variable
+  const unsigned* guard;  // not null: the dense kernels return at once when *guard == 1 (another kernel of the
+                          // module has produced the result: kernels/keops_radial_mfma.h)
   const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
 };
 
@@ -319,6 +321,7 @@ __device__ __forceinline__ void keops_sweep(const KeopsParams& P, const i64* col
 // ---- dense scheme ---------------------------------------------------------------------------
 
 extern "C" __global__ void __launch_bounds__(KEOPS_BLOCK) keops_conv_dense(const KeopsParams P) {
+  if (P.guard != nullptr && *P.guard == 1u) return;
   __shared__ __attribute__((aligned(16))) T ys[KEOPS_TILE_J * (KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1)];
   const i64 zero_off[8 + KEOPS_NARGS] = {};
   const i64 row0 = (i64)blockIdx.x * KEOPS_ROWS_PER_BLOCK + threadIdx.x;
@@ -360,6 +363,7 @@ extern "C" __global__ void __launch_bounds__(KEOPS_BLOCK) keops_conv_dense(const
 // Second pass of the slab scheme: merge the per-slab partial accumulators of every row in slab
 // order (ReducePair) and finalize (GpuReduc2D.py:85-125).
 extern "C" __global__ void __launch_bounds__(KEOPS_BLOCK) keops_reduce_partials(const KeopsParams P) {
+  if (P.guard != nullptr && *P.guard == 1u) return;
   const i64 i = (i64)blockIdx.x * KEOPS_BLOCK + threadIdx.x;
   if (i >= P.nx) return;
   KeopsAcc<TACC> acc;

@@ -1,0 +1,320 @@
+// Low-dimensional radial sums on the matrix cores:
+//     out_i = sum_j exp(c * |x_i - y_j|^2) * B(y_j-variables, parameters),      x, y of RAD_D <= 8 components.
+//
+// Counterpart of keopscore/keopscore/mapreduce/gpu/GpuReduc1D.py:43-96 for this family (the Gaussian kernel sum of
+// the reference's benchmarks): the general-purpose kernel of keops_conv.h spends 3*D + 3 of its 9 vector
+// instructions per pair on the exponent.  Here the exponent of a whole 32 x 32 tile of pairs,
+//     t_ij = k |x_i - y_j|^2 = k |x_i|^2 + k |y_j|^2 - 2 k <x_i, y_j>,        k = c * log2(e),
+// comes out of v_mfma_f32_32x32x16_bf16 as ONE scalar product of two "slot vectors", and the vector ALU is left
+// with v_exp_f32 and one fused multiply-add per pair and output component.
+//
+// Exact operands.  bfloat16 products are exact in float32 (8 x 8 significant bits), so a float32 number split as
+// h + m + l (three bfloat16 terms, 24 bits) multiplies exactly term by term.  Row side: u = -2 k x^ (x^ = x minus
+// the mean of y, formed in double precision, rounded once to float32) in three terms, p = k |x^|^2 from double
+// precision in four terms; column side: y^ in three terms, q = k |y^|^2 in four.  The slots of the scalar product
+// are the term products (h,h) (h,m) (m,h) (m,m) (h,l) (l,h) (m,l) of every component plus (p_n, 1) and (1, q_n):
+// 7 D + 8 slots, ordered by magnitude so that the big terms, which cancel, share one 8-slot group of the first
+// instruction (the hardware adds the products of a group exactly up to 24 bits below the largest and truncates
+// each instruction's result to float32; measured on a million pairs: |dt| <= 8 * 2^-24 |k| (|x^|^2 + |y^|^2), no
+// bias).  Dropped: (l,m), (l,l), below 2^-24 |u||y|.  The error of a kernel value is therefore at most
+// ln(2) |dt| <= 3.3e-7 |k| (|x^|^2 + |y^|^2), typically a third of it: the float32 class of the reference's own
+// exponent as long as the kernel is not much narrower than the cloud.  keops_rad_decide checks exactly that on the
+// device, |k| (max |x^|^2 + max |y^|^2) <= RAD_LIMIT, and sets a flag: when it does not hold, the kernels of this
+// file return at once and the general-purpose kernel of the same module, which is launched behind them and returns
+// at once in the other case, computes the sum from exact float32 differences.  No host synchronisation.
+//
+// Work decomposition: lane l of a wavefront owns column j = l % 32 of the staged sub-tile (its slot vector is the B
+// operand, its weights B_j sit in registers) and, after the instruction, the 16 exponents of rows
+// 8 (v / 4) + 4 (l / 32) + v % 4; it accumulates exp2(t) * B_j per row and component in registers for the whole
+// sweep.  A wavefront holds RAD_RB blocks of 32 rows (A operands in VGPRs), RAD_WAVES wavefronts share the staged
+// column tile (slot vectors pre-formatted by keops_rad_prep: straight 16-byte copies, conflict-free 16-byte reads).
+// The lanes of a row are summed with shuffles once at the end; slabs over the reduced axis (blockIdx.y) are added
+// in order by keops_rad_reduce: deterministic.
+//
+// The plug-in defines RAD_D, RAD_DV, RAD_NKB (16-slot blocks), RAD_RB, RAD_WAVES, RAD_XARG, RAD_YARG, RAD_LIMIT,
+// the slot tables rad_slot_kind / rad_slot_comp / rad_slot_term for both sides, the tables of the variables of B
+// (rad_col_arg / rad_col_dim / rad_col_off, RAD_NCOLVARS, RAD_DIMY) and of the parameters (keops_par_*), and
+// struct KeopsRadFormula { kappa(p); weights(yj, p, w) }.
+#pragma once
+
+typedef __bf16 rad_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float rad_f32x16 __attribute__((ext_vector_type(16)));
+
+#define RAD_TJ 128                 // columns per staged tile
+#define RAD_NSUB (RAD_TJ / 32)
+#define RAD_SLOTS (16 * RAD_NKB)
+#define RAD_BLOCK (64 * RAD_WAVES)
+#define RAD_ROWS_PER_BLOCK (32 * RAD_RB * RAD_WAVES)
+
+struct RadParams {
+  i64 nx, ny;
+  __bf16* xa;         // [nx][RAD_SLOTS] row-side slot vectors
+  __bf16* yb;         // [tile][RAD_NKB][2][RAD_TJ][8] column-side slot vectors, tile by tile
+  float* bw;          // [ntiles * RAD_TJ][RAD_DV] weights B_j (zero past the last column)
+  float* colsum;      // [RAD_D] column sums of y
+  float* colpart;     // [nparts][RAD_D]
+  unsigned* scal;     // [0], [1]: bit patterns of max |x^|^2, max |y^|^2; [2]: 1 when the matrix-core path is taken
+  T* out;             // [nx][RAD_DV]
+  float* partial;     // [nslabs][nx][RAD_DV]
+  i64 slab_len;       // reduced rows per slab (multiple of RAD_TJ)
+  int nslabs;
+  int nparts;
+  const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
+};
+
+__device__ __forceinline__ void rad_load_params(const RadParams& P, T (&p)[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1]) {
+#pragma unroll
+  for (int v = 0; v < KEOPS_NPARVARS; v++) {
+    const T* src = P.arg[keops_par_arg[v]];
+#pragma unroll
+    for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
+  }
+}
+
+// ---- pre-pass ---------------------------------------------------------------------------------------------------
+
+// column sums of y in two deterministic stages (fixed order, no atomics)
+extern "C" __global__ void __launch_bounds__(256) keops_rad_colsum(const RadParams P) {
+  __shared__ float part[256];
+  const T* y = P.arg[RAD_YARG];
+  const i64 rows_per_block = (P.ny + gridDim.x - 1) / gridDim.x;
+  const i64 r0 = (i64)blockIdx.x * rows_per_block, r1 = keops_min(P.ny, r0 + rows_per_block);
+#pragma unroll
+  for (int c = 0; c < RAD_D; c++) {
+    float s = 0.f;
+    for (i64 r = r0 + threadIdx.x; r < r1; r += 256) s += (float)y[r * RAD_D + c];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+      if ((int)threadIdx.x < o) part[threadIdx.x] += part[threadIdx.x + o];
+      __syncthreads();
+    }
+    if (threadIdx.x == 0) P.colpart[(i64)blockIdx.x * RAD_D + c] = part[0];
+    __syncthreads();
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(64) keops_rad_colsum_final(const RadParams P) {
+  const int c = threadIdx.x;
+  if (c < RAD_D) {
+    double s = 0.0;
+    for (int b = 0; b < P.nparts; b++) s += (double)P.colpart[(i64)b * RAD_D + c];
+    P.colsum[c] = (float)(s / (double)P.ny);  // the mean
+  }
+  if (c < 3) P.scal[c] = 0u;
+}
+
+__device__ __forceinline__ void rad_split3(float v, __bf16 (&t)[3]) {
+  t[0] = (__bf16)v;
+  const float r1 = v - (float)t[0];
+  t[1] = (__bf16)r1;
+  t[2] = (__bf16)(r1 - (float)t[1]);
+}
+__device__ __forceinline__ void rad_split4(double v, __bf16 (&t)[4]) {
+  double r = v;
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    t[k] = (__bf16)(float)r;
+    r -= (double)(float)t[k];
+  }
+}
+
+// Slot vector of one point.  which = 0: rows (x), 1: columns (y; one thread per column of the padded tile grid).
+extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams P, int which) {
+  const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+  const i64 n = which ? P.ny : P.nx;
+  const i64 ntot = which ? (P.ny + RAD_TJ - 1) / RAD_TJ * RAD_TJ : P.nx;
+  if (i >= ntot) return;
+  T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+  rad_load_params(P, p);
+  const double kappa = (double)KeopsRadFormula::kappa(p);
+  __bf16 slot[RAD_SLOTS];
+  float w[RAD_DV];
+#pragma unroll
+  for (int d = 0; d < RAD_DV; d++) w[d] = 0.f;
+  if (i < n) {
+    const T* src = P.arg[which ? RAD_YARG : RAD_XARG] + i * RAD_D;
+    __bf16 ct[RAD_D][3], nt[4];
+    double nrm = 0.0;
+#pragma unroll
+    for (int k = 0; k < RAD_D; k++) {
+      const double c = (double)src[k] - (double)P.colsum[k];
+      nrm += c * c;
+      rad_split3((float)(which ? c : -2.0 * kappa * c), ct[k]);
+    }
+    rad_split4(kappa * nrm, nt);
+    // largest centred squared norm (bit pattern of a non-negative float, rounded up): order-independent maximum
+    atomicMax(P.scal + which, __float_as_uint((float)nrm * 1.000001f));
+#pragma unroll
+    for (int s = 0; s < RAD_SLOTS; s++) {
+      const int kind = which ? rad_col_kind[s] : rad_row_kind[s];
+      const int comp = which ? rad_col_comp[s] : rad_row_comp[s];
+      const int term = which ? rad_col_term[s] : rad_row_term[s];
+      slot[s] = kind == 0 ? (__bf16)0.0f : (kind == 1 ? (__bf16)1.0f : (kind == 2 ? ct[comp][term] : nt[term]));
+    }
+    if (which) {
+      T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
+#pragma unroll
+      for (int v = 0; v < RAD_NCOLVARS; v++) {
+        const T* a = P.arg[rad_col_arg[v]] + i * rad_col_dim[v];
+#pragma unroll
+        for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
+      }
+      T wv[RAD_DV];
+      KeopsRadFormula::weights(yj, p, wv);
+#pragma unroll
+      for (int d = 0; d < RAD_DV; d++) w[d] = (float)wv[d];
+    }
+  } else {
+#pragma unroll
+    for (int s = 0; s < RAD_SLOTS; s++) slot[s] = (__bf16)0.0f;
+  }
+  if (!which) {
+#pragma unroll
+    for (int c8 = 0; c8 < RAD_SLOTS / 8; c8++) {
+      rad_bf16x8 v8;
+#pragma unroll
+      for (int e = 0; e < 8; e++) v8[e] = slot[c8 * 8 + e];
+      *reinterpret_cast<rad_bf16x8*>(P.xa + i * RAD_SLOTS + c8 * 8) = v8;
+    }
+  } else {
+    const i64 tile = i / RAD_TJ;
+    const int c = (int)(i % RAD_TJ);
+#pragma unroll
+    for (int kb = 0; kb < RAD_NKB; kb++)
+#pragma unroll
+      for (int hf = 0; hf < 2; hf++) {
+        rad_bf16x8 v8;
+#pragma unroll
+        for (int e = 0; e < 8; e++) v8[e] = slot[kb * 16 + hf * 8 + e];
+        *reinterpret_cast<rad_bf16x8*>(P.yb + (((tile * RAD_NKB + kb) * 2 + hf) * RAD_TJ + c) * 8) = v8;
+      }
+#pragma unroll
+    for (int d = 0; d < RAD_DV; d++) P.bw[i * RAD_DV + d] = w[d];
+  }
+}
+
+// the matrix-core path is taken when the kernel is not too narrow for the cloud (see the head of this file)
+extern "C" __global__ void __launch_bounds__(64) keops_rad_decide(const RadParams P) {
+  if (threadIdx.x != 0) return;
+  T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+  rad_load_params(P, p);
+  const float kappa = (float)KeopsRadFormula::kappa(p);
+  const float R = __uint_as_float(P.scal[0]) + __uint_as_float(P.scal[1]);
+  P.scal[2] = (__builtin_fabsf(kappa) * R <= (float)RAD_LIMIT) ? 1u : 0u;  // false for NaN
+}
+
+// ---- main kernel ------------------------------------------------------------------------------------------------
+
+extern "C" __global__ void __launch_bounds__(RAD_BLOCK) keops_rad_main(const RadParams P) {
+  if (P.scal[2] != 1u) return;
+  __shared__ __attribute__((aligned(16))) __bf16 ys[RAD_NKB * 2 * RAD_TJ * 8];  // [kb][half][col][8]
+  __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_DV];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+  const i64 row0 = ((i64)blockIdx.x * RAD_WAVES + wave) * (32 * RAD_RB);
+  rad_bf16x8 a[RAD_RB][RAD_NKB];
+#pragma unroll
+  for (int r = 0; r < RAD_RB; r++) {
+    i64 i = row0 + r * 32 + col;
+    if (i >= P.nx) i = P.nx - 1;  // clamped rows compute, never store
+#pragma unroll
+    for (int kb = 0; kb < RAD_NKB; kb++) a[r][kb] = *reinterpret_cast<const rad_bf16x8*>(P.xa + i * RAD_SLOTS + kb * 16 + 8 * half);
+  }
+  float acc[RAD_RB][16][RAD_DV];
+#pragma unroll
+  for (int r = 0; r < RAD_RB; r++)
+#pragma unroll
+    for (int v = 0; v < 16; v++)
+#pragma unroll
+      for (int d = 0; d < RAD_DV; d++) acc[r][v][d] = 0.f;
+
+  const i64 jbeg = (i64)blockIdx.y * P.slab_len, jend = keops_min(P.ny, jbeg + P.slab_len);
+  // software pipeline: tile t+1 travels to registers while tile t is consumed
+  constexpr int CH = RAD_NKB * 2 * RAD_TJ;  // 16-byte chunks of the slot vectors of a tile
+  constexpr int NPF = (CH + RAD_BLOCK - 1) / RAD_BLOCK;
+  constexpr int NPW = (RAD_TJ * RAD_DV + RAD_BLOCK - 1) / RAD_BLOCK;
+  uint4 pf[NPF];
+  float pfw[NPW];
+  auto prefetch = [&](i64 j0) {
+    const uint4* src = reinterpret_cast<const uint4*>(P.yb + (j0 / RAD_TJ) * (RAD_NKB * 2 * RAD_TJ * 8));
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * RAD_BLOCK;
+      pf[u] = e < CH ? src[e] : make_uint4(0u, 0u, 0u, 0u);
+    }
+    const float* wsrc = P.bw + j0 * RAD_DV;  // padded to whole tiles
+#pragma unroll
+    for (int u = 0; u < NPW; u++) {
+      const int e = tid + u * RAD_BLOCK;
+      pfw[u] = e < RAD_TJ * RAD_DV ? wsrc[e] : 0.f;
+    }
+  };
+  if (jbeg < jend) prefetch(jbeg);
+  for (i64 j0 = jbeg; j0 < jend; j0 += RAD_TJ) {
+    __syncthreads();  // the previous tile has been consumed by every wavefront
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * RAD_BLOCK;
+      if (e < CH) reinterpret_cast<uint4*>(ys)[e] = pf[u];
+    }
+#pragma unroll
+    for (int u = 0; u < NPW; u++) {
+      const int e = tid + u * RAD_BLOCK;
+      if (e < RAD_TJ * RAD_DV) bs[e] = pfw[u];
+    }
+    __syncthreads();
+    if (j0 + RAD_TJ < jend) prefetch(j0 + RAD_TJ);
+#pragma unroll
+    for (int sub = 0; sub < RAD_NSUB; sub++) {
+      const int c = sub * 32 + col;
+      rad_bf16x8 b[RAD_NKB];
+#pragma unroll
+      for (int kb = 0; kb < RAD_NKB; kb++) b[kb] = *reinterpret_cast<const rad_bf16x8*>(ys + ((kb * 2 + half) * RAD_TJ + c) * 8);
+      float w[RAD_DV];
+#pragma unroll
+      for (int d = 0; d < RAD_DV; d++) w[d] = bs[c * RAD_DV + d];
+      rad_f32x16 t[RAD_RB];
+#pragma unroll
+      for (int r = 0; r < RAD_RB; r++) {
+        rad_f32x16 z;
+#pragma unroll
+        for (int v = 0; v < 16; v++) z[v] = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < RAD_NKB; kb++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r][kb], b[kb], z, 0, 0, 0);
+        t[r] = z;
+      }
+#pragma unroll
+      for (int r = 0; r < RAD_RB; r++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const float e = __builtin_amdgcn_exp2f(t[r][v]);
+#pragma unroll
+          for (int d = 0; d < RAD_DV; d++) acc[r][v][d] = __builtin_fmaf(e, w[d], acc[r][v][d]);
+        }
+    }
+  }
+  // the 32 lanes of a half hold the same rows for different columns: shuffle sums, then one lane stores
+#pragma unroll
+  for (int r = 0; r < RAD_RB; r++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const i64 i = row0 + r * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+#pragma unroll
+      for (int d = 0; d < RAD_DV; d++) {
+        float s = acc[r][v][d];
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o);
+        if (col == 0 && i < P.nx) P.partial[((i64)blockIdx.y * P.nx + i) * RAD_DV + d] = s;
+      }
+    }
+}
+
+// slabs are added in order
+extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadParams P) {
+  if (P.scal[2] != 1u) return;
+  const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (e >= P.nx * RAD_DV) return;
+  float s = P.partial[e];
+  for (int k = 1; k < P.nslabs; k++) s += P.partial[(i64)k * P.nx * RAD_DV + e];
+  P.out[e] = (T)s;
+}

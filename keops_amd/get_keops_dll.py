@@ -685,6 +685,168 @@ def generate_final_plugin(red, match, sum_scheme, nargs, irregular=False):
     return "\n".join(src) + "\n", meta
 
 
+def _linear_coef(E, svar):
+    """Uniform (parameter-only) formula C with E = C * svar, or None when E is not of that form."""
+    from .formulas import ops as O
+
+    def uniform(f):
+        return all(v.cat == 2 for v in f.variables)
+
+    if E == svar:
+        return O.IntCst(1)
+    if E.name == "Minus":
+        c = _linear_coef(E.children[0], svar)
+        return None if c is None else O.Minus(c)
+    if E.name == "Mult" and len(E.children) == 2:
+        for a, b in (E.children, E.children[::-1]):
+            if uniform(a) and a.dim == 1:
+                c = _linear_coef(b, svar)
+                if c is not None:
+                    return O.Mult(a, c)
+    if E.name == "Divide" and len(E.children) == 2:
+        a, b = E.children
+        if uniform(b) and b.dim == 1:
+            c = _linear_coef(a, svar)
+            if c is not None:
+                return O.Divide(c, b)
+    return None
+
+
+def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id, pairs=0):
+    """dict(x, y, coef, W) when ``red`` is Sum_Reduction(Exp(C * SqDist(x, y)) * W) in float32 on the dense scheme,
+    with x an output-indexed and y a reduced-index variable of at most config.radial_max_dim (8) components, C a
+    scalar formula of the parameters and W (optional) a formula of reduced-index variables and parameters of at most
+    config.radial_max_dv (8) components: the Gaussian kernel sums.  Such sums take their exponents from the matrix
+    cores (kernels/keops_radial_mfma.h) when the data allow it.  ``pairs``: when not 0, the call holds less than
+    2**pairs pairs; small calls stay on the general-purpose kernel alone, whose fixed cost is lower."""
+    from .formulas import ops as O
+    from .formulas.reductions import KIND_SUM
+
+    if (not config.radial or red.kind != KIND_SUM or dtype != "float" or dtypeacc != "float" or not use_fast_math
+            or "_ranges" in map_reduce_id or sum_scheme == "kahan_scheme"):
+        return None
+    if pairs and int(pairs) < config.radial_min_pairs_log2:
+        return None
+    F = red.formula
+    if F.name == "Exp":
+        expnode, W = F, None
+    elif F.name == "Mult" and len(F.children) == 2:
+        # the factor that is the exponential of a formula of both indices
+        pick = [k for k, c in enumerate(F.children) if c.name == "Exp" and c.depends_on_cat(0) and c.depends_on_cat(1)]
+        if len(pick) != 1:
+            return None
+        expnode, W = F.children[pick[0]], F.children[1 - pick[0]]
+    else:
+        return None
+    if expnode.dim != 1:
+        return None
+    E = expnode.children[0]
+    found = []
+    for node in E.walk():
+        if node.name == "Sum" and node.children[0].name == "Square" and node.children[0].children[0].name == "Subtract":
+            a, b = node.children[0].children[0].children
+            if (isinstance(a, O.Var) and isinstance(b, O.Var) and a.dim == b.dim and 1 <= a.dim <= config.radial_max_dim
+                    and {a.cat, b.cat} == {0, 1} and node not in [f[0] for f in found]):
+                found.append((node, a, b))
+    if len(found) != 1:
+        return None
+    node, a, b = found[0]
+    svar = O.Var(1 << 30, 1, 3)
+    coef = _linear_coef(E.replace(node, svar), svar)
+    if coef is None:
+        return None
+    x, y = (a, b) if a.cat == red.tagI else (b, a)
+    if W is not None:
+        if W.dim != F.dim or not 1 <= W.dim <= config.radial_max_dv:
+            return None
+        if any(v.cat not in (1 - red.tagI, 2) for v in W.variables):
+            return None
+    return dict(x=x, y=y, coef=coef, W=W)
+
+
+def generate_radial_section(red, match, nargs):
+    """Source text appended to a general-purpose module: tables, the two straight-line bodies of struct
+    KeopsRadFormula and the template kernels/keops_radial_mfma.h; returns (text, meta entries)."""
+    from .formulas import ops as O
+    from .formulas.lir import LOG2E
+
+    x, y, coef, W = match["x"], match["y"], match["coef"], match["W"]
+    D = x.dim
+    Dv = 1 if W is None else W.dim
+    # slots of the scalar product, by decreasing magnitude: (row term, column term) of every component, the terms
+    # of the two squared norms against 1.  kind 0: zero, 1: one, 2: component term (comp, term), 3: norm term
+    H, Mi, Lo = 0, 1, 2
+    rows, cols = [], []
+
+    def prod(tr, tc):
+        for k in range(D):
+            rows.append((2, k, tr))
+            cols.append((2, k, tc))
+
+    def norm(n):
+        rows.append((3, 0, n)); cols.append((1, 0, 0))
+        rows.append((1, 0, 0)); cols.append((3, 0, n))
+
+    def pad(mult):
+        while len(rows) % mult:
+            rows.append((0, 0, 0)); cols.append((0, 0, 0))
+
+    prod(H, H); norm(0)
+    if D + 2 <= 8:
+        pad(8)  # the big terms, which cancel, share one 8-slot group: the hardware adds a group exactly
+    prod(H, Mi); prod(Mi, H); norm(1)
+    prod(Mi, Mi); prod(H, Lo); prod(Lo, H); norm(2)
+    prod(Mi, Lo); norm(3)
+    pad(16)
+    nkb = len(rows) // 16
+    if nkb > 4:
+        return None, None
+    # output rows per wavefront (32-row blocks) and wavefronts per workgroup: the accumulators (16 per block and
+    # output component) live in registers
+    rb = 2 if Dv <= 2 else 1
+    waves = 8
+
+    class _W:
+        formula, tagI = (W if W is not None else O.IntCst(1)), red.tagI
+
+    layout = VarLayout(_W)
+    if layout.rowvars:
+        return None, None
+    # the parameter table serves both bodies: the one of the whole reduction (as the general-purpose kernel's)
+    full = VarLayout(red)
+    pnames = {key: name for key, name in full.names.items() if key[0] == 2}
+    w_names = dict(layout.names)
+    w_names.update(pnames)
+    L = Lir(row_cat=red.tagI, fast_math=True, dtype="float")
+    w_lines, w_exprs = L.emit(lower(_W.formula, L), w_names, indent="    ")
+    w_prelude = list(L.prelude)
+    Lk = Lir(row_cat=red.tagI, fast_math=True, dtype="float")
+    k_lines, k_exprs = Lk.emit(lower(coef, Lk), pnames, indent="    ")
+    ca, cd, co = VarLayout.table(layout.colvars)
+    meta = dict(radial=1, rad_d=D, rad_dv=Dv, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind, rad_yarg=y.ind)
+    src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
+    defs = dict(RAD_D=D, RAD_DV=Dv, RAD_NKB=nkb, RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind,
+                RAD_LIMIT=f"{float(config.radial_limit)!r}f", RAD_NCOLVARS=len(layout.colvars), RAD_DIMY=layout.dimy)
+    src += [f"#define {k} {v}" for k, v in defs.items()]
+    for name, vals in (("row_kind", [r[0] for r in rows]), ("row_comp", [r[1] for r in rows]), ("row_term", [r[2] for r in rows]),
+                       ("col_kind", [c[0] for c in cols]), ("col_comp", [c[1] for c in cols]), ("col_term", [c[2] for c in cols]),
+                       ("col_arg", ca), ("col_dim", cd), ("col_off", co)):
+        src.append(f"static __device__ constexpr int rad_{name}[] = {_c_list(vals)};")
+    dy, dp = max(1, layout.dimy), max(1, full.dimp)
+    src += w_prelude + list(Lk.prelude)
+    src.append("struct KeopsRadFormula {")
+    src.append(f"  // log2(e) times the coefficient of the squared distance in the exponent")
+    src.append(f"  static __device__ __forceinline__ T kappa(const T (&p)[{dp}]) {{")
+    src += k_lines
+    src.append(f"    return ({k_exprs[0]}) * {LOG2E!r}f;")
+    src.append("  }")
+    src.append(f"  static __device__ __forceinline__ void weights(const T (&yj)[{dy}], const T (&p)[{dp}], T (&w)[{Dv}]) {{")
+    src += w_lines + [f"    w[{k}] = {e};" for k, e in enumerate(w_exprs)]
+    src.append("  }\n};")
+    src.append('#include "keops_radial_mfma.h"')
+    return "\n".join(src) + "\n", meta
+
+
 def get_keops_dll(
     map_reduce_id, red_formula_string, enable_chunks, enable_finalchunks, mul_var_highdim, aliases, nargs, dtype,
     dtypeacc, sum_scheme_string, tagHostDevice, tagCPUGPU, tag1D2D, use_half, use_fast_math, device_id, nx=None,
@@ -761,6 +923,13 @@ def get_keops_dll(
         if source is None:
             source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint,
                                            irregular=irregular)
+            rad = match_radial(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, map_reduce_id, pairs) if mc else None
+            if rad is not None:
+                section, rmeta = generate_radial_section(red, rad, nargs)
+                if section is not None:
+                    meta.update(rmeta)
+                    head, body = source.split("\n", 1)
+                    source = "//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()) + "\n" + body + section
         tag = hashlib.sha256((source + binder.templates_digest() + str(use_fast_math)).encode()).hexdigest()[:16]
         folder = config.get_build_folder()
         target = os.path.join(folder, f"hsaco_{tag}")

@@ -182,6 +182,7 @@ class LoadKeOps_hip:
 
 
 _loaders = {}
+last_loader = None  # the object the most recent call resolved to (diagnostics, tests)
 
 
 def load_keops_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula, aliases, nargs, dtype,
@@ -203,10 +204,12 @@ def load_keops_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_requ
         pairs = 0
     key = (tagCPUGPU, tag1D2D, tagHostDevice, bool(use_ranges), device_id_request, formula, tuple(aliases), nargs,
            dtype, lang, tuple(sorted(optional_flags.items())), _rows_bucket(rows_hint), batch_loop, pairs)
+    global last_loader
     obj = _loaders.get(key)
     if obj is None:
         obj = _loaders[key] = LoadKeOps_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula,
                                             aliases, nargs, dtype, lang, optional_flags, nx=nx, batch_loop=batch_loop, pairs=pairs)
+    last_loader = obj
     return obj
 
 

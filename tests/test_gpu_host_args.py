@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 NO_RANGES = np.array([-1], np.int64)
 
 
-def _module(formula, aliases, red="Sum", axis=1, ranges=False, nx=None):
+def _module(formula, aliases, red="Sum", axis=1, ranges=False, nx=None, ny=None):
     from keops_amd.keops_io import load_keops_hip
     from keops_amd.common.operations import preprocess
     from keops_amd.common.parse_type import axis2cat, get_optional_flags
@@ -23,7 +23,7 @@ def _module(formula, aliases, red="Sum", axis=1, ranges=False, nx=None):
     red_int, f2 = preprocess(red, None)
     flags = get_optional_flags(red_int, "auto", False, "auto", True, True)
     full = f"{red_int}_Reduction({formula},{axis2cat(axis)}{',' + f2 if f2 else ''})"
-    return load_keops_hip(1, 0, 0, ranges, 0, full, aliases, len(aliases), "float32", "torch", flags, nx=nx)
+    return load_keops_hip(1, 0, 0, ranges, 0, full, aliases, len(aliases), "float32", "torch", flags, nx=nx, ny=ny)
 
 
 def test_abi_takes_numpy_pointers_directly():
@@ -31,7 +31,7 @@ def test_abi_takes_numpy_pointers_directly():
     rng = np.random.default_rng(0)
     x, y = rng.standard_normal((M, 3)).astype(np.float32), rng.standard_normal((N, 3)).astype(np.float32)
     b, g = rng.standard_normal((N, 2)).astype(np.float32), np.array([0.7], np.float32)
-    ld = _module("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)", "g=Pm(1)"], nx=M)
+    ld = _module("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)", "g=Pm(1)"], nx=M, ny=N)
     p = ld.params
     out = np.full((M, 2), np.nan, np.float32)
     args = [x, y, b, g]

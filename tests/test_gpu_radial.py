@@ -1,0 +1,145 @@
+"""Gaussian kernel sums whose exponents come from the matrix cores (kernels/keops_radial_mfma.h): parity with the CPU
+oracle where the device takes that path, and bit-identity with the general-purpose kernel where the device decides
+against it (kernels much narrower than the cloud, clouds far from their mean)."""
+import numpy as np
+import pytest
+import torch
+
+from common import assert_sum_parity, to_dev
+from oracle.cpu_oracle import cpu_reduc
+
+pytestmark = pytest.mark.gpu
+
+GAUSS = "Exp(-g*SqDist(x,y))*b"
+
+
+def _genred(D, Dv, axis=1, **kw):
+    from keops_amd.torch import Genred
+
+    bcat = "Vj" if axis == 1 else "Vi"
+    return Genred(GAUSS, [f"x=Vi({D})", f"y=Vj({D})", f"b={bcat}({Dv})", "g=Pm(1)"], reduction_op="Sum", axis=axis, **kw)
+
+
+def _plain(D, Dv, axis=1):
+    """The same reduction with the matrix-core schemes switched off: the general-purpose kernel alone."""
+    return _genred(D, Dv, axis, enable_chunks=False)
+
+
+def _last_meta(key):
+    from keops_amd import keops_io
+
+    return keops_io.last_loader.module.meta(key)
+
+
+@pytest.mark.parametrize("D,Dv,M,N", [(3, 1, 30011, 30500), (3, 8, 20000, 21000), (3, 2, 300000, 777), (5, 3, 17000, 23001),
+                                      (8, 1, 16000, 18000), (2, 4, 33333, 10001)])
+def test_gaussian_sums_with_matrix_core_exponents_vs_oracle(D, Dv, M, N):
+    rng = np.random.default_rng(100 * D + Dv)
+    x = rng.standard_normal((M, D)).astype(np.float32)
+    y = (rng.standard_normal((N, D)) + 0.3).astype(np.float32)   # not centred on the origin: the kernels centre on mean(y)
+    b = rng.standard_normal((N, Dv)).astype(np.float32)
+    g = np.array([0.7], np.float32)
+    dev = to_dev(x, y, b, g)
+    got = _genred(D, Dv)(*dev)
+    assert _last_meta("radial") == "1"
+    rows = np.sort(rng.choice(M, 1500, replace=False)).astype(np.int64)
+    ref = cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
+    scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, Dv, rows=rows)
+    assert_sum_parity(got[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
+    # the matrix-core path really ran: the general-purpose kernel gives (slightly) different bits
+    plain = _plain(D, Dv)(*dev)
+    assert _last_meta("radial") is None
+    assert not torch.equal(plain, got)
+    assert_sum_parity(plain[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
+    # exact linearity in the weights, deterministic from call to call
+    assert torch.equal(_genred(D, Dv)(dev[0], dev[1], 2 * dev[2], dev[3]), 2 * got)
+    assert torch.equal(_genred(D, Dv)(*dev), got)
+
+
+def test_reduction_over_i_and_formula_spellings():
+    from keops_amd.torch import Genred
+
+    M, N, D = 21000, 19000, 3
+    rng = np.random.default_rng(9)
+    x, y = rng.standard_normal((M, D)).astype(np.float32), rng.standard_normal((N, D)).astype(np.float32)
+    a = rng.standard_normal((M, 2)).astype(np.float32)
+    s = np.array([1.3], np.float32)
+    conv = Genred("Exp(-SqDist(x,y)/(2*s*s))*a", [f"x=Vi({D})", f"y=Vj({D})", "a=Vi(2)", "s=Pm(1)"], reduction_op="Sum", axis=0)
+    got = conv(*to_dev(x, y, a, s)).cpu().numpy()
+    assert _last_meta("radial") == "1" and got.shape == (N, 2)
+    g = np.array([1 / (2 * 1.3 ** 2)], np.float32)
+    rows = np.arange(0, N, 13, dtype=np.int64)
+    ref = cpu_reduc("gauss", [y, x, a, g], N, M, 2, rows=rows)   # roles of i and j exchanged
+    scale = cpu_reduc("gauss", [y, x, np.abs(a), g], N, M, 2, rows=rows)
+    assert_sum_parity(got[rows], ref, scale)
+    # no weights at all: sum_j exp(-|x - y|^2)
+    ones = Genred("Exp(-SqDist(x,y))", [f"x=Vi({D})", f"y=Vj({D})"], reduction_op="Sum", axis=1)(*to_dev(x, y)).cpu().numpy()
+    assert _last_meta("radial") == "1"
+    ref1 = cpu_reduc("gauss", [x, y, np.ones((N, 1), np.float32), np.ones(1, np.float32)], M, N, 1, rows=rows[:800])
+    assert_sum_parity(ones[rows[:800]], ref1, ref1)
+
+
+@pytest.mark.parametrize("case", ["narrow", "far", "outlier"])
+def test_device_side_decision_falls_back_to_exact_differences(case):
+    """Where |c| log2(e) (max |x^|^2 + max |y^|^2) exceeds the bound, the expansion of |x - y|^2 would lose the digits
+    that matter: the device skips the matrix-core kernels and the general-purpose kernel of the same module runs.
+    Same code, same slabs: bit-identical to the module built without the matrix-core kernels."""
+    M, N, D = 20000, 20000, 3
+    rng = np.random.default_rng(3)
+    x, y = rng.random((M, D)).astype(np.float32), rng.random((N, D)).astype(np.float32)
+    g = np.array([1.0], np.float32)
+    if case == "narrow":
+        g = np.array([1 / 0.05 ** 2], np.float32)              # kernel width 0.05 in the unit cube
+    elif case == "far":
+        x, y, g = x * 100, y * 100, np.array([0.5], np.float32)  # width 1 in a cube of side 100
+    else:
+        x[5] += 40.0                                             # one far outlier
+    b = rng.standard_normal((N, 1)).astype(np.float32)
+    dev = to_dev(x, y, b, g)
+    got = _genred(D, 1)(*dev)
+    assert _last_meta("radial") == "1"
+    plain = _plain(D, 1)(*dev)
+    assert torch.equal(got, plain)
+    rows = np.arange(0, M, 17, dtype=np.int64)
+    ref = cpu_reduc("gauss", [x, y, b, g], M, N, 1, rows=rows)
+    scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, 1, rows=rows)
+    assert_sum_parity(got[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale + 1e-30)
+
+
+def test_small_calls_other_sum_schemes_and_dtypes_stay_on_the_general_purpose_kernel():
+    rng = np.random.default_rng(4)
+    x, y = rng.standard_normal((2000, 3)).astype(np.float32), rng.standard_normal((3000, 3)).astype(np.float32)
+    b, g = rng.standard_normal((3000, 1)).astype(np.float32), np.array([1.0], np.float32)
+    _genred(3, 1)(*to_dev(x, y, b, g))
+    assert _last_meta("radial") is None                                   # 6e6 pairs: not worth the pre-pass
+    big = [np.repeat(a, 12, 0) for a in (x, y, b)]
+    _genred(3, 1, sum_scheme="kahan_scheme")(*to_dev(*big, g))
+    assert _last_meta("radial") is None
+    _genred(3, 1, use_fast_math=False)(*to_dev(*big, g))
+    assert _last_meta("radial") is None
+    _genred(3, 1)(*[t.double() for t in to_dev(*big, g)])
+    assert _last_meta("radial") is None
+
+
+def test_matrix_core_exponents_under_graph_capture():
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    r = lambda *s: torch.randn(*s, device="cuda", generator=gen)
+    x, y, b, g = r(20000, 3), r(21000, 3), r(21000, 2), torch.tensor([0.5], device="cuda")
+    conv = _genred(3, 2)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        conv(x, y, b, g)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = conv(x, y, b, g)
+    for scale in (1.0, 0.5, 30.0):   # the last one flips the device-side decision inside the same graph
+        x.copy_(r(20000, 3) * scale)
+        y.copy_(r(21000, 3) * scale)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        assert torch.equal(got, conv(x, y, b, g))
