@@ -617,7 +617,7 @@ int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* arg
   if (int rc = launch_raw(m, "keops_rad_decide", 1, 1, 64, buf.data(), psize, stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
   if (int rc = launch_raw(m, "keops_rad_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)(64 * WAVES), buf.data(), psize, stream)) return rc;
-  if (int rc = launch_raw(m, "keops_rad_reduce", (unsigned)((nx * DV + 255) / 256), 1, 256, buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_reduce", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), psize, stream)) return rc;
   *guard = (const unsigned*)(ws + o_scal) + 2;
   return 0;
 }

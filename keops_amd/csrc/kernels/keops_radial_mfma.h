@@ -1,5 +1,10 @@
 // Low-dimensional radial sums on the matrix cores:
-//     out_i = sum_j exp(c * |x_i - y_j|^2) * B(y_j-variables, parameters),      x, y of RAD_D <= 8 components.
+//     out_i = A(i-variables) sum_j exp(c * |x_i - y_j|^2) * W(j-variables),          x, y of RAD_D <= 8 components,
+// and, with the difference factor of the gradients with respect to the points (RAD_DIFF = +-1),
+//     out_i = +- A_i sum_j exp(c * |x_i - y_j|^2) w_j (x_i - y_j)  =  +- A_i (x^_i S_i - sum_j K_ij w_j y^_j),
+// where the kernel accumulates the RAD_D + 1 sums of K_ij w_j [y^_j, 1] and x^, y^ are the points minus the mean of y
+// (the two terms that are subtracted are then as small as the cloud allows; what remains is a cancellation of
+// order 2^-24 |x^_i| / |x_i - y_j|, small wherever the device-side check below lets this path run).
 //
 // Counterpart of keopscore/keopscore/mapreduce/gpu/GpuReduc1D.py:43-96 for this family (the Gaussian kernel sum of
 // the reference's benchmarks): the general-purpose kernel of keops_conv.h spends 3*D + 3 of its 9 vector
@@ -34,7 +39,8 @@
 // The plug-in defines RAD_D, RAD_DV, RAD_NKB (16-slot blocks), RAD_RB, RAD_WAVES, RAD_XARG, RAD_YARG, RAD_LIMIT,
 // the slot tables rad_slot_kind / rad_slot_comp / rad_slot_term for both sides, the tables of the variables of B
 // (rad_col_arg / rad_col_dim / rad_col_off, RAD_NCOLVARS, RAD_DIMY) and of the parameters (keops_par_*), and
-// struct KeopsRadFormula { kappa(p); weights(yj, p, w) }.
+// the tables of the variables of A (rad_row_*, RAD_NROWVARS, RAD_DIMX), RAD_DW (components of W), RAD_DOUT, RAD_DIFF,
+// RAD_SIGN and struct KeopsRadFormula { kappa(p); weights(yj, p, w); rowscale(xi, p) }.
 #pragma once
 
 typedef __bf16 rad_bf16x8 __attribute__((ext_vector_type(8)));
@@ -135,10 +141,12 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
   if (i < n) {
     const T* src = P.arg[which ? RAD_YARG : RAD_XARG] + i * RAD_D;
     __bf16 ct[RAD_D][3], nt[4];
+    float cf[RAD_D];
     double nrm = 0.0;
 #pragma unroll
     for (int k = 0; k < RAD_D; k++) {
       const double c = (double)src[k] - (double)P.colsum[k];
+      cf[k] = (float)c;
       nrm += c * c;
       rad_split3((float)(which ? c : -2.0 * kappa * c), ct[k]);
     }
@@ -160,10 +168,16 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
 #pragma unroll
         for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
       }
-      T wv[RAD_DV];
+      T wv[RAD_DW];
       KeopsRadFormula::weights(yj, p, wv);
+#if RAD_DIFF != 0
+#pragma unroll
+      for (int k = 0; k < RAD_D; k++) w[k] = (float)wv[0] * cf[k];
+      w[RAD_D] = (float)wv[0];
+#else
 #pragma unroll
       for (int d = 0; d < RAD_DV; d++) w[d] = (float)wv[d];
+#endif
     }
   } else {
 #pragma unroll
@@ -309,12 +323,37 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK) keops_rad_main(const Rad
     }
 }
 
-// slabs are added in order
+// slabs are added in order; the factors of the output index and, for the gradients with respect to the points, the
+// difference x^_i S - sum_j K_ij w_j y^_j are applied here, once per output row
 extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadParams P) {
   if (P.scal[2] != 1u) return;
-  const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
-  if (e >= P.nx * RAD_DV) return;
-  float s = P.partial[e];
-  for (int k = 1; k < P.nslabs; k++) s += P.partial[(i64)k * P.nx * RAD_DV + e];
-  P.out[e] = (T)s;
+  const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (i >= P.nx) return;
+  float s[RAD_DV];
+#pragma unroll
+  for (int d = 0; d < RAD_DV; d++) s[d] = P.partial[i * RAD_DV + d];
+  for (int k = 1; k < P.nslabs; k++)
+#pragma unroll
+    for (int d = 0; d < RAD_DV; d++) s[d] += P.partial[((i64)k * P.nx + i) * RAD_DV + d];
+  T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+  rad_load_params(P, p);
+  T xi[RAD_DIMX > 0 ? RAD_DIMX : 1];
+#pragma unroll
+  for (int v = 0; v < RAD_NROWVARS; v++) {
+    const T* a = P.arg[rad_row_arg[v]] + i * rad_row_dim[v];
+#pragma unroll
+    for (int d = 0; d < rad_row_dim[v]; d++) xi[rad_row_off[v] + d] = a[d];
+  }
+  const float ai = (float)KeopsRadFormula::rowscale(xi, p) * RAD_SIGN;
+#if RAD_DIFF != 0
+  const T* x = P.arg[RAD_XARG] + i * RAD_D;
+#pragma unroll
+  for (int k = 0; k < RAD_D; k++) {
+    const float xc = (float)((double)x[k] - (double)P.colsum[k]);
+    P.out[i * RAD_DOUT + k] = (T)(ai * (float)RAD_DIFF * __builtin_fmaf(xc, s[RAD_D], -s[k]));
+  }
+#else
+#pragma unroll
+  for (int d = 0; d < RAD_DOUT; d++) P.out[i * RAD_DOUT + d] = (T)(ai * s[d]);
+#endif
 }

@@ -713,12 +713,18 @@ def _linear_coef(E, svar):
 
 
 def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id, pairs=0):
-    """dict(x, y, coef, W) when ``red`` is Sum_Reduction(Exp(C * SqDist(x, y)) * W) in float32 on the dense scheme,
-    with x an output-indexed and y a reduced-index variable of at most config.radial_max_dim (8) components, C a
-    scalar formula of the parameters and W (optional) a formula of reduced-index variables and parameters of at most
-    config.radial_max_dv (8) components: the Gaussian kernel sums.  Such sums take their exponents from the matrix
-    cores (kernels/keops_radial_mfma.h) when the data allow it.  ``pairs``: when not 0, the call holds less than
-    2**pairs pairs; small calls stay on the general-purpose kernel alone, whose fixed cost is lower."""
+    """dict(x, y, coef, A, W, diff) when the formula of a float32 Sum reduction on the dense scheme is a product
+
+        [+-]  A(i-variables)  *  Exp(C * SqDist(x, y))  *  W(j-variables)  [ * (x - y) | (y - x) ]
+
+    with x an output-indexed and y a reduced-index variable of at most config.radial_max_dim (8) components, C a scalar
+    formula of the parameters, A scalar, W of at most config.radial_max_dv (8) components (scalar when the difference
+    factor is present): the Gaussian kernel sums and their gradients with respect to the points and the weights.  Here
+    "i" means indexed like the output.  Such sums take their exponents from the matrix cores
+    (kernels/keops_radial_mfma.h) when the data allow it; with the difference factor, the kernel accumulates
+    sum_j K_ij w_j [y^_j, 1] and the last pass forms A_i (x^_i S - sum_j K_ij w_j y^_j) for the points centred on the
+    mean of y.  ``pairs``: when not 0, the call holds less than 2**pairs pairs; small calls stay on the
+    general-purpose kernel alone, whose fixed cost is lower."""
     from .formulas import ops as O
     from .formulas.reductions import KIND_SUM
 
@@ -727,20 +733,22 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
         return None
     if pairs and int(pairs) < config.radial_min_pairs_log2:
         return None
-    F = red.formula
-    if F.name == "Exp":
-        expnode, W = F, None
-    elif F.name == "Mult" and len(F.children) == 2:
-        # the factor that is the exponential of a formula of both indices
-        pick = [k for k, c in enumerate(F.children) if c.name == "Exp" and c.depends_on_cat(0) and c.depends_on_cat(1)]
-        if len(pick) != 1:
-            return None
-        expnode, W = F.children[pick[0]], F.children[1 - pick[0]]
-    else:
+    row_cat, col_cat = red.tagI, 1 - red.tagI
+    # the factors of the product, signs and scalar constants pulled out
+    sign, factors, stack = 1, [], [red.formula]
+    while stack:
+        f = stack.pop()
+        if f.name == "Minus":
+            sign = -sign
+            stack.append(f.children[0])
+        elif f.name == "Mult" and len(f.children) == 2:
+            stack.extend(f.children[::-1])
+        else:
+            factors.append(f)
+    exps = [f for f in factors if f.name == "Exp" and f.depends_on_cat(0) and f.depends_on_cat(1)]
+    if len(exps) != 1 or exps[0].dim != 1:
         return None
-    if expnode.dim != 1:
-        return None
-    E = expnode.children[0]
+    E = exps[0].children[0]
     found = []
     for node in E.walk():
         if node.name == "Sum" and node.children[0].name == "Square" and node.children[0].children[0].name == "Subtract":
@@ -755,24 +763,53 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
     coef = _linear_coef(E.replace(node, svar), svar)
     if coef is None:
         return None
-    x, y = (a, b) if a.cat == red.tagI else (b, a)
-    if W is not None:
-        if W.dim != F.dim or not 1 <= W.dim <= config.radial_max_dv:
+    x, y = (a, b) if a.cat == row_cat else (b, a)
+    A, Wf, diff = [], [], 0
+    for f in factors:
+        if f is exps[0]:
+            continue
+        if f.name == "Subtract" and set(f.children) == {x, y} and f.dim == x.dim and x.dim > 1:
+            if diff:
+                return None
+            diff = 1 if f.children[0] == x else -1
+        elif not f.depends_on_cat(col_cat) and f.depends_on_cat(row_cat):
+            if f.dim != 1:
+                return None
+            A.append(f)
+        elif not f.depends_on_cat(row_cat):
+            Wf.append(f)
+        else:
+            return None  # a factor of both indices other than the exponential
+    vec = [f for f in Wf if f.dim != 1]
+    if len(vec) > 1 or (diff and vec):
+        return None
+    dimw = vec[0].dim if vec else 1
+    if diff:
+        if x.dim + 1 > config.radial_max_dv or red.formula.dim != x.dim:
             return None
-        if any(v.cat not in (1 - red.tagI, 2) for v in W.variables):
-            return None
-    return dict(x=x, y=y, coef=coef, W=W)
+    elif dimw != red.formula.dim or not 1 <= dimw <= config.radial_max_dv:
+        return None
+
+    def product(fs):
+        out = None
+        for f in sorted(fs, key=lambda f: f.dim):  # scalars first: one multiplication per component at the end
+            out = f if out is None else O.Mult(out, f)
+        return out
+
+    return dict(x=x, y=y, coef=coef, A=product(A), W=product(Wf), diff=diff, sign=sign)
 
 
 def generate_radial_section(red, match, nargs):
-    """Source text appended to a general-purpose module: tables, the two straight-line bodies of struct
+    """Source text appended to a general-purpose module: tables, the straight-line bodies of struct
     KeopsRadFormula and the template kernels/keops_radial_mfma.h; returns (text, meta entries)."""
     from .formulas import ops as O
     from .formulas.lir import LOG2E
 
-    x, y, coef, W = match["x"], match["y"], match["coef"], match["W"]
+    x, y, coef, A, W, diff, sign = (match[k] for k in ("x", "y", "coef", "A", "W", "diff", "sign"))
     D = x.dim
-    Dv = 1 if W is None else W.dim
+    dimw = 1 if W is None else W.dim
+    Dv = D + 1 if diff else dimw       # components accumulated per pair
+    dout = D if diff else dimw         # components of the output
     # slots of the scalar product, by decreasing magnitude: (row term, column term) of every component, the terms
     # of the two squared norms against 1.  kind 0: zero, 1: one, 2: component term (comp, term), 3: norm term
     H, Mi, Lo = 0, 1, 2
@@ -802,46 +839,63 @@ def generate_radial_section(red, match, nargs):
     if nkb > 4:
         return None, None
     # output rows per wavefront (32-row blocks) and wavefronts per workgroup: the accumulators (16 per block and
-    # output component) live in registers
+    # accumulated component) live in registers
     rb = 2 if Dv <= 2 else 1
     waves = 8
+    one = O.IntCst(1)
 
     class _W:
-        formula, tagI = (W if W is not None else O.IntCst(1)), red.tagI
+        formula, tagI = (W if W is not None else one), red.tagI
 
-    layout = VarLayout(_W)
-    if layout.rowvars:
+    class _A:
+        formula, tagI = (A if A is not None else one), red.tagI
+
+    wl, al = VarLayout(_W), VarLayout(_A)
+    if wl.rowvars or al.colvars:
         return None, None
-    # the parameter table serves both bodies: the one of the whole reduction (as the general-purpose kernel's)
+    # the parameter table serves every body: the one of the whole reduction (as the general-purpose kernel's)
     full = VarLayout(red)
     pnames = {key: name for key, name in full.names.items() if key[0] == 2}
-    w_names = dict(layout.names)
-    w_names.update(pnames)
-    L = Lir(row_cat=red.tagI, fast_math=True, dtype="float")
-    w_lines, w_exprs = L.emit(lower(_W.formula, L), w_names, indent="    ")
-    w_prelude = list(L.prelude)
-    Lk = Lir(row_cat=red.tagI, fast_math=True, dtype="float")
-    k_lines, k_exprs = Lk.emit(lower(coef, Lk), pnames, indent="    ")
-    ca, cd, co = VarLayout.table(layout.colvars)
-    meta = dict(radial=1, rad_d=D, rad_dv=Dv, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind, rad_yarg=y.ind)
+
+    def body(formula, names):
+        L = Lir(row_cat=red.tagI, fast_math=True, dtype="float")
+        nm = dict(names)
+        nm.update(pnames)
+        lines, exprs = L.emit(lower(formula, L), nm, indent="    ")
+        return list(L.prelude), lines, exprs
+
+    w_pre, w_lines, w_exprs = body(_W.formula, wl.names)
+    a_pre, a_lines, a_exprs = body(_A.formula, al.names)
+    k_pre, k_lines, k_exprs = body(coef, {})
+    ca, cd, co = VarLayout.table(wl.colvars)
+    ra, rd, ro = VarLayout.table(al.rowvars)
+    meta = dict(radial=1, rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
+                rad_yarg=y.ind)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
-    defs = dict(RAD_D=D, RAD_DV=Dv, RAD_NKB=nkb, RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind,
-                RAD_LIMIT=f"{float(config.radial_limit)!r}f", RAD_NCOLVARS=len(layout.colvars), RAD_DIMY=layout.dimy)
+    defs = dict(RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
+                RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit)!r}f",
+                RAD_NCOLVARS=len(wl.colvars), RAD_DIMY=wl.dimy, RAD_NROWVARS=len(al.rowvars), RAD_DIMX=al.dimx)
     src += [f"#define {k} {v}" for k, v in defs.items()]
     for name, vals in (("row_kind", [r[0] for r in rows]), ("row_comp", [r[1] for r in rows]), ("row_term", [r[2] for r in rows]),
                        ("col_kind", [c[0] for c in cols]), ("col_comp", [c[1] for c in cols]), ("col_term", [c[2] for c in cols]),
-                       ("col_arg", ca), ("col_dim", cd), ("col_off", co)):
+                       ("col_arg", ca), ("col_dim", cd), ("col_off", co), ("row_arg", ra), ("row_dim", rd), ("row_off", ro)):
         src.append(f"static __device__ constexpr int rad_{name}[] = {_c_list(vals)};")
-    dy, dp = max(1, layout.dimy), max(1, full.dimp)
-    src += w_prelude + list(Lk.prelude)
+    dy, dx, dp = max(1, wl.dimy), max(1, al.dimx), max(1, full.dimp)
+    src += w_pre + a_pre + k_pre
     src.append("struct KeopsRadFormula {")
-    src.append(f"  // log2(e) times the coefficient of the squared distance in the exponent")
+    src.append("  // log2(e) times the coefficient of the squared distance in the exponent")
     src.append(f"  static __device__ __forceinline__ T kappa(const T (&p)[{dp}]) {{")
     src += k_lines
     src.append(f"    return ({k_exprs[0]}) * {LOG2E!r}f;")
     src.append("  }")
-    src.append(f"  static __device__ __forceinline__ void weights(const T (&yj)[{dy}], const T (&p)[{dp}], T (&w)[{Dv}]) {{")
+    src.append("  // factors that depend on the reduced index: the weights of a column")
+    src.append(f"  static __device__ __forceinline__ void weights(const T (&yj)[{dy}], const T (&p)[{dp}], T (&w)[{dimw}]) {{")
     src += w_lines + [f"    w[{k}] = {e};" for k, e in enumerate(w_exprs)]
+    src.append("  }")
+    src.append("  // factors that depend on the output index: applied once per output row")
+    src.append(f"  static __device__ __forceinline__ T rowscale(const T (&xi)[{dx}], const T (&p)[{dp}]) {{")
+    src += a_lines
+    src.append(f"    return {a_exprs[0]};")
     src.append("  }\n};")
     src.append('#include "keops_radial_mfma.h"')
     return "\n".join(src) + "\n", meta

@@ -143,3 +143,37 @@ def test_matrix_core_exponents_under_graph_capture():
         torch.cuda.synchronize()
         got = out.clone()
         assert torch.equal(got, conv(x, y, b, g))
+
+
+@pytest.mark.parametrize("D", [3, 2])
+def test_gradients_wrt_points_and_weights_with_matrix_core_exponents(D):
+    """Backward pass of the Gaussian kernel sum: the gradients with respect to x, y and b are again Gaussian sums
+    (with a difference factor for the points) and take the same path; against the oracle's gradient body."""
+    from keops_amd import keops_io
+
+    M, N = 24000, 26000
+    rng = np.random.default_rng(50 + D)
+    x = rng.standard_normal((M, D)).astype(np.float32)
+    y = (rng.standard_normal((N, D)) - 0.2).astype(np.float32)
+    b = rng.standard_normal((N, 1)).astype(np.float32)
+    e = rng.standard_normal((M, 1)).astype(np.float32)     # incoming gradient
+    g = np.array([0.6], np.float32)
+    xd, yd, bd, gd = to_dev(x, y, b, g)
+    xd.requires_grad_(True), yd.requires_grad_(True), bd.requires_grad_(True)
+    out = _genred(D, 1)(xd, yd, bd, gd)
+    gx, gy, gb = torch.autograd.grad(out, [xd, yd, bd], torch.from_numpy(e).cuda())
+    # the two gradients with respect to the points accumulate D + 1 sums per row on the matrix-core path
+    assert sum(m.meta("rad_dv") == str(D + 1) and m.meta("rad_d") == str(D) for m in keops_io._modules.values()) >= 2
+    rows = np.sort(rng.choice(M, 1200, replace=False)).astype(np.int64)
+    ref = cpu_reduc("gauss_gradx", [x, y, b, g, e], M, N, D, rows=rows)
+    scale = cpu_reduc("gauss_gradx_abs", [x, y, b, g, e], M, N, D, rows=rows)
+    assert_sum_parity(gx[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
+    # gradient with respect to y_j: the same body with the roles of the two clouds (and of b and e) exchanged
+    cols = np.sort(rng.choice(N, 1200, replace=False)).astype(np.int64)
+    refy = cpu_reduc("gauss_gradx", [y, x, e, g, b], N, M, D, rows=cols)
+    scaley = cpu_reduc("gauss_gradx_abs", [y, x, e, g, b], N, M, D, rows=cols)
+    assert_sum_parity(gy[torch.from_numpy(cols).cuda()].cpu().numpy(), refy, scaley)
+    # gradient with respect to b_j: sum_i e_i K_ij
+    refb = cpu_reduc("gauss", [y, x, e, g], N, M, 1, rows=cols)
+    scaleb = cpu_reduc("gauss", [y, x, np.abs(e), g], N, M, 1, rows=cols)
+    assert_sum_parity(gb[torch.from_numpy(cols).cuda()].cpu().numpy(), refb, scaleb)
