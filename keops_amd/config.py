@@ -22,6 +22,8 @@ dimfinalchunk = 64
 block_size = 256           # threads per workgroup (4 wavefronts)
 max_rows_per_lane = int(os.environ.get("KEOPS_AMD_MAX_ROWS", 4))      # output rows held in the registers of one lane
 lds_tile_bytes = 16384     # LDS bytes of one staged column tile
+# block-sparse / batched launches: workgroups per compute unit that the choice of rows per lane keeps
+irregular_wg_per_cu = int(os.environ.get("KEOPS_AMD_IRREGULAR_WG_PER_CU", 16))
 # formula bodies of more than segment_threshold statements are cut into functions of segment_statements each
 segment_threshold = int(os.environ.get("KEOPS_AMD_SEGMENT_MIN", 1024))
 segment_statements = int(os.environ.get("KEOPS_AMD_SEGMENT", 512))

@@ -57,7 +57,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float knn_f32x4;
 #ifndef KNN_SPLIT
 #define KNN_SPLIT 0
 #endif
-static_assert(KNN_FQSETS <= 2 && KNN_SQSETS <= 2, "one lane per query owns its list in the replay and sampling kernels");
+static_assert(KNN_FQSETS <= 4 && KNN_SQSETS <= 2, "a lane owns the lists of at most two queries in the replay kernel, of one in the sampling kernel");
 #ifndef KNN_FTJ
 #define KNN_FTJ KNN_TJ                 // reference rows per staged tile of the fixed-threshold filter
 #endif
@@ -688,6 +688,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_thresholds(const Knn
 // bins (one LDS atomic each) that the owners fold into their lists.
 extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParams P, int fgrid_x) {
   constexpr int QW = 32 * KNN_FQSETS;
+  constexpr int QPL = (QW + 63) / 64;  // queries owned by a lane: l, l + 64, ...
   __shared__ int bin_n[QW];
   __shared__ float bin_d[QW * KNN_BIN];
   __shared__ int bin_j[QW * KNN_BIN];
@@ -700,23 +701,27 @@ extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParam
   const i64 logid = (slab * fgrid_x + bx) * KNN_FWAVES + wave;
   const i64 qw0 = bx * (KNN_FWAVES * QW) + (i64)wave * QW;
   const float inf = __builtin_huge_valf();
-  float ld[KNN_K];
-  int lj[KNN_K];
+  float ld[QPL][KNN_K];
+  int lj[QPL][KNN_K];
 #pragma unroll
-  for (int k = 0; k < KNN_K; k++) {
-    ld[k] = inf;
-    lj[k] = 0;
-  }
+  for (int o = 0; o < QPL; o++)
+#pragma unroll
+    for (int k = 0; k < KNN_K; k++) {
+      ld[o][k] = inf;
+      lj[o][k] = 0;
+    }
   volatile int* bn = bin_n;
   volatile float* bd = bin_d;
   volatile int* bj = bin_j;
   volatile float* kd = kth_d;
   volatile int* kj = kth_j;
-  if (lane < QW) {
-    bn[lane] = 0;
-    kd[lane] = inf;
-    kj[lane] = 0x7fffffff;
-  }
+#pragma unroll
+  for (int o = 0; o < QPL; o++)
+    if (lane + 64 * o < QW) {
+      bn[lane + 64 * o] = 0;
+      kd[lane + 64 * o] = inf;
+      kj[lane + 64 * o] = 0x7fffffff;
+    }
   __threadfence_block();
   const int count = P.logcount[logid];
   const int2* mylog = P.log + logid * P.logcap;
@@ -741,28 +746,32 @@ extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParam
         }
       }
       __threadfence_block();
-      if (lane < QW) {
-        const int n = min(bn[lane], KNN_BIN);
-        if (n > 0) {
-          bn[lane] = 0;
-          for (int i = 0; i < n; i++) {
-            const float cd = bd[lane * KNN_BIN + i];
-            const int cj = bj[lane * KNN_BIN + i];
-            // sorted insertion in registers: entry k becomes old[k-1] when the candidate goes before old[k-1],
-            // the candidate when it goes before old[k] only, and stays otherwise
-            bool before_cur = knn_better(cd, cj, ld[KNN_K - 1], lj[KNN_K - 1]);
 #pragma unroll
-            for (int k = KNN_K - 1; k > 0; k--) {
-              const bool before_prev = knn_better(cd, cj, ld[k - 1], lj[k - 1]);
-              ld[k] = before_prev ? ld[k - 1] : (before_cur ? cd : ld[k]);
-              lj[k] = before_prev ? lj[k - 1] : (before_cur ? cj : lj[k]);
-              before_cur = before_prev;
+      for (int o = 0; o < QPL; o++) {
+        const int qo = lane + 64 * o;
+        if (qo < QW) {
+          const int n = min(bn[qo], KNN_BIN);
+          if (n > 0) {
+            bn[qo] = 0;
+            for (int i = 0; i < n; i++) {
+              const float cd = bd[qo * KNN_BIN + i];
+              const int cj = bj[qo * KNN_BIN + i];
+              // sorted insertion in registers: entry k becomes old[k-1] when the candidate goes before old[k-1],
+              // the candidate when it goes before old[k] only, and stays otherwise
+              bool before_cur = knn_better(cd, cj, ld[o][KNN_K - 1], lj[o][KNN_K - 1]);
+#pragma unroll
+              for (int k = KNN_K - 1; k > 0; k--) {
+                const bool before_prev = knn_better(cd, cj, ld[o][k - 1], lj[o][k - 1]);
+                ld[o][k] = before_prev ? ld[o][k - 1] : (before_cur ? cd : ld[o][k]);
+                lj[o][k] = before_prev ? lj[o][k - 1] : (before_cur ? cj : lj[o][k]);
+                before_cur = before_prev;
+              }
+              ld[o][0] = before_cur ? cd : ld[o][0];
+              lj[o][0] = before_cur ? cj : lj[o][0];
             }
-            ld[0] = before_cur ? cd : ld[0];
-            lj[0] = before_cur ? cj : lj[0];
+            kd[qo] = ld[o][KNN_K - 1];
+            kj[qo] = lj[o][KNN_K - 1];
           }
-          kd[lane] = ld[KNN_K - 1];
-          kj[lane] = lj[KNN_K - 1];
         }
       }
       __threadfence_block();
@@ -770,13 +779,16 @@ extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParam
       pending = pending && knn_better(d, j, kd[ql], kj[ql]);
     }
   }
-  const i64 q = qw0 + lane;
-  if (lane < QW && q < P.nq) {
 #pragma unroll
-    for (int l = 0; l < KNN_K; l++) {
-      const i64 o = (slab * P.nq + q) * KNN_K + l;
-      P.plist_d[o] = ld[l];
-      P.plist_i[o] = lj[l];
+  for (int o = 0; o < QPL; o++) {
+    const i64 q = qw0 + lane + 64 * o;
+    if (lane + 64 * o < QW && q < P.nq) {
+#pragma unroll
+      for (int l = 0; l < KNN_K; l++) {
+        const i64 e = (slab * P.nq + q) * KNN_K + l;
+        P.plist_d[e] = ld[o][l];
+        P.plist_i[e] = lj[o][l];
+      }
     }
   }
 }

@@ -72,7 +72,7 @@ def choose_geometry(red, layout, nops, sizeof_t, nx=None, irregular=False):
         rows //= 2
     if nx is not None:
         # keep at least ~2 workgroups per compute unit when the row count allows it
-        while rows > 1 and nx < (16 if irregular else 2) * 256 * block * rows:
+        while rows > 1 and nx < (config.irregular_wg_per_cu if irregular else 2) * 256 * block * rows:
             rows //= 2
     tile_j = config.lds_tile_bytes // max(1, dimy_pad * sizeof_t)
     tile_j = max(64, min(1024, 1 << (tile_j.bit_length() - 1)))
@@ -172,8 +172,8 @@ def generate_knn_plugin(red, rowvar, colvar, nargs):
     # low dimensions: neighbours are close compared with the norms, the operands are split as hi + lo
     split = int(D < 32)
     qsets, tj = config.knn_qsets, config.knn_tile_j
-    if not (1 <= config.knn_filter_qsets <= 2 and 1 <= config.knn_sample_qsets <= 2 and 1 <= qsets <= 2):
-        raise ValueError("[KeOps] the KNN kernels take one or two 32-query operand sets per wavefront")
+    if not (1 <= config.knn_filter_qsets <= 4 and 1 <= config.knn_sample_qsets <= 2 and 1 <= qsets <= 2):
+        raise ValueError("[KeOps] the KNN kernels take one or two 32-query operand sets per wavefront (the filter: up to four)")
     # as many wavefronts as the LDS budget allows share one staged reference tile: the K-lists of the
     # 32*qsets queries of every wavefront live in LDS (8 bytes per entry)
     fixed = tj * (dpad * 2 * (1 + split) + 16) + tj * 4
