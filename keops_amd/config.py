@@ -42,6 +42,9 @@ chunk_max_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MAX_DIM", 1024))  # largest 
 
 # exponents of low-dimensional Gaussian kernel sums on the matrix cores (csrc/kernels/keops_radial_mfma.h)
 radial = os.environ.get("KEOPS_AMD_RADIAL", "1") != "0"
+# scalar weights join the exponents (columns partitioned by sign, add/subtract instead of fma: a few percent faster);
+# off by default: doubling the weights then no longer doubles the result bit for bit
+radial_fold = os.environ.get("KEOPS_AMD_RADIAL_FOLD", "0") == "1"
 radial_max_dim = 8                  # components of the points (7 D + 8 slots of the scalar product fit four instructions)
 radial_max_dv = 8                   # components of the weights (16 accumulators per component in every lane)
 # the path is taken when |c| log2(e) (max |x^|^2 + max |y^|^2) <= this bound for the centred points (checked on the

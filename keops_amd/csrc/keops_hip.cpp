@@ -571,6 +571,7 @@ struct RadHeader {
   void* colsum;
   void* colpart;
   void* scal;
+  void* blk;
   void* out;
   void* partial;
   int64_t slab_len;
@@ -586,16 +587,21 @@ int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* arg
   const int64_t D = m.meta_int("rad_d", 0), DV = m.meta_int("rad_dv", 0), NKB = m.meta_int("rad_nkb", 0);
   const int64_t RB = m.meta_int("rad_rb", 0), WAVES = m.meta_int("rad_waves", 0), TJ = 128;
   if (D <= 0 || DV <= 0 || NKB <= 0 || RB <= 0 || WAVES <= 0) return fail(-1, "corrupt radial module metadata");
-  const int64_t ntiles = (ny + TJ - 1) / TJ, rows_per_wg = 32 * RB * WAVES, row_blocks = (nx + rows_per_wg - 1) / rows_per_wg;
+  const bool fold = m.meta_int("rad_fold", 0) != 0;  // weights folded into the exponents, columns partitioned by sign
+  // (the partition pads both groups of columns to whole tiles: one more tile)
+  const int64_t ntiles = (ny + TJ - 1) / TJ + (fold ? 1 : 0), rows_per_wg = 32 * RB * WAVES, row_blocks = (nx + rows_per_wg - 1) / rows_per_wg;
   // slabs over the reduced axis: about 16 workgroups per compute unit, whole tiles per slab
   int64_t nslabs = std::max<int64_t>(1, (16 * (int64_t)m.cu_count + row_blocks - 1) / row_blocks);
   nslabs = std::min<int64_t>(nslabs, std::max<int64_t>(1, ntiles / 8));
-  int64_t slab_len = ((ny + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ;
-  nslabs = std::max<int64_t>(1, (ny + slab_len - 1) / slab_len);
+  const int64_t ncols = fold ? ntiles * TJ : ny;
+  int64_t slab_len = ((ncols + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ;
+  nslabs = std::max<int64_t>(1, (ncols + slab_len - 1) / slab_len);
   const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(256, ny / 1024));
+  const int64_t nblk = (ny + 255) / 256;
   size_t off = align_up(reserved, 256);
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
-  const size_t o_scal = take(16), o_colsum = take((size_t)D * 4), o_colpart = take((size_t)nparts * D * 4);
+  const size_t o_scal = take(32), o_colsum = take((size_t)D * 4), o_colpart = take((size_t)nparts * D * 4);
+  const size_t o_blk = take(fold ? (size_t)nblk * 4 : 0);
   const size_t o_xa = take((size_t)nx * NKB * 32), o_yb = take((size_t)ntiles * TJ * NKB * 32), o_bw = take((size_t)ntiles * TJ * DV * 4);
   const size_t o_part = take((size_t)nslabs * nx * DV * 4);
   if (int rc = m.partial.reserve(off)) return rc;
@@ -603,17 +609,26 @@ int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* arg
   std::vector<char> buf(sizeof(RadHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 16);
   RadHeader h{};
   h.nx = nx; h.ny = ny; h.xa = ws + o_xa; h.yb = ws + o_yb; h.bw = ws + o_bw; h.colsum = ws + o_colsum; h.colpart = ws + o_colpart;
-  h.scal = ws + o_scal; h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs; h.nparts = nparts;
+  h.scal = ws + o_scal; h.blk = ws + o_blk; h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs; h.nparts = nparts;
   std::memcpy(buf.data(), &h, sizeof(h));
   for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
   const size_t psize = sizeof(RadHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs);
   auto with_which = [&](int w) { std::memcpy(buf.data() + psize, &w, 4); return psize + 4; };
   if (int rc = launch_raw(m, "keops_rad_colsum", (unsigned)nparts, 1, 256, buf.data(), psize, stream)) return rc;
   if (int rc = launch_raw(m, "keops_rad_colsum_final", 1, 1, 64, buf.data(), psize, stream)) return rc;
+  if (fold) {
+    if (int rc = launch_raw(m, "keops_rad_sign_count", (unsigned)nblk, 1, 256, buf.data(), psize, stream)) return rc;
+    int nb32 = (int)nblk;
+    std::memcpy(buf.data() + psize, &nb32, 4);
+    if (int rc = launch_raw(m, "keops_rad_sign_scan", 1, 1, 1024, buf.data(), psize + 4, stream)) return rc;
+    const int64_t nc = ntiles * TJ;
+    std::memcpy(buf.data() + psize, &nc, 8);
+    if (int rc = launch_raw(m, "keops_rad_fill_dead", (unsigned)((nc + 255) / 256), 1, 256, buf.data(), psize + 8, stream)) return rc;
+  }
   size_t sz = with_which(0);
   if (int rc = launch_raw(m, "keops_rad_prep", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
   sz = with_which(1);
-  if (int rc = launch_raw(m, "keops_rad_prep", (unsigned)((ntiles * TJ + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_prep", (unsigned)(fold ? nblk : (ntiles * TJ + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
   if (int rc = launch_raw(m, "keops_rad_decide", 1, 1, 64, buf.data(), psize, stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
   if (int rc = launch_raw(m, "keops_rad_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)(64 * WAVES), buf.data(), psize, stream)) return rc;

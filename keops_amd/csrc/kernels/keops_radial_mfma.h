@@ -36,6 +36,16 @@
 // The lanes of a row are summed with shuffles once at the end; slabs over the reduced axis (blockIdx.y) are added
 // in order by keops_rad_reduce: deterministic.
 //
+// RAD_FOLD (a scalar weight w_j and no difference factor: the plain Gaussian kernel sum): exp2(t) w_j =
+// +- exp2(t + log2 |w_j|), so log2 |w_j| joins the column's squared-norm term (formed in double precision) and the
+// columns are partitioned by the sign of their weight (stable, deterministic: keops_rad_sign_count / _scan, then
+// keops_rad_prep scatters every column to its place; unused places hold "dead" columns whose exponent is -16384).
+// Tiles of non-negative weights are accumulated with one v_add_f32 per pair, the others with one v_sub_f32: half
+// the cost of the fused multiply-add (v_exp_f32 takes 8 issue cycles per wavefront, v_fmac_f32 4, v_add_f32 2).
+// The sweep alternates between the two groups tile by tile (rad_tile_of), so that the running sums stay as small
+// as with the weights in their original order: summing one sign after the other would carry rounding errors
+// relative to sum_j K_ij |w_j| into a result that may be much smaller.
+//
 // The plug-in defines RAD_D, RAD_DV, RAD_NKB (16-slot blocks), RAD_RB, RAD_WAVES, RAD_XARG, RAD_YARG, RAD_LIMIT,
 // the slot tables rad_slot_kind / rad_slot_comp / rad_slot_term for both sides, the tables of the variables of B
 // (rad_col_arg / rad_col_dim / rad_col_off, RAD_NCOLVARS, RAD_DIMY) and of the parameters (keops_par_*), and
@@ -59,7 +69,9 @@ struct RadParams {
   float* bw;          // [ntiles * RAD_TJ][RAD_DV] weights B_j (zero past the last column)
   float* colsum;      // [RAD_D] column sums of y
   float* colpart;     // [nparts][RAD_D]
-  unsigned* scal;     // [0], [1]: bit patterns of max |x^|^2, max |y^|^2; [2]: 1 when the matrix-core path is taken
+  unsigned* scal;     // [0], [1]: bit patterns of max |x^|^2, max |y^|^2; [2]: 1 when the matrix-core path is taken;
+                      // [3] (RAD_FOLD): number of tiles of columns with non-negative weights
+  int* blk;           // RAD_FOLD: [nblk] non-negative weights per block of 256 columns, then their exclusive scan
   T* out;             // [nx][RAD_DV]
   float* partial;     // [nslabs][nx][RAD_DV]
   i64 slab_len;       // reduced rows per slab (multiple of RAD_TJ)
@@ -107,8 +119,86 @@ extern "C" __global__ void __launch_bounds__(64) keops_rad_colsum_final(const Ra
     for (int b = 0; b < P.nparts; b++) s += (double)P.colpart[(i64)b * RAD_D + c];
     P.colsum[c] = (float)(s / (double)P.ny);  // the mean
   }
-  if (c < 3) P.scal[c] = 0u;
+  if (c < 4) P.scal[c] = 0u;
 }
+
+#ifndef RAD_FOLD
+#define RAD_FOLD 0
+#endif
+
+__device__ __forceinline__ float rad_column_weight(const RadParams& P, i64 j, const T (&p)[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1]) {
+  T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
+#pragma unroll
+  for (int v = 0; v < RAD_NCOLVARS; v++) {
+    const T* a = P.arg[rad_col_arg[v]] + j * rad_col_dim[v];
+#pragma unroll
+    for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
+  }
+  T wv[RAD_DW];
+  KeopsRadFormula::weights(yj, p, wv);
+  return (float)wv[0];
+}
+
+#if RAD_FOLD
+// columns with a non-negative weight, per block of 256 columns (a NaN weight counts as non-negative)
+extern "C" __global__ void __launch_bounds__(256) keops_rad_sign_count(const RadParams P) {
+  __shared__ int cnt[4];
+  const i64 j = (i64)blockIdx.x * 256 + threadIdx.x;
+  T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+  rad_load_params(P, p);
+  const bool pos = j < P.ny && !(rad_column_weight(P, j, p) < 0.f);
+  const unsigned long long bal = __ballot(pos);
+  if ((threadIdx.x & 63) == 0) cnt[threadIdx.x >> 6] = __popcll(bal);
+  __syncthreads();
+  if (threadIdx.x == 0) P.blk[blockIdx.x] = cnt[0] + cnt[1] + cnt[2] + cnt[3];
+}
+
+// exclusive scan of the block counts (one workgroup, sequential over chunks of 1024 blocks); scal[3] = tiles of
+// non-negative columns
+extern "C" __global__ void __launch_bounds__(1024) keops_rad_sign_scan(const RadParams P, int nblk) {
+  __shared__ int part[1024];
+  __shared__ int carry;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (int base = 0; base < nblk; base += 1024) {
+    const int b = base + threadIdx.x;
+    const int v = b < nblk ? P.blk[b] : 0;
+    part[threadIdx.x] = v;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) {  // inclusive scan in shared memory
+      const int t = (int)threadIdx.x >= o ? part[threadIdx.x - o] : 0;
+      __syncthreads();
+      part[threadIdx.x] += t;
+      __syncthreads();
+    }
+    if (b < nblk) P.blk[b] = carry + part[threadIdx.x] - v;
+    __syncthreads();
+    if (threadIdx.x == 1023) carry += part[1023];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) P.scal[3] = (unsigned)((carry + RAD_TJ - 1) / RAD_TJ);
+}
+
+// every place of the column operand starts as a dead column: exponent -16384 for every row
+extern "C" __global__ void __launch_bounds__(256) keops_rad_fill_dead(const RadParams P, i64 ncols) {
+  const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (i >= ncols) return;
+  const i64 tile = i / RAD_TJ;
+  const int c = (int)(i % RAD_TJ);
+#pragma unroll
+  for (int kb = 0; kb < RAD_NKB; kb++)
+#pragma unroll
+    for (int hf = 0; hf < 2; hf++) {
+      rad_bf16x8 v8;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const int s = kb * 16 + hf * 8 + e;
+        v8[e] = (rad_col_kind[s] == 3 && rad_col_term[s] == 0) ? (__bf16)(-16384.0f) : (__bf16)0.0f;
+      }
+      *reinterpret_cast<rad_bf16x8*>(P.yb + (((tile * RAD_NKB + kb) * 2 + hf) * RAD_TJ + c) * 8) = v8;
+    }
+}
+#endif
 
 __device__ __forceinline__ void rad_split3(float v, __bf16 (&t)[3]) {
   t[0] = (__bf16)v;
@@ -129,7 +219,11 @@ __device__ __forceinline__ void rad_split4(double v, __bf16 (&t)[4]) {
 extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams P, int which) {
   const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
   const i64 n = which ? P.ny : P.nx;
+#if RAD_FOLD
+  const i64 ntot = which ? (P.ny + 255) / 256 * 256 : P.nx;  // whole blocks: every lane takes part in the ranking
+#else
   const i64 ntot = which ? (P.ny + RAD_TJ - 1) / RAD_TJ * RAD_TJ : P.nx;
+#endif
   if (i >= ntot) return;
   T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
   rad_load_params(P, p);
@@ -150,7 +244,17 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
       nrm += c * c;
       rad_split3((float)(which ? c : -2.0 * kappa * c), ct[k]);
     }
+#if RAD_FOLD
+    // the weight joins the exponent: exp2(t) w = +- exp2(t + log2 |w|)
+    float wfold = 1.f;
+    if (which) {
+      wfold = rad_column_weight(P, i, p);
+      w[0] = wfold;
+    }
+    rad_split4(which ? kappa * nrm + (double)__ocml_log2_f64((double)__builtin_fabsf(wfold)) : kappa * nrm, nt);
+#else
     rad_split4(kappa * nrm, nt);
+#endif
     // largest centred squared norm (bit pattern of a non-negative float, rounded up): order-independent maximum
     atomicMax(P.scal + which, __float_as_uint((float)nrm * 1.000001f));
 #pragma unroll
@@ -160,7 +264,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
       const int term = which ? rad_col_term[s] : rad_row_term[s];
       slot[s] = kind == 0 ? (__bf16)0.0f : (kind == 1 ? (__bf16)1.0f : (kind == 2 ? ct[comp][term] : nt[term]));
     }
-    if (which) {
+    if (which && !RAD_FOLD) {
       T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
 #pragma unroll
       for (int v = 0; v < RAD_NCOLVARS; v++) {
@@ -192,8 +296,25 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
       *reinterpret_cast<rad_bf16x8*>(P.xa + i * RAD_SLOTS + c8 * 8) = v8;
     }
   } else {
+#if RAD_FOLD
+    // stable partition by the sign of the weight: rank of this column among the non-negative (or negative) ones
+    __shared__ int wcnt[4];
+    const bool real = i < n, posw = real && !(w[0] < 0.f);
+    const unsigned long long bal = __ballot(posw);
+    const int lane = threadIdx.x & 63, wv_ = threadIdx.x >> 6;
+    if (lane == 0) wcnt[wv_] = __popcll(bal);
+    __syncthreads();
+    int before = __popcll(bal & ((1ull << lane) - 1ull));
+    for (int k = 0; k < wv_; k++) before += wcnt[k];
+    const i64 npos_before = (i64)P.blk[blockIdx.x] + before;
+    if (!real || w[0] == 0.f) return;  // zero weights: the place stays dead
+    const i64 dst = posw ? npos_before : (i64)P.scal[3] * RAD_TJ + (i - npos_before);
+    const i64 tile = dst / RAD_TJ;
+    const int c = (int)(dst % RAD_TJ);
+#else
     const i64 tile = i / RAD_TJ;
     const int c = (int)(i % RAD_TJ);
+#endif
 #pragma unroll
     for (int kb = 0; kb < RAD_NKB; kb++)
 #pragma unroll
@@ -203,8 +324,10 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
         for (int e = 0; e < 8; e++) v8[e] = slot[kb * 16 + hf * 8 + e];
         *reinterpret_cast<rad_bf16x8*>(P.yb + (((tile * RAD_NKB + kb) * 2 + hf) * RAD_TJ + c) * 8) = v8;
       }
+#if !RAD_FOLD
 #pragma unroll
     for (int d = 0; d < RAD_DV; d++) P.bw[i * RAD_DV + d] = w[d];
+#endif
   }
 }
 
@@ -218,12 +341,29 @@ extern "C" __global__ void __launch_bounds__(64) keops_rad_decide(const RadParam
   P.scal[2] = (__builtin_fabsf(kappa) * R <= (float)RAD_LIMIT) ? 1u : 0u;  // false for NaN
 }
 
+#if RAD_FOLD
+// k-th tile of the sweep: tiles of the two sign groups alternate while both last, then the rest of the larger group
+__device__ __forceinline__ i64 rad_tile_of(i64 k, i64 pos_tiles, i64 all_tiles, bool& negative) {
+  const i64 neg_tiles = all_tiles - pos_tiles, m = pos_tiles < neg_tiles ? pos_tiles : neg_tiles;
+  if (k < 2 * m) {
+    negative = (k & 1) != 0;
+    return negative ? pos_tiles + (k >> 1) : (k >> 1);
+  }
+  negative = pos_tiles <= neg_tiles;
+  return (negative ? pos_tiles : 0) + m + (k - 2 * m);
+}
+#endif
+
 // ---- main kernel ------------------------------------------------------------------------------------------------
 
-extern "C" __global__ void __launch_bounds__(RAD_BLOCK) keops_rad_main(const RadParams P) {
+// with at most 32 accumulators per lane the kernel fits 128 registers: four wavefronts per SIMD, two workgroups per CU
+#define RAD_MIN_WAVES ((RAD_RB * 16 * RAD_DV <= 32) ? 4 : 1)
+extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad_main(const RadParams P) {
   if (P.scal[2] != 1u) return;
   __shared__ __attribute__((aligned(16))) __bf16 ys[RAD_NKB * 2 * RAD_TJ * 8];  // [kb][half][col][8]
+#if !RAD_FOLD
   __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_DV];
+#endif
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
   const i64 row0 = ((i64)blockIdx.x * RAD_WAVES + wave) * (32 * RAD_RB);
   rad_bf16x8 a[RAD_RB][RAD_NKB];
@@ -242,26 +382,40 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK) keops_rad_main(const Rad
 #pragma unroll
       for (int d = 0; d < RAD_DV; d++) acc[r][v][d] = 0.f;
 
-  const i64 jbeg = (i64)blockIdx.y * P.slab_len, jend = keops_min(P.ny, jbeg + P.slab_len);
+  // (RAD_FOLD: the partition by sign pads both groups to whole tiles: one more tile than the columns need)
+  const i64 ncols = RAD_FOLD ? ((P.ny + RAD_TJ - 1) / RAD_TJ + 1) * RAD_TJ : P.ny;
+  const i64 jbeg = (i64)blockIdx.y * P.slab_len, jend = keops_min(ncols, jbeg + P.slab_len);
   // software pipeline: tile t+1 travels to registers while tile t is consumed
   constexpr int CH = RAD_NKB * 2 * RAD_TJ;  // 16-byte chunks of the slot vectors of a tile
   constexpr int NPF = (CH + RAD_BLOCK - 1) / RAD_BLOCK;
   constexpr int NPW = (RAD_TJ * RAD_DV + RAD_BLOCK - 1) / RAD_BLOCK;
   uint4 pf[NPF];
+#if !RAD_FOLD
   float pfw[NPW];
+#else
+  const i64 pos_tiles = keops_uniform((i64)P.scal[3]);  // tiles of columns with non-negative weights come first
+#endif
   auto prefetch = [&](i64 j0) {
-    const uint4* src = reinterpret_cast<const uint4*>(P.yb + (j0 / RAD_TJ) * (RAD_NKB * 2 * RAD_TJ * 8));
+#if RAD_FOLD
+    bool neg_;
+    const i64 tile = rad_tile_of(j0 / RAD_TJ, pos_tiles, ncols / RAD_TJ, neg_);
+#else
+    const i64 tile = j0 / RAD_TJ;
+#endif
+    const uint4* src = reinterpret_cast<const uint4*>(P.yb + tile * (RAD_NKB * 2 * RAD_TJ * 8));
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * RAD_BLOCK;
       pf[u] = e < CH ? src[e] : make_uint4(0u, 0u, 0u, 0u);
     }
+#if !RAD_FOLD
     const float* wsrc = P.bw + j0 * RAD_DV;  // padded to whole tiles
 #pragma unroll
     for (int u = 0; u < NPW; u++) {
       const int e = tid + u * RAD_BLOCK;
       pfw[u] = e < RAD_TJ * RAD_DV ? wsrc[e] : 0.f;
     }
+#endif
   };
   if (jbeg < jend) prefetch(jbeg);
   for (i64 j0 = jbeg; j0 < jend; j0 += RAD_TJ) {
@@ -271,22 +425,30 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK) keops_rad_main(const Rad
       const int e = tid + u * RAD_BLOCK;
       if (e < CH) reinterpret_cast<uint4*>(ys)[e] = pf[u];
     }
+#if !RAD_FOLD
 #pragma unroll
     for (int u = 0; u < NPW; u++) {
       const int e = tid + u * RAD_BLOCK;
       if (e < RAD_TJ * RAD_DV) bs[e] = pfw[u];
     }
+#endif
     __syncthreads();
     if (j0 + RAD_TJ < jend) prefetch(j0 + RAD_TJ);
+#if RAD_FOLD
+    bool negative;  // uniform: one sign per tile
+    (void)rad_tile_of(j0 / RAD_TJ, pos_tiles, ncols / RAD_TJ, negative);
+#endif
 #pragma unroll
     for (int sub = 0; sub < RAD_NSUB; sub++) {
       const int c = sub * 32 + col;
       rad_bf16x8 b[RAD_NKB];
 #pragma unroll
       for (int kb = 0; kb < RAD_NKB; kb++) b[kb] = *reinterpret_cast<const rad_bf16x8*>(ys + ((kb * 2 + half) * RAD_TJ + c) * 8);
+#if !RAD_FOLD
       float w[RAD_DV];
 #pragma unroll
       for (int d = 0; d < RAD_DV; d++) w[d] = bs[c * RAD_DV + d];
+#endif
       rad_f32x16 t[RAD_RB];
 #pragma unroll
       for (int r = 0; r < RAD_RB; r++) {
@@ -297,6 +459,19 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK) keops_rad_main(const Rad
         for (int kb = 0; kb < RAD_NKB; kb++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r][kb], b[kb], z, 0, 0, 0);
         t[r] = z;
       }
+#if RAD_FOLD
+      if (!negative) {
+#pragma unroll
+        for (int r = 0; r < RAD_RB; r++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) acc[r][v][0] += __builtin_amdgcn_exp2f(t[r][v]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < RAD_RB; r++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) acc[r][v][0] -= __builtin_amdgcn_exp2f(t[r][v]);
+      }
+#else
 #pragma unroll
       for (int r = 0; r < RAD_RB; r++)
 #pragma unroll
@@ -305,6 +480,7 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK) keops_rad_main(const Rad
 #pragma unroll
           for (int d = 0; d < RAD_DV; d++) acc[r][v][d] = __builtin_fmaf(e, w[d], acc[r][v][d]);
         }
+#endif
     }
   }
   // the 32 lanes of a half hold the same rows for different columns: shuffle sums, then one lane stores

@@ -869,10 +869,12 @@ def generate_radial_section(red, match, nargs):
     k_pre, k_lines, k_exprs = body(coef, {})
     ca, cd, co = VarLayout.table(wl.colvars)
     ra, rd, ro = VarLayout.table(al.rowvars)
+    # a scalar weight and no difference factor: the weight joins the exponent, columns are partitioned by its sign
+    fold = int(config.radial_fold and dimw == 1 and not diff)
     meta = dict(radial=1, rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
-                rad_yarg=y.ind)
+                rad_yarg=y.ind, rad_fold=fold)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
-    defs = dict(RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
+    defs = dict(RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
                 RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit)!r}f",
                 RAD_NCOLVARS=len(wl.colvars), RAD_DIMY=wl.dimy, RAD_NROWVARS=len(al.rowvars), RAD_DIMX=al.dimx)
     src += [f"#define {k} {v}" for k, v in defs.items()]
@@ -925,7 +927,7 @@ def get_keops_dll(
         rows_hint = nx if nx < 64 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
            use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs),
-           binder.templates_digest())
+           binder.templates_digest(), bool(config.radial), bool(config.radial_fold))
     with _lock:
         hit = _cache.get(key)
     if hit is not None:

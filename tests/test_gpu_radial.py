@@ -56,6 +56,37 @@ def test_gaussian_sums_with_matrix_core_exponents_vs_oracle(D, Dv, M, N):
     assert torch.equal(_genred(D, Dv)(*dev), got)
 
 
+@pytest.mark.parametrize("D,M,N,signs", [(3, 30011, 30500, "mixed"), (8, 16000, 18000, "positive"), (2, 9000, 40000, "negative")])
+def test_scalar_weights_folded_into_the_exponents_vs_oracle(D, M, N, signs):
+    """Opt-in variant (config.radial_fold): log2|b_j| joins the exponent, the columns are partitioned by the sign of
+    b_j and the main loop adds or subtracts exp2 of whole tiles.  Same parity bar; zero weights contribute nothing."""
+    from keops_amd import config, keops_io
+
+    rng = np.random.default_rng(7 * D)
+    x = rng.standard_normal((M, D)).astype(np.float32)
+    y = rng.standard_normal((N, D)).astype(np.float32)
+    b = rng.standard_normal((N, 1)).astype(np.float32)
+    b = b if signs == "mixed" else np.abs(b) if signs == "positive" else -np.abs(b)
+    b[::97] = 0.0
+    g = np.array([0.7], np.float32)
+    dev = to_dev(x, y, b, g)
+    saved, loaders = config.radial_fold, dict(keops_io._loaders)
+    try:
+        config.radial_fold = True
+        keops_io._loaders.clear()
+        got = _genred(D, 1)(*dev)
+        assert _last_meta("rad_fold") == "1"
+        assert torch.equal(_genred(D, 1)(*dev), got)
+    finally:
+        config.radial_fold = saved
+        keops_io._loaders.clear()
+        keops_io._loaders.update(loaders)
+    rows = np.sort(rng.choice(M, 1500, replace=False)).astype(np.int64)
+    ref = cpu_reduc("gauss", [x, y, b, g], M, N, 1, rows=rows)
+    scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, 1, rows=rows)
+    assert_sum_parity(got[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
+
+
 def test_reduction_over_i_and_formula_spellings():
     from keops_amd.torch import Genred
 
