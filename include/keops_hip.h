@@ -79,7 +79,14 @@ void keops_hip_module_destroy(void* module);
  *   indsi/j/p, dims*  argument indices and dimensions of the i, j and parameter variables
  *   ranges            7 pointers: ranges_i, slices_i, redranges_j, ranges_j, slices_j, redranges_i
  *                     (int64, on the data's device) and a HOST int64[6] with their row counts;
- *                     ranges[6][0] == -1 means "no ranges" (LoadKeOps.py:11-12,194-202)
+ *                     ranges[6][0] == -1 means "no ranges" (LoadKeOps.py:11-12,194-202).  The first launch of a
+ *                     module with a given set of range tensors (same pointers and sizes) reads them back, checks
+ *                     every index against its axis and fails with a message otherwise, as the reference reads
+ *                     ranges_i back at every call (keops_nvrtc.cpp:195-197).  Later launches with the same tensors
+ *                     build the workgroup table on the device from the tensors' current contents: no read-back,
+ *                     no synchronisation, can be recorded in a HIP graph; indices that are out of bounds by then
+ *                     are clamped and reported by keops_hip_ranges_status (KEOPS_HIP_DEVICE_RANGES=0: always the
+ *                     first kind)
  *   shapeout          shape of out; out has prod(shapeout) elements
  *   args, argshapes   nargs device pointers; their shapes are concatenated in argshapes_flat,
  *                     argndims[k] entries each
@@ -137,6 +144,14 @@ int keops_hip_launch_noalloc(void* module, int64_t nx, int64_t ny, int tagI, int
                              const int64_t* shapeout, int nshapeout, void* out, void* const* args,
                              const int64_t* argshapes_flat, const int* argndims, void* hip_stream);
 size_t keops_hip_noalloc_scratch_bytes(void);
+
+/*
+ * Status of the module's last block-sparse launch whose table was built on the device (see `ranges` above); waits for
+ * that launch.  *status: 0 fine (or no such launch yet), bit 0: an index of the ranges was out of bounds and has
+ * been clamped to its axis, bit 1: the row ranges overlap so much that they need more workgroups than rows allow
+ * (the surplus was dropped).  No counterpart in the reference, which validates nothing (Sizes.h:12).
+ */
+int keops_hip_ranges_status(void* module, unsigned* status);
 
 /*
  * Loop-only calibration of the instruction issue rates the roofline fractions are held against: runs a grid of

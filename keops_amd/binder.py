@@ -55,6 +55,7 @@ def lib():
         ]
         L.keops_hip_noalloc_scratch_bytes.restype = ctypes.c_size_t
         L.keops_hip_calibrate.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 2
+        L.keops_hip_ranges_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint)]
         _lib = L
     return _lib
 
@@ -126,6 +127,14 @@ class Module:
 
     def set_timing(self, enabled):
         lib().keops_hip_module_set_timing(self.handle, int(bool(enabled)))
+
+    def ranges_status(self):
+        """Status bits of the last block-sparse launch whose table was built on the device
+        (keops_hip_ranges_status of include/keops_hip.h); waits for that launch."""
+        st = ctypes.c_uint(0)
+        if lib().keops_hip_ranges_status(self.handle, ctypes.byref(st)) != 0:
+            raise KeOpsHipError(last_error())
+        return int(st.value)
 
     def last_kernel_ms(self):
         return lib().keops_hip_module_last_kernel_ms(self.handle)

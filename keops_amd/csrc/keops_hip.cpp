@@ -262,6 +262,11 @@ struct Module {
   bool tables_in_flight = false;
   std::vector<int64_t> tables_key;  // batch mode: shape signature of the cached tables
   int64_t cached_nblocks = 0;
+  // block-sparse mode: signature (pointers, sizes, geometry) of the ranges the host path has read and validated, the
+  // number of workgroups it found, and where the device path keeps its status word
+  std::vector<int64_t> ranges_key;
+  int64_t ranges_nblocks = 0;
+  const unsigned* ranges_status = nullptr;
   DeviceBuffer staging;  // host-pointer launches (tagHostDevice = 0): device copies of the arguments and of out
   // a launch was recorded into a HIP graph: workspaces and tables keep their address and contents from then on
   bool captured = false;
@@ -330,6 +335,15 @@ bool stream_is_capturing(hipStream_t stream) {
   return st != hipStreamCaptureStatusNone;
 }
 
+// KEOPS_HIP_DEVICE_RANGES=0 keeps every block-sparse launch on the host path (read-back and validation per call)
+bool device_ranges_enabled() {
+  static const bool on = [] {
+    const char* e = std::getenv("KEOPS_HIP_DEVICE_RANGES");
+    return !(e && e[0] == '0');
+  }();
+  return on;
+}
+
 int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ranges, int64_t* const* ranges,
                          int64_t rows_total, int64_t cols_total, int64_t rows_per_block, bool by_arg, const std::vector<int>& rowvars,
                          const std::vector<int>& colvars, const std::vector<int>& vP, hipStream_t stream, RangeTables& rt) {
@@ -342,16 +356,57 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
   std::vector<int64_t> synth;  // batch mode: [slices (nbatches)] [ranges_y (2*nbatches)]
   std::vector<int64_t> range_work;  // block-sparse mode: reduced rows per row range
 
+  std::vector<int64_t> ukey;  // signature of a block-sparse call
   if (user_ranges) {
     const int sel = tagI == 0 ? 0 : 3;
     nranges = ranges[6][sel];
     rx_dev = ranges[sel];
     slices_dev = ranges[sel + 1];
     ry_dev = ranges[sel + 2];
+    const int64_t nred_u = ranges[6][sel + 2];
+    ukey = {tagI, by_arg ? 1 : 0, rows_per_block, (int64_t)(intptr_t)rx_dev, (int64_t)(intptr_t)slices_dev,
+            (int64_t)(intptr_t)ry_dev, nranges, ranges[6][sel + 1], nred_u, rows_total, cols_total};
+    if (device_ranges_enabled() && nb == 0 && nranges >= 0 && nred_u >= 0 && ukey == m.ranges_key) {
+      // These ranges (same tensors, same sizes) have been read and validated by an earlier call: the table is now
+      // built on the device from their current contents, with every index clamped to its axis.  No read-back, no
+      // synchronisation; the launch can be recorded in a HIP graph.
+      if (g_noalloc) return fail(-1, "keops_hip_launch_noalloc: block-sparse and batched launches build device tables");
+      const int64_t nblocks_max = std::max(nranges + rows_total / rows_per_block, m.ranges_nblocks);
+      const size_t words = keops_static_range_build_words(nranges, nred_u, nblocks_max);
+      const bool capturing = stream_is_capturing(stream);
+      if (!capturing && m.tables.frozen && m.tables.ptr != nullptr) m.tables.retire();
+      if (m.tables_in_flight) {
+        HIP_TRY(hipEventSynchronize(m.tables_copied));
+        m.tables_in_flight = false;
+      }
+      if (int rc = m.tables.reserve(words * sizeof(int64_t))) return rc;
+      m.tables_key.clear();  // whatever batch tables the buffer held are gone
+      long long* base = (long long*)m.tables.ptr;
+      KeopsRangeBuild B;
+      B.rx = (const long long*)rx_dev; B.sl = (const long long*)slices_dev; B.ry = (const long long*)ry_dev;
+      B.nranges = nranges; B.nred = nred_u; B.rows_total = rows_total; B.cols_total = cols_total;
+      B.rows_per_block = rows_per_block; B.nblocks_max = nblocks_max;
+      B.lookup = base;
+      B.sl_clean = B.lookup + 3 * nblocks_max;
+      B.ry_clean = B.sl_clean + nranges;
+      B.nb = B.ry_clean + 2 * nred_u;
+      B.work = B.nb + nranges;
+      B.order = B.work + nranges;
+      B.offs = B.order + nranges;
+      B.status = (unsigned*)(B.offs + nranges);
+      if (int e = keops_static_build_ranges(&B, stream)) return fail(e, "building the range tables on the device failed");
+      m.ranges_status = B.status;
+      rt.nblocks = nblocks_max;
+      rt.lookup = (const int64_t*)B.lookup;
+      rt.offsets = nullptr;
+      rt.slices_x = (const int64_t*)B.sl_clean;
+      rt.ranges_y = (const int64_t*)B.ry_clean;
+      return 0;
+    }
     rx_host.resize((size_t)2 * nranges);
     if (stream_is_capturing(stream))
-      return fail(-1, "block-sparse ranges are read back from the device at every call: such a launch cannot be "
-                      "captured in a HIP graph");
+      return fail(-1, "the first launch with a set of block-sparse ranges reads them back from the device to validate "
+                      "them: it cannot be captured in a HIP graph (run the call once eagerly, then capture it)");
     // same synchronous read-back as the reference (keops_nvrtc.cpp:195-197)
     if (nranges) HIP_TRY(hipMemcpyAsync(rx_host.data(), rx_dev, sizeof(int64_t) * 2 * nranges, hipMemcpyDeviceToHost, stream));
     // the slices and reduced ranges too: workgroups are issued longest first (below)
@@ -482,13 +537,21 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
       }
     }
     if (n_syn) std::memcpy(syn, synth.data(), n_syn * sizeof(int64_t));
-    if (int rc = m.tables.reserve(total * sizeof(int64_t))) return rc;
+    // (block-sparse mode: room for the tables that later calls with these ranges build on the device)
+    const size_t dev_words = (user_ranges && nb == 0)
+        ? keops_static_range_build_words(nranges, ranges[6][(tagI == 0 ? 0 : 3) + 2], std::max(nranges + rows_total / rows_per_block, nblocks)) : 0;
+    if (int rc = m.tables.reserve(std::max(total, dev_words) * sizeof(int64_t))) return rc;
     HIP_TRY(hipMemcpyAsync(m.tables.ptr, m.pinned, total * sizeof(int64_t), hipMemcpyHostToDevice, stream));
     if (!m.tables_copied) HIP_TRY(hipEventCreateWithFlags(&m.tables_copied, hipEventDisableTiming));
     HIP_TRY(hipEventRecord(m.tables_copied, stream));
     m.tables_in_flight = true;
     m.tables_key = key;
     m.cached_nblocks = nblocks;
+  }
+  if (user_ranges) {
+    m.ranges_key = ukey;  // read and validated: later calls build the table on the device
+    m.ranges_nblocks = nblocks;
+    m.ranges_status = nullptr;
   }
   const int64_t* tab = (const int64_t*)m.tables.ptr;
   rt.nblocks = nblocks;
@@ -1530,6 +1593,17 @@ int keops_hip_launch_noalloc(void* module, int64_t nx, int64_t ny, int tagI, int
   g_noalloc = false;
   std::swap(m.partial, view);
   return rc;
+}
+
+int keops_hip_ranges_status(void* module, unsigned* status) {
+  if (!module || !status) return fail(-1, "keops_hip_ranges_status: null argument");
+  Module& m = *static_cast<Module*>(module);
+  *status = 0u;
+  if (!m.ranges_status) return 0;
+  HIP_TRY(hipSetDevice(m.device));
+  if (m.has_last) HIP_TRY(hipEventSynchronize(m.last_done));
+  HIP_TRY(hipMemcpy(status, m.ranges_status, sizeof(unsigned), hipMemcpyDeviceToHost));
+  return 0;
 }
 
 size_t keops_hip_noalloc_scratch_bytes(void) { return (size_t)KEOPS_STATIC_SCRATCH_BYTES; }

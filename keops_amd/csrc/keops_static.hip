@@ -1,6 +1,7 @@
 // Device code that is compiled into libkeops_hip.so itself (everything else is JIT-compiled per formula):
 //   * the static scratch buffer of the entry point that allocates nothing (keops_hip_launch_noalloc),
 //   * a fill kernel (zero formulas: a kernel instead of hipMemsetAsync, which must stay out of captured graphs),
+//   * the kernels that build the lookup table of a block-sparse launch from the caller's ranges on the device,
 //   * loop-only calibration kernels for the vector ALU and the matrix cores (keops_hip_calibrate): they measure
 //     what an instruction stream without memory traffic sustains, the ceiling the map-reduce kernels are held to.
 #include <hip/hip_runtime.h>
@@ -52,6 +53,131 @@ int keops_static_fill_zero(void* dst, size_t bytes, void* stream) {
   const long long n = (long long)(bytes / 4);
   if (n == 0) return 0;
   hipLaunchKernelGGL(keops_fill_zero_u32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, (uint32_t*)dst, n);
+  return (int)hipGetLastError();
+}
+
+// ---- lookup table of block-sparse launches, built on the device --------------------------------------------------
+//
+// Counterpart of range_preprocess_from_device (keopscore/keopscore/binders/nvrtc/keops_nvrtc.cpp:152-248), which
+// copies the row ranges to the host at every call, builds the table there and copies it back.  Here the table is
+// built by a few small kernels on the launch stream: no read-back, no synchronisation, and the launch can be
+// recorded in a HIP graph.  The number of workgroups is not known on the host, so the grid has nblocks_max =
+// nranges + rows_total / rows_per_block workgroups (enough for disjoint row ranges) and the surplus ones find an
+// empty entry and return.  Every index is clamped to its axis (the map-reduce kernels sweep the ranges unchecked);
+// status records that something had to be clamped.  Row ranges are ordered by the reduced rows they sweep, longest
+// first, as the host path does (stable: ties keep their order), up to 16384 ranges; beyond, in table order.
+
+static __global__ void __launch_bounds__(256) keops_ranges_clean_y(const KeopsRangeBuild B) {
+  const long long k = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (k >= B.nred) return;
+  const long long a = B.ry[2 * k], b = B.ry[2 * k + 1];
+  const long long a2 = a < 0 ? 0 : (a > B.cols_total ? B.cols_total : a);
+  const long long b2 = b < a2 ? a2 : (b > B.cols_total ? B.cols_total : b);
+  B.ry_clean[2 * k] = a2;
+  B.ry_clean[2 * k + 1] = b2;
+  if (a2 != a || b2 != b) atomicOr(B.status, 1u);
+}
+
+static __global__ void __launch_bounds__(256) keops_ranges_rows(const KeopsRangeBuild B) {
+  const long long r = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (r >= B.nranges) return;
+  const long long s = B.rx[2 * r], e = B.rx[2 * r + 1];
+  const long long s2 = s < 0 ? 0 : (s > B.rows_total ? B.rows_total : s);
+  const long long e2 = e < s2 ? s2 : (e > B.rows_total ? B.rows_total : e);
+  auto clamp_slice = [&](long long v) { return v < 0 ? 0 : (v > B.nred ? B.nred : v); };
+  const long long a = r == 0 ? 0 : clamp_slice(B.sl[r - 1]), b = clamp_slice(B.sl[r]);
+  if (s2 != s || e2 != e || b != B.sl[r]) atomicOr(B.status, 1u);
+  B.sl_clean[r] = b;
+  B.nb[r] = (e2 - s2 + B.rows_per_block - 1) / B.rows_per_block;
+  long long w = 0;
+  for (long long k = a; k < b; k++) w += B.ry_clean[2 * k + 1] - B.ry_clean[2 * k];
+  B.work[r] = w;
+}
+
+// order[rank] = r with rank = number of ranges that come before r in a stable sort by decreasing work
+static __global__ void __launch_bounds__(256) keops_ranges_rank(const KeopsRangeBuild B, int sorted) {
+  __shared__ long long ws[256];
+  const long long r = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (!sorted) {
+    if (r < B.nranges) B.order[r] = r;
+    return;
+  }
+  const long long w = r < B.nranges ? B.work[r] : 0;
+  long long rank = 0;
+  for (long long q0 = 0; q0 < B.nranges; q0 += 256) {
+    __syncthreads();
+    ws[threadIdx.x] = q0 + threadIdx.x < B.nranges ? B.work[q0 + threadIdx.x] : -1;
+    __syncthreads();
+    const int n = (int)(B.nranges - q0 < 256 ? B.nranges - q0 : 256);
+    for (int t = 0; t < n; t++) {
+      const long long wq = ws[t];
+      rank += (wq > w || (wq == w && q0 + t < r)) ? 1 : 0;
+    }
+  }
+  if (r < B.nranges) B.order[rank] = r;
+}
+
+// offs[i] = first workgroup of the i-th range in issue order (one workgroup of 1024 threads scans everything)
+static __global__ void __launch_bounds__(1024) keops_ranges_scan(const KeopsRangeBuild B) {
+  __shared__ long long part[1024];
+  const int t = threadIdx.x;
+  const long long per = (B.nranges + 1023) / 1024, lo = t * per, hi = lo + per < B.nranges ? lo + per : B.nranges;
+  long long s = 0;
+  for (long long i = lo; i < hi; i++) s += B.nb[B.order[i]];
+  part[t] = s;
+  __syncthreads();
+  for (int o = 1; o < 1024; o <<= 1) {
+    const long long v = t >= o ? part[t - o] : 0;
+    __syncthreads();
+    part[t] += v;
+    __syncthreads();
+  }
+  long long run = part[t] - s;  // exclusive
+  for (long long i = lo; i < hi; i++) {
+    B.offs[i] = run;
+    run += B.nb[B.order[i]];
+  }
+  if (t == 1023 && part[1023] > B.nblocks_max) atomicOr(B.status, 2u);
+}
+
+// every entry starts empty (range 0, no rows)
+static __global__ void __launch_bounds__(256) keops_ranges_clear(const KeopsRangeBuild B) {
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (e < 3 * B.nblocks_max) B.lookup[e] = 0;
+}
+
+static __global__ void __launch_bounds__(256) keops_ranges_fill(const KeopsRangeBuild B) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= B.nranges) return;
+  const long long r = B.order[i];
+  const long long s = B.rx[2 * r], e = B.rx[2 * r + 1];
+  const long long s2 = s < 0 ? 0 : (s > B.rows_total ? B.rows_total : s);
+  const long long e2 = e < s2 ? s2 : (e > B.rows_total ? B.rows_total : e);
+  long long idx = B.offs[i];
+  for (long long j = s2; j < e2 && idx < B.nblocks_max; j += B.rows_per_block, idx++) {
+    B.lookup[3 * idx] = r;
+    B.lookup[3 * idx + 1] = j;
+    B.lookup[3 * idx + 2] = j + B.rows_per_block < e2 ? j + B.rows_per_block : e2;
+  }
+}
+
+size_t keops_static_range_build_words(long long nranges, long long nred, long long nblocks_max) {
+  return (size_t)(3 * nblocks_max + nranges + 2 * nred + 4 * nranges + 2);
+}
+
+int keops_static_build_ranges(const KeopsRangeBuild* b, void* stream) {
+  const KeopsRangeBuild B = *b;
+  hipStream_t st = (hipStream_t)stream;
+  auto grid = [](long long n) { return dim3((unsigned)((n + 255) / 256 > 0 ? (n + 255) / 256 : 1)); };
+  hipLaunchKernelGGL(keops_fill_zero_u32, dim3(1), dim3(256), 0, st, (uint32_t*)B.status, 1LL);
+  hipLaunchKernelGGL(keops_ranges_clear, grid(3 * B.nblocks_max), dim3(256), 0, st, B);
+  if (B.nred > 0) hipLaunchKernelGGL(keops_ranges_clean_y, grid(B.nred), dim3(256), 0, st, B);
+  if (B.nranges > 0) {
+    hipLaunchKernelGGL(keops_ranges_rows, grid(B.nranges), dim3(256), 0, st, B);
+    hipLaunchKernelGGL(keops_ranges_rank, grid(B.nranges), dim3(256), 0, st, B, B.nranges <= 16384 ? 1 : 0);
+    hipLaunchKernelGGL(keops_ranges_scan, dim3(1), dim3(1024), 0, st, B);
+    hipLaunchKernelGGL(keops_ranges_fill, grid(B.nranges), dim3(256), 0, st, B);
+  }
   return (int)hipGetLastError();
 }
 

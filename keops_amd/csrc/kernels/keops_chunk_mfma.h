@@ -300,6 +300,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
   const int half = lane >> 5, col = lane & 31;
   KeopsTileGeom G;
   G.init(P.rt, P.nx, CHK_QB);
+  if (G.row_first >= G.row_end) return;  // empty entry: tables built on the device round the grid up
   // CHK_NC wavefronts share 32 output rows: wavefront `chunk` of group `grp` contracts k blocks
   // [chunk * CHK_KBC, (chunk + 1) * CHK_KBC) and evaluates values [chunk * CHK_VS, (chunk + 1) * CHK_VS) of each tile
   const int grp = wave / CHK_NC, chunk = wave % CHK_NC;
@@ -786,6 +787,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
   const int half = lane >> 5, col = lane & 31;
   KeopsTileGeom G;
   G.init(P.rt, P.nx, CHK_QB);
+  if (G.row_first >= G.row_end) return;  // empty entry: tables built on the device round the grid up
   const i64 row0 = G.row_first + wave * 32;  // first output row of this wavefront
   const bool wave_live = row0 < G.row_end;   // a wavefront without rows only helps staging the tiles
   i64 q = row0 + col;
@@ -1038,6 +1040,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
   const int half = lane >> 5, col = lane & 31;
   KeopsTileGeom G;
   G.init(P.rt, P.nx, CHK_QB);
+  if (G.row_first >= G.row_end) return;  // empty entry: tables built on the device round the grid up
   const i64 row0 = G.row_first + wave * 32;  // first output row of this wavefront
   const bool wave_live = row0 < G.row_end;   // a wavefront without rows only helps staging the tiles
   i64 q = row0 + col;

@@ -406,6 +406,7 @@ extern "C" __global__ void __launch_bounds__(KEOPS_BLOCK) keops_conv_ranges(cons
   const i64 range_id = P.lookup[3 * (i64)blockIdx.x];
   const i64 start_x = P.lookup[3 * (i64)blockIdx.x + 1];
   const i64 end_x = P.lookup[3 * (i64)blockIdx.x + 2];
+  if (end_x <= start_x) return;  // empty entry: tables built on the device round the grid up
   const i64 start_slice = range_id < 1 ? 0 : P.slices_x[range_id - 1];
   const i64 end_slice = P.slices_x[range_id];
   const bool batched = P.nbatchdims > 0;

@@ -54,6 +54,7 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
   const int half = lane >> 5, col = lane & 31;
   KeopsTileGeom G;
   G.init(P.rt, P.nx, FIN_QB);
+  if (G.row_first >= G.row_end) return;  // empty entry: tables built on the device round the grid up
   const i64 row0 = G.row_first + wave * 32;  // first output row of this wavefront
   const bool wave_live = row0 < G.row_end;   // a wavefront without rows only helps staging the tiles
   i64 q = row0 + col;
@@ -265,6 +266,7 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
   const int half = lane >> 5, col = lane & 31;
   KeopsTileGeom G;
   G.init(P.rt, P.nx, FIN_QB);
+  if (G.row_first >= G.row_end) return;  // empty entry: tables built on the device round the grid up
   const i64 row0 = G.row_first + wave * 32;  // first output row of this wavefront
   const bool wave_live = row0 < G.row_end;   // a wavefront without rows only helps staging the tiles
   i64 q = row0 + col;

@@ -1,7 +1,7 @@
 """HIP graph capture of launches (torch.cuda.graph): after one eager call with the same shapes, which sizes the
 workspaces, a launch records kernels and copies only, so the replayed graph must reproduce the eager result bit for
 bit on new input values.  Launches that have to wait for the device adapt (the KNN scheme takes its adaptive
-schedule) or refuse with a clear error (block-sparse ranges)."""
+schedule); block-sparse ranges are validated on the host once and then served without a read-back."""
 import pytest
 import torch
 
@@ -85,22 +85,90 @@ def test_knn_scheme_takes_its_adaptive_schedule_under_capture():
     assert _scheme_of_last_module() == "knn"
 
 
-def test_block_sparse_ranges_refuse_capture_with_a_clear_error():
+def _block_ranges(edges_i, edges_j, keep):
+    """ranges tuple (device int64 tensors) of a block-sparse pattern: keep[a] lists the column blocks of row block a."""
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device="cuda")
+    ranges_i = [[edges_i[a], edges_i[a + 1]] for a in range(len(edges_i) - 1)]
+    ranges_j = [[edges_j[b], edges_j[b + 1]] for b in range(len(edges_j) - 1)]
+    red_j, slices_i = [], []
+    for a in range(len(ranges_i)):
+        red_j += [ranges_j[b] for b in keep[a]]
+        slices_i.append(len(red_j))
+    red_i, slices_j = [], []
+    for b in range(len(ranges_j)):
+        red_i += [ranges_i[a] for a in range(len(ranges_i)) if b in keep[a]]
+        slices_j.append(len(red_i))
+    return (i64(ranges_i), i64(slices_i), i64(red_j), i64(ranges_j), i64(slices_j), i64(red_i))
+
+
+def _masked_dense(x, y, b, ranges):
+    ri, sl, rj = (t.cpu().tolist() for t in ranges[:3])
+    out = torch.zeros(x.shape[0], b.shape[1], dtype=torch.float64, device="cuda")
+    for a, (s, e) in enumerate(ri):
+        for k in range(0 if a == 0 else sl[a - 1], sl[a]):
+            js, je = rj[k]
+            K = torch.exp(-torch.cdist(x[s:e].double(), y[js:je].double()) ** 2)
+            out[s:e] += K @ b[js:je].double()
+    return out
+
+
+def test_block_sparse_ranges_under_graph_capture():
+    """The first launch with a set of range tensors reads them back and validates them (it refuses capture, with a
+    message that says so); from the second on the workgroup table is built on the device, so the launch records into
+    a graph, replays follow new input values and in-place changes of the ranges, and indices that have gone out of
+    bounds are clamped and flagged instead of faulting."""
+    from keops_amd import keops_io
     from keops_amd.torch import Genred
 
-    x, y, b = (torch.randn(n, d, device="cuda") for n, d in ((1000, 3), (1200, 3), (1200, 1)))
-    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device="cuda")
-    ranges = (i64([[0, 500], [500, 1000]]), i64([1, 2]), i64([[0, 600], [600, 1200]]),
-              i64([[0, 600], [600, 1200]]), i64([1, 2]), i64([[0, 500], [500, 1000]]))
-    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(1)"], reduction_op="Sum", axis=1)
-    ref = conv(x, y, b, ranges=ranges)
-    torch.cuda.synchronize()
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    x, y, b = (torch.randn(n, d, device="cuda", generator=gen) for n, d in ((3000, 3), (3500, 3), (3500, 2)))
+    ranges = _block_ranges([0, 700, 1500, 1501, 3000], [0, 900, 2000, 3500], [[0, 1], [1], [0, 2], [2]])
+    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)"], reduction_op="Sum", axis=1)
+
+    fresh = tuple(t.clone() for t in ranges)          # tensors the module has not seen: host path only
     graph = torch.cuda.CUDAGraph()
     with pytest.raises(RuntimeError, match="cannot be captured"):
         with torch.cuda.graph(graph):
-            conv(x, y, b, ranges=ranges)
+            conv(x, y, b, ranges=fresh)
     torch.cuda.synchronize()
-    assert torch.equal(conv(x, y, b, ranges=ranges), ref)             # the stream is usable again
+
+    ref = conv(x, y, b, ranges=ranges)                 # host path: read back, validated
+    err = (ref.double() - _masked_dense(x, y, b, ranges)).norm() / _masked_dense(x, y, b, ranges).norm()
+    assert float(err) < 1e-5
+    again = conv(x, y, b, ranges=ranges)               # device path
+    assert torch.equal(again, ref)
+    module = keops_io.last_loader.module
+    assert module.ranges_status() == 0
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        conv(x, y, b, ranges=ranges)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = conv(x, y, b, ranges=ranges)
+    for k in range(3):
+        x.copy_(torch.randn(x.shape, device="cuda", generator=gen))
+        b.copy_(torch.randn(b.shape, device="cuda", generator=gen))
+        if k == 2:                                      # the pattern changes in place: row block 0 loses column block 1
+            ranges[2][1] = torch.tensor([0, 0], device="cuda")
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = _masked_dense(x, y, b, ranges)
+        assert float((got.double() - want).norm() / want.norm()) < 1e-5
+        assert torch.equal(conv(x, y, b, ranges=ranges), got)      # eager work between the replays
+    # an index beyond the reduced axis: clamped (the kernels sweep the ranges unchecked) and flagged
+    ranges[2][2] = torch.tensor([2000, 10 ** 9], device="cuda")
+    clamped = conv(x, y, b, ranges=ranges)
+    torch.cuda.synchronize()
+    assert module.ranges_status() & 1
+    ranges[2][2] = torch.tensor([2000, 3500], device="cuda")
+    assert torch.equal(conv(x, y, b, ranges=ranges), clamped)
+    assert module.ranges_status() == 0
 
 
 def test_captured_graph_survives_later_eager_calls_at_other_shapes():
