@@ -71,6 +71,11 @@ void keops_hip_module_destroy(void* module);
  *                     nothing else runs.  A module is still required (it gives the element size); the engine
  *                     compiles none for a zero formula, so keops_amd/keops_io.py fills out itself and never
  *                     passes 1 here
+ *   use_half          1: out and the arguments are arrays of IEEE half precision (device pointers, plain row-major
+ *                     layout -- not the half2 interleaving that pykeops/pykeops/torch/half2_convert.py produces for
+ *                     the CUDA kernels); the module must be compiled for float: the library converts the arguments
+ *                     into a staging buffer owned by the module, computes in float32 and rounds the result to half
+ *                     once (the reference computes in half2 arithmetic)
  *   tag1D2D           0: one pass over the reduced axis; 1: force the column-slab (2D) scheme
  *   dimred, dimout    accumulator and output dimensions per row
  *   block_size        upper bound for the workgroup size (0 = module default)
@@ -101,7 +106,7 @@ void keops_hip_module_destroy(void* module);
  */
 #define KEOPS_HIP_NOT_CERTIFIED (-7)
 int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, int64_t ny, int tagI,
-                     int tagZero, int tag1D2D, int64_t dimred, int64_t block_size, int use_chunk_mode,
+                     int tagZero, int use_half, int tag1D2D, int64_t dimred, int64_t block_size, int use_chunk_mode,
                      const int* indsi, int ni, const int* indsj, int nj, const int* indsp, int np,
                      int64_t dimout, const int64_t* dimsx, const int64_t* dimsy, const int64_t* dimsp,
                      int64_t* const* ranges, const int64_t* shapeout, int nshapeout, void* out,

@@ -45,7 +45,7 @@ def lib():
         L.keops_hip_compile.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int]
         I64, P = ctypes.c_int64, ctypes.c_void_p
         L.keops_hip_launch.argtypes = [
-            P, ctypes.c_int, I64, I64, I64, ctypes.c_int, ctypes.c_int, ctypes.c_int, I64, I64, ctypes.c_int,
+            P, ctypes.c_int, I64, I64, I64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, I64, I64, ctypes.c_int,
             P, ctypes.c_int, P, ctypes.c_int, P, ctypes.c_int, I64, P, P, P, P, P, ctypes.c_int, P, P, P, P, P,
             ctypes.c_int,
         ]
@@ -144,8 +144,6 @@ class Module:
                  out_ptr, args_ptr, argshapes, stream=0, sync=False):
         """Same positional arguments as KeOps_module_python::operator() (pykeops_nvrtc.cpp:17-23),
         plus the stream to launch on and whether to wait for completion."""
-        if use_half:
-            raise KeOpsHipError("float16 data is not supported")
         ci, cj, cp = _iarr(ctypes.c_int, indsi), _iarr(ctypes.c_int, indsj), _iarr(ctypes.c_int, indsp)
         dx, dy, dp = _iarr(ctypes.c_int64, dimsx), _iarr(ctypes.c_int64, dimsy), _iarr(ctypes.c_int64, dimsp)
         rp = (ctypes.c_void_p * 7)(*ranges_ptr)
@@ -155,7 +153,7 @@ class Module:
         sh = _iarr(ctypes.c_int64, flat)
         nd = _iarr(ctypes.c_int, [len(shp) for shp in argshapes])
         rc = lib().keops_hip_launch(
-            self.handle, int(tagHostDevice), int(dimy), int(nx), int(ny), int(tagI), int(tagZero), int(tag1D2D),
+            self.handle, int(tagHostDevice), int(dimy), int(nx), int(ny), int(tagI), int(tagZero), int(bool(use_half)), int(tag1D2D),
             int(dimred), int(block_size), int(use_chunk_mode), ci, len(indsi), cj, len(indsj), cp, len(indsp),
             int(dimout), dx, dy, dp, rp, so, len(shapeout), ctypes.c_void_p(out_ptr), ap, sh, nd,
             ctypes.c_void_p(stream), int(bool(sync)),

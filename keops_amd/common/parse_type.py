@@ -100,5 +100,8 @@ def parse_dtype_acc(dtype_acc, dtype):
     if dtype == "float64" and dtype_acc != "float64":
         raise ValueError("[KeOps] invalid parameter dtype_acc : should be 'float64' when dtype is 'float64'")
     if dtype == "float16":
-        raise ValueError("[KeOps] float16 data is not supported by the HIP backend")
+        # half-precision data is computed and accumulated in float32 by the HIP backend, whatever is asked for
+        if dtype_acc not in ("float16", "float32"):
+            raise ValueError("[KeOps] invalid parameter dtype_acc : should be either 'float16' or 'float32' when dtype is 'float16'")
+        return "float"
     return dict(float32="float", float64="double")[dtype_acc]

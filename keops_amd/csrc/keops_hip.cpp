@@ -1104,7 +1104,7 @@ int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
 
 extern "C" {
 
-int keops_hip_abi_version(void) { return 2; }
+int keops_hip_abi_version(void) { return 3; }
 
 const char* keops_hip_templates_digest(void) { return keops_templates_digest; }
 
@@ -1540,8 +1540,56 @@ static int launch_from_host(Module& m, int64_t nx, int64_t ny, int tagI, int tag
   return 0;
 }
 
+// Half-precision data (use_half = 1; KeOps_module<TYPE>::launch_kernel's use_half, keops_nvrtc.cpp:390-400, and
+// pykeops/pykeops/torch/half2_convert.py): out and the arguments are plain row-major arrays of IEEE half on the
+// device.  The kernels of this library compute in float32: the arguments are converted into the module's staging
+// buffer, the float32 module runs on those copies and the result is rounded to half once, at the end (the reference
+// computes in half2 arithmetic; results here are at least as accurate).
+static int launch_half(Module& m, int64_t nx, int64_t ny, int tagI, int tagZero, int tag1D2D, int64_t dimred,
+                       const int* indsi, int ni, const int* indsj, int nj, const int* indsp, int np,
+                       int64_t dimout, const int64_t* dimsx, const int64_t* dimsy, const int64_t* dimsp,
+                       int64_t* const* ranges, const int64_t* shapeout, int nshapeout, void* out,
+                       void* const* args, const int64_t* argshapes_flat, const int* argndims, hipStream_t stream, int sync) {
+  if (m.sizeof_t != 4) return fail(-1, "use_half needs a module compiled for float (half data is computed in float32)");
+  int64_t sizeout = 1;
+  for (int k = 0; k < nshapeout; k++) sizeout *= shapeout[k];
+  if (sizeout < 0) return fail(-1, "negative output shape");
+  std::vector<int64_t> arg_n((size_t)m.nargs);
+  std::vector<size_t> arg_off((size_t)m.nargs);
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+  const int64_t* p = argshapes_flat;
+  for (int k = 0; k < m.nargs; k++) {
+    int64_t n = 1;
+    for (int d = 0; d < argndims[k]; d++) {
+      if (p[d] < 0) return fail(-1, "negative dimension in the shape of argument " + std::to_string(k));
+      n *= p[d];
+    }
+    p += argndims[k];
+    arg_n[k] = n;
+    arg_off[k] = take((size_t)n * sizeof(float));
+  }
+  const size_t out_off = take((size_t)sizeout * sizeof(float));
+  if (stream_is_capturing(stream)) m.staging.frozen = true;
+  if (int rc = m.staging.reserve(std::max<size_t>(off, 256))) return rc;
+  char* base = (char*)m.staging.ptr;
+  std::vector<void*> fargs((size_t)std::max(1, m.nargs));
+  for (int k = 0; k < m.nargs; k++) {
+    fargs[k] = base + arg_off[k];
+    if (int e = keops_static_convert_half(fargs[k], args[k], arg_n[k], 1, stream))
+      return fail(e, std::string("half -> float conversion failed: ") + hipGetErrorString((hipError_t)e));
+  }
+  if (int rc = launch_on_device(m, nx, ny, tagI, tagZero, tag1D2D, dimred, indsi, ni, indsj, nj, indsp, np, dimout, dimsx, dimsy,
+                                dimsp, ranges, shapeout, nshapeout, base + out_off, fargs.data(), argshapes_flat, argndims, stream, 0))
+    return rc;
+  if (int e = keops_static_convert_half(out, base + out_off, sizeout, 0, stream))
+    return fail(e, std::string("float -> half conversion failed: ") + hipGetErrorString((hipError_t)e));
+  if (sync) HIP_TRY(hipStreamSynchronize(stream));
+  return 0;
+}
+
 int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, int64_t ny, int tagI,
-                     int tagZero, int tag1D2D, int64_t dimred, int64_t block_size, int use_chunk_mode,
+                     int tagZero, int use_half, int tag1D2D, int64_t dimred, int64_t block_size, int use_chunk_mode,
                      const int* indsi, int ni, const int* indsj, int nj, const int* indsp, int np,
                      int64_t dimout, const int64_t* dimsx, const int64_t* dimsy, const int64_t* dimsp,
                      int64_t* const* ranges, const int64_t* shapeout, int nshapeout, void* out,
@@ -1554,6 +1602,12 @@ int keops_hip_launch(void* module, int tagHostDevice, int64_t dimY, int64_t nx, 
   if (tagHostDevice != 0 && tagHostDevice != 1) return fail(-1, "tagHostDevice must be 0 (host pointers) or 1 (device pointers)");
   hipStream_t stream = (hipStream_t)hip_stream;
   HIP_TRY(hipSetDevice(m.device));
+  if (use_half != 0 && use_half != 1) return fail(-1, "use_half must be 0 or 1");
+  if (use_half) {
+    if (tagHostDevice == 0) return fail(-1, "use_half takes device pointers (tagHostDevice = 1)");
+    return launch_half(m, nx, ny, tagI, tagZero, tag1D2D, dimred, indsi, ni, indsj, nj, indsp, np, dimout, dimsx, dimsy, dimsp,
+                       ranges, shapeout, nshapeout, out, args, argshapes_flat, argndims, stream, sync);
+  }
   if (tagHostDevice == 0)
     return launch_from_host(m, nx, ny, tagI, tagZero, tag1D2D, dimred, indsi, ni, indsj, nj, indsp, np, dimout, dimsx, dimsy, dimsp,
                             ranges, shapeout, nshapeout, out, args, argshapes_flat, argndims, stream);

@@ -9,6 +9,8 @@
 
 int keops_static_scratch(int device, void** ptr, size_t* bytes);
 int keops_static_fill_zero(void* dst, size_t bytes, void* stream);
+// n elements: IEEE half -> float (to_float != 0) or float -> half (round to nearest even)
+int keops_static_convert_half(void* dst, const void* src, long long n, int to_float, void* stream);
 int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* out, void* stream, double* instr_per_wave);
 
 // Lookup table of a block-sparse launch built on the device (no read-back of the ranges): see keops_static.hip.

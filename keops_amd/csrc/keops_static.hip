@@ -1,5 +1,6 @@
 // Device code that is compiled into libkeops_hip.so itself (everything else is JIT-compiled per formula):
 //   * the static scratch buffer of the entry point that allocates nothing (keops_hip_launch_noalloc),
+//   * half <-> float conversion kernels (use_half launches compute in float32),
 //   * a fill kernel (zero formulas: a kernel instead of hipMemsetAsync, which must stay out of captured graphs),
 //   * the kernels that build the lookup table of a block-sparse launch from the caller's ranges on the device,
 //   * loop-only calibration kernels for the vector ALU and the matrix cores (keops_hip_calibrate): they measure
@@ -53,6 +54,27 @@ int keops_static_fill_zero(void* dst, size_t bytes, void* stream) {
   const long long n = (long long)(bytes / 4);
   if (n == 0) return 0;
   hipLaunchKernelGGL(keops_fill_zero_u32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, (uint32_t*)dst, n);
+  return (int)hipGetLastError();
+}
+
+// ---- half precision <-> float -------------------------------------------------------------------------------------
+
+static __global__ void __launch_bounds__(256) keops_half_to_float(float* dst, const _Float16* src, long long n) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = (float)src[i];
+}
+static __global__ void __launch_bounds__(256) keops_float_to_half(_Float16* dst, const float* src, long long n) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = (_Float16)src[i];
+}
+
+int keops_static_convert_half(void* dst, const void* src, long long n, int to_float, void* stream) {
+  if (n <= 0) return 0;
+  const dim3 grid((unsigned)((n + 255) / 256));
+  if (to_float)
+    hipLaunchKernelGGL(keops_half_to_float, grid, dim3(256), 0, (hipStream_t)stream, (float*)dst, (const _Float16*)src, n);
+  else
+    hipLaunchKernelGGL(keops_float_to_half, grid, dim3(256), 0, (hipStream_t)stream, (_Float16*)dst, (const float*)src, n);
   return (int)hipGetLastError();
 }
 

@@ -36,9 +36,12 @@ class LoadKeOps_hip:
         p.aliases_old, p.aliases = list(aliases), aliases_new
         p.red_formula_string = formula
         p.dtype = dtype
-        p.c_dtype = dict(float32="float", float64="double").get(dtype)
+        # half-precision data is computed in float32: the library converts the arguments and rounds the result once
+        # (use_half of keops_hip_launch; pykeops/pykeops/torch/half2_convert.py computes in half2 arithmetic)
+        self.half = dtype == "float16"
+        p.c_dtype = dict(float16="float", float32="float", float64="double").get(dtype)
         if p.c_dtype is None:
-            raise ValueError("not implemented")
+            raise ValueError(f"[KeOps] data of type {dtype} is not supported (float16, float32, float64 are)")
         p.c_dtype_acc = parse_dtype_acc(optional_flags["dtype_acc"], dtype)
         p.sum_scheme = optional_flags["sum_scheme"]
         p.enable_chunks = optional_flags["enable_chunks"]
@@ -58,8 +61,10 @@ class LoadKeOps_hip:
             plan, tagI = self.plan, red.tagI
             D = plan["row"].dim
             width = 64 if D > 128 else 128
+            sub_flags = dict(optional_flags, dtype_acc="auto") if self.half else optional_flags
             sub = lambda f, extra: LoadKeOps_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, f,
-                                                 list(aliases) + extra, nargs + len(extra), dtype, lang, optional_flags,
+                                                 list(aliases) + extra, nargs + len(extra),
+                                                 "float32" if self.half else dtype, lang, sub_flags,
                                                  nx=nx, batch_loop=batch_loop, pairs=pairs)
             self.sub_slices, self.ones_column = [], False
             if plan["c"]:
@@ -134,6 +139,14 @@ class LoadKeOps_hip:
 
     def genred_pytorch(self, device_args, ranges, nx, ny, nbatchdims, out, *args):
         if self.plan is not None:
+            if self.half:
+                # several float32 launches combined with torch operations: the conversions happen here
+                res = self._row_col_product(device_args, ranges, nx, ny, nbatchdims, None, *[a.float() for a in args]).half()
+                if out is None:
+                    return res
+                if tuple(out.shape) != tuple(res.shape) or not out.is_contiguous():
+                    raise ValueError(f"[KeOps] 'out' must be a contiguous tensor of shape {tuple(res.shape)}")
+                return out.copy_(res)
             return self._row_col_product(device_args, ranges, nx, ny, nbatchdims, out, *args)
         p = self.params
         if not ranges:
@@ -162,7 +175,7 @@ class LoadKeOps_hip:
         stream = torch.cuda.current_stream(dev).cuda_stream
         try:
             self.module(
-                p.tagHostDevice, p.dimy, nx, ny, p.tagI, p.tagZero, p.use_half, p.tag1D2D, p.dimred, p.cuda_block_size,
+                p.tagHostDevice, p.dimy, nx, ny, p.tagI, p.tagZero, int(self.half), p.tag1D2D, p.dimred, p.cuda_block_size,
                 p.use_chunk_mode, p.indsi, p.indsj, p.indsp, p.dim, p.dimsx, p.dimsy, p.dimsp, ranges_ptr,
                 tuple(out.shape), int(out.data_ptr()), args_ptr, argshapes, stream=stream, sync=False,
             )

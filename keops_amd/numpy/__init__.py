@@ -23,8 +23,8 @@ def _to_device(args, dev):
     out = []
     for a in args:
         a = np.ascontiguousarray(a)
-        if a.dtype not in (np.float32, np.float64):
-            raise ValueError("[KeOps] only float32 and float64 arrays are supported")
+        if a.dtype not in (np.float16, np.float32, np.float64):
+            raise ValueError("[KeOps] only float16, float32 and float64 arrays are supported")
         out.append(torch.from_numpy(a).to(dev))
     return out
 
@@ -54,8 +54,8 @@ class Genred:
         host = []
         for a in args:
             a = np.ascontiguousarray(a)
-            if a.dtype not in (np.float32, np.float64):
-                raise ValueError("[KeOps] only float32 and float64 arrays are supported")
+            if a.dtype not in (np.float16, np.float32, np.float64):
+                raise ValueError("[KeOps] only float16, float32 and float64 arrays are supported")
             host.append(torch.from_numpy(a))
         if ranges is not None:
             ranges = tuple(torch.from_numpy(np.ascontiguousarray(r).astype(np.int64)) for r in ranges)
@@ -134,8 +134,8 @@ class LazyTensor(_TorchLazyTensor):
 
     def __init__(self, x=None, axis=None):
         if isinstance(x, np.ndarray):
-            if x.dtype not in (np.float32, np.float64):
-                raise ValueError("[KeOps] only float32 and float64 arrays are supported")
+            if x.dtype not in (np.float16, np.float32, np.float64):
+                raise ValueError("[KeOps] only float16, float32 and float64 arrays are supported")
             x = torch.from_numpy(np.ascontiguousarray(x)).to(_device(-1))
         elif isinstance(x, (np.floating, np.integer)):
             x = x.item()

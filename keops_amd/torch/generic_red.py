@@ -86,9 +86,10 @@ class GenredAutograd_base:
             if not torch.cuda.is_available():
                 raise ValueError("[KeOps] the HIP backend needs a GPU: none is visible to torch")
             myconv = binder_for(0)
-            if myconv.plan is not None:
+            if myconv.plan is not None or params.dtype == "float16":
                 # ... except for reductions that the binding layer evaluates as several launches combined with
-                # torch operations on the device: those are staged here
+                # torch operations on the device, and for half-precision data (use_half takes device pointers):
+                # those are staged here
                 dev = torch.device("cuda", device_id)
                 args = tuple(a.to(dev) for a in args)
                 if params.ranges:

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(binder.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert binder.lib().keops_hip_abi_version() == 2
+    assert binder.lib().keops_hip_abi_version() == 3
     assert re.fullmatch(r"[0-9a-f]{64}", binder.templates_digest())
 
 
