@@ -38,7 +38,7 @@ MEASURED_TRAFFIC_BYTES = {
     # profiles/keops_knn_filter__knn_d64.md: dominant kernel keops_knn_filter
     "knn_d64": int(2 * (391283 * 2.0 + 43486) * 1024),
     # profiles/keops_chk_final__laplace_d256.md
-    "laplace_d256": int((5070320 * 2.0 + 666150) * 1024),
+    "laplace_d256": int((5045781 * 2.0 + 672429) * 1024),
     # profiles/keops_chk_softmax__softmax_d64.md
     "softmax_d64": int((204925 * 2.0 + 33804) * 1024),
     # profiles/keops_fin_main3__gauss_dv256.md
