@@ -38,6 +38,11 @@ chunk_min_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MIN_DIM", 24))    # smallest
 # norms), the order of the rounding of the reference's own float32 sum; 1/8 below 32 components, where random pairs
 # come that close often enough for the recomputation to cost more than it is worth (+50 % at D = 24)
 chunk_near = os.environ.get("KEOPS_AMD_CHUNK_NEAR", "auto")
+# float64 contractions on the float64 matrix instruction (csrc/kernels/keops_chunk_f64.h)
+chunk64 = os.environ.get("KEOPS_AMD_CHUNK64", "1") != "0"
+chunk64_min_dim = int(os.environ.get("KEOPS_AMD_CHUNK64_MIN_DIM", 32))
+chunk64_max_dim = 256          # the operands of 16 output rows fill 128 registers of a wavefront
+chunk64_min_rows = int(os.environ.get("KEOPS_AMD_CHUNK64_MIN_ROWS", 4096))
 chunk_max_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MAX_DIM", 1024))  # largest contraction served by the matrix-core chunked scheme
 
 # exponents of low-dimensional Gaussian kernel sums on the matrix cores (csrc/kernels/keops_radial_mfma.h)

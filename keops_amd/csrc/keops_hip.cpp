@@ -1035,6 +1035,63 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   return 0;
 }
 
+// ---- float64 matrix-core chunked scheme (kernels/keops_chunk_f64.h) --------------------------------
+
+// must match struct C64Params of kernels/keops_chunk_f64.h (argument pointers follow)
+struct C64Header {
+  int64_t nx, ny;
+  void* xs;
+  void* ys;
+  void* xn;
+  void* yn;
+  void* colsum;
+  void* colpart;
+  void* out;
+  int64_t nxs, nys;
+  RangeHeader rt;
+};
+
+int launch_chunk64(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, hipStream_t stream, const RangeLaunch* rg,
+                   int64_t nxs, int64_t nys) {
+  const int64_t D = m.meta_int("chk_d", 0), DP = m.meta_int("chk_dpad", 0), QB = m.meta_int("chk_qb", 128);
+  const int mode = m.meta_int("chk_mode", 0);
+  if (D <= 0 || DP <= 0 || DP % 8 != 0) return fail(-1, "corrupt chunk module metadata");
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(256, nys / 64));
+  const size_t o_colsum = take((size_t)DP * 8), o_colpart = take((size_t)nparts * DP * 8);
+  const size_t o_xs = take((size_t)nxs * DP * 8), o_ys = take((size_t)nys * DP * 8);
+  const size_t o_xn = take((size_t)nxs * 8), o_yn = take((size_t)nys * 8);
+  if (int rc = m.partial.reserve(off)) return rc;
+  char* ws = (char*)m.partial.ptr;
+  const int64_t row_blocks = rg ? rg->tables.nblocks : (nx + QB - 1) / QB;
+  std::vector<char> buf(sizeof(C64Header) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 32);
+  C64Header h{};
+  h.nx = nx; h.ny = ny; h.xs = ws + o_xs; h.ys = ws + o_ys; h.xn = ws + o_xn; h.yn = ws + o_yn; h.colsum = ws + o_colsum;
+  h.colpart = ws + o_colpart; h.out = out; h.nxs = nxs; h.nys = nys;
+  if (rg) h.rt = rg->header(m.nargs);
+  std::memcpy(buf.data(), &h, sizeof(h));
+  for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
+  const size_t psize = sizeof(C64Header) + sizeof(void*) * (size_t)std::max(1, m.nargs);
+  int32_t which = 0;
+  auto with_which = [&](int w) { which = w; std::memcpy(buf.data() + psize, &which, 4); return psize + 4; };
+  if (mode == 0) {
+    if (int rc = launch_raw(m, "keops_c64_colsum", (unsigned)nparts, 1, 256, buf.data(), psize, stream)) return rc;
+    const size_t szp = with_which(nparts);
+    if (int rc = launch_raw(m, "keops_c64_colsum_final", 1, 1, 256, buf.data(), szp, stream)) return rc;
+  }
+  size_t sz = with_which(0);
+  if (int rc = launch_raw(m, "keops_c64_prep", (unsigned)((nxs * 8 + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  sz = with_which(1);
+  if (int rc = launch_raw(m, "keops_c64_prep", (unsigned)((nys * 8 + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  if (rg && rg->user_ranges)
+    if (int rc = launch_raw(m, "keops_c64_fill_neutral", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), psize, stream)) return rc;
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
+  if (int rc = launch_raw(m, "keops_c64_main", (unsigned)row_blocks, 1, (unsigned)m.block, buf.data(), psize, stream)) return rc;
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
+  return 0;
+}
+
 // ---- matrix-core final-product scheme (kernels/keops_final_mfma.h) ----------------------------------
 
 // must match struct FinParams of kernels/keops_final_mfma.h (argument pointers follow)
@@ -1361,7 +1418,7 @@ static int launch_on_device(Module& m, int64_t nx, int64_t ny, int tagI, int tag
       if (rc) return rc;
       if (timing) HIP_TRY(hipEventRecord(m.ev1, stream));
     }
-  } else if (m.scheme == "final" || m.scheme == "chunk") {
+  } else if (m.scheme == "final" || m.scheme == "chunk" || m.scheme == "chunk64") {
     const bool built_for_ranges = m.meta_int("ranges", 0) != 0;
     if (use_ranges != built_for_ranges)
       return fail(-1, built_for_ranges ? "this module was built for block-sparse or batched reductions"
@@ -1389,7 +1446,9 @@ static int launch_on_device(Module& m, int64_t nx, int64_t ny, int tagI, int tag
       if (xarg < 0 || yarg < 0 || xarg >= m.nargs || yarg >= m.nargs) return fail(-1, "corrupt chunk module metadata");
       const int64_t nxs = nb > 0 ? arg_rows(xarg, tagI == 0 ? S.M : S.N) : rows_total;
       const int64_t nys = nb > 0 ? arg_rows(yarg, tagI == 0 ? S.N : S.M) : cols_total;
-      if (int rc = launch_chunk(m, rows_total, cols_total, out, args, tag1D2D, stream, use_ranges ? &rg : nullptr, nxs, nys))
+      if (m.scheme == "chunk64") {
+        if (int rc = launch_chunk64(m, rows_total, cols_total, out, args, stream, use_ranges ? &rg : nullptr, nxs, nys)) return rc;
+      } else if (int rc = launch_chunk(m, rows_total, cols_total, out, args, tag1D2D, stream, use_ranges ? &rg : nullptr, nxs, nys))
         return rc;
     }
   } else if (!use_ranges) {

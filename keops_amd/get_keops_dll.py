@@ -417,7 +417,7 @@ def generate_knn_highdim_plugin(red, match, nargs):
     return head + "\n" + body.replace(marker, marker + defs, 1), meta
 
 
-def match_chunk(red, dtype, map_reduce_id, use_fast_math):
+def match_chunk(red, dtype, map_reduce_id, use_fast_math, want="float"):
     """(mode, node, row variable, column variable) when the formula of a Sum / log-sum-exp reduction
     contains exactly one high-dimensional contraction SqDist(x_i, y_j) (mode 0) or <x_i, y_j> (mode 1)
     between plain variables of dimension config.chunk_min_dim..config.chunk_max_dim (24..1024) that appear nowhere else in the formula (the
@@ -426,8 +426,9 @@ def match_chunk(red, dtype, map_reduce_id, use_fast_math):
     from .formulas import ops as O
     from .formulas.reductions import KIND_LSE, KIND_SUM
 
-    if red.kind not in (KIND_SUM, KIND_LSE) or dtype != "float" or not use_fast_math:
+    if red.kind not in (KIND_SUM, KIND_LSE) or dtype != want or not use_fast_math:
         return None
+    dmin, dmax = (config.chunk_min_dim, config.chunk_max_dim) if want == "float" else (config.chunk64_min_dim, config.chunk64_max_dim)
     found = []
     for node in red.formula.walk():
         mode = pair = None
@@ -438,7 +439,7 @@ def match_chunk(red, dtype, map_reduce_id, use_fast_math):
         if mode is None:
             continue
         a, b = pair
-        if isinstance(a, O.Var) and isinstance(b, O.Var) and a.dim == b.dim and config.chunk_min_dim <= a.dim <= config.chunk_max_dim and {a.cat, b.cat} == {0, 1}:
+        if isinstance(a, O.Var) and isinstance(b, O.Var) and a.dim == b.dim and dmin <= a.dim <= dmax and {a.cat, b.cat} == {0, 1}:
             if node not in [f[1] for f in found]:
                 found.append((mode, node, a, b))
     if len(found) != 1:
@@ -605,6 +606,63 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
     src += lines + [f"    fout[{k}] = {e};" for k, e in enumerate(exprs)]
     src.append("  }\n};")
     src.append('#include "keops_chunk_mfma.h"')
+    return "\n".join(src) + "\n", meta
+
+
+def generate_chunk64_plugin(red, match, sum_scheme, nargs, irregular=False):
+    """Module source for the float64 matrix-core chunked scheme (kernels/keops_chunk_f64.h): the contraction on
+    v_mfma_f64_16x16x4_f64, the post-chunk formula in double precision on the vector ALU; ``irregular``: the
+    block-sparse / batched variant."""
+    from .formulas import ops as O
+
+    mode, node, xvar, yvar = match
+    svar = O.Var(1 << 30, 1, 3)
+    post = red.formula.replace(node, svar)
+
+    class _Post:  # what VarLayout needs: the post-chunk formula with the reduction's orientation
+        formula, tagI = post, red.tagI
+
+    layout = VarLayout(_Post)
+    layout.names[(3, svar.ind, 0)] = "s"
+    L = Lir(row_cat=red.tagI, fast_math=True, dtype="double")
+    outs = lower(post, L)
+    lines, exprs = L.emit(outs, layout.names, indent="    ")
+    D = xvar.dim
+    dpad = -(-D // 8) * 8
+    dimy_pad = 0 if layout.dimy == 0 else -(-layout.dimy // 2) * 2
+    waves = 8
+    rb = 2 if dpad <= 128 else 1   # 16-row blocks per wavefront: the operands of 2 x 128 or 1 x 256 components take 128 registers
+    lds = 32 * (dpad * 8 + 16) + 32 * 8 + 32 * max(1, dimy_pad) * 8
+    if max(lds, 8 * 16 * rb * waves * 3 * red.dimred) > config.knn_lds_budget:
+        return None, None
+    ra, rd, ro = VarLayout.table(layout.rowvars)
+    ca, cd, co = VarLayout.table(layout.colvars)
+    pa, pd, po = VarLayout.table(layout.parvars)
+    meta = dict(scheme="chunk64", block=64 * waves, rows=1, tile_j=32, dimred=red.dimred, dimout=red.dim, sizeof_t=8,
+                sizeof_acc=8, nrowvars=len(layout.rowvars) + 1, ncolvars=len(layout.colvars) + 1,
+                nparvars=len(layout.parvars), chk_d=D, chk_dpad=dpad, chk_mode=mode, chk_qb=16 * rb * waves,
+                chk_xarg=xvar.ind, chk_yarg=yvar.ind, ranges=int(irregular), nops=L.count_ops(outs))
+    src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
+           "typedef double T;\ntypedef double TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
+           '#include "keops_common.h"']
+    defs = dict(
+        KEOPS_NARGS=nargs, CHK_D=D, CHK_DPAD=dpad, CHK_MODE=mode, CHK_XARG=xvar.ind, CHK_YARG=yvar.ind, CHK_WAVES=waves, CHK_RB=rb,
+        KEOPS_DIMX=layout.dimx, KEOPS_DIMY=layout.dimy, KEOPS_DIMY_PAD=dimy_pad, KEOPS_DIMP=layout.dimp,
+        KEOPS_DIMFOUT=post.dim, KEOPS_DIMRED=red.dimred, KEOPS_DIMOUT=red.dim, KEOPS_RED_KIND=red.kind,
+        KEOPS_RED_KEEP=red.keep, KEOPS_RED_K=red.K, KEOPS_SUM_SCHEME=SUM_SCHEMES[sum_scheme],
+        KEOPS_NROWVARS=len(layout.rowvars), KEOPS_NCOLVARS=len(layout.colvars), KEOPS_NPARVARS=len(layout.parvars),
+    )
+    src += [f"#define {k} {v}" for k, v in defs.items()]
+    for name, vals in (("row_arg", ra), ("row_dim", rd), ("row_off", ro), ("col_arg", ca), ("col_dim", cd),
+                       ("col_off", co), ("par_arg", pa), ("par_dim", pd), ("par_off", po)):
+        src.append(f"static __device__ constexpr int keops_{name}[] = {_c_list(vals)};")
+    dx, dy, dp = max(1, layout.dimx), max(1, dimy_pad), max(1, layout.dimp)
+    src.append("struct KeopsFormula {")
+    src.append(f"  static __device__ __forceinline__ void eval(const T (&xi)[{dx}], const T (&yj)[{dy}], "
+               f"const T (&p)[{dp}], const T s, T (&fout)[{post.dim}]) {{")
+    src += lines + [f"    fout[{k}] = {e};" for k, e in enumerate(exprs)]
+    src.append("  }\n};")
+    src.append('#include "keops_chunk_f64.h"')
     return "\n".join(src) + "\n", meta
 
 
@@ -953,6 +1011,11 @@ def get_keops_dll(
         knn = match_knn_sqdist(red_k, dtype, map_reduce_id, batch_loop, pairs) if mc else None
         knn_hd = match_knn_highdim(red_k, dtype, map_reduce_id, use_fast_math) if (mc and knn is None) else None
         chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (mc and knn is None) else None
+        # double precision: the contraction on the float64 matrix instruction, when there are enough output rows to
+        # fill the chip without column slabs (the vector-ALU chunked kernel has them)
+        chk64 = None
+        if mc and dtype == "double" and dtypeacc == "double" and config.chunk64 and (rows_hint is None or rows_hint >= config.chunk64_min_rows):
+            chk64 = match_chunk(red, dtype, map_reduce_id, use_fast_math, want="double")
         fin = None
         if enable_finalchunks and mc and knn is None and chk is None:
             fin = match_final(red, dtype, dtypeacc, sum_scheme_string, map_reduce_id, use_fast_math)
@@ -967,6 +1030,9 @@ def get_keops_dll(
             use_chunk_mode = 1 if source is not None else 0
         elif knn_hd is not None:
             source, meta = generate_knn_highdim_plugin(red_k, knn_hd, nargs)
+            use_chunk_mode = 1 if source is not None else 0
+        elif chk64 is not None:
+            source, meta = generate_chunk64_plugin(red, chk64, sum_scheme_string, nargs, irregular=irregular)
             use_chunk_mode = 1 if source is not None else 0
         else:
             source = None
