@@ -256,7 +256,7 @@ __device__ __forceinline__ void chk_fix_near(const ChkParams& P, float (&sv)[NV]
   float m = sv[0];
 #pragma unroll
   for (int u = 1; u < NV; u++) m = __builtin_fminf(m, sv[u]);
-  if (__builtin_expect(!__any(m < near_bound), 1)) return;
+  if (__builtin_expect(!keops_any(m < near_bound), 1)) return;
   unsigned mask = 0u;
 #pragma unroll
   for (int u = 0; u < NV; u++) {
@@ -1212,7 +1212,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
     }
     mx = __builtin_fmaxf(mx, __shfl_xor(mx, 32));  // the partner lane holds the other 16 reduced rows of this output row
     const float m_new = __builtin_fmaxf(__builtin_fmaxf(m_run, mx), -3.0e38f);
-    if (__any(m_new != m_run)) {
+    if (keops_any(m_new != m_run)) {
       // rescale: alpha_i = exp(m_old - m_new) for the rows of this wavefront, moved to the accumulator layout
       const float alpha = keops_red_exp(m_run - m_new);
       l_run *= alpha;

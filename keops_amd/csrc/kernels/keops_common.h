@@ -81,6 +81,10 @@ __device__ __forceinline__ i64 keops_uniform(i64 v) {
   return (i64)(((unsigned long long)hi << 32) | lo);
 }
 
+// true when the predicate holds in some lane: one compare into a scalar register pair and a scalar test (the
+// library's __any goes through an integer per lane: two more vector instructions)
+__device__ __forceinline__ bool keops_any(bool p) { return __builtin_amdgcn_ballot_w64(p) != 0ull; }
+
 struct KeopsRangeTables {
   const i64* lookup;    // [nblocks][3] = (range id, first row, end row)
   const i64* slices_x;  // end slice of every row range

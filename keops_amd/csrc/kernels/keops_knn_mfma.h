@@ -318,7 +318,7 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
       ql = qq[wave][lane];
       u = __int_as_float(qj[wave][lane]);
     }
-    while (__any(pending)) {
+    while (keops_any(pending)) {
       if (pending) {
         const int pos = atomicAdd(const_cast<int*>(&bin_n[ql]), 1);
         if (pos < KNN_BIN) {
@@ -368,7 +368,7 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
     const int slot = wave * QW + ql;
     volatile int* ow = owner;
     bool done = !act;
-    while (__any(!done)) {
+    while (keops_any(!done)) {
       if (!done) ow[slot] = lane;
       __threadfence_block();
       if (!done && ow[slot] == lane) {
@@ -468,7 +468,7 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
 #pragma unroll
         for (int v = 3; v < 15; v += 2) m = __builtin_fminf(__builtin_fminf(m, acc[h][v]), acc[h][v + 1]);
         m = __builtin_fminf(__builtin_fminf(m, acc[h][15]), KNN_FLT_MAX);
-        if (__builtin_expect(!__any(m <= t[h]), 1)) continue;
+        if (__builtin_expect(!keops_any(m <= t[h]), 1)) continue;
         if (MODE == 2) {
           // A threshold estimate may ignore candidates (the bound only gets looser): every lane offers the
           // smallest of its 16 pairs of this sub-tile, which is nearly every candidate once they are sparse.
@@ -736,7 +736,7 @@ extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParam
       d = knn_exact_sqdist(P.xq + (qw0 + ql) * KNN_D, P.yr + (i64)j * KNN_D);
     }
     bool pending = act && knn_better(d, j, kd[ql], kj[ql]);
-    while (__any(pending)) {
+    while (keops_any(pending)) {
       if (pending) {
         const int pos = atomicAdd(&bin_n[ql], 1);
         if (pos < KNN_BIN) {
