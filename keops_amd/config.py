@@ -37,6 +37,8 @@ chunk_min_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MIN_DIM", 24))    # smallest
 # bounds the relative error of every squared distance by 4 * 1.4e-7 (the expansion is off by about 1.4e-7 of the
 # norms), the order of the rounding of the reference's own float32 sum; 1/8 below 32 components, where random pairs
 # come that close often enough for the recomputation to cost more than it is worth (+50 % at D = 24)
+# K-nearest-neighbour reductions with block-sparse ranges on the matrix-core scheme (0: the general-purpose ranges kernel)
+knn_ranges = os.environ.get("KEOPS_AMD_KNN_RANGES", "1") != "0"
 chunk_near = os.environ.get("KEOPS_AMD_CHUNK_NEAR", "auto")
 # float64 contractions on the float64 matrix instruction (csrc/kernels/keops_chunk_f64.h)
 chunk64 = os.environ.get("KEOPS_AMD_CHUNK64", "1") != "0"

@@ -898,6 +898,46 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   return 0;
 }
 
+// Block-sparse launch of a K-nearest-neighbour module built for ranges (KNN_RANGES): pre-pass, neutral lists, the
+// adaptive kernel with one workgroup per patch of a row range, merge (which writes the output layout).
+int launch_knn_ranges(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr, void* out, hipStream_t stream,
+                      const RangeLaunch& rg) {
+  const int64_t D = m.meta_int("knn_d", 0), DP = m.meta_int("knn_dpad", 0), K = m.meta_int("knn_k", 0);
+  if (D <= 0 || DP <= 0 || K <= 0) return fail(-1, "corrupt knn module metadata");
+  if (nr > 2147483647LL) return fail(-1, "too many reference rows for 32-bit indices");
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+  const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(512, nr / 64));
+  const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
+  const int64_t RW = DP * (m.meta_int("knn_split", 0) ? 2 : 1);
+  const size_t o_xh = take((size_t)nq * RW * 2), o_yh = take((size_t)nr * RW * 2);
+  const size_t o_xkey = take((size_t)nq * 4), o_ykey = take((size_t)nr * 4);
+  const size_t o_pd = take((size_t)nq * K * 4), o_pi = take((size_t)nq * K * 4);
+  if (int rc = m.partial.reserve(off)) return rc;
+  char* ws = (char*)m.partial.ptr;
+  struct Packed { KnnHeader h; RangeHeader rt; int64_t extra[2]; } p{};
+  static_assert(sizeof(KnnHeader) % 8 == 0, "the range tables follow the header without padding");
+  KnnHeader& h = p.h;
+  h.nq = nq; h.nr = nr; h.xq = xq; h.yr = yr;
+  h.xh = ws + o_xh; h.yh = ws + o_yh; h.xkey = ws + o_xkey; h.ykey = ws + o_ykey; h.colsum = ws + o_colsum; h.colpart = ws + o_colpart;
+  h.plist_d = ws + o_pd; h.plist_i = ws + o_pi; h.out = out; h.ref_step = 1; h.nslabs = 1; h.slab_len = nr;
+  p.rt = rg.header(m.nargs);
+  const size_t HS = sizeof(KnnHeader) + sizeof(RangeHeader);
+  auto run = [&](const char* k, unsigned gx, unsigned block, size_t size) { return launch_raw(m, k, gx, 1, block, &p, size, stream); };
+  auto with_int = [&](int v) { std::memcpy(p.extra, &v, 4); return HS + 4; };
+  if (int rc = run("keops_knn_colsum", (unsigned)nparts, 256, HS)) return rc;
+  if (int rc = run("keops_knn_colsum_final", 1, 256, with_int(nparts))) return rc;
+  const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
+  if (int rc = run("keops_knn_prep", (unsigned)((nq * lpr + 255) / 256), 256, with_int(0))) return rc;
+  if (int rc = run("keops_knn_prep", (unsigned)((nr * lpr + 255) / 256), 256, with_int(1))) return rc;
+  if (int rc = run("keops_knn_fill_lists", (unsigned)((nq * K + 255) / 256), 256, HS)) return rc;
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
+  if (int rc = run("keops_knn_main", (unsigned)rg.tables.nblocks, (unsigned)m.block, HS)) return rc;
+  if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
+  if (int rc = run("keops_knn_merge", (unsigned)((nq + 255) / 256), 256, HS)) return rc;
+  return 0;
+}
+
 // ---- matrix-core chunked scheme (kernels/keops_chunk_mfma.h) ---------------------------------------
 
 // must match struct ChkParams of kernels/keops_chunk_mfma.h (argument pointers follow)
@@ -1388,10 +1428,21 @@ static int launch_on_device(Module& m, int64_t nx, int64_t ny, int tagI, int tag
   h.slab_len = cols_total;
 
   if (m.scheme == "knn") {
-    if (user_ranges) return fail(-1, "the matrix-core KNN module does not handle block-sparse ranges");
+    const bool built_for_ranges = m.meta_int("ranges", 0) != 0;
+    if (user_ranges != built_for_ranges || (built_for_ranges && nb > 0))
+      return fail(-1, built_for_ranges ? "this K-nearest-neighbour module was built for block-sparse ranges without batch dimensions"
+                                       : "this K-nearest-neighbour module does not handle block-sparse ranges");
     const int rowarg = m.meta_int("rowarg", 0), colarg = m.meta_int("colarg", 1);
     if (rowarg < 0 || colarg < 0 || rowarg >= m.nargs || colarg >= m.nargs) return fail(-1, "corrupt knn module metadata");
-    if (nb == 0) {
+    if (user_ranges) {
+      RangeLaunch rg;
+      rg.nbatchdims = 0;
+      rg.user_ranges = true;
+      if (int rc = prepare_range_tables(m, S, tagI, true, ranges, rows_total, cols_total, m.meta_int("knn_qb", 256), true, rowvars,
+                                        colvars, vP, stream, rg.tables))
+        return rc;
+      if (int rc = launch_knn_ranges(m, rows_total, cols_total, args[rowarg], args[colarg], out, stream, rg)) return rc;
+    } else if (nb == 0) {
       if (int rc = launch_knn(m, rows_total, cols_total, args[rowarg], args[colarg], out, tag1D2D, stream)) return rc;
     } else {
       // batch dimensions: one pass of the dense pipeline per batch on the same stream (indices are relative to

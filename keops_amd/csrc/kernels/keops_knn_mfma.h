@@ -54,6 +54,9 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 knn_bf16x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float knn_f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float knn_f32x4;
 
+#ifndef KNN_RANGES
+#define KNN_RANGES 0                   // 1: module for block-sparse launches (adaptive kernel with a range cursor)
+#endif
 #ifndef KNN_SPLIT
 #define KNN_SPLIT 0
 #endif
@@ -101,6 +104,9 @@ struct KnnParams {
   i64 logcap;
   int stage;             // filter / replay: which slabs this launch covers (knn_stage_slab)
   int pad_;
+#if KNN_RANGES
+  KeopsRangeTables rt;   // block-sparse launches: workgroup table and reduced-index ranges (keops_knn_main only)
+#endif
 };
 
 // Slab handled by workgroup row y of a filter (or replay) launch.  stage 0: all slabs in order;
@@ -268,7 +274,18 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
   constexpr int BLOCK = 64 * WAVES, QW = 32 * QSETS, QB = WAVES * QW;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
-  const i64 qw0 = (i64)blockIdx.x * QB + (i64)wave * QW;  // first query of this wavefront
+#if KNN_RANGES
+  // block-sparse launch (adaptive kernel only): the workgroup serves a patch of one row range and sweeps the
+  // reduced-index ranges of that row range, as GpuReduc1D_ranges.py:127-165 does for any reduction
+  static_assert(MODE == 0, "block-sparse launches run the adaptive kernel");
+  KeopsTileGeom G;
+  G.init(P.rt, P.nq, QB);
+  if (G.row_first >= G.row_end) return;  // empty entry: tables built on the device round the grid up
+  const i64 qbase = G.row_first, qlimit = G.row_end;
+#else
+  const i64 qbase = (i64)blockIdx.x * QB, qlimit = P.nq;
+#endif
+  const i64 qw0 = qbase + (i64)wave * QW;  // first query of this wavefront
   const float inf = __builtin_huge_valf();
 
   // queries of this wavefront as MFMA B operands
@@ -279,8 +296,8 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
 #pragma unroll
   for (int h = 0; h < QSETS; h++) {
     i64 q = qw0 + h * 32 + col;
-    valid[h] = q < P.nq;
-    if (!valid[h]) q = P.nq - 1;
+    valid[h] = q < qlimit;
+    if (!valid[h]) q = qlimit - 1;
 #pragma unroll
     for (int kb = 0; kb < KNN_KB; kb++) {
       bq[h][kb] = *reinterpret_cast<const knn_bf16x8*>(P.xh + q * KNN_RW + kb * 16 + 8 * half);
@@ -393,8 +410,12 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
     }
   };
 
+#if KNN_RANGES
+  i64 jbeg = 0, jend = 0;
+#else
   const i64 jbeg = (i64)slab * P.slab_len;
   const i64 jend = keops_min(P.nr, jbeg + P.slab_len);
+#endif
   // software pipeline: the rows of tile t+1 travel from HBM/L2 to registers while tile t is consumed
   constexpr int CH = KNN_RW / 8;                            // 16-byte chunks per staged row
   constexpr int NPF = (TJ * CH + BLOCK - 1) / BLOCK;    // chunks per thread and tile
@@ -414,6 +435,12 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
   // this lane's operand row and keys inside a sub-tile of 32 staged rows
   const unsigned char* const abase = ys + col * KNN_STRIDE + 16 * half;
   const float* const kbase = ykey_s + 4 * half;
+#if KNN_RANGES
+  G.rewind(P.rt);
+  while (G.next(P.rt, jbeg, jend)) {
+#else
+  {
+#endif
   if (jbeg < jend) prefetch(jbeg);
   for (i64 j0 = jbeg; j0 < jend; j0 += TJ) {
     const int n = (int)keops_min((i64)TJ, jend - j0);
@@ -528,6 +555,7 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
       }
     }
   }
+  }
   if (MODE == 2) {
     // lists of this slab straight from the owners' registers
     drain(qcount);
@@ -554,8 +582,8 @@ __device__ __forceinline__ void knn_sweep(const KnnParams& P, unsigned char* ys,
   // partial lists of this slab
   for (int e = tid; e < QB * KNN_K; e += BLOCK) {
     const int ql = e / KNN_K, l = e - ql * KNN_K;
-    const i64 q = (i64)blockIdx.x * QB + ql;
-    if (q < P.nq) {
+    const i64 q = qbase + ql;
+    if (q < qlimit) {
       const i64 o = ((i64)blockIdx.y * P.nq + q) * KNN_K + l;
       P.plist_d[o] = lv[ql][l];
       P.plist_i[o] = li[ql][l];
@@ -575,6 +603,7 @@ extern "C" __global__ void __launch_bounds__(64 * KNN_WAVES) keops_knn_main(cons
   knn_sweep<0, KNN_WAVES, KNN_QSETS>(P, ys, ykey_s, lv, li, owner, qq, qj);
 }
 
+#if !KNN_RANGES
 // threshold estimate from a subset of the references: K-lists of upper bounds, no memory access per candidate
 extern "C" __global__ void __launch_bounds__(64 * KNN_SWAVES) keops_knn_sample(const KnnParams P) {
   __shared__ __attribute__((aligned(16))) unsigned char ys[KNN_TJ * KNN_STRIDE];
@@ -606,6 +635,8 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_gather_sample(const 
   reinterpret_cast<uint4*>(yh_s)[e] = reinterpret_cast<const uint4*>(P.yh)[row * step * CH + c];
   if (c == 0) ykey_sm[row] = P.ykey[row * step];
 }
+
+#endif  // !KNN_RANGES
 
 // ---- merge of the per-slab lists ----------------------------------------------------------------
 
@@ -640,6 +671,17 @@ __device__ __forceinline__ void knn_merge_lists(const KnnParams& P, i64 q, float
   }
 }
 
+#if KNN_RANGES
+// block-sparse launches: queries that no row range covers (and lists that fewer than K references reach) keep the
+// neutral entries (infinite distance, index 0)
+extern "C" __global__ void __launch_bounds__(256) keops_knn_fill_lists(const KnnParams P) {
+  const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (e >= P.nq * KNN_K) return;
+  P.plist_d[e] = __builtin_huge_valf();
+  P.plist_i[e] = 0;
+}
+#endif
+
 extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParams P) {
   const i64 q = (i64)blockIdx.x * 256 + threadIdx.x;
   if (q >= P.nq) return;
@@ -660,6 +702,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParam
   }
 }
 
+#if !KNN_RANGES
 // Thresholds of a filter pass from K-lists of a subset of the references (any such K-th distance is
 // an upper bound of the final one).  refine = 0: lists of upper bounds U of the sampling pass (slabs
 // 0 .. nslabs-1): K references have an exact float32 distance <= U_K (1 + delta), so every final neighbour has a
@@ -792,3 +835,4 @@ extern "C" __global__ void __launch_bounds__(64) keops_knn_rerank(const KnnParam
     }
   }
 }
+#endif  // !KNN_RANGES

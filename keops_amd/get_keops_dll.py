@@ -147,7 +147,11 @@ def match_knn_sqdist(red, dtype, map_reduce_id, batch_loop=0, pairs=0):
     2**pairs pairs; small problems stay on the general-purpose kernel, whose fixed cost is lower."""
     from .formulas import ops as O
 
+    # batch_loop: 0 none; > 0: few large batches served one at a time (log2 bucket of the pairs per batch);
+    # -1: block-sparse ranges without batch dimensions (the adaptive kernel with a range cursor)
     if red.kind != KIND_KMIN or dtype != "float" or ("_ranges" in map_reduce_id and not batch_loop) or red.K > 64:
+        return None
+    if batch_loop == -1 and not config.knn_ranges:
         return None
     f = red.formula
     if f.name != "Sum" or f.children[0].name != "Square" or f.children[0].children[0].name != "Subtract":
@@ -160,13 +164,15 @@ def match_knn_sqdist(red, dtype, map_reduce_id, batch_loop=0, pairs=0):
     if pairs and (1 << (int(pairs) - 1)) * max(a.dim, 16) < config.knn_min_work:
         # the pre-pass, the warm-up of the adaptive lists and the merge cost about 0.3 ms whatever the size
         return None
-    if "_ranges" in map_reduce_id and (1 << (int(batch_loop) - 1)) * max(a.dim, 8) < config.knn_batch_min_work:
+    if "_ranges" in map_reduce_id and batch_loop > 0 and (1 << (int(batch_loop) - 1)) * max(a.dim, 8) < config.knn_batch_min_work:
         # one pass per batch costs about 0.3 ms of launches: below this the batched general-purpose kernel wins
         return None
     return (a, b) if a.cat == red.tagI else (b, a)
 
 
-def generate_knn_plugin(red, rowvar, colvar, nargs):
+def generate_knn_plugin(red, rowvar, colvar, nargs, block_sparse=False):
+    """Module source for the matrix-core K-nearest-neighbour scheme (kernels/keops_knn_mfma.h); ``block_sparse``: the
+    variant for launches with a ``ranges`` tuple (adaptive kernel only, GpuReduc1D_ranges.py:127-165)."""
     D = rowvar.dim
     dpad = -(-D // 16) * 16
     # low dimensions: neighbours are close compared with the norms, the operands are split as hi + lo
@@ -193,8 +199,10 @@ def generate_knn_plugin(red, rowvar, colvar, nargs):
                 sizeof_acc=4, nrowvars=1, ncolvars=1, nparvars=0, knn_d=D, knn_dpad=dpad, knn_k=red.K,
                 knn_qb=waves * 32 * qsets, knn_fwaves=config.knn_filter_waves, knn_fqsets=config.knn_filter_qsets,
                 knn_sample=config.knn_sample, knn_split=split, knn_ftj=ftj, knn_sqb=swaves * 32 * sqsets, knn_sblock=64 * swaves,
-                rowarg=rowvar.ind, colarg=colvar.ind)
+                rowarg=rowvar.ind, colarg=colvar.ind, ranges=int(block_sparse))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}", "typedef float T;"]
+    if block_sparse:
+        src += ["#define KEOPS_MC_RANGES 1", "#define KNN_RANGES 1"]
     defs = dict(KEOPS_NARGS=nargs, KNN_D=D, KNN_DPAD=dpad, KNN_K=red.K, KEOPS_RED_KEEP=red.keep, KEOPS_DIMOUT=red.dim,
                 KNN_QSETS=qsets, KNN_TJ=tj, KNN_WAVES=waves, KNN_FWAVES=config.knn_filter_waves,
                 KNN_FQSETS=config.knn_filter_qsets, KNN_FTJ=ftj, KNN_SWAVES=swaves, KNN_SQSETS=sqsets, KNN_SPLIT=split)
@@ -1020,7 +1028,7 @@ def get_keops_dll(
         if enable_finalchunks and mc and knn is None and chk is None:
             fin = match_final(red, dtype, dtypeacc, sum_scheme_string, map_reduce_id, use_fast_math)
         if knn is not None:
-            source, meta = generate_knn_plugin(red_k, knn[0], knn[1], nargs)
+            source, meta = generate_knn_plugin(red_k, knn[0], knn[1], nargs, block_sparse=(irregular and batch_loop == -1))
             use_chunk_mode = 3  # matrix-core filter scheme (no counterpart among the reference's chunk modes)
         elif fin is not None:
             source, meta = generate_final_plugin(red, fin, sum_scheme_string, nargs, irregular=irregular)

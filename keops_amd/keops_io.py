@@ -210,7 +210,9 @@ def load_keops_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_requ
 
     rows_hint = nx if (nx is not None and nx < 64 * 256 * config.block_size) else None
     # log2 bucket of the pairs per batch when there are few batches: the engine weighs it against the formula
-    batch_loop = int(batch[1] * batch[2]).bit_length() if (batch and batch[0] <= config.knn_batch_max) else 0
+    batch_loop = int(batch[1] * batch[2]).bit_length() if (batch and 0 < batch[0] <= config.knn_batch_max) else 0
+    if batch and batch[0] == 0:
+        batch_loop = -1  # block-sparse ranges without batch dimensions
     # log2 bucket of the pairs of the call (of each batch), 0: unknown or beyond every threshold of the engine
     pairs = int(nx * ny).bit_length() if (nx is not None and ny is not None) else 0
     if pairs > 40:

@@ -72,6 +72,8 @@ class GenredAutograd_base:
             for d in range(nbatchdims):
                 nbatches *= max(a.shape[d] if a.dim() == nbatchdims + 2 else 1 for a in args)
             batch = (nbatches, params.nx, params.ny)
+        elif nbatchdims == 0 and params.ranges is not None:
+            batch = (0, params.nx, params.ny)  # block-sparse ranges, no batch dimensions
 
         def binder_for(tag_hd):
             return keops_binder["hip"](

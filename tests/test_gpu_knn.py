@@ -206,6 +206,46 @@ def test_batched_knn_one_dense_pass_per_batch(monkeypatch):
         assert np.array_equal(vals[b].cpu().numpy(), np.take_along_axis(d, ref, 1)), b
 
 
+@pytest.mark.parametrize("D,K,op", [(16, 5, "KMin_ArgKMin"), (64, 10, "ArgKMin"), (40, 3, "KMin")])
+def test_knn_with_block_sparse_ranges_bit_exact(D, K, op):
+    """K nearest neighbours restricted by a block-sparse pattern (cluster-to-cluster search): the adaptive matrix-core
+    kernel with a range cursor, bit-identical to the oracle's ranges loop; rows that no range covers and rows whose
+    ranges hold fewer than K references keep the neutral entries."""
+    from keops_amd import keops_io
+
+    rng = np.random.default_rng(D)
+    M, N = 5200, 6100
+    x = rng.random((M, D)).astype(np.float32)
+    y = rng.random((N, D)).astype(np.float32)
+    y[4000] = y[4500]          # ties across two ranges of the same row range: lower index first
+    # four row ranges (rows 1000..1199 uncovered; the last one sees only 2 references, fewer than K)
+    ranges_i = np.array([[0, 1000], [1200, 3000], [3000, 5190], [5190, 5200]], np.int64)
+    slices_i = np.array([2, 3, 6, 7], np.int64)
+    red_j = np.array([[0, 1500], [4000, 6100], [1500, 4000], [0, 700], [700, 1500], [4200, 5000], [6000, 6002]], np.int64)
+    # the other three arrays describe the transposed pattern (not used by a reduction over j)
+    ranges_j = np.array([[0, N]], np.int64)
+    slices_j = np.array([1], np.int64)
+    red_i = np.array([[0, M]], np.int64)
+    ranges = tuple(torch.from_numpy(r).cuda() for r in (ranges_i, slices_i, red_j, ranges_j, slices_j, red_i))
+    got = _knn(D, K, op)(*to_dev(x, y), ranges=ranges)
+    assert keops_io.last_loader.module.meta("scheme") == "knn" and keops_io.last_loader.module.meta("ranges") == "1"
+    ref = cpu_reduc("sqdist", [x, y], M, N, 1, reduction="KMin_ArgKMin", K=K, scheme="direct_sum",
+                    ranges=(ranges_i, slices_i, red_j))
+    rv, ri = ref[:, 0::2], ref[:, 1::2].astype(np.int64)
+    if op == "KMin_ArgKMin":
+        vals, idx = (t.cpu().numpy().reshape(M, K) for t in got)
+        assert np.array_equal(idx, ri) and np.array_equal(vals, rv)
+    elif op == "ArgKMin":
+        assert np.array_equal(got.cpu().numpy().reshape(M, K), ri)
+    else:
+        assert np.array_equal(got.cpu().numpy().reshape(M, K), rv)
+    assert np.isinf(rv[1100]).all() and np.isinf(rv[5195, 2:]).all()      # the cases above are really there
+    # second call with the same range tensors: table built on the device, same result
+    again = _knn(D, K, op)(*to_dev(x, y), ranges=ranges)
+    a0, g0 = (again[0], got[0]) if isinstance(got, tuple) else (again, got)
+    assert torch.equal(a0, g0)
+
+
 def test_small_problem_stays_on_the_general_purpose_kernel(monkeypatch):
     """Below config.knn_min_work the fixed cost of the matrix-core pipeline does not pay: same results from the
     general-purpose kernel."""
