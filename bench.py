@@ -248,14 +248,15 @@ def calibration(mfma):
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     simds, clock = 4 * cus, 2.4e9
     rows = []
-    kinds = [(3, "v_mfma_f32_32x32x16_bf16", (1, 2, 4)), (4, "v_mfma_f32_32x32x16_f16", (1, 2, 4))] if mfma else [
+    kinds = [(3, "v_mfma_f32_32x32x16_bf16", (1, 2, 4)), (4, "v_mfma_f32_32x32x16_f16", (1, 2, 4)),
+             (5, "two chains of v_mfma_f32_32x32x16_bf16 with `chains` v_fmac_f32 after every matrix instruction", (0, 1, 2, 4, 8))] if mfma else [
         (0, "v_fmac_f32 chains", (1, 2, 4, 8)), (1, "Gaussian pair mix with v_exp_f32 (9 instr)", (1, 2, 4, 8)),
         (2, "Gaussian pair mix without v_exp_f32 (8 instr)", (1, 2, 4, 8))]
     for kind, label, chain_set in kinds:
         for chains in chain_set:
             for waves in (1, 2, 4):
                 blocks = cus * waves  # one workgroup = 4 wavefronts = one per SIMD of a CU
-                iters = 200_000 // chains if kind < 3 else 100_000 // chains
+                iters = 200_000 // chains if kind < 3 else (100_000 // chains if kind < 5 else 50_000)
                 ms, ipw = binder.calibrate(kind, chains, blocks, iters)
                 total = ipw * blocks * 4  # wavefront instructions
                 per_cycle = total / (ms * 1e-3) / simds / clock

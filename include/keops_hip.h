@@ -164,7 +164,9 @@ int keops_hip_ranges_status(void* module, unsigned* status);
  * chains, and returns the elapsed time in ms and the counted instructions per wavefront.
  *   kind 0: v_fmac_f32 only (8 per chain and round); kind 1: the 9-instruction mix of a Gaussian pair (3 sub,
  *   mul, 2 fma, mul, v_exp_f32, fma); kind 2: the same without v_exp_f32; kind 3: v_mfma_f32_32x32x16_bf16
- *   (4 per chain and round); kind 4: v_mfma_f32_32x32x16_f16.  chains: 1, 2, 4, 8 (kinds 0-2) or 1, 2, 4 (kinds 3, 4).
+ *   (4 per chain and round); kind 4: v_mfma_f32_32x32x16_f16; kind 5: two chains of the bf16 instruction (8 per round)
+ *   with `chains` independent v_fmac_f32 after every matrix instruction (what fits beside a saturated matrix pipe).
+ *   chains: 1, 2, 4, 8 (kinds 0-2), 1, 2, 4 (kinds 3, 4) or 0, 1, 2, 4, 8 (kind 5).
  * Measurement aid without counterpart in the reference; used by bench.py --valu-calibration / --mfma-calibration.
  */
 int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave);

@@ -283,8 +283,55 @@ static __global__ void __launch_bounds__(256) keops_mfma_loop(float* out, int it
   out[(size_t)blockIdx.x * 256 + threadIdx.x] = r;
 }
 
+// `iters` rounds of 8 v_mfma_f32_32x32x16_bf16 (two dependent chains of 4, the shape of the K-nearest-neighbour
+// filter) with NV independent v_fmac_f32 between them: how much vector work fits beside a saturated matrix pipe
+template <int NV>
+static __global__ void __launch_bounds__(256) keops_mix_loop(float* out, int iters, float c0, float c1) {
+  keops_f32x16 acc[2];
+  keops_bf16x8 a, b;
+  unsigned h = 0x9e3779b9u * (threadIdx.x + 1u);
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    h = h * 1664525u + 1013904223u;
+    a[e] = (__bf16)(1.0f + (float)(h >> 8) * (1.0f / 16777216.0f));
+    h = h * 1664525u + 1013904223u;
+    b[e] = (__bf16)(((h & 1u) ? -1.0f : 1.0f) * (0.5f + (float)(h >> 8) * (0.5f / 16777216.0f)));
+  }
+#pragma unroll
+  for (int k = 0; k < 2; k++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[k][e] = 0.f;
+  float v[8];
+#pragma unroll
+  for (int k = 0; k < 8; k++) v[k] = 1.0f + 1e-3f * (float)(threadIdx.x + k);
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+#pragma unroll
+      for (int k = 0; k < 2; k++) {
+        acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[k], 0, 0, 0);
+#pragma unroll
+        for (int w = 0; w < NV / 8; w++) {
+          const int c = (u * 2 + k + w) & 7;
+          v[c] = __builtin_fmaf(v[c], c0, c1);
+          asm volatile("" : "+v"(v[c]));
+        }
+      }
+    }
+  }
+  float r = 0.f;
+#pragma unroll
+  for (int k = 0; k < 2; k++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) r += acc[k][e];
+#pragma unroll
+  for (int k = 0; k < 8; k++) r += v[k];
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = r;
+}
+
 // Runs one calibration loop on `stream`: grid of `blocks` workgroups of 256 lanes (4 wavefronts), `iters` rounds.
-// kind 0/1/2: vector loop with MIX = kind; kind 3 / 4: matrix loop on bf16 / f16 operands.  chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
+// kind 0/1/2: vector loop with MIX = kind; kind 3 / 4: matrix loop on bf16 / f16 operands; kind 5: 8 bf16 matrix
+// instructions per round with `chains` v_fmac_f32 after each of them (0, 1, 2, 4, 8).  chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
 // instr_per_lane receives the number of counted instructions one wavefront issues (vector: per lane = per wavefront
 // instruction count; matrix: v_mfma instructions).  out must hold blocks * 256 floats.
 int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* out, void* stream, double* instr_per_wave) {
@@ -313,6 +360,13 @@ int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* o
     else if (chains == 4) MFMA_CASE(4);
     else return (int)hipErrorInvalidValue;
 #undef MFMA_CASE
+  } else if (kind == 5) {
+    // chains = vector instructions per matrix instruction: 0, 1, 2, 4, 8
+    *instr_per_wave = 8.0 * (double)iters;
+#define MIX_CASE(N) hipLaunchKernelGGL((keops_mix_loop<N>), g, b, 0, s, out, iters, 1.0009765625f, 0.99951171875f)
+    if (chains == 0) MIX_CASE(0); else if (chains == 1) MIX_CASE(8); else if (chains == 2) MIX_CASE(16);
+    else if (chains == 4) MIX_CASE(32); else if (chains == 8) MIX_CASE(64); else return (int)hipErrorInvalidValue;
+#undef MIX_CASE
   } else {
     return (int)hipErrorInvalidValue;
   }
