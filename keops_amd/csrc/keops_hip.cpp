@@ -1680,7 +1680,10 @@ static int launch_half(Module& m, int64_t nx, int64_t ny, int tagI, int tagZero,
     arg_off[k] = take((size_t)n * sizeof(float));
   }
   const size_t out_off = take((size_t)sizeout * sizeof(float));
-  if (stream_is_capturing(stream)) m.staging.frozen = true;
+  const bool capturing = stream_is_capturing(stream);
+  if (capturing) m.staging.frozen = true;
+  // the staging buffer is shared by all launches of the module: a launch on another stream first waits for the last one
+  if (!capturing && m.has_last && m.last_stream != stream) HIP_TRY(hipStreamWaitEvent(stream, m.last_done, 0));
   if (int rc = m.staging.reserve(std::max<size_t>(off, 256))) return rc;
   char* base = (char*)m.staging.ptr;
   std::vector<void*> fargs((size_t)std::max(1, m.nargs));
@@ -1694,6 +1697,7 @@ static int launch_half(Module& m, int64_t nx, int64_t ny, int tagI, int tagZero,
     return rc;
   if (int e = keops_static_convert_half(out, base + out_off, sizeout, 0, stream))
     return fail(e, std::string("float -> half conversion failed: ") + hipGetErrorString((hipError_t)e));
+  if (!capturing && m.last_done) HIP_TRY(hipEventRecord(m.last_done, stream));  // the conversion reads the staging buffer too
   if (sync) HIP_TRY(hipStreamSynchronize(stream));
   return 0;
 }

@@ -92,3 +92,37 @@ def test_use_half_through_the_abi_refuses_what_it_cannot_serve():
         ld.module(1, p.dimy, 100, 120, p.tagI, 0, 1, p.tag1D2D, p.dimred, p.cuda_block_size, p.use_chunk_mode, p.indsi,
                   p.indsj, p.indsp, p.dim, p.dimsx, p.dimsy, p.dimsp, ld.empty_ranges, (100, 1), out.data_ptr(),
                   (x.data_ptr(), y.data_ptr()), ((100, 3), (120, 3)))
+
+
+def test_half_precision_launch_under_graph_capture():
+    """After an eager call that sizes the staging buffer, the conversions and the launch record into a HIP graph; replays
+    follow new input values bit for bit."""
+    from keops_amd.torch import Genred
+
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    x, y, b = (torch.randn(n, d, device="cuda", generator=gen).half() for n, d in ((3000, 3), (4000, 3), (4000, 2)))
+    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)"], reduction_op="Sum", axis=1)
+
+    def replays_like_eager(fn, inputs, replays=3):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                fn(*inputs)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = fn(*inputs)
+        for _ in range(replays):
+            for t in inputs:
+                t.copy_(torch.randn(t.shape, device="cuda", generator=gen).half())
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = out.clone()
+            if not torch.equal(got, fn(*inputs)):
+                return False
+        return True
+
+    assert replays_like_eager(conv, [x, y, b])
