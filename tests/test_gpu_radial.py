@@ -208,3 +208,46 @@ def test_gradients_wrt_points_and_weights_with_matrix_core_exponents(D):
     refb = cpu_reduc("gauss", [y, x, e, g], N, M, 1, rows=cols)
     scaleb = cpu_reduc("gauss", [y, x, np.abs(e), g], N, M, 1, rows=cols)
     assert_sum_parity(gb[torch.from_numpy(cols).cuda()].cpu().numpy(), refb, scaleb)
+
+
+@pytest.mark.parametrize("seed", [0, 7])
+def test_random_clouds_and_kernel_widths_vs_oracle(seed):
+    """Seeded sweep over dimensions, cloud shapes (anisotropic, two clumps, far from the origin), weight scales and
+    kernel widths from 5 times narrower to 30 times wider than the cloud: the device-side check sends each case to
+    the matrix-core exponents or to the exact differences, and every one meets the parity bar against the oracle
+    (rows whose whole sum underflows in float32 are left out)."""
+    rng = np.random.default_rng(seed)
+    served = 0
+    for case in range(20):
+        D, Dv = int(rng.integers(2, 9)), int(rng.integers(1, 9))
+        M = int(rng.integers(12000, 40000))
+        N = max(1, (1 << 27) // M + int(rng.integers(1, 3000)))
+        spread = float(10 ** rng.uniform(-2, 1.5))
+        offset = float(rng.choice([0, 0, 1, 30, 1000])) * spread
+        aniso = rng.uniform(0.05, 1, D) if rng.random() < 0.5 else np.ones(D)
+        x = (rng.standard_normal((M, D)) * aniso * spread + offset).astype(np.float32)
+        y = (rng.standard_normal((N, D)) * aniso * spread + offset * (1 + 0.01 * rng.random())).astype(np.float32)
+        if rng.random() < 0.3:
+            y[: N // 2] += 5 * spread
+        b = rng.standard_normal((N, Dv)).astype(np.float32) * float(10 ** rng.uniform(-3, 3))
+        if rng.random() < 0.3:
+            b = np.abs(b)
+        # (not narrower than a fifth of the cloud: below, every row sums exponents of -50 and less, where the hardware
+        # exp2 of this build and the reference's own fast exponential are both beyond 1e-5 of the libm value)
+        width = float(10 ** rng.uniform(-0.7, 1.5)) * spread
+        g = np.array([1.0 / (2 * width * width)], np.float32)
+        got = _genred(D, Dv)(*to_dev(x, y, b, g))
+        served += _last_meta("radial") == "1"
+        rows = np.sort(rng.choice(M, 400, replace=False)).astype(np.int64)
+        ref = cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
+        scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, Dv, rows=rows)
+        live = scale.max(axis=1) > 1e-30
+        if not live.any():
+            continue
+        out = got[torch.from_numpy(rows).cuda()].cpu().numpy()
+        try:
+            assert_sum_parity(out[live], ref[live], np.maximum(scale[live], 1e-30))
+        except AssertionError as e:
+            raise AssertionError(f"case {case}: D={D} Dv={Dv} M={M} N={N} spread={spread:.3g} offset={offset:.3g} "
+                                 f"width={width:.3g}: {e}") from None
+    assert served >= 15
