@@ -906,7 +906,7 @@ def generate_radial_section(red, match, nargs):
         return None, None
     # output rows per wavefront (32-row blocks) and wavefronts per workgroup: the accumulators (16 per block and
     # accumulated component) live in registers
-    rb = 2 if Dv <= 2 else 1
+    rb = 2 if Dv <= config.radial_rb2_max_dv else 1
     waves = 8
     one = O.IntCst(1)
 
