@@ -57,6 +57,9 @@ radial_max_dv = 8                   # components of the weights (16 accumulators
 # the path is taken when |c| log2(e) (max |x^|^2 + max |y^|^2) <= this bound for the centred points (checked on the
 # device): the exponent is then off by at most 8 * 2^-24 of it, a kernel value by 7e-5 at worst and 1e-6 typically
 radial_rb2_max_dv = int(os.environ.get("KEOPS_AMD_RADIAL_RB2_MAX_DV", 4))  # two 32-row blocks per wavefront up to this many accumulated components
+# columns per staged tile (multiple of 32); auto: 128 up to two accumulated components per pair, 512 beyond (the
+# vector work of a sub-tile grows with the components while the cost of a tile change does not)
+radial_tile_j = os.environ.get("KEOPS_AMD_RADIAL_TJ", "auto")
 radial_limit = float(os.environ.get("KEOPS_AMD_RADIAL_LIMIT", 128.0))
 radial_min_pairs_log2 = int(os.environ.get("KEOPS_AMD_RADIAL_MIN_PAIRS", 28))  # calls below 2**27 pairs: general-purpose kernel only
 

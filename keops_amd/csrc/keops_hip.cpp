@@ -648,7 +648,7 @@ struct RadHeader {
 int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, hipStream_t stream, size_t reserved,
                   const unsigned** guard) {
   const int64_t D = m.meta_int("rad_d", 0), DV = m.meta_int("rad_dv", 0), NKB = m.meta_int("rad_nkb", 0);
-  const int64_t RB = m.meta_int("rad_rb", 0), WAVES = m.meta_int("rad_waves", 0), TJ = 128;
+  const int64_t RB = m.meta_int("rad_rb", 0), WAVES = m.meta_int("rad_waves", 0), TJ = m.meta_int("rad_tj", 128);
   if (D <= 0 || DV <= 0 || NKB <= 0 || RB <= 0 || WAVES <= 0) return fail(-1, "corrupt radial module metadata");
   const bool fold = m.meta_int("rad_fold", 0) != 0;  // weights folded into the exponents, columns partitioned by sign
   // (the partition pads both groups of columns to whole tiles: one more tile)

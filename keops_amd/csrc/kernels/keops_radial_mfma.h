@@ -56,7 +56,9 @@
 typedef __bf16 rad_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float rad_f32x16 __attribute__((ext_vector_type(16)));
 
+#ifndef RAD_TJ
 #define RAD_TJ 128                 // columns per staged tile
+#endif
 #define RAD_NSUB (RAD_TJ / 32)
 #define RAD_SLOTS (16 * RAD_NKB)
 #define RAD_BLOCK (64 * RAD_WAVES)

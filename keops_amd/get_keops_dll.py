@@ -907,6 +907,9 @@ def generate_radial_section(red, match, nargs):
     # output rows per wavefront (32-row blocks) and wavefronts per workgroup: the accumulators (16 per block and
     # accumulated component) live in registers
     rb = 2 if Dv <= config.radial_rb2_max_dv else 1
+    tj = (128 if Dv <= 2 else 512) if config.radial_tile_j == "auto" else int(config.radial_tile_j)
+    if tj % 32 or not 32 <= tj <= 1024:
+        raise ValueError("[KeOps] KEOPS_AMD_RADIAL_TJ must be a multiple of 32 between 32 and 1024")
     waves = 8
     one = O.IntCst(1)
 
@@ -938,9 +941,9 @@ def generate_radial_section(red, match, nargs):
     # a scalar weight and no difference factor: the weight joins the exponent, columns are partitioned by its sign
     fold = int(config.radial_fold and dimw == 1 and not diff)
     meta = dict(radial=1, rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
-                rad_yarg=y.ind, rad_fold=fold)
+                rad_yarg=y.ind, rad_fold=fold, rad_tj=tj)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
-    defs = dict(RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
+    defs = dict(RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
                 RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit)!r}f",
                 RAD_NCOLVARS=len(wl.colvars), RAD_DIMY=wl.dimy, RAD_NROWVARS=len(al.rowvars), RAD_DIMX=al.dimx)
     src += [f"#define {k} {v}" for k, v in defs.items()]
