@@ -970,7 +970,9 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
   const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(128, nys / 64));
   const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
-  const size_t o_xs = take((size_t)nxs * DP * 4), o_ys = take((size_t)nys * DP * 4);
+  // one half-precision term per component when the data are half-precision numbers (no lo parts, no centring)
+  const bool single = m.meta_int("chk_single", 0) != 0;
+  const size_t o_xs = take((size_t)nxs * DP * (single ? 2 : 4)), o_ys = take((size_t)nys * DP * (single ? 2 : 4));
   const size_t o_xn = take((size_t)nxs * 4), o_yn = take((size_t)nys * 4), o_scal = take(8);
   // final-product variant: slabs over the reduced axis fill the chip and round the grid to whole
   // rounds of workgroups (one 8-wavefront workgroup per CU, all taking the same time)
@@ -1026,7 +1028,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   const size_t psize = sizeof(ChkHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs);
   int32_t which = 0;
   auto with_which = [&](int w) { which = w; std::memcpy(buf.data() + psize, &which, 4); return psize + 4; };
-  if (mode == 0) {
+  if (mode == 0 && !single) {
     if (int rc = launch_raw(m, "keops_chk_colsum", (unsigned)nparts, 1, 256, buf.data(), psize, stream)) return rc;
     const size_t szp = with_which(nparts);
     const int64_t cw = D > 128 ? 256 : (D > 64 ? 128 : (D > 32 ? 64 : 32));  // CHK_CW: columns per workgroup

@@ -62,7 +62,14 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float chk_f32x4;
 #define CHK_KB (CHK_DPAD / 16)
 #define CHK_KBC (CHK_KB / CHK_NC)            // 16-wide k blocks per wavefront
 #define CHK_VS (16 / CHK_NC)                 // values of a 32 x 32 tile each lane evaluates
-#define CHK_ROWBYTES (CHK_DPAD * 4)          // hi part then lo part, half precision each
+// CHK_SINGLE: the data are half-precision numbers (use_half launches: float32 copies of float16 arrays).  Their
+// products are exact in float32, so one term per operand is enough: no lo parts, one matrix instruction per k block
+// instead of three, and no centring (which would leave values that one half-precision number cannot hold).
+#ifndef CHK_SINGLE
+#define CHK_SINGLE 0
+#endif
+#define CHK_RW (CHK_DPAD * (CHK_SINGLE ? 1 : 2))  // half-precision elements per stored row: [hi] or [hi | lo]
+#define CHK_ROWBYTES (CHK_RW * 2)
 #define CHK_STRIDE (CHK_ROWBYTES + 16)       // padded LDS row
 #define CHK_TJ 32                            // reduced rows per staged tile
 #define CHK_DY (KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1)
@@ -216,15 +223,15 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
       float v = 0.f;
       if (c < CHK_D) {
         v = src[row * CHK_D + c];
-        if (CHK_MODE == 0) v -= P.colsum[c] * inv;
+        if (CHK_MODE == 0 && !CHK_SINGLE) v -= P.colsum[c] * inv;
       }
       nrm += v * v;
       v *= scale;
       hi[e] = (_Float16)v;
       lo[e] = (_Float16)(v - (float)hi[e]);
     }
-    *reinterpret_cast<chk_h4*>(dst + row * 2 * CHK_DPAD + c0) = hi;
-    *reinterpret_cast<chk_h4*>(dst + row * 2 * CHK_DPAD + CHK_DPAD + c0) = lo;
+    *reinterpret_cast<chk_h4*>(dst + row * CHK_RW + c0) = hi;
+    if (!CHK_SINGLE) *reinterpret_cast<chk_h4*>(dst + row * CHK_RW + CHK_DPAD + c0) = lo;
   }
 #pragma unroll
   for (int o = CHK_LPR / 2; o > 0; o >>= 1) nrm += __shfl_xor(nrm, o, CHK_LPR);
@@ -312,12 +319,14 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
   const i64 qx = G.row(CHK_XARG, q);
 
   // B operands: split rows of the chunked row variable
-  chk_h8 bh[CHK_KBC], bl[CHK_KBC];
+  chk_h8 bh[CHK_KBC], bl[CHK_SINGLE ? 1 : CHK_KBC];
 #pragma unroll
   for (int kb = 0; kb < CHK_KBC; kb++) {
     const int k0 = (chunk * CHK_KBC + kb) * 16 + 8 * half;
-    bh[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + k0);
-    bl[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + k0);
+    bh[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * CHK_RW + k0);
+#if !CHK_SINGLE
+    bl[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * CHK_RW + CHK_DPAD + k0);
+#endif
   }
   const float xnq = CHK_MODE == 0 ? P.xn[qx] : 0.f;
   // the tile comes out of the matrix cores times chk_sc (a power of two: the scales of the two operands)
@@ -357,7 +366,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
   auto prefetch = [&](i64 j0, i64 jend) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
     const i64 jy = G.col(CHK_YARG, j0);
-    const uint4* src = reinterpret_cast<const uint4*>(P.ys + jy * 2 * CHK_DPAD);
+    const uint4* src = reinterpret_cast<const uint4*>(P.ys + jy * CHK_RW);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * CHK_BLOCK;
@@ -426,9 +435,11 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
 #pragma unroll
     for (int kb = 0; kb < CHK_KB; kb++) {
       const chk_h8 ah = *reinterpret_cast<const chk_h8*>(arow + kb * 32);
+#if !CHK_SINGLE
       const chk_h8 al = *reinterpret_cast<const chk_h8*>(arow + CHK_DPAD * 2 + kb * 32);
       s = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[kb], s, 0, 0, 0);
       s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[kb], s, 0, 0, 0);
+#endif
       s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[kb], s, 0, 0, 0);
     }
 #else
@@ -441,9 +452,11 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_main(const Chk
 #pragma unroll
       for (int kb = 0; kb < CHK_KBC; kb++) {
         const chk_h8 ah = *reinterpret_cast<const chk_h8*>(arow + kb * 32);
+#if !CHK_SINGLE
         const chk_h8 al = *reinterpret_cast<const chk_h8*>(arow + CHK_DPAD * 2 + kb * 32);
         s = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[kb], s, 0, 0, 0);
         s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[kb], s, 0, 0, 0);
+#endif
         s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[kb], s, 0, 0, 0);
       }
 #pragma unroll
@@ -794,11 +807,13 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
   if (q >= G.row_end) q = G.row_end - 1;
   const i64 qx = G.row(CHK_XARG, q);  // clamped rows compute, never store
 
-  chk_h8 bh[CHK_KB], bl[CHK_KB];
+  chk_h8 bh[CHK_KB], bl[CHK_SINGLE ? 1 : CHK_KB];
 #pragma unroll
   for (int kb = 0; kb < CHK_KB; kb++) {
-    bh[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + kb * 16 + 8 * half);
-    bl[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+    bh[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * CHK_RW + kb * 16 + 8 * half);
+#if !CHK_SINGLE
+    bl[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * CHK_RW + CHK_DPAD + kb * 16 + 8 * half);
+#endif
   }
   const float xnq = CHK_MODE == 0 ? P.xn[qx] : 0.f;
   // the tile comes out of the matrix cores times chk_sc (a power of two: the scales of the two operands)
@@ -863,7 +878,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
   auto prefetch = [&](i64 j0, i64 jend) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
     const i64 jy = G.col(CHK_YARG, j0), jv = G.col(CHK_FV_ARG, j0);
-    const uint4* src = reinterpret_cast<const uint4*>(P.ys + jy * 2 * CHK_DPAD);
+    const uint4* src = reinterpret_cast<const uint4*>(P.ys + jy * CHK_RW);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * CHK_BLOCK;
@@ -949,9 +964,11 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_final(const Ch
 #pragma unroll
     for (int kb = 0; kb < CHK_KB; kb++) {
       const chk_h8 ah = *reinterpret_cast<const chk_h8*>(arow + kb * 32);
+#if !CHK_SINGLE
       const chk_h8 al = *reinterpret_cast<const chk_h8*>(arow + CHK_DPAD * 2 + kb * 32);
       s = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[kb], s, 0, 0, 0);
       s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[kb], s, 0, 0, 0);
+#endif
       s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[kb], s, 0, 0, 0);
     }
     float sq[16];
@@ -1047,11 +1064,13 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
   if (q >= G.row_end) q = G.row_end - 1;
   const i64 qx = G.row(CHK_XARG, q);
 
-  chk_h8 bh[CHK_KB], bl[CHK_KB];
+  chk_h8 bh[CHK_KB], bl[CHK_SINGLE ? 1 : CHK_KB];
 #pragma unroll
   for (int kb = 0; kb < CHK_KB; kb++) {
-    bh[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + kb * 16 + 8 * half);
-    bl[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * 2 * CHK_DPAD + CHK_DPAD + kb * 16 + 8 * half);
+    bh[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * CHK_RW + kb * 16 + 8 * half);
+#if !CHK_SINGLE
+    bl[kb] = *reinterpret_cast<const chk_h8*>(P.xs + qx * CHK_RW + CHK_DPAD + kb * 16 + 8 * half);
+#endif
   }
   const float xnq = CHK_MODE == 0 ? P.xn[qx] : 0.f;
   // the tile comes out of the matrix cores times chk_sc (a power of two: the scales of the two operands)
@@ -1097,7 +1116,7 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
   auto prefetch = [&](i64 j0, i64 jend) {
     const int n = (int)keops_min((i64)CHK_TJ, jend - j0);
     const i64 jy = G.col(CHK_YARG, j0), jv = G.col(CHK_FV_ARG, j0);
-    const uint4* src = reinterpret_cast<const uint4*>(P.ys + jy * 2 * CHK_DPAD);
+    const uint4* src = reinterpret_cast<const uint4*>(P.ys + jy * CHK_RW);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * CHK_BLOCK;
@@ -1181,9 +1200,11 @@ extern "C" __global__ void __launch_bounds__(CHK_BLOCK) keops_chk_softmax(const 
 #pragma unroll
     for (int kb = 0; kb < CHK_KB; kb++) {
       const chk_h8 ah = *reinterpret_cast<const chk_h8*>(arow + kb * 32);
+#if !CHK_SINGLE
       const chk_h8 al = *reinterpret_cast<const chk_h8*>(arow + CHK_DPAD * 2 + kb * 32);
       s = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[kb], s, 0, 0, 0);
       s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[kb], s, 0, 0, 0);
+#endif
       s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[kb], s, 0, 0, 0);
     }
     float sq[16];

@@ -502,7 +502,7 @@ def plan_row_col_product(red, dtype, use_fast_math, enable_chunks):
     return None
 
 
-def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=False):
+def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=False, half_data=False):
     """Module source for the matrix-core chunked scheme (kernels/keops_chunk_mfma.h); ``irregular``: the
     block-sparse / batched variant (GpuReduc1D_ranges_chunks.py:21-183)."""
     from .formulas import ops as O
@@ -581,7 +581,8 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
                 ncolvars=len(layout.colvars) + ncol_extra, nparvars=len(layout.parvars), chk_d=D, chk_dpad=dpad,
                 chk_mode=mode, chk_qb=32 * waves // nc, chk_final=int(final is not None), chk_softmax=int(softmax is not None),
                 chk_xarg=xvar.ind, chk_yarg=yvar.ind, ranges=int(irregular), chk_split3=int(split3 and config.chunk_presplit),
-                chk_vcols=0 if wvar is None else -(-wvar.dim // 32) * 32, nops=L.count_ops(outs))
+                chk_vcols=0 if wvar is None else -(-wvar.dim // 32) * 32, nops=L.count_ops(outs),
+                chk_single=int(bool(half_data)))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
            f"typedef float T;\ntypedef {dtypeacc} TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
            '#include "keops_common.h"']
@@ -600,6 +601,11 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
         defs.update(KEOPS_DIMFOUT=full_post.dim, CHK_SOFTMAX=1, CHK_SM_ONE=softmax[2], CHK_FV_ARG=softmax[1].ind,
                     CHK_FV_DIM=softmax[1].dim, CHK_FNB=-(-softmax[1].dim // 32))
     near = (0.125 if D < 32 else 0.25) if config.chunk_near == "auto" else float(config.chunk_near)
+    if half_data:
+        # half-precision data: exact products of single terms, no centring; the expansion of a squared distance is off
+        # by 2^-24 of the norms only, so far fewer values need the recomputation (and uncentred norms are large)
+        near = min(near, 1.0 / 256)
+        defs["CHK_SINGLE"] = 1
     defs["CHK_NEAR"] = f"{near!r}f"
     defs["CHK_SPLIT3"] = split3
     defs["CHK_PRESPLIT"] = int(config.chunk_presplit)
@@ -982,9 +988,11 @@ def get_keops_dll(
     rows per lane, and ``batch_loop``: when not 0, the "_ranges" of the scheme id stand for a few batches
     of less than 2**batch_loop pairs each without block-sparse ranges, which a dense module may serve one batch
     at a time; ``pairs``: when not 0, the call (each batch of it) holds less than 2**pairs pairs.  ``dtype`` / ``dtypeacc`` are C
-    type names ("float" | "double")."""
-    if use_half or dtype not in ("float", "double"):
-        raise ValueError("[KeOps] only float32 and float64 data are supported by the HIP backend")
+    type names ("float" | "double").  ``use_half``: the data are half-precision numbers (converted to float32 copies by
+    the library before the launch): modules are compiled for float, and the chunked matrix-core scheme keeps one
+    half-precision term per component instead of two."""
+    if dtype not in ("float", "double") or (use_half and dtype != "float"):
+        raise ValueError("[KeOps] the HIP backend computes in float32 (also for half-precision data) or float64")
     if "Gpu" not in map_reduce_id:
         raise ValueError("[KeOps] the HIP engine only builds Gpu map-reduce schemes")
     red = parse_reduction(red_formula_string, aliases)
@@ -996,7 +1004,7 @@ def get_keops_dll(
         rows_hint = nx if nx < 64 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
            use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs),
-           binder.templates_digest(), bool(config.radial), bool(config.radial_fold))
+           binder.templates_digest(), bool(config.radial), bool(config.radial_fold), bool(use_half))
     with _lock:
         hit = _cache.get(key)
     if hit is not None:
@@ -1037,7 +1045,8 @@ def get_keops_dll(
             source, meta = generate_final_plugin(red, fin, sum_scheme_string, nargs, irregular=irregular)
             use_chunk_mode = 2  # as the reference's final-chunk mode (get_keops_dll.py:101-108)
         elif chk is not None:
-            source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs, irregular=irregular)
+            source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs, irregular=irregular,
+                                                 half_data=bool(use_half))
             use_chunk_mode = 1 if source is not None else 0
         elif knn_hd is not None:
             source, meta = generate_knn_highdim_plugin(red_k, knn_hd, nargs)
@@ -1074,7 +1083,7 @@ def get_keops_dll(
             binder.compile_module(target, source, use_fast_math, max(0, device_id))
             config.message("OK", flush=True)
     res = (
-        tag, src_file, target, red.tagI, tagZero, 0, int(bool(use_fast_math)), config.block_size, use_chunk_mode,
+        tag, src_file, target, red.tagI, tagZero, int(bool(use_half)), int(bool(use_fast_math)), config.block_size, use_chunk_mode,
         0 if tagZero else tag1D2D, red.dimred, red.dim, layout.dimy,
         tuple(v.ind for v in layout.rowvars), tuple(v.ind for v in layout.colvars), tuple(v.ind for v in layout.parvars),
         tuple(v.dim for v in layout.rowvars), tuple(v.dim for v in layout.colvars), tuple(v.dim for v in layout.parvars),

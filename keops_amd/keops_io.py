@@ -86,7 +86,7 @@ class LoadKeOps_hip:
          p.cuda_block_size, p.use_chunk_mode, p.tag1D2D, p.dimred, p.dim, p.dimy, indsi, indsj, indsp, dimsx,
          dimsy, dimsp) = get_keops_dll(
             map_reduce_id, formula, p.enable_chunks, -1, p.mult_var_highdim, p.aliases, nargs, p.c_dtype,
-            p.c_dtype_acc, p.sum_scheme, tagHostDevice, tagCPUGPU, tag1D2D, False, optional_flags["use_fast_math"],
+            p.c_dtype_acc, p.sum_scheme, tagHostDevice, tagCPUGPU, tag1D2D, self.half, optional_flags["use_fast_math"],
             device_id_request, nx=nx, batch_loop=batch_loop, pairs=pairs,
         )
         # the engine reports (output-indexed, reduced) variable lists; the ABI takes (i, j) lists

@@ -51,7 +51,23 @@ def test_half_precision_other_schemes_and_gradients():
     lap = Genred("Exp(-Norm2(x-y))*b", ["x=Vi(64)", "y=Vj(64)", "b=Vj(4)"], reduction_op="Sum", axis=1)
     got = lap(x, y, b)
     assert keops_io.last_loader.module.meta("scheme") == "chunk"
-    assert torch.equal(got, lap(x.float(), y.float(), b.float()).half())
+    # half-precision numbers multiply exactly in float32: the contraction keeps one term per component (one matrix
+    # instruction per block instead of three, no centring); the float32 result behind the final rounding is as
+    # good as the two-term one of float32 data
+    assert keops_io.last_loader.module.meta("chk_single") == "1"
+    K = torch.exp(-torch.cdist(x.double(), y.double()))
+    ref, scale = K @ b.double(), K @ b.double().abs()
+    assert float(((got.double() - ref).abs() / scale).max()) < 6e-4          # the rounding of the result to half
+    f32 = lap(x.float(), y.float(), b.float())
+    assert keops_io.last_loader.module.meta("chk_single") == "0"
+    assert float(((f32.double() - ref).abs() / scale).max()) < 1e-5
+    # scalar products of half data, and data far from the origin (uncentred norms, near-pair recomputation)
+    lin = Genred("(x|y)*b", ["x=Vi(64)", "y=Vj(64)", "b=Vj(4)"], reduction_op="Sum", axis=1)
+    refl, scl = (x.double() @ y.double().T) @ b.double(), (x.double() @ y.double().T).abs() @ b.double().abs()
+    assert float(((lin(x, y, b).double() - refl).abs() / scl).max()) < 6e-4
+    xo, yo = (x.float() + 3.0).half(), (y.float() + 3.0).half()
+    Ko = torch.exp(-torch.cdist(xo.double(), yo.double()))
+    assert float(((lap(xo, yo, b).double() - Ko @ b.double()).abs() / (Ko @ b.double().abs())).max()) < 6e-4
     lse = Genred("-SqDist(x,y)", ["x=Vi(64)", "y=Vj(64)"], reduction_op="LogSumExp", axis=1)
     # (the kernel returns the pair (max, sum of shifted exponentials), which is rounded to half before the layer above
     # takes the logarithm, as in the reference: close, not bit-equal)
