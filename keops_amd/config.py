@@ -61,7 +61,9 @@ radial_rb2_max_dv = int(os.environ.get("KEOPS_AMD_RADIAL_RB2_MAX_DV", 4))  # two
 # vector work of a sub-tile grows with the components while the cost of a tile change does not)
 radial_tile_j = os.environ.get("KEOPS_AMD_RADIAL_TJ", "auto")
 radial_limit = float(os.environ.get("KEOPS_AMD_RADIAL_LIMIT", 128.0))
-radial_min_pairs_log2 = int(os.environ.get("KEOPS_AMD_RADIAL_MIN_PAIRS", 28))  # calls below 2**27 pairs: general-purpose kernel only
+# calls below 2**28 pairs (16384 x 16384) stay on the general-purpose kernel: measured 0.061 vs 0.074 ms at 12000^2, equal at
+# 16000^2, 0.150 vs 0.126 ms at 23000^2 (the pre-pass of the matrix-core scheme is seven small launches)
+radial_min_pairs_log2 = int(os.environ.get("KEOPS_AMD_RADIAL_MIN_PAIRS", 29))
 
 # matrix-core final-product scheme (csrc/kernels/keops_final_mfma.h): Sum_j f(x_i,y_j) * v_j with dim(v) large
 final_chunk_min_dim = int(os.environ.get("KEOPS_AMD_FINAL_MIN_DIM", 24))   # smallest dim(v) that selects the scheme
