@@ -43,8 +43,8 @@ MEASURED_TRAFFIC_BYTES = {
     "softmax_d64": int((204925 * 2.0 + 33804) * 1024),
     # profiles/keops_fin_main3__gauss_dv256.md
     "gauss_dv256": int((10715900 * 2.0 + 10797000) * 1024),
-    # profiles/keops_conv_ranges__sparse_100x10k.md, keops_conv_ranges__lse_b16.md
-    "sparse_100x10k": int((109492 * 2.0 + 3906.25) * 1024),
+    # profiles/keops_radr_main__sparse_100x10k.md (all kernels of a launch), keops_conv_ranges__lse_b16.md
+    "sparse_100x10k": int((638070 * 2.0 + 179582) * 1024),
     "lse_b16": int((55625 * 2.0 + 6250) * 1024),
     # profiles/keops_conv_dense_vchunk__knn_l1_d784.md
     "knn_l1_d784": int((4176921 * 2.0 + 39063) * 1024),

@@ -159,6 +159,15 @@ size_t keops_hip_noalloc_scratch_bytes(void);
 int keops_hip_ranges_status(void* module, unsigned* status);
 
 /*
+ * Which kernel family served the module's last launch; waits for that launch.  Modules of Gaussian-type sums carry
+ * two families (meta key radial=1): exponents from the matrix cores, chosen on the device when the kernel is not
+ * too narrow for the cloud (for block-sparse launches: for every row range), and the general-purpose kernel from
+ * exact differences otherwise.  *taken: 1 the matrix-core family ran, 0 the general-purpose one (or the module has
+ * one family only, or the launch was too small to try).  No counterpart in the reference.
+ */
+int keops_hip_radial_status(void* module, unsigned* taken);
+
+/*
  * Loop-only calibration of the instruction issue rates the roofline fractions are held against: runs a grid of
  * `blocks` workgroups of 4 wavefronts, each wavefront issuing `iters` rounds of `chains` independent dependency
  * chains, and returns the elapsed time in ms and the counted instructions per wavefront.

@@ -63,6 +63,7 @@ radial_tile_j = os.environ.get("KEOPS_AMD_RADIAL_TJ", "auto")
 radial_limit = float(os.environ.get("KEOPS_AMD_RADIAL_LIMIT", 128.0))
 # calls below 2**28 pairs (16384 x 16384) stay on the general-purpose kernel: measured 0.061 vs 0.074 ms at 12000^2, equal at
 # 16000^2, 0.150 vs 0.126 ms at 23000^2 (the pre-pass of the matrix-core scheme is seven small launches)
+radial_ranges = os.environ.get("KEOPS_AMD_RADIAL_RANGES", "1") != "0"  # block-sparse launches too (one centre per row range)
 radial_min_pairs_log2 = int(os.environ.get("KEOPS_AMD_RADIAL_MIN_PAIRS", 29))
 
 # matrix-core final-product scheme (csrc/kernels/keops_final_mfma.h): Sum_j f(x_i,y_j) * v_j with dim(v) large

@@ -266,6 +266,9 @@ struct Module {
   // number of workgroups it found, and where the device path keeps its status word
   std::vector<int64_t> ranges_key;
   int64_t ranges_nblocks = 0;
+  const unsigned* last_guard = nullptr;  // flag of the last launch's device-side choice between two kernel families
+  int64_t ranges_work_total = 0;  // of the validated ranges: reduced rows swept, summed over the row ranges
+  double ranges_pairs = 0.0;      // ... and their pairs
   const unsigned* ranges_status = nullptr;
   DeviceBuffer staging;  // host-pointer launches (tagHostDevice = 0): device copies of the arguments and of out
   // a launch was recorded into a HIP graph: workspaces and tables keep their address and contents from then on
@@ -302,6 +305,11 @@ struct Module {
 struct RangeTables {
   const int64_t *lookup = nullptr, *slices_x = nullptr, *ranges_y = nullptr, *offsets = nullptr;
   int64_t nblocks = 0;
+  // block-sparse mode: the caller's row ranges (device) and what the validating launch measured on the host
+  const int64_t* rx = nullptr;
+  int64_t nranges = 0;
+  int64_t work_total = 0;   // reduced rows swept, summed over the row ranges
+  double pairs = 0.0;       // pairs of the pattern
 };
 
 int ensure_pinned(Module& m, size_t bytes);
@@ -401,6 +409,7 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
       rt.offsets = nullptr;
       rt.slices_x = (const int64_t*)B.sl_clean;
       rt.ranges_y = (const int64_t*)B.ry_clean;
+      rt.rx = rx_dev; rt.nranges = nranges; rt.work_total = m.ranges_work_total; rt.pairs = m.ranges_pairs;
       return 0;
     }
     rx_host.resize((size_t)2 * nranges);
@@ -552,6 +561,13 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
     m.ranges_key = ukey;  // read and validated: later calls build the table on the device
     m.ranges_nblocks = nblocks;
     m.ranges_status = nullptr;
+    m.ranges_work_total = 0;
+    m.ranges_pairs = 0.0;
+    for (int64_t r = 0; r < nranges; r++) {
+      m.ranges_work_total += range_work[r];
+      m.ranges_pairs += (double)range_work[r] * (double)(rx_host[2 * r + 1] - rx_host[2 * r]);
+    }
+    rt.rx = rx_dev; rt.nranges = nranges; rt.work_total = m.ranges_work_total; rt.pairs = m.ranges_pairs;
   }
   const int64_t* tab = (const int64_t*)m.tables.ptr;
   rt.nblocks = nblocks;
@@ -696,6 +712,64 @@ int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* arg
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
   if (int rc = launch_raw(m, "keops_rad_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)(64 * WAVES), buf.data(), psize, stream)) return rc;
   if (int rc = launch_raw(m, "keops_rad_reduce", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), psize, stream)) return rc;
+  *guard = (const unsigned*)(ws + o_scal) + 2;
+  return 0;
+}
+
+// must match struct RadRParams of kernels/keops_radial_ranges.h (argument pointers follow)
+struct RadRHeader {
+  int64_t nx, ny, nranges, nblocks;
+  const void* rx;
+  RangeHeader rt;
+  void *xa, *yb, *bw, *ctr, *vt, *rmax, *scal;
+  int64_t vt_capacity;
+  void *out, *partial;
+};
+
+// Block-sparse launches of a module built with radial=1 and rad_ranges=1: every row range gets its own centre and
+// its own formatted copy of the columns it sweeps (kernels/keops_radial_ranges.h).  Worth it when the row ranges are
+// long (the copy is one column per range and column, the work one pair per row and column) and the pattern holds
+// enough pairs; otherwise *guard stays null and the general-purpose kernel runs alone.  All launches asynchronous.
+int launch_radial_ranges(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, hipStream_t stream, const RangeTables& rt,
+                         const unsigned** guard) {
+  *guard = nullptr;
+  const int64_t D = m.meta_int("rad_d", 0), DV = m.meta_int("rad_dv", 0), NKB = m.meta_int("rad_nkb", 0);
+  const int64_t RB = m.meta_int("rad_rb", 0), WAVES = m.meta_int("rad_waves", 0), TJ = m.meta_int("rad_tj", 128);
+  if (D <= 0 || DV <= 0 || NKB <= 0 || RB <= 0 || WAVES <= 0) return fail(-1, "corrupt radial module metadata");
+  const int64_t RPB = 32 * RB * WAVES;
+  if (RPB != (int64_t)m.block * m.rows) return fail(-1, "corrupt radial module metadata: rows per workgroup");
+  static const double min_pairs = [] {
+    const char* e = std::getenv("KEOPS_HIP_RADIAL_RANGES_MIN_PAIRS");
+    return e ? std::atof(e) : 268435456.0;  // 2^28, as for dense launches
+  }();
+  // rows per formatted column: at 128 the copy costs about a tenth of the sweep
+  if (rt.nranges <= 0 || rt.pairs < min_pairs || rt.pairs < 128.0 * (double)rt.work_total || rt.nblocks < (int64_t)m.cu_count) return 0;
+  const int64_t vt_capacity = rt.work_total / TJ + rt.nranges;  // every range pads less than one tile
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+  const size_t o_scal = take(32), o_ctr = take((size_t)rt.nranges * D * 4), o_vt = take((size_t)rt.nranges * 16), o_rmax = take((size_t)rt.nranges * 8);
+  const size_t o_xa = take((size_t)rt.nblocks * RPB * NKB * 32), o_yb = take((size_t)vt_capacity * TJ * NKB * 32);
+  const size_t o_bw = take((size_t)vt_capacity * TJ * DV * 4), o_part = take((size_t)rt.nblocks * RPB * DV * 4);
+  if (off > ((size_t)4 << 30)) return 0;  // the formatted operands stay within 4 GiB
+  if (int rc = m.partial.reserve(off)) return rc;
+  char* ws = (char*)m.partial.ptr;
+  std::vector<char> buf(sizeof(RadRHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs));
+  RadRHeader h{};
+  h.nx = nx; h.ny = ny; h.nranges = rt.nranges; h.nblocks = rt.nblocks; h.rx = rt.rx;
+  h.rt.lookup = rt.lookup; h.rt.slices_x = rt.slices_x; h.rt.ranges_y = rt.ranges_y; h.rt.offsets = nullptr;
+  h.rt.nbatchdims = 0; h.rt.nargs = m.nargs;
+  h.xa = ws + o_xa; h.yb = ws + o_yb; h.bw = ws + o_bw; h.ctr = ws + o_ctr; h.vt = ws + o_vt; h.rmax = ws + o_rmax; h.scal = ws + o_scal;
+  h.vt_capacity = vt_capacity; h.out = out; h.partial = ws + o_part;
+  std::memcpy(buf.data(), &h, sizeof(h));
+  for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
+  const size_t psize = buf.size();
+  if (int rc = launch_raw(m, "keops_radr_centres", (unsigned)rt.nranges, 1, 256, buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_radr_scan", 1, 1, 1024, buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_radr_prep_rows", (unsigned)rt.nblocks, 1, (unsigned)RPB, buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_radr_prep_cols", (unsigned)rt.nranges, 8, 256, buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_radr_decide", 1, 1, 256, buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_radr_main", (unsigned)rt.nblocks, 1, (unsigned)(64 * WAVES), buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_radr_finish", (unsigned)rt.nblocks, 1, (unsigned)RPB, buf.data(), psize, stream)) return rc;
   *guard = (const unsigned*)(ws + o_scal) + 2;
   return 0;
 }
@@ -1541,6 +1615,7 @@ static int launch_on_device(Module& m, int64_t nx, int64_t ny, int tagI, int tag
       // exponents on the matrix cores when the data allow it (decided on the device); the kernels below then return
       // at once, and the other way round.  Both share the workspace: slab partials first.
       if (int rc = launch_radial(m, rows_total, cols_total, out, args, stream, slab_bytes, &h.guard)) return rc;
+      m.last_guard = h.guard;
     } else if (slab_bytes) {
       if (int rc = m.partial.reserve(slab_bytes)) return rc;
     }
@@ -1567,6 +1642,11 @@ static int launch_on_device(Module& m, int64_t nx, int64_t ny, int tagI, int tag
     if (user_ranges) {
       const int64_t gb = (rows_total + m.block - 1) / m.block;
       if (int rc = launch(m, "keops_fill_neutral", (unsigned)gb, 1, h, args, stream)) return rc;
+      // exponents on the matrix cores when the pattern and the data allow it (the latter is decided on the device):
+      // keops_conv_ranges then returns at once, and the other way round
+      if (m.meta_int("radial", 0) != 0 && m.meta_int("rad_ranges", 0) != 0)
+        if (int rc = launch_radial_ranges(m, rows_total, cols_total, out, args, stream, rt, &h.guard)) return rc;
+      m.last_guard = h.guard;
     }
     if (int rc = launch(m, "keops_conv_ranges", (unsigned)nblocks, 1, h, args, stream)) return rc;
     if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
@@ -1763,6 +1843,17 @@ int keops_hip_launch_noalloc(void* module, int64_t nx, int64_t ny, int tagI, int
   g_noalloc = false;
   std::swap(m.partial, view);
   return rc;
+}
+
+int keops_hip_radial_status(void* module, unsigned* taken) {
+  if (!module || !taken) return fail(-1, "keops_hip_radial_status: null argument");
+  Module& m = *static_cast<Module*>(module);
+  *taken = 0u;
+  if (!m.last_guard) return 0;
+  HIP_TRY(hipSetDevice(m.device));
+  if (m.has_last) HIP_TRY(hipEventSynchronize(m.last_done));
+  HIP_TRY(hipMemcpy(taken, m.last_guard, sizeof(unsigned), hipMemcpyDeviceToHost));
+  return 0;
 }
 
 int keops_hip_ranges_status(void* module, unsigned* status) {

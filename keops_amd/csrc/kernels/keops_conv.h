@@ -394,6 +394,7 @@ extern "C" __global__ void __launch_bounds__(KEOPS_BLOCK) keops_fill_neutral(con
 // (GpuReduc1D_ranges.py:127-165).  With batch dimensions, rows and columns are addressed relative
 // to per-variable offsets (broadcasting over batch dimensions, keops_nvrtc.cpp:75-149).
 extern "C" __global__ void __launch_bounds__(KEOPS_BLOCK) keops_conv_ranges(const KeopsParams P) {
+  if (P.guard != nullptr && *P.guard == 1u) return;
   __shared__ __attribute__((aligned(16))) T ys[KEOPS_TILE_J * (KEOPS_DIMY_PAD > 0 ? KEOPS_DIMY_PAD : 1)];
   constexpr int NV = KEOPS_NROWVARS + KEOPS_NCOLVARS + KEOPS_NPARVARS;
   i64 offs[NV > 0 ? NV : 1];

@@ -93,6 +93,11 @@ __device__ __forceinline__ void rad_load_params(const RadParams& P, T (&p)[KEOPS
 
 // ---- pre-pass ---------------------------------------------------------------------------------------------------
 
+#ifndef RAD_RANGES
+#define RAD_RANGES 0
+#endif
+
+#if !RAD_RANGES
 // column sums of y in two deterministic stages (fixed order, no atomics)
 extern "C" __global__ void __launch_bounds__(256) keops_rad_colsum(const RadParams P) {
   __shared__ float part[256];
@@ -123,6 +128,8 @@ extern "C" __global__ void __launch_bounds__(64) keops_rad_colsum_final(const Ra
   }
   if (c < 4) P.scal[c] = 0u;
 }
+
+#endif  // !RAD_RANGES
 
 #ifndef RAD_FOLD
 #define RAD_FOLD 0
@@ -217,6 +224,7 @@ __device__ __forceinline__ void rad_split4(double v, __bf16 (&t)[4]) {
   }
 }
 
+#if !RAD_RANGES
 // Slot vector of one point.  which = 0: rows (x), 1: columns (y; one thread per column of the padded tile grid).
 extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams P, int which) {
   const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
@@ -342,6 +350,7 @@ extern "C" __global__ void __launch_bounds__(64) keops_rad_decide(const RadParam
   const float R = __uint_as_float(P.scal[0]) + __uint_as_float(P.scal[1]);
   P.scal[2] = (__builtin_fabsf(kappa) * R <= (float)RAD_LIMIT) ? 1u : 0u;  // false for NaN
 }
+#endif  // !RAD_RANGES
 
 #if RAD_FOLD
 // k-th tile of the sweep: tiles of the two sign groups alternate while both last, then the rest of the larger group
@@ -360,21 +369,29 @@ __device__ __forceinline__ i64 rad_tile_of(i64 k, i64 pos_tiles, i64 all_tiles, 
 
 // with at most 32 accumulators per lane the kernel fits 128 registers: four wavefronts per SIMD, two workgroups per CU
 #define RAD_MIN_WAVES ((RAD_RB * 16 * RAD_DV <= 32) ? 4 : 1)
-extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad_main(const RadParams P) {
-  if (P.scal[2] != 1u) return;
-  __shared__ __attribute__((aligned(16))) __bf16 ys[RAD_NKB * 2 * RAD_TJ * 8];  // [kb][half][col][8]
-#if !RAD_FOLD
-  __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_DV];
-#endif
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
-  const i64 row0 = ((i64)blockIdx.x * RAD_WAVES + wave) * (32 * RAD_RB);
+
+// What one wavefront sweeps: its 32 * RAD_RB rows against the columns [jbeg, jend) of the pre-formatted operand.
+struct RadSweep {
+  const __bf16* xa;    // slot vectors of the wavefront's rows: [rows_avail][RAD_SLOTS]
+  i64 rows_avail;      // rows past the last one are clamped to it (they compute, never store)
+  const __bf16* yb;    // column tiles
+  const float* bw;     // weights, padded to whole tiles
+  i64 jbeg, jend;      // jbeg a multiple of RAD_TJ
+  float* part;         // [rows_store][RAD_DV] sums of the wavefront's rows
+  i64 rows_store;
+  i64 pos_tiles, all_tiles;  // RAD_FOLD
+};
+
+// All wavefronts of the workgroup call this together with the same columns (they share the staged tile).
+__device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* bs) {
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, col = lane & 31;
   rad_bf16x8 a[RAD_RB][RAD_NKB];
 #pragma unroll
   for (int r = 0; r < RAD_RB; r++) {
-    i64 i = row0 + r * 32 + col;
-    if (i >= P.nx) i = P.nx - 1;  // clamped rows compute, never store
+    i64 i = r * 32 + col;
+    if (i >= S.rows_avail) i = S.rows_avail - 1;
 #pragma unroll
-    for (int kb = 0; kb < RAD_NKB; kb++) a[r][kb] = *reinterpret_cast<const rad_bf16x8*>(P.xa + i * RAD_SLOTS + kb * 16 + 8 * half);
+    for (int kb = 0; kb < RAD_NKB; kb++) a[r][kb] = *reinterpret_cast<const rad_bf16x8*>(S.xa + i * RAD_SLOTS + kb * 16 + 8 * half);
   }
   float acc[RAD_RB][16][RAD_DV];
 #pragma unroll
@@ -384,9 +401,7 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
 #pragma unroll
       for (int d = 0; d < RAD_DV; d++) acc[r][v][d] = 0.f;
 
-  // (RAD_FOLD: the partition by sign pads both groups to whole tiles: one more tile than the columns need)
-  const i64 ncols = RAD_FOLD ? ((P.ny + RAD_TJ - 1) / RAD_TJ + 1) * RAD_TJ : P.ny;
-  const i64 jbeg = (i64)blockIdx.y * P.slab_len, jend = keops_min(ncols, jbeg + P.slab_len);
+  const i64 jbeg = S.jbeg, jend = S.jend;
   // software pipeline: tile t+1 travels to registers while tile t is consumed
   constexpr int CH = RAD_NKB * 2 * RAD_TJ;  // 16-byte chunks of the slot vectors of a tile
   constexpr int NPF = (CH + RAD_BLOCK - 1) / RAD_BLOCK;
@@ -394,24 +409,22 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
   uint4 pf[NPF];
 #if !RAD_FOLD
   float pfw[NPW];
-#else
-  const i64 pos_tiles = keops_uniform((i64)P.scal[3]);  // tiles of columns with non-negative weights come first
 #endif
   auto prefetch = [&](i64 j0) {
 #if RAD_FOLD
     bool neg_;
-    const i64 tile = rad_tile_of(j0 / RAD_TJ, pos_tiles, ncols / RAD_TJ, neg_);
+    const i64 tile = rad_tile_of(j0 / RAD_TJ, S.pos_tiles, S.all_tiles, neg_);
 #else
     const i64 tile = j0 / RAD_TJ;
 #endif
-    const uint4* src = reinterpret_cast<const uint4*>(P.yb + tile * (RAD_NKB * 2 * RAD_TJ * 8));
+    const uint4* src = reinterpret_cast<const uint4*>(S.yb + tile * (RAD_NKB * 2 * RAD_TJ * 8));
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * RAD_BLOCK;
       pf[u] = e < CH ? src[e] : make_uint4(0u, 0u, 0u, 0u);
     }
 #if !RAD_FOLD
-    const float* wsrc = P.bw + j0 * RAD_DV;  // padded to whole tiles
+    const float* wsrc = S.bw + j0 * RAD_DV;  // padded to whole tiles
 #pragma unroll
     for (int u = 0; u < NPW; u++) {
       const int e = tid + u * RAD_BLOCK;
@@ -438,7 +451,7 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
     if (j0 + RAD_TJ < jend) prefetch(j0 + RAD_TJ);
 #if RAD_FOLD
     bool negative;  // uniform: one sign per tile
-    (void)rad_tile_of(j0 / RAD_TJ, pos_tiles, ncols / RAD_TJ, negative);
+    (void)rad_tile_of(j0 / RAD_TJ, S.pos_tiles, S.all_tiles, negative);
 #endif
 #pragma unroll
     for (int sub = 0; sub < RAD_NSUB; sub++) {
@@ -490,17 +503,48 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
   for (int r = 0; r < RAD_RB; r++)
 #pragma unroll
     for (int v = 0; v < 16; v++) {
-      const i64 i = row0 + r * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+      const i64 i = r * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
 #pragma unroll
       for (int d = 0; d < RAD_DV; d++) {
         float s = acc[r][v][d];
 #pragma unroll
         for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o);
-        if (col == 0 && i < P.nx) P.partial[((i64)blockIdx.y * P.nx + i) * RAD_DV + d] = s;
+        if (col == 0 && i < S.rows_store) S.part[i * RAD_DV + d] = s;
       }
     }
 }
 
+#if !RAD_RANGES
+extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad_main(const RadParams P) {
+  if (P.scal[2] != 1u) return;
+  __shared__ __attribute__((aligned(16))) __bf16 ys[RAD_NKB * 2 * RAD_TJ * 8];  // [kb][half][col][8]
+#if !RAD_FOLD
+  __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_DV];
+#else
+  float* bs = nullptr;
+#endif
+  const int wave = threadIdx.x >> 6;
+  const i64 row0 = ((i64)blockIdx.x * RAD_WAVES + wave) * (32 * RAD_RB);
+  // (RAD_FOLD: the partition by sign pads both groups to whole tiles: one more tile than the columns need)
+  const i64 ncols = RAD_FOLD ? ((P.ny + RAD_TJ - 1) / RAD_TJ + 1) * RAD_TJ : P.ny;
+  RadSweep S;
+  // a wavefront past the last row sweeps the last row again (the workgroup's barriers need it) and stores nothing
+  const i64 first = row0 < P.nx ? row0 : P.nx - 1;
+  S.xa = P.xa + first * RAD_SLOTS;
+  S.rows_avail = P.nx - first;
+  S.yb = P.yb;
+  S.bw = P.bw;
+  S.jbeg = (i64)blockIdx.y * P.slab_len;
+  S.jend = keops_min(ncols, S.jbeg + P.slab_len);
+  S.part = P.partial + ((i64)blockIdx.y * P.nx + first) * RAD_DV;
+  S.rows_store = row0 < P.nx ? P.nx - row0 : 0;
+  S.pos_tiles = RAD_FOLD ? keops_uniform((i64)P.scal[3]) : 0;  // tiles of columns with non-negative weights come first
+  S.all_tiles = ncols / RAD_TJ;
+  rad_sweep(S, ys, bs);
+}
+#endif
+
+#if !RAD_RANGES
 // slabs are added in order; the factors of the output index and, for the gradients with respect to the points, the
 // difference x^_i S - sum_j K_ij w_j y^_j are applied here, once per output row
 extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadParams P) {
@@ -535,3 +579,6 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadPara
   for (int d = 0; d < RAD_DOUT; d++) P.out[i * RAD_DOUT + d] = (T)(ai * s[d]);
 #endif
 }
+#else
+#include "keops_radial_ranges.h"
+#endif

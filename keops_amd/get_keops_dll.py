@@ -784,7 +784,7 @@ def _linear_coef(E, svar):
     return None
 
 
-def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id, pairs=0):
+def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id, pairs=0, block_sparse=False):
     """dict(x, y, coef, A, W, diff) when the formula of a float32 Sum reduction on the dense scheme is a product
 
         [+-]  A(i-variables)  *  Exp(C * SqDist(x, y))  *  W(j-variables)  [ * (x - y) | (y - x) ]
@@ -801,7 +801,10 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
     from .formulas.reductions import KIND_SUM
 
     if (not config.radial or red.kind != KIND_SUM or dtype != "float" or dtypeacc != "float" or not use_fast_math
-            or "_ranges" in map_reduce_id or sum_scheme == "kahan_scheme"):
+            or sum_scheme == "kahan_scheme"):
+        return None
+    # launches with ranges: block-sparse patterns only (no batch dimensions), where every row range gets its own centre
+    if "_ranges" in map_reduce_id and not (block_sparse and config.radial_ranges):
         return None
     if pairs and int(pairs) < config.radial_min_pairs_log2:
         return None
@@ -871,9 +874,11 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
     return dict(x=x, y=y, coef=coef, A=product(A), W=product(Wf), diff=diff, sign=sign)
 
 
-def generate_radial_section(red, match, nargs):
+def generate_radial_section(red, match, nargs, rows_per_block=0):
     """Source text appended to a general-purpose module: tables, the straight-line bodies of struct
-    KeopsRadFormula and the template kernels/keops_radial_mfma.h; returns (text, meta entries)."""
+    KeopsRadFormula and the template kernels/keops_radial_mfma.h; returns (text, meta entries).
+    ``rows_per_block`` > 0: block-sparse variant (kernels/keops_radial_ranges.h), whose workgroups own that many rows,
+    like the general-purpose kernel of the same module: both read one lookup table."""
     from .formulas import ops as O
     from .formulas.lir import LOG2E
 
@@ -917,6 +922,10 @@ def generate_radial_section(red, match, nargs):
     if tj % 32 or not 32 <= tj <= 1024:
         raise ValueError("[KeOps] KEOPS_AMD_RADIAL_TJ must be a multiple of 32 between 32 and 1024")
     waves = 8
+    if rows_per_block:
+        if rows_per_block % (32 * rb) or not 2 <= rows_per_block // (32 * rb) <= 16:
+            return None, None
+        waves = rows_per_block // (32 * rb)
     one = O.IntCst(1)
 
     class _W:
@@ -945,11 +954,11 @@ def generate_radial_section(red, match, nargs):
     ca, cd, co = VarLayout.table(wl.colvars)
     ra, rd, ro = VarLayout.table(al.rowvars)
     # a scalar weight and no difference factor: the weight joins the exponent, columns are partitioned by its sign
-    fold = int(config.radial_fold and dimw == 1 and not diff)
-    meta = dict(radial=1, rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
+    fold = int(config.radial_fold and dimw == 1 and not diff and not rows_per_block)
+    meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
                 rad_yarg=y.ind, rad_fold=fold, rad_tj=tj)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
-    defs = dict(RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
+    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
                 RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit)!r}f",
                 RAD_NCOLVARS=len(wl.colvars), RAD_DIMY=wl.dimy, RAD_NROWVARS=len(al.rowvars), RAD_DIMX=al.dimx)
     src += [f"#define {k} {v}" for k, v in defs.items()]
@@ -1004,7 +1013,7 @@ def get_keops_dll(
         rows_hint = nx if nx < 64 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
            use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs),
-           binder.templates_digest(), bool(config.radial), bool(config.radial_fold), bool(use_half))
+           binder.templates_digest(), bool(config.radial), bool(config.radial_fold), bool(config.radial_ranges), bool(use_half))
     with _lock:
         hit = _cache.get(key)
     if hit is not None:
@@ -1065,9 +1074,11 @@ def get_keops_dll(
         if source is None:
             source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint,
                                            irregular=irregular)
-            rad = match_radial(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, map_reduce_id, pairs) if mc else None
+            block_sparse = irregular and batch_loop == -1
+            rad = match_radial(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, map_reduce_id, pairs, block_sparse) if mc else None
             if rad is not None:
-                section, rmeta = generate_radial_section(red, rad, nargs)
+                section, rmeta = generate_radial_section(red, rad, nargs,
+                                                         int(meta["block"]) * int(meta["rows"]) if block_sparse else 0)
                 if section is not None:
                     meta.update(rmeta)
                     head, body = source.split("\n", 1)
