@@ -7,6 +7,7 @@ Environment variables:
   KEOPS_HIP_ARCH      offload architecture used when no GPU is visible (default gfx950)
 """
 import os
+import sys
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 
@@ -59,6 +60,10 @@ radial_max_dv = 8                   # components of the weights (16 accumulators
 radial_rb2_max_dv = int(os.environ.get("KEOPS_AMD_RADIAL_RB2_MAX_DV", 4))  # two 32-row blocks per wavefront up to this many accumulated components
 # columns per staged tile (multiple of 32); auto: 128 up to two accumulated components per pair, 512 beyond (the
 # vector work of a sub-tile grows with the components while the cost of a tile change does not)
+# accumulated components from which the weighted sum of the radial scheme runs on the matrix cores (per pair the vector
+# ALU then issues v_exp_f32 and a three-term split instead of one fused multiply-add per component); 99: never
+radial_mm_min_dv = int(os.environ.get("KEOPS_AMD_RADIAL_MM_MIN_DV", 7))
+radial_mm_rb = int(os.environ.get("KEOPS_AMD_RADIAL_MM_RB", 1))   # 32-row blocks per wavefront in that variant
 radial_tile_j = os.environ.get("KEOPS_AMD_RADIAL_TJ", "auto")
 radial_limit = float(os.environ.get("KEOPS_AMD_RADIAL_LIMIT", 128.0))
 # calls below 2**28 pairs (16384 x 16384) stay on the general-purpose kernel: measured 0.061 vs 0.074 ms at 12000^2, equal at
@@ -111,5 +116,7 @@ def set_build_folder(path=None):
 
 
 def message(*args, **kwargs):
+    # progress messages go to stderr: stdout belongs to the caller (bench.py prints one JSON line there)
     if verbose:
+        kwargs.setdefault("file", sys.stderr)
         print("[keops_amd]", *args, **kwargs)

@@ -59,6 +59,10 @@ typedef float rad_f32x16 __attribute__((ext_vector_type(16)));
 #ifndef RAD_TJ
 #define RAD_TJ 128                 // columns per staged tile
 #endif
+#ifndef RAD_MM
+#define RAD_MM 0                   // 1: the weighted sum runs on the matrix cores too (see rad_sweep_mm)
+#endif
+#define RAD_MM_FOLD 4096           // columns between two folds of the running sums (block summation)
 #define RAD_NSUB (RAD_TJ / 32)
 #define RAD_SLOTS (16 * RAD_NKB)
 #define RAD_BLOCK (64 * RAD_WAVES)
@@ -224,6 +228,29 @@ __device__ __forceinline__ void rad_split4(double v, __bf16 (&t)[4]) {
   }
 }
 
+
+#if RAD_MM
+// Weights of column j in the layout of the B operand of the weighted sum (rad_sweep_mm): 32 operand columns
+// [w_h | w_m | w_l | 0] (the three bfloat16 terms of the RAD_DV weights side by side), contraction index = the 32
+// columns of a sub-tile in the order in which the exponent tile leaves them in the registers of a lane: registers
+// 0-7 (k block 0) of lanes 0-31 hold columns {0,1,2,3,8,9,10,11}, of lanes 32-63 {4,...,7,12,...,15}; registers 8-15
+// (k block 1) the same plus 16.  Layout [32-column sub-tile][k block][half][operand column][8].
+__device__ __forceinline__ void rad_store_weights_mm(__bf16* bwm, i64 j, const float (&w)[RAD_DV]) {
+  const int jj = (int)(j & 31), kb = jj >> 4, q = jj & 15, hf = (q >> 2) & 1, e = (q & 3) + 4 * (q >> 3);
+  __bf16* dst = bwm + ((((j >> 5) * 2 + kb) * 2 + hf) * 32) * 8 + e;
+#pragma unroll
+  for (int n = 0; n < 32; n++) {
+    __bf16 v = (__bf16)0.0f;
+    if (n < 3 * RAD_DV) {
+      __bf16 t3[3];
+      rad_split3(w[n % RAD_DV], t3);
+      v = t3[n / RAD_DV];
+    }
+    dst[n * 8] = v;
+  }
+}
+#endif
+
 #if !RAD_RANGES
 // Slot vector of one point.  which = 0: rows (x), 1: columns (y; one thread per column of the padded tile grid).
 extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams P, int which) {
@@ -334,7 +361,9 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
         for (int e = 0; e < 8; e++) v8[e] = slot[kb * 16 + hf * 8 + e];
         *reinterpret_cast<rad_bf16x8*>(P.yb + (((tile * RAD_NKB + kb) * 2 + hf) * RAD_TJ + c) * 8) = v8;
       }
-#if !RAD_FOLD
+#if RAD_MM
+    rad_store_weights_mm(reinterpret_cast<__bf16*>(P.bw), i, w);
+#elif !RAD_FOLD
 #pragma unroll
     for (int d = 0; d < RAD_DV; d++) P.bw[i * RAD_DV + d] = w[d];
 #endif
@@ -368,7 +397,11 @@ __device__ __forceinline__ i64 rad_tile_of(i64 k, i64 pos_tiles, i64 all_tiles, 
 // ---- main kernel ------------------------------------------------------------------------------------------------
 
 // with at most 32 accumulators per lane the kernel fits 128 registers: four wavefronts per SIMD, two workgroups per CU
+#if RAD_MM
+#define RAD_MIN_WAVES (RAD_RB == 1 ? 4 : 2)
+#else
 #define RAD_MIN_WAVES ((RAD_RB * 16 * RAD_DV <= 32) ? 4 : 1)
+#endif
 
 // What one wavefront sweeps: its 32 * RAD_RB rows against the columns [jbeg, jend) of the pre-formatted operand.
 struct RadSweep {
@@ -514,11 +547,152 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
     }
 }
 
+
+#if RAD_MM
+// The same sweep with the weighted sum on the matrix cores (3 * RAD_DV <= 32 accumulated components):
+//     out[i][d] = sum_j K_ij w_j[d]   is the matrix product   K (32 rows x 32 columns of a sub-tile) x W (32 x RAD_DV).
+// The exponent tile is computed transposed (columns as the A operand, the wavefront's rows as B), so that lane l
+// receives the 16 values of ITS row l % 32: registers 0-7 and 8-15 are then A operands of two k blocks of the second
+// product as they stand.  Float32 accuracy from bfloat16 products: K = h + m + l by truncation (two v_and, two exact
+// v_sub, byte permutes to pack: 26 issue cycles per pair with v_exp_f32, whatever RAD_DV is, against 8 + 4 RAD_DV),
+// and the three terms of the weights sit side by side in the 32 operand columns, so three instructions per k block
+// form all nine term products; the column groups are added once at the end.  Running sums are folded into a second
+// accumulator every RAD_MM_FOLD columns.
+__device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf16* ws) {
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, col = lane & 31;
+  rad_bf16x8 a[RAD_RB][RAD_NKB];
+#pragma unroll
+  for (int r = 0; r < RAD_RB; r++) {
+    i64 i = r * 32 + col;
+    if (i >= S.rows_avail) i = S.rows_avail - 1;
+#pragma unroll
+    for (int kb = 0; kb < RAD_NKB; kb++) a[r][kb] = *reinterpret_cast<const rad_bf16x8*>(S.xa + i * RAD_SLOTS + kb * 16 + 8 * half);
+  }
+  rad_f32x16 acc[RAD_RB], tot[RAD_RB];
+#pragma unroll
+  for (int r = 0; r < RAD_RB; r++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[r][v] = tot[r][v] = 0.f;
+
+  const i64 jbeg = S.jbeg, jend = S.jend;
+  constexpr int CH = RAD_NKB * 2 * RAD_TJ;  // 16-byte chunks of the slot vectors of a tile
+  constexpr int NPF = (CH + RAD_BLOCK - 1) / RAD_BLOCK;
+  constexpr int CW = RAD_TJ * 4;            // 16-byte chunks of the weights of a tile (64 bytes per column)
+  constexpr int NPW = (CW + RAD_BLOCK - 1) / RAD_BLOCK;
+  uint4 pf[NPF], pfw[NPW];
+  const __bf16* bwm = reinterpret_cast<const __bf16*>(S.bw);
+  auto prefetch = [&](i64 j0) {
+    const uint4* src = reinterpret_cast<const uint4*>(S.yb + (j0 / RAD_TJ) * (RAD_NKB * 2 * RAD_TJ * 8));
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * RAD_BLOCK;
+      pf[u] = e < CH ? src[e] : make_uint4(0u, 0u, 0u, 0u);
+    }
+    const uint4* wsrc = reinterpret_cast<const uint4*>(bwm + j0 * 32);  // padded to whole tiles
+#pragma unroll
+    for (int u = 0; u < NPW; u++) {
+      const int e = tid + u * RAD_BLOCK;
+      pfw[u] = e < CW ? wsrc[e] : make_uint4(0u, 0u, 0u, 0u);
+    }
+  };
+  if (jbeg < jend) prefetch(jbeg);
+  i64 since_fold = 0;
+  for (i64 j0 = jbeg; j0 < jend; j0 += RAD_TJ) {
+    __syncthreads();  // the previous tile has been consumed by every wavefront
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * RAD_BLOCK;
+      if (e < CH) reinterpret_cast<uint4*>(ys)[e] = pf[u];
+    }
+#pragma unroll
+    for (int u = 0; u < NPW; u++) {
+      const int e = tid + u * RAD_BLOCK;
+      if (e < CW) reinterpret_cast<uint4*>(ws)[e] = pfw[u];
+    }
+    __syncthreads();
+    if (j0 + RAD_TJ < jend) prefetch(j0 + RAD_TJ);
+#pragma unroll
+    for (int sub = 0; sub < RAD_NSUB; sub++) {
+      const int c = sub * 32 + col;
+      rad_bf16x8 b[RAD_NKB], wk[2];
+#pragma unroll
+      for (int kb = 0; kb < RAD_NKB; kb++) b[kb] = *reinterpret_cast<const rad_bf16x8*>(ys + ((kb * 2 + half) * RAD_TJ + c) * 8);
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++) wk[kb] = *reinterpret_cast<const rad_bf16x8*>(ws + (((sub * 2 + kb) * 2 + half) * 32 + col) * 8);
+#pragma unroll
+      for (int r = 0; r < RAD_RB; r++) {
+        rad_f32x16 z;
+#pragma unroll
+        for (int v = 0; v < 16; v++) z[v] = 0.f;
+        // transposed: z[v] = exponent of (row l % 32, column 8 (v / 4) + 4 (l / 32) + v % 4 of the sub-tile)
+#pragma unroll
+        for (int kb = 0; kb < RAD_NKB; kb++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[kb], a[r][kb], z, 0, 0, 0);
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+          unsigned hb[8], mb[8], lb[8];
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const float x = __builtin_amdgcn_exp2f(z[8 * kb + e]);
+            hb[e] = __float_as_uint(x);
+            const float r1 = x - __uint_as_float(hb[e] & 0xffff0000u);   // exact
+            mb[e] = __float_as_uint(r1);
+            const float r2 = r1 - __uint_as_float(mb[e] & 0xffff0000u);  // exact, at most 8 significant bits
+            lb[e] = __float_as_uint(r2);
+          }
+          // pack the high halves of two floats into one register: truncated bfloat16 terms
+          uint4 ph, pm, pl;
+          unsigned* php = reinterpret_cast<unsigned*>(&ph);
+          unsigned* pmp = reinterpret_cast<unsigned*>(&pm);
+          unsigned* plp = reinterpret_cast<unsigned*>(&pl);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            php[e] = __builtin_amdgcn_perm(hb[2 * e + 1], hb[2 * e], 0x07060302u);
+            pmp[e] = __builtin_amdgcn_perm(mb[2 * e + 1], mb[2 * e], 0x07060302u);
+            plp[e] = __builtin_amdgcn_perm(lb[2 * e + 1], lb[2 * e], 0x07060302u);
+          }
+          const rad_bf16x8 kh = __builtin_bit_cast(rad_bf16x8, ph), km = __builtin_bit_cast(rad_bf16x8, pm),
+                           kl = __builtin_bit_cast(rad_bf16x8, pl);
+          // smallest terms first
+          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kl, wk[kb], acc[r], 0, 0, 0);
+          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(km, wk[kb], acc[r], 0, 0, 0);
+          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, wk[kb], acc[r], 0, 0, 0);
+        }
+      }
+    }
+    since_fold += RAD_TJ;
+    if (since_fold >= RAD_MM_FOLD) {
+      since_fold = 0;
+#pragma unroll
+      for (int r = 0; r < RAD_RB; r++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          tot[r][v] += acc[r][v];
+          acc[r][v] = 0.f;
+        }
+    }
+  }
+  // lane l holds operand column l % 32 of rows 8 (v / 4) + 4 (l / 32) + v % 4: the three column groups
+  // (terms of the weights) are added with shuffles, lanes d < RAD_DV store
+#pragma unroll
+  for (int r = 0; r < RAD_RB; r++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const float s0 = tot[r][v] + acc[r][v];
+      // (smallest group first)
+      const float s = (__shfl(s0, lane + 2 * RAD_DV) + __shfl(s0, lane + RAD_DV)) + s0;
+      const i64 i = r * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+      if (col < RAD_DV && i < S.rows_store) S.part[i * RAD_DV + col] = s;
+    }
+}
+#endif
+
 #if !RAD_RANGES
 extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad_main(const RadParams P) {
   if (P.scal[2] != 1u) return;
   __shared__ __attribute__((aligned(16))) __bf16 ys[RAD_NKB * 2 * RAD_TJ * 8];  // [kb][half][col][8]
-#if !RAD_FOLD
+#if RAD_MM
+  __shared__ __attribute__((aligned(16))) __bf16 ws[RAD_TJ * 32];  // [sub-tile][k block][half][operand column][8]
+#elif !RAD_FOLD
   __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_DV];
 #else
   float* bs = nullptr;
@@ -540,7 +714,11 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
   S.rows_store = row0 < P.nx ? P.nx - row0 : 0;
   S.pos_tiles = RAD_FOLD ? keops_uniform((i64)P.scal[3]) : 0;  // tiles of columns with non-negative weights come first
   S.all_tiles = ncols / RAD_TJ;
+#if RAD_MM
+  rad_sweep_mm(S, ys, ws);
+#else
   rad_sweep(S, ys, bs);
+#endif
 }
 #endif
 

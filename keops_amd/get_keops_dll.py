@@ -917,8 +917,11 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
         return None, None
     # output rows per wavefront (32-row blocks) and wavefronts per workgroup: the accumulators (16 per block and
     # accumulated component) live in registers
-    rb = 2 if Dv <= config.radial_rb2_max_dv else 1
-    tj = (128 if Dv <= 2 else 512) if config.radial_tile_j == "auto" else int(config.radial_tile_j)
+    # from config.radial_mm_min_dv accumulated components on, the weighted sum runs on the matrix cores too (the three
+    # bfloat16 terms of the weights side by side in the 32 operand columns): 16 accumulators per block of 32 rows
+    mm = int(config.radial_mm_min_dv <= Dv and 3 * Dv <= 32 and not rows_per_block)
+    rb = (config.radial_mm_rb if mm else 2) if (mm or Dv <= config.radial_rb2_max_dv) else 1
+    tj = ((256 if mm else 128 if Dv <= 2 else 512) if config.radial_tile_j == "auto" else int(config.radial_tile_j))
     if tj % 32 or not 32 <= tj <= 1024:
         raise ValueError("[KeOps] KEOPS_AMD_RADIAL_TJ must be a multiple of 32 between 32 and 1024")
     waves = 8
@@ -954,11 +957,11 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     ca, cd, co = VarLayout.table(wl.colvars)
     ra, rd, ro = VarLayout.table(al.rowvars)
     # a scalar weight and no difference factor: the weight joins the exponent, columns are partitioned by its sign
-    fold = int(config.radial_fold and dimw == 1 and not diff and not rows_per_block)
-    meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
+    fold = int(config.radial_fold and dimw == 1 and not diff and not rows_per_block and not mm)
+    meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
                 rad_yarg=y.ind, rad_fold=fold, rad_tj=tj)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
-    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
+    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
                 RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit)!r}f",
                 RAD_NCOLVARS=len(wl.colvars), RAD_DIMY=wl.dimy, RAD_NROWVARS=len(al.rowvars), RAD_DIMX=al.dimx)
     src += [f"#define {k} {v}" for k, v in defs.items()]
@@ -1013,7 +1016,8 @@ def get_keops_dll(
         rows_hint = nx if nx < 64 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
            use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs),
-           binder.templates_digest(), bool(config.radial), bool(config.radial_fold), bool(config.radial_ranges), bool(use_half))
+           binder.templates_digest(), bool(config.radial), bool(config.radial_fold), bool(config.radial_ranges), int(config.radial_mm_min_dv),
+           int(config.radial_mm_rb), bool(use_half))
     with _lock:
         hit = _cache.get(key)
     if hit is not None:

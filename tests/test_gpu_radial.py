@@ -32,7 +32,7 @@ def _last_meta(key):
 
 
 @pytest.mark.parametrize("D,Dv,M,N", [(3, 1, 30011, 30500), (3, 8, 20000, 21000), (3, 2, 300000, 1001), (5, 3, 17000, 23001),
-                                      (8, 1, 16000, 18000), (2, 4, 33333, 10001)])
+                                      (8, 1, 16000, 18000), (2, 4, 33333, 10001), (6, 7, 18011, 19003)])
 def test_gaussian_sums_with_matrix_core_exponents_vs_oracle(D, Dv, M, N):
     rng = np.random.default_rng(100 * D + Dv)
     x = rng.standard_normal((M, D)).astype(np.float32)
@@ -42,6 +42,8 @@ def test_gaussian_sums_with_matrix_core_exponents_vs_oracle(D, Dv, M, N):
     dev = to_dev(x, y, b, g)
     got = _genred(D, Dv)(*dev)
     assert _last_meta("radial") == "1"
+    # from seven components on, the weighted sum runs on the matrix cores too (three-term operands)
+    assert _last_meta("rad_mm") == ("1" if Dv >= 7 else "0")
     rows = np.sort(rng.choice(M, 1500, replace=False)).astype(np.int64)
     ref = cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
     scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, Dv, rows=rows)
@@ -176,10 +178,11 @@ def test_matrix_core_exponents_under_graph_capture():
         assert torch.equal(got, conv(x, y, b, g))
 
 
-@pytest.mark.parametrize("D", [3, 2])
+@pytest.mark.parametrize("D", [3, 2, 7])
 def test_gradients_wrt_points_and_weights_with_matrix_core_exponents(D):
     """Backward pass of the Gaussian kernel sum: the gradients with respect to x, y and b are again Gaussian sums
-    (with a difference factor for the points) and take the same path; against the oracle's gradient body."""
+    (with a difference factor for the points) and take the same path; against the oracle's gradient body.  (D = 7:
+    eight sums per row, which the variant with the weighted sum on the matrix cores accumulates.)"""
     from keops_amd import keops_io
 
     M, N = 24000, 26000
