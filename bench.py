@@ -25,6 +25,7 @@ if ROOT not in sys.path:
 PEAK_FP32_VECTOR_TFLOPS = 157.3
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_BF16_MFMA_TFLOPS = 2500.0
+PEAK_INT8_MFMA_TOPS = 5000.0
 # reference number for this metric: PyKeOps Gaussian conv, M=N=1M, RTX 2080 Ti, 1.39 s
 # (reference benchmarks/README.md:14) -> 7.2e11 pairs/s
 PUBLISHED_PAIRS_PER_S = 1e12 / 1.39
@@ -35,8 +36,8 @@ MEASURED_TRAFFIC_BYTES = {
     # profiles/keops_rad_main__gauss_1m_dv1.md: FETCH_SIZE 2302881 KiB x 2.0 (copy calibration) + WRITE_SIZE 11718.75 KiB
     # (column slot vectors re-read by every row block, 98 % from L2 / Infinity Cache; 52 GB/s, not the limiter)
     "gauss_1m_dv1": int((2302881 * 2.0 + 11718.75) * 1024),
-    # profiles/keops_knn_filter__knn_d64.md: dominant kernel keops_knn_filter
-    "knn_d64": int(2 * (391283 * 2.0 + 43486) * 1024),
+    # profiles/keops_knn_filter_i8__knn_d64.md: dominant kernel keops_knn_filter_i8 (two launches per call)
+    "knn_d64": int(2 * (200093 * 2.0 + 45852) * 1024),
     # profiles/keops_chk_final__laplace_d256.md
     "laplace_d256": int((5045781 * 2.0 + 672429) * 1024),
     # profiles/keops_chk_softmax__softmax_d64.md
@@ -58,7 +59,8 @@ WORKLOADS = {
     "gauss_10k": ("Gaussian kernel sum 1e4 x 1e4, D=3, Dv=1, float32 (benchmark configuration 1)", 14, "valu"),
     "gauss_100k": ("Gaussian kernel sum 1e5 x 1e5, D=3, Dv=1, float32 (reference benchmarks/README.md:13)", 14, "valu"),
     # 2*D flop of the <x,y> contraction per pair (the matrix-core work); filter and re-rank are not counted
-    "knn_d64": ("KMin_ArgKMin K=10, 1e5 queries x 1e6 references, D=64 (benchmark configuration 3)", 128, "mfma"),
+    # (the filter runs on signed bytes, v_mfma_i32_32x32x32_i8: the line is priced against the int8 matrix peak)
+    "knn_d64": ("KMin_ArgKMin K=10, 1e5 queries x 1e6 references, D=64 (benchmark configuration 3)", 128, "mfma8"),
     # nearest neighbours among MNIST-sized rows (784 components): squared distances on the chunked matrix-core
     # sweep + exact re-rank (2*D flop of the contraction per pair), Manhattan distances on the vector-ALU chunked
     # variant of the general-purpose kernel (subtract, absolute value, add per component)
@@ -249,6 +251,7 @@ def calibration(mfma):
     simds, clock = 4 * cus, 2.4e9
     rows = []
     kinds = [(3, "v_mfma_f32_32x32x16_bf16", (1, 2, 4)), (4, "v_mfma_f32_32x32x16_f16", (1, 2, 4)),
+             (6, "v_mfma_i32_32x32x32_i8", (1, 2, 4)),
              (5, "two chains of v_mfma_f32_32x32x16_bf16 with `chains` v_fmac_f32 after every matrix instruction", (0, 1, 2, 4, 8))] if mfma else [
         (0, "v_fmac_f32 chains", (1, 2, 4, 8)), (1, "Gaussian pair mix with v_exp_f32 (9 instr)", (1, 2, 4, 8)),
         (2, "Gaussian pair mix without v_exp_f32 (8 instr)", (1, 2, 4, 8))]
@@ -256,14 +259,15 @@ def calibration(mfma):
         for chains in chain_set:
             for waves in (1, 2, 4):
                 blocks = cus * waves  # one workgroup = 4 wavefronts = one per SIMD of a CU
-                iters = 200_000 // chains if kind < 3 else (100_000 // chains if kind < 5 else 50_000)
+                iters = 200_000 // chains if kind < 3 else (100_000 // chains if kind != 5 else 50_000)
                 ms, ipw = binder.calibrate(kind, chains, blocks, iters)
                 total = ipw * blocks * 4  # wavefront instructions
                 per_cycle = total / (ms * 1e-3) / simds / clock
                 row = dict(kind=label, chains=chains, waves_per_simd=waves, ms=round(ms, 3),
                            wave_instr_per_cycle_per_simd_at_2p4GHz=round(per_cycle, 4))
                 if kind >= 3:
-                    row["PFLOP_per_s"] = round(total * 32 * 32 * 16 * 2 / (ms * 1e-3) / 1e15, 3)
+                    # (kind 6: integer operations, 32 x 32 x 32 per instruction)
+                    row["PFLOP_per_s"] = round(total * 32 * 32 * (32 if kind == 6 else 16) * 2 / (ms * 1e-3) / 1e15, 3)
                 else:
                     row["lane_instr_per_s"] = total * 64 / (ms * 1e-3)
                 rows.append(row)
@@ -331,12 +335,18 @@ def main():
 
     kms = sum(kernel_ms) / len(kernel_ms)
     achieved = pairs * flop_per_pair / (kms * 1e-3) / 1e12
-    peak = {"valu": PEAK_FP32_VECTOR_TFLOPS, "mfma": PEAK_BF16_MFMA_TFLOPS, "mfma32": PEAK_FP32_MFMA_TFLOPS}[bound]
+    peak = {"valu": PEAK_FP32_VECTOR_TFLOPS, "mfma": PEAK_BF16_MFMA_TFLOPS, "mfma32": PEAK_FP32_MFMA_TFLOPS,
+            "mfma8": PEAK_INT8_MFMA_TOPS}[bound]
     note = {"valu": "peak is the packed-FP32 vector figure; packed FP32 instructions are disabled in this build. "
                     "Gaussian sums take their exponents from the matrix cores when the device-side check allows it "
                     "(kernels/keops_radial_mfma.h): the vector ALU then issues v_exp_f32 + one fma per pair and output "
                     "component, and the algorithmic flop of the exponent are not vector-ALU work any more",
-            "mfma": "peak is the dense bf16 matrix figure", "mfma32": "peak is the dense fp32 matrix figure"}[bound]
+            "mfma": "peak is the dense bf16 matrix figure", "mfma32": "peak is the dense fp32 matrix figure",
+            "mfma8": "peak is the dense int8 matrix figure (5.0 POP/s): the fixed-threshold filter runs on signed bytes when "
+                     "the device finds the quantisation slack small against the search radii (kernels/keops_knn_mfma.h, "
+                     "keops_knn_filter_i8); with KEOPS_AMD_KNN_I8=0 the same call runs its filter in bfloat16 "
+                     "(12.7 ms, 0.40 of the 2.5 PFLOP/s bf16 peak).  `achieved` counts the 2*D operations of <x,y> per "
+                     "pair once; sampling pass and exact re-rank are not counted"}[bound]
     out = {
         "metric": "pair interactions/sec (M*N/s), 1e6x1e6 D=3 Gauss sum" if args.workload == "gauss_1m_dv1"
         else "pair interactions/sec (M*N/s)",

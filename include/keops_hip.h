@@ -159,13 +159,16 @@ size_t keops_hip_noalloc_scratch_bytes(void);
 int keops_hip_ranges_status(void* module, unsigned* status);
 
 /*
- * Which kernel family served the module's last launch; waits for that launch.  Modules of Gaussian-type sums carry
- * two families (meta key radial=1): exponents from the matrix cores, chosen on the device when the kernel is not
- * too narrow for the cloud (for block-sparse launches: for every row range), and the general-purpose kernel from
- * exact differences otherwise.  *taken: 1 the matrix-core family ran, 0 the general-purpose one (or the module has
- * one family only, or the launch was too small to try).  No counterpart in the reference.
+ * Which of a module's two kernel families served its last launch; waits for that launch.  Two kinds of module
+ * choose on the device, per launch, without host synchronisation: (1) Gaussian-type sums (meta key radial=1):
+ * exponents from the matrix cores when the kernel is not too narrow for the cloud (block-sparse launches: for every
+ * row range), the general-purpose kernel from exact differences otherwise; (2) K-nearest-neighbour modules with
+ * knn_i8=1: the fixed-threshold filter on signed bytes when the quantisation slack is small against the search
+ * radii, the bfloat16 filter otherwise (the returned neighbours are the same either way).  *taken: 1 the first of
+ * the two ran, 0 the other one (or the module has one family only, or the launch was too small to try).
+ * No counterpart in the reference.
  */
-int keops_hip_radial_status(void* module, unsigned* taken);
+int keops_hip_path_status(void* module, unsigned* taken);
 
 /*
  * Loop-only calibration of the instruction issue rates the roofline fractions are held against: runs a grid of
@@ -175,7 +178,8 @@ int keops_hip_radial_status(void* module, unsigned* taken);
  *   mul, 2 fma, mul, v_exp_f32, fma); kind 2: the same without v_exp_f32; kind 3: v_mfma_f32_32x32x16_bf16
  *   (4 per chain and round); kind 4: v_mfma_f32_32x32x16_f16; kind 5: two chains of the bf16 instruction (8 per round)
  *   with `chains` independent v_fmac_f32 after every matrix instruction (what fits beside a saturated matrix pipe).
- *   chains: 1, 2, 4, 8 (kinds 0-2), 1, 2, 4 (kinds 3, 4) or 0, 1, 2, 4, 8 (kind 5).
+ *   chains: 1, 2, 4, 8 (kinds 0-2), 1, 2, 4 (kinds 3, 4, 6) or 0, 1, 2, 4, 8 (kind 5); kind 6: v_mfma_i32_32x32x32_i8
+ *   (4 per chain and round).
  * Measurement aid without counterpart in the reference; used by bench.py --valu-calibration / --mfma-calibration.
  */
 int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave);

@@ -56,7 +56,7 @@ def lib():
         L.keops_hip_noalloc_scratch_bytes.restype = ctypes.c_size_t
         L.keops_hip_calibrate.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 2
         L.keops_hip_ranges_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint)]
-        L.keops_hip_radial_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint)]
+        L.keops_hip_path_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint)]
         _lib = L
     return _lib
 
@@ -137,11 +137,12 @@ class Module:
             raise KeOpsHipError(last_error())
         return int(st.value)
 
-    def radial_status(self):
-        """1 when the matrix-core exponent kernels served the last launch, 0 when the general-purpose kernel did
-        (keops_hip_radial_status of include/keops_hip.h); waits for that launch."""
+    def path_status(self):
+        """1 when the first of the module's two kernel families served the last launch (matrix-core exponents of a
+        Gaussian-type sum, byte filter of a K-nearest-neighbour search), 0 when the other one did
+        (keops_hip_path_status of include/keops_hip.h); waits for that launch."""
         st = ctypes.c_uint(0)
-        if lib().keops_hip_radial_status(self.handle, ctypes.byref(st)) != 0:
+        if lib().keops_hip_path_status(self.handle, ctypes.byref(st)) != 0:
             raise KeOpsHipError(last_error())
         return int(st.value)
 

@@ -96,6 +96,7 @@ knn_min_work = int(os.environ.get("KEOPS_AMD_KNN_MIN_WORK", 1 << 32))      # sma
 knn_batch_max = int(os.environ.get("KEOPS_AMD_KNN_BATCH_MAX", 64))    # batched KNN: at most this many batches are served one by one
 knn_batch_min_work = int(os.environ.get("KEOPS_AMD_KNN_BATCH_MIN_WORK", 1 << 33))  # ... of at least this many pairs x max(D, 8) each
 knn_lds_budget = 150 * 1024                                        # LDS bytes a KNN workgroup may use (160 KB per CU)
+knn_i8 = os.environ.get("KEOPS_AMD_KNN_I8", "1") != "0"           # fixed-threshold filter on signed bytes (v_mfma_i32_32x32x32_i8) when its slack allows
 knn_qsets = int(os.environ.get("KEOPS_AMD_KNN_QSETS", 1))          # 32-query operand sets per wavefront (<= 2)
 
 

@@ -800,6 +800,8 @@ struct KnnHeader {
   void* overflow;
   int64_t logcap;
   int32_t stage, pad_;
+  // filter on signed bytes (modules with knn_i8=1, two-phase launches; null otherwise)
+  void *xq8, *yq8, *ykey_i, *xnorm_i, *xres, *thr_i, *scal;
 };
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -903,6 +905,14 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   const size_t o_yhs = take((size_t)nsample * RW * 2), o_ykeys = take((size_t)nsample * 4);
   const size_t o_thr = take((size_t)nq * 4), o_flag = take(256);
   const size_t o_logcount = take((size_t)(two_phase ? nlogs : 0) * 4), o_log = take((size_t)(two_phase ? nlogs : 0) * logcap * 8);
+  // the filter also runs on signed bytes (twice the matrix rate, half the staged bytes) when the device finds its
+  // slack small against the search radii
+  const bool i8 = two_phase && m.meta_int("knn_i8", 0) != 0;
+  const int64_t DP8 = (D + 31) / 32 * 32;
+  const size_t o_xq8 = take(i8 ? (size_t)nq * DP8 : 0), o_yq8 = take(i8 ? (size_t)nr * DP8 : 0);
+  const size_t o_ykeyi = take(i8 ? (size_t)nr * 4 : 0), o_xnormi = take(i8 ? (size_t)nq * 4 : 0), o_thri = take(i8 ? (size_t)nq * 4 : 0);
+  const size_t o_xres = take(i8 ? (size_t)nq * 4 : 0);
+  const size_t o_scal = take(64);
   if (int rc = m.partial.reserve(off)) return rc;
   char* ws = (char*)m.partial.ptr;
   struct Packed { KnnHeader h; int64_t extra[4]; } p{};
@@ -911,6 +921,11 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   h.xh = ws + o_xh; h.yh = ws + o_yh; h.xkey = ws + o_xkey; h.ykey = ws + o_ykey; h.colsum = ws + o_colsum; h.colpart = ws + o_colpart;
   h.plist_d = ws + o_pd; h.plist_i = ws + o_pi; h.out = out; h.ref_step = 1;
   h.thr = ws + o_thr; h.log = ws + o_log; h.logcount = ws + o_logcount; h.overflow = ws + o_flag; h.logcap = logcap;
+  if (i8) {
+    h.xq8 = ws + o_xq8; h.yq8 = ws + o_yq8; h.ykey_i = ws + o_ykeyi; h.xnorm_i = ws + o_xnormi; h.xres = ws + o_xres;
+    h.thr_i = ws + o_thri; h.scal = ws + o_scal;
+  }
+  m.last_guard = i8 ? (const unsigned*)(ws + o_scal) + 3 : nullptr;
   const size_t HS = sizeof(KnnHeader);
   auto run = [&](const char* k, unsigned gx, unsigned gy, unsigned block, size_t size) {
     return launch_raw(m, k, gx, gy, block, &p, size, stream);
@@ -923,6 +938,12 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
   if (int rc = run("keops_knn_prep", (unsigned)((nq * lpr + 255) / 256), 1, 256, with_int(0))) return rc;
   if (int rc = run("keops_knn_prep", (unsigned)((nr * lpr + 255) / 256), 1, 256, with_int(1))) return rc;
+  if (i8) {
+    // (after both bf16 passes: they find the largest centred component, which sets the quantisation step)
+    const int64_t lpr8 = DP8 / 4 <= 8 ? 8 : (DP8 / 4 <= 16 ? 16 : (DP8 / 4 <= 32 ? 32 : 64));
+    if (int rc = run("keops_knn_quant", (unsigned)((nq * lpr8 + 255) / 256), 1, 256, with_int(0))) return rc;
+    if (int rc = run("keops_knn_quant", (unsigned)((nr * lpr8 + 255) / 256), 1, 256, with_int(1))) return rc;
+  }
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
 
   auto adaptive = [&](const char* kernel, int64_t refs, void* yh, void* ykey, int step, int64_t slabs, int64_t len) -> int {
@@ -948,11 +969,16 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
     // Staged: every 4th slab first, thresholds refined from its replay, then the other slabs.
     h.nr = nr; h.yh = ws + o_yh; h.ykey = ws + o_ykey; h.ref_step = 1; h.nslabs = (int32_t)f_slabs; h.slab_len = f_len;
     h.stage = staged ? 1 : 0;
+    // (one of the two filters returns at once: the choice was made on the device by keops_knn_thresholds)
+    if (i8)
+      if (int rc = run("keops_knn_filter_i8", (unsigned)f_qblocks, (unsigned)fa_slabs, (unsigned)(64 * FW), HS)) return rc;
     if (int rc = run("keops_knn_filter", (unsigned)f_qblocks, (unsigned)fa_slabs, (unsigned)(64 * FW), HS)) return rc;
     if (int rc = run("keops_knn_rerank", (unsigned)(f_qblocks * fa_slabs * FW), 1, 64, with_int((int)f_qblocks))) return rc;
     if (staged) {
       if (int rc = run("keops_knn_thresholds", (unsigned)((nq + 255) / 256), 1, 256, with_2int(1, (int)fa_slabs))) return rc;
       h.stage = 2;
+      if (i8)
+        if (int rc = run("keops_knn_filter_i8", (unsigned)f_qblocks, (unsigned)fb_slabs, (unsigned)(64 * FW), HS)) return rc;
       if (int rc = run("keops_knn_filter", (unsigned)f_qblocks, (unsigned)fb_slabs, (unsigned)(64 * FW), HS)) return rc;
       if (int rc = run("keops_knn_rerank", (unsigned)(f_qblocks * fb_slabs * FW), 1, 64, with_int((int)f_qblocks))) return rc;
       h.stage = 0;
@@ -1847,8 +1873,8 @@ int keops_hip_launch_noalloc(void* module, int64_t nx, int64_t ny, int tagI, int
   return rc;
 }
 
-int keops_hip_radial_status(void* module, unsigned* taken) {
-  if (!module || !taken) return fail(-1, "keops_hip_radial_status: null argument");
+int keops_hip_path_status(void* module, unsigned* taken) {
+  if (!module || !taken) return fail(-1, "keops_hip_path_status: null argument");
   Module& m = *static_cast<Module*>(module);
   *taken = 0u;
   if (!m.last_guard) return 0;

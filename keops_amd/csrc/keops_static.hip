@@ -283,6 +283,42 @@ static __global__ void __launch_bounds__(256) keops_mfma_loop(float* out, int it
   out[(size_t)blockIdx.x * 256 + threadIdx.x] = r;
 }
 
+
+typedef int keops_i32x16 __attribute__((ext_vector_type(16)));
+typedef int keops_i32x4 __attribute__((ext_vector_type(4)));
+
+// `iters` rounds of CHAINS independent v_mfma_i32_32x32x32_i8 accumulation chains per wavefront (4 instructions per
+// chain and round) on random signed bytes
+template <int CHAINS>
+static __global__ void __launch_bounds__(256) keops_mfma_i8_loop(float* out, int iters) {
+  keops_i32x16 acc[CHAINS];
+  keops_i32x4 a, b;
+  unsigned h = 0x9e3779b9u * (threadIdx.x + 1u);
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    h = h * 1664525u + 1013904223u;
+    a[e] = (int)h;
+    h = h * 1664525u + 1013904223u;
+    b[e] = (int)h;
+  }
+#pragma unroll
+  for (int k = 0; k < CHAINS; k++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[k][e] = 0;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+#pragma unroll
+      for (int k = 0; k < CHAINS; k++) acc[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[k], 0, 0, 0);
+  }
+  int r = 0;
+#pragma unroll
+  for (int k = 0; k < CHAINS; k++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) r += acc[k][e];
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = (float)r;
+}
+
 // `iters` rounds of 8 v_mfma_f32_32x32x16_bf16 (two dependent chains of 4, the shape of the K-nearest-neighbour
 // filter) with NV independent v_fmac_f32 between them: how much vector work fits beside a saturated matrix pipe
 template <int NV>
@@ -330,7 +366,8 @@ static __global__ void __launch_bounds__(256) keops_mix_loop(float* out, int ite
 }
 
 // Runs one calibration loop on `stream`: grid of `blocks` workgroups of 256 lanes (4 wavefronts), `iters` rounds.
-// kind 0/1/2: vector loop with MIX = kind; kind 3 / 4: matrix loop on bf16 / f16 operands; kind 5: 8 bf16 matrix
+// kind 0/1/2: vector loop with MIX = kind; kind 3 / 4: matrix loop on bf16 / f16 operands; kind 6: on signed bytes
+// (v_mfma_i32_32x32x32_i8); kind 5: 8 bf16 matrix
 // instructions per round with `chains` v_fmac_f32 after each of them (0, 1, 2, 4, 8).  chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
 // instr_per_lane receives the number of counted instructions one wavefront issues (vector: per lane = per wavefront
 // instruction count; matrix: v_mfma instructions).  out must hold blocks * 256 floats.
@@ -360,6 +397,12 @@ int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* o
     else if (chains == 4) MFMA_CASE(4);
     else return (int)hipErrorInvalidValue;
 #undef MFMA_CASE
+  } else if (kind == 6) {
+    *instr_per_wave = 4.0 * chains * (double)iters;
+    if (chains == 1) hipLaunchKernelGGL((keops_mfma_i8_loop<1>), g, b, 0, s, out, iters);
+    else if (chains == 2) hipLaunchKernelGGL((keops_mfma_i8_loop<2>), g, b, 0, s, out, iters);
+    else if (chains == 4) hipLaunchKernelGGL((keops_mfma_i8_loop<4>), g, b, 0, s, out, iters);
+    else return (int)hipErrorInvalidValue;
   } else if (kind == 5) {
     // chains = vector instructions per matrix instruction: 0, 1, 2, 4, 8
     *instr_per_wave = 8.0 * (double)iters;

@@ -64,6 +64,11 @@ static_assert(KNN_FQSETS <= 4 && KNN_SQSETS <= 2, "a lane owns the lists of at m
 #ifndef KNN_FTJ
 #define KNN_FTJ KNN_TJ                 // reference rows per staged tile of the fixed-threshold filter
 #endif
+#ifndef KNN_I8
+#define KNN_I8 0                       // 1: the fixed-threshold filter also exists on signed bytes (keops_knn_filter_i8)
+#endif
+#define KNN_DP8 ((KNN_D + 31) / 32 * 32)  // bytes per quantised row: whole k blocks of v_mfma_i32_32x32x32_i8
+#define KNN_I8_ETA 0.08f               // the byte filter is used when its slack is below this fraction of the search radius
 #define KNN_KB (KNN_DPAD / 16)         // 16-wide k blocks
 #define KNN_RW (KNN_DPAD * (1 + KNN_SPLIT))  // bf16 elements per stored row: [hi] or [hi | lo]
 #define KNN_STRIDE (KNN_RW * 2 + 16)   // bytes per staged reference row (16 B pad: conflict-free b128 reads)
@@ -104,6 +109,16 @@ struct KnnParams {
   i64 logcap;
   int stage;             // filter / replay: which slabs this launch covers (knn_stage_slab)
   int pad_;
+  // filter on signed bytes (KNN_I8; null otherwise)
+  signed char* xq8;      // [nq][KNN_DP8] minus the quantised centred queries
+  signed char* yq8;      // [nr][KNN_DP8] quantised centred references
+  int* ykey_i;           // [nr] floor(|y~|^2 / 2) in quantisation steps
+  int* xnorm_i;          // [nq] |x~|^2
+  float* xres;           // [nq] distance between a centred query and its quantised copy (rounded up)
+  int* thr_i;            // [nq] integer thresholds
+  unsigned* scal;        // [0]: bit pattern of the largest |centred component|; [1]: queries for which the byte filter
+                         // would be too loose; [2]: bit pattern of the largest distance between a centred reference
+                         // and its quantised copy; [3]: 1 when the byte filter served the call (written at the end)
 #if KNN_RANGES
   KeopsRangeTables rt;   // block-sparse launches: workgroup table and reduced-index ranges (keops_knn_main only)
 #endif
@@ -152,6 +167,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_colsum(const KnnPara
 
 extern "C" __global__ void __launch_bounds__(256) keops_knn_colsum_final(const KnnParams P, int nparts) {
   __shared__ float part[256];
+  if (KNN_I8 && P.scal != nullptr && threadIdx.x < 4) P.scal[threadIdx.x] = 0u;
   constexpr int RG = 256 / KNN_CW;
   const int cw = threadIdx.x % KNN_CW, rg = threadIdx.x / KNN_CW;
   for (int c0 = 0; c0 < KNN_DPAD; c0 += KNN_CW) {
@@ -181,7 +197,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_prep(const KnnParams
   const int sub = threadIdx.x % KNN_LPR;
   const i64 row = ((i64)blockIdx.x * 256 + threadIdx.x) / KNN_LPR;
   const float inv = 1.0f / (float)P.nr;
-  float nrm = 0.f;
+  float nrm = 0.f, vmax = 0.f;
   const bool live = row < n && sub * 4 < KNN_DPAD;
   if (live) {
     knn_bf16x4 h, l;
@@ -190,6 +206,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_prep(const KnnParams
       const int c = sub * 4 + e;
       float v = 0.f;
       if (c < KNN_D) v = src[row * KNN_D + c] - P.colsum[c] * inv;
+      vmax = __builtin_fmaxf(vmax, __builtin_fabsf(v));
       h[e] = (__bf16)v;
       float r = (float)h[e];
       if (KNN_SPLIT) {
@@ -210,6 +227,14 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_prep(const KnnParams
 #pragma unroll
   for (int o = KNN_LPR / 2; o > 0; o >>= 1) nrm += __shfl_xor(nrm, o, KNN_LPR);
   if (live && sub == 0) key[row] = (1.0f - KNN_C) * nrm;
+  if (KNN_I8 && P.scal != nullptr) {
+    // largest centred component of both sets (a NaN never wins: the byte filter is then simply not exact about
+    // that row, as the bf16 one, and the exact re-rank decides); one atomic per wavefront
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) vmax = __builtin_fmaxf(vmax, __shfl_xor(vmax, o));
+    // (most wavefronts find the current maximum at least as large and skip the atomic)
+    if ((threadIdx.x & 63) == 0 && __float_as_uint(vmax) > *const_cast<volatile unsigned*>(P.scal)) atomicMax(P.scal, __float_as_uint(vmax));
+  }
 }
 
 // ---- exact re-rank ----------------------------------------------------------------------------
@@ -603,6 +628,218 @@ extern "C" __global__ void __launch_bounds__(64 * KNN_WAVES) keops_knn_main(cons
   knn_sweep<0, KNN_WAVES, KNN_QSETS>(P, ys, ykey_s, lv, li, owner, qq, qj);
 }
 
+#if KNN_I8 && !KNN_RANGES
+typedef int knn_i32x16 __attribute__((ext_vector_type(16)));
+typedef int knn_i32x4 __attribute__((ext_vector_type(4)));
+#ifndef KNN_I8_PAD
+#define KNN_I8_PAD 16
+#endif
+#define KNN_I8_STRIDE (KNN_DP8 + KNN_I8_PAD)   // bytes per staged byte row (padded against bank conflicts)
+#define KNN_I8_KB (KNN_DP8 / 32)       // 32-wide k blocks
+
+// Quantisation step of the byte filter: the largest centred component of both sets maps to 127.
+__device__ __forceinline__ float knn_i8_step(const KnnParams& P) {
+  return __builtin_fmaxf(__uint_as_float(P.scal[0]), 1e-30f) * (1.0f / 127.0f);
+}
+// The distance between two quantised points differs from the true one by at most the distances of the two points to
+// their quantised copies (triangle inequality): the query's own, the largest one among the references
+__device__ __forceinline__ float knn_i8_slack(const KnnParams& P, i64 q) { return P.xres[q] + __uint_as_float(P.scal[2]); }
+// true while the byte filter serves this call (few queries for which its slack is large against their search radius)
+__device__ __forceinline__ bool knn_i8_taken(const KnnParams& P) { return (i64)P.scal[1] * 8 <= P.nq; }
+
+// Rows as signed bytes: round((v - mean) / step), the queries negated, with the integer squared norms.  The metric is
+// exact on the quantised points (integer products), so the filter only needs the triangle inequality:
+// | |x - y| - step |x~ - y~| | <= slack.  which = 0: queries, 1: references; one row per group of KNN_LPR8 lanes.
+#define KNN_LPR8 (KNN_DP8 / 4 <= 8 ? 8 : (KNN_DP8 / 4 <= 16 ? 16 : (KNN_DP8 / 4 <= 32 ? 32 : 64)))
+extern "C" __global__ void __launch_bounds__(256) keops_knn_quant(const KnnParams P, int which) {
+  const i64 n = which ? P.nr : P.nq;
+  const float* src = which ? P.yr : P.xq;
+  signed char* dst = which ? P.yq8 : P.xq8;
+  const int sub = threadIdx.x % KNN_LPR8;
+  const i64 row = ((i64)blockIdx.x * 256 + threadIdx.x) / KNN_LPR8;
+  const float inv = 1.0f / (float)P.nr, step = knn_i8_step(P), rstep = 1.0f / step;
+  int nrm = 0;
+  float res2 = 0.f;
+  const bool live = row < n && sub * 4 < KNN_DP8;
+  if (live) {
+    unsigned packed = 0u;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const int c = sub * 4 + e;
+      int q = 0;
+      if (c < KNN_D) {
+        const float v = src[row * KNN_D + c] - P.colsum[c] * inv;
+        q = (int)__builtin_rintf(__builtin_fminf(__builtin_fmaxf(v * rstep, -127.0f), 127.0f));  // (NaN -> -127 -> a finite byte)
+        const float r = v - (float)q * step;
+        res2 = __builtin_fmaf(r, r, res2);
+      }
+      nrm += q * q;
+      packed |= ((unsigned)((which ? q : -q) & 0xff)) << (8 * e);
+    }
+    *reinterpret_cast<unsigned*>(dst + row * KNN_DP8 + sub * 4) = packed;
+  }
+#pragma unroll
+  for (int o = KNN_LPR8 / 2; o > 0; o >>= 1) {
+    nrm += __shfl_xor(nrm, o, KNN_LPR8);
+    res2 += __shfl_xor(res2, o, KNN_LPR8);
+  }
+  // distance to the quantised copy, rounded up (float32 evaluation of the sum; the centring itself is rounded to 2^-24
+  // of the uncentred component, counted as 2^-20 of the largest centred one per component)
+  const float res = __builtin_sqrtf(res2) * 1.00001f + 1.0e-6f * __builtin_sqrtf((float)KNN_D) * (127.0f * step);
+  if (live && sub == 0) {
+    if (which) P.ykey_i[row] = nrm >> 1;  // floor: never excludes a pair
+    else {
+      P.xnorm_i[row] = nrm;
+      P.xres[row] = res;
+    }
+  }
+  if (which) {
+    // largest one among the references (a NaN row is left out: its exact distances are NaN and never inserted)
+    float rmax = (live && res == res) ? res : 0.f;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) rmax = __builtin_fmaxf(rmax, __shfl_xor(rmax, o));
+    if ((threadIdx.x & 63) == 0 && __float_as_uint(rmax) > *const_cast<volatile unsigned*>(P.scal + 2)) atomicMax(P.scal + 2, __float_as_uint(rmax));
+  }
+}
+
+// Integer threshold of query q for the K-th distance bound tau (squared, already inflated for rounding): a pair
+// with |x - y|^2 <= tau has step |x~ - y~| <= sqrt(tau) + slack, i.e. |y~|^2 / 2 - <x~, y~> <= (R^2 - |x~|^2) / 2 with
+// R = (sqrt(tau) + slack) / step.
+__device__ __forceinline__ int knn_i8_threshold(const KnnParams& P, i64 q, float tau) {
+  const double R = ((double)__builtin_sqrtf(__builtin_fmaxf(tau, 0.f)) * 1.000001 + (double)knn_i8_slack(P, q)) / (double)knn_i8_step(P);
+  const double t = (R * R * 1.000001 - (double)P.xnorm_i[q]) * 0.5 + 1.0;
+  return t >= 1.0e9 ? 1000000000 : (t <= -1.0e9 ? -1000000000 : (int)t);  // (NaN: the last branch, 0 on this hardware)
+}
+
+// Fixed-threshold filter on signed bytes: the geometry, the logs and the replay of keops_knn_filter, with
+// v_mfma_i32_32x32x32_i8 (half as many matrix instructions and staged bytes per pair).  The accumulators start from
+// floor(|y~|^2 / 2), the B operands hold -x~: a lane's 16 results are |y~|^2 / 2 - <x~, y~> for 16 references.
+extern "C" __global__ void __launch_bounds__(64 * KNN_FWAVES) keops_knn_filter_i8(const KnnParams P) {
+  if (!knn_i8_taken(P)) return;
+  constexpr int WAVES = KNN_FWAVES, QSETS = KNN_FQSETS, TJ = KNN_FTJ;
+  constexpr int BLOCK = 64 * WAVES, QW = 32 * QSETS, QB = WAVES * QW;
+  __shared__ __attribute__((aligned(16))) unsigned char ys[TJ * KNN_I8_STRIDE];
+  __shared__ __attribute__((aligned(16))) int ykey_s[TJ];
+  __shared__ int qq[WAVES][64];
+  __shared__ int qj[WAVES][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+  const i64 qw0 = (i64)blockIdx.x * QB + (i64)wave * QW;
+  knn_i32x4 bq[QSETS][KNN_I8_KB];
+  int t[QSETS];
+#pragma unroll
+  for (int h = 0; h < QSETS; h++) {
+    i64 q = qw0 + h * 32 + col;
+    const bool valid = q < P.nq;
+    if (!valid) q = P.nq - 1;
+#pragma unroll
+    for (int kb = 0; kb < KNN_I8_KB; kb++) bq[h][kb] = *reinterpret_cast<const knn_i32x4*>(P.xq8 + q * KNN_DP8 + kb * 32 + 16 * half);
+    t[h] = valid ? P.thr_i[q] : -2147483647 - 1;
+  }
+  int qcount = 0;    // wave-uniform number of queued candidates
+  i64 logged = 0;    // wave-uniform number of entries already in this wavefront's log
+  const int slab = knn_stage_slab(P.stage, blockIdx.y);
+  const i64 logid = ((i64)slab * gridDim.x + blockIdx.x) * WAVES + wave;
+  int2* mylog = P.log + logid * P.logcap;
+  auto flush = [&](int nb) {
+    if (logged + nb <= P.logcap) {
+      if (lane < nb) mylog[logged + lane] = make_int2(qq[wave][lane], qj[wave][lane]);
+      logged += nb;
+    } else {
+      if (lane == 0) *P.overflow = 1;
+    }
+  };
+  const i64 jbeg = (i64)slab * P.slab_len, jend = keops_min(P.nr, jbeg + P.slab_len);
+  constexpr int CH = KNN_DP8 / 16;                       // 16-byte chunks per staged row
+  constexpr int NPF = (TJ * CH + BLOCK - 1) / BLOCK;
+  uint4 pf[NPF];
+  int pfkey = 1000000000;
+  auto prefetch = [&](i64 j0) {
+    const int n = (int)keops_min((i64)TJ, jend - j0);
+    const uint4* src = reinterpret_cast<const uint4*>(P.yq8 + j0 * KNN_DP8);
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * BLOCK;
+      pf[u] = (e < n * CH) ? src[e] : make_uint4(0u, 0u, 0u, 0u);
+    }
+    pfkey = (tid < n) ? P.ykey_i[j0 + tid] : 1000000000;  // padded rows never pass
+  };
+  static_assert(TJ <= BLOCK, "one key per thread");
+  const unsigned char* const abase = ys + col * KNN_I8_STRIDE + 16 * half;
+  const int* const kbase = ykey_s + 4 * half;
+  if (jbeg < jend) prefetch(jbeg);
+  for (i64 j0 = jbeg; j0 < jend; j0 += TJ) {
+    const int n = (int)keops_min((i64)TJ, jend - j0);
+    __syncthreads();  // every wavefront is done with the previous tile
+#pragma unroll
+    for (int u = 0; u < NPF; u++) {
+      const int e = tid + u * BLOCK;
+      if (e < TJ * CH) {
+        const int row = e / CH, c = e - row * CH;
+        *reinterpret_cast<uint4*>(ys + row * KNN_I8_STRIDE + c * 16) = pf[u];
+      }
+    }
+    if (tid < TJ) ykey_s[tid] = pfkey;
+    __syncthreads();
+    if (j0 + TJ < jend) prefetch(j0 + TJ);
+    const int nsub = (n + 31) / 32;
+    for (int sub = 0; sub < nsub; sub++) {
+      // accumulator register v of this lane is reference row 8*(v/4) + 4*half + v%4 of the sub-tile:
+      // start from the keys of those rows (they are the C operand of the first matrix instruction)
+      knn_i32x4 kk[4];
+#pragma unroll
+      for (int b = 0; b < 4; b++) kk[b] = *reinterpret_cast<const knn_i32x4*>(kbase + sub * 32 + 8 * b);
+      knn_i32x16 acc[QSETS];
+#pragma unroll
+      for (int h = 0; h < QSETS; h++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[h][v] = kk[v >> 2][v & 3];
+      const unsigned char* arow = abase + sub * (32 * KNN_I8_STRIDE);
+#pragma unroll
+      for (int kb = 0; kb < KNN_I8_KB; kb++) {
+        const knn_i32x4 a = *reinterpret_cast<const knn_i32x4*>(arow + kb * 32);
+#pragma unroll
+        for (int h = 0; h < QSETS; h++) acc[h] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bq[h][kb], acc[h], 0, 0, 0);
+      }
+#pragma unroll
+      for (int h = 0; h < QSETS; h++) {
+        // cheap screen first: the smallest of the lane's 16 values against the threshold (three-operand minima)
+        int m = min(min(acc[h][0], acc[h][1]), acc[h][2]);
+#pragma unroll
+        for (int v = 3; v < 15; v += 2) m = min(min(m, acc[h][v]), acc[h][v + 1]);
+        m = min(m, acc[h][15]);
+        if (__builtin_expect(!keops_any(m <= t[h]), 1)) continue;
+        unsigned long long bals[16];
+#pragma unroll
+        for (int v = 0; v < 16; v++) bals[v] = __ballot(acc[h][v] <= t[h]);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          unsigned long long bal = bals[v];
+          bool mine = (bal >> lane) & 1ull;
+          while (__builtin_expect(bal != 0ull, 0)) {
+            const int slot = qcount + __popcll(bal & ((1ull << lane) - 1ull));
+            if (mine && slot < 64) {
+              qq[wave][slot] = h * 32 + col;
+              qj[wave][slot] = (int)(j0 + sub * 32 + 8 * (v >> 2) + 4 * half + (v & 3));
+              mine = false;
+            }
+            qcount += __popcll(bal);
+            if (qcount >= 64) {
+              flush(64);
+              qcount = 0;
+              bal = __ballot(mine);  // lanes that found the queue full retry
+            } else {
+              bal = 0ull;
+            }
+          }
+        }
+      }
+    }
+  }
+  if (qcount > 0) flush(qcount);
+  if (lane == 0) P.logcount[logid] = (int)logged;
+}
+#endif
+
 #if !KNN_RANGES
 // threshold estimate from a subset of the references: K-lists of upper bounds, no memory access per candidate
 extern "C" __global__ void __launch_bounds__(64 * KNN_SWAVES) keops_knn_sample(const KnnParams P) {
@@ -617,6 +854,9 @@ extern "C" __global__ void __launch_bounds__(64 * KNN_SWAVES) keops_knn_sample(c
 
 // fixed-threshold filter: KNN_FWAVES wavefronts of 32*KNN_FQSETS queries share every staged tile
 extern "C" __global__ void __launch_bounds__(64 * KNN_FWAVES) keops_knn_filter(const KnnParams P) {
+#if KNN_I8
+  if (P.scal != nullptr && knn_i8_taken(P)) return;  // keops_knn_filter_i8 serves this call
+#endif
   __shared__ __attribute__((aligned(16))) unsigned char ys[KNN_FTJ * KNN_STRIDE];
   __shared__ __attribute__((aligned(16))) float ykey_s[KNN_FTJ];
   __shared__ int qq[KNN_FWAVES][64];
@@ -684,6 +924,9 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_fill_lists(const Knn
 
 extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParams P) {
   const i64 q = (i64)blockIdx.x * 256 + threadIdx.x;
+#if KNN_I8 && !KNN_RANGES
+  if (q == 0 && P.scal != nullptr) P.scal[3] = knn_i8_taken(P) ? 1u : 0u;  // which filter served the call
+#endif
   if (q >= P.nq) return;
   float bv[KNN_K];
   int bi[KNN_K];
@@ -717,9 +960,19 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_thresholds(const Knn
   if (refine) knn_merge_lists(P, q, bv, bi, 0, 4, count);
   else knn_merge_lists(P, q, bv, bi, 0, 1, P.nslabs);
   const float tau = bv[KNN_K - 1];
-  float t = __builtin_fminf((tau + tau * (refine ? KNN_DELTA : 3.0f * KNN_DELTA)) - P.xkey[q], KNN_FLT_MAX);
+  const float tau_up = tau + tau * (refine ? KNN_DELTA : 3.0f * KNN_DELTA);
+  float t = __builtin_fminf(tau_up - P.xkey[q], KNN_FLT_MAX);
   if (refine) t = __builtin_fminf(t, P.thr[q]);
   P.thr[q] = t;
+#if KNN_I8
+  if (P.scal != nullptr) {
+    int ti = knn_i8_threshold(P, q, tau_up);
+    if (refine) ti = min(ti, P.thr_i[q]);
+    P.thr_i[q] = ti;
+    // first estimate: is the slack of the byte filter small against the search radius of this query?
+    if (!refine && !(knn_i8_slack(P, q) <= KNN_I8_ETA * __builtin_sqrtf(__builtin_fmaxf(tau_up, 0.f)))) atomicAdd(P.scal + 1, 1u);
+  }
+#endif
 }
 
 // ---- replay of the candidate logs ---------------------------------------------------------------

@@ -195,7 +195,9 @@ def generate_knn_plugin(red, rowvar, colvar, nargs, block_sparse=False):
     ftj = max(tj, min(config.knn_filter_tile_j, 64 * config.knn_filter_waves))
     while ftj > tj and ftj * (dpad * 2 * (1 + split) + 16) > 96 * 1024:
         ftj //= 2
-    meta = dict(scheme="knn", block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
+    # dense launches in 32 dimensions and more: the fixed-threshold filter also exists on signed bytes
+    i8 = int(config.knn_i8 and not split and not block_sparse and D >= 32)
+    meta = dict(scheme="knn", knn_i8=i8, block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
                 sizeof_acc=4, nrowvars=1, ncolvars=1, nparvars=0, knn_d=D, knn_dpad=dpad, knn_k=red.K,
                 knn_qb=waves * 32 * qsets, knn_fwaves=config.knn_filter_waves, knn_fqsets=config.knn_filter_qsets,
                 knn_sample=config.knn_sample, knn_split=split, knn_ftj=ftj, knn_sqb=swaves * 32 * sqsets, knn_sblock=64 * swaves,
@@ -205,7 +207,7 @@ def generate_knn_plugin(red, rowvar, colvar, nargs, block_sparse=False):
         src += ["#define KEOPS_MC_RANGES 1", "#define KNN_RANGES 1"]
     defs = dict(KEOPS_NARGS=nargs, KNN_D=D, KNN_DPAD=dpad, KNN_K=red.K, KEOPS_RED_KEEP=red.keep, KEOPS_DIMOUT=red.dim,
                 KNN_QSETS=qsets, KNN_TJ=tj, KNN_WAVES=waves, KNN_FWAVES=config.knn_filter_waves,
-                KNN_FQSETS=config.knn_filter_qsets, KNN_FTJ=ftj, KNN_SWAVES=swaves, KNN_SQSETS=sqsets, KNN_SPLIT=split)
+                KNN_FQSETS=config.knn_filter_qsets, KNN_FTJ=ftj, KNN_SWAVES=swaves, KNN_SQSETS=sqsets, KNN_SPLIT=split, KNN_I8=i8)
     src += [f"#define {k} {v}" for k, v in defs.items()]
     src.append('#include "keops_knn_mfma.h"')
     return "\n".join(src) + "\n", meta
@@ -1017,7 +1019,7 @@ def get_keops_dll(
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
            use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs),
            binder.templates_digest(), bool(config.radial), bool(config.radial_fold), bool(config.radial_ranges), int(config.radial_mm_min_dv),
-           int(config.radial_mm_rb), bool(use_half))
+           int(config.radial_mm_rb), bool(config.knn_i8), bool(use_half))
     with _lock:
         hit = _cache.get(key)
     if hit is not None:

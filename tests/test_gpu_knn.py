@@ -82,6 +82,10 @@ def test_knn_config3_query_subset():
     x = rng.random((M, D), dtype=np.float32)
     y = rng.random((N, D), dtype=np.float32)
     vals, idx = _knn(D, K)(*to_dev(x, y))
+    from keops_amd import keops_io
+
+    # bounded data: the device lets the fixed-threshold filter run on signed bytes (keops_knn_filter_i8)
+    assert keops_io.last_loader.module.meta("knn_i8") == "1" and keops_io.last_loader.module.path_status() == 1
     rows = np.sort(np.random.default_rng(7).choice(M, 512, replace=False)).astype(np.int64)
     ref = cpu_reduc("sqdist", [x, y], M, N, 1, reduction="KMin_ArgKMin", K=K, scheme="direct_sum", rows=rows)
     sel = torch.from_numpy(rows).cuda()
@@ -97,6 +101,45 @@ def test_knn_config3_query_subset():
     xq, yq = torch.from_numpy(x).cuda()[q], torch.from_numpy(y).cuda()[idx[q, 0]]
     d0 = ((xq.double() - yq.double()) ** 2).sum(1)
     assert torch.allclose(vals[q, 0].double(), d0, rtol=1e-5)
+
+
+@pytest.mark.parametrize("kind,D,K,taken", [("uniform", 64, 10, 1), ("gauss", 100, 3, 1), ("ties", 40, 5, 1), ("offset", 33, 16, 1),
+                                            ("outlier", 64, 10, 0), ("heavy", 48, 3, 0), ("tight_clusters", 128, 10, 0)])
+def test_byte_filter_or_bf16_filter_chosen_on_the_device(kind, D, K, taken):
+    """Two-phase launches in 32 dimensions and more quantise both sets to signed bytes (step = largest centred component
+    / 127) and filter with v_mfma_i32_32x32x32_i8: integer products are exact, so |x - y| differs from the distance of
+    the quantised points by at most the two quantisation residuals.  Where that slack is large against the search
+    radii (outliers, heavy tails, clusters much tighter than their spread) the device keeps the bfloat16 filter.
+    Either way the exact re-rank returns the oracle's bits."""
+    from keops_amd import keops_io
+
+    M, N = 2500, 60000
+    rng = np.random.default_rng(1000 + D + K)
+    if kind in ("uniform", "outlier", "offset"):
+        x, y = rng.random((M, D)), rng.random((N, D))
+        if kind == "outlier":
+            y[7, 3], x[11, 0] = 5000.0, -800.0
+        if kind == "offset":
+            x, y = x + 1000.0, y + 1000.0
+    elif kind == "gauss":
+        x, y = rng.standard_normal((M, D)), rng.standard_normal((N, D))
+    elif kind == "heavy":
+        x, y = rng.standard_t(2, (M, D)), rng.standard_t(2, (N, D))
+    elif kind == "ties":
+        y = rng.integers(0, 4, (N, D)).astype(np.float64)           # many equal distances: the index decides
+        x = y[rng.integers(0, N, M)] + (rng.random((M, D)) < 0.02)
+    else:
+        c = 3 * rng.standard_normal((20, D))
+        x = c[rng.integers(0, 20, M)] + 0.1 * rng.standard_normal((M, D))
+        y = c[rng.integers(0, 20, N)] + 0.1 * rng.standard_normal((N, D))
+    x, y = x.astype(np.float32), y.astype(np.float32)
+    vals, idx = _knn(D, K)(*to_dev(x, y))
+    module = keops_io.last_loader.module
+    assert module.meta("knn_i8") == "1" and module.path_status() == taken
+    rows = np.sort(rng.choice(M, 400, replace=False)).astype(np.int64)
+    ref = cpu_reduc("sqdist", [x, y], M, N, 1, reduction="KMin_ArgKMin", K=K, scheme="direct_sum", rows=rows)
+    assert np.array_equal(idx.cpu().numpy().reshape(M, K)[rows], ref[:, 1::2].astype(np.int64))
+    assert np.array_equal(vals.cpu().numpy().reshape(M, K)[rows], ref[:, 0::2])
 
 
 @pytest.mark.parametrize("M,N,D,K", [(3000, 70000, 3, 10), (1500, 40000, 2, 4), (2000, 50000, 16, 50), (500, 900, 3, 10),

@@ -1,7 +1,7 @@
 """GPU parity of block-sparse Gaussian-type sums whose exponents come from the matrix cores
 (kernels/keops_radial_ranges.h: one centre per row range, the columns of every range formatted relative to it)
 against the CPU oracle (CpuReduc_ranges.py:150-228).  Tolerances: float32 sums 1e-5, norm-wise and relative to
-sum_j |F_ij|.  `Module.radial_status()` tells which kernel family served a launch."""
+sum_j |F_ij|.  `Module.path_status()` tells which kernel family served a launch."""
 import numpy as np
 import pytest
 import torch
@@ -57,9 +57,9 @@ def test_block_sparse_gaussian_sums_on_the_matrix_cores_vs_oracle(D, Dv, sigma):
     rd = tuple(r.cuda() for r in ranges)
     conv = _genred(D, Dv)
     got = conv(*dev, ranges=rd)                        # the ranges are read back and validated on the host
-    assert _module().meta("rad_ranges") == "1" and _module().radial_status() == 1
+    assert _module().meta("rad_ranges") == "1" and _module().path_status() == 1
     again = conv(*dev, ranges=rd)                      # workgroup table built on the device
-    assert _module().radial_status() == 1 and _module().ranges_status() == 0
+    assert _module().path_status() == 1 and _module().ranges_status() == 0
     assert torch.equal(again, got)
     rows = np.sort(np.random.default_rng(1).choice(M, 1500, replace=False)).astype(np.int64)
     r3 = tuple(r.numpy() for r in ranges[:3])
@@ -78,7 +78,7 @@ def test_reduction_over_i_uses_the_last_three_ranges():
     ranges, keep = _pattern(c, rx, ry)
     M, N = x.shape[0], y.shape[0]
     got = _genred(D, Dv, axis=0)(*to_dev(x, y, a, g), ranges=tuple(r.cuda() for r in ranges))
-    assert got.shape == (N, Dv) and _module().radial_status() == 1
+    assert got.shape == (N, Dv) and _module().path_status() == 1
     cols = np.sort(np.random.default_rng(2).choice(N, 1500, replace=False)).astype(np.int64)
     r3t = tuple(r.numpy() for r in ranges[3:])
     ref = cpu_reduc("gauss", [y, x, a, g], N, M, Dv, ranges=r3t, rows=cols)   # roles of i and j exchanged
@@ -100,7 +100,7 @@ def test_rows_without_columns_and_rows_outside_every_range_are_zero():
     dev = to_dev(x, y, b, g)
     out = torch.full((M, Dv), 7.0, device="cuda")
     got = _genred(D, Dv)(*dev, ranges=tuple(r.cuda() for r in ranges), out=out)
-    assert _module().radial_status() == 1
+    assert _module().path_status() == 1
     for k in (5, 11):
         assert torch.all(got[int(rx[k, 0]):int(rx[k, 1])] == 0)
     rows = np.sort(np.random.default_rng(3).choice(M, 1500, replace=False)).astype(np.int64)
@@ -124,7 +124,7 @@ def test_gradient_with_respect_to_the_points_under_ranges_vs_oracle():
     a = _genred(D, 1)(xd, yd, bd, gd, ranges=rd)
     e = np.random.default_rng(4).standard_normal((M, 1)).astype(np.float32)
     (gx,) = torch.autograd.grad(a, [xd], torch.from_numpy(e).cuda())
-    assert _module().meta("rad_ranges") == "1" and _module().radial_status() == 1
+    assert _module().meta("rad_ranges") == "1" and _module().path_status() == 1
     rows = np.sort(np.random.default_rng(5).choice(M, 1500, replace=False)).astype(np.int64)
     r3 = tuple(r.numpy() for r in ranges[:3])
     ref = cpu_reduc("gauss_gradx", [x, y, b, g, e], M, N, D, ranges=r3, rows=rows)
@@ -143,7 +143,7 @@ def test_kernel_too_narrow_for_the_clusters_falls_back_to_exact_differences():
     dev = to_dev(x, y, b, g)
     rd = tuple(r.cuda() for r in ranges)
     got = _genred(D, Dv)(*dev, ranges=rd)
-    assert _module().meta("rad_ranges") == "1" and _module().radial_status() == 0
+    assert _module().meta("rad_ranges") == "1" and _module().path_status() == 0
     plain = _genred(D, Dv, enable_chunks=False)(*dev, ranges=rd)   # matrix-core schemes switched off
     assert _module().meta("radial") is None
     assert torch.equal(got, plain)
@@ -161,7 +161,7 @@ def test_short_row_ranges_and_small_patterns_stay_on_the_general_purpose_kernel(
     ranges, keep = _pattern(c, rx, ry)
     M, N = x.shape[0], y.shape[0]
     got = _genred(D, Dv)(*to_dev(x, y, b, g), ranges=tuple(r.cuda() for r in ranges))
-    assert _module().radial_status() == 0
+    assert _module().path_status() == 0
     r3 = tuple(r.numpy() for r in ranges[:3])
     ref = cpu_reduc("gauss", [x, y, b, g], M, N, Dv, ranges=r3)
     scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, Dv, ranges=r3)
@@ -181,12 +181,12 @@ def test_ranges_edited_in_place_follow_and_an_outgrown_workspace_falls_back():
     rd = tuple(r.cuda() for r in ranges)
     conv = _genred(D, Dv)
     conv(*dev, ranges=rd)
-    assert _module().radial_status() == 1
+    assert _module().path_status() == 1
     rows = np.sort(np.random.default_rng(8).choice(M, 800, replace=False)).astype(np.int64)
 
     def check(expect_taken):
         got = conv(*dev, ranges=rd)
-        assert _module().radial_status() == expect_taken and _module().ranges_status() == 0
+        assert _module().path_status() == expect_taken and _module().ranges_status() == 0
         r3 = tuple(r.cpu().numpy() for r in rd[:3])
         ref = cpu_reduc("gauss", [x, y, b, g], M, N, Dv, ranges=r3, rows=rows)
         scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, Dv, ranges=r3, rows=rows)
@@ -208,7 +208,7 @@ def test_block_sparse_matrix_core_sums_under_graph_capture():
     conv = _genred(D, Dv)
     conv(xd, yd, bd, gd, ranges=rd)
     eager = conv(xd, yd, bd, gd, ranges=rd)
-    assert _module().radial_status() == 1
+    assert _module().path_status() == 1
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):

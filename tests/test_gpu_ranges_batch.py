@@ -74,7 +74,7 @@ def test_config4_block_sparse_100x10k_row_subset():
 
     # the clusters are about three kernel widths across: every row range passes the device-side check and the
     # exponents come from the matrix cores (kernels/keops_radial_ranges.h)
-    assert keops_io.last_loader.module.radial_status() == 1
+    assert keops_io.last_loader.module.path_status() == 1
     rows = np.sort(np.random.default_rng(1).choice(M, 2048, replace=False)).astype(np.int64)
     r3 = tuple(r.numpy() for r in ranges[:3])
     ref = cpu_reduc("gauss", [x, y, b, g], M, N, 1, ranges=r3, rows=rows)
