@@ -554,7 +554,7 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
 // The exponent tile is computed transposed (columns as the A operand, the wavefront's rows as B), so that lane l
 // receives the 16 values of ITS row l % 32: registers 0-7 and 8-15 are then A operands of two k blocks of the second
 // product as they stand.  Float32 accuracy from bfloat16 products: K = h + m + l by truncation (two v_and, two exact
-// v_sub, byte permutes to pack: 26 issue cycles per pair with v_exp_f32, whatever RAD_DV is, against 8 + 4 RAD_DV),
+// v_sub, byte permutes to pack: the same vector work per pair whatever RAD_DV is, against v_exp_f32 + RAD_DV fma),
 // and the three terms of the weights sit side by side in the 32 operand columns, so three instructions per k block
 // form all nine term products; the column groups are added once at the end.  Running sums are folded into a second
 // accumulator every RAD_MM_FOLD columns.
@@ -629,26 +629,23 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
         for (int kb = 0; kb < RAD_NKB; kb++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[kb], a[r][kb], z, 0, 0, 0);
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
-          unsigned hb[8], mb[8], lb[8];
-#pragma unroll
-          for (int e = 0; e < 8; e++) {
-            const float x = __builtin_amdgcn_exp2f(z[8 * kb + e]);
-            hb[e] = __float_as_uint(x);
-            const float r1 = x - __uint_as_float(hb[e] & 0xffff0000u);   // exact
-            mb[e] = __float_as_uint(r1);
-            const float r2 = r1 - __uint_as_float(mb[e] & 0xffff0000u);  // exact, at most 8 significant bits
-            lb[e] = __float_as_uint(r2);
-          }
-          // pack the high halves of two floats into one register: truncated bfloat16 terms
+          // K = h + m + l, each the truncation of what is left to 8 significant bits (the subtractions are exact); a
+          // byte permute packs the high halves of two floats: the bfloat16 terms.  (v_dot2_f32_bf16 against the pairs
+          // (-1, 0) / (0, -1) subtracts a packed term in one instruction instead of v_and + v_sub: measured, same time.)
           uint4 ph, pm, pl;
           unsigned* php = reinterpret_cast<unsigned*>(&ph);
           unsigned* pmp = reinterpret_cast<unsigned*>(&pm);
           unsigned* plp = reinterpret_cast<unsigned*>(&pl);
 #pragma unroll
           for (int e = 0; e < 4; e++) {
-            php[e] = __builtin_amdgcn_perm(hb[2 * e + 1], hb[2 * e], 0x07060302u);
-            pmp[e] = __builtin_amdgcn_perm(mb[2 * e + 1], mb[2 * e], 0x07060302u);
-            plp[e] = __builtin_amdgcn_perm(lb[2 * e + 1], lb[2 * e], 0x07060302u);
+            const float x0 = __builtin_amdgcn_exp2f(z[8 * kb + 2 * e]), x1 = __builtin_amdgcn_exp2f(z[8 * kb + 2 * e + 1]);
+            php[e] = __builtin_amdgcn_perm(__float_as_uint(x1), __float_as_uint(x0), 0x07060302u);
+            const float r0 = x0 - __uint_as_float(__float_as_uint(x0) & 0xffff0000u);
+            const float r1 = x1 - __uint_as_float(__float_as_uint(x1) & 0xffff0000u);
+            pmp[e] = __builtin_amdgcn_perm(__float_as_uint(r1), __float_as_uint(r0), 0x07060302u);
+            const float s0 = r0 - __uint_as_float(__float_as_uint(r0) & 0xffff0000u);
+            const float s1 = r1 - __uint_as_float(__float_as_uint(r1) & 0xffff0000u);
+            plp[e] = __builtin_amdgcn_perm(__float_as_uint(s1), __float_as_uint(s0), 0x07060302u);
           }
           const rad_bf16x8 kh = __builtin_bit_cast(rad_bf16x8, ph), km = __builtin_bit_cast(rad_bf16x8, pm),
                            kl = __builtin_bit_cast(rad_bf16x8, pl);
