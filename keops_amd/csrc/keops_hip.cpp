@@ -802,6 +802,7 @@ struct KnnHeader {
   int32_t stage, pad_;
   // filter on signed bytes (modules with knn_i8=1, two-phase launches; null otherwise)
   void *xq8, *yq8, *ykey_i, *xnorm_i, *xres, *thr_i, *scal;
+  int64_t batch_rows, batch_cols;  // batches served as row ranges: indices relative to the batch
 };
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -1003,7 +1004,7 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
 // Block-sparse launch of a K-nearest-neighbour module built for ranges (KNN_RANGES): pre-pass, neutral lists, the
 // adaptive kernel with one workgroup per patch of a row range, merge (which writes the output layout).
 int launch_knn_ranges(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr, void* out, hipStream_t stream,
-                      const RangeLaunch& rg) {
+                      const RangeLaunch& rg, int64_t batch_rows = 0, int64_t batch_cols = 0) {
   const int64_t D = m.meta_int("knn_d", 0), DP = m.meta_int("knn_dpad", 0), K = m.meta_int("knn_k", 0);
   if (D <= 0 || DP <= 0 || K <= 0) return fail(-1, "corrupt knn module metadata");
   if (nr > 2147483647LL) return fail(-1, "too many reference rows for 32-bit indices");
@@ -1023,6 +1024,7 @@ int launch_knn_ranges(Module& m, int64_t nq, int64_t nr, const void* xq, const v
   h.nq = nq; h.nr = nr; h.xq = xq; h.yr = yr;
   h.xh = ws + o_xh; h.yh = ws + o_yh; h.xkey = ws + o_xkey; h.ykey = ws + o_ykey; h.colsum = ws + o_colsum; h.colpart = ws + o_colpart;
   h.plist_d = ws + o_pd; h.plist_i = ws + o_pi; h.out = out; h.ref_step = 1; h.nslabs = 1; h.slab_len = nr;
+  h.batch_rows = batch_rows; h.batch_cols = batch_cols;
   p.rt = rg.header(m.nargs);
   const size_t HS = sizeof(KnnHeader) + sizeof(RangeHeader);
   auto run = [&](const char* k, unsigned gx, unsigned block, size_t size) { return launch_raw(m, k, gx, 1, block, &p, size, stream); };
@@ -1533,12 +1535,37 @@ static int launch_on_device(Module& m, int64_t nx, int64_t ny, int tagI, int tag
 
   if (m.scheme == "knn") {
     const bool built_for_ranges = m.meta_int("ranges", 0) != 0;
-    if (user_ranges != built_for_ranges || (built_for_ranges && nb > 0))
-      return fail(-1, built_for_ranges ? "this K-nearest-neighbour module was built for block-sparse ranges without batch dimensions"
-                                       : "this K-nearest-neighbour module does not handle block-sparse ranges");
     const int rowarg = m.meta_int("rowarg", 0), colarg = m.meta_int("colarg", 1);
     if (rowarg < 0 || colarg < 0 || rowarg >= m.nargs || colarg >= m.nargs) return fail(-1, "corrupt knn module metadata");
-    if (user_ranges) {
+    // many batches on a module built for ranges: every batch is one row range with one reduced-index range, provided
+    // queries and references carry every batch dimension in full (no broadcasting)
+    bool batches_as_ranges = false;
+    if (built_for_ranges && nb > 0 && !user_ranges) {
+      auto full = [&](int arg) {
+        const int64_t* r = S.row(arg + 1);
+        for (int b = 0; b < nb; b++)
+          if (r[b] != S.shapes[b]) return false;
+        return true;
+      };
+      if (!full(rowarg) || !full(colarg))
+        return fail(-1, "this K-nearest-neighbour module serves batches as row ranges: queries and references must carry "
+                        "every batch dimension (no broadcasting)");
+      batches_as_ranges = true;
+    }
+    if (!batches_as_ranges && (user_ranges != built_for_ranges || (built_for_ranges && nb > 0)))
+      return fail(-1, built_for_ranges ? "this K-nearest-neighbour module was built for block-sparse ranges without batch dimensions"
+                                       : "this K-nearest-neighbour module does not handle block-sparse ranges");
+    if (batches_as_ranges) {
+      RangeLaunch rg;
+      rg.nbatchdims = 0;  // rows are addressed globally: the kernel sees plain ranges over the flattened batches
+      rg.user_ranges = false;
+      if (int rc = prepare_range_tables(m, S, tagI, false, ranges, rows_total, cols_total, m.meta_int("knn_qb", 256), true, rowvars,
+                                        colvars, vP, stream, rg.tables))
+        return rc;
+      rg.tables.offsets = nullptr;
+      const int64_t R = tagI == 0 ? S.M : S.N, C = tagI == 0 ? S.N : S.M;
+      if (int rc = launch_knn_ranges(m, rows_total, cols_total, args[rowarg], args[colarg], out, stream, rg, R, C)) return rc;
+    } else if (user_ranges) {
       RangeLaunch rg;
       rg.nbatchdims = 0;
       rg.user_ranges = true;

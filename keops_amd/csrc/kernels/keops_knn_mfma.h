@@ -119,6 +119,8 @@ struct KnnParams {
   unsigned* scal;        // [0]: bit pattern of the largest |centred component|; [1]: queries for which the byte filter
                          // would be too loose; [2]: bit pattern of the largest distance between a centred reference
                          // and its quantised copy; [3]: 1 when the byte filter served the call (written at the end)
+  i64 batch_rows, batch_cols;  // > 0: the row ranges are batches of that many queries / references, and the indices
+                         // returned are relative to the batch (GpuReduc1D_ranges.py:151-158)
 #if KNN_RANGES
   KeopsRangeTables rt;   // block-sparse launches: workgroup table and reduced-index ranges (keops_knn_main only)
 #endif
@@ -932,6 +934,14 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParam
   int bi[KNN_K];
   knn_merge_lists(P, q, bv, bi, 0, 1, P.nslabs);
   T* out = P.out + q * KEOPS_DIMOUT;
+#if KNN_RANGES
+  if (P.batch_rows > 0) {
+    // (neutral entries, infinite distance and index 0, stay as they are)
+    const int first = (int)((q / P.batch_rows) * P.batch_cols);
+#pragma unroll
+    for (int l = 0; l < KNN_K; l++) bi[l] = bv[l] < __builtin_huge_valf() ? bi[l] - first : bi[l];
+  }
+#endif
 #pragma unroll
   for (int l = 0; l < KNN_K; l++) {
 #if KEOPS_RED_KEEP == 0

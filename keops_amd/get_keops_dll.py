@@ -995,13 +995,14 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
 def get_keops_dll(
     map_reduce_id, red_formula_string, enable_chunks, enable_finalchunks, mul_var_highdim, aliases, nargs, dtype,
     dtypeacc, sum_scheme_string, tagHostDevice, tagCPUGPU, tag1D2D, use_half, use_fast_math, device_id, nx=None,
-    batch_loop=0, pairs=0,
+    batch_loop=0, pairs=0, batch_total=0,
 ):
     """Same arguments and same 19-tuple as the reference's get_keops_dll (get_keops_dll.py:78-159),
     plus ``nx``: the number of output rows of the call being prepared, used to pick the number of
     rows per lane, and ``batch_loop``: when not 0, the "_ranges" of the scheme id stand for a few batches
     of less than 2**batch_loop pairs each without block-sparse ranges, which a dense module may serve one batch
-    at a time; ``pairs``: when not 0, the call (each batch of it) holds less than 2**pairs pairs.  ``dtype`` / ``dtypeacc`` are C
+    at a time; ``pairs``: when not 0, the call (each batch of it) holds less than 2**pairs pairs; ``batch_total``: when
+    not 0, all batches together hold less than 2**batch_total pairs and no variable is broadcast over a batch dimension.  ``dtype`` / ``dtypeacc`` are C
     type names ("float" | "double").  ``use_half``: the data are half-precision numbers (converted to float32 copies by
     the library before the launch): modules are compiled for float, and the chunked matrix-core scheme keeps one
     half-precision term per component instead of two."""
@@ -1017,7 +1018,7 @@ def get_keops_dll(
         # only the bucket matters for the cache key
         rows_hint = nx if nx < 64 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
-           use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs),
+           use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs), int(batch_total),
            binder.templates_digest(), bool(config.radial), bool(config.radial_fold), bool(config.radial_ranges), int(config.radial_mm_min_dv),
            int(config.radial_mm_rb), bool(config.knn_i8), bool(use_half))
     with _lock:
@@ -1043,6 +1044,12 @@ def get_keops_dll(
         # arithmetic in the reference's order) but the vector-ALU chunked variant for long sums
         mc = int(enable_chunks) > 0
         knn = match_knn_sqdist(red_k, dtype, map_reduce_id, batch_loop, pairs) if mc else None
+        knn_batches = False
+        if knn is None and mc and irregular and batch_loop >= 0 and batch_total and config.knn_ranges:
+            # many batches, none of them large enough to be served on its own: every batch becomes a row range of the
+            # block-sparse variant (queries and references carry every batch dimension in full)
+            knn = match_knn_sqdist(red_k, dtype, map_reduce_id, -1, batch_total)
+            knn_batches = knn is not None
         knn_hd = match_knn_highdim(red_k, dtype, map_reduce_id, use_fast_math) if (mc and knn is None) else None
         chk = match_chunk(red, dtype, map_reduce_id, use_fast_math) if (mc and knn is None) else None
         # double precision: the contraction on the float64 matrix instruction, when there are enough output rows to
@@ -1054,7 +1061,7 @@ def get_keops_dll(
         if enable_finalchunks and mc and knn is None and chk is None:
             fin = match_final(red, dtype, dtypeacc, sum_scheme_string, map_reduce_id, use_fast_math)
         if knn is not None:
-            source, meta = generate_knn_plugin(red_k, knn[0], knn[1], nargs, block_sparse=(irregular and batch_loop == -1))
+            source, meta = generate_knn_plugin(red_k, knn[0], knn[1], nargs, block_sparse=(irregular and (batch_loop == -1 or knn_batches)))
             use_chunk_mode = 3  # matrix-core filter scheme (no counterpart among the reference's chunk modes)
         elif fin is not None:
             source, meta = generate_final_plugin(red, fin, sum_scheme_string, nargs, irregular=irregular)

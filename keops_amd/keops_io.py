@@ -22,7 +22,7 @@ class LoadKeOps_hip:
     empty_ranges = tuple([_NULL_RANGE.ctypes.data] * 7)
 
     def __init__(self, tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula, aliases, nargs,
-                 dtype, lang, optional_flags, nx=None, batch_loop=0, pairs=0):
+                 dtype, lang, optional_flags, nx=None, batch_loop=0, pairs=0, batch_total=0):
         if lang not in ("torch", "pytorch"):
             raise ValueError("[KeOps] the HIP backend binds torch tensors only")
         if tagCPUGPU != 1 or tagHostDevice not in (0, 1):
@@ -65,7 +65,7 @@ class LoadKeOps_hip:
             sub = lambda f, extra: LoadKeOps_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, f,
                                                  list(aliases) + extra, nargs + len(extra),
                                                  "float32" if self.half else dtype, lang, sub_flags,
-                                                 nx=nx, batch_loop=batch_loop, pairs=pairs)
+                                                 nx=nx, batch_loop=batch_loop, pairs=pairs, batch_total=batch_total)
             self.sub_slices, self.ones_column = [], False
             if plan["c"]:
                 for c0 in range(0, D, width):
@@ -87,7 +87,7 @@ class LoadKeOps_hip:
          dimsy, dimsp) = get_keops_dll(
             map_reduce_id, formula, p.enable_chunks, -1, p.mult_var_highdim, p.aliases, nargs, p.c_dtype,
             p.c_dtype_acc, p.sum_scheme, tagHostDevice, tagCPUGPU, tag1D2D, self.half, optional_flags["use_fast_math"],
-            device_id_request, nx=nx, batch_loop=batch_loop, pairs=pairs,
+            device_id_request, nx=nx, batch_loop=batch_loop, pairs=pairs, batch_total=batch_total,
         )
         # the engine reports (output-indexed, reduced) variable lists; the ABI takes (i, j) lists
         if p.tagI == 1:
@@ -203,8 +203,9 @@ def load_keops_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_requ
     """Cached constructor (the reference keeps one LoadKeOps object per parameter set as well,
     pykeops/pykeops/common/keops_io/LoadKeOps.py:23-31): parsing the formula and resolving the
     module happen once, later calls only launch.  ``nx`` / ``ny``: output and reduced rows of the call (of each
-    batch); ``batch``: (number of batches, M, N) of a call with batch dimensions and no block-sparse ranges: a few
-    large batches may be served one at a time by a dense module."""
+    batch); ``batch``: (number of batches, M, N[, full]) of a call with batch dimensions and no block-sparse ranges: a
+    few large batches may be served one at a time by a dense module, many batches as row ranges by a block-sparse one
+    (``full``: every tensor variable carries every batch dimension, nothing is broadcast)."""
     from .get_keops_dll import _rows_bucket
     from . import config
 
@@ -213,17 +214,22 @@ def load_keops_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_requ
     batch_loop = int(batch[1] * batch[2]).bit_length() if (batch and 0 < batch[0] <= config.knn_batch_max) else 0
     if batch and batch[0] == 0:
         batch_loop = -1  # block-sparse ranges without batch dimensions
+    # log2 bucket of the pairs of all batches together when nothing is broadcast, else 0
+    batch_total = int(batch[0] * batch[1] * batch[2]).bit_length() if (batch and batch[0] > 0 and len(batch) > 3 and batch[3]) else 0
+    if batch_total > 44:
+        batch_total = 44
     # log2 bucket of the pairs of the call (of each batch), 0: unknown or beyond every threshold of the engine
     pairs = int(nx * ny).bit_length() if (nx is not None and ny is not None) else 0
     if pairs > 40:
         pairs = 0
     key = (tagCPUGPU, tag1D2D, tagHostDevice, bool(use_ranges), device_id_request, formula, tuple(aliases), nargs,
-           dtype, lang, tuple(sorted(optional_flags.items())), _rows_bucket(rows_hint), batch_loop, pairs)
+           dtype, lang, tuple(sorted(optional_flags.items())), _rows_bucket(rows_hint), batch_loop, pairs, batch_total)
     global last_loader
     obj = _loaders.get(key)
     if obj is None:
         obj = _loaders[key] = LoadKeOps_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_request, formula,
-                                            aliases, nargs, dtype, lang, optional_flags, nx=nx, batch_loop=batch_loop, pairs=pairs)
+                                            aliases, nargs, dtype, lang, optional_flags, nx=nx, batch_loop=batch_loop, pairs=pairs,
+                                            batch_total=batch_total)
     last_loader = obj
     return obj
 

@@ -71,7 +71,10 @@ class GenredAutograd_base:
             nbatches = 1
             for d in range(nbatchdims):
                 nbatches *= max(a.shape[d] if a.dim() == nbatchdims + 2 else 1 for a in args)
-            batch = (nbatches, params.nx, params.ny)
+            shape = tuple(max(a.shape[d] if a.dim() == nbatchdims + 2 else 1 for a in args) for d in range(nbatchdims))
+            # (every tensor variable carries every batch dimension in full: many small batches can be served as row ranges)
+            full = all(a.dim() != nbatchdims + 2 or tuple(a.shape[:nbatchdims]) == shape for a in args)
+            batch = (nbatches, params.nx, params.ny, full)
         elif nbatchdims == 0 and params.ranges is not None:
             batch = (0, params.nx, params.ny)  # block-sparse ranges, no batch dimensions
 

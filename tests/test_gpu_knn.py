@@ -142,6 +142,38 @@ def test_byte_filter_or_bf16_filter_chosen_on_the_device(kind, D, K, taken):
     assert np.array_equal(vals.cpu().numpy().reshape(M, K)[rows], ref[:, 0::2])
 
 
+@pytest.mark.parametrize("shape,M,N,D,K,axis", [((40,), 2048, 4096, 3, 8, 1), ((3, 8), 3000, 2500, 40, 10, 1), ((24,), 2500, 3000, 64, 5, 0)])
+def test_many_batches_served_as_row_ranges(shape, M, N, D, K, axis):
+    """Batches too small to be served one by one: every batch becomes a row range of the block-sparse variant of the
+    scheme (queries and references carry every batch dimension), indices relative to the batch as in
+    GpuReduc1D_ranges.py:151-158; bit-identical to the oracle run batch by batch."""
+    from keops_amd import keops_io
+
+    rng = np.random.default_rng(77 + D)
+    x = rng.random(shape + (M, D)).astype(np.float32)
+    y = rng.random(shape + (N, D)).astype(np.float32)
+    y[..., 5, :] = y[..., 40, :]                                   # ties: the lower index wins
+    vals, idx = _knn(D, K, axis=axis)(*to_dev(x, y))
+    module = keops_io.last_loader.module
+    assert module.meta("scheme") == "knn" and module.meta("ranges") == "1"
+    nout, nred = (M, N) if axis == 1 else (N, M)
+    assert idx.shape == shape + (nout, K)
+    for b in [tuple(0 for _ in shape), tuple(s - 1 for s in shape)]:
+        q, r = (x[b], y[b]) if axis == 1 else (y[b], x[b])
+        ref = cpu_reduc("sqdist", [q, r], nout, nred, 1, reduction="KMin_ArgKMin", K=K, scheme="direct_sum")
+        assert np.array_equal(idx[b].cpu().numpy(), ref[:, 1::2].astype(np.int64))
+        assert np.array_equal(vals[b].cpu().numpy(), ref[:, 0::2])
+    if axis == 1:
+        # a broadcast batch dimension cannot be served that way: the general-purpose kernel takes the call
+        y1 = y[(0,) * len(shape)]                                   # one reference set for every batch
+        _, idx_b = _knn(D, K)(*to_dev(x, y1[(None,) * len(shape)]))
+        module = keops_io.last_loader.module
+        assert not (module.meta("scheme") == "knn" and module.meta("ranges") == "1")
+        b = tuple(s - 1 for s in shape)
+        ref = cpu_reduc("sqdist", [x[b], y1], M, N, 1, reduction="ArgKMin", K=K, scheme="direct_sum")
+        assert np.array_equal(idx_b[b].cpu().numpy(), ref.astype(np.int64))
+
+
 @pytest.mark.parametrize("M,N,D,K", [(3000, 70000, 3, 10), (1500, 40000, 2, 4), (2000, 50000, 16, 50), (500, 900, 3, 10),
                                      (1200, 33000, 7, 1)])
 def test_knn_low_dimension_split_operands(M, N, D, K):
