@@ -179,7 +179,9 @@ int keops_hip_path_status(void* module, unsigned* taken);
  *   (4 per chain and round); kind 4: v_mfma_f32_32x32x16_f16; kind 5: two chains of the bf16 instruction (8 per round)
  *   with `chains` independent v_fmac_f32 after every matrix instruction (what fits beside a saturated matrix pipe).
  *   chains: 1, 2, 4, 8 (kinds 0-2), 1, 2, 4 (kinds 3, 4, 6) or 0, 1, 2, 4, 8 (kind 5); kind 6: v_mfma_i32_32x32x32_i8
- *   (4 per chain and round).
+ *   (4 per chain and round); kind 7: two chains of 16 matrix instructions per round whose operands change with every
+ *   instruction (16 A x 16 B register sets of random data, as when tiles stream through a kernel), chains = 0: the
+ *   bf16 instruction, 1: f16, 2: signed bytes.
  * Measurement aid without counterpart in the reference; used by bench.py --valu-calibration / --mfma-calibration.
  */
 int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave);

@@ -319,6 +319,58 @@ static __global__ void __launch_bounds__(256) keops_mfma_i8_loop(float* out, int
   out[(size_t)blockIdx.x * 256 + threadIdx.x] = (float)r;
 }
 
+// `iters` rounds of 32 matrix instructions (two chains) whose operands change with every instruction, as in a kernel
+// that streams tiles: 16 A and 16 B register sets of random data per lane, instruction k of chain c multiplies
+// A[k] by B[(k + c) % 16].  TYPE 0: v_mfma_f32_32x32x16_bf16, 1: ..._f16, 2: v_mfma_i32_32x32x32_i8.  The loops above
+// feed the same two registers to every instruction, which keeps the operand buses quiet; here they toggle as they do
+// on real data, the multipliers draw more power and the sustained clock is lower.
+template <int TYPE>
+static __global__ void __launch_bounds__(256) keops_mfma_stream_loop(float* out, int iters) {
+  typedef typename std::conditional<TYPE == 2, keops_i32x16, keops_f32x16>::type accT;
+  keops_i32x4 a[16], b[16];
+  unsigned h = 0x9e3779b9u * (threadIdx.x + 1u);
+#pragma unroll
+  for (int k = 0; k < 16; k++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      // two 16-bit floats of magnitude 2^-3 .. 2 (sign and significand random), or four random bytes
+      h = h * 1664525u + 1013904223u;
+      a[k][e] = TYPE == 2 ? (int)h : (int)((h & (TYPE == 1 ? 0x8fff8fffu : 0x81ff81ffu)) | (TYPE == 1 ? 0x30003000u : 0x3e003e00u));
+      h = h * 1664525u + 1013904223u;
+      b[k][e] = TYPE == 2 ? (int)h : (int)((h & (TYPE == 1 ? 0x8fff8fffu : 0x81ff81ffu)) | (TYPE == 1 ? 0x30003000u : 0x3e003e00u));
+    }
+  accT acc[2];
+#pragma unroll
+  for (int c = 0; c < 2; c++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[c][e] = 0;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int k = 0; k < 16; k++)
+#pragma unroll
+      for (int c = 0; c < 2; c++) {
+        const keops_i32x4 av = a[k], bv = b[(k + c) & 15];
+        if constexpr (TYPE == 2) acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, acc[c], 0, 0, 0);
+        else if constexpr (TYPE == 1)
+          acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(keops_f16x8, av), __builtin_bit_cast(keops_f16x8, bv), acc[c], 0, 0, 0);
+        else
+          acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(keops_bf16x8, av), __builtin_bit_cast(keops_bf16x8, bv), acc[c], 0, 0, 0);
+      }
+    if (TYPE != 2) {  // keep the float sums bounded
+#pragma unroll
+      for (int c = 0; c < 2; c++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[c][e] *= 0.0009765625f;
+    }
+  }
+  float r = 0.f;
+#pragma unroll
+  for (int c = 0; c < 2; c++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) r += (float)acc[c][e];
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = r;
+}
+
 // `iters` rounds of 8 v_mfma_f32_32x32x16_bf16 (two dependent chains of 4, the shape of the K-nearest-neighbour
 // filter) with NV independent v_fmac_f32 between them: how much vector work fits beside a saturated matrix pipe
 template <int NV>
@@ -368,7 +420,9 @@ static __global__ void __launch_bounds__(256) keops_mix_loop(float* out, int ite
 // Runs one calibration loop on `stream`: grid of `blocks` workgroups of 256 lanes (4 wavefronts), `iters` rounds.
 // kind 0/1/2: vector loop with MIX = kind; kind 3 / 4: matrix loop on bf16 / f16 operands; kind 6: on signed bytes
 // (v_mfma_i32_32x32x32_i8); kind 5: 8 bf16 matrix
-// instructions per round with `chains` v_fmac_f32 after each of them (0, 1, 2, 4, 8).  chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
+// instructions per round with `chains` v_fmac_f32 after each of them (0, 1, 2, 4, 8); kind 7: 32 matrix instructions
+// per round whose operands change with every instruction, `chains` = 0 bf16, 1 f16, 2 signed bytes.
+// chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
 // instr_per_lane receives the number of counted instructions one wavefront issues (vector: per lane = per wavefront
 // instruction count; matrix: v_mfma instructions).  out must hold blocks * 256 floats.
 int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* out, void* stream, double* instr_per_wave) {
@@ -402,6 +456,13 @@ int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* o
     if (chains == 1) hipLaunchKernelGGL((keops_mfma_i8_loop<1>), g, b, 0, s, out, iters);
     else if (chains == 2) hipLaunchKernelGGL((keops_mfma_i8_loop<2>), g, b, 0, s, out, iters);
     else if (chains == 4) hipLaunchKernelGGL((keops_mfma_i8_loop<4>), g, b, 0, s, out, iters);
+    else return (int)hipErrorInvalidValue;
+  } else if (kind == 7) {
+    // chains = operand type: 0 bf16, 1 f16, 2 signed bytes
+    *instr_per_wave = 32.0 * (double)iters;
+    if (chains == 0) hipLaunchKernelGGL((keops_mfma_stream_loop<0>), g, b, 0, s, out, iters);
+    else if (chains == 1) hipLaunchKernelGGL((keops_mfma_stream_loop<1>), g, b, 0, s, out, iters);
+    else if (chains == 2) hipLaunchKernelGGL((keops_mfma_stream_loop<2>), g, b, 0, s, out, iters);
     else return (int)hipErrorInvalidValue;
   } else if (kind == 5) {
     // chains = vector instructions per matrix instruction: 0, 1, 2, 4, 8
