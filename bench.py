@@ -253,6 +253,8 @@ def calibration(mfma):
     kinds = [(3, "v_mfma_f32_32x32x16_bf16", (1, 2, 4)), (4, "v_mfma_f32_32x32x16_f16", (1, 2, 4)),
              (6, "v_mfma_i32_32x32x32_i8", (1, 2, 4)),
              (7, "two chains, operands change with every instruction (chains = 0: bf16, 1: f16, 2: i8)", (0, 1, 2)),
+             (8, "byte filter loop without memory traffic: 4 v_mfma_i32_32x32x32_i8 and two 16-value minima per round "
+                 "(chains = 0: minima over the results, 1: over other registers, 2: no minima)", (2, 1, 0)),
              (5, "two chains of v_mfma_f32_32x32x16_bf16 with `chains` v_fmac_f32 after every matrix instruction", (0, 1, 2, 4, 8))] if mfma else [
         (0, "v_fmac_f32 chains", (1, 2, 4, 8)), (1, "Gaussian pair mix with v_exp_f32 (9 instr)", (1, 2, 4, 8)),
         (2, "Gaussian pair mix without v_exp_f32 (8 instr)", (1, 2, 4, 8))]
@@ -260,7 +262,7 @@ def calibration(mfma):
         for chains in chain_set:
             for waves in (1, 2, 4):
                 blocks = cus * waves  # one workgroup = 4 wavefronts = one per SIMD of a CU
-                iters = 200_000 // chains if kind < 3 else (12_500 if kind == 7 else (100_000 // chains if kind != 5 else 50_000))
+                iters = 200_000 // chains if kind < 3 else (12_500 if kind == 7 else (100_000 if kind == 8 else (100_000 // chains if kind != 5 else 50_000)))
                 ms, ipw = binder.calibrate(kind, chains, blocks, iters)
                 total = ipw * blocks * 4  # wavefront instructions
                 per_cycle = total / (ms * 1e-3) / simds / clock
@@ -268,7 +270,7 @@ def calibration(mfma):
                            wave_instr_per_cycle_per_simd_at_2p4GHz=round(per_cycle, 4))
                 if kind >= 3:
                     # (kind 6: integer operations, 32 x 32 x 32 per instruction)
-                    depth = 32 if kind == 6 or (kind == 7 and chains == 2) else 16
+                    depth = 32 if kind in (6, 8) or (kind == 7 and chains == 2) else 16
                     row["PFLOP_per_s"] = round(total * 32 * 32 * depth * 2 / (ms * 1e-3) / 1e15, 3)
                 else:
                     row["lane_instr_per_s"] = total * 64 / (ms * 1e-3)

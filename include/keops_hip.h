@@ -181,7 +181,10 @@ int keops_hip_path_status(void* module, unsigned* taken);
  *   chains: 1, 2, 4, 8 (kinds 0-2), 1, 2, 4 (kinds 3, 4, 6) or 0, 1, 2, 4, 8 (kind 5); kind 6: v_mfma_i32_32x32x32_i8
  *   (4 per chain and round); kind 7: two chains of 16 matrix instructions per round whose operands change with every
  *   instruction (16 A x 16 B register sets of random data, as when tiles stream through a kernel), chains = 0: the
- *   bf16 instruction, 1: f16, 2: signed bytes.
+ *   bf16 instruction, 1: f16, 2: signed bytes; kind 8: the inner loop of the signed-byte nearest-neighbour filter
+ *   without its memory traffic (per round two query sets of two dependent v_mfma_i32_32x32x32_i8 and the minimum
+ *   over the 16 results of a set), chains = 0: minima over the results, 1: over registers that no matrix instruction
+ *   writes, 2: no vector work.
  * Measurement aid without counterpart in the reference; used by bench.py --valu-calibration / --mfma-calibration.
  */
 int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave);

@@ -371,6 +371,60 @@ static __global__ void __launch_bounds__(256) keops_mfma_stream_loop(float* out,
   out[(size_t)blockIdx.x * 256 + threadIdx.x] = r;
 }
 
+// The inner loop of the signed-byte nearest-neighbour filter without its memory traffic: per round two query sets,
+// each two dependent v_mfma_i32_32x32x32_i8 from a constant accumulator, and the minimum over the 16 results of a
+// set (v_min3_i32 chain, one compare) taken while the other set's instructions are in the pipe.  MODE 0: as
+// described; 1: the minima read registers that no matrix instruction writes (same instruction count, no dependence
+// on the matrix results); 2: no vector work.
+template <int MODE>
+static __global__ void __launch_bounds__(256) keops_mfma_screen_loop(float* out, int iters) {
+  keops_i32x4 a[2], b[2];
+  unsigned h = 0x9e3779b9u * (threadIdx.x + 1u);
+#pragma unroll
+  for (int k = 0; k < 2; k++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      h = h * 1664525u + 1013904223u;
+      a[k][e] = (int)h;
+      h = h * 1664525u + 1013904223u;
+      b[k][e] = (int)h;
+    }
+  keops_i32x16 c0, acc[2], other;
+#pragma unroll
+  for (int e = 0; e < 16; e++) {
+    c0[e] = (int)(h >> 20) + e;
+    other[e] = (int)(h >> 12) - e;
+    acc[0][e] = acc[1][e] = 0;
+  }
+  int hits = 0;
+  int thr = -(1 << 30);
+  asm volatile("" : "+v"(thr));
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[0], b[c], c0, 0, 0, 0);
+      acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[1], b[1 - c], acc[c], 0, 0, 0);
+      if (MODE != 2) {
+        keops_i32x16 src = MODE == 0 ? acc[1 - c] : other;
+        if (MODE == 1) asm volatile("" : "+v"(src));
+        int m = src[0] < src[1] ? src[0] : src[1];
+#pragma unroll
+        for (int e = 2; e < 16; e += 2) {
+          const int t = m < src[e] ? m : src[e];
+          m = t < src[e + 1] ? t : src[e + 1];
+        }
+        hits += m <= thr ? 1 : 0;
+      }
+    }
+  }
+  int r = hits;
+#pragma unroll
+  for (int c = 0; c < 2; c++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) r += acc[c][e];
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = (float)r;
+}
+
 // `iters` rounds of 8 v_mfma_f32_32x32x16_bf16 (two dependent chains of 4, the shape of the K-nearest-neighbour
 // filter) with NV independent v_fmac_f32 between them: how much vector work fits beside a saturated matrix pipe
 template <int NV>
@@ -421,7 +475,8 @@ static __global__ void __launch_bounds__(256) keops_mix_loop(float* out, int ite
 // kind 0/1/2: vector loop with MIX = kind; kind 3 / 4: matrix loop on bf16 / f16 operands; kind 6: on signed bytes
 // (v_mfma_i32_32x32x32_i8); kind 5: 8 bf16 matrix
 // instructions per round with `chains` v_fmac_f32 after each of them (0, 1, 2, 4, 8); kind 7: 32 matrix instructions
-// per round whose operands change with every instruction, `chains` = 0 bf16, 1 f16, 2 signed bytes.
+// per round whose operands change with every instruction, `chains` = 0 bf16, 1 f16, 2 signed bytes; kind 8: the loop of
+// the signed-byte nearest-neighbour filter without memory traffic, `chains` = 0, 1, 2 (see keops_mfma_screen_loop).
 // chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
 // instr_per_lane receives the number of counted instructions one wavefront issues (vector: per lane = per wavefront
 // instruction count; matrix: v_mfma instructions).  out must hold blocks * 256 floats.
@@ -463,6 +518,13 @@ int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* o
     if (chains == 0) hipLaunchKernelGGL((keops_mfma_stream_loop<0>), g, b, 0, s, out, iters);
     else if (chains == 1) hipLaunchKernelGGL((keops_mfma_stream_loop<1>), g, b, 0, s, out, iters);
     else if (chains == 2) hipLaunchKernelGGL((keops_mfma_stream_loop<2>), g, b, 0, s, out, iters);
+    else return (int)hipErrorInvalidValue;
+  } else if (kind == 8) {
+    // chains = 0: minima over the other set's results, 1: over registers no matrix instruction writes, 2: none
+    *instr_per_wave = 4.0 * (double)iters;
+    if (chains == 0) hipLaunchKernelGGL((keops_mfma_screen_loop<0>), g, b, 0, s, out, iters);
+    else if (chains == 1) hipLaunchKernelGGL((keops_mfma_screen_loop<1>), g, b, 0, s, out, iters);
+    else if (chains == 2) hipLaunchKernelGGL((keops_mfma_screen_loop<2>), g, b, 0, s, out, iters);
     else return (int)hipErrorInvalidValue;
   } else if (kind == 5) {
     // chains = vector instructions per matrix instruction: 0, 1, 2, 4, 8
