@@ -55,6 +55,11 @@ def set_device(tagCPUGPU, tagHostDevice, device_id_request, *args):
 class GenredAutograd_base:
     @staticmethod
     def _forward(params, *args):
+        result, dimout, tagIJ = GenredAutograd_base._launch(params, *args)
+        return result, torch.tensor([dimout, tagIJ])
+
+    @staticmethod
+    def _launch(params, *args):
         params.optional_flags["multVar_highdim"] = (
             1 if isinstance(params.rec_multVar_highdim, int) and not isinstance(params.rec_multVar_highdim, bool)
             or params.rec_multVar_highdim else 0
@@ -123,7 +128,7 @@ class GenredAutograd_base:
             result = host_out
         elif staged:
             result = result.cpu()
-        return result, torch.tensor([myconv.dimout, myconv.tagIJ])
+        return result, myconv.dimout, myconv.tagIJ
 
     @staticmethod
     def _setup_context(ctx, inputs, outputs):
@@ -232,8 +237,19 @@ class GenredAutograd(torch.autograd.Function):
         return GenredAutograd_base._backward(ctx, G, _)
 
 
-def GenredAutograd_fun(*inputs):
-    return GenredAutograd.apply(*inputs)[0]
+def _nothing_to_differentiate(args):
+    """No argument asks for a gradient, no forward-mode level and no function transform (vmap, grad, jvp) is active."""
+    if torch._C._functorch.peek_interpreter_stack() is not None or torch.autograd.forward_ad._current_level >= 0:
+        return False
+    return not (torch.is_grad_enabled() and any(a.requires_grad for a in args))
+
+
+def GenredAutograd_fun(params, *args):
+    # the autograd machinery around a launch (argument binding, context, saved tensors) costs as much as a small
+    # launch itself: when there is nothing to differentiate the result is the same without it
+    if _nothing_to_differentiate(args):
+        return GenredAutograd_base._launch(params, *args)[0]
+    return GenredAutograd.apply(params, *args)[0]
 
 
 class Genred:
