@@ -39,6 +39,24 @@ def _broadcast_batch(a, b):
 
 
 _genred_cache = {}
+_constants = {}
+
+
+def _constant_tensor(value, dtype, device):
+    """Device tensor of a Python number or list of numbers used as a parameter; the same constants recur on every
+    pass of an iterative algorithm, and building one costs a host-to-device copy."""
+    key = (tuple(value) if isinstance(value, (list, tuple)) else value, dtype, device)
+    try:
+        t = _constants.get(key)
+    except TypeError:  # nested lists and the like
+        return torch.tensor(value, dtype=dtype, device=device)
+    if t is None:
+        if len(_constants) >= 256:
+            _constants.clear()
+        t = _constants[key] = torch.tensor(value, dtype=dtype, device=device)
+    return t
+
+
 
 
 class LazyTensor:
@@ -552,7 +570,7 @@ class LazyTensor:
             if pos[pid] not in cats:
                 continue
             if not isinstance(t, torch.Tensor):
-                t = torch.tensor(t, dtype=dtype, device=dev)
+                t = _constant_tensor(t, dtype, dev)
             want = nb + (1 if cats[pos[pid]] == 2 else 2)
             if t.dim() < want:
                 t = t.view((1,) * (want - t.dim()) + tuple(t.shape))
