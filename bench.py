@@ -255,16 +255,20 @@ def calibration(mfma):
              (7, "two chains, operands change with every instruction (chains = 0: bf16, 1: f16, 2: i8)", (0, 1, 2)),
              (8, "byte filter loop without memory traffic: 4 v_mfma_i32_32x32x32_i8 and two 16-value minima per round "
                  "(chains = 0: minima over the results, 1: over other registers, 2: no minima)", (2, 1, 0)),
+             (9, "contraction loop of the chunked kernel alone: hi/lo half-precision rows in registers, tiles streamed "
+                 "through LDS, 48 v_mfma_f32_32x32x16_f16 per round (chains = 0: constant operands, 1: random)", (0, 1)),
              (5, "two chains of v_mfma_f32_32x32x16_bf16 with `chains` v_fmac_f32 after every matrix instruction", (0, 1, 2, 4, 8))] if mfma else [
         (0, "v_fmac_f32 chains", (1, 2, 4, 8)), (1, "Gaussian pair mix with v_exp_f32 (9 instr)", (1, 2, 4, 8)),
         (2, "Gaussian pair mix without v_exp_f32 (8 instr)", (1, 2, 4, 8))]
     for kind, label, chain_set in kinds:
         for chains in chain_set:
-            for waves in (1, 2, 4):
-                blocks = cus * waves  # one workgroup = 4 wavefronts = one per SIMD of a CU
-                iters = 200_000 // chains if kind < 3 else (12_500 if kind == 7 else (100_000 if kind == 8 else (100_000 // chains if kind != 5 else 50_000)))
+            # one workgroup = 4 wavefronts = one per SIMD of a CU (kind 9: 8 wavefronts, at most two workgroups per CU)
+            wg_waves = 8 if kind == 9 else 4
+            for wgs in ((1, 2) if kind == 9 else (1, 2, 4)):
+                blocks, waves = cus * wgs, wgs * wg_waves // 4
+                iters = {7: 12_500, 8: 100_000, 5: 50_000, 9: 4_000}.get(kind) or (200_000 if kind < 3 else 100_000) // chains
                 ms, ipw = binder.calibrate(kind, chains, blocks, iters)
-                total = ipw * blocks * 4  # wavefront instructions
+                total = ipw * blocks * wg_waves  # wavefront instructions
                 per_cycle = total / (ms * 1e-3) / simds / clock
                 row = dict(kind=label, chains=chains, waves_per_simd=waves, ms=round(ms, 3),
                            wave_instr_per_cycle_per_simd_at_2p4GHz=round(per_cycle, 4))

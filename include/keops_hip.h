@@ -184,7 +184,10 @@ int keops_hip_path_status(void* module, unsigned* taken);
  *   bf16 instruction, 1: f16, 2: signed bytes; kind 8: the inner loop of the signed-byte nearest-neighbour filter
  *   without its memory traffic (per round two query sets of two dependent v_mfma_i32_32x32x32_i8 and the minimum
  *   over the 16 results of a set), chains = 0: minima over the results, 1: over registers that no matrix instruction
- *   writes, 2: no vector work.
+ *   writes, 2: no vector work; kind 9: the contraction loop of the high-dimensional chunked kernel on its own
+ *   (workgroups of 8 wavefronts, 32 rows of 256 components per wavefront in registers as hi and lo half-precision
+ *   operands, 32-row tiles streamed through LDS, 48 v_mfma_f32_32x32x16_f16 per round and wavefront, no vector
+ *   work), chains = 0: every operand the same constant, 1: random operands with the magnitudes of real data.
  * Measurement aid without counterpart in the reference; used by bench.py --valu-calibration / --mfma-calibration.
  */
 int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave);

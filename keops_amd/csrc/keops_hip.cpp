@@ -1928,7 +1928,7 @@ int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int ite
   if (!ms || !instr_per_wave || blocks <= 0 || iters <= 0) return fail(-1, "keops_hip_calibrate: bad arguments");
   HIP_TRY(hipSetDevice(device_id < 0 ? 0 : device_id));
   float* out = nullptr;
-  HIP_TRY(hipMalloc((void**)&out, (size_t)blocks * 256 * sizeof(float)));
+  HIP_TRY(hipMalloc((void**)&out, (size_t)blocks * 256 * sizeof(float) + KEOPS_STATIC_STREAM_BYTES));
   hipEvent_t e0 = nullptr, e1 = nullptr;
   int rc = 0;
   auto cleanup = [&] { if (e0) (void)hipEventDestroy(e0); if (e1) (void)hipEventDestroy(e1); (void)hipFree(out); };
@@ -1943,7 +1943,7 @@ int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int ite
   float t = 0.f;
   if (rc == 0 && hipEventElapsedTime(&t, e0, e1) != hipSuccess) rc = -1;
   cleanup();
-  if (rc != 0) return fail(rc, "calibration loop failed (kind 0-2: chains 1, 2, 4, 8; kind 3: chains 1, 2, 4)");
+  if (rc != 0) return fail(rc, "calibration loop failed: kind or chains out of range (see keops_hip_calibrate in keops_hip.h)");
   *ms = t;
   return 0;
 }

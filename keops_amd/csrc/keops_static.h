@@ -11,6 +11,8 @@ int keops_static_scratch(int device, void** ptr, size_t* bytes);
 int keops_static_fill_zero(void* dst, size_t bytes, void* stream);
 // n elements: IEEE half -> float (to_float != 0) or float -> half (round to nearest even)
 int keops_static_convert_half(void* dst, const void* src, long long n, int to_float, void* stream);
+// out: blocks * 256 floats, followed by KEOPS_STATIC_STREAM_BYTES of tile data for the kinds that stream tiles
+#define KEOPS_STATIC_STREAM_BYTES ((size_t)64 * 32 * 512 * 2)
 int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* out, void* stream, double* instr_per_wave);
 
 // Lookup table of a block-sparse launch built on the device (no read-back of the ranges): see keops_static.hip.

@@ -371,6 +371,81 @@ static __global__ void __launch_bounds__(256) keops_mfma_stream_loop(float* out,
   out[(size_t)blockIdx.x * 256 + threadIdx.x] = r;
 }
 
+// The contraction loop of the high-dimensional chunked kernel on its own: 8 wavefronts per workgroup, each with 32
+// rows of 256 components in registers as hi and lo half-precision operands, a 32-row tile (hi | lo, 1024 bytes per
+// row) brought straight from memory to LDS one round ahead (two buffers, one barrier per round), per k block two LDS
+// reads and three v_mfma_f32_32x32x16_f16 (lo*hi, hi*lo, hi*hi).  No vector work, no weighted sum.  RANDOM = 0: every
+// operand is the same constant; 1: random signs and significands, hi parts near 2^11, lo parts near 1, like the split
+// operands of real data.  `tiles`: KEOPS_STREAM_TILES tiles of 32 x 512 half-precision numbers, swept cyclically.
+#define KEOPS_STREAM_TILES 64
+template <int RANDOM>
+static __global__ void __launch_bounds__(256) keops_stream_fill(_Float16* tiles) {
+  const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;   // one half-precision number each
+  unsigned h = 0x9e3779b9u * (unsigned)(e + 1u);
+  h = h * 1664525u + 1013904223u;
+  const float u = (float)((h >> 8) & 0xffff) * (1.0f / 32768.0f) - 1.0f;
+  tiles[e] = RANDOM ? (_Float16)(((e & 511) < 256 ? 4000.f : 2.f) * u) : (_Float16)1.0586f;
+}
+
+template <int RANDOM>
+static __global__ void __launch_bounds__(512) keops_stream_loop(float* out, const _Float16* tiles, int iters) {
+  constexpr int STRIDE = 1024 + 16;
+  __shared__ __attribute__((aligned(16))) unsigned char as[2][32 * STRIDE];
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, col = lane & 31;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  keops_f16x8 bh[16], bl[16];
+  unsigned h = 0x9e3779b9u * (unsigned)(blockIdx.x * 512 + tid + 1u);
+#pragma unroll
+  for (int kb = 0; kb < 16; kb++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      h = h * 1664525u + 1013904223u;
+      const float u = (float)((h >> 8) & 0xffff) * (1.0f / 32768.0f) - 1.0f;
+      bh[kb][e] = RANDOM ? (_Float16)(4000.f * u) : (_Float16)1.0586f;
+      h = h * 1664525u + 1013904223u;
+      const float w = (float)((h >> 8) & 0xffff) * (1.0f / 32768.0f) - 1.0f;
+      bl[kb][e] = RANDOM ? (_Float16)(2.f * w) : (_Float16)1.0586f;
+    }
+  if (tid < 2) as[tid][0] = 0;  // (an array the compiler sees no store to would count as uninitialised)
+  __syncthreads();
+  auto stage = [&](int t) {
+    const _Float16* src = tiles + (size_t)(t % KEOPS_STREAM_TILES) * 32 * 512;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int row = wave + 8 * r;
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src + row * 512) + lane,
+                                       &as[0][0] + __builtin_amdgcn_readfirstlane((t & 1) * 32 * STRIDE + row * STRIDE), 16, 0, 0);
+    }
+  };
+  keops_f32x16 tot;
+#pragma unroll
+  for (int v = 0; v < 16; v++) tot[v] = 0.f;
+  stage(0);
+  for (int t = 0; t < iters; t++) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's rows of tile t have landed
+    __syncthreads();                     // everybody's have, and tile t - 1 has been consumed
+    if (t + 1 < iters) stage(t + 1);
+    const unsigned char* arow = as[t & 1] + col * STRIDE + 16 * half;
+    keops_f32x16 s;
+#pragma unroll
+    for (int v = 0; v < 16; v++) s[v] = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 16; kb++) {
+      const keops_f16x8 ah = *reinterpret_cast<const keops_f16x8*>(arow + kb * 32);
+      const keops_f16x8 al = *reinterpret_cast<const keops_f16x8*>(arow + 512 + kb * 32);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[kb], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[kb], s, 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) tot[v] += s[v] * 1e-12f;
+  }
+  float r = 0.f;
+#pragma unroll
+  for (int v = 0; v < 16; v++) r += tot[v];
+  out[(size_t)blockIdx.x * 256 + (tid & 255)] = r;
+}
+
 // The inner loop of the signed-byte nearest-neighbour filter without its memory traffic: per round two query sets,
 // each two dependent v_mfma_i32_32x32x32_i8 from a constant accumulator, and the minimum over the 16 results of a
 // set (v_min3_i32 chain, one compare) taken while the other set's instructions are in the pipe.  MODE 0: as
@@ -476,7 +551,9 @@ static __global__ void __launch_bounds__(256) keops_mix_loop(float* out, int ite
 // (v_mfma_i32_32x32x32_i8); kind 5: 8 bf16 matrix
 // instructions per round with `chains` v_fmac_f32 after each of them (0, 1, 2, 4, 8); kind 7: 32 matrix instructions
 // per round whose operands change with every instruction, `chains` = 0 bf16, 1 f16, 2 signed bytes; kind 8: the loop of
-// the signed-byte nearest-neighbour filter without memory traffic, `chains` = 0, 1, 2 (see keops_mfma_screen_loop).
+// the signed-byte nearest-neighbour filter without memory traffic, `chains` = 0, 1, 2 (see keops_mfma_screen_loop);
+// kind 9: the contraction loop of the high-dimensional chunked kernel on its own (keops_stream_loop; workgroups of 8
+// wavefronts, `chains` = 0 constant / 1 random operands; out needs KEOPS_STATIC_STREAM_BYTES more bytes).
 // chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
 // instr_per_lane receives the number of counted instructions one wavefront issues (vector: per lane = per wavefront
 // instruction count; matrix: v_mfma instructions).  out must hold blocks * 256 floats.
@@ -519,6 +596,21 @@ int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* o
     else if (chains == 1) hipLaunchKernelGGL((keops_mfma_stream_loop<1>), g, b, 0, s, out, iters);
     else if (chains == 2) hipLaunchKernelGGL((keops_mfma_stream_loop<2>), g, b, 0, s, out, iters);
     else return (int)hipErrorInvalidValue;
+  } else if (kind == 9) {
+    // workgroups of 8 wavefronts; chains = 0: constant operands, 1: random ones; 48 matrix instructions per round.
+    // out: blocks * 256 floats followed by KEOPS_STREAM_TILES * 32 * 512 half-precision numbers of tile data
+    *instr_per_wave = 48.0 * (double)iters;
+    _Float16* tiles = reinterpret_cast<_Float16*>(out + (size_t)blocks * 256);
+    const dim3 gf(KEOPS_STREAM_TILES * 32 * 512 / 256), b8(512);
+    if (chains == 0) {
+      hipLaunchKernelGGL((keops_stream_fill<0>), gf, b, 0, s, tiles);
+      hipLaunchKernelGGL((keops_stream_loop<0>), g, b8, 0, s, out, tiles, iters);
+    } else if (chains == 1) {
+      hipLaunchKernelGGL((keops_stream_fill<1>), gf, b, 0, s, tiles);
+      hipLaunchKernelGGL((keops_stream_loop<1>), g, b8, 0, s, out, tiles, iters);
+    } else {
+      return (int)hipErrorInvalidValue;
+    }
   } else if (kind == 8) {
     // chains = 0: minima over the other set's results, 1: over registers no matrix instruction writes, 2: none
     *instr_per_wave = 4.0 * (double)iters;
