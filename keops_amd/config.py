@@ -55,6 +55,7 @@ radial = os.environ.get("KEOPS_AMD_RADIAL", "1") != "0"
 radial_fold = os.environ.get("KEOPS_AMD_RADIAL_FOLD", "0") == "1"
 radial_max_dim = 8                  # components of the points (7 D + 8 slots of the scalar product fit four instructions)
 radial_max_dv = 8                   # components of the weights (16 accumulators per component in every lane)
+radial_mm_max_dv = 10               # ... when the weighted sum runs on the matrix cores (three terms of the weights in 32 operand columns)
 # the path is taken when |c| log2(e) (max |x^|^2 + max |y^|^2) <= this bound for the centred points (checked on the
 # device): the exponent is then off by at most 8 * 2^-24 of it, a kernel value by 7e-5 at worst and 1e-6 typically
 radial_rb2_max_dv = int(os.environ.get("KEOPS_AMD_RADIAL_RB2_MAX_DV", 4))  # two 32-row blocks per wavefront up to this many accumulated components
@@ -63,6 +64,11 @@ radial_rb2_max_dv = int(os.environ.get("KEOPS_AMD_RADIAL_RB2_MAX_DV", 4))  # two
 # accumulated components from which the weighted sum of the radial scheme runs on the matrix cores (per pair the vector
 # ALU then issues v_exp_f32 and a three-term split instead of one fused multiply-add per component); 99: never
 radial_mm_min_dv = int(os.environ.get("KEOPS_AMD_RADIAL_MM_MIN_DV", 7))
+# bfloat16 terms of a kernel value in that product: 3 (24 bits: the float32 class) or 2 (both rounded to nearest:
+# every kernel value is then off by up to 2^-17, 2.4e-6 rms, forty times the float32 rounding, which sums with
+# cancellation do not forgive; 199 against 263 ms at eight components on 10^6 x 10^6 points, and the matrix cores
+# then win from five components on: KEOPS_AMD_RADIAL_MM_MIN_DV=5)
+radial_mm_terms = int(os.environ.get("KEOPS_AMD_RADIAL_MM_TERMS", 3))
 radial_mm_rb = int(os.environ.get("KEOPS_AMD_RADIAL_MM_RB", 1))   # 32-row blocks per wavefront in that variant
 radial_tile_j = os.environ.get("KEOPS_AMD_RADIAL_TJ", "auto")
 radial_limit = float(os.environ.get("KEOPS_AMD_RADIAL_LIMIT", 128.0))
@@ -77,6 +83,9 @@ final_max_blocks = int(os.environ.get("KEOPS_AMD_FINAL_NB", 8))            # 32-
 final_waves = int(os.environ.get("KEOPS_AMD_FINAL_WAVES", 8))              # wavefronts (32 output rows each) per workgroup
 final_tile_j = int(os.environ.get("KEOPS_AMD_FINAL_TJ", 32))               # reduced rows per staged tile (even)
 final_split3 = os.environ.get("KEOPS_AMD_FINAL_SPLIT3", "1") != "0"          # product in three bfloat16 terms per operand
+# ... of the staged vectors and of the per-pair weights; 2: the weights in two terms, both rounded to nearest (off by up
+# to 2^-17 each, 2.4e-6 rms: not the float32 class; C5b 68.8 against 70.6 ms, softmax_d64 4.70 against 5.09 ms)
+final_weight_terms = int(os.environ.get("KEOPS_AMD_FINAL_WEIGHT_TERMS", 3))
 final_period = int(os.environ.get("KEOPS_AMD_FINAL_PERIOD", 4096))         # block-sum period in reduced rows
 
 # matrix-core KNN kernel (csrc/kernels/keops_knn_mfma.h)

@@ -744,7 +744,12 @@ __device__ __forceinline__ void chk_v3_scatter(__bf16* bt3, int tid, const float
   }
 }
 
-// acc[b] += W (32 output rows x 32 reduced rows, the 16 weights w of this lane) * v (staged terms bt3)
+// acc[b] += W (32 output rows x 32 reduced rows, the 16 weights w of this lane) * v (staged terms bt3).
+// CHK_WTERMS bfloat16 terms per weight: 3 (24 bits, six term products) or 2 (w = h + m with both terms rounded to
+// nearest: |w - h - m| <= 2^-17 |w|, either sign; five term products, less vector work; not the float32 class).
+#ifndef CHK_WTERMS
+#define CHK_WTERMS 3
+#endif
 __device__ __forceinline__ void chk_v3_product(const float (&w)[16], const __bf16* bt3, int col, int half,
                                                chk_f32x16 (&acc)[CHK_FNB]) {
 #pragma unroll
@@ -758,7 +763,7 @@ __device__ __forceinline__ void chk_v3_product(const float (&w)[16], const __bf1
       const __bf16 m = (__bf16)r1;
       ah[e] = h;
       am[e] = m;
-      al[e] = (__bf16)(r1 - (float)m);
+      if (CHK_WTERMS == 3) al[e] = (__bf16)(r1 - (float)m);
     }
     const __bf16* brow = bt3 + col * CHK_TS + 16 * kb + 8 * half;
 #pragma unroll
@@ -768,7 +773,7 @@ __device__ __forceinline__ void chk_v3_product(const float (&w)[16], const __bf1
       const chk_bf16x8 bl = *reinterpret_cast<const chk_bf16x8*>(brow + (2 * CHK_VCOLS + 32 * b) * CHK_TS);
       // smallest terms first
       acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am, bm, acc[b], 0, 0, 0);
-      acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh, acc[b], 0, 0, 0);
+      if (CHK_WTERMS == 3) acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh, acc[b], 0, 0, 0);
       acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl, acc[b], 0, 0, 0);
       acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am, bh, acc[b], 0, 0, 0);
       acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bm, acc[b], 0, 0, 0);

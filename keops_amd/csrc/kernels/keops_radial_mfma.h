@@ -55,6 +55,8 @@
 
 typedef __bf16 rad_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float rad_f32x16 __attribute__((ext_vector_type(16)));
+typedef float rad_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 rad_bf16x2 __attribute__((ext_vector_type(2)));
 
 #ifndef RAD_TJ
 #define RAD_TJ 128                 // columns per staged tile
@@ -63,6 +65,9 @@ typedef float rad_f32x16 __attribute__((ext_vector_type(16)));
 #define RAD_MM 0                   // 1: the weighted sum runs on the matrix cores too (see rad_sweep_mm)
 #endif
 #define RAD_MM_FOLD 4096           // columns between two folds of the running sums (block summation)
+#ifndef RAD_MM_TERMS
+#define RAD_MM_TERMS 3             // bfloat16 terms of a kernel value in the second product (3: truncated, exact; 2: rounded)
+#endif
 #define RAD_NSUB (RAD_TJ / 32)
 #define RAD_SLOTS (16 * RAD_NKB)
 #define RAD_BLOCK (64 * RAD_WAVES)
@@ -629,6 +634,26 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
         for (int kb = 0; kb < RAD_NKB; kb++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[kb], a[r][kb], z, 0, 0, 0);
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
+#if RAD_MM_TERMS == 2
+          // K = h + m: h the bfloat16 nearest to K, m the bfloat16 nearest to the (exact) rest, |K - h - m| <= 2^-17 K
+          // with either sign (an option: forty times the float32 rounding).  v_cvt_pk_bf16_f32 rounds and packs two values at once; a shift / a mask give h back as
+          // a float.
+          uint4 ph, pm;
+          unsigned* php = reinterpret_cast<unsigned*>(&ph);
+          unsigned* pmp = reinterpret_cast<unsigned*>(&pm);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float x0 = __builtin_amdgcn_exp2f(z[8 * kb + 2 * e]), x1 = __builtin_amdgcn_exp2f(z[8 * kb + 2 * e + 1]);
+            const rad_f32x2 xx = {x0, x1};
+            const unsigned hp = __builtin_bit_cast(unsigned, __builtin_convertvector(xx, rad_bf16x2));
+            php[e] = hp;
+            const rad_f32x2 rr = {x0 - __uint_as_float(hp << 16), x1 - __uint_as_float(hp & 0xffff0000u)};
+            pmp[e] = __builtin_bit_cast(unsigned, __builtin_convertvector(rr, rad_bf16x2));
+          }
+          const rad_bf16x8 kh = __builtin_bit_cast(rad_bf16x8, ph), km = __builtin_bit_cast(rad_bf16x8, pm);
+          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(km, wk[kb], acc[r], 0, 0, 0);
+          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, wk[kb], acc[r], 0, 0, 0);
+#else
           // K = h + m + l, each the truncation of what is left to 8 significant bits (the subtractions are exact); a
           // byte permute packs the high halves of two floats: the bfloat16 terms.  (v_dot2_f32_bf16 against the pairs
           // (-1, 0) / (0, -1) subtracts a packed term in one instruction instead of v_and + v_sub: measured, same time.)
@@ -653,6 +678,7 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
           acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kl, wk[kb], acc[r], 0, 0, 0);
           acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(km, wk[kb], acc[r], 0, 0, 0);
           acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, wk[kb], acc[r], 0, 0, 0);
+#endif
         }
       }
     }

@@ -610,6 +610,7 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
         defs["CHK_SINGLE"] = 1
     defs["CHK_NEAR"] = f"{near!r}f"
     defs["CHK_SPLIT3"] = split3
+    defs["CHK_WTERMS"] = int(config.final_weight_terms)
     defs["CHK_PRESPLIT"] = int(config.chunk_presplit)
     src += [f"#define {k} {v}" for k, v in defs.items()]
     for name, vals in (("row_arg", ra), ("row_dim", rd), ("row_off", ro), ("col_arg", ca), ("col_dim", cd),
@@ -864,7 +865,7 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
     if diff:
         if x.dim + 1 > config.radial_max_dv or red.formula.dim != x.dim:
             return None
-    elif dimw != red.formula.dim or not 1 <= dimw <= config.radial_max_dv:
+    elif dimw != red.formula.dim or not 1 <= dimw <= max(config.radial_max_dv, config.radial_mm_max_dv if config.radial_mm_min_dv <= dimw else 0):
         return None
 
     def product(fs):
@@ -922,6 +923,8 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     # from config.radial_mm_min_dv accumulated components on, the weighted sum runs on the matrix cores too (the three
     # bfloat16 terms of the weights side by side in the 32 operand columns): 16 accumulators per block of 32 rows
     mm = int(config.radial_mm_min_dv <= Dv and 3 * Dv <= 32 and not rows_per_block)
+    if Dv > config.radial_max_dv and not mm:
+        return None, None  # the accumulators of that many components do not fit the registers
     rb = (config.radial_mm_rb if mm else 2) if (mm or Dv <= config.radial_rb2_max_dv) else 1
     tj = ((256 if mm else 128 if Dv <= 2 else 512) if config.radial_tile_j == "auto" else int(config.radial_tile_j))
     if tj % 32 or not 32 <= tj <= 1024:
@@ -963,7 +966,7 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
                 rad_yarg=y.ind, rad_fold=fold, rad_tj=tj)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
-    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
+    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
                 RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit)!r}f",
                 RAD_NCOLVARS=len(wl.colvars), RAD_DIMY=wl.dimy, RAD_NROWVARS=len(al.rowvars), RAD_DIMX=al.dimx)
     src += [f"#define {k} {v}" for k, v in defs.items()]
@@ -1020,7 +1023,7 @@ def get_keops_dll(
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
            use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs), int(batch_total),
            binder.templates_digest(), bool(config.radial), bool(config.radial_fold), bool(config.radial_ranges), int(config.radial_mm_min_dv),
-           int(config.radial_mm_rb), bool(config.knn_i8), bool(use_half))
+           int(config.radial_mm_rb), int(config.radial_mm_terms), bool(config.knn_i8), bool(use_half))
     with _lock:
         hit = _cache.get(key)
     if hit is not None:

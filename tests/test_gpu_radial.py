@@ -32,7 +32,7 @@ def _last_meta(key):
 
 
 @pytest.mark.parametrize("D,Dv,M,N", [(3, 1, 30011, 30500), (3, 8, 20000, 21000), (3, 2, 300000, 1001), (5, 3, 17000, 23001),
-                                      (8, 1, 16000, 18000), (2, 4, 33333, 10001), (6, 7, 18011, 19003)])
+                                      (8, 1, 16000, 18000), (2, 4, 33333, 10001), (6, 7, 18011, 19003), (3, 10, 17000, 16500)])
 def test_gaussian_sums_with_matrix_core_exponents_vs_oracle(D, Dv, M, N):
     rng = np.random.default_rng(100 * D + Dv)
     x = rng.standard_normal((M, D)).astype(np.float32)
