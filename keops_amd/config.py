@@ -55,7 +55,7 @@ radial = os.environ.get("KEOPS_AMD_RADIAL", "1") != "0"
 radial_fold = os.environ.get("KEOPS_AMD_RADIAL_FOLD", "0") == "1"
 radial_max_dim = 8                  # components of the points (7 D + 8 slots of the scalar product fit four instructions)
 radial_max_dv = 8                   # components of the weights (16 accumulators per component in every lane)
-radial_mm_max_dv = 10               # ... when the weighted sum runs on the matrix cores (three terms of the weights in 32 operand columns)
+radial_mm_max_dv = 32               # ... when the weighted sum runs on the matrix cores (the three terms of the weights in up to three blocks of 32 operand columns)
 # the path is taken when |c| log2(e) (max |x^|^2 + max |y^|^2) <= this bound for the centred points (checked on the
 # device): the exponent is then off by at most 8 * 2^-24 of it, a kernel value by 7e-5 at worst and 1e-6 typically
 radial_rb2_max_dv = int(os.environ.get("KEOPS_AMD_RADIAL_RB2_MAX_DV", 4))  # two 32-row blocks per wavefront up to this many accumulated components

@@ -682,7 +682,8 @@ int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* arg
   const size_t o_scal = take(32), o_colsum = take((size_t)D * 4), o_colpart = take((size_t)nparts * D * 4);
   const size_t o_blk = take(fold ? (size_t)nblk * 4 : 0);
   // weights of a column: RAD_DV floats, or 32 bfloat16 operand columns when the weighted sum runs on the matrix cores
-  const size_t wbytes = m.meta_int("rad_mm", 0) != 0 ? 64 : (size_t)DV * 4;
+  // (three terms of every weight: one block of 32 columns up to ten weights, rad_mm_nb blocks beyond)
+  const size_t wbytes = m.meta_int("rad_mm", 0) != 0 ? 64 * (size_t)std::max<int64_t>(1, m.meta_int("rad_mm_nb", 1)) : (size_t)DV * 4;
   const size_t o_xa = take((size_t)nx * NKB * 32), o_yb = take((size_t)ntiles * TJ * NKB * 32), o_bw = take((size_t)ntiles * TJ * wbytes);
   const size_t o_part = take((size_t)nslabs * nx * DV * 4);
   if (int rc = m.partial.reserve(off)) return rc;

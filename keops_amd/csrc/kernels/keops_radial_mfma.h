@@ -65,6 +65,7 @@ typedef __bf16 rad_bf16x2 __attribute__((ext_vector_type(2)));
 #define RAD_MM 0                   // 1: the weighted sum runs on the matrix cores too (see rad_sweep_mm)
 #endif
 #define RAD_MM_FOLD 4096           // columns between two folds of the running sums (block summation)
+#define RAD_MM_NB ((3 * RAD_DV + 31) / 32)  // 32-column blocks of the B operand of the second product
 #ifndef RAD_MM_TERMS
 #define RAD_MM_TERMS 3             // bfloat16 terms of a kernel value in the second product (3: truncated, exact; 2: rounded)
 #endif
@@ -239,12 +240,13 @@ __device__ __forceinline__ void rad_split4(double v, __bf16 (&t)[4]) {
 // [w_h | w_m | w_l | 0] (the three bfloat16 terms of the RAD_DV weights side by side), contraction index = the 32
 // columns of a sub-tile in the order in which the exponent tile leaves them in the registers of a lane: registers
 // 0-7 (k block 0) of lanes 0-31 hold columns {0,1,2,3,8,9,10,11}, of lanes 32-63 {4,...,7,12,...,15}; registers 8-15
-// (k block 1) the same plus 16.  Layout [32-column sub-tile][k block][half][operand column][8].
+// (k block 1) the same plus 16.  Layout [32-column sub-tile][k block][half][operand column][8]; beyond ten weights the
+// 3 * RAD_DV operand columns take RAD_MM_NB blocks of 32.
 __device__ __forceinline__ void rad_store_weights_mm(__bf16* bwm, i64 j, const float (&w)[RAD_DV]) {
   const int jj = (int)(j & 31), kb = jj >> 4, q = jj & 15, hf = (q >> 2) & 1, e = (q & 3) + 4 * (q >> 3);
-  __bf16* dst = bwm + ((((j >> 5) * 2 + kb) * 2 + hf) * 32) * 8 + e;
+  __bf16* dst = bwm + ((((j >> 5) * 2 + kb) * 2 + hf) * (32 * RAD_MM_NB)) * 8 + e;
 #pragma unroll
-  for (int n = 0; n < 32; n++) {
+  for (int n = 0; n < 32 * RAD_MM_NB; n++) {
     __bf16 v = (__bf16)0.0f;
     if (n < 3 * RAD_DV) {
       __bf16 t3[3];
@@ -403,7 +405,7 @@ __device__ __forceinline__ i64 rad_tile_of(i64 k, i64 pos_tiles, i64 all_tiles, 
 
 // with at most 32 accumulators per lane the kernel fits 128 registers: four wavefronts per SIMD, two workgroups per CU
 #if RAD_MM
-#define RAD_MIN_WAVES (RAD_RB == 1 ? 4 : 2)
+#define RAD_MIN_WAVES (RAD_MM_NB > 1 ? 1 : (RAD_RB == 1 ? 4 : 2))  // (several operand blocks: 32 accumulators each)
 #else
 #define RAD_MIN_WAVES ((RAD_RB * 16 * RAD_DV <= 32) ? 4 : 1)
 #endif
@@ -573,16 +575,18 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
 #pragma unroll
     for (int kb = 0; kb < RAD_NKB; kb++) a[r][kb] = *reinterpret_cast<const rad_bf16x8*>(S.xa + i * RAD_SLOTS + kb * 16 + 8 * half);
   }
-  rad_f32x16 acc[RAD_RB], tot[RAD_RB];
+  rad_f32x16 acc[RAD_RB][RAD_MM_NB], tot[RAD_RB][RAD_MM_NB];
 #pragma unroll
   for (int r = 0; r < RAD_RB; r++)
 #pragma unroll
-    for (int v = 0; v < 16; v++) acc[r][v] = tot[r][v] = 0.f;
+    for (int nb = 0; nb < RAD_MM_NB; nb++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[r][nb][v] = tot[r][nb][v] = 0.f;
 
   const i64 jbeg = S.jbeg, jend = S.jend;
   constexpr int CH = RAD_NKB * 2 * RAD_TJ;  // 16-byte chunks of the slot vectors of a tile
   constexpr int NPF = (CH + RAD_BLOCK - 1) / RAD_BLOCK;
-  constexpr int CW = RAD_TJ * 4;            // 16-byte chunks of the weights of a tile (64 bytes per column)
+  constexpr int CW = RAD_TJ * 4 * RAD_MM_NB;  // 16-byte chunks of the weights of a tile (64 bytes per column and block)
   constexpr int NPW = (CW + RAD_BLOCK - 1) / RAD_BLOCK;
   uint4 pf[NPF], pfw[NPW];
   const __bf16* bwm = reinterpret_cast<const __bf16*>(S.bw);
@@ -593,7 +597,7 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
       const int e = tid + u * RAD_BLOCK;
       pf[u] = e < CH ? src[e] : make_uint4(0u, 0u, 0u, 0u);
     }
-    const uint4* wsrc = reinterpret_cast<const uint4*>(bwm + j0 * 32);  // padded to whole tiles
+    const uint4* wsrc = reinterpret_cast<const uint4*>(bwm + j0 * (32 * RAD_MM_NB));  // padded to whole tiles
 #pragma unroll
     for (int u = 0; u < NPW; u++) {
       const int e = tid + u * RAD_BLOCK;
@@ -619,11 +623,14 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
 #pragma unroll
     for (int sub = 0; sub < RAD_NSUB; sub++) {
       const int c = sub * 32 + col;
-      rad_bf16x8 b[RAD_NKB], wk[2];
+      rad_bf16x8 b[RAD_NKB], wk[2][RAD_MM_NB];
 #pragma unroll
       for (int kb = 0; kb < RAD_NKB; kb++) b[kb] = *reinterpret_cast<const rad_bf16x8*>(ys + ((kb * 2 + half) * RAD_TJ + c) * 8);
 #pragma unroll
-      for (int kb = 0; kb < 2; kb++) wk[kb] = *reinterpret_cast<const rad_bf16x8*>(ws + (((sub * 2 + kb) * 2 + half) * 32 + col) * 8);
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int nb = 0; nb < RAD_MM_NB; nb++)
+          wk[kb][nb] = *reinterpret_cast<const rad_bf16x8*>(ws + (((sub * 2 + kb) * 2 + half) * (32 * RAD_MM_NB) + 32 * nb + col) * 8);
 #pragma unroll
       for (int r = 0; r < RAD_RB; r++) {
         rad_f32x16 z;
@@ -651,8 +658,11 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
             pmp[e] = __builtin_bit_cast(unsigned, __builtin_convertvector(rr, rad_bf16x2));
           }
           const rad_bf16x8 kh = __builtin_bit_cast(rad_bf16x8, ph), km = __builtin_bit_cast(rad_bf16x8, pm);
-          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(km, wk[kb], acc[r], 0, 0, 0);
-          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, wk[kb], acc[r], 0, 0, 0);
+#pragma unroll
+          for (int nb = 0; nb < RAD_MM_NB; nb++) {
+            acc[r][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(km, wk[kb][nb], acc[r][nb], 0, 0, 0);
+            acc[r][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, wk[kb][nb], acc[r][nb], 0, 0, 0);
+          }
 #else
           // K = h + m + l, each the truncation of what is left to 8 significant bits (the subtractions are exact); a
           // byte permute packs the high halves of two floats: the bfloat16 terms.  (v_dot2_f32_bf16 against the pairs
@@ -675,9 +685,12 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
           const rad_bf16x8 kh = __builtin_bit_cast(rad_bf16x8, ph), km = __builtin_bit_cast(rad_bf16x8, pm),
                            kl = __builtin_bit_cast(rad_bf16x8, pl);
           // smallest terms first
-          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kl, wk[kb], acc[r], 0, 0, 0);
-          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(km, wk[kb], acc[r], 0, 0, 0);
-          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, wk[kb], acc[r], 0, 0, 0);
+#pragma unroll
+          for (int nb = 0; nb < RAD_MM_NB; nb++) {
+            acc[r][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kl, wk[kb][nb], acc[r][nb], 0, 0, 0);
+            acc[r][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(km, wk[kb][nb], acc[r][nb], 0, 0, 0);
+            acc[r][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, wk[kb][nb], acc[r][nb], 0, 0, 0);
+          }
 #endif
         }
       }
@@ -688,10 +701,12 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
 #pragma unroll
       for (int r = 0; r < RAD_RB; r++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-          tot[r][v] += acc[r][v];
-          acc[r][v] = 0.f;
-        }
+        for (int nb = 0; nb < RAD_MM_NB; nb++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) {
+            tot[r][nb][v] += acc[r][nb][v];
+            acc[r][nb][v] = 0.f;
+          }
     }
   }
   // lane l holds operand column l % 32 of rows 8 (v / 4) + 4 (l / 32) + v % 4: the three column groups
@@ -700,9 +715,22 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
   for (int r = 0; r < RAD_RB; r++)
 #pragma unroll
     for (int v = 0; v < 16; v++) {
-      const float s0 = tot[r][v] + acc[r][v];
+      // term t of component d = lane % 32 sits in operand column t * RAD_DV + d: block (column / 32), lane (column % 32)
+      // of the same half
+      float term[3];
+#pragma unroll
+      for (int t = 0; t < 3; t++) {
+        const int c = t * RAD_DV + col;
+        float got = 0.f;
+#pragma unroll
+        for (int nb = 0; nb < RAD_MM_NB; nb++) {
+          const float cand = __shfl(tot[r][nb][v] + acc[r][nb][v], 32 * half + (c & 31));
+          got = (c >> 5) == nb ? cand : got;
+        }
+        term[t] = got;
+      }
       // (smallest group first)
-      const float s = (__shfl(s0, lane + 2 * RAD_DV) + __shfl(s0, lane + RAD_DV)) + s0;
+      const float s = (term[2] + term[1]) + term[0];
       const i64 i = r * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
       if (col < RAD_DV && i < S.rows_store) S.part[i * RAD_DV + col] = s;
     }
@@ -714,7 +742,7 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
   if (P.scal[2] != 1u) return;
   __shared__ __attribute__((aligned(16))) __bf16 ys[RAD_NKB * 2 * RAD_TJ * 8];  // [kb][half][col][8]
 #if RAD_MM
-  __shared__ __attribute__((aligned(16))) __bf16 ws[RAD_TJ * 32];  // [sub-tile][k block][half][operand column][8]
+  __shared__ __attribute__((aligned(16))) __bf16 ws[RAD_TJ * 32 * RAD_MM_NB];  // [sub-tile][k block][half][operand column][8]
 #elif !RAD_FOLD
   __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_DV];
 #else

@@ -922,7 +922,7 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     # accumulated component) live in registers
     # from config.radial_mm_min_dv accumulated components on, the weighted sum runs on the matrix cores too (the three
     # bfloat16 terms of the weights side by side in the 32 operand columns): 16 accumulators per block of 32 rows
-    mm = int(config.radial_mm_min_dv <= Dv and 3 * Dv <= 32 and not rows_per_block)
+    mm = int(config.radial_mm_min_dv <= Dv <= config.radial_mm_max_dv and not rows_per_block)
     if Dv > config.radial_max_dv and not mm:
         return None, None  # the accumulators of that many components do not fit the registers
     rb = (config.radial_mm_rb if mm else 2) if (mm or Dv <= config.radial_rb2_max_dv) else 1
@@ -963,7 +963,7 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     ra, rd, ro = VarLayout.table(al.rowvars)
     # a scalar weight and no difference factor: the weight joins the exponent, columns are partitioned by its sign
     fold = int(config.radial_fold and dimw == 1 and not diff and not rows_per_block and not mm)
-    meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
+    meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_mm_nb=-(-3 * Dv // 32), rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
                 rad_yarg=y.ind, rad_fold=fold, rad_tj=tj)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
     defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,

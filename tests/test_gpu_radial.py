@@ -32,7 +32,8 @@ def _last_meta(key):
 
 
 @pytest.mark.parametrize("D,Dv,M,N", [(3, 1, 30011, 30500), (3, 8, 20000, 21000), (3, 2, 300000, 1001), (5, 3, 17000, 23001),
-                                      (8, 1, 16000, 18000), (2, 4, 33333, 10001), (6, 7, 18011, 19003), (3, 10, 17000, 16500)])
+                                      (8, 1, 16000, 18000), (2, 4, 33333, 10001), (6, 7, 18011, 19003), (3, 10, 17000, 16500),
+                                      (3, 16, 16400, 16700), (4, 23, 16500, 16400)])
 def test_gaussian_sums_with_matrix_core_exponents_vs_oracle(D, Dv, M, N):
     rng = np.random.default_rng(100 * D + Dv)
     x = rng.standard_normal((M, D)).astype(np.float32)
@@ -42,7 +43,8 @@ def test_gaussian_sums_with_matrix_core_exponents_vs_oracle(D, Dv, M, N):
     dev = to_dev(x, y, b, g)
     got = _genred(D, Dv)(*dev)
     assert _last_meta("radial") == "1"
-    # from seven components on, the weighted sum runs on the matrix cores too (three-term operands)
+    # from seven components on, the weighted sum runs on the matrix cores too (three-term operands; beyond ten components
+    # the operand columns take two or three blocks)
     assert _last_meta("rad_mm") == ("1" if Dv >= 7 else "0")
     rows = np.sort(rng.choice(M, 1500, replace=False)).astype(np.int64)
     ref = cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
