@@ -443,7 +443,11 @@ static __global__ void __launch_bounds__(512) keops_stream_loop(float* out, cons
   float r = 0.f;
 #pragma unroll
   for (int v = 0; v < 16; v++) r += tot[v];
-  out[(size_t)blockIdx.x * 256 + (tid & 255)] = r;
+  // (blocks * 256 floats of output for workgroups of 512 lanes: the two halves of a workgroup add up)
+  __syncthreads();  // every wavefront is done with the last tile
+  if (tid >= 256) reinterpret_cast<float*>(as[0])[tid - 256] = r;
+  __syncthreads();
+  if (tid < 256) out[(size_t)blockIdx.x * 256 + tid] = r + reinterpret_cast<float*>(as[0])[tid];
 }
 
 // The inner loop of the signed-byte nearest-neighbour filter without its memory traffic: per round two query sets,
