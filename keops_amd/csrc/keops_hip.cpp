@@ -445,13 +445,15 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
     nranges = S.nbatches;
     const int64_t R = tagI == 0 ? S.M : S.N, C = tagI == 0 ? S.N : S.M;
     rx_host.resize((size_t)2 * nranges);
-    synth.resize((size_t)3 * nranges);
+    synth.resize((size_t)5 * nranges);  // [slices][ranges_y][row ranges]
     for (int64_t b = 0; b < nranges; b++) {
       rx_host[2 * b] = b * R;
       rx_host[2 * b + 1] = (b + 1) * R;
       synth[b] = b + 1;
       synth[nranges + 2 * b] = b * C;
       synth[nranges + 2 * b + 1] = (b + 1) * C;
+      synth[3 * nranges + 2 * b] = b * R;
+      synth[3 * nranges + 2 * b + 1] = (b + 1) * R;
     }
   }
 
@@ -579,6 +581,12 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
   } else {
     rt.slices_x = tab + n_lookup + n_off;
     rt.ranges_y = tab + n_lookup + n_off + nranges;
+    // the batches as row ranges over the flattened arrays (kernels that give every range its own centre)
+    const int64_t R = tagI == 0 ? S.M : S.N, C = tagI == 0 ? S.N : S.M;
+    rt.rx = tab + n_lookup + n_off + 3 * nranges;
+    rt.nranges = nranges;
+    rt.work_total = nranges * C;
+    rt.pairs = (double)nranges * (double)R * (double)C;
   }
   return 0;
 }
@@ -1701,6 +1709,16 @@ static int launch_on_device(Module& m, int64_t nx, int64_t ny, int tagI, int tag
       // exponents on the matrix cores when the pattern and the data allow it (the latter is decided on the device):
       // keops_conv_ranges then returns at once, and the other way round
       if (m.meta_int("radial", 0) != 0 && m.meta_int("rad_ranges", 0) != 0)
+        if (int rc = launch_radial_ranges(m, rows_total, cols_total, out, args, stream, rt, &h.guard)) return rc;
+      m.last_guard = h.guard;
+    } else if (m.meta_int("radial", 0) != 0 && m.meta_int("rad_ranges", 0) != 0) {
+      // batches: row ranges over the flattened arrays when every row and column variable carries every batch
+      // dimension and no parameter does (the kernels of that family address rows globally and read one parameter set)
+      bool plain = true;
+      for (int v : rowvars) { const int64_t* r = S.row(v + 1); for (int b = 0; b < nb; b++) plain = plain && r[b] == S.shapes[b]; }
+      for (int v : colvars) { const int64_t* r = S.row(v + 1); for (int b = 0; b < nb; b++) plain = plain && r[b] == S.shapes[b]; }
+      for (int v : vP) { const int64_t* r = S.row(v + 1); for (int b = 0; b < nb; b++) plain = plain && r[b] == 1; }
+      if (plain)
         if (int rc = launch_radial_ranges(m, rows_total, cols_total, out, args, stream, rt, &h.guard)) return rc;
       m.last_guard = h.guard;
     }

@@ -787,7 +787,7 @@ def _linear_coef(E, svar):
     return None
 
 
-def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id, pairs=0, block_sparse=False):
+def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id, pairs=0, block_sparse=False, batch_total=0):
     """dict(x, y, coef, A, W, diff) when the formula of a float32 Sum reduction on the dense scheme is a product
 
         [+-]  A(i-variables)  *  Exp(C * SqDist(x, y))  *  W(j-variables)  [ * (x - y) | (y - x) ]
@@ -806,9 +806,14 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
     if (not config.radial or red.kind != KIND_SUM or dtype != "float" or dtypeacc != "float" or not use_fast_math
             or sum_scheme == "kahan_scheme"):
         return None
-    # launches with ranges: block-sparse patterns only (no batch dimensions), where every row range gets its own centre
-    if "_ranges" in map_reduce_id and not (block_sparse and config.radial_ranges):
-        return None
+    # launches with ranges: block-sparse patterns without batch dimensions, where every row range gets its own centre,
+    # and batches that no variable is broadcast over (``batch_total``: log2 bucket of their pairs together), which
+    # are row ranges with one reduced range each
+    if "_ranges" in map_reduce_id:
+        if not config.radial_ranges or not (block_sparse or batch_total):
+            return None
+        if not block_sparse:
+            pairs = batch_total
     if pairs and int(pairs) < config.radial_min_pairs_log2:
         return None
     row_cat, col_cat = red.tagI, 1 - red.tagI
@@ -1091,10 +1096,12 @@ def get_keops_dll(
             source, meta = generate_plugin(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, nargs, nx=rows_hint,
                                            irregular=irregular)
             block_sparse = irregular and batch_loop == -1
-            rad = match_radial(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, map_reduce_id, pairs, block_sparse) if mc else None
+            batched = irregular and batch_loop >= 0 and batch_total > 0
+            rad = match_radial(red, dtype, dtypeacc, sum_scheme_string, use_fast_math, map_reduce_id, pairs, block_sparse,
+                               batch_total if batched else 0) if mc else None
             if rad is not None:
                 section, rmeta = generate_radial_section(red, rad, nargs,
-                                                         int(meta["block"]) * int(meta["rows"]) if block_sparse else 0)
+                                                         int(meta["block"]) * int(meta["rows"]) if (block_sparse or batched) else 0)
                 if section is not None:
                     meta.update(rmeta)
                     head, body = source.split("\n", 1)

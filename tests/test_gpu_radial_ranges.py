@@ -226,3 +226,55 @@ def test_block_sparse_matrix_core_sums_under_graph_capture():
         torch.cuda.synchronize()
         got = out.clone()
         assert torch.equal(got, conv(xd, yd, bd, gd, ranges=rd))   # eager launches between the replays
+
+
+def test_batches_are_served_as_row_ranges_with_one_centre_each():
+    """Batch dimensions that no variable is broadcast over (GpuReduc1D_ranges.py:74-173 with the block-diagonal
+    ranges of Ranges.h:40-86): every batch is one row range of the flattened arrays with its own centre.  Batches far
+    from each other (offsets of 50 kernel widths) would fail a check on one common centre."""
+    D, Dv, B, M, N = 3, 2, 7, 9500, 6700   # (at least one workgroup per compute unit: 7 x 38 row blocks)
+    rng = np.random.default_rng(61)
+    off = (50.0 * rng.standard_normal((B, 1, D))).astype(np.float32)
+    x = (rng.standard_normal((B, M, D)) + off).astype(np.float32)
+    y = (rng.standard_normal((B, N, D)) + off).astype(np.float32)
+    b = rng.standard_normal((B, N, Dv)).astype(np.float32)
+    g = np.array([0.6], np.float32)
+    dev = to_dev(x, y, b, g)
+    got = _genred(D, Dv)(*dev)
+    assert got.shape == (B, M, Dv)
+    assert _module().meta("rad_ranges") == "1" and _module().path_status() == 1
+    rows = np.sort(rng.choice(M, 400, replace=False)).astype(np.int64)
+    for k in range(B):
+        ref = cpu_reduc("gauss", [x[k], y[k], b[k], g], M, N, Dv, rows=rows)
+        scale = cpu_reduc("gauss", [x[k], y[k], np.abs(b[k]), g], M, N, Dv, rows=rows)
+        assert_sum_parity(got[k][torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
+    # the general-purpose kernel gives (slightly) different bits; deterministic from call to call
+    plain = _genred(D, Dv, enable_chunks=False)(*dev)
+    assert _module().meta("radial") is None and not torch.equal(plain, got)
+    assert torch.equal(_genred(D, Dv)(*dev), got)
+    # a variable shared by the batches (broadcast) or a parameter per batch keeps the call on the general-purpose kernel
+    shared = _genred(D, Dv)(dev[0], dev[1][:1], dev[2], dev[3])
+    assert _module().path_status() == 0
+    ref = cpu_reduc("gauss", [x[3], y[0], b[3], g], M, N, Dv, rows=rows)
+    scale = cpu_reduc("gauss", [x[3], y[0], np.abs(b[3]), g], M, N, Dv, rows=rows)
+    assert_sum_parity(shared[3][torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
+    gs = torch.full((B, 1), 0.6, device="cuda")
+    per_batch = _genred(D, Dv)(dev[0], dev[1], dev[2], gs)
+    assert _module().path_status() == 0
+    assert_sum_parity(per_batch[2][torch.from_numpy(rows).cuda()].cpu().numpy(),
+                      cpu_reduc("gauss", [x[2], y[2], b[2], g], M, N, Dv, rows=rows),
+                      cpu_reduc("gauss", [x[2], y[2], np.abs(b[2]), g], M, N, Dv, rows=rows))
+
+
+def test_batches_with_a_kernel_too_narrow_for_them_fall_back():
+    D, Dv, B, M, N = 3, 1, 5, 14000, 7800
+    rng = np.random.default_rng(62)
+    x = rng.standard_normal((B, M, D)).astype(np.float32)
+    y = rng.standard_normal((B, N, D)).astype(np.float32)
+    b = rng.standard_normal((B, N, Dv)).astype(np.float32)
+    g = np.array([400.0], np.float32)
+    dev = to_dev(x, y, b, g)
+    got = _genred(D, Dv)(*dev)
+    assert _module().meta("rad_ranges") == "1" and _module().path_status() == 0
+    plain = _genred(D, Dv, enable_chunks=False)(*dev)
+    assert torch.equal(got, plain)
