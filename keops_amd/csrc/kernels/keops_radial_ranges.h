@@ -33,7 +33,7 @@ struct RadRParams {
   KeopsRangeTables rt;   // lookup (one entry per workgroup), slices and reduced-index ranges, validated or clamped
   __bf16* xa;            // [nblocks * RAD_ROWS_PER_BLOCK][RAD_SLOTS] row-side slot vectors, by lookup entry
   __bf16* yb;            // [virtual tile][RAD_NKB][2][RAD_TJ][8]
-  float* bw;             // [virtual tile * RAD_TJ][RAD_DV]
+  float* bw;             // [virtual tile * RAD_TJ][RAD_DV] (RAD_MM: the operand layout of rad_store_weights_mm)
   float* ctr;            // [nranges][RAD_D] centre of every row range
   i64* vt;               // [nranges][2] = (first virtual tile, number of virtual tiles)
   unsigned* rmax;        // [nranges][2] bit patterns of max |x^|^2 and max |y~|^2
@@ -224,8 +224,12 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_prep_cols(const Rad
         for (int q = 0; q < 8; q++) v8[q] = slot[kb * 16 + hf * 8 + q];
         *reinterpret_cast<rad_bf16x8*>(P.yb + (((tile * RAD_NKB + kb) * 2 + hf) * RAD_TJ + c) * 8) = v8;
       }
+#if RAD_MM
+    rad_store_weights_mm(reinterpret_cast<__bf16*>(P.bw), tile * RAD_TJ + c, w);  // B operand of the second product
+#else
 #pragma unroll
     for (int d = 0; d < RAD_DV; d++) P.bw[(tile * RAD_TJ + c) * RAD_DV + d] = w[d];
+#endif
   };
 
   i64 k0, k1;
@@ -312,7 +316,11 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_decide(const RadRPa
 extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_radr_main(const RadRParams P) {
   if (P.scal[2] != 1u) return;
   __shared__ __attribute__((aligned(16))) __bf16 ys[RAD_NKB * 2 * RAD_TJ * 8];  // [kb][half][col][8]
+#if RAD_MM
+  __shared__ __attribute__((aligned(16))) __bf16 ws[RAD_TJ * 32 * RAD_MM_NB];  // [sub-tile][k block][half][operand column][8]
+#else
   __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_DV];
+#endif
   const i64 e = blockIdx.x;
   const i64 r = keops_uniform(P.rt.lookup[3 * e]), r0 = keops_uniform(P.rt.lookup[3 * e + 1]), r1 = keops_uniform(P.rt.lookup[3 * e + 2]);
   if (r1 <= r0) return;
@@ -328,7 +336,11 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
   S.part = P.partial + local0 * RAD_DV;
   S.rows_store = 32 * RAD_RB;
   S.pos_tiles = S.all_tiles = 0;
+#if RAD_MM
+  rad_sweep_mm(S, ys, ws);
+#else
   rad_sweep(S, ys, bs);
+#endif
 }
 
 // the factors of the output index and, for the gradients with respect to the points, the difference

@@ -927,7 +927,7 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     # accumulated component) live in registers
     # from config.radial_mm_min_dv accumulated components on, the weighted sum runs on the matrix cores too (the three
     # bfloat16 terms of the weights side by side in the 32 operand columns): 16 accumulators per block of 32 rows
-    mm = int(config.radial_mm_min_dv <= Dv <= config.radial_mm_max_dv and not rows_per_block)
+    mm = int(config.radial_mm_min_dv <= Dv <= config.radial_mm_max_dv)
     if Dv > config.radial_max_dv and not mm:
         return None, None  # the accumulators of that many components do not fit the registers
     rb = (config.radial_mm_rb if mm else 2) if (mm or Dv <= config.radial_rb2_max_dv) else 1

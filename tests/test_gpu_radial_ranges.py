@@ -47,7 +47,7 @@ def _pattern(c, rx, ry, thr=1.0):
     return from_matrix(rx, ry, keep), keep
 
 
-@pytest.mark.parametrize("D,Dv,sigma", [(3, 1, 0.05), (3, 3, 0.05), (2, 8, 0.05), (5, 2, 0.04), (8, 1, 0.03)])
+@pytest.mark.parametrize("D,Dv,sigma", [(3, 1, 0.05), (3, 3, 0.05), (2, 8, 0.05), (5, 2, 0.04), (8, 1, 0.03), (3, 12, 0.05)])
 def test_block_sparse_gaussian_sums_on_the_matrix_cores_vs_oracle(D, Dv, sigma):
     c, x, y, b, rx, ry = _clusters(D, Dv, 64, 10 * D + Dv, sigma=sigma, box=4.0 if D <= 3 else 2.0)
     g = np.array([100.0], np.float32)
