@@ -159,7 +159,8 @@ class LoadKeOps_hip:
         argshapes = tuple(tuple(a.shape) for a in args)
         M = nx if p.tagI == 0 else ny
         if nbatchdims:
-            bshape = np.maximum.reduce([list(a.shape[:nbatchdims]) for a in args])
+            # (an argument with fewer leading dimensions, e.g. a parameter given as (dim,), is broadcast over them)
+            bshape = np.maximum.reduce([list(a.shape[:nbatchdims]) if a.dim() > nbatchdims else [1] * nbatchdims for a in args])
             shapeout = tuple(int(b) for b in bshape) + (M, p.dim)
         else:
             shapeout = (M, p.dim)

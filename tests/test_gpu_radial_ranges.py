@@ -266,6 +266,22 @@ def test_batches_are_served_as_row_ranges_with_one_centre_each():
                       cpu_reduc("gauss", [x[2], y[2], np.abs(b[2]), g], M, N, Dv, rows=rows))
 
 
+def test_batched_reduction_over_i_and_two_batch_dimensions():
+    D, Dv, B1, B2, M, N = 2, 1, 3, 4, 5200, 5700     # 12 batches of 23 workgroups (the output is indexed by j)
+    rng = np.random.default_rng(63)
+    x = rng.standard_normal((B1, B2, M, D)).astype(np.float32)
+    y = rng.standard_normal((B1, B2, N, D)).astype(np.float32)
+    a = rng.standard_normal((B1, B2, M, Dv)).astype(np.float32)
+    g = np.array([0.8], np.float32)
+    got = _genred(D, Dv, axis=0)(*to_dev(x, y, a, g))
+    assert got.shape == (B1, B2, N, Dv) and _module().path_status() == 1
+    cols = np.sort(rng.choice(N, 300, replace=False)).astype(np.int64)
+    for k1, k2 in ((0, 0), (2, 3), (1, 2)):
+        ref = cpu_reduc("gauss", [y[k1, k2], x[k1, k2], a[k1, k2], g], N, M, Dv, rows=cols)   # roles of i and j exchanged
+        scale = cpu_reduc("gauss", [y[k1, k2], x[k1, k2], np.abs(a[k1, k2]), g], N, M, Dv, rows=cols)
+        assert_sum_parity(got[k1, k2][torch.from_numpy(cols).cuda()].cpu().numpy(), ref, scale)
+
+
 def test_batches_with_a_kernel_too_narrow_for_them_fall_back():
     D, Dv, B, M, N = 3, 1, 5, 14000, 7800
     rng = np.random.default_rng(62)
