@@ -294,3 +294,33 @@ def test_batches_with_a_kernel_too_narrow_for_them_fall_back():
     assert _module().meta("rad_ranges") == "1" and _module().path_status() == 0
     plain = _genred(D, Dv, enable_chunks=False)(*dev)
     assert torch.equal(got, plain)
+
+
+def test_batched_matrix_core_sums_under_graph_capture():
+    D, Dv, B, M, N = 3, 1, 8, 8448, 8200
+    rng = np.random.default_rng(64)
+    x = rng.standard_normal((B, M, D)).astype(np.float32)
+    y = rng.standard_normal((B, N, D)).astype(np.float32)
+    b = rng.standard_normal((B, N, Dv)).astype(np.float32)
+    xd, yd, bd, gd = to_dev(x, y, b, np.array([0.5], np.float32))
+    conv = _genred(D, Dv)
+    conv(xd, yd, bd, gd)
+    assert _module().path_status() == 1
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        conv(xd, yd, bd, gd)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = conv(xd, yd, bd, gd)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for k in range(3):
+        bd.copy_(torch.randn(bd.shape, device="cuda", generator=gen))
+        xd.add_(0.01)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        assert torch.equal(got, conv(xd, yd, bd, gd))   # eager launches between the replays
