@@ -324,3 +324,24 @@ def test_batched_matrix_core_sums_under_graph_capture():
         torch.cuda.synchronize()
         got = out.clone()
         assert torch.equal(got, conv(xd, yd, bd, gd))   # eager launches between the replays
+
+
+def test_gradient_with_respect_to_the_points_of_batched_sums_vs_dense_float64():
+    """The gradient is another batched map-reduce (generic_red.py:165-214) of the same family: it takes the same
+    kernels, one centre per batch."""
+    D, Dv, B, M, N = 3, 1, 8, 8448, 8300   # (scalar weights: <b_j, e_i> is then a product of a row and a column factor)
+    gen = torch.Generator(device="cuda").manual_seed(65)
+    x = torch.randn(B, M, D, device="cuda", generator=gen) + 30.0 * torch.randn(B, 1, D, device="cuda", generator=gen)
+    y = x[:, :N].clone() + 0.3 * torch.randn(B, N, D, device="cuda", generator=gen)
+    b = torch.randn(B, N, Dv, device="cuda", generator=gen)
+    e = torch.randn(B, M, Dv, device="cuda", generator=gen)
+    g = torch.tensor([0.7], device="cuda")
+    x.requires_grad_(True)
+    (_genred(D, Dv)(x, y, b, g) * e).sum().backward()
+    assert _module().meta("rad_ranges") == "1" and _module().path_status() == 1
+    for k in (0, 5):
+        xk = x[k].detach().double().requires_grad_(True)
+        K = torch.exp(-0.7 * torch.cdist(xk, y[k].double()) ** 2)
+        ((K @ b[k].double()) * e[k].double()).sum().backward()
+        err = (x.grad[k].double() - xk.grad).norm() / xk.grad.norm()
+        assert float(err) <= 1e-5, float(err)
