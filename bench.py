@@ -68,6 +68,9 @@ WORKLOADS = {
     "knn_l1_d784": ("ArgKMin K=10 of the L1 distance, 1e4 queries x 6e4 references, D=784", 2352, "valu"),
     "sparse_100x10k": ("block-sparse Gaussian sum, 100 clusters x 10,000 points (benchmark configuration 4)", 14, "valu"),
     "lse_b16": ("batched LogSumExp softmin B=16, 50,000 x 50,000, D=3 (benchmark configuration 5a)", 17, "valu"),
+    # the shape of configuration 5a with a Gaussian sum instead of the log-sum-exp: batches as row ranges of the
+    # matrix-core exponent kernels, one centre per batch (kernels/keops_radial_ranges.h)
+    "gauss_b16": ("batched Gaussian kernel sum B=16, 50,000 x 50,000, D=3, Dv=1", 14, "valu"),
     # 2*D flop of the contraction + sqrt, neg, exp + 2*Dv of the weighted accumulation
     "laplace_d256": ("Laplace kernel sum 2e5 x 2e5, D=256, Dv=16 (benchmark configuration 5b)", 547, "mfma"),
     # softmax-weighted sum of an inner product (attention-like): 2*D flop of the scores, exp, 2*Dv of the weighted
@@ -121,13 +124,13 @@ def _np_inputs(name):
         y = (np.repeat(c, per, 0) + 0.05 * rng.standard_normal((C * per, 3))).astype(np.float32)
         b = rng.standard_normal((C * per, 1)).astype(np.float32)
         return dict(M=C * per, N=C * per, Dv=1, centres=c, per=per, arrays=[x, y, b, np.array([100.0], np.float32)])
-    if name == "lse_b16":
+    if name in ("lse_b16", "gauss_b16"):
         rng = np.random.default_rng(4)
         B, M, N = 16, 50_000, 50_000
         x = rng.standard_normal((B, M, 3)).astype(np.float32)
         y = rng.standard_normal((B, N, 3)).astype(np.float32)
         l = rng.standard_normal((B, N, 1)).astype(np.float32)
-        return dict(M=M, N=N, Dv=1, B=B, arrays=[x, y, l, np.array([20.0], np.float32)])
+        return dict(M=M, N=N, Dv=1, B=B, arrays=[x, y, l, np.array([20.0 if name == "lse_b16" else 0.5], np.float32)])
     raise SystemExit(f"workload {name} is not available in this build")
 
 
@@ -156,6 +159,9 @@ def build_step(name):
     if name == "lse_b16":
         lse = Genred("l-SqDist(x,y)*e", ["x=Vi(3)", "y=Vj(3)", "l=Vj(1)", "e=Pm(1)"], reduction_op="LogSumExp", axis=1)
         return (lambda: lse(*dev)), inp["B"] * M * N, inp
+    if name == "gauss_b16":
+        gs = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(1)", "g=Pm(1)"], reduction_op="Sum", axis=1)
+        return (lambda: gs(*dev)), inp["B"] * M * N, inp
     if name == "sparse_100x10k":
         from keops_amd.torch.cluster import from_matrix
 
