@@ -49,7 +49,8 @@
 // The plug-in defines RAD_D, RAD_DV, RAD_NKB (16-slot blocks), RAD_RB, RAD_WAVES, RAD_XARG, RAD_YARG, RAD_LIMIT,
 // the slot tables rad_slot_kind / rad_slot_comp / rad_slot_term for both sides, the tables of the variables of B
 // (rad_col_arg / rad_col_dim / rad_col_off, RAD_NCOLVARS, RAD_DIMY) and of the parameters (keops_par_*), and
-// the tables of the variables of A (rad_row_*, RAD_NROWVARS, RAD_DIMX), RAD_DW (components of W), RAD_DOUT, RAD_DIFF,
+// the tables of the variables of A (rad_row_*, RAD_NROWVARS, RAD_DIMX), RAD_DW (components of W), RAD_DU (components of
+// a row vector u_i that multiplies W as <u_i, W_j>: KeopsRadFormula::rowvec), RAD_DOUT, RAD_DIFF,
 // RAD_SIGN and struct KeopsRadFormula { kappa(p); weights(yj, p, w); rowscale(xi, p) }.
 #pragma once
 
@@ -60,6 +61,9 @@ typedef __bf16 rad_bf16x2 __attribute__((ext_vector_type(2)));
 
 #ifndef RAD_TJ
 #define RAD_TJ 128                 // columns per staged tile
+#endif
+#ifndef RAD_DU
+#define RAD_DU 0                   // components of a row factor u_i that enters as <u_i, v_j> (0: none)
 #endif
 #ifndef RAD_MM
 #define RAD_MM 0                   // 1: the weighted sum runs on the matrix cores too (see rad_sweep_mm)
@@ -319,9 +323,13 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
       T wv[RAD_DW];
       KeopsRadFormula::weights(yj, p, wv);
 #if RAD_DIFF != 0
+      // component d of the weights against [y^_j, 1]
 #pragma unroll
-      for (int k = 0; k < RAD_D; k++) w[k] = (float)wv[0] * cf[k];
-      w[RAD_D] = (float)wv[0];
+      for (int d = 0; d < RAD_DW; d++) {
+#pragma unroll
+        for (int k = 0; k < RAD_D; k++) w[d * (RAD_D + 1) + k] = (float)wv[d] * cf[k];
+        w[d * (RAD_D + 1) + RAD_D] = (float)wv[d];
+      }
 #else
 #pragma unroll
       for (int d = 0; d < RAD_DV; d++) w[d] = (float)wv[d];
@@ -796,13 +804,30 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadPara
     for (int d = 0; d < rad_row_dim[v]; d++) xi[rad_row_off[v] + d] = a[d];
   }
   const float ai = (float)KeopsRadFormula::rowscale(xi, p) * RAD_SIGN;
+  // a factor <u_i, v_j> of both indices: the sums were accumulated per component of v, u_i contracts them here
+#if RAD_DU > 0
+  T uv[RAD_DU];
+  KeopsRadFormula::rowvec(xi, p, uv);
+#endif
 #if RAD_DIFF != 0
   const T* x = P.arg[RAD_XARG] + i * RAD_D;
 #pragma unroll
   for (int k = 0; k < RAD_D; k++) {
     const float xc = (float)((double)x[k] - (double)P.colsum[k]);
+#if RAD_DU > 0
+    float acc = 0.f;
+#pragma unroll
+    for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], __builtin_fmaf(xc, s[d * (RAD_D + 1) + RAD_D], -s[d * (RAD_D + 1) + k]), acc);
+    P.out[i * RAD_DOUT + k] = (T)(ai * (float)RAD_DIFF * acc);
+#else
     P.out[i * RAD_DOUT + k] = (T)(ai * (float)RAD_DIFF * __builtin_fmaf(xc, s[RAD_D], -s[k]));
+#endif
   }
+#elif RAD_DU > 0
+  float acc = 0.f;
+#pragma unroll
+  for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], s[d], acc);
+  P.out[i] = (T)(ai * acc);
 #else
 #pragma unroll
   for (int d = 0; d < RAD_DOUT; d++) P.out[i * RAD_DOUT + d] = (T)(ai * s[d]);

@@ -260,9 +260,13 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_prep_cols(const Rad
         T wv[RAD_DW];
         KeopsRadFormula::weights(yj, p, wv);
 #if RAD_DIFF != 0
+        // component d of the weights against [y~_j, 1]
 #pragma unroll
-        for (int q = 0; q < RAD_D; q++) w[q] = (float)wv[0] * cf[q];
-        w[RAD_D] = (float)wv[0];
+        for (int d = 0; d < RAD_DW; d++) {
+#pragma unroll
+          for (int q = 0; q < RAD_D; q++) w[d * (RAD_D + 1) + q] = (float)wv[d] * cf[q];
+          w[d * (RAD_D + 1) + RAD_D] = (float)wv[d];
+        }
 #else
 #pragma unroll
         for (int d = 0; d < RAD_DV; d++) w[d] = (float)wv[d];
@@ -362,13 +366,30 @@ extern "C" __global__ void __launch_bounds__(RAD_ROWS_PER_BLOCK) keops_radr_fini
     for (int d = 0; d < rad_row_dim[v]; d++) xi[rad_row_off[v] + d] = a[d];
   }
   const float ai = (float)KeopsRadFormula::rowscale(xi, p) * RAD_SIGN;
+  // a factor <u_i, v_j> of both indices: the sums were accumulated per component of v, u_i contracts them here
+#if RAD_DU > 0
+  T uv[RAD_DU];
+  KeopsRadFormula::rowvec(xi, p, uv);
+#endif
 #if RAD_DIFF != 0
   const T* x = P.arg[RAD_XARG] + i * RAD_D;
 #pragma unroll
   for (int k = 0; k < RAD_D; k++) {
     const float xc = (float)((double)x[k] - (double)P.ctr[r * RAD_D + k]);
+#if RAD_DU > 0
+    float acc = 0.f;
+#pragma unroll
+    for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], __builtin_fmaf(xc, s[d * (RAD_D + 1) + RAD_D], -s[d * (RAD_D + 1) + k]), acc);
+    P.out[i * RAD_DOUT + k] = (T)(ai * (float)RAD_DIFF * acc);
+#else
     P.out[i * RAD_DOUT + k] = (T)(ai * (float)RAD_DIFF * __builtin_fmaf(xc, s[RAD_D], -s[k]));
+#endif
   }
+#elif RAD_DU > 0
+  float acc = 0.f;
+#pragma unroll
+  for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], s[d], acc);
+  P.out[i] = (T)(ai * acc);
 #else
 #pragma unroll
   for (int d = 0; d < RAD_DOUT; d++) P.out[i * RAD_DOUT + d] = (T)(ai * s[d]);

@@ -795,7 +795,9 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
     with x an output-indexed and y a reduced-index variable of at most config.radial_max_dim (8) components, C a scalar
     formula of the parameters, A scalar, W of at most config.radial_max_dv (8) components (scalar when the difference
     factor is present): the Gaussian kernel sums and their gradients with respect to the points and the weights.  Here
-    "i" means indexed like the output.  Such sums take their exponents from the matrix cores
+    "i" means indexed like the output.  One factor may be a scalar product <u_i, v_j> of an output-indexed and a
+    reduced-index vector: the sums are then accumulated per component of v_j and contracted with u_i once per output
+    row.  Such sums take their exponents from the matrix cores
     (kernels/keops_radial_mfma.h) when the data allow it; with the difference factor, the kernel accumulates
     sum_j K_ij w_j [y^_j, 1] and the last pass forms A_i (x^_i S - sum_j K_ij w_j y^_j) for the points centred on the
     mean of y.  ``pairs``: when not 0, the call holds less than 2**pairs pairs; small calls stay on the
@@ -847,7 +849,7 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
     if coef is None:
         return None
     x, y = (a, b) if a.cat == row_cat else (b, a)
-    A, Wf, diff = [], [], 0
+    A, Wf, diff, U = [], [], 0, None
     for f in factors:
         if f is exps[0]:
             continue
@@ -855,6 +857,13 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
             if diff:
                 return None
             diff = 1 if f.children[0] == x else -1
+        elif (f.name == "Scalprod" and len(f.children) == 2 and U is None and f.children[0].dim == f.children[1].dim > 1
+              and any(not c.depends_on_cat(col_cat) and c.depends_on_cat(row_cat) for c in f.children)
+              and any(not c.depends_on_cat(row_cat) and c.depends_on_cat(col_cat) for c in f.children)):
+            # <u_i, v_j>: the sums are accumulated per component of v_j, u_i contracts them once per output row
+            u, v = f.children if f.children[0].depends_on_cat(row_cat) else f.children[::-1]
+            U = u
+            Wf.append(v)
         elif not f.depends_on_cat(col_cat) and f.depends_on_cat(row_cat):
             if f.dim != 1:
                 return None
@@ -864,13 +873,22 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
         else:
             return None  # a factor of both indices other than the exponential
     vec = [f for f in Wf if f.dim != 1]
-    if len(vec) > 1 or (diff and vec):
+    if len(vec) > 1 or (diff and vec and U is None):
         return None
     dimw = vec[0].dim if vec else 1
+
+    def fits(n):  # accumulated components per pair
+        return 1 <= n <= max(config.radial_max_dv, config.radial_mm_max_dv if config.radial_mm_min_dv <= n else 0)
+
     if diff:
-        if x.dim + 1 > config.radial_max_dv or red.formula.dim != x.dim:
+        # (with vector weights the general-purpose kernel contracts <u_i, v_j> first and keeps D sums per pair, while
+        # this family keeps dim(v) (D + 1): measured, it only wins while the fused-multiply-add variant holds them)
+        if dimw * (x.dim + 1) > (config.radial_max_dv if U is not None else 10 ** 9) or not fits(dimw * (x.dim + 1)) or red.formula.dim != x.dim:
             return None
-    elif dimw != red.formula.dim or not 1 <= dimw <= max(config.radial_max_dv, config.radial_mm_max_dv if config.radial_mm_min_dv <= dimw else 0):
+    elif U is not None:
+        if red.formula.dim != 1 or not fits(dimw):
+            return None
+    elif dimw != red.formula.dim or not fits(dimw):
         return None
 
     def product(fs):
@@ -879,7 +897,7 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
             out = f if out is None else O.Mult(out, f)
         return out
 
-    return dict(x=x, y=y, coef=coef, A=product(A), W=product(Wf), diff=diff, sign=sign)
+    return dict(x=x, y=y, coef=coef, A=product(A), W=product(Wf), diff=diff, sign=sign, U=U)
 
 
 def generate_radial_section(red, match, nargs, rows_per_block=0):
@@ -891,10 +909,12 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     from .formulas.lir import LOG2E
 
     x, y, coef, A, W, diff, sign = (match[k] for k in ("x", "y", "coef", "A", "W", "diff", "sign"))
+    U = match.get("U")                 # row factor u_i of a scalar product <u_i, v_j> (v_j is then the vector in W)
     D = x.dim
     dimw = 1 if W is None else W.dim
-    Dv = D + 1 if diff else dimw       # components accumulated per pair
-    dout = D if diff else dimw         # components of the output
+    du = 0 if U is None else U.dim
+    Dv = dimw * (D + 1) if diff else dimw                    # components accumulated per pair
+    dout = D if diff else (1 if U is not None else dimw)     # components of the output
     # slots of the scalar product, by decreasing magnitude: (row term, column term) of every component, the terms
     # of the two squared norms against 1.  kind 0: zero, 1: one, 2: component term (comp, term), 3: norm term
     H, Mi, Lo = 0, 1, 2
@@ -947,7 +967,10 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     class _A:
         formula, tagI = (A if A is not None else one), red.tagI
 
-    wl, al = VarLayout(_W), VarLayout(_A)
+    class _AU:  # the variables of both row factors share one table
+        formula, tagI = (_A.formula if U is None else O.Mult(_A.formula, O.Sum(U))), red.tagI
+
+    wl, al = VarLayout(_W), VarLayout(_AU)
     if wl.rowvars or al.colvars:
         return None, None
     # the parameter table serves every body: the one of the whole reduction (as the general-purpose kernel's)
@@ -963,6 +986,7 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
 
     w_pre, w_lines, w_exprs = body(_W.formula, wl.names)
     a_pre, a_lines, a_exprs = body(_A.formula, al.names)
+    u_pre, u_lines, u_exprs = body(U, al.names) if U is not None else ([], [], [])
     k_pre, k_lines, k_exprs = body(coef, {})
     ca, cd, co = VarLayout.table(wl.colvars)
     ra, rd, ro = VarLayout.table(al.rowvars)
@@ -971,7 +995,7 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_mm_nb=-(-3 * Dv // 32), rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
                 rad_yarg=y.ind, rad_fold=fold, rad_tj=tj)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
-    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
+    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DU=du, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
                 RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit)!r}f",
                 RAD_NCOLVARS=len(wl.colvars), RAD_DIMY=wl.dimy, RAD_NROWVARS=len(al.rowvars), RAD_DIMX=al.dimx)
     src += [f"#define {k} {v}" for k, v in defs.items()]
@@ -980,7 +1004,7 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
                        ("col_arg", ca), ("col_dim", cd), ("col_off", co), ("row_arg", ra), ("row_dim", rd), ("row_off", ro)):
         src.append(f"static __device__ constexpr int rad_{name}[] = {_c_list(vals)};")
     dy, dx, dp = max(1, wl.dimy), max(1, al.dimx), max(1, full.dimp)
-    src += w_pre + a_pre + k_pre
+    src += w_pre + a_pre + u_pre + k_pre
     src.append("struct KeopsRadFormula {")
     src.append("  // log2(e) times the coefficient of the squared distance in the exponent")
     src.append(f"  static __device__ __forceinline__ T kappa(const T (&p)[{dp}]) {{")
@@ -995,7 +1019,13 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     src.append(f"  static __device__ __forceinline__ T rowscale(const T (&xi)[{dx}], const T (&p)[{dp}]) {{")
     src += a_lines
     src.append(f"    return {a_exprs[0]};")
-    src.append("  }\n};")
+    src.append("  }")
+    if U is not None:
+        src.append("  // row factor of a scalar product with the weights: contracts the accumulated sums once per output row")
+        src.append(f"  static __device__ __forceinline__ void rowvec(const T (&xi)[{dx}], const T (&p)[{dp}], T (&u)[{du}]) {{")
+        src += u_lines + [f"    u[{k}] = {e};" for k, e in enumerate(u_exprs)]
+        src.append("  }")
+    src.append("};")
     src.append('#include "keops_radial_mfma.h"')
     return "\n".join(src) + "\n", meta
 

@@ -256,3 +256,59 @@ def test_random_clouds_and_kernel_widths_vs_oracle(seed):
             raise AssertionError(f"case {case}: D={D} Dv={Dv} M={M} N={N} spread={spread:.3g} offset={offset:.3g} "
                                  f"width={width:.3g}: {e}") from None
     assert served >= 15
+
+
+def _path_status():
+    from keops_amd import keops_io
+
+    return keops_io.last_loader.module.path_status()
+
+
+@pytest.mark.parametrize("D,Dw", [(3, 4), (3, 8), (2, 13)])
+def test_scalar_product_of_a_row_and_a_column_vector_as_weight(D, Dw):
+    """sum_j K_ij <u_i, v_j> (the kernel energy of shape models): one factor depends on both indices, but it is a
+    scalar product, so the sums are accumulated per component of v_j and contracted with u_i once per row.  Reference:
+    dense float64."""
+    from keops_amd.torch import Genred
+
+    M, N = 17000, 16500
+    gen = torch.Generator(device="cuda").manual_seed(70 + Dw)
+    x, y = torch.randn(M, D, device="cuda", generator=gen), torch.randn(N, D, device="cuda", generator=gen) + 0.2
+    u, v = torch.randn(M, Dw, device="cuda", generator=gen), torch.randn(N, Dw, device="cuda", generator=gen)
+    g = torch.tensor([0.6], device="cuda")
+    f = Genred("Exp(-g*SqDist(x,y))*(u|v)", [f"x=Vi({D})", f"y=Vj({D})", f"u=Vi({Dw})", f"v=Vj({Dw})", "g=Pm(1)"],
+               reduction_op="Sum", axis=1)
+    got = f(x, y, u, v, g)
+    assert got.shape == (M, 1)
+    assert _last_meta("radial") == "1" and _last_meta("rad_mm") == ("1" if Dw >= 7 else "0")
+    assert _path_status() == 1
+    K = torch.exp(-0.6 * torch.cdist(x.double(), y.double()) ** 2)
+    ref = ((K @ v.double()) * u.double()).sum(1, keepdim=True)
+    scale = ((K @ v.double().abs()) * u.double().abs()).sum(1, keepdim=True)
+    assert_sum_parity(got.cpu().numpy(), ref.cpu().numpy(), scale.cpu().numpy())
+    plain = Genred("Exp(-g*SqDist(x,y))*(u|v)", [f"x=Vi({D})", f"y=Vj({D})", f"u=Vi({Dw})", f"v=Vj({Dw})", "g=Pm(1)"],
+                   reduction_op="Sum", axis=1, enable_chunks=False)(x, y, u, v, g)
+    assert _last_meta("radial") is None
+    assert_sum_parity(plain.cpu().numpy(), ref.cpu().numpy(), scale.cpu().numpy())
+
+
+def test_gradient_with_respect_to_the_points_with_vector_weights():
+    """sum_j K_ij <e_i, b_j> (x_i - y_j) with two-component weights in the plane: 2 x 3 sums per pair, contracted with
+    e_i at the end (more components stay on the general-purpose kernel, which contracts <e_i, b_j> per pair)."""
+    D, Dv, M, N = 2, 2, 17000, 16500
+    gen = torch.Generator(device="cuda").manual_seed(81)
+    x, y = torch.randn(M, D, device="cuda", generator=gen), torch.randn(N, D, device="cuda", generator=gen)
+    b, e = torch.randn(N, Dv, device="cuda", generator=gen), torch.randn(M, Dv, device="cuda", generator=gen)
+    g = torch.tensor([0.6], device="cuda")
+    xr = x.clone().requires_grad_(True)
+    (_genred(D, Dv)(xr, y, b, g) * e).sum().backward()
+    assert _last_meta("radial") == "1" and _last_meta("rad_dv") == "6" and _path_status() == 1
+    xd = x.double().requires_grad_(True)
+    ((torch.exp(-0.6 * torch.cdist(xd, y.double()) ** 2) @ b.double()) * e.double()).sum().backward()
+    assert float((xr.grad.double() - xd.grad).norm() / xd.grad.norm()) <= 1e-5
+    # three components in space: 12 sums, left to the general-purpose kernel
+    x3, y3 = torch.randn(M, 3, device="cuda", generator=gen), torch.randn(N, 3, device="cuda", generator=gen)
+    b3, e3 = torch.randn(N, 3, device="cuda", generator=gen), torch.randn(M, 3, device="cuda", generator=gen)
+    xr3 = x3.clone().requires_grad_(True)
+    (_genred(3, 3)(xr3, y3, b3, g) * e3).sum().backward()
+    assert _last_meta("radial") is None
