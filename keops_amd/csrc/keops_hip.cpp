@@ -691,7 +691,8 @@ int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* arg
   const size_t o_blk = take(fold ? (size_t)nblk * 4 : 0);
   // weights of a column: RAD_DV floats, or 32 bfloat16 operand columns when the weighted sum runs on the matrix cores
   // (three terms of every weight: one block of 32 columns up to ten weights, rad_mm_nb blocks beyond)
-  const size_t wbytes = m.meta_int("rad_mm", 0) != 0 ? 64 * (size_t)std::max<int64_t>(1, m.meta_int("rad_mm_nb", 1)) : (size_t)DV * 4;
+  const size_t wbytes = m.meta_int("rad_mm", 0) != 0 ? 64 * (size_t)std::max<int64_t>(1, m.meta_int("rad_mm_nb", 1))
+                                                      : (size_t)std::max<int64_t>(DV, m.meta_int("rad_ws", 0)) * 4;
   const size_t o_xa = take((size_t)nx * NKB * 32), o_yb = take((size_t)ntiles * TJ * NKB * 32), o_bw = take((size_t)ntiles * TJ * wbytes);
   const size_t o_part = take((size_t)nslabs * nx * DV * 4);
   if (int rc = m.partial.reserve(off)) return rc;
@@ -761,7 +762,8 @@ int launch_radial_ranges(Module& m, int64_t nx, int64_t ny, void* out, void* con
   const size_t o_scal = take(32), o_ctr = take((size_t)rt.nranges * D * 4), o_vt = take((size_t)rt.nranges * 16), o_rmax = take((size_t)rt.nranges * 8);
   const size_t o_xa = take((size_t)rt.nblocks * RPB * NKB * 32), o_yb = take((size_t)vt_capacity * TJ * NKB * 32);
   // weights of a formatted column: RAD_DV floats, or the operand columns of the second matrix product
-  const size_t wbytes = m.meta_int("rad_mm", 0) != 0 ? 64 * (size_t)std::max<int64_t>(1, m.meta_int("rad_mm_nb", 1)) : (size_t)DV * 4;
+  const size_t wbytes = m.meta_int("rad_mm", 0) != 0 ? 64 * (size_t)std::max<int64_t>(1, m.meta_int("rad_mm_nb", 1))
+                                                      : (size_t)std::max<int64_t>(DV, m.meta_int("rad_ws", 0)) * 4;
   const size_t o_bw = take((size_t)vt_capacity * TJ * wbytes), o_part = take((size_t)rt.nblocks * RPB * DV * 4);
   if (off > ((size_t)4 << 30)) return 0;  // the formatted operands stay within 4 GiB
   if (int rc = m.partial.reserve(off)) return rc;

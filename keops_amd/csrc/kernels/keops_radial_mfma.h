@@ -65,6 +65,10 @@ typedef __bf16 rad_bf16x2 __attribute__((ext_vector_type(2)));
 #ifndef RAD_DU
 #define RAD_DU 0                   // components of a row factor u_i that enters as <u_i, v_j> (0: none)
 #endif
+#ifndef RAD_UPAIR
+#define RAD_UPAIR 0                // 1 (with RAD_DIFF and RAD_DU): <u_i, v_j> is formed per pair and D + 1 sums are kept
+#endif
+#define RAD_WS (RAD_UPAIR ? RAD_DW + RAD_D + 1 : RAD_DV)  // floats staged per column: the weights as the sweep needs them
 #ifndef RAD_MM
 #define RAD_MM 0                   // 1: the weighted sum runs on the matrix cores too (see rad_sweep_mm)
 #endif
@@ -277,9 +281,9 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
   rad_load_params(P, p);
   const double kappa = (double)KeopsRadFormula::kappa(p);
   __bf16 slot[RAD_SLOTS];
-  float w[RAD_DV];
+  float w[RAD_WS];
 #pragma unroll
-  for (int d = 0; d < RAD_DV; d++) w[d] = 0.f;
+  for (int d = 0; d < RAD_WS; d++) w[d] = 0.f;
   if (i < n) {
     const T* src = P.arg[which ? RAD_YARG : RAD_XARG] + i * RAD_D;
     __bf16 ct[RAD_D][3], nt[4];
@@ -322,7 +326,14 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
       }
       T wv[RAD_DW];
       KeopsRadFormula::weights(yj, p, wv);
-#if RAD_DIFF != 0
+#if RAD_UPAIR
+      // the weights as they are, then [y^_j, 1]: the sweep forms <u_i, v_j> itself
+#pragma unroll
+      for (int d = 0; d < RAD_DW; d++) w[d] = (float)wv[d];
+#pragma unroll
+      for (int k = 0; k < RAD_D; k++) w[RAD_DW + k] = cf[k];
+      w[RAD_DW + RAD_D] = 1.f;
+#elif RAD_DIFF != 0
       // component d of the weights against [y^_j, 1]
 #pragma unroll
       for (int d = 0; d < RAD_DW; d++) {
@@ -380,7 +391,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
     rad_store_weights_mm(reinterpret_cast<__bf16*>(P.bw), i, w);
 #elif !RAD_FOLD
 #pragma unroll
-    for (int d = 0; d < RAD_DV; d++) P.bw[i * RAD_DV + d] = w[d];
+    for (int d = 0; d < RAD_WS; d++) P.bw[i * RAD_WS + d] = w[d];
 #endif
   }
 }
@@ -428,7 +439,19 @@ struct RadSweep {
   float* part;         // [rows_store][RAD_DV] sums of the wavefront's rows
   i64 rows_store;
   i64 pos_tiles, all_tiles;  // RAD_FOLD
+  const T* const* arg;       // RAD_UPAIR: the arguments, for the row factor u_i of the wavefront's rows ...
+  i64 row_first, row_last;   // ... which are rows row_first + k of the arguments, clamped to row_last
 };
+
+// parameters of the formula from the argument table
+__device__ __forceinline__ void rad_params_of(const T* const* arg, T (&p)[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1]) {
+#pragma unroll
+  for (int v = 0; v < KEOPS_NPARVARS; v++) {
+    const T* src = arg[keops_par_arg[v]];
+#pragma unroll
+    for (int d = 0; d < keops_par_dim[v]; d++) p[keops_par_off[v] + d] = src[d];
+  }
+}
 
 // All wavefronts of the workgroup call this together with the same columns (they share the staged tile).
 __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* bs) {
@@ -448,12 +471,37 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
     for (int v = 0; v < 16; v++)
 #pragma unroll
       for (int d = 0; d < RAD_DV; d++) acc[r][v][d] = 0.f;
+#if RAD_UPAIR
+  // the row factor u_i of the 16 rows this lane accumulates, from the arguments themselves
+  float ur[RAD_RB][16][RAD_DW];
+  {
+    T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+    rad_params_of(S.arg, p);
+#pragma unroll
+    for (int r = 0; r < RAD_RB; r++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const i64 gi = keops_min(S.row_first + r * 32 + 8 * (v >> 2) + 4 * half + (v & 3), S.row_last);
+        T xi[RAD_DIMX > 0 ? RAD_DIMX : 1];
+#pragma unroll
+        for (int q = 0; q < RAD_NROWVARS; q++) {
+          const T* a_ = S.arg[rad_row_arg[q]] + gi * rad_row_dim[q];
+#pragma unroll
+          for (int d = 0; d < rad_row_dim[q]; d++) xi[rad_row_off[q] + d] = a_[d];
+        }
+        T uv[RAD_DU > 0 ? RAD_DU : 1];
+        KeopsRadFormula::rowvec(xi, p, uv);
+#pragma unroll
+        for (int d = 0; d < RAD_DW; d++) ur[r][v][d] = (float)uv[d];
+      }
+  }
+#endif
 
   const i64 jbeg = S.jbeg, jend = S.jend;
   // software pipeline: tile t+1 travels to registers while tile t is consumed
   constexpr int CH = RAD_NKB * 2 * RAD_TJ;  // 16-byte chunks of the slot vectors of a tile
   constexpr int NPF = (CH + RAD_BLOCK - 1) / RAD_BLOCK;
-  constexpr int NPW = (RAD_TJ * RAD_DV + RAD_BLOCK - 1) / RAD_BLOCK;
+  constexpr int NPW = (RAD_TJ * RAD_WS + RAD_BLOCK - 1) / RAD_BLOCK;
   uint4 pf[NPF];
 #if !RAD_FOLD
   float pfw[NPW];
@@ -472,11 +520,11 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
       pf[u] = e < CH ? src[e] : make_uint4(0u, 0u, 0u, 0u);
     }
 #if !RAD_FOLD
-    const float* wsrc = S.bw + j0 * RAD_DV;  // padded to whole tiles
+    const float* wsrc = S.bw + j0 * RAD_WS;  // padded to whole tiles
 #pragma unroll
     for (int u = 0; u < NPW; u++) {
       const int e = tid + u * RAD_BLOCK;
-      pfw[u] = e < RAD_TJ * RAD_DV ? wsrc[e] : 0.f;
+      pfw[u] = e < RAD_TJ * RAD_WS ? wsrc[e] : 0.f;
     }
 #endif
   };
@@ -492,7 +540,7 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
 #pragma unroll
     for (int u = 0; u < NPW; u++) {
       const int e = tid + u * RAD_BLOCK;
-      if (e < RAD_TJ * RAD_DV) bs[e] = pfw[u];
+      if (e < RAD_TJ * RAD_WS) bs[e] = pfw[u];
     }
 #endif
     __syncthreads();
@@ -508,9 +556,9 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
 #pragma unroll
       for (int kb = 0; kb < RAD_NKB; kb++) b[kb] = *reinterpret_cast<const rad_bf16x8*>(ys + ((kb * 2 + half) * RAD_TJ + c) * 8);
 #if !RAD_FOLD
-      float w[RAD_DV];
+      float w[RAD_WS];
 #pragma unroll
-      for (int d = 0; d < RAD_DV; d++) w[d] = bs[c * RAD_DV + d];
+      for (int d = 0; d < RAD_WS; d++) w[d] = bs[c * RAD_WS + d];
 #endif
       rad_f32x16 t[RAD_RB];
 #pragma unroll
@@ -540,8 +588,18 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
 #pragma unroll
         for (int v = 0; v < 16; v++) {
           const float e = __builtin_amdgcn_exp2f(t[r][v]);
+#if RAD_UPAIR
+          // K_ij <u_i, v_j> [y^_j, 1]
+          float sp = ur[r][v][0] * w[0];
+#pragma unroll
+          for (int d = 1; d < RAD_DW; d++) sp = __builtin_fmaf(ur[r][v][d], w[d], sp);
+          const float es = e * sp;
+#pragma unroll
+          for (int d = 0; d < RAD_DV; d++) acc[r][v][d] = __builtin_fmaf(es, w[RAD_DW + d], acc[r][v][d]);
+#else
 #pragma unroll
           for (int d = 0; d < RAD_DV; d++) acc[r][v][d] = __builtin_fmaf(e, w[d], acc[r][v][d]);
+#endif
         }
 #endif
     }
@@ -752,7 +810,7 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
 #if RAD_MM
   __shared__ __attribute__((aligned(16))) __bf16 ws[RAD_TJ * 32 * RAD_MM_NB];  // [sub-tile][k block][half][operand column][8]
 #elif !RAD_FOLD
-  __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_DV];
+  __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_WS];
 #else
   float* bs = nullptr;
 #endif
@@ -773,6 +831,9 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
   S.rows_store = row0 < P.nx ? P.nx - row0 : 0;
   S.pos_tiles = RAD_FOLD ? keops_uniform((i64)P.scal[3]) : 0;  // tiles of columns with non-negative weights come first
   S.all_tiles = ncols / RAD_TJ;
+  S.arg = P.arg;
+  S.row_first = first;
+  S.row_last = P.nx - 1;
 #if RAD_MM
   rad_sweep_mm(S, ys, ws);
 #else
@@ -805,7 +866,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadPara
   }
   const float ai = (float)KeopsRadFormula::rowscale(xi, p) * RAD_SIGN;
   // a factor <u_i, v_j> of both indices: the sums were accumulated per component of v, u_i contracts them here
-#if RAD_DU > 0
+#if RAD_DU > 0 && !RAD_UPAIR
   T uv[RAD_DU];
   KeopsRadFormula::rowvec(xi, p, uv);
 #endif
@@ -814,7 +875,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadPara
 #pragma unroll
   for (int k = 0; k < RAD_D; k++) {
     const float xc = (float)((double)x[k] - (double)P.colsum[k]);
-#if RAD_DU > 0
+#if RAD_DU > 0 && !RAD_UPAIR
     float acc = 0.f;
 #pragma unroll
     for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], __builtin_fmaf(xc, s[d * (RAD_D + 1) + RAD_D], -s[d * (RAD_D + 1) + k]), acc);

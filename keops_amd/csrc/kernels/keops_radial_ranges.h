@@ -33,7 +33,7 @@ struct RadRParams {
   KeopsRangeTables rt;   // lookup (one entry per workgroup), slices and reduced-index ranges, validated or clamped
   __bf16* xa;            // [nblocks * RAD_ROWS_PER_BLOCK][RAD_SLOTS] row-side slot vectors, by lookup entry
   __bf16* yb;            // [virtual tile][RAD_NKB][2][RAD_TJ][8]
-  float* bw;             // [virtual tile * RAD_TJ][RAD_DV] (RAD_MM: the operand layout of rad_store_weights_mm)
+  float* bw;             // [virtual tile * RAD_TJ][RAD_WS] (RAD_MM: the operand layout of rad_store_weights_mm)
   float* ctr;            // [nranges][RAD_D] centre of every row range
   i64* vt;               // [nranges][2] = (first virtual tile, number of virtual tiles)
   unsigned* rmax;        // [nranges][2] bit patterns of max |x^|^2 and max |y~|^2
@@ -213,7 +213,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_prep_cols(const Rad
   const float* ctr = P.ctr + r * RAD_D;
   float nmax = 0.f;
 
-  auto store = [&](i64 t, int c, const __bf16 (&slot)[RAD_SLOTS], const float (&w)[RAD_DV]) {
+  auto store = [&](i64 t, int c, const __bf16 (&slot)[RAD_SLOTS], const float (&w)[RAD_WS]) {
     const i64 tile = tile0 + t;
 #pragma unroll
     for (int kb = 0; kb < RAD_NKB; kb++)
@@ -228,7 +228,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_prep_cols(const Rad
     rad_store_weights_mm(reinterpret_cast<__bf16*>(P.bw), tile * RAD_TJ + c, w);  // B operand of the second product
 #else
 #pragma unroll
-    for (int d = 0; d < RAD_DV; d++) P.bw[(tile * RAD_TJ + c) * RAD_DV + d] = w[d];
+    for (int d = 0; d < RAD_WS; d++) P.bw[(tile * RAD_TJ + c) * RAD_WS + d] = w[d];
 #endif
   };
 
@@ -247,7 +247,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_prep_cols(const Rad
         if (v < base || v >= base + len) continue;
         const i64 j = s + (v - base);
         __bf16 slot[RAD_SLOTS];
-        float cf[RAD_D], w[RAD_DV];
+        float cf[RAD_D], w[RAD_WS];
         const float nrm = radr_slots(P.arg[RAD_YARG] + j * RAD_D, ctr, kappa, true, slot, cf);
         nmax = nrm > nmax ? nrm : nmax;
         T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
@@ -259,7 +259,14 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_prep_cols(const Rad
         }
         T wv[RAD_DW];
         KeopsRadFormula::weights(yj, p, wv);
-#if RAD_DIFF != 0
+#if RAD_UPAIR
+        // the weights as they are, then [y~_j, 1]: the sweep forms <u_i, v_j> itself
+#pragma unroll
+        for (int d = 0; d < RAD_DW; d++) w[d] = (float)wv[d];
+#pragma unroll
+        for (int q = 0; q < RAD_D; q++) w[RAD_DW + q] = cf[q];
+        w[RAD_DW + RAD_D] = 1.f;
+#elif RAD_DIFF != 0
         // component d of the weights against [y~_j, 1]
 #pragma unroll
         for (int d = 0; d < RAD_DW; d++) {
@@ -279,11 +286,11 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_prep_cols(const Rad
   const i64 last = ntiles - 1;
   if (last % RADR_NCH == chunk) {
     __bf16 slot[RAD_SLOTS];
-    float w[RAD_DV];
+    float w[RAD_WS];
 #pragma unroll
     for (int s = 0; s < RAD_SLOTS; s++) slot[s] = (__bf16)0.0f;
 #pragma unroll
-    for (int d = 0; d < RAD_DV; d++) w[d] = 0.f;
+    for (int d = 0; d < RAD_WS; d++) w[d] = 0.f;
     for (int c = tid; c < RAD_TJ; c += 256)
       if (last * RAD_TJ + c >= base) store(last, c, slot, w);
   }
@@ -323,7 +330,7 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
 #if RAD_MM
   __shared__ __attribute__((aligned(16))) __bf16 ws[RAD_TJ * 32 * RAD_MM_NB];  // [sub-tile][k block][half][operand column][8]
 #else
-  __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_DV];
+  __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_WS];
 #endif
   const i64 e = blockIdx.x;
   const i64 r = keops_uniform(P.rt.lookup[3 * e]), r0 = keops_uniform(P.rt.lookup[3 * e + 1]), r1 = keops_uniform(P.rt.lookup[3 * e + 2]);
@@ -340,6 +347,9 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
   S.part = P.partial + local0 * RAD_DV;
   S.rows_store = 32 * RAD_RB;
   S.pos_tiles = S.all_tiles = 0;
+  S.arg = P.arg;
+  S.row_first = r0 + (i64)wave * (32 * RAD_RB);
+  S.row_last = r1 - 1;
 #if RAD_MM
   rad_sweep_mm(S, ys, ws);
 #else
@@ -367,7 +377,7 @@ extern "C" __global__ void __launch_bounds__(RAD_ROWS_PER_BLOCK) keops_radr_fini
   }
   const float ai = (float)KeopsRadFormula::rowscale(xi, p) * RAD_SIGN;
   // a factor <u_i, v_j> of both indices: the sums were accumulated per component of v, u_i contracts them here
-#if RAD_DU > 0
+#if RAD_DU > 0 && !RAD_UPAIR
   T uv[RAD_DU];
   KeopsRadFormula::rowvec(xi, p, uv);
 #endif
@@ -376,7 +386,7 @@ extern "C" __global__ void __launch_bounds__(RAD_ROWS_PER_BLOCK) keops_radr_fini
 #pragma unroll
   for (int k = 0; k < RAD_D; k++) {
     const float xc = (float)((double)x[k] - (double)P.ctr[r * RAD_D + k]);
-#if RAD_DU > 0
+#if RAD_DU > 0 && !RAD_UPAIR
     float acc = 0.f;
 #pragma unroll
     for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], __builtin_fmaf(xc, s[d * (RAD_D + 1) + RAD_D], -s[d * (RAD_D + 1) + k]), acc);

@@ -883,7 +883,12 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
     if diff:
         # (with vector weights the general-purpose kernel contracts <u_i, v_j> first and keeps D sums per pair, while
         # this family keeps dim(v) (D + 1): measured, it only wins while the fused-multiply-add variant holds them)
-        if dimw * (x.dim + 1) > (config.radial_max_dv if U is not None else 10 ** 9) or not fits(dimw * (x.dim + 1)) or red.formula.dim != x.dim:
+        # beyond 8 sums the sweep forms <u_i, v_j> per pair itself and keeps D + 1 sums (u_i of its rows in registers)
+        if red.formula.dim != x.dim or x.dim + 1 > config.radial_max_dv:
+            return None
+        if U is not None and dimw * (x.dim + 1) > config.radial_max_dv and dimw > config.radial_upair_max_dw:
+            return None
+        if U is None and not fits(x.dim + 1):
             return None
     elif U is not None:
         if red.formula.dim != 1 or not fits(dimw):
@@ -913,8 +918,9 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     D = x.dim
     dimw = 1 if W is None else W.dim
     du = 0 if U is None else U.dim
-    Dv = dimw * (D + 1) if diff else dimw                    # components accumulated per pair
-    dout = D if diff else (1 if U is not None else dimw)     # components of the output
+    upair = int(bool(diff and U is not None and dimw * (D + 1) > config.radial_max_dv))  # <u_i, v_j> formed per pair
+    Dv = (D + 1 if upair else dimw * (D + 1)) if diff else dimw   # components accumulated per pair
+    dout = D if diff else (1 if U is not None else dimw)          # components of the output
     # slots of the scalar product, by decreasing magnitude: (row term, column term) of every component, the terms
     # of the two squared norms against 1.  kind 0: zero, 1: one, 2: component term (comp, term), 3: norm term
     H, Mi, Lo = 0, 1, 2
@@ -947,10 +953,12 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     # accumulated component) live in registers
     # from config.radial_mm_min_dv accumulated components on, the weighted sum runs on the matrix cores too (the three
     # bfloat16 terms of the weights side by side in the 32 operand columns): 16 accumulators per block of 32 rows
-    mm = int(config.radial_mm_min_dv <= Dv <= config.radial_mm_max_dv)
+    mm = int(config.radial_mm_min_dv <= Dv <= config.radial_mm_max_dv and not upair)
     if Dv > config.radial_max_dv and not mm:
         return None, None  # the accumulators of that many components do not fit the registers
     rb = (config.radial_mm_rb if mm else 2) if (mm or Dv <= config.radial_rb2_max_dv) else 1
+    if upair:
+        rb = 1  # 16 x dim(u) registers per 32-row block hold the row factors
     tj = ((256 if mm else 128 if Dv <= 2 else 512) if config.radial_tile_j == "auto" else int(config.radial_tile_j))
     if tj % 32 or not 32 <= tj <= 1024:
         raise ValueError("[KeOps] KEOPS_AMD_RADIAL_TJ must be a multiple of 32 between 32 and 1024")
@@ -992,10 +1000,10 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     ra, rd, ro = VarLayout.table(al.rowvars)
     # a scalar weight and no difference factor: the weight joins the exponent, columns are partitioned by its sign
     fold = int(config.radial_fold and dimw == 1 and not diff and not rows_per_block and not mm)
-    meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_mm_nb=-(-3 * Dv // 32), rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
+    meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_mm_nb=-(-3 * Dv // 32), rad_ws=(dimw + D + 1 if upair else Dv), rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
                 rad_yarg=y.ind, rad_fold=fold, rad_tj=tj)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
-    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DU=du, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
+    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DU=du, RAD_UPAIR=upair, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
                 RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit)!r}f",
                 RAD_NCOLVARS=len(wl.colvars), RAD_DIMY=wl.dimy, RAD_NROWVARS=len(al.rowvars), RAD_DIMX=al.dimx)
     src += [f"#define {k} {v}" for k, v in defs.items()]

@@ -294,7 +294,7 @@ def test_scalar_product_of_a_row_and_a_column_vector_as_weight(D, Dw):
 
 def test_gradient_with_respect_to_the_points_with_vector_weights():
     """sum_j K_ij <e_i, b_j> (x_i - y_j) with two-component weights in the plane: 2 x 3 sums per pair, contracted with
-    e_i at the end (more components stay on the general-purpose kernel, which contracts <e_i, b_j> per pair)."""
+    e_i at the end; with more components the sweep forms <e_i, b_j> per pair, as the general-purpose kernel does."""
     D, Dv, M, N = 2, 2, 17000, 16500
     gen = torch.Generator(device="cuda").manual_seed(81)
     x, y = torch.randn(M, D, device="cuda", generator=gen), torch.randn(N, D, device="cuda", generator=gen)
@@ -306,9 +306,17 @@ def test_gradient_with_respect_to_the_points_with_vector_weights():
     xd = x.double().requires_grad_(True)
     ((torch.exp(-0.6 * torch.cdist(xd, y.double()) ** 2) @ b.double()) * e.double()).sum().backward()
     assert float((xr.grad.double() - xd.grad).norm() / xd.grad.norm()) <= 1e-5
-    # three components in space: 12 sums, left to the general-purpose kernel
+    # three components in space would be 12 sums: the sweep forms <e_i, b_j> per pair instead and keeps 4
     x3, y3 = torch.randn(M, 3, device="cuda", generator=gen), torch.randn(N, 3, device="cuda", generator=gen)
     b3, e3 = torch.randn(N, 3, device="cuda", generator=gen), torch.randn(M, 3, device="cuda", generator=gen)
     xr3 = x3.clone().requires_grad_(True)
     (_genred(3, 3)(xr3, y3, b3, g) * e3).sum().backward()
+    assert _last_meta("radial") == "1" and _last_meta("rad_dv") == "4" and _path_status() == 1
+    xd3 = x3.double().requires_grad_(True)
+    ((torch.exp(-0.6 * torch.cdist(xd3, y3.double()) ** 2) @ b3.double()) * e3.double()).sum().backward()
+    assert float((xr3.grad.double() - xd3.grad).norm() / xd3.grad.norm()) <= 1e-5
+    # eight components: the general-purpose kernel
+    b8, e8 = torch.randn(N, 8, device="cuda", generator=gen), torch.randn(M, 8, device="cuda", generator=gen)
+    xr8 = x3.clone().requires_grad_(True)
+    (_genred(3, 8)(xr8, y3, b8, g) * e8).sum().backward()
     assert _last_meta("radial") is None

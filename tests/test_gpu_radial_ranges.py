@@ -345,3 +345,24 @@ def test_gradient_with_respect_to_the_points_of_batched_sums_vs_dense_float64():
         ((K @ b[k].double()) * e[k].double()).sum().backward()
         err = (x.grad[k].double() - xk.grad).norm() / xk.grad.norm()
         assert float(err) <= 1e-5, float(err)
+
+
+def test_batched_gradient_with_vector_weights_forms_the_scalar_product_per_pair():
+    """Momentum-weighted gradient of shape models, batched: sum_j K_ij <e_i, b_j> (x_i - y_j) with three-component
+    e and b; the range kernels read e_i of their rows from the arguments (rows of a batch, clamped to its end)."""
+    D, Dv, B, M, N = 3, 3, 9, 7500, 7600     # 7500 rows: the last workgroup of every batch is ragged
+    gen = torch.Generator(device="cuda").manual_seed(66)
+    x = torch.randn(B, M, D, device="cuda", generator=gen) + 20.0 * torch.randn(B, 1, D, device="cuda", generator=gen)
+    y = x[:, :N].clone() if N <= M else torch.randn(B, N, D, device="cuda", generator=gen) + x.mean(1, keepdim=True)
+    b = torch.randn(B, N, Dv, device="cuda", generator=gen)
+    e = torch.randn(B, M, Dv, device="cuda", generator=gen)
+    g = torch.tensor([0.7], device="cuda")
+    x.requires_grad_(True)
+    (_genred(D, Dv)(x, y, b, g) * e).sum().backward()
+    assert _module().meta("rad_ranges") == "1" and _module().meta("rad_dv") == "4" and _module().path_status() == 1
+    for k in (0, 8):
+        xk = x[k].detach().double().requires_grad_(True)
+        K = torch.exp(-0.7 * torch.cdist(xk, y[k].double()) ** 2)
+        ((K @ b[k].double()) * e[k].double()).sum().backward()
+        err = (x.grad[k].double() - xk.grad).norm() / xk.grad.norm()
+        assert float(err) <= 1e-5, float(err)
