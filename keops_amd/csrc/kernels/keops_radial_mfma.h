@@ -69,6 +69,15 @@ typedef __bf16 rad_bf16x2 __attribute__((ext_vector_type(2)));
 #define RAD_UPAIR 0                // 1 (with RAD_DIFF and RAD_DU): <u_i, v_j> is formed per pair and D + 1 sums are kept
 #endif
 #define RAD_WS (RAD_UPAIR ? RAD_DW + RAD_D + 1 : RAD_DV)  // floats staged per column: the weights as the sweep needs them
+// RAD_BIL: a factor <u_i, v_j> comes out of the matrix cores like the exponent: the k blocks RAD_NKE .. RAD_NKB - 1 of
+// the slot vectors hold the term products of u_i (rows) and v_j (columns), slot kind 4, and a second accumulator
+// receives their sum for the 32 x 32 tile; the vector ALU multiplies it with the kernel value.
+#ifndef RAD_BIL
+#define RAD_BIL 0
+#endif
+#ifndef RAD_NKE
+#define RAD_NKE RAD_NKB            // k blocks of the exponent
+#endif
 #ifndef RAD_MM
 #define RAD_MM 0                   // 1: the weighted sum runs on the matrix cores too (see rad_sweep_mm)
 #endif
@@ -307,6 +316,34 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
 #else
     rad_split4(kappa * nrm, nt);
 #endif
+#if RAD_BIL
+    // three bfloat16 terms of every component of u_i (rows) or v_j (columns)
+    __bf16 bt[RAD_DW][3];
+    {
+      T vals[RAD_DW];
+      if (which) {
+        T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
+#pragma unroll
+        for (int v = 0; v < RAD_NCOLVARS; v++) {
+          const T* a = P.arg[rad_col_arg[v]] + i * rad_col_dim[v];
+#pragma unroll
+          for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
+        }
+        KeopsRadFormula::weights(yj, p, vals);
+      } else {
+        T xi[RAD_DIMX > 0 ? RAD_DIMX : 1];
+#pragma unroll
+        for (int v = 0; v < RAD_NROWVARS; v++) {
+          const T* a = P.arg[rad_row_arg[v]] + i * rad_row_dim[v];
+#pragma unroll
+          for (int d = 0; d < rad_row_dim[v]; d++) xi[rad_row_off[v] + d] = a[d];
+        }
+        KeopsRadFormula::rowvec(xi, p, vals);
+      }
+#pragma unroll
+      for (int d = 0; d < RAD_DW; d++) rad_split3((float)vals[d], bt[d]);
+    }
+#endif
     // largest centred squared norm (bit pattern of a non-negative float, rounded up): order-independent maximum
     atomicMax(P.scal + which, __float_as_uint((float)nrm * 1.000001f));
 #pragma unroll
@@ -314,7 +351,11 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
       const int kind = which ? rad_col_kind[s] : rad_row_kind[s];
       const int comp = which ? rad_col_comp[s] : rad_row_comp[s];
       const int term = which ? rad_col_term[s] : rad_row_term[s];
+#if RAD_BIL
+      slot[s] = kind == 0 ? (__bf16)0.0f : (kind == 1 ? (__bf16)1.0f : (kind == 2 ? ct[comp][term] : (kind == 3 ? nt[term] : bt[comp][term])));
+#else
       slot[s] = kind == 0 ? (__bf16)0.0f : (kind == 1 ? (__bf16)1.0f : (kind == 2 ? ct[comp][term] : nt[term]));
+#endif
     }
     if (which && !RAD_FOLD) {
       T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
@@ -326,7 +367,17 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
       }
       T wv[RAD_DW];
       KeopsRadFormula::weights(yj, p, wv);
-#if RAD_UPAIR
+#if RAD_BIL
+      // the weights sit in the slot vectors: what is left per column is [y^_j, 1], or 1
+      (void)wv;
+#if RAD_DIFF != 0
+#pragma unroll
+      for (int k = 0; k < RAD_D; k++) w[k] = cf[k];
+      w[RAD_D] = 1.f;
+#else
+      w[0] = 1.f;
+#endif
+#elif RAD_UPAIR
       // the weights as they are, then [y^_j, 1]: the sweep forms <u_i, v_j> itself
 #pragma unroll
       for (int d = 0; d < RAD_DW; d++) w[d] = (float)wv[d];
@@ -426,7 +477,7 @@ __device__ __forceinline__ i64 rad_tile_of(i64 k, i64 pos_tiles, i64 all_tiles, 
 #if RAD_MM
 #define RAD_MIN_WAVES (RAD_MM_NB > 1 ? 1 : (RAD_RB == 1 ? 4 : 2))  // (several operand blocks: 32 accumulators each)
 #else
-#define RAD_MIN_WAVES ((RAD_RB * 16 * RAD_DV <= 32) ? 4 : 1)
+#define RAD_MIN_WAVES ((RAD_RB * 16 * RAD_DV <= 32) ? (RAD_BIL ? 2 : 4) : 1)  // (RAD_BIL: a second tile of 16 values per block)
 #endif
 
 // What one wavefront sweeps: its 32 * RAD_RB rows against the columns [jbeg, jend) of the pre-formatted operand.
@@ -561,14 +612,24 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
       for (int d = 0; d < RAD_WS; d++) w[d] = bs[c * RAD_WS + d];
 #endif
       rad_f32x16 t[RAD_RB];
+#if RAD_BIL
+      rad_f32x16 t2[RAD_RB];  // <u_i, v_j> of the same pairs
+#endif
 #pragma unroll
       for (int r = 0; r < RAD_RB; r++) {
         rad_f32x16 z;
 #pragma unroll
         for (int v = 0; v < 16; v++) z[v] = 0.f;
 #pragma unroll
-        for (int kb = 0; kb < RAD_NKB; kb++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r][kb], b[kb], z, 0, 0, 0);
+        for (int kb = 0; kb < RAD_NKE; kb++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r][kb], b[kb], z, 0, 0, 0);
         t[r] = z;
+#if RAD_BIL
+#pragma unroll
+        for (int v = 0; v < 16; v++) z[v] = 0.f;
+#pragma unroll
+        for (int kb = RAD_NKE; kb < RAD_NKB; kb++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r][kb], b[kb], z, 0, 0, 0);
+        t2[r] = z;
+#endif
       }
 #if RAD_FOLD
       if (!negative) {
@@ -588,7 +649,11 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
 #pragma unroll
         for (int v = 0; v < 16; v++) {
           const float e = __builtin_amdgcn_exp2f(t[r][v]);
-#if RAD_UPAIR
+#if RAD_BIL
+          const float es = e * t2[r][v];
+#pragma unroll
+          for (int d = 0; d < RAD_DV; d++) acc[r][v][d] = __builtin_fmaf(es, w[d], acc[r][v][d]);
+#elif RAD_UPAIR
           // K_ij <u_i, v_j> [y^_j, 1]
           float sp = ur[r][v][0] * w[0];
 #pragma unroll
@@ -704,7 +769,7 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
         for (int v = 0; v < 16; v++) z[v] = 0.f;
         // transposed: z[v] = exponent of (row l % 32, column 8 (v / 4) + 4 (l / 32) + v % 4 of the sub-tile)
 #pragma unroll
-        for (int kb = 0; kb < RAD_NKB; kb++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[kb], a[r][kb], z, 0, 0, 0);
+        for (int kb = 0; kb < RAD_NKE; kb++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[kb], a[r][kb], z, 0, 0, 0);
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
 #if RAD_MM_TERMS == 2
@@ -866,7 +931,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadPara
   }
   const float ai = (float)KeopsRadFormula::rowscale(xi, p) * RAD_SIGN;
   // a factor <u_i, v_j> of both indices: the sums were accumulated per component of v, u_i contracts them here
-#if RAD_DU > 0 && !RAD_UPAIR
+#if RAD_DU > 0 && !RAD_UPAIR && !RAD_BIL
   T uv[RAD_DU];
   KeopsRadFormula::rowvec(xi, p, uv);
 #endif
@@ -875,7 +940,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadPara
 #pragma unroll
   for (int k = 0; k < RAD_D; k++) {
     const float xc = (float)((double)x[k] - (double)P.colsum[k]);
-#if RAD_DU > 0 && !RAD_UPAIR
+#if RAD_DU > 0 && !RAD_UPAIR && !RAD_BIL
     float acc = 0.f;
 #pragma unroll
     for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], __builtin_fmaf(xc, s[d * (RAD_D + 1) + RAD_D], -s[d * (RAD_D + 1) + k]), acc);
@@ -884,7 +949,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadPara
     P.out[i * RAD_DOUT + k] = (T)(ai * (float)RAD_DIFF * __builtin_fmaf(xc, s[RAD_D], -s[k]));
 #endif
   }
-#elif RAD_DU > 0
+#elif RAD_DU > 0 && !RAD_BIL
   float acc = 0.f;
 #pragma unroll
   for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], s[d], acc);

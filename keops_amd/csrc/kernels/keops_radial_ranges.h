@@ -61,9 +61,15 @@ __device__ __forceinline__ void radr_slices(const RadRParams& P, i64 r, i64& k0,
 }
 
 // Slot vector of one point relative to a centre; returns the squared norm of the centred point.
+// (RAD_BIL: bil holds the RAD_DW components of u_i resp. v_j, whose terms fill the slots of kind 4)
 __device__ __forceinline__ float radr_slots(const T* src, const float* ctr, double kappa, bool column, __bf16 (&slot)[RAD_SLOTS],
-                                            float (&cf)[RAD_D]) {
+                                            float (&cf)[RAD_D], const T* bil = nullptr) {
   __bf16 ct[RAD_D][3], nt[4];
+#if RAD_BIL
+  __bf16 bt[RAD_DW][3];
+#pragma unroll
+  for (int d = 0; d < RAD_DW; d++) rad_split3((float)bil[d], bt[d]);
+#endif
   double nrm = 0.0;
 #pragma unroll
   for (int k = 0; k < RAD_D; k++) {
@@ -78,7 +84,11 @@ __device__ __forceinline__ float radr_slots(const T* src, const float* ctr, doub
     const int kind = column ? rad_col_kind[s] : rad_row_kind[s];
     const int comp = column ? rad_col_comp[s] : rad_row_comp[s];
     const int term = column ? rad_col_term[s] : rad_row_term[s];
+#if RAD_BIL
+    slot[s] = kind == 0 ? (__bf16)0.0f : (kind == 1 ? (__bf16)1.0f : (kind == 2 ? ct[comp][term] : (kind == 3 ? nt[term] : bt[comp][term])));
+#else
     slot[s] = kind == 0 ? (__bf16)0.0f : (kind == 1 ? (__bf16)1.0f : (kind == 2 ? ct[comp][term] : nt[term]));
+#endif
   }
   return (float)nrm * 1.000001f;
 }
@@ -182,7 +192,19 @@ extern "C" __global__ void __launch_bounds__(RAD_ROWS_PER_BLOCK) keops_radr_prep
   float cf[RAD_D];
   float nrm = 0.f;
   if (i < r1) {
+#if RAD_BIL
+    T xi[RAD_DIMX > 0 ? RAD_DIMX : 1], uv[RAD_DW];
+#pragma unroll
+    for (int v = 0; v < RAD_NROWVARS; v++) {
+      const T* a = P.arg[rad_row_arg[v]] + i * rad_row_dim[v];
+#pragma unroll
+      for (int d = 0; d < rad_row_dim[v]; d++) xi[rad_row_off[v] + d] = a[d];
+    }
+    KeopsRadFormula::rowvec(xi, p, uv);
+    nrm = radr_slots(P.arg[RAD_XARG] + i * RAD_D, P.ctr + r * RAD_D, kappa, false, slot, cf, uv);
+#else
     nrm = radr_slots(P.arg[RAD_XARG] + i * RAD_D, P.ctr + r * RAD_D, kappa, false, slot, cf);
+#endif
   } else {
 #pragma unroll
     for (int s = 0; s < RAD_SLOTS; s++) slot[s] = (__bf16)0.0f;
@@ -248,8 +270,6 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_prep_cols(const Rad
         const i64 j = s + (v - base);
         __bf16 slot[RAD_SLOTS];
         float cf[RAD_D], w[RAD_WS];
-        const float nrm = radr_slots(P.arg[RAD_YARG] + j * RAD_D, ctr, kappa, true, slot, cf);
-        nmax = nrm > nmax ? nrm : nmax;
         T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
 #pragma unroll
         for (int q = 0; q < RAD_NCOLVARS; q++) {
@@ -259,7 +279,18 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_prep_cols(const Rad
         }
         T wv[RAD_DW];
         KeopsRadFormula::weights(yj, p, wv);
-#if RAD_UPAIR
+        const float nrm = radr_slots(P.arg[RAD_YARG] + j * RAD_D, ctr, kappa, true, slot, cf, wv);
+        nmax = nrm > nmax ? nrm : nmax;
+#if RAD_BIL
+        // the weights sit in the slot vectors: what is left per column is [y~_j, 1], or 1
+#if RAD_DIFF != 0
+#pragma unroll
+        for (int q = 0; q < RAD_D; q++) w[q] = cf[q];
+        w[RAD_D] = 1.f;
+#else
+        w[0] = 1.f;
+#endif
+#elif RAD_UPAIR
         // the weights as they are, then [y~_j, 1]: the sweep forms <u_i, v_j> itself
 #pragma unroll
         for (int d = 0; d < RAD_DW; d++) w[d] = (float)wv[d];
@@ -377,7 +408,7 @@ extern "C" __global__ void __launch_bounds__(RAD_ROWS_PER_BLOCK) keops_radr_fini
   }
   const float ai = (float)KeopsRadFormula::rowscale(xi, p) * RAD_SIGN;
   // a factor <u_i, v_j> of both indices: the sums were accumulated per component of v, u_i contracts them here
-#if RAD_DU > 0 && !RAD_UPAIR
+#if RAD_DU > 0 && !RAD_UPAIR && !RAD_BIL
   T uv[RAD_DU];
   KeopsRadFormula::rowvec(xi, p, uv);
 #endif
@@ -386,7 +417,7 @@ extern "C" __global__ void __launch_bounds__(RAD_ROWS_PER_BLOCK) keops_radr_fini
 #pragma unroll
   for (int k = 0; k < RAD_D; k++) {
     const float xc = (float)((double)x[k] - (double)P.ctr[r * RAD_D + k]);
-#if RAD_DU > 0 && !RAD_UPAIR
+#if RAD_DU > 0 && !RAD_UPAIR && !RAD_BIL
     float acc = 0.f;
 #pragma unroll
     for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], __builtin_fmaf(xc, s[d * (RAD_D + 1) + RAD_D], -s[d * (RAD_D + 1) + k]), acc);
@@ -395,7 +426,7 @@ extern "C" __global__ void __launch_bounds__(RAD_ROWS_PER_BLOCK) keops_radr_fini
     P.out[i * RAD_DOUT + k] = (T)(ai * (float)RAD_DIFF * __builtin_fmaf(xc, s[RAD_D], -s[k]));
 #endif
   }
-#elif RAD_DU > 0
+#elif RAD_DU > 0 && !RAD_BIL
   float acc = 0.f;
 #pragma unroll
   for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], s[d], acc);

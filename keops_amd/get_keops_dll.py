@@ -918,6 +918,9 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     D = x.dim
     dimw = 1 if W is None else W.dim
     du = 0 if U is None else U.dim
+    # a factor <u_i, v_j>: out of the matrix cores like the exponent when its term products fit the slot vectors
+    # (decided below, once the exponent's slots are counted), else expanded per component of v_j or formed per pair
+    bil = 0
     upair = int(bool(diff and U is not None and dimw * (D + 1) > config.radial_max_dv))  # <u_i, v_j> formed per pair
     Dv = (D + 1 if upair else dimw * (D + 1)) if diff else dimw   # components accumulated per pair
     dout = D if diff else (1 if U is not None else dimw)          # components of the output
@@ -946,14 +949,26 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     prod(Mi, Mi); prod(H, Lo); prod(Lo, H); norm(2)
     prod(Mi, Lo); norm(3)
     pad(16)
-    nkb = len(rows) // 16
+    nkb = nke = len(rows) // 16
     if nkb > 4:
         return None, None
+    # (with the difference factor only: a plain sum over <u_i, v_j> is cheaper expanded per component of v_j, 15.0
+    # against 16.8 ms at three components)
+    if U is not None and diff and config.radial_bilinear and nke + -(-6 * dimw // 16) <= 4:
+        # slot kind 4: term of a component of u_i (rows) / v_j (columns); six term products per component
+        bil, upair = 1, 0
+        for tr, tc in ((H, H), (H, Mi), (Mi, H), (Mi, Mi), (H, Lo), (Lo, H)):
+            for k in range(dimw):
+                rows.append((4, k, tr))
+                cols.append((4, k, tc))
+        pad(16)
+        nkb = len(rows) // 16
+        Dv = D + 1 if diff else 1
     # output rows per wavefront (32-row blocks) and wavefronts per workgroup: the accumulators (16 per block and
     # accumulated component) live in registers
     # from config.radial_mm_min_dv accumulated components on, the weighted sum runs on the matrix cores too (the three
     # bfloat16 terms of the weights side by side in the 32 operand columns): 16 accumulators per block of 32 rows
-    mm = int(config.radial_mm_min_dv <= Dv <= config.radial_mm_max_dv and not upair)
+    mm = int(config.radial_mm_min_dv <= Dv <= config.radial_mm_max_dv and not upair and not bil)
     if Dv > config.radial_max_dv and not mm:
         return None, None  # the accumulators of that many components do not fit the registers
     rb = (config.radial_mm_rb if mm else 2) if (mm or Dv <= config.radial_rb2_max_dv) else 1
@@ -1000,10 +1015,10 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     ra, rd, ro = VarLayout.table(al.rowvars)
     # a scalar weight and no difference factor: the weight joins the exponent, columns are partitioned by its sign
     fold = int(config.radial_fold and dimw == 1 and not diff and not rows_per_block and not mm)
-    meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_mm_nb=-(-3 * Dv // 32), rad_ws=(dimw + D + 1 if upair else Dv), rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
+    meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_mm_nb=-(-3 * Dv // 32), rad_ws=(dimw + D + 1 if upair else Dv), rad_bil=bil, rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
                 rad_yarg=y.ind, rad_fold=fold, rad_tj=tj)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
-    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DU=du, RAD_UPAIR=upair, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
+    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DU=du, RAD_UPAIR=upair, RAD_BIL=bil, RAD_NKE=nke, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
                 RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit)!r}f",
                 RAD_NCOLVARS=len(wl.colvars), RAD_DIMY=wl.dimy, RAD_NROWVARS=len(al.rowvars), RAD_DIMX=al.dimx)
     src += [f"#define {k} {v}" for k, v in defs.items()]
@@ -1066,7 +1081,7 @@ def get_keops_dll(
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
            use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs), int(batch_total),
            binder.templates_digest(), bool(config.radial), bool(config.radial_fold), bool(config.radial_ranges), int(config.radial_mm_min_dv),
-           int(config.radial_mm_rb), int(config.radial_mm_terms), bool(config.knn_i8), bool(use_half))
+           int(config.radial_mm_rb), int(config.radial_mm_terms), bool(config.radial_bilinear), bool(config.knn_i8), bool(use_half))
     with _lock:
         hit = _cache.get(key)
     if hit is not None:

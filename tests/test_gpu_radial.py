@@ -302,19 +302,34 @@ def test_gradient_with_respect_to_the_points_with_vector_weights():
     g = torch.tensor([0.6], device="cuda")
     xr = x.clone().requires_grad_(True)
     (_genred(D, Dv)(xr, y, b, g) * e).sum().backward()
-    assert _last_meta("radial") == "1" and _last_meta("rad_dv") == "6" and _path_status() == 1
+    assert _last_meta("radial") == "1" and _last_meta("rad_dv") == "3" and _path_status() == 1
     xd = x.double().requires_grad_(True)
     ((torch.exp(-0.6 * torch.cdist(xd, y.double()) ** 2) @ b.double()) * e.double()).sum().backward()
     assert float((xr.grad.double() - xd.grad).norm() / xd.grad.norm()) <= 1e-5
-    # three components in space would be 12 sums: the sweep forms <e_i, b_j> per pair instead and keeps 4
+    assert _last_meta("rad_bil") == "1"   # <e_i, b_j> out of the matrix cores, next to the exponent
+    # the same with the expanded sums (2 x 3 per pair, contracted with e_i at the end)
+    import keops_amd.config as cfg
+    cfg.radial_bilinear = False
+    try:
+        xe = x.clone().requires_grad_(True)
+        (_genred(D, Dv, sum_scheme="direct_sum")(xe, y, b, g) * e).sum().backward()   # (another module: the option is part of its key)
+        assert _last_meta("radial") == "1" and _last_meta("rad_bil") == "0" and _last_meta("rad_dv") == "6" and _path_status() == 1
+        assert float((xe.grad.double() - xd.grad).norm() / xd.grad.norm()) <= 1e-5
+    finally:
+        cfg.radial_bilinear = True
+    # three components in space: 4 sums per pair either way; in six dimensions the slot vectors have no room for the
+    # second product and the sweep forms <e_i, b_j> per pair on the vector ALU
+    for D3, mode in ((3, "bil"), (6, "upair")):
+        x3, y3 = torch.randn(M, D3, device="cuda", generator=gen), torch.randn(N, D3, device="cuda", generator=gen)
+        b3, e3 = torch.randn(N, 3, device="cuda", generator=gen), torch.randn(M, 3, device="cuda", generator=gen)
+        xr3 = x3.clone().requires_grad_(True)
+        (_genred(D3, 3)(xr3, y3, b3, g) * e3).sum().backward()
+        assert _last_meta("radial") == "1" and _last_meta("rad_dv") == str(D3 + 1) and _path_status() == 1
+        assert _last_meta("rad_bil") == ("1" if mode == "bil" else "0")
+        xd3 = x3.double().requires_grad_(True)
+        ((torch.exp(-0.6 * torch.cdist(xd3, y3.double()) ** 2) @ b3.double()) * e3.double()).sum().backward()
+        assert float((xr3.grad.double() - xd3.grad).norm() / xd3.grad.norm()) <= 1e-5
     x3, y3 = torch.randn(M, 3, device="cuda", generator=gen), torch.randn(N, 3, device="cuda", generator=gen)
-    b3, e3 = torch.randn(N, 3, device="cuda", generator=gen), torch.randn(M, 3, device="cuda", generator=gen)
-    xr3 = x3.clone().requires_grad_(True)
-    (_genred(3, 3)(xr3, y3, b3, g) * e3).sum().backward()
-    assert _last_meta("radial") == "1" and _last_meta("rad_dv") == "4" and _path_status() == 1
-    xd3 = x3.double().requires_grad_(True)
-    ((torch.exp(-0.6 * torch.cdist(xd3, y3.double()) ** 2) @ b3.double()) * e3.double()).sum().backward()
-    assert float((xr3.grad.double() - xd3.grad).norm() / xd3.grad.norm()) <= 1e-5
     # eight components: the general-purpose kernel
     b8, e8 = torch.randn(N, 8, device="cuda", generator=gen), torch.randn(M, 8, device="cuda", generator=gen)
     xr8 = x3.clone().requires_grad_(True)
