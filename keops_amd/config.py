@@ -60,6 +60,11 @@ radial_max_dv = 8                   # components of the weights (16 accumulators
 # 45.3 against 42.5 ms at 8; 300 000 x 300 000 points in space)
 radial_upair_max_dw = int(os.environ.get("KEOPS_AMD_RADIAL_UPAIR_MAX_DW", 5))
 radial_bilinear = os.environ.get("KEOPS_AMD_RADIAL_BILINEAR", "1") != "0"   # a factor <u_i, v_j> out of the matrix cores, like the exponent
+# ... up to this many components and k blocks of the slot vectors together (300 000 x 300 000 points in space, gradient
+# with 8 weight components, five k blocks: 31.6 against 43.8 ms on the general-purpose kernel; 10 components, six k
+# blocks: 64.8 against 49.8 ms)
+radial_bilinear_max_dw = int(os.environ.get("KEOPS_AMD_RADIAL_BILINEAR_MAX_DW", 8))
+radial_bilinear_max_nkb = int(os.environ.get("KEOPS_AMD_RADIAL_BILINEAR_MAX_NKB", 5))
 radial_mm_max_dv = 32               # ... when the weighted sum runs on the matrix cores (the three terms of the weights in up to three blocks of 32 operand columns)
 # the path is taken when |c| log2(e) (max |x^|^2 + max |y^|^2) <= this bound for the centred points (checked on the
 # device): the exponent is then off by at most 8 * 2^-24 of it, a kernel value by 7e-5 at worst and 1e-6 typically

@@ -886,7 +886,8 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
         # beyond 8 sums the sweep forms <u_i, v_j> per pair itself and keeps D + 1 sums (u_i of its rows in registers)
         if red.formula.dim != x.dim or x.dim + 1 > config.radial_max_dv:
             return None
-        if U is not None and dimw * (x.dim + 1) > config.radial_max_dv and dimw > config.radial_upair_max_dw:
+        if U is not None and dimw * (x.dim + 1) > config.radial_max_dv and dimw > max(config.radial_upair_max_dw,
+                                                                                         config.radial_bilinear_max_dw if config.radial_bilinear else 0):
             return None
         if U is None and not fits(x.dim + 1):
             return None
@@ -954,7 +955,7 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
         return None, None
     # (with the difference factor only: a plain sum over <u_i, v_j> is cheaper expanded per component of v_j, 15.0
     # against 16.8 ms at three components)
-    if U is not None and diff and config.radial_bilinear and nke + -(-6 * dimw // 16) <= 4:
+    if U is not None and diff and config.radial_bilinear and dimw <= config.radial_bilinear_max_dw and nke + -(-6 * dimw // 16) <= config.radial_bilinear_max_nkb:
         # slot kind 4: term of a component of u_i (rows) / v_j (columns); six term products per component
         bil, upair = 1, 0
         for tr, tc in ((H, H), (H, Mi), (Mi, H), (Mi, Mi), (H, Lo), (Lo, H)):
@@ -968,6 +969,8 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     # accumulated component) live in registers
     # from config.radial_mm_min_dv accumulated components on, the weighted sum runs on the matrix cores too (the three
     # bfloat16 terms of the weights side by side in the 32 operand columns): 16 accumulators per block of 32 rows
+    if upair and dimw > config.radial_upair_max_dw:
+        return None, None  # too wide for the per-pair form, and the slot vectors had no room
     mm = int(config.radial_mm_min_dv <= Dv <= config.radial_mm_max_dv and not upair and not bil)
     if Dv > config.radial_max_dv and not mm:
         return None, None  # the accumulators of that many components do not fit the registers

@@ -330,8 +330,12 @@ def test_gradient_with_respect_to_the_points_with_vector_weights():
         ((torch.exp(-0.6 * torch.cdist(xd3, y3.double()) ** 2) @ b3.double()) * e3.double()).sum().backward()
         assert float((xr3.grad.double() - xd3.grad).norm() / xd3.grad.norm()) <= 1e-5
     x3, y3 = torch.randn(M, 3, device="cuda", generator=gen), torch.randn(N, 3, device="cuda", generator=gen)
-    # eight components: the general-purpose kernel
-    b8, e8 = torch.randn(N, 8, device="cuda", generator=gen), torch.randn(M, 8, device="cuda", generator=gen)
-    xr8 = x3.clone().requires_grad_(True)
-    (_genred(3, 8)(xr8, y3, b8, g) * e8).sum().backward()
-    assert _last_meta("radial") is None
+    # eight components: three more k blocks, five in all; twelve: the general-purpose kernel
+    for Dv8, radial in ((8, "1"), (12, None)):
+        b8, e8 = torch.randn(N, Dv8, device="cuda", generator=gen), torch.randn(M, Dv8, device="cuda", generator=gen)
+        xr8 = x3.clone().requires_grad_(True)
+        (_genred(3, Dv8)(xr8, y3, b8, g) * e8).sum().backward()
+        assert _last_meta("radial") == radial
+        xd8 = x3.double().requires_grad_(True)
+        ((torch.exp(-0.6 * torch.cdist(xd8, y3.double()) ** 2) @ b8.double()) * e8.double()).sum().backward()
+        assert float((xr8.grad.double() - xd8.grad).norm() / xd8.grad.norm()) <= 1e-5
