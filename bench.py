@@ -56,6 +56,9 @@ WORKLOADS = {
     "gauss_1m_dv1": ("Gaussian kernel sum 1e6 x 1e6, D=3, Dv=1, float32 (benchmark configuration 2)", 14, "valu"),
     "gauss_1m_dv8": ("Gaussian kernel sum 1e6 x 1e6, D=3, Dv=8, float32 (benchmark configuration 2)", 28, "valu"),
     "gauss_1m_grad": ("gradient wrt x of the Gaussian kernel sum 1e6 x 1e6, D=3, Dv=1 (benchmark configuration 2)", 21, "valu"),
+    # sum_j K_ij <e_i, b_j> (x_i - y_j) with three-component e and b (momentum-weighted gradient of shape models):
+    # 12 flop of the kernel, 6 of the scalar product, 3 differences, 1 + 6 of the weighted accumulation
+    "gauss_300k_grad_dv3": ("gradient wrt x of the Gaussian kernel sum 3e5 x 3e5, D=3, three weight components", 28, "valu"),
     "gauss_10k": ("Gaussian kernel sum 1e4 x 1e4, D=3, Dv=1, float32 (benchmark configuration 1)", 14, "valu"),
     "gauss_100k": ("Gaussian kernel sum 1e5 x 1e5, D=3, Dv=1, float32 (reference benchmarks/README.md:13)", 14, "valu"),
     # 2*D flop of the <x,y> contraction per pair (the matrix-core work); filter and re-rank are not counted
@@ -87,9 +90,9 @@ WORKLOADS = {
 def _np_inputs(name):
     import numpy as np
 
-    if name.startswith("gauss_1m") or name in ("gauss_10k", "gauss_100k", "gauss_dv256"):
-        M = N = {"gauss_10k": 10_000, "gauss_100k": 100_000, "gauss_dv256": 200_000}.get(name, 1_000_000)
-        Dv = 8 if name.endswith("dv8") else (256 if name == "gauss_dv256" else 1)
+    if name.startswith("gauss_1m") or name in ("gauss_10k", "gauss_100k", "gauss_dv256", "gauss_300k_grad_dv3"):
+        M = N = {"gauss_10k": 10_000, "gauss_100k": 100_000, "gauss_dv256": 200_000, "gauss_300k_grad_dv3": 300_000}.get(name, 1_000_000)
+        Dv = 8 if name.endswith("dv8") else (256 if name == "gauss_dv256" else (3 if name.endswith("dv3") else 1))
         rng = np.random.default_rng(0 if name == "gauss_10k" else 1)
         x = rng.standard_normal((M, 3)).astype(np.float32)
         y = rng.standard_normal((N, 3)).astype(np.float32)
@@ -174,12 +177,12 @@ def build_step(name):
         kept_pairs = int(keep.sum().item()) * per * per  # effective pairs: kept cluster pairs only
         return (lambda: sp(*dev, ranges=ranges)), kept_pairs, inp
     conv = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", f"b=Vj({Dv})", "g=Pm(1)"], reduction_op="Sum", axis=1)
-    if name == "gauss_1m_grad":
+    if name in ("gauss_1m_grad", "gauss_300k_grad_dv3"):
         # the gradient is another map-reduce (pykeops generic_red.py:165-214): run the forward once,
-        # then every step back-propagates G = ones through it, which launches the gradient kernel only
+        # then every step back-propagates G through it, which launches the gradient kernel only
         dev[0].requires_grad_(True)
         a = conv(*dev)
-        G = torch.ones_like(a)
+        G = torch.ones_like(a) if Dv == 1 else torch.randn(a.shape, device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
 
         def step():
             return torch.autograd.grad(a, [dev[0]], G, retain_graph=True)[0]
