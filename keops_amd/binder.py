@@ -54,7 +54,6 @@ def lib():
             P, ctypes.c_int, P, P, P, P, P,
         ]
         L.keops_hip_noalloc_scratch_bytes.restype = ctypes.c_size_t
-        L.keops_hip_calibrate.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 2
         L.keops_hip_ranges_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint)]
         L.keops_hip_path_status.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint)]
         _lib = L
@@ -65,13 +64,25 @@ def noalloc_scratch_bytes():
     return int(lib().keops_hip_noalloc_scratch_bytes())
 
 
+_calib = None
+
+
 def calibrate(kind, chains, blocks, iters, device_id=0):
-    """(milliseconds, counted instructions per wavefront) of one loop-only calibration kernel
-    (keops_hip_calibrate of include/keops_hip.h)."""
+    """(milliseconds, counted instructions per wavefront) of one loop-only calibration kernel: keops_calibrate of
+    csrc/keops_calibrate.h, in the benchmark-only library libkeops_calibrate.so (built by csrc/build_lib.py)."""
+    global _calib
+    if _calib is None:
+        from .csrc import build_lib
+
+        path = build_lib.CALIB_LIB
+        if not os.path.exists(path):
+            build_lib.build()
+        _calib = ctypes.CDLL(path)
+        _calib.keops_calibrate.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 2
     ms, ipw = ctypes.c_double(0), ctypes.c_double(0)
-    rc = lib().keops_hip_calibrate(int(device_id), int(kind), int(chains), int(blocks), int(iters), ctypes.byref(ms), ctypes.byref(ipw))
+    rc = _calib.keops_calibrate(int(device_id), int(kind), int(chains), int(blocks), int(iters), ctypes.byref(ms), ctypes.byref(ipw))
     if rc != 0:
-        raise KeOpsHipError(f"calibration failed (code {rc}): {last_error()}")
+        raise KeOpsHipError(f"calibration failed (code {rc}): kind or chains out of range, or no device")
     return ms.value, ipw.value
 
 

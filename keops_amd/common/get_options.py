@@ -1,6 +1,7 @@
 """Backend string -> (tagCPUGPU, tag1D2D, tagHostDevice), as
-pykeops/pykeops/common/get_options.py:14-140.  The HIP engine only computes on device-resident
-torch tensors: "CPU" and host-memory variants are rejected when the call is made."""
+pykeops/pykeops/common/get_options.py:14-140.  Every GPU backend is served: device-resident tensors travel as
+device pointers (tagHostDevice = 1), host tensors and NumPy arrays as host pointers that the library stages
+(tagHostDevice = 0).  "CPU" is rejected when the call is made: there is no CPU engine behind this front end."""
 
 POSSIBLE_BACKENDS = [
     "auto", "CPU", "GPU", "GPU_1D", "GPU_1D_device", "GPU_1D_host", "GPU_2D", "GPU_2D_device", "GPU_2D_host",

@@ -191,6 +191,10 @@ int64_t broadcast_index(int64_t i, int nbatchdims, const int64_t* full_shape, co
 
 // set for the duration of keops_hip_launch_noalloc on the calling thread: nothing may be allocated or freed
 thread_local bool g_noalloc = false;
+// set while a host-pointer launch runs: its ranges are host memory, so they are validated on the host at every call
+thread_local bool g_host_ranges = false;
+// set while a use_half launch runs on the float32 copies of half-precision arguments
+thread_local bool g_half_data = false;
 
 struct DeviceBuffer {
   void* ptr = nullptr;
@@ -269,7 +273,10 @@ struct Module {
   const unsigned* last_guard = nullptr;  // flag of the last launch's device-side choice between two kernel families
   int64_t ranges_work_total = 0;  // of the validated ranges: reduced rows swept, summed over the row ranges
   double ranges_pairs = 0.0;      // ... and their pairs
-  const unsigned* ranges_status = nullptr;
+  // status words of the tables built on the device, in pinned host memory that the kernels write directly (no
+  // read-back): [0] an index was clamped, [1] workgroups were dropped.  Sticky until the host has looked at them.
+  unsigned* ranges_status = nullptr;      // host address
+  unsigned* ranges_status_dev = nullptr;  // the same words as the device sees them
   DeviceBuffer staging;  // host-pointer launches (tagHostDevice = 0): device copies of the arguments and of out
   // a launch was recorded into a HIP graph: workspaces and tables keep their address and contents from then on
   bool captured = false;
@@ -374,11 +381,22 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
     const int64_t nred_u = ranges[6][sel + 2];
     ukey = {tagI, by_arg ? 1 : 0, rows_per_block, (int64_t)(intptr_t)rx_dev, (int64_t)(intptr_t)slices_dev,
             (int64_t)(intptr_t)ry_dev, nranges, ranges[6][sel + 1], nred_u, rows_total, cols_total};
-    if (device_ranges_enabled() && nb == 0 && nranges >= 0 && nred_u >= 0 && ukey == m.ranges_key) {
-      // These ranges (same tensors, same sizes) have been read and validated by an earlier call: the table is now
-      // built on the device from their current contents, with every index clamped to its axis.  No read-back, no
-      // synchronisation; the launch can be recorded in a HIP graph.
+    if (device_ranges_enabled() && !g_host_ranges && nb == 0 && nranges >= 0 && nred_u >= 0 && ukey == m.ranges_key && m.ranges_status) {
+      // These ranges (same addresses, same sizes: the key is the identity of the buffers, not their contents) have
+      // been read and validated by an earlier call: the table is now built on the device from their current
+      // contents, with every index clamped to its axis.  No read-back, no synchronisation; the launch can be
+      // recorded in a HIP graph.  What had to be clamped is reported through two sticky status words that the
+      // kernels write into pinned host memory: keops_hip_ranges_status reads and clears them, and a launch that finds
+      // them set by an earlier launch fails, so out-of-bounds ranges never go unnoticed.
       if (g_noalloc) return fail(-1, "keops_hip_launch_noalloc: block-sparse and batched launches build device tables");
+      if (const unsigned pending = (m.ranges_status[0] ? 1u : 0u) | (m.ranges_status[1] ? 2u : 0u)) {
+        m.ranges_status[0] = m.ranges_status[1] = 0u;
+        return fail(-1, std::string("an earlier block-sparse launch of this module found its ranges invalid (") +
+                        ((pending & 1u) ? "an index was out of bounds and has been clamped to its axis" : "") +
+                        ((pending & 3u) == 3u ? "; " : "") +
+                        ((pending & 2u) ? "the row ranges overlap so much that workgroups were dropped" : "") +
+                        "): its result is not the reduction over the ranges as given");
+      }
       const int64_t nblocks_max = std::max(nranges + rows_total / rows_per_block, m.ranges_nblocks);
       const size_t words = keops_static_range_build_words(nranges, nred_u, nblocks_max);
       const bool capturing = stream_is_capturing(stream);
@@ -401,9 +419,8 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
       B.work = B.nb + nranges;
       B.order = B.work + nranges;
       B.offs = B.order + nranges;
-      B.status = (unsigned*)(B.offs + nranges);
+      B.status = m.ranges_status_dev;
       if (int e = keops_static_build_ranges(&B, stream)) return fail(e, "building the range tables on the device failed");
-      m.ranges_status = B.status;
       rt.nblocks = nblocks_max;
       rt.lookup = (const int64_t*)B.lookup;
       rt.offsets = nullptr;
@@ -560,9 +577,13 @@ int prepare_range_tables(Module& m, const ShapeTable& S, int tagI, bool user_ran
     m.cached_nblocks = nblocks;
   }
   if (user_ranges) {
+    if (!m.ranges_status && !g_noalloc && !g_host_ranges) {
+      HIP_TRY(hipHostMalloc((void**)&m.ranges_status, 64, hipHostMallocMapped));
+      m.ranges_status[0] = m.ranges_status[1] = 0u;
+      HIP_TRY(hipHostGetDevicePointer((void**)&m.ranges_status_dev, m.ranges_status, 0));
+    }
     m.ranges_key = ukey;  // read and validated: later calls build the table on the device
     m.ranges_nblocks = nblocks;
-    m.ranges_status = nullptr;
     m.ranges_work_total = 0;
     m.ranges_pairs = 0.0;
     for (int64_t r = 0; r < nranges; r++) {
@@ -1089,6 +1110,12 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
   // one half-precision term per component when the data are half-precision numbers (no lo parts, no centring)
   const bool single = m.meta_int("chk_single", 0) != 0;
+  // one half-precision term per component is only exact for data that IS half precision
+  if (single != g_half_data)
+    return fail(-1, single ? "this module was compiled for half-precision data (use_half = 1 in get_keops_dll): launch it with "
+                             "use_half = 1; float32 operands would be truncated to 11 bits"
+                           : "this module was compiled for float32 data: a use_half launch needs the module that get_keops_dll "
+                             "returns for use_half = 1");
   const size_t o_xs = take((size_t)nxs * DP * (single ? 2 : 4)), o_ys = take((size_t)nys * DP * (single ? 2 : 4));
   const size_t o_xn = take((size_t)nxs * 4), o_yn = take((size_t)nys * 4), o_scal = take(8);
   // final-product variant: slabs over the reduced axis fill the chip and round the grid to whole
@@ -1438,6 +1465,8 @@ void keops_hip_module_destroy(void* module) {
   m->staging.release();
   if (m->last_done) (void)hipEventDestroy(m->last_done);
   if (m->pinned) (void)hipHostFree(m->pinned);
+  // (the status words are not read here: at interpreter exit the runtime may already have unmapped pinned memory)
+  if (m->ranges_status) (void)hipHostFree(m->ranges_status);
   for (void* p : m->retired_pinned) (void)hipHostFree(p);
   if (m->tables_copied) (void)hipEventDestroy(m->tables_copied);
   if (m->ev0) (void)hipEventDestroy(m->ev0);
@@ -1801,10 +1830,13 @@ static int launch_from_host(Module& m, int64_t nx, int64_t ny, int tagI, int tag
     }
     dranges[6] = ranges[6];
   }
-  if (int rc = launch_on_device(m, nx, ny, tagI, tagZero, tag1D2D, dimred, indsi, ni, indsj, nj, indsp, np, dimout, dimsx, dimsy,
-                                dimsp, user_ranges ? dranges : ranges, shapeout, nshapeout, base + out_off, dargs.data(),
-                                argshapes_flat, argndims, stream, 0))
-    return rc;
+  // (the ranges are host memory: validated on the host at every call, never through the device-built tables)
+  g_host_ranges = true;
+  const int rc_launch = launch_on_device(m, nx, ny, tagI, tagZero, tag1D2D, dimred, indsi, ni, indsj, nj, indsp, np, dimout, dimsx,
+                                         dimsy, dimsp, user_ranges ? dranges : ranges, shapeout, nshapeout, base + out_off,
+                                         dargs.data(), argshapes_flat, argndims, stream, 0);
+  g_host_ranges = false;
+  if (rc_launch) return rc_launch;
   if (out_bytes) HIP_TRY(hipMemcpyAsync(out, base + out_off, out_bytes, hipMemcpyDeviceToHost, stream));
   HIP_TRY(hipStreamSynchronize(stream));
   return 0;
@@ -1852,9 +1884,12 @@ static int launch_half(Module& m, int64_t nx, int64_t ny, int tagI, int tagZero,
     if (int e = keops_static_convert_half(fargs[k], args[k], arg_n[k], 1, stream))
       return fail(e, std::string("half -> float conversion failed: ") + hipGetErrorString((hipError_t)e));
   }
-  if (int rc = launch_on_device(m, nx, ny, tagI, tagZero, tag1D2D, dimred, indsi, ni, indsj, nj, indsp, np, dimout, dimsx, dimsy,
-                                dimsp, ranges, shapeout, nshapeout, base + out_off, fargs.data(), argshapes_flat, argndims, stream, 0))
-    return rc;
+  g_half_data = true;
+  const int rc_launch = launch_on_device(m, nx, ny, tagI, tagZero, tag1D2D, dimred, indsi, ni, indsj, nj, indsp, np, dimout, dimsx,
+                                         dimsy, dimsp, ranges, shapeout, nshapeout, base + out_off, fargs.data(), argshapes_flat,
+                                         argndims, stream, 0);
+  g_half_data = false;
+  if (rc_launch) return rc_launch;
   if (int e = keops_static_convert_half(out, base + out_off, sizeout, 0, stream))
     return fail(e, std::string("float -> half conversion failed: ") + hipGetErrorString((hipError_t)e));
   if (!capturing && m.last_done) HIP_TRY(hipEventRecord(m.last_done, stream));  // the conversion reads the staging buffer too
@@ -1941,34 +1976,11 @@ int keops_hip_ranges_status(void* module, unsigned* status) {
   if (!m.ranges_status) return 0;
   HIP_TRY(hipSetDevice(m.device));
   if (m.has_last) HIP_TRY(hipEventSynchronize(m.last_done));
-  HIP_TRY(hipMemcpy(status, m.ranges_status, sizeof(unsigned), hipMemcpyDeviceToHost));
+  *status = (m.ranges_status[0] ? 1u : 0u) | (m.ranges_status[1] ? 2u : 0u);
+  m.ranges_status[0] = m.ranges_status[1] = 0u;  // read: the next launch starts clean
   return 0;
 }
 
 size_t keops_hip_noalloc_scratch_bytes(void) { return (size_t)KEOPS_STATIC_SCRATCH_BYTES; }
-
-int keops_hip_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave) {
-  if (!ms || !instr_per_wave || blocks <= 0 || iters <= 0) return fail(-1, "keops_hip_calibrate: bad arguments");
-  HIP_TRY(hipSetDevice(device_id < 0 ? 0 : device_id));
-  float* out = nullptr;
-  HIP_TRY(hipMalloc((void**)&out, (size_t)blocks * 256 * sizeof(float) + KEOPS_STATIC_STREAM_BYTES));
-  hipEvent_t e0 = nullptr, e1 = nullptr;
-  int rc = 0;
-  auto cleanup = [&] { if (e0) (void)hipEventDestroy(e0); if (e1) (void)hipEventDestroy(e1); (void)hipFree(out); };
-  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { cleanup(); return fail(-1, "hipEventCreate failed"); }
-  // one untimed pass (code upload, clocks), then the timed one
-  for (int pass = 0; pass < 2 && rc == 0; pass++) {
-    (void)hipEventRecord(e0, nullptr);
-    rc = keops_static_calibrate(kind, chains, blocks, iters, out, nullptr, instr_per_wave);
-    (void)hipEventRecord(e1, nullptr);
-    if (rc == 0 && hipEventSynchronize(e1) != hipSuccess) rc = -1;
-  }
-  float t = 0.f;
-  if (rc == 0 && hipEventElapsedTime(&t, e0, e1) != hipSuccess) rc = -1;
-  cleanup();
-  if (rc != 0) return fail(rc, "calibration loop failed: kind or chains out of range (see keops_hip_calibrate in keops_hip.h)");
-  *ms = t;
-  return 0;
-}
 
 }  // extern "C"

@@ -11,9 +11,6 @@ int keops_static_scratch(int device, void** ptr, size_t* bytes);
 int keops_static_fill_zero(void* dst, size_t bytes, void* stream);
 // n elements: IEEE half -> float (to_float != 0) or float -> half (round to nearest even)
 int keops_static_convert_half(void* dst, const void* src, long long n, int to_float, void* stream);
-// out: blocks * 256 floats, followed by KEOPS_STATIC_STREAM_BYTES of tile data for the kinds that stream tiles
-#define KEOPS_STATIC_STREAM_BYTES ((size_t)64 * 32 * 512 * 2)
-int keops_static_calibrate(int kind, int chains, int blocks, int iters, float* out, void* stream, double* instr_per_wave);
 
 // Lookup table of a block-sparse launch built on the device (no read-back of the ranges): see keops_static.hip.
 struct KeopsRangeBuild {
@@ -22,7 +19,8 @@ struct KeopsRangeBuild {
   long long *lookup;              // out: [nblocks_max][3] (range id, first row, end row); unused entries are empty
   long long *sl_clean, *ry_clean; // out: copies of sl / ry with every index clamped to its axis
   long long *nb, *work, *order, *offs;  // work arrays [nranges] each
-  unsigned *status;               // out: bit 0 an index was out of bounds (clamped), bit 1 more workgroups than nblocks_max
+  unsigned *status;               // out, host memory mapped into the device, never cleared here: [0] = 1 an index was out of
+                                  // bounds (clamped), [1] = 1 more workgroups than nblocks_max
 };
 // number of long long words the arrays above take (lookup, sl_clean, ry_clean, nb, work, order, offs, status)
 size_t keops_static_range_build_words(long long nranges, long long nred, long long nblocks_max);

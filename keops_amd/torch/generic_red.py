@@ -67,6 +67,10 @@ class GenredAutograd_base:
         tagCPUGPU, tag1D2D, tagHostDevice = get_tag_backend(params.backend, args)
         # where the data lives decides what kind of pointers the library receives, whatever the backend string says
         tagHostDevice = 1 if all(a.is_cuda for a in args) else 0
+        # (get_tag_backend has rejected arguments that are partly on the host and partly on a GPU; the output buffer a
+        # caller hands in must live where the arguments live, as in the reference)
+        if params.out is not None and bool(params.out.is_cuda) != bool(tagHostDevice):
+            raise ValueError("[KeOps] Input arrays must be all located on the same device.")
         nbatchdims = max(len(a.shape) for a in args) - 2
         use_ranges = nbatchdims > 0 or params.ranges is not None
         device_id, device_args = set_device(tagCPUGPU, tagHostDevice, params.device_id_request, *args)
@@ -121,7 +125,9 @@ class GenredAutograd_base:
             )
             args = tuple(a.contiguous() for a in args)
         if params.ranges:
-            params.ranges = tuple(r.to(memory_format=torch.contiguous_format, dtype=torch.int64) for r in params.ranges)
+            # the kernels read the ranges where they read the data (keops_nvrtc.cpp:190-208)
+            rdev = device_args if tagHostDevice == 1 else torch.device("cpu")
+            params.ranges = tuple(r.to(device=rdev, memory_format=torch.contiguous_format, dtype=torch.int64) for r in params.ranges)
         result = myconv.genred_pytorch(device_args, params.ranges, params.nx, params.ny, nbatchdims, params.out, *args)
         if host_out is not None:
             host_out.copy_(result.view(host_out.shape))

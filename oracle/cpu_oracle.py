@@ -6,7 +6,9 @@ product package imports this module; it serves the test-suite, the smoke test an
 cpu_baseline leg as the checker.
 """
 import ctypes
+import hashlib
 import os
+import shutil
 import subprocess
 
 import numpy as np
@@ -23,18 +25,31 @@ REDUCTIONS = dict(
 SCHEMES = dict(direct_sum=0, block_sum=1, kahan_scheme=2)
 
 
+def _source_digest():
+    h = hashlib.sha256()
+    for name in ("cpu_reduc.c", "Makefile"):
+        with open(os.path.join(_HERE, name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def build(force=False):
-    """Compile oracle/cpu_reduc.c into oracle/liboracle_cpu.so (make; gcc only)."""
+    """Compile oracle/cpu_reduc.c into oracle/liboracle_cpu.so (make; gcc only).  A failing compilation is an error.
+    Only a machine without make or without a C compiler uses the library that travelled with the tree, and only if
+    the digest written when it was built matches the sources beside it."""
     target = os.path.join(_HERE, "liboracle_cpu.so")
+    stamp = os.path.join(_HERE, "liboracle_cpu.digest")
+    have_tools = shutil.which("make") and (shutil.which(os.environ.get("CC", "cc")) or shutil.which("gcc"))
+    if not have_tools:
+        if not os.path.exists(target) or not os.path.exists(stamp) or open(stamp).read().strip() != _source_digest():
+            raise RuntimeError("oracle: no make / C compiler here and no liboracle_cpu.so built from these sources")
+        return target
     if force:
         subprocess.run(["make", "-C", _HERE, "clean"], check=True, stdout=subprocess.DEVNULL)
     # make is incremental: a library older than cpu_reduc.c is rebuilt, an up-to-date one is left alone
-    # (no compiler on the machine: use the library that travelled with the tree)
-    try:
-        subprocess.run(["make", "-C", _HERE], check=True, stdout=subprocess.DEVNULL)
-    except (OSError, subprocess.CalledProcessError):
-        if not os.path.exists(target):
-            raise
+    subprocess.run(["make", "-C", _HERE], check=True, stdout=subprocess.DEVNULL)
+    with open(stamp, "w") as f:
+        f.write(_source_digest())
     return target
 
 

@@ -135,3 +135,18 @@ def test_reference_named_helpers_exist_and_health_check_runs(capsys):
     assert keops_amd.check_health() is True
     out = capsys.readouterr().out
     assert "libkeops_hip.so" in out and "cache folder" in out
+
+
+def test_arguments_in_different_memories_are_rejected():
+    """x on a GPU and a parameter on the host (or an output buffer that lives elsewhere than the arguments) is the
+    reference's ValueError, not a launch with mismatched pointers (pykeops/pykeops/common/get_options.py)."""
+    from keops_amd.common.get_options import get_tag_backend
+
+    class Fake:
+        def __init__(self, cuda):
+            self.is_cuda = cuda
+
+    with pytest.raises(ValueError, match="different memory locations"):
+        get_tag_backend("auto", [Fake(True), Fake(True), Fake(False)])
+    assert get_tag_backend("auto", [Fake(True), Fake(True)]) == (1, 0, 1)
+    assert get_tag_backend("GPU_2D", [Fake(False), Fake(False)]) == (1, 1, 0)

@@ -50,7 +50,7 @@ def test_config5b_laplace_d256_row_subset():
     x, y, b = _laplace_inputs(M, N, 256, 16, 5)
     conv = Genred("Exp(-Norm2(x-y))*b", ["x=Vi(256)", "y=Vj(256)", "b=Vj(16)"], reduction_op="Sum", axis=1)
     got = conv(*to_dev(x, y, b))
-    rows = np.sort(np.random.default_rng(9).choice(M, 512, replace=False)).astype(np.int64)
+    rows = np.sort(np.random.default_rng(9).choice(M, 1024, replace=False)).astype(np.int64)
     ref = cpu_reduc("laplace", [x, y, b], M, N, 16, rows=rows)
     scale = cpu_reduc("laplace", [x, y, np.abs(b)], M, N, 16, rows=rows)
     assert_sum_parity(got[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)

@@ -142,3 +142,35 @@ def test_half_precision_launch_under_graph_capture():
         return True
 
     assert replays_like_eager(conv, [x, y, b])
+
+
+def test_module_compiled_for_half_data_refuses_float32_operands():
+    """A chunked module built for half-precision data keeps one half-precision term per component: exact for data that
+    is half precision, an 11-bit truncation for float32 data.  The ABI ties the two together: such a module only runs
+    with use_half = 1 (and a float32 module only with use_half = 0)."""
+    from keops_amd import binder, keops_io
+    from keops_amd.torch import Genred
+
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    r = lambda *s: torch.randn(*s, device="cuda", generator=gen)
+    x, y, b = (r(600, 64) / 8).half(), (r(700, 64) / 8).half(), r(700, 4).half()
+    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(64)", "y=Vj(64)", "b=Vj(4)"], reduction_op="Sum", axis=1)
+    conv(x, y, b)
+    ld = keops_io.last_loader
+    assert ld.module.meta("chk_single") == "1"
+    p = ld.params
+    xf, yf, bf = x.float(), y.float(), b.float()
+    out = torch.empty(600, 4, device="cuda")
+    with pytest.raises(binder.KeOpsHipError, match="compiled for half-precision data"):
+        ld.module(1, p.dimy, 600, 700, p.tagI, 0, 0, p.tag1D2D, p.dimred, p.cuda_block_size, p.use_chunk_mode, p.indsi,
+                  p.indsj, p.indsp, p.dim, p.dimsx, p.dimsy, p.dimsp, ld.empty_ranges, (600, 4), out.data_ptr(),
+                  (xf.data_ptr(), yf.data_ptr(), bf.data_ptr()), ((600, 64), (700, 64), (700, 4)))
+    # and the other way round: the float32 module of the same formula does not take use_half = 1
+    conv(xf, yf, bf)
+    ld32 = keops_io.last_loader
+    assert ld32.module.meta("chk_single") == "0"
+    outh = torch.empty(600, 4, device="cuda", dtype=torch.float16)
+    with pytest.raises(binder.KeOpsHipError, match="compiled for float32 data"):
+        ld32.module(1, p.dimy, 600, 700, p.tagI, 0, 1, p.tag1D2D, p.dimred, p.cuda_block_size, p.use_chunk_mode, p.indsi,
+                    p.indsj, p.indsp, p.dim, p.dimsx, p.dimsy, p.dimsp, ld32.empty_ranges, (600, 4), outh.data_ptr(),
+                    (x.data_ptr(), y.data_ptr(), b.data_ptr()), ((600, 64), (700, 64), (700, 4)))

@@ -104,3 +104,49 @@ def test_malformed_ranges_are_an_error_not_a_fault():
     with pytest.raises(binder.KeOpsHipError, match="out of bounds"):
         conv(x, y, b, ranges=negative)
     assert torch.equal(conv(x, y, b, ranges=good), ref)
+
+
+def test_host_ranges_are_validated_at_every_call():
+    """Host-pointer launches copy their ranges into the same staging addresses call after call: the second call with
+    an out-of-bounds range must fail like the first (validation on the host every time, never the device-built
+    tables that clamp)."""
+    from keops_amd import binder
+    from keops_amd.torch import Genred
+
+    x, y, b = (torch.randn(n, d) for n, d in ((1000, 3), (1200, 3), (1200, 1)))
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64)
+    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(1)"], reduction_op="Sum", axis=1)
+    good = (i64([[0, 500], [500, 1000]]), i64([1, 2]), i64([[0, 600], [600, 1200]]),
+            i64([[0, 600], [600, 1200]]), i64([1, 2]), i64([[0, 500], [500, 1000]]))
+    bad = (good[0], good[1], i64([[0, 600], [600, 1300]])) + good[3:]
+    ref = conv(x, y, b, ranges=good)
+    assert torch.equal(conv(x, y, b, ranges=good), ref)
+    for _ in range(2):
+        with pytest.raises(binder.KeOpsHipError, match="out of bounds"):
+            conv(x, y, b, ranges=bad)
+    assert torch.equal(conv(x, y, b, ranges=good), ref)
+
+
+def test_ranges_clamped_by_the_device_built_tables_fail_the_next_launch():
+    """Device tensors that an earlier call has validated are not read back again: the tables are built on the device
+    and out-of-bounds indices are clamped.  That never passes silently: unless the caller reads the status
+    (keops_hip_ranges_status), the module's next block-sparse launch fails and says why."""
+    from keops_amd import binder, keops_io
+    from keops_amd.torch import Genred
+
+    x, y, b = (torch.randn(n, d, device="cuda") for n, d in ((1000, 3), (1200, 3), (1200, 2)))
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device="cuda")
+    conv = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)"], reduction_op="Sum", axis=1)
+    rg = (i64([[0, 500], [500, 1000]]), i64([1, 2]), i64([[0, 600], [600, 1200]]),
+          i64([[0, 600], [600, 1200]]), i64([1, 2]), i64([[0, 500], [500, 1000]]))
+    ref = conv(x, y, b, ranges=rg)               # validated on the host
+    assert torch.equal(conv(x, y, b, ranges=rg), ref)   # tables built on the device
+    rg[2][1, 1] = 10 ** 9                        # edited in place: same tensors, now out of bounds
+    clamped = conv(x, y, b, ranges=rg)           # clamped to the axis, flagged
+    torch.cuda.synchronize()
+    assert torch.equal(clamped, ref)
+    with pytest.raises(binder.KeOpsHipError, match="clamped"):
+        conv(x, y, b, ranges=rg)
+    rg[2][1, 1] = 1200
+    assert torch.equal(conv(x, y, b, ranges=rg), ref)
+    assert keops_io.last_loader.module.ranges_status() == 0

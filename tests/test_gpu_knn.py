@@ -86,7 +86,7 @@ def test_knn_config3_query_subset():
 
     # bounded data: the device lets the fixed-threshold filter run on signed bytes (keops_knn_filter_i8)
     assert keops_io.last_loader.module.meta("knn_i8") == "1" and keops_io.last_loader.module.path_status() == 1
-    rows = np.sort(np.random.default_rng(7).choice(M, 512, replace=False)).astype(np.int64)
+    rows = np.sort(np.random.default_rng(7).choice(M, 1024, replace=False)).astype(np.int64)
     ref = cpu_reduc("sqdist", [x, y], M, N, 1, reduction="KMin_ArgKMin", K=K, scheme="direct_sum", rows=rows)
     sel = torch.from_numpy(rows).cuda()
     assert np.array_equal(idx[sel].cpu().numpy(), ref[:, 1::2].astype(np.int64))
