@@ -249,6 +249,41 @@ def cpu_baseline(name, inp):
     return res
 
 
+def cpu_baseline_config1():
+    """The oracle on the reference's own CPU-runnable case in full (benchmark configuration 1: Gaussian sum, M = N =
+    10,000, D = 3): median of 5 calls after one warm-up, on all host threads and on one."""
+    import numpy as np
+
+    from oracle.cpu_oracle import cpu_reduc
+
+    inp = _np_inputs("gauss_10k")
+    M, N, Dv = inp["M"], inp["N"], inp["Dv"]
+
+    def median_time():
+        cpu_reduc("gauss", inp["arrays"], M, N, Dv)
+        ts = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            cpu_reduc("gauss", inp["arrays"], M, N, Dv)
+            ts.append(time.perf_counter() - t0)
+        return float(np.median(ts))
+
+    res = {"workload": WORKLOADS["gauss_10k"][0]}
+    try:
+        gomp = ctypes.CDLL("libgomp.so.1")
+        threads = int(gomp.omp_get_max_threads())
+    except Exception:
+        gomp, threads = None, None
+    t_all = median_time()
+    res.update(value=M * N / t_all, unit="pairs/s", cores=threads, seconds=t_all)
+    if gomp is not None and threads and threads > 1:
+        gomp.omp_set_num_threads(1)
+        t1 = median_time()
+        gomp.omp_set_num_threads(threads)
+        res.update(value_1_thread=M * N / t1, seconds_1_thread=t1)
+    return res
+
+
 def calibration(mfma):
     """Issue rates of loop-only kernels (keops_hip_calibrate): wavefront instructions per cycle and SIMD at the
     nominal 2.4 GHz clock, for 1, 2 and 4 wavefronts per SIMD (256 CUs x 4 SIMDs; a workgroup is 4 wavefronts)."""
@@ -291,6 +326,77 @@ def calibration(mfma):
     return {"calibration": "mfma" if mfma else "valu", "cus": cus, "rows": rows}
 
 
+# the other targets of the hot path: reported beside the headline line so that one default run shows all of them
+SIDE_WORKLOADS = ["gauss_1m_dv8", "gauss_1m_grad", "knn_d64", "sparse_100x10k", "lse_b16", "laplace_d256"]
+
+
+def measure(workload, steps, warmup):
+    """Times `steps` passes of one workload (after `warmup` untimed ones, synchronised on both sides) and the main
+    kernels of a pass between HIP events on the launch stream."""
+    import torch
+
+    desc, flop_per_pair, bound = WORKLOADS[workload]
+    before = set(id(m) for m in kernel_modules())
+    step, pairs, inp = build_step(workload)
+    for _ in range(max(1, warmup)):
+        step()
+    torch.cuda.synchronize()
+    # kernel-only time: HIP events recorded by the library around the launch, on the launch stream; only the
+    # modules this workload loaded are asked
+    mods = [m for m in kernel_modules() if id(m) not in before] or kernel_modules()
+    for m in mods:
+        m.set_timing(True)
+    kernel_ms = []
+    for _ in range(min(3, steps)):
+        step()
+        kernel_ms.append(max(m.last_kernel_ms() for m in mods))
+    for m in mods:
+        m.set_timing(False)
+    torch.cuda.synchronize()
+
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+
+    kms = sum(kernel_ms) / len(kernel_ms)
+    achieved = pairs * flop_per_pair / (kms * 1e-3) / 1e12
+    peak = {"valu": PEAK_FP32_VECTOR_TFLOPS, "mfma": PEAK_BF16_MFMA_TFLOPS, "mfma32": PEAK_FP32_MFMA_TFLOPS,
+            "mfma8": PEAK_INT8_MFMA_TOPS}[bound]
+    note = {"valu": "peak is the packed-FP32 vector figure; packed FP32 instructions are disabled in this build. "
+                    "Gaussian sums take their exponents from the matrix cores when the device-side check allows it "
+                    "(kernels/keops_radial_mfma.h): the vector ALU then issues v_exp_f32 + one fma per pair and output "
+                    "component, and the algorithmic flop of the exponent are not vector-ALU work any more",
+            "mfma": "peak is the dense bf16 matrix figure", "mfma32": "peak is the dense fp32 matrix figure",
+            "mfma8": "peak is the dense int8 matrix figure (5.0 POP/s): the fixed-threshold filter runs on signed bytes when "
+                     "the device finds the quantisation slack small against the search radii (kernels/keops_knn_mfma.h, "
+                     "keops_knn_filter_i8); with KEOPS_AMD_KNN_I8=0 the same call runs its filter in bfloat16 "
+                     "(12.7 ms, 0.40 of the 2.5 PFLOP/s bf16 peak).  `achieved` counts the 2*D operations of <x,y> per "
+                     "pair once; sampling pass and exact re-rank are not counted"}[bound]
+    return dict(desc=desc, flop_per_pair=flop_per_pair, bound=bound, pairs=pairs, inp=inp, dt=dt, kernel_ms=kms,
+                achieved=achieved, peak=peak, note=note)
+
+
+def side_configs(steps=3, warmup=1):
+    """{workload: {ms, kernel_ms, pairs_per_s, frac, bound, peak}} for the other targets of the hot path, a few steps each."""
+    import gc
+
+    import torch
+
+    res = {}
+    for name in SIDE_WORKLOADS:
+        r = measure(name, steps, warmup)
+        res[name] = {"workload": r["desc"], "ms": r["dt"] * 1e3, "kernel_ms": r["kernel_ms"], "pairs_per_s": r["pairs"] / r["dt"],
+                     "achieved": r["achieved"], "peak": r["peak"], "unit": "TFLOP/s" if r["bound"] != "mfma8" else "TOP/s",
+                     "frac": r["achieved"] / r["peak"], "bound": "mfma" if r["bound"].startswith("mfma") else r["bound"],
+                     "flop_per_pair": r["flop_per_pair"], "steps": steps}
+        del r
+        gc.collect()
+        torch.cuda.empty_cache()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -298,6 +404,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="gauss_1m_dv1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-side-configs", action="store_true",
+                    help="default workload only: skip the short runs of the other targets (the `configs` object of the line)")
     ap.add_argument("--valu-calibration", action="store_true",
                     help="loop-only kernels: what the vector ALU sustains on chains of v_fmac_f32 and on the "
                          "instruction mix of a Gaussian pair, with and without v_exp_f32, at 1/2/4 wavefronts per SIMD")
@@ -326,44 +434,9 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4, "copies": args.steps}))
         return
-    desc, flop_per_pair, bound = WORKLOADS[args.workload]
-    step, pairs, inp = build_step(args.workload)
-
-    for _ in range(max(1, args.warmup)):
-        step()
-    torch.cuda.synchronize()
-    # kernel-only time: HIP events recorded by the library around the launch, on the launch stream
-    mods = kernel_modules()
-    for m in mods:
-        m.set_timing(True)
-    kernel_ms = []
-    for _ in range(min(3, args.steps)):
-        step()
-        kernel_ms.append(max(m.last_kernel_ms() for m in mods))
-    for m in mods:
-        m.set_timing(False)
-    torch.cuda.synchronize()
-
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
-
-    kms = sum(kernel_ms) / len(kernel_ms)
-    achieved = pairs * flop_per_pair / (kms * 1e-3) / 1e12
-    peak = {"valu": PEAK_FP32_VECTOR_TFLOPS, "mfma": PEAK_BF16_MFMA_TFLOPS, "mfma32": PEAK_FP32_MFMA_TFLOPS,
-            "mfma8": PEAK_INT8_MFMA_TOPS}[bound]
-    note = {"valu": "peak is the packed-FP32 vector figure; packed FP32 instructions are disabled in this build. "
-                    "Gaussian sums take their exponents from the matrix cores when the device-side check allows it "
-                    "(kernels/keops_radial_mfma.h): the vector ALU then issues v_exp_f32 + one fma per pair and output "
-                    "component, and the algorithmic flop of the exponent are not vector-ALU work any more",
-            "mfma": "peak is the dense bf16 matrix figure", "mfma32": "peak is the dense fp32 matrix figure",
-            "mfma8": "peak is the dense int8 matrix figure (5.0 POP/s): the fixed-threshold filter runs on signed bytes when "
-                     "the device finds the quantisation slack small against the search radii (kernels/keops_knn_mfma.h, "
-                     "keops_knn_filter_i8); with KEOPS_AMD_KNN_I8=0 the same call runs its filter in bfloat16 "
-                     "(12.7 ms, 0.40 of the 2.5 PFLOP/s bf16 peak).  `achieved` counts the 2*D operations of <x,y> per "
-                     "pair once; sampling pass and exact re-rank are not counted"}[bound]
+    r = measure(args.workload, args.steps, args.warmup)
+    desc, flop_per_pair, bound, pairs, inp, dt, kms, achieved, peak, note = (
+        r["desc"], r["flop_per_pair"], r["bound"], r["pairs"], r["inp"], r["dt"], r["kernel_ms"], r["achieved"], r["peak"], r["note"])
     out = {
         "metric": "pair interactions/sec (M*N/s), 1e6x1e6 D=3 Gauss sum" if args.workload == "gauss_1m_dv1"
         else "pair interactions/sec (M*N/s)",
@@ -387,8 +460,13 @@ def main():
             "note": note,
         },
     }
+    if args.workload == "gauss_1m_dv1" and not args.no_side_configs:
+        del r, inp
+        out["configs"] = side_configs()
     if args.workload == "gauss_1m_dv1" and not args.no_cpu_baseline:
+        inp = _np_inputs(args.workload)
         out["cpu_baseline"] = cpu_baseline(args.workload, inp)
+        out["cpu_baseline"]["config1"] = cpu_baseline_config1()
     print(json.dumps(out))
 
 
