@@ -50,9 +50,6 @@ chunk_max_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MAX_DIM", 1024))  # largest 
 
 # exponents of low-dimensional Gaussian kernel sums on the matrix cores (csrc/kernels/keops_radial_mfma.h)
 radial = os.environ.get("KEOPS_AMD_RADIAL", "1") != "0"
-# scalar weights join the exponents (columns partitioned by sign, add/subtract instead of fma: a few percent faster);
-# off by default: doubling the weights then no longer doubles the result bit for bit
-radial_fold = os.environ.get("KEOPS_AMD_RADIAL_FOLD", "0") == "1"
 radial_max_dim = 8                  # components of the points (7 D + 8 slots of the scalar product fit four instructions)
 radial_max_dv = 8                   # components of the weights (16 accumulators per component in every lane)
 # components of v up to which gradients with a factor <u_i, v_j> form it per pair in the matrix-core exponent kernels
@@ -66,8 +63,6 @@ radial_bilinear = os.environ.get("KEOPS_AMD_RADIAL_BILINEAR", "1") != "0"   # a 
 radial_bilinear_max_dw = int(os.environ.get("KEOPS_AMD_RADIAL_BILINEAR_MAX_DW", 8))
 radial_bilinear_max_nkb = int(os.environ.get("KEOPS_AMD_RADIAL_BILINEAR_MAX_NKB", 5))
 radial_mm_max_dv = 32               # ... when the weighted sum runs on the matrix cores (the three terms of the weights in up to three blocks of 32 operand columns)
-# the path is taken when |c| log2(e) (max |x^|^2 + max |y^|^2) <= this bound for the centred points (checked on the
-# device): the exponent is then off by at most 8 * 2^-24 of it, a kernel value by 7e-5 at worst and 1e-6 typically
 radial_rb2_max_dv = int(os.environ.get("KEOPS_AMD_RADIAL_RB2_MAX_DV", 4))  # two 32-row blocks per wavefront up to this many accumulated components
 # columns per staged tile (multiple of 32); auto: 128 up to two accumulated components per pair, 512 beyond (the
 # vector work of a sub-tile grows with the components while the cost of a tile change does not)
@@ -81,7 +76,16 @@ radial_mm_min_dv = int(os.environ.get("KEOPS_AMD_RADIAL_MM_MIN_DV", 7))
 radial_mm_terms = int(os.environ.get("KEOPS_AMD_RADIAL_MM_TERMS", 3))
 radial_mm_rb = int(os.environ.get("KEOPS_AMD_RADIAL_MM_RB", 1))   # 32-row blocks per wavefront in that variant
 radial_tile_j = os.environ.get("KEOPS_AMD_RADIAL_TJ", "auto")
-radial_limit = float(os.environ.get("KEOPS_AMD_RADIAL_LIMIT", 128.0))
+# Dense launches decide per tile: a wavefront takes the exponents of a 32-column sub-tile from the matrix cores when
+# |c| log2(e) (max |x^|^2 of its rows + max |y^|^2 of the sub-tile) <= this bound for the centred points (both clouds
+# are sorted by that quantity); an exponent is off by at most 8 * 2^-24 of it, a kernel value by 3.3e-7 * limit <= 1e-5.
+# The other sub-tiles are computed from exact differences in the same sweep.
+radial_limit = float(os.environ.get("KEOPS_AMD_RADIAL_LIMIT", 30.0))
+# ... unless more than this share of the pairs would be (estimated on the device from the sort's bucket counts): then
+# the general-purpose kernel computes the whole sum
+radial_exact_frac = float(os.environ.get("KEOPS_AMD_RADIAL_EXACT_FRAC", 0.25))
+# block-sparse launches: one centre and one check per row range, |c| log2(e) (R_x^2 + min(R_y, R_x + reach)^2) <= this
+radial_ranges_limit = float(os.environ.get("KEOPS_AMD_RADIAL_RANGES_LIMIT", 128.0))
 # calls below 2**28 pairs (16384 x 16384) stay on the general-purpose kernel: measured 0.061 vs 0.074 ms at 12000^2, equal at
 # 16000^2, 0.150 vs 0.126 ms at 23000^2 (the pre-pass of the matrix-core scheme is seven small launches)
 radial_ranges = os.environ.get("KEOPS_AMD_RADIAL_RANGES", "1") != "0"  # block-sparse launches too (one centre per row range)

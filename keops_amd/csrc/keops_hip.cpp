@@ -679,71 +679,99 @@ struct RadHeader {
   void* colsum;
   void* colpart;
   void* scal;
-  void* blk;
+  void* hist[2];
+  void* btot[2];
+  void* bkt[2];
+  void* perm[2];
+  void* qn[2];
+  void* gmax[2];
   void* out;
   void* partial;
-  int64_t slab_len;
-  int32_t nslabs, nparts;
+  void* xpart;
+  void* segmax;
+  int64_t slab_len, seg_len;
+  int32_t nslabs, nseg, nparts;
 };
 
-// Launches the pre-pass, the decision kernel and the matrix-core sweep of a module built with radial=1, all
-// asynchronous; *guard receives the device address of the flag that the general-purpose kernels, launched by the
-// caller right after, test before doing anything.  Workspace: the first `reserved` bytes of m.partial stay free for
-// the caller (slab partials of the general-purpose kernel).
+// Launches the pre-pass (centre, counting sort of both clouds by their centred norms, slot vectors in sorted order,
+// tile maxima), the decision kernel and the matrix-core sweep of a module built with radial=1, all asynchronous;
+// *guard receives the device address of the flag that the general-purpose kernels, launched by the caller right
+// after, test before doing anything.  Workspace: the first `reserved` bytes of m.partial stay free for the caller
+// (slab partials of the general-purpose kernel).
 int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, hipStream_t stream, size_t reserved,
                   const unsigned** guard) {
   const int64_t D = m.meta_int("rad_d", 0), DV = m.meta_int("rad_dv", 0), NKB = m.meta_int("rad_nkb", 0);
   const int64_t RB = m.meta_int("rad_rb", 0), WAVES = m.meta_int("rad_waves", 0), TJ = m.meta_int("rad_tj", 128);
+  const int64_t NBK = m.meta_int("rad_nbk", 128), CHUNK = m.meta_int("rad_sort_chunk", 1024);
   if (D <= 0 || DV <= 0 || NKB <= 0 || RB <= 0 || WAVES <= 0) return fail(-1, "corrupt radial module metadata");
-  const bool fold = m.meta_int("rad_fold", 0) != 0;  // weights folded into the exponents, columns partitioned by sign
-  // (the partition pads both groups of columns to whole tiles: one more tile)
-  const int64_t ntiles = (ny + TJ - 1) / TJ + (fold ? 1 : 0), rows_per_wg = 32 * RB * WAVES, row_blocks = (nx + rows_per_wg - 1) / rows_per_wg;
+  if (nx >= (int64_t)1 << 31 || ny >= ((int64_t)1 << 31) - TJ) return fail(-1, "radial scheme: more than 2^31 points");
+  const int64_t ntiles = (ny + TJ - 1) / TJ, rows_per_wg = 32 * RB * WAVES, row_blocks = (nx + rows_per_wg - 1) / rows_per_wg;
   // slabs over the reduced axis: about 16 workgroups per compute unit, whole tiles per slab
   int64_t nslabs = std::max<int64_t>(1, (16 * (int64_t)m.cu_count + row_blocks - 1) / row_blocks);
   nslabs = std::min<int64_t>(nslabs, std::max<int64_t>(1, ntiles / 8));
-  const int64_t ncols = fold ? ntiles * TJ : ny;
-  int64_t slab_len = ((ncols + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ;
-  nslabs = std::max<int64_t>(1, (ncols + slab_len - 1) / slab_len);
+  int64_t slab_len = ((ny + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ;
+  nslabs = std::max<int64_t>(1, (ny + slab_len - 1) / slab_len);
   const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(256, ny / 1024));
-  const int64_t nblk = (ny + 255) / 256;
+  const int64_t ncols = ntiles * TJ;  // columns of the padded tile grid
+  const int nblk_r = (int)((nx + CHUNK - 1) / CHUNK), nblk_c = (int)((ny + CHUNK - 1) / CHUNK);
   size_t off = align_up(reserved, 256);
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
   const size_t o_scal = take(32), o_colsum = take((size_t)D * 4), o_colpart = take((size_t)nparts * D * 4);
-  const size_t o_blk = take(fold ? (size_t)nblk * 4 : 0);
+  const size_t o_hist_r = take((size_t)NBK * nblk_r * 4), o_hist_c = take((size_t)NBK * nblk_c * 4);
+  const size_t o_btot_r = take((size_t)NBK * 4), o_btot_c = take((size_t)NBK * 4);
+  const size_t o_bkt_r = take((size_t)nx), o_bkt_c = take((size_t)ny);
+  const size_t o_perm_r = take((size_t)nx * 4), o_perm_c = take((size_t)ncols * 4);
+  const size_t o_qn_r = take((size_t)nx * 4), o_qn_c = take((size_t)ncols * 4);
+  const int64_t groups_r = (nx + 32 * RB - 1) / (32 * RB);
+  const size_t o_gmax_r = take((size_t)groups_r * 4), o_gmax_c = take((size_t)ntiles * 4);
   // weights of a column: RAD_DV floats, or 32 bfloat16 operand columns when the weighted sum runs on the matrix cores
   // (three terms of every weight: one block of 32 columns up to ten weights, rad_mm_nb blocks beyond)
   const size_t wbytes = m.meta_int("rad_mm", 0) != 0 ? 64 * (size_t)std::max<int64_t>(1, m.meta_int("rad_mm_nb", 1))
                                                       : (size_t)std::max<int64_t>(DV, m.meta_int("rad_ws", 0)) * 4;
-  const size_t o_xa = take((size_t)nx * NKB * 32), o_yb = take((size_t)ntiles * TJ * NKB * 32), o_bw = take((size_t)ntiles * TJ * wbytes);
+  const size_t o_xa = take((size_t)nx * NKB * 32), o_yb = take((size_t)ncols * NKB * 32), o_bw = take((size_t)ncols * wbytes);
   const size_t o_part = take((size_t)nslabs * nx * DV * 4);
+  // column segments of the kernel that computes the left-out tiles from exact differences: finer than the slabs (its
+  // work sits in a corner of the pair matrix), at most 16 and at most 256 MiB of sums
+  int64_t nseg = std::max<int64_t>(1, std::min<int64_t>(16, ((int64_t)256 << 20) / std::max<int64_t>(1, nx * DV * 4)));
+  nseg = std::min<int64_t>(nseg, ntiles);
+  const int64_t seg_len = ((ny + nseg - 1) / nseg + TJ - 1) / TJ * TJ;
+  nseg = std::max<int64_t>(1, (ny + seg_len - 1) / seg_len);
+  const size_t o_xpart = take((size_t)nseg * nx * DV * 4), o_segmax = take((size_t)nseg * 4);
   if (int rc = m.partial.reserve(off)) return rc;
   char* ws = (char*)m.partial.ptr;
   std::vector<char> buf(sizeof(RadHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 16);
   RadHeader h{};
   h.nx = nx; h.ny = ny; h.xa = ws + o_xa; h.yb = ws + o_yb; h.bw = ws + o_bw; h.colsum = ws + o_colsum; h.colpart = ws + o_colpart;
-  h.scal = ws + o_scal; h.blk = ws + o_blk; h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs; h.nparts = nparts;
+  h.scal = ws + o_scal;
+  h.hist[0] = ws + o_hist_r; h.hist[1] = ws + o_hist_c; h.btot[0] = ws + o_btot_r; h.btot[1] = ws + o_btot_c; h.bkt[0] = ws + o_bkt_r; h.bkt[1] = ws + o_bkt_c;
+  h.perm[0] = ws + o_perm_r; h.perm[1] = ws + o_perm_c; h.qn[0] = ws + o_qn_r; h.qn[1] = ws + o_qn_c;
+  h.gmax[0] = ws + o_gmax_r; h.gmax[1] = ws + o_gmax_c;
+  h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs; h.nparts = nparts;
+  h.xpart = ws + o_xpart; h.segmax = ws + o_segmax; h.seg_len = seg_len; h.nseg = (int32_t)nseg;
   std::memcpy(buf.data(), &h, sizeof(h));
   for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
   const size_t psize = sizeof(RadHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs);
   auto with_which = [&](int w) { std::memcpy(buf.data() + psize, &w, 4); return psize + 4; };
+  auto with_nblk = [&]() { std::memcpy(buf.data() + psize, &nblk_r, 4); std::memcpy(buf.data() + psize + 4, &nblk_c, 4); return psize + 8; };
   if (int rc = launch_raw(m, "keops_rad_colsum", (unsigned)nparts, 1, 256, buf.data(), psize, stream)) return rc;
   if (int rc = launch_raw(m, "keops_rad_colsum_final", 1, 1, 64, buf.data(), psize, stream)) return rc;
-  if (fold) {
-    if (int rc = launch_raw(m, "keops_rad_sign_count", (unsigned)nblk, 1, 256, buf.data(), psize, stream)) return rc;
-    int nb32 = (int)nblk;
-    std::memcpy(buf.data() + psize, &nb32, 4);
-    if (int rc = launch_raw(m, "keops_rad_sign_scan", 1, 1, 1024, buf.data(), psize + 4, stream)) return rc;
-    const int64_t nc = ntiles * TJ;
-    std::memcpy(buf.data() + psize, &nc, 8);
-    if (int rc = launch_raw(m, "keops_rad_fill_dead", (unsigned)((nc + 255) / 256), 1, 256, buf.data(), psize + 8, stream)) return rc;
-  }
   size_t sz = with_which(0);
-  if (int rc = launch_raw(m, "keops_rad_prep", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_bucket", (unsigned)nblk_r, 1, 256, buf.data(), sz, stream)) return rc;
   sz = with_which(1);
-  if (int rc = launch_raw(m, "keops_rad_prep", (unsigned)(fold ? nblk : (ntiles * TJ + 255) / 256), 1, 256, buf.data(), sz, stream)) return rc;
-  if (int rc = launch_raw(m, "keops_rad_decide", 1, 1, 64, buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_bucket", (unsigned)nblk_c, 1, 256, buf.data(), sz, stream)) return rc;
+  sz = with_nblk();
+  if (int rc = launch_raw(m, "keops_rad_scan", (unsigned)NBK, 2, 256, buf.data(), sz, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_decide", 1, 1, (unsigned)NBK, buf.data(), psize, stream)) return rc;
+  sz = with_which(0);
+  if (int rc = launch_raw(m, "keops_rad_prep", (unsigned)nblk_r, 1, 256, buf.data(), sz, stream)) return rc;
+  sz = with_which(1);
+  if (int rc = launch_raw(m, "keops_rad_prep", (unsigned)((ncols + CHUNK - 1) / CHUNK), 1, 256, buf.data(), sz, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_groupmax", (unsigned)((groups_r + ntiles + 3) / 4), 1, 256, buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_segmax", (unsigned)nseg, 1, 64, buf.data(), psize, stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
   if (int rc = launch_raw(m, "keops_rad_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)(64 * WAVES), buf.data(), psize, stream)) return rc;
+  const int64_t xrows = m.meta_int("rad_exact_rows", 64);
+  if (int rc = launch_raw(m, "keops_rad_exact", (unsigned)((nx + xrows - 1) / xrows), (unsigned)nseg, 256, buf.data(), psize, stream)) return rc;
   if (int rc = launch_raw(m, "keops_rad_reduce", (unsigned)((nx + 255) / 256), 1, 256, buf.data(), psize, stream)) return rc;
   *guard = (const unsigned*)(ws + o_scal) + 2;
   return 0;

@@ -23,10 +23,18 @@
 // each instruction's result to float32; measured on a million pairs: |dt| <= 8 * 2^-24 |k| (|x^|^2 + |y^|^2), no
 // bias).  Dropped: (l,m), (l,l), below 2^-24 |u||y|.  The error of a kernel value is therefore at most
 // ln(2) |dt| <= 3.3e-7 |k| (|x^|^2 + |y^|^2), typically a third of it: the float32 class of the reference's own
-// exponent as long as the kernel is not much narrower than the cloud.  keops_rad_decide checks exactly that on the
-// device, |k| (max |x^|^2 + max |y^|^2) <= RAD_LIMIT, and sets a flag: when it does not hold, the kernels of this
+// exponent wherever |k| (|x^|^2 + |y^|^2) is moderate, which the kernels check PER TILE: both clouds are sorted by
+// that quantity (a stable counting sort on RAD_NBK buckets, so that the points of a tile have similar norms and the
+// summation order is reproducible), and a wavefront takes the exponents of a 32-column sub-tile from the matrix cores
+// only when  max over its rows + max over the sub-tile's columns <= RAD_LIMIT  (a-priori error of a kernel value
+// 3.3e-7 * RAD_LIMIT).  The other sub-tiles -- the shell of the cloud against itself, an outlier against everything --
+// are left out by the sweep and computed by keops_rad_exact, launched behind it, from exact float32 differences in the
+// reference's own operation order (difference, square, sum without contraction, one rounded product with the
+// coefficient, then an exponential good to 2 ulp); it adds its sums to the sweep's.
+// keops_rad_decide estimates the share of such pairs from the bucket counts and sets a flag: when more than
+// RAD_EXACT_FRAC of the pairs would take the slow path (a kernel much narrower than the cloud), the kernels of this
 // file return at once and the general-purpose kernel of the same module, which is launched behind them and returns
-// at once in the other case, computes the sum from exact float32 differences.  No host synchronisation.
+// at once in the other case, computes the whole sum from exact differences.  No host synchronisation.
 //
 // Work decomposition: lane l of a wavefront owns column j = l % 32 of the staged sub-tile (its slot vector is the B
 // operand, its weights B_j sit in registers) and, after the instruction, the 16 exponents of rows
@@ -36,22 +44,12 @@
 // The lanes of a row are summed with shuffles once at the end; slabs over the reduced axis (blockIdx.y) are added
 // in order by keops_rad_reduce: deterministic.
 //
-// RAD_FOLD (a scalar weight w_j and no difference factor: the plain Gaussian kernel sum): exp2(t) w_j =
-// +- exp2(t + log2 |w_j|), so log2 |w_j| joins the column's squared-norm term (formed in double precision) and the
-// columns are partitioned by the sign of their weight (stable, deterministic: keops_rad_sign_count / _scan, then
-// keops_rad_prep scatters every column to its place; unused places hold "dead" columns whose exponent is -16384).
-// Tiles of non-negative weights are accumulated with one v_add_f32 per pair, the others with one v_sub_f32: half
-// the cost of the fused multiply-add (v_exp_f32 takes 8 issue cycles per wavefront, v_fmac_f32 4, v_add_f32 2).
-// The sweep alternates between the two groups tile by tile (rad_tile_of), so that the running sums stay as small
-// as with the weights in their original order: summing one sign after the other would carry rounding errors
-// relative to sum_j K_ij |w_j| into a result that may be much smaller.
-//
 // The plug-in defines RAD_D, RAD_DV, RAD_NKB (16-slot blocks), RAD_RB, RAD_WAVES, RAD_XARG, RAD_YARG, RAD_LIMIT,
 // the slot tables rad_slot_kind / rad_slot_comp / rad_slot_term for both sides, the tables of the variables of B
 // (rad_col_arg / rad_col_dim / rad_col_off, RAD_NCOLVARS, RAD_DIMY) and of the parameters (keops_par_*), and
 // the tables of the variables of A (rad_row_*, RAD_NROWVARS, RAD_DIMX), RAD_DW (components of W), RAD_DU (components of
 // a row vector u_i that multiplies W as <u_i, W_j>: KeopsRadFormula::rowvec), RAD_DOUT, RAD_DIFF,
-// RAD_SIGN and struct KeopsRadFormula { kappa(p); weights(yj, p, w); rowscale(xi, p) }.
+// RAD_SIGN and struct KeopsRadFormula { coef(p); kappa(p); weights(yj, p, w); rowscale(xi, p) }.
 #pragma once
 
 typedef __bf16 rad_bf16x8 __attribute__((ext_vector_type(8)));
@@ -91,20 +89,40 @@ typedef __bf16 rad_bf16x2 __attribute__((ext_vector_type(2)));
 #define RAD_BLOCK (64 * RAD_WAVES)
 #define RAD_ROWS_PER_BLOCK (32 * RAD_RB * RAD_WAVES)
 
+#ifndef RAD_RANGES
+#define RAD_RANGES 0
+#endif
+// Per-tile choice between matrix-core exponents and exact differences (dense launches; the block-sparse variant has
+// one centre per row range and decides per range).
+#define RAD_TILEWISE (!RAD_RANGES)
+#define RAD_NBK 128                // buckets of the counting sort by |k| |x^|^2: [0, RAD_LIMIT) in equal parts, the last one open
+#define RAD_SORT_CHUNK 1024        // points per workgroup of the sort (4 rounds of 256)
+#ifndef RAD_EXACT_FRAC
+#define RAD_EXACT_FRAC 0.25f       // largest estimated share of pairs from exact differences for which this family still runs
+#endif
+
 struct RadParams {
   i64 nx, ny;
-  __bf16* xa;         // [nx][RAD_SLOTS] row-side slot vectors
-  __bf16* yb;         // [tile][RAD_NKB][2][RAD_TJ][8] column-side slot vectors, tile by tile
+  __bf16* xa;         // [nx][RAD_SLOTS] row-side slot vectors, rows in sorted order
+  __bf16* yb;         // [tile][RAD_NKB][2][RAD_TJ][8] column-side slot vectors, tile by tile, columns in sorted order
   float* bw;          // [ntiles * RAD_TJ][RAD_DV] weights B_j (zero past the last column)
   float* colsum;      // [RAD_D] column sums of y
   float* colpart;     // [nparts][RAD_D]
-  unsigned* scal;     // [0], [1]: bit patterns of max |x^|^2, max |y^|^2; [2]: 1 when the matrix-core path is taken;
-                      // [3] (RAD_FOLD): number of tiles of columns with non-negative weights
-  int* blk;           // RAD_FOLD: [nblk] non-negative weights per block of 256 columns, then their exclusive scan
-  T* out;             // [nx][RAD_DV]
-  float* partial;     // [nslabs][nx][RAD_DV]
+  unsigned* scal;     // [0], [1]: bit patterns of max |x^|^2, max |y^|^2; [2]: 1 when the matrix-core path is taken
+  int* hist[2];       // rows, columns: [RAD_NBK][nblk] points per bucket and sort chunk, then their exclusive scan per bucket
+  int* btot[2];       // [RAD_NBK] points per bucket, then (keops_rad_decide) their exclusive scan: first sorted position of a bucket
+  unsigned char* bkt[2];  // [n] bucket of every point
+  int* perm[2];       // [n (columns: padded to whole tiles)] sorted position -> point (-1: padding)
+  float* qn[2];       // ... and |k| |x^|^2 of that point, rounded up
+  float* gmax[2];     // largest qn of every group of sorted points: rows by 32 * RAD_RB (a wavefront's rows), columns by RAD_TJ (a tile)
+  T* out;             // [nx][RAD_DOUT]
+  float* partial;     // [nslabs][nx][RAD_DV], rows in sorted order
+  float* xpart;       // [nseg][nx][RAD_DV] sums of keops_rad_exact (only the rows that meet a tile beyond the bound are written)
+  float* segmax;      // [nseg] largest qn of the columns of every segment
   i64 slab_len;       // reduced rows per slab (multiple of RAD_TJ)
+  i64 seg_len;        // reduced rows per segment of keops_rad_exact (multiple of RAD_TJ)
   int nslabs;
+  int nseg;
   int nparts;
   const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
 };
@@ -119,10 +137,6 @@ __device__ __forceinline__ void rad_load_params(const RadParams& P, T (&p)[KEOPS
 }
 
 // ---- pre-pass ---------------------------------------------------------------------------------------------------
-
-#ifndef RAD_RANGES
-#define RAD_RANGES 0
-#endif
 
 #if !RAD_RANGES
 // column sums of y in two deterministic stages (fixed order, no atomics)
@@ -156,85 +170,88 @@ extern "C" __global__ void __launch_bounds__(64) keops_rad_colsum_final(const Ra
   if (c < 4) P.scal[c] = 0u;
 }
 
-#endif  // !RAD_RANGES
-
-#ifndef RAD_FOLD
-#define RAD_FOLD 0
-#endif
-
-__device__ __forceinline__ float rad_column_weight(const RadParams& P, i64 j, const T (&p)[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1]) {
-  T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
+// |k| |x^|^2 of a point (x^: the point minus the mean of y, in double precision) and its bucket
+__device__ __forceinline__ double rad_centred_norm(const RadParams& P, const T* src) {
+  double nrm = 0.0;
 #pragma unroll
-  for (int v = 0; v < RAD_NCOLVARS; v++) {
-    const T* a = P.arg[rad_col_arg[v]] + j * rad_col_dim[v];
-#pragma unroll
-    for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
+  for (int k = 0; k < RAD_D; k++) {
+    const double c = (double)src[k] - (double)P.colsum[k];
+    nrm += c * c;
   }
-  T wv[RAD_DW];
-  KeopsRadFormula::weights(yj, p, wv);
-  return (float)wv[0];
+  return nrm;
+}
+__device__ __forceinline__ int rad_bucket_of(double q) {
+  // NaN and everything from RAD_LIMIT on: the last bucket
+  return q < (double)RAD_LIMIT ? (int)(q * ((double)(RAD_NBK - 1) / (double)RAD_LIMIT)) : RAD_NBK - 1;
 }
 
-#if RAD_FOLD
-// columns with a non-negative weight, per block of 256 columns (a NaN weight counts as non-negative)
-extern "C" __global__ void __launch_bounds__(256) keops_rad_sign_count(const RadParams P) {
-  __shared__ int cnt[4];
-  const i64 j = (i64)blockIdx.x * 256 + threadIdx.x;
+// Counting sort by |k| |x^|^2, pass 1: bucket of every point and points per (bucket, chunk of RAD_SORT_CHUNK points).
+// which = 0: rows (x), 1: columns (y).
+extern "C" __global__ void __launch_bounds__(256) keops_rad_bucket(const RadParams P, int which) {
+  __shared__ int h[RAD_NBK];
+  const i64 n = which ? P.ny : P.nx;
+  for (int b = threadIdx.x; b < RAD_NBK; b += 256) h[b] = 0;
+  __syncthreads();
   T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
   rad_load_params(P, p);
-  const bool pos = j < P.ny && !(rad_column_weight(P, j, p) < 0.f);
-  const unsigned long long bal = __ballot(pos);
-  if ((threadIdx.x & 63) == 0) cnt[threadIdx.x >> 6] = __popcll(bal);
+  const double ak = __builtin_fabs((double)KeopsRadFormula::kappa(p));
+  const T* base = P.arg[which ? RAD_YARG : RAD_XARG];
+  float nmax = 0.f;
+#pragma unroll
+  for (int r = 0; r < RAD_SORT_CHUNK / 256; r++) {
+    const i64 i = (i64)blockIdx.x * RAD_SORT_CHUNK + r * 256 + threadIdx.x;
+    if (i < n) {
+      const double nrm = rad_centred_norm(P, base + i * RAD_D);
+      const int b = rad_bucket_of(ak * nrm);
+      P.bkt[which][i] = (unsigned char)b;
+      atomicAdd(&h[b], 1);
+      const float nf = (float)nrm * 1.000001f;
+      nmax = nf > nmax ? nf : nmax;
+    }
+  }
+  // largest centred squared norm (bit pattern of a non-negative float, rounded up): order-independent maximum, one
+  // atomic per wavefront
+  {
+    unsigned bits = __float_as_uint(nmax);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const unsigned other = (unsigned)__shfl_xor((int)bits, o);
+      bits = other > bits ? other : bits;
+    }
+    if ((threadIdx.x & 63) == 0) atomicMax(P.scal + which, bits);
+  }
   __syncthreads();
-  if (threadIdx.x == 0) P.blk[blockIdx.x] = cnt[0] + cnt[1] + cnt[2] + cnt[3];
+  for (int b = threadIdx.x; b < RAD_NBK; b += 256) P.hist[which][(i64)b * gridDim.x + blockIdx.x] = h[b];
 }
 
-// exclusive scan of the block counts (one workgroup, sequential over chunks of 1024 blocks); scal[3] = tiles of
-// non-negative columns
-extern "C" __global__ void __launch_bounds__(1024) keops_rad_sign_scan(const RadParams P, int nblk) {
-  __shared__ int part[1024];
-  __shared__ int carry;
-  if (threadIdx.x == 0) carry = 0;
+// pass 2: exclusive scan of the counts of every bucket over the chunks (one workgroup per bucket and cloud, the
+// counts of a bucket are contiguous) and the points per bucket.  The first sorted position of (bucket, chunk) is the
+// scan of the bucket totals, done by keops_rad_decide, plus this.
+extern "C" __global__ void __launch_bounds__(256) keops_rad_scan(const RadParams P, int nblk_r, int nblk_c) {
+  __shared__ int part[256];
+  const int which = blockIdx.y, b = blockIdx.x, t = threadIdx.x;
+  const int nblk = which ? nblk_c : nblk_r;
+  int* h = P.hist[which] + (i64)b * nblk;
+  const int per = (nblk + 255) / 256, lo = keops_min(nblk, t * per), hi = keops_min(nblk, lo + per);
+  int s = 0;
+  for (int k = lo; k < hi; k++) s += h[k];
+  part[t] = s;
   __syncthreads();
-  for (int base = 0; base < nblk; base += 1024) {
-    const int b = base + threadIdx.x;
-    const int v = b < nblk ? P.blk[b] : 0;
-    part[threadIdx.x] = v;
+  for (int o = 1; o < 256; o <<= 1) {
+    const int v = t >= o ? part[t - o] : 0;
     __syncthreads();
-    for (int o = 1; o < 1024; o <<= 1) {  // inclusive scan in shared memory
-      const int t = (int)threadIdx.x >= o ? part[threadIdx.x - o] : 0;
-      __syncthreads();
-      part[threadIdx.x] += t;
-      __syncthreads();
-    }
-    if (b < nblk) P.blk[b] = carry + part[threadIdx.x] - v;
-    __syncthreads();
-    if (threadIdx.x == 1023) carry += part[1023];
+    part[t] += v;
     __syncthreads();
   }
-  if (threadIdx.x == 0) P.scal[3] = (unsigned)((carry + RAD_TJ - 1) / RAD_TJ);
+  int run = part[t] - s;
+  for (int k = lo; k < hi; k++) {
+    const int c = h[k];
+    h[k] = run;
+    run += c;
+  }
+  if (t == 255) P.btot[which][b] = part[255];
 }
-
-// every place of the column operand starts as a dead column: exponent -16384 for every row
-extern "C" __global__ void __launch_bounds__(256) keops_rad_fill_dead(const RadParams P, i64 ncols) {
-  const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
-  if (i >= ncols) return;
-  const i64 tile = i / RAD_TJ;
-  const int c = (int)(i % RAD_TJ);
-#pragma unroll
-  for (int kb = 0; kb < RAD_NKB; kb++)
-#pragma unroll
-    for (int hf = 0; hf < 2; hf++) {
-      rad_bf16x8 v8;
-#pragma unroll
-      for (int e = 0; e < 8; e++) {
-        const int s = kb * 16 + hf * 8 + e;
-        v8[e] = (rad_col_kind[s] == 3 && rad_col_term[s] == 0) ? (__bf16)(-16384.0f) : (__bf16)0.0f;
-      }
-      *reinterpret_cast<rad_bf16x8*>(P.yb + (((tile * RAD_NKB + kb) * 2 + hf) * RAD_TJ + c) * 8) = v8;
-    }
-}
-#endif
+#endif  // !RAD_RANGES
 
 __device__ __forceinline__ void rad_split3(float v, __bf16 (&t)[3]) {
   t[0] = (__bf16)v;
@@ -276,51 +293,102 @@ __device__ __forceinline__ void rad_store_weights_mm(__bf16* bwm, i64 j, const f
 #endif
 
 #if !RAD_RANGES
-// Slot vector of one point.  which = 0: rows (x), 1: columns (y; one thread per column of the padded tile grid).
+// pass 3: slot vector of every point, written at its sorted position.  which = 0: rows (x), 1: columns (y; the
+// places past the last column of the padded tile grid receive zero vectors and zero weights).  Stable: the points of
+// a bucket keep their order (chunks in order, rounds in order, wavefronts in order, lanes in order).
 extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams P, int which) {
-  const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+  __shared__ int cnt[RAD_NBK];
   const i64 n = which ? P.ny : P.nx;
-#if RAD_FOLD
-  const i64 ntot = which ? (P.ny + 255) / 256 * 256 : P.nx;  // whole blocks: every lane takes part in the ranking
-#else
   const i64 ntot = which ? (P.ny + RAD_TJ - 1) / RAD_TJ * RAD_TJ : P.nx;
-#endif
-  if (i >= ntot) return;
+  const int nblk = (int)((n + RAD_SORT_CHUNK - 1) / RAD_SORT_CHUNK);  // chunks that hold points (the grid may be longer)
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int b = threadIdx.x; b < RAD_NBK; b += 256) cnt[b] = 0;
+  __syncthreads();
   T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
   rad_load_params(P, p);
   const double kappa = (double)KeopsRadFormula::kappa(p);
-  __bf16 slot[RAD_SLOTS];
-  float w[RAD_WS];
+  for (int r = 0; r < RAD_SORT_CHUNK / 256; r++) {
+    const i64 i = (i64)blockIdx.x * RAD_SORT_CHUNK + r * 256 + threadIdx.x;
+    const bool real = i < n;
+    // rank of the point among the points of its bucket in this chunk
+    const int b = real ? (int)P.bkt[which][i] : 0;
+    unsigned long long same = __ballot(real);
 #pragma unroll
-  for (int d = 0; d < RAD_WS; d++) w[d] = 0.f;
-  if (i < n) {
-    const T* src = P.arg[which ? RAD_YARG : RAD_XARG] + i * RAD_D;
-    __bf16 ct[RAD_D][3], nt[4];
-    float cf[RAD_D];
-    double nrm = 0.0;
+    for (int bit = 0; bit < 7; bit++) {
+      const bool set = (b >> bit) & 1;
+      const unsigned long long bal = __ballot(set);
+      same &= set ? bal : ~bal;
+    }
+    int rank = 0;
+    for (int w = 0; w < 4; w++) {
+      if (wave == w && real) {
+        const int before = cnt[b];
+        rank = before + __popcll(same & ((1ull << lane) - 1ull));
+        if ((same >> lane) == 1ull) cnt[b] = before + __popcll(same);  // the highest lane of the group
+      }
+      __syncthreads();
+    }
+    if (i >= ntot) continue;
+    const i64 pos = real ? (i64)P.btot[which][b] + P.hist[which][(i64)b * nblk + blockIdx.x] + rank : i;
+
+    __bf16 slot[RAD_SLOTS];
+    float w[RAD_WS];
 #pragma unroll
-    for (int k = 0; k < RAD_D; k++) {
-      const double c = (double)src[k] - (double)P.colsum[k];
-      cf[k] = (float)c;
-      nrm += c * c;
-      rad_split3((float)(which ? c : -2.0 * kappa * c), ct[k]);
-    }
-#if RAD_FOLD
-    // the weight joins the exponent: exp2(t) w = +- exp2(t + log2 |w|)
-    float wfold = 1.f;
-    if (which) {
-      wfold = rad_column_weight(P, i, p);
-      w[0] = wfold;
-    }
-    rad_split4(which ? kappa * nrm + (double)__ocml_log2_f64((double)__builtin_fabsf(wfold)) : kappa * nrm, nt);
-#else
-    rad_split4(kappa * nrm, nt);
-#endif
+    for (int d = 0; d < RAD_WS; d++) w[d] = 0.f;
+    float q = 0.f;
+    if (real) {
+      const T* src = P.arg[which ? RAD_YARG : RAD_XARG] + i * RAD_D;
+      __bf16 ct[RAD_D][3], nt[4];
+      float cf[RAD_D];
+      double nrm = 0.0;
+#pragma unroll
+      for (int k = 0; k < RAD_D; k++) {
+        const double c = (double)src[k] - (double)P.colsum[k];
+        cf[k] = (float)c;
+        nrm += c * c;
+        rad_split3((float)(which ? c : -2.0 * kappa * c), ct[k]);
+      }
+      rad_split4(kappa * nrm, nt);
+      q = (float)(__builtin_fabs(kappa) * nrm) * 1.000001f;
 #if RAD_BIL
-    // three bfloat16 terms of every component of u_i (rows) or v_j (columns)
-    __bf16 bt[RAD_DW][3];
-    {
-      T vals[RAD_DW];
+      // three bfloat16 terms of every component of u_i (rows) or v_j (columns)
+      __bf16 bt[RAD_DW][3];
+      {
+        T vals[RAD_DW];
+        if (which) {
+          T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
+#pragma unroll
+          for (int v = 0; v < RAD_NCOLVARS; v++) {
+            const T* a = P.arg[rad_col_arg[v]] + i * rad_col_dim[v];
+#pragma unroll
+            for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
+          }
+          KeopsRadFormula::weights(yj, p, vals);
+        } else {
+          T xi[RAD_DIMX > 0 ? RAD_DIMX : 1];
+#pragma unroll
+          for (int v = 0; v < RAD_NROWVARS; v++) {
+            const T* a = P.arg[rad_row_arg[v]] + i * rad_row_dim[v];
+#pragma unroll
+            for (int d = 0; d < rad_row_dim[v]; d++) xi[rad_row_off[v] + d] = a[d];
+          }
+          KeopsRadFormula::rowvec(xi, p, vals);
+        }
+#pragma unroll
+        for (int d = 0; d < RAD_DW; d++) rad_split3((float)vals[d], bt[d]);
+      }
+#endif
+#pragma unroll
+      for (int s = 0; s < RAD_SLOTS; s++) {
+        const int kind = which ? rad_col_kind[s] : rad_row_kind[s];
+        const int comp = which ? rad_col_comp[s] : rad_row_comp[s];
+        const int term = which ? rad_col_term[s] : rad_row_term[s];
+#if RAD_BIL
+        slot[s] = kind == 0 ? (__bf16)0.0f : (kind == 1 ? (__bf16)1.0f : (kind == 2 ? ct[comp][term] : (kind == 3 ? nt[term] : bt[comp][term])));
+#else
+        slot[s] = kind == 0 ? (__bf16)0.0f : (kind == 1 ? (__bf16)1.0f : (kind == 2 ? ct[comp][term] : nt[term]));
+#endif
+      }
       if (which) {
         T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
 #pragma unroll
@@ -329,147 +397,144 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
 #pragma unroll
           for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
         }
-        KeopsRadFormula::weights(yj, p, vals);
-      } else {
-        T xi[RAD_DIMX > 0 ? RAD_DIMX : 1];
-#pragma unroll
-        for (int v = 0; v < RAD_NROWVARS; v++) {
-          const T* a = P.arg[rad_row_arg[v]] + i * rad_row_dim[v];
-#pragma unroll
-          for (int d = 0; d < rad_row_dim[v]; d++) xi[rad_row_off[v] + d] = a[d];
-        }
-        KeopsRadFormula::rowvec(xi, p, vals);
-      }
-#pragma unroll
-      for (int d = 0; d < RAD_DW; d++) rad_split3((float)vals[d], bt[d]);
-    }
-#endif
-    // largest centred squared norm (bit pattern of a non-negative float, rounded up): order-independent maximum
-    atomicMax(P.scal + which, __float_as_uint((float)nrm * 1.000001f));
-#pragma unroll
-    for (int s = 0; s < RAD_SLOTS; s++) {
-      const int kind = which ? rad_col_kind[s] : rad_row_kind[s];
-      const int comp = which ? rad_col_comp[s] : rad_row_comp[s];
-      const int term = which ? rad_col_term[s] : rad_row_term[s];
+        T wv[RAD_DW];
+        KeopsRadFormula::weights(yj, p, wv);
 #if RAD_BIL
-      slot[s] = kind == 0 ? (__bf16)0.0f : (kind == 1 ? (__bf16)1.0f : (kind == 2 ? ct[comp][term] : (kind == 3 ? nt[term] : bt[comp][term])));
-#else
-      slot[s] = kind == 0 ? (__bf16)0.0f : (kind == 1 ? (__bf16)1.0f : (kind == 2 ? ct[comp][term] : nt[term]));
-#endif
-    }
-    if (which && !RAD_FOLD) {
-      T yj[RAD_DIMY > 0 ? RAD_DIMY : 1];
-#pragma unroll
-      for (int v = 0; v < RAD_NCOLVARS; v++) {
-        const T* a = P.arg[rad_col_arg[v]] + i * rad_col_dim[v];
-#pragma unroll
-        for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
-      }
-      T wv[RAD_DW];
-      KeopsRadFormula::weights(yj, p, wv);
-#if RAD_BIL
-      // the weights sit in the slot vectors: what is left per column is [y^_j, 1], or 1
-      (void)wv;
+        // the weights sit in the slot vectors: what is left per column is [y^_j, 1], or 1
+        (void)wv;
 #if RAD_DIFF != 0
 #pragma unroll
-      for (int k = 0; k < RAD_D; k++) w[k] = cf[k];
-      w[RAD_D] = 1.f;
+        for (int k = 0; k < RAD_D; k++) w[k] = cf[k];
+        w[RAD_D] = 1.f;
 #else
-      w[0] = 1.f;
+        w[0] = 1.f;
 #endif
 #elif RAD_UPAIR
-      // the weights as they are, then [y^_j, 1]: the sweep forms <u_i, v_j> itself
+        // the weights as they are, then [y^_j, 1]: the sweep forms <u_i, v_j> itself
 #pragma unroll
-      for (int d = 0; d < RAD_DW; d++) w[d] = (float)wv[d];
+        for (int d = 0; d < RAD_DW; d++) w[d] = (float)wv[d];
 #pragma unroll
-      for (int k = 0; k < RAD_D; k++) w[RAD_DW + k] = cf[k];
-      w[RAD_DW + RAD_D] = 1.f;
+        for (int k = 0; k < RAD_D; k++) w[RAD_DW + k] = cf[k];
+        w[RAD_DW + RAD_D] = 1.f;
 #elif RAD_DIFF != 0
-      // component d of the weights against [y^_j, 1]
+        // component d of the weights against [y^_j, 1]
 #pragma unroll
-      for (int d = 0; d < RAD_DW; d++) {
+        for (int d = 0; d < RAD_DW; d++) {
 #pragma unroll
-        for (int k = 0; k < RAD_D; k++) w[d * (RAD_D + 1) + k] = (float)wv[d] * cf[k];
-        w[d * (RAD_D + 1) + RAD_D] = (float)wv[d];
+          for (int k = 0; k < RAD_D; k++) w[d * (RAD_D + 1) + k] = (float)wv[d] * cf[k];
+          w[d * (RAD_D + 1) + RAD_D] = (float)wv[d];
+        }
+#else
+#pragma unroll
+        for (int d = 0; d < RAD_DV; d++) w[d] = (float)wv[d];
+#endif
       }
-#else
+    } else {
 #pragma unroll
-      for (int d = 0; d < RAD_DV; d++) w[d] = (float)wv[d];
-#endif
+      for (int s = 0; s < RAD_SLOTS; s++) slot[s] = (__bf16)0.0f;
     }
-  } else {
+    P.perm[which][pos] = real ? (int)i : -1;
+    P.qn[which][pos] = q;
+    if (!which) {
 #pragma unroll
-    for (int s = 0; s < RAD_SLOTS; s++) slot[s] = (__bf16)0.0f;
-  }
-  if (!which) {
-#pragma unroll
-    for (int c8 = 0; c8 < RAD_SLOTS / 8; c8++) {
-      rad_bf16x8 v8;
-#pragma unroll
-      for (int e = 0; e < 8; e++) v8[e] = slot[c8 * 8 + e];
-      *reinterpret_cast<rad_bf16x8*>(P.xa + i * RAD_SLOTS + c8 * 8) = v8;
-    }
-  } else {
-#if RAD_FOLD
-    // stable partition by the sign of the weight: rank of this column among the non-negative (or negative) ones
-    __shared__ int wcnt[4];
-    const bool real = i < n, posw = real && !(w[0] < 0.f);
-    const unsigned long long bal = __ballot(posw);
-    const int lane = threadIdx.x & 63, wv_ = threadIdx.x >> 6;
-    if (lane == 0) wcnt[wv_] = __popcll(bal);
-    __syncthreads();
-    int before = __popcll(bal & ((1ull << lane) - 1ull));
-    for (int k = 0; k < wv_; k++) before += wcnt[k];
-    const i64 npos_before = (i64)P.blk[blockIdx.x] + before;
-    if (!real || w[0] == 0.f) return;  // zero weights: the place stays dead
-    const i64 dst = posw ? npos_before : (i64)P.scal[3] * RAD_TJ + (i - npos_before);
-    const i64 tile = dst / RAD_TJ;
-    const int c = (int)(dst % RAD_TJ);
-#else
-    const i64 tile = i / RAD_TJ;
-    const int c = (int)(i % RAD_TJ);
-#endif
-#pragma unroll
-    for (int kb = 0; kb < RAD_NKB; kb++)
-#pragma unroll
-      for (int hf = 0; hf < 2; hf++) {
+      for (int c8 = 0; c8 < RAD_SLOTS / 8; c8++) {
         rad_bf16x8 v8;
 #pragma unroll
-        for (int e = 0; e < 8; e++) v8[e] = slot[kb * 16 + hf * 8 + e];
-        *reinterpret_cast<rad_bf16x8*>(P.yb + (((tile * RAD_NKB + kb) * 2 + hf) * RAD_TJ + c) * 8) = v8;
+        for (int e = 0; e < 8; e++) v8[e] = slot[c8 * 8 + e];
+        *reinterpret_cast<rad_bf16x8*>(P.xa + pos * RAD_SLOTS + c8 * 8) = v8;
       }
-#if RAD_MM
-    rad_store_weights_mm(reinterpret_cast<__bf16*>(P.bw), i, w);
-#elif !RAD_FOLD
+    } else {
+      const i64 tile = pos / RAD_TJ;
+      const int c = (int)(pos % RAD_TJ);
 #pragma unroll
-    for (int d = 0; d < RAD_WS; d++) P.bw[i * RAD_WS + d] = w[d];
+      for (int kb = 0; kb < RAD_NKB; kb++)
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+          rad_bf16x8 v8;
+#pragma unroll
+          for (int e = 0; e < 8; e++) v8[e] = slot[kb * 16 + hf * 8 + e];
+          *reinterpret_cast<rad_bf16x8*>(P.yb + (((tile * RAD_NKB + kb) * 2 + hf) * RAD_TJ + c) * 8) = v8;
+        }
+#if RAD_MM
+      rad_store_weights_mm(reinterpret_cast<__bf16*>(P.bw), pos, w);
+#else
+#pragma unroll
+      for (int d = 0; d < RAD_WS; d++) P.bw[pos * RAD_WS + d] = w[d];
 #endif
+    }
   }
 }
 
-// the matrix-core path is taken when the kernel is not too narrow for the cloud (see the head of this file)
-extern "C" __global__ void __launch_bounds__(64) keops_rad_decide(const RadParams P) {
-  if (threadIdx.x != 0) return;
+// pass 4: largest |k| |x^|^2 of the rows of every wavefront of the sweep (32 * RAD_RB sorted rows) and of the columns
+// of every tile (RAD_TJ sorted columns); one wavefront per group
+extern "C" __global__ void __launch_bounds__(256) keops_rad_groupmax(const RadParams P) {
+  const i64 gr = (P.nx + 32 * RAD_RB - 1) / (32 * RAD_RB), gc = (P.ny + RAD_TJ - 1) / RAD_TJ;
+  i64 g = (i64)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (g >= gr + gc) return;
+  const int which = g >= gr, lane = threadIdx.x & 63;
+  if (which) g -= gr;
+  const i64 len = which ? RAD_TJ : 32 * RAD_RB, n = which ? gc * RAD_TJ : P.nx;
+  const float* q = P.qn[which] + g * len;
+  float m = 0.f;
+  for (i64 k = lane; k < len && g * len + k < n; k += 64) m = q[k] > m ? q[k] : m;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float other = __shfl_xor(m, o);
+    m = other > m ? other : m;
+  }
+  if (lane == 0) P.gmax[which][g] = m;
+}
+
+// largest |k| |y^|^2 of every column segment of keops_rad_exact (one wavefront per segment)
+extern "C" __global__ void __launch_bounds__(64) keops_rad_segmax(const RadParams P) {
+  const i64 ntile = (P.ny + RAD_TJ - 1) / RAD_TJ, per = P.seg_len / RAD_TJ;
+  const i64 t0 = (i64)blockIdx.x * per, t1 = keops_min(ntile, t0 + per);
+  float m = 0.f;
+  for (i64 t = t0 + threadIdx.x; t < t1; t += 64) {
+    const float q = P.gmax[1][t];
+    m = q > m ? q : m;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float other = __shfl_xor(m, o);
+    m = other > m ? other : m;
+  }
+  if (threadIdx.x == 0) P.segmax[blockIdx.x] = m;
+}
+
+// The matrix-core path is taken unless too many pairs would fall back to exact differences.  Estimate from the
+// bucket counts: a pair of buckets (a, b) needs exact differences when a + b + 1 > RAD_NBK - 1 (mid-point rule on
+// the bucket edges); the last bucket (everything from RAD_LIMIT on) is bad against every column.
+extern "C" __global__ void __launch_bounds__(RAD_NBK) keops_rad_decide(const RadParams P) {
+  __shared__ double hy[RAD_NBK], bad[RAD_NBK];
+  __shared__ int cnt[2][RAD_NBK];
+  const int b = threadIdx.x;
+  cnt[0][b] = P.btot[0][b];
+  cnt[1][b] = P.btot[1][b];
+  hy[b] = (double)cnt[1][b];
+  __syncthreads();
+  double suffix = 0.0;  // columns in buckets >= RAD_NBK - 1 - b
+  for (int k = RAD_NBK - 1 - b; k < RAD_NBK; k++) suffix += hy[k];
+  bad[b] = (double)cnt[0][b] * suffix;
+  // first sorted position of every bucket
+  if (b < 2) {
+    int run = 0;
+    for (int k = 0; k < RAD_NBK; k++) {
+      P.btot[b][k] = run;
+      run += cnt[b][k];
+    }
+  }
+  __syncthreads();
+  if (b != 0) return;
+  double total = 0.0;
+  for (int k = 0; k < RAD_NBK; k++) total += bad[k];
   T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
   rad_load_params(P, p);
   const float kappa = (float)KeopsRadFormula::kappa(p);
-  const float R = __uint_as_float(P.scal[0]) + __uint_as_float(P.scal[1]);
-  P.scal[2] = (__builtin_fabsf(kappa) * R <= (float)RAD_LIMIT) ? 1u : 0u;  // false for NaN
+  const bool finite = __builtin_fabsf(kappa) <= 3.0e38f;  // false for NaN
+  P.scal[2] = (finite && total <= (double)RAD_EXACT_FRAC * (double)P.nx * (double)P.ny) ? 1u : 0u;
 }
 #endif  // !RAD_RANGES
-
-#if RAD_FOLD
-// k-th tile of the sweep: tiles of the two sign groups alternate while both last, then the rest of the larger group
-__device__ __forceinline__ i64 rad_tile_of(i64 k, i64 pos_tiles, i64 all_tiles, bool& negative) {
-  const i64 neg_tiles = all_tiles - pos_tiles, m = pos_tiles < neg_tiles ? pos_tiles : neg_tiles;
-  if (k < 2 * m) {
-    negative = (k & 1) != 0;
-    return negative ? pos_tiles + (k >> 1) : (k >> 1);
-  }
-  negative = pos_tiles <= neg_tiles;
-  return (negative ? pos_tiles : 0) + m + (k - 2 * m);
-}
-#endif
 
 // ---- main kernel ------------------------------------------------------------------------------------------------
 
@@ -489,9 +554,13 @@ struct RadSweep {
   i64 jbeg, jend;      // jbeg a multiple of RAD_TJ
   float* part;         // [rows_store][RAD_DV] sums of the wavefront's rows
   i64 rows_store;
-  i64 pos_tiles, all_tiles;  // RAD_FOLD
-  const T* const* arg;       // RAD_UPAIR: the arguments, for the row factor u_i of the wavefront's rows ...
-  i64 row_first, row_last;   // ... which are rows row_first + k of the arguments, clamped to row_last
+  const T* const* arg;       // the arguments (RAD_UPAIR: the row factor u_i of the wavefront's rows; exact sub-tiles: x, y) ...
+  i64 row_first, row_last;   // ... whose rows row_first + k, clamped to row_last, are the wavefront's rows
+  // RAD_TILEWISE: sorted position -> point for the rows (indexed by row_first + k), the largest |k| |y^|^2 of every
+  // tile of sorted columns and the largest |k| |x^|^2 of the wavefront's rows
+  const int* rperm;
+  const float* ctmax;
+  float xq;
 };
 
 // parameters of the formula from the argument table
@@ -504,6 +573,43 @@ __device__ __forceinline__ void rad_params_of(const T* const* arg, T (&p)[KEOPS_
   }
 }
 
+// exp(coef * s) the way the reference evaluates it: one rounded product, then an exponential good to 2 ulp whatever the
+// size of the argument (the product with log2(e) in two parts: the hardware exp2 of a single rounded product would be
+// off by 2^-24 |argument|)
+__device__ __forceinline__ float rad_exp_of(float coef, float s) {
+#pragma clang fp contract(off)
+  const float u = coef * s;
+  const float th = u * 1.44269502162933349609375f;
+  const float tl = __builtin_fmaf(u, 1.925963033500011e-08f, __builtin_fmaf(u, 1.44269502162933349609375f, -th));
+  const float e = __builtin_amdgcn_exp2f(th);
+  return __builtin_fmaf(e, tl * 0.693147180559945f, e);
+}
+
+// squared distance in the reference's operation order (difference, square, sequential sum; no contraction)
+__device__ __forceinline__ float rad_sqdist_exact(const float* x, const float (&y)[RAD_D]) {
+#pragma clang fp contract(off)
+  const float d0 = x[0] - y[0];
+  float s = d0 * d0;
+#pragma unroll
+  for (int k = 1; k < RAD_D; k++) {
+    const float d = x[k] - y[k];
+    const float sq = d * d;
+    s = s + sq;
+  }
+  return s;
+}
+
+// original row of the wavefront's k-th row
+__device__ __forceinline__ i64 rad_row_of(const RadSweep& S, i64 k) {
+  const i64 i = keops_min(S.row_first + k, S.row_last);
+#if RAD_TILEWISE
+  return (i64)S.rperm[i];
+#else
+  return i;
+#endif
+}
+
+// All wavefronts of the workgroup call this together with the same columns (they share the staged tile).
 // All wavefronts of the workgroup call this together with the same columns (they share the staged tile).
 __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* bs) {
   const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, col = lane & 31;
@@ -532,7 +638,7 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
     for (int r = 0; r < RAD_RB; r++)
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        const i64 gi = keops_min(S.row_first + r * 32 + 8 * (v >> 2) + 4 * half + (v & 3), S.row_last);
+        const i64 gi = rad_row_of(S, r * 32 + 8 * (v >> 2) + 4 * half + (v & 3));
         T xi[RAD_DIMX > 0 ? RAD_DIMX : 1];
 #pragma unroll
         for (int q = 0; q < RAD_NROWVARS; q++) {
@@ -554,29 +660,26 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
   constexpr int NPF = (CH + RAD_BLOCK - 1) / RAD_BLOCK;
   constexpr int NPW = (RAD_TJ * RAD_WS + RAD_BLOCK - 1) / RAD_BLOCK;
   uint4 pf[NPF];
-#if !RAD_FOLD
   float pfw[NPW];
+#if RAD_TILEWISE
+  float pfq = 0.f;  // largest |k| |y^|^2 of the tile in flight
 #endif
   auto prefetch = [&](i64 j0) {
-#if RAD_FOLD
-    bool neg_;
-    const i64 tile = rad_tile_of(j0 / RAD_TJ, S.pos_tiles, S.all_tiles, neg_);
-#else
     const i64 tile = j0 / RAD_TJ;
-#endif
     const uint4* src = reinterpret_cast<const uint4*>(S.yb + tile * (RAD_NKB * 2 * RAD_TJ * 8));
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * RAD_BLOCK;
       pf[u] = e < CH ? src[e] : make_uint4(0u, 0u, 0u, 0u);
     }
-#if !RAD_FOLD
     const float* wsrc = S.bw + j0 * RAD_WS;  // padded to whole tiles
 #pragma unroll
     for (int u = 0; u < NPW; u++) {
       const int e = tid + u * RAD_BLOCK;
       pfw[u] = e < RAD_TJ * RAD_WS ? wsrc[e] : 0.f;
     }
+#if RAD_TILEWISE
+    pfq = S.ctmax[tile];
 #endif
   };
   if (jbeg < jend) prefetch(jbeg);
@@ -587,18 +690,20 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
       const int e = tid + u * RAD_BLOCK;
       if (e < CH) reinterpret_cast<uint4*>(ys)[e] = pf[u];
     }
-#if !RAD_FOLD
 #pragma unroll
     for (int u = 0; u < NPW; u++) {
       const int e = tid + u * RAD_BLOCK;
       if (e < RAD_TJ * RAD_WS) bs[e] = pfw[u];
     }
+#if RAD_TILEWISE
+    // the tile's norms, with those of the wavefront's rows, beyond what the matrix-core exponents are good for: the
+    // wavefront leaves the tile to keops_rad_exact (same test there; wavefront-uniform)
+    const bool skip = !(pfq + S.xq <= (float)RAD_LIMIT);
 #endif
     __syncthreads();
     if (j0 + RAD_TJ < jend) prefetch(j0 + RAD_TJ);
-#if RAD_FOLD
-    bool negative;  // uniform: one sign per tile
-    (void)rad_tile_of(j0 / RAD_TJ, S.pos_tiles, S.all_tiles, negative);
+#if RAD_TILEWISE
+    if (skip) continue;
 #endif
 #pragma unroll
     for (int sub = 0; sub < RAD_NSUB; sub++) {
@@ -606,11 +711,9 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
       rad_bf16x8 b[RAD_NKB];
 #pragma unroll
       for (int kb = 0; kb < RAD_NKB; kb++) b[kb] = *reinterpret_cast<const rad_bf16x8*>(ys + ((kb * 2 + half) * RAD_TJ + c) * 8);
-#if !RAD_FOLD
       float w[RAD_WS];
 #pragma unroll
       for (int d = 0; d < RAD_WS; d++) w[d] = bs[c * RAD_WS + d];
-#endif
       rad_f32x16 t[RAD_RB];
 #if RAD_BIL
       rad_f32x16 t2[RAD_RB];  // <u_i, v_j> of the same pairs
@@ -631,19 +734,6 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
         t2[r] = z;
 #endif
       }
-#if RAD_FOLD
-      if (!negative) {
-#pragma unroll
-        for (int r = 0; r < RAD_RB; r++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) acc[r][v][0] += __builtin_amdgcn_exp2f(t[r][v]);
-      } else {
-#pragma unroll
-        for (int r = 0; r < RAD_RB; r++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) acc[r][v][0] -= __builtin_amdgcn_exp2f(t[r][v]);
-      }
-#else
 #pragma unroll
       for (int r = 0; r < RAD_RB; r++)
 #pragma unroll
@@ -666,7 +756,6 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
           for (int d = 0; d < RAD_DV; d++) acc[r][v][d] = __builtin_fmaf(e, w[d], acc[r][v][d]);
 #endif
         }
-#endif
     }
   }
   // the 32 lanes of a half hold the same rows for different columns: shuffle sums, then one lane stores
@@ -720,6 +809,9 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
   constexpr int CW = RAD_TJ * 4 * RAD_MM_NB;  // 16-byte chunks of the weights of a tile (64 bytes per column and block)
   constexpr int NPW = (CW + RAD_BLOCK - 1) / RAD_BLOCK;
   uint4 pf[NPF], pfw[NPW];
+#if RAD_TILEWISE
+  float pfq = 0.f;  // largest |k| |y^|^2 of the tile in flight
+#endif
   const __bf16* bwm = reinterpret_cast<const __bf16*>(S.bw);
   auto prefetch = [&](i64 j0) {
     const uint4* src = reinterpret_cast<const uint4*>(S.yb + (j0 / RAD_TJ) * (RAD_NKB * 2 * RAD_TJ * 8));
@@ -734,6 +826,9 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
       const int e = tid + u * RAD_BLOCK;
       pfw[u] = e < CW ? wsrc[e] : make_uint4(0u, 0u, 0u, 0u);
     }
+#if RAD_TILEWISE
+    pfq = S.ctmax[j0 / RAD_TJ];
+#endif
   };
   if (jbeg < jend) prefetch(jbeg);
   i64 since_fold = 0;
@@ -749,8 +844,14 @@ __device__ __forceinline__ void rad_sweep_mm(const RadSweep& S, __bf16* ys, __bf
       const int e = tid + u * RAD_BLOCK;
       if (e < CW) reinterpret_cast<uint4*>(ws)[e] = pfw[u];
     }
+#if RAD_TILEWISE
+    const bool skip = !(pfq + S.xq <= (float)RAD_LIMIT);  // left to keops_rad_exact (see rad_sweep)
+#endif
     __syncthreads();
     if (j0 + RAD_TJ < jend) prefetch(j0 + RAD_TJ);
+#if RAD_TILEWISE
+    if (skip) continue;
+#endif
 #pragma unroll
     for (int sub = 0; sub < RAD_NSUB; sub++) {
       const int c = sub * 32 + col;
@@ -874,15 +975,14 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
   __shared__ __attribute__((aligned(16))) __bf16 ys[RAD_NKB * 2 * RAD_TJ * 8];  // [kb][half][col][8]
 #if RAD_MM
   __shared__ __attribute__((aligned(16))) __bf16 ws[RAD_TJ * 32 * RAD_MM_NB];  // [sub-tile][k block][half][operand column][8]
-#elif !RAD_FOLD
-  __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_WS];
 #else
-  float* bs = nullptr;
+  __shared__ __attribute__((aligned(16))) float bs[RAD_TJ * RAD_WS];
 #endif
   const int wave = threadIdx.x >> 6;
-  const i64 row0 = ((i64)blockIdx.x * RAD_WAVES + wave) * (32 * RAD_RB);
-  // (RAD_FOLD: the partition by sign pads both groups to whole tiles: one more tile than the columns need)
-  const i64 ncols = RAD_FOLD ? ((P.ny + RAD_TJ - 1) / RAD_TJ + 1) * RAD_TJ : P.ny;
+  // (both clouds are sorted by increasing norm: the workgroups of the last rows and the last slab leave the most
+  // tiles to keops_rad_exact, so the launch ends on the workgroups that have the least to do)
+  const i64 bx = (i64)blockIdx.x, by = (i64)blockIdx.y;
+  const i64 row0 = (bx * RAD_WAVES + wave) * (32 * RAD_RB);
   RadSweep S;
   // a wavefront past the last row sweeps the last row again (the workgroup's barriers need it) and stores nothing
   const i64 first = row0 < P.nx ? row0 : P.nx - 1;
@@ -890,36 +990,218 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
   S.rows_avail = P.nx - first;
   S.yb = P.yb;
   S.bw = P.bw;
-  S.jbeg = (i64)blockIdx.y * P.slab_len;
-  S.jend = keops_min(ncols, S.jbeg + P.slab_len);
-  S.part = P.partial + ((i64)blockIdx.y * P.nx + first) * RAD_DV;
+  S.jbeg = by * P.slab_len;
+  S.jend = keops_min(P.ny, S.jbeg + P.slab_len);
+  S.part = P.partial + (by * P.nx + first) * RAD_DV;
   S.rows_store = row0 < P.nx ? P.nx - row0 : 0;
-  S.pos_tiles = RAD_FOLD ? keops_uniform((i64)P.scal[3]) : 0;  // tiles of columns with non-negative weights come first
-  S.all_tiles = ncols / RAD_TJ;
   S.arg = P.arg;
   S.row_first = first;
   S.row_last = P.nx - 1;
+  S.rperm = P.perm[0];
+  S.ctmax = P.gmax[1];
+  // largest |k| |x^|^2 of the wavefront's rows (a wavefront past the last row recomputes the last row: that row's group)
+  S.xq = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, P.gmax[0][first / (32 * RAD_RB)])));
 #if RAD_MM
   rad_sweep_mm(S, ys, ws);
 #else
   rad_sweep(S, ys, bs);
 #endif
 }
+
+// The tiles that the sweep left out, from exact differences.  RADX_LPR lanes share an output row (its original
+// coordinates in their registers) and take every RADX_LPR-th column of a staged chunk; the 256 columns of a chunk are
+// staged in LDS with everything a pair needs -- original coordinates, centred coordinates (gradients with respect to
+// the points) and the weights as the formula gives them -- and read back 16 bytes at a time.  The test of a
+// (wavefront of the sweep, tile) pair is the sweep's own, on the same numbers, so every pair is computed exactly once.
+// The work sits where both norms are large (the last rows against the last columns): it is cut finer than the sweep,
+// in workgroups of 256 / RADX_LPR rows and column segments of seg_len, heaviest first, and the sums of a segment go to
+// their own array, which keops_rad_reduce adds for the rows that have any (same test again).
+#define RADX_LPR 4
+#define RADX_ROWS (256 / RADX_LPR)
+extern "C" __global__ void __launch_bounds__(256) keops_rad_exact(const RadParams P) {
+  if (P.scal[2] != 1u) return;
+  // floats per staged column: original coordinates | centred coordinates (RAD_DIFF) | weights, each padded to 16 bytes
+  constexpr int XD = (RAD_D + 3) / 4 * 4, XC = RAD_DIFF != 0 ? XD : 0, XWT = (RAD_DW + 3) / 4 * 4, XW = XD + XC + XWT;
+  __shared__ __attribute__((aligned(16))) float cs[256 * XW];
+  __shared__ float wgmax[4];
+  const int tid = threadIdx.x, lane = tid & 63, sub = tid % RADX_LPR;
+  // (the last rows and the last segment hold the work: they are issued first)
+  const i64 bx = (i64)gridDim.x - 1 - blockIdx.x, seg = (i64)gridDim.y - 1 - blockIdx.y;
+  const i64 k = bx * RADX_ROWS + tid / RADX_LPR;  // sorted position of the lane's row
+  const bool valid = k < P.nx;
+  const float xq = valid ? P.gmax[0][k / (32 * RAD_RB)] : 0.f;
+  // nothing to do for the whole workgroup?  (the rows are sorted: most workgroups meet no tile beyond the bound)
+  {
+    float m = valid ? xq : 0.f;
+    m = !(m == m) ? 3.0e38f : m;  // a NaN norm: every tile
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float other = __shfl_xor(m, o);
+      m = other > m ? other : m;
+    }
+    if (lane == 0) wgmax[tid >> 6] = m;
+  }
+  __syncthreads();
+  const float xq_wg = fmaxf(fmaxf(wgmax[0], wgmax[1]), fmaxf(wgmax[2], wgmax[3]));
+  if (P.segmax[seg] + xq_wg <= (float)RAD_LIMIT) return;  // (uniform over the workgroup)
+  const i64 jbeg = seg * P.seg_len, jend = keops_min(P.ny, jbeg + P.seg_len);
+  const i64 tile0 = jbeg / RAD_TJ, ntile = jend > jbeg ? (jend - jbeg + RAD_TJ - 1) / RAD_TJ : 0;
+  T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
+  rad_load_params(P, p);
+  const float coef = (float)KeopsRadFormula::coef(p);
+  const i64 i = valid ? (i64)P.perm[0][k] : 0;
+  float xv[RAD_D];
+#pragma unroll
+  for (int d = 0; d < RAD_D; d++) xv[d] = (float)P.arg[RAD_XARG][i * RAD_D + d];
+#if RAD_BIL || RAD_UPAIR
+  float uv[RAD_DW];
+  {
+    T xi[RAD_DIMX > 0 ? RAD_DIMX : 1], u_[RAD_DU > 0 ? RAD_DU : 1];
+#pragma unroll
+    for (int v = 0; v < RAD_NROWVARS; v++) {
+      const T* a = P.arg[rad_row_arg[v]] + i * rad_row_dim[v];
+#pragma unroll
+      for (int d = 0; d < rad_row_dim[v]; d++) xi[rad_row_off[v] + d] = a[d];
+    }
+    KeopsRadFormula::rowvec(xi, p, u_);
+#pragma unroll
+    for (int d = 0; d < RAD_DW; d++) uv[d] = (float)u_[d];
+  }
+#endif
+  float acc[RAD_DV];
+#pragma unroll
+  for (int d = 0; d < RAD_DV; d++) acc[d] = 0.f;
+
+  // one pair: column `col` of the staged chunk against the lane's row
+  auto pair = [&](const float* col) {
+    float yv[RAD_D];
+    {
+      float yy[XD];
+#pragma unroll
+      for (int q = 0; q < XD / 4; q++) *reinterpret_cast<float4*>(yy + 4 * q) = reinterpret_cast<const float4*>(col)[q];
+#pragma unroll
+      for (int d = 0; d < RAD_D; d++) yv[d] = yy[d];
+    }
+    float wv[XWT];
+#pragma unroll
+    for (int q = 0; q < XWT / 4; q++) *reinterpret_cast<float4*>(wv + 4 * q) = reinterpret_cast<const float4*>(col + XD + XC)[q];
+#if RAD_DIFF != 0
+    float cf[XD];
+#pragma unroll
+    for (int q = 0; q < XD / 4; q++) *reinterpret_cast<float4*>(cf + 4 * q) = reinterpret_cast<const float4*>(col + XD)[q];
+#endif
+    const float e = rad_exp_of(coef, rad_sqdist_exact(xv, yv));
+#if RAD_BIL || RAD_UPAIR
+    float sp = uv[0] * wv[0];
+#pragma unroll
+    for (int d = 1; d < RAD_DW; d++) sp = __builtin_fmaf(uv[d], wv[d], sp);
+    const float es = e * sp;
+#if RAD_DIFF != 0
+#pragma unroll
+    for (int d = 0; d < RAD_D; d++) acc[d] = __builtin_fmaf(es, cf[d], acc[d]);
+    acc[RAD_D] += es;
+#else
+    acc[0] += es;
+#endif
+#elif RAD_DIFF != 0
+    // component d of the weights against [y^_j, 1]
+#pragma unroll
+    for (int d = 0; d < RAD_DW; d++) {
+      const float ew = e * wv[d];
+#pragma unroll
+      for (int q = 0; q < RAD_D; q++) acc[d * (RAD_D + 1) + q] = __builtin_fmaf(ew, cf[q], acc[d * (RAD_D + 1) + q]);
+      acc[d * (RAD_D + 1) + RAD_D] += ew;
+    }
+#else
+#pragma unroll
+    for (int d = 0; d < RAD_DV; d++) acc[d] = __builtin_fmaf(e, wv[d], acc[d]);
+#endif
+  };
+
+  // the tiles of the segment, 64 at a time: lane t looks at tile base + t, the workgroup visits those that some row needs
+  for (i64 base = 0; base < ntile; base += 64) {
+    const float tqv = base + lane < ntile ? P.gmax[1][tile0 + base + lane] : 0.f;
+    unsigned long long todo = __ballot(base + lane < ntile && !(tqv + xq_wg <= (float)RAD_LIMIT));
+    while (todo != 0ull) {
+      const int t = __builtin_ctzll(todo);
+      todo &= todo - 1ull;
+      const i64 j0 = (tile0 + base + t) * RAD_TJ;
+      const float tq = __shfl(tqv, t);
+      const bool mine = valid && !(tq + xq <= (float)RAD_LIMIT);  // the sweep's test for this row's wavefront
+      for (int c0 = 0; c0 < RAD_TJ; c0 += 256) {
+        const i64 ncol = keops_min((i64)256, keops_min((i64)RAD_TJ - c0, P.ny - (j0 + c0)));  // places past the last column are left out
+        if (ncol <= 0) break;
+        __syncthreads();
+        if (tid < ncol) {
+          const i64 j = (i64)P.perm[1][j0 + c0 + tid];
+          float* dst = cs + tid * XW;
+          const T* y = P.arg[RAD_YARG] + j * RAD_D;
+#pragma unroll
+          for (int d = 0; d < RAD_D; d++) dst[d] = (float)y[d];
+#if RAD_DIFF != 0
+#pragma unroll
+          for (int d = 0; d < RAD_D; d++) dst[XD + d] = (float)((double)y[d] - (double)P.colsum[d]);
+#endif
+          T yj[RAD_DIMY > 0 ? RAD_DIMY : 1], wv[RAD_DW];
+#pragma unroll
+          for (int v = 0; v < RAD_NCOLVARS; v++) {
+            const T* a = P.arg[rad_col_arg[v]] + j * rad_col_dim[v];
+#pragma unroll
+            for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
+          }
+          KeopsRadFormula::weights(yj, p, wv);
+#pragma unroll
+          for (int d = 0; d < RAD_DW; d++) dst[XD + XC + d] = (float)wv[d];
+        }
+        __syncthreads();
+        if (!mine) continue;
+        int c = sub;
+        for (; c + 3 * RADX_LPR < (int)ncol; c += 4 * RADX_LPR) {  // four independent pairs in flight
+#pragma unroll
+          for (int u = 0; u < 4; u++) pair(cs + (c + u * RADX_LPR) * XW);
+        }
+        for (; c < (int)ncol; c += RADX_LPR) pair(cs + c * XW);
+      }
+    }
+  }
+  // the RADX_LPR lanes of a row are neighbours
+#pragma unroll
+  for (int d = 0; d < RAD_DV; d++) {
+#pragma unroll
+    for (int o = 1; o < RADX_LPR; o <<= 1) acc[d] += __shfl_xor(acc[d], o);
+  }
+  if (valid && sub == 0 && !(P.segmax[seg] + xq <= (float)RAD_LIMIT)) {
+    float* dst = P.xpart + (seg * P.nx + k) * RAD_DV;
+#pragma unroll
+    for (int d = 0; d < RAD_DV; d++) dst[d] = acc[d];
+  }
+}
 #endif
 
 #if !RAD_RANGES
 // slabs are added in order; the factors of the output index and, for the gradients with respect to the points, the
-// difference x^_i S - sum_j K_ij w_j y^_j are applied here, once per output row
+// difference x^_i S - sum_j K_ij w_j y^_j are applied here, once per output row (the sweep's rows are in sorted order:
+// row k of the sums belongs to point perm[k])
 extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadParams P) {
   if (P.scal[2] != 1u) return;
-  const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
-  if (i >= P.nx) return;
+  const i64 k = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (k >= P.nx) return;
+  const i64 i = (i64)P.perm[0][k];
   float s[RAD_DV];
 #pragma unroll
-  for (int d = 0; d < RAD_DV; d++) s[d] = P.partial[i * RAD_DV + d];
-  for (int k = 1; k < P.nslabs; k++)
+  for (int d = 0; d < RAD_DV; d++) s[d] = P.partial[k * RAD_DV + d];
+  for (int sl = 1; sl < P.nslabs; sl++)
 #pragma unroll
-    for (int d = 0; d < RAD_DV; d++) s[d] += P.partial[((i64)k * P.nx + i) * RAD_DV + d];
+    for (int d = 0; d < RAD_DV; d++) s[d] += P.partial[((i64)sl * P.nx + k) * RAD_DV + d];
+  // the sums of keops_rad_exact, for the segments in which this row's wavefront left tiles out (its test)
+  {
+    const float xq = P.gmax[0][k / (32 * RAD_RB)];
+    for (int sg = 0; sg < P.nseg; sg++)
+      if (!(P.segmax[sg] + xq <= (float)RAD_LIMIT)) {
+#pragma unroll
+        for (int d = 0; d < RAD_DV; d++) s[d] += P.xpart[((i64)sg * P.nx + k) * RAD_DV + d];
+      }
+  }
   T p[KEOPS_DIMP > 0 ? KEOPS_DIMP : 1];
   rad_load_params(P, p);
   T xi[RAD_DIMX > 0 ? RAD_DIMX : 1];
@@ -938,15 +1220,15 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_reduce(const RadPara
 #if RAD_DIFF != 0
   const T* x = P.arg[RAD_XARG] + i * RAD_D;
 #pragma unroll
-  for (int k = 0; k < RAD_D; k++) {
-    const float xc = (float)((double)x[k] - (double)P.colsum[k]);
+  for (int c = 0; c < RAD_D; c++) {
+    const float xc = (float)((double)x[c] - (double)P.colsum[c]);
 #if RAD_DU > 0 && !RAD_UPAIR && !RAD_BIL
     float acc = 0.f;
 #pragma unroll
-    for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], __builtin_fmaf(xc, s[d * (RAD_D + 1) + RAD_D], -s[d * (RAD_D + 1) + k]), acc);
-    P.out[i * RAD_DOUT + k] = (T)(ai * (float)RAD_DIFF * acc);
+    for (int d = 0; d < RAD_DW; d++) acc = __builtin_fmaf((float)uv[d], __builtin_fmaf(xc, s[d * (RAD_D + 1) + RAD_D], -s[d * (RAD_D + 1) + c]), acc);
+    P.out[i * RAD_DOUT + c] = (T)(ai * (float)RAD_DIFF * acc);
 #else
-    P.out[i * RAD_DOUT + k] = (T)(ai * (float)RAD_DIFF * __builtin_fmaf(xc, s[RAD_D], -s[k]));
+    P.out[i * RAD_DOUT + c] = (T)(ai * (float)RAD_DIFF * __builtin_fmaf(xc, s[RAD_D], -s[c]));
 #endif
   }
 #elif RAD_DU > 0 && !RAD_BIL

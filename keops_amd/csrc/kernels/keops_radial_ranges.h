@@ -377,10 +377,12 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
   S.jend = S.jbeg + keops_uniform(P.vt[2 * r + 1]) * RAD_TJ;
   S.part = P.partial + local0 * RAD_DV;
   S.rows_store = 32 * RAD_RB;
-  S.pos_tiles = S.all_tiles = 0;
   S.arg = P.arg;
   S.row_first = r0 + (i64)wave * (32 * RAD_RB);
   S.row_last = r1 - 1;
+  S.rperm = nullptr;  // (the per-tile choice belongs to the dense launches: here every range has been checked)
+  S.ctmax = nullptr;
+  S.xq = 0.f;
 #if RAD_MM
   rad_sweep_mm(S, ys, ws);
 #else

@@ -1016,13 +1016,11 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     k_pre, k_lines, k_exprs = body(coef, {})
     ca, cd, co = VarLayout.table(wl.colvars)
     ra, rd, ro = VarLayout.table(al.rowvars)
-    # a scalar weight and no difference factor: the weight joins the exponent, columns are partitioned by its sign
-    fold = int(config.radial_fold and dimw == 1 and not diff and not rows_per_block and not mm)
     meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_mm_nb=-(-3 * Dv // 32), rad_ws=(dimw + D + 1 if upair else Dv), rad_bil=bil, rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
-                rad_yarg=y.ind, rad_fold=fold, rad_tj=tj)
+                rad_yarg=y.ind, rad_tj=tj)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
-    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_FOLD=fold, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DU=du, RAD_UPAIR=upair, RAD_BIL=bil, RAD_NKE=nke, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
-                RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit)!r}f",
+    defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DU=du, RAD_UPAIR=upair, RAD_BIL=bil, RAD_NKE=nke, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
+                RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit if not rows_per_block else config.radial_ranges_limit)!r}f", RAD_EXACT_FRAC=f"{float(config.radial_exact_frac)!r}f",
                 RAD_NCOLVARS=len(wl.colvars), RAD_DIMY=wl.dimy, RAD_NROWVARS=len(al.rowvars), RAD_DIMX=al.dimx)
     src += [f"#define {k} {v}" for k, v in defs.items()]
     for name, vals in (("row_kind", [r[0] for r in rows]), ("row_comp", [r[1] for r in rows]), ("row_term", [r[2] for r in rows]),
@@ -1032,7 +1030,12 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     dy, dx, dp = max(1, wl.dimy), max(1, al.dimx), max(1, full.dimp)
     src += w_pre + a_pre + u_pre + k_pre
     src.append("struct KeopsRadFormula {")
-    src.append("  // log2(e) times the coefficient of the squared distance in the exponent")
+    src.append("  // the coefficient of the squared distance in the exponent")
+    src.append(f"  static __device__ __forceinline__ T coef(const T (&p)[{dp}]) {{")
+    src += k_lines
+    src.append(f"    return {k_exprs[0]};")
+    src.append("  }")
+    src.append("  // log2(e) times that coefficient")
     src.append(f"  static __device__ __forceinline__ T kappa(const T (&p)[{dp}]) {{")
     src += k_lines
     src.append(f"    return ({k_exprs[0]}) * {LOG2E!r}f;")
@@ -1083,7 +1086,7 @@ def get_keops_dll(
         rows_hint = nx if nx < 64 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
            use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs), int(batch_total),
-           binder.templates_digest(), bool(config.radial), bool(config.radial_fold), bool(config.radial_ranges), int(config.radial_mm_min_dv),
+           binder.templates_digest(), bool(config.radial), float(config.radial_limit), float(config.radial_exact_frac), bool(config.radial_ranges), int(config.radial_mm_min_dv),
            int(config.radial_mm_rb), int(config.radial_mm_terms), bool(config.radial_bilinear), bool(config.knn_i8), bool(use_half))
     with _lock:
         hit = _cache.get(key)
