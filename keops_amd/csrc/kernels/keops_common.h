@@ -38,6 +38,20 @@ __device__ __forceinline__ float keops_atan2(float y, float x) { return __ocml_a
 __device__ __forceinline__ double keops_atan2(double y, double x) { return __ocml_atan2_f64(y, x); }
 __device__ __forceinline__ float keops_pow(float x, float y) { return __ocml_pow_f32(x, y); }
 __device__ __forceinline__ double keops_pow(double x, double y) { return __ocml_pow_f64(x, y); }
+// a sum, a difference, a product rounded on its own: never contracted into a fused multiply-add with a neighbour
+// (the arguments of exponentials: an exponential magnifies a relative error of its argument by the argument's size)
+template <typename U> __device__ __forceinline__ U keops_add_rounded(U a, U b) {
+#pragma clang fp contract(off)
+  return a + b;
+}
+template <typename U> __device__ __forceinline__ U keops_sub_rounded(U a, U b) {
+#pragma clang fp contract(off)
+  return a - b;
+}
+template <typename U> __device__ __forceinline__ U keops_mul_rounded(U a, U b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
 __device__ __forceinline__ float keops_fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double keops_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
 __device__ __forceinline__ float keops_floor(float x) { return __builtin_floorf(x); }

@@ -4,9 +4,13 @@ Every value is one scalar; vector-valued formula nodes become Python lists of va
 are hash-consed (common sub-expressions are shared), constants are folded, and a few algebraic
 peepholes keep the per-pair instruction count of the generated HIP code minimal:
 
-* ``exp(u)`` is emitted as the hardware base-2 exponential ``exp2(u * log2(e))`` and, when fast
-  math is allowed, the ``log2(e)`` factor is merged into any uniform (parameter-only) factor of
-  ``u``; the merged product is invariant in the pair loop, so one multiply per pair disappears.
+* ``exp(u)`` is emitted as the hardware base-2 exponential ``exp2(u * log2(e))``.  The argument ``u`` itself is
+  computed the way the reference computes it -- its operations in the reference's order, every product and sum
+  rounded on its own (no fused multiply-adds), the factor ``log2(e)`` applied to the rounded ``u`` and not merged into
+  a factor of it: an exponential magnifies a relative error of its argument by ``|u|``, so a kernel value deep in the
+  tail (``u = -80``) is only as good as ``u`` is bit for bit, and rows whose every term lies there exist (a kernel much
+  narrower than the spacing of the points).  On this GPU a product and a sum issue in the time of one fused
+  multiply-add, so the only cost is the separate ``log2(e)`` multiplication.
 * negations are pushed outwards (they are free source modifiers on the VALU).
 
 The program is printed as straight-line C++ (``const T t7 = t3 * t5;``): with every index a
@@ -37,6 +41,7 @@ class Lir:
         self.level = []
         self.index = {}
         self.loads = {}  # (cat, ind) -> set of component indices actually read
+        self.rounded = set()  # values whose operation must not be contracted with a neighbour (arguments of exp)
 
     # ------------------------------------------------------------------ construction
     def _mk(self, key, level):
@@ -166,8 +171,29 @@ class Lir:
         if self.is_const(a):
             return self.const(math.exp(self.cval(a)))
         if self.dtype == "float" and self.fast_fn:
-            return self._mk(("exp2", self.mul(a, self.const(LOG2E))), self.level[a])
+            if self.exact:
+                return self._mk(("exp2", self.mul(a, self.const(LOG2E))), self.level[a])
+            # u as the reference rounds it, then one product with log2(e): see the head of this file
+            neg = self.nodes[a][0] == "neg"
+            u = self.nodes[a][1] if neg else a
+            self._keep_rounded(u)
+            c = self.const(LOG2E)
+            t = self._mk(("mul", min(u, c), max(u, c)), self.level[a])
+            self.rounded.add(t)
+            return self._mk(("exp2", self._mk(("neg", t), self.level[a]) if neg else t), self.level[a])
         return self._mk(("exp", a), self.level[a])
+
+    def _keep_rounded(self, a):
+        """Marks the sums and products below ``a`` that change with the pair or the output row."""
+        stack = [a]
+        while stack:
+            i = stack.pop()
+            n = self.nodes[i]
+            if i in self.rounded or n[0] in ("const", "load") or self.level[i] == UNIFORM:
+                continue
+            if n[0] in ("add", "sub", "mul"):
+                self.rounded.add(i)
+            stack.extend(n[2:] if n[0] == "call" else n[1:])
 
     def log(self, a):
         if self.is_const(a) and self.cval(a) > 0:
@@ -294,6 +320,8 @@ class Lir:
             boolean = False
             if op == "neg":
                 e = f"-{a[0]}"
+            elif op in ("add", "sub", "mul") and i in self.rounded:
+                e = f"keops_{op}_rounded({a[0]}, {a[1]})"
             elif op in ("add", "sub", "mul", "div"):
                 e = f"{a[0]} {dict(add='+', sub='-', mul='*', div='/')[op]} {a[1]}"
             elif op == "fma":

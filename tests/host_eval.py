@@ -30,6 +30,9 @@ static inline T keops_atan(T x) { return std::atan(x); }
 static inline T keops_atan2(T y, T x) { return std::atan2(y, x); }
 static inline T keops_pow(T x, T y) { return std::pow(x, y); }
 static inline T keops_fma(T a, T b, T c) { return std::fma(a, b, c); }
+static inline T keops_add_rounded(T a, T b) { return a + b; }
+static inline T keops_sub_rounded(T a, T b) { return a - b; }
+static inline T keops_mul_rounded(T a, T b) { return a * b; }
 static inline T keops_floor(T x) { return std::floor(x); }
 static inline T keops_round(T x) { return std::round(x); }
 static inline float __builtin_amdgcn_exp2f(float x) { return std::exp2(x); }

@@ -175,15 +175,26 @@ def test_simplifications():
 
 
 def test_gaussian_lowering_is_minimal():
-    """The Gaussian kernel must cost 3 sub + 3 mul/fma + 1 scale + exp + weight per pair."""
+    """The Gaussian kernel costs 3 sub + 3 mul + 2 add (the squared distance in the reference's order, nothing fused:
+    a product and a sum issue in the time of one fused multiply-add), the product with g, the product with log2(e),
+    exp2 and the weight per pair.  The argument of the exponential is the reference's own, rounding for rounding, and
+    log2(e) multiplies the rounded argument: a coefficient merged with log2(e) would shift every exponent by up to
+    2^-24 of its size, which a kernel value in the far tail (exponent -80) shows as 1e-5."""
     al = ["x=Var(0,3,0)", "y=Var(1,3,1)", "b=Var(2,1,1)", "g=Var(3,1,2)"]
     red = parse_reduction("Sum_Reduction(Exp(-g*SqDist(x,y))*b,0)", al)
     L = Lir(row_cat=0, fast_math=True)
     outs = lower(red.formula, L)
-    assert L.count_ops(outs) == 11  # sub x3, mul x3, add x2, scale, exp2, weight (mul+add fuse to fma)
+    assert L.count_ops(outs) == 12  # sub x3, mul x3, add x2, g, log2(e), exp2, weight
+    names = {(v.cat, v.ind, k): f"a{v.ind}[{k}]" for v in red.formula.variables for k in range(v.dim)}
+    lines, _ = L.emit(outs, names)
+    text = "\n".join(lines)
+    # the reference's operation order (Subtract.py:21-24, Square.py:17-18, Sum.py:20-24, Mult.py:25), every operation
+    # of the argument rounded on its own, then one product with log2(e)
+    assert text.count("keops_sub_rounded") == 3 and text.count("keops_mul_rounded") == 5 and text.count("keops_add_rounded") == 2
+    assert "keops_mul_rounded(a3[0], " in text and "1.4426950408889634f" in text
     g = parse_reduction("Grad_WithSavedForward(Sum_Reduction(Exp(-g*SqDist(x,y))*b,0),Var(0,3,0),Var(4,1,0),Var(5,1,0))", al)
     L = Lir(row_cat=0, fast_math=True)
-    assert L.count_ops(lower(g.formula, L)) <= 16
+    assert L.count_ops(lower(g.formula, L)) <= 19
 
 
 def test_parser_errors_and_aliases():

@@ -211,6 +211,48 @@ def test_one_far_outlier_in_a_large_cloud_keeps_the_matrix_core_path():
     assert_sum_parity(got[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
 
 
+@pytest.mark.parametrize("D,Dv,M,N,ratio,offset", [
+    (7, 23, 24918, 13490, 0.101, 0.0),     # every live term of a row has an exponent of -50 ... -87
+    (8, 20, 16004, 18283, 0.0448, 30.0),
+    (7, 1, 17000, 16500, 0.16, 0.0),
+    (8, 3, 6000, 7000, 0.08, 1.0),         # (a small call: the module has no matrix-core kernels at all)
+    (3, 1, 9000, 8000, 0.02, 0.0),
+])
+def test_kernels_far_narrower_than_the_cloud_keep_parity_in_the_deep_tail(D, Dv, M, N, ratio, offset):
+    """A kernel 5 to 50 times narrower than the cloud in 7-8 dimensions: nearly every pair is tens of widths apart, the
+    rows sum kernel values of 1e-22 ... 1e-38, and an exponential magnifies the relative error of its argument 50 to
+    87 times.  The general-purpose kernel (these calls end there: the device-side estimate finds nearly every tile
+    beyond the matrix cores' bound) forms the argument as the reference does, rounding for rounding, so the values
+    agree with the oracle to the bar where they are not denormal; against float64 the error is the reference's own
+    plus a few 1e-6."""
+    rng = np.random.default_rng(int(1000 * ratio) + D)
+    spread = 0.3
+    x = (rng.standard_normal((M, D)) * spread + offset * spread).astype(np.float32)
+    y = (rng.standard_normal((N, D)) * spread + offset * spread).astype(np.float32)
+    b = np.abs(rng.standard_normal((N, Dv))).astype(np.float32)
+    width = ratio * spread
+    g = np.array([1.0 / (2 * width * width)], np.float32)
+    got = _genred(D, Dv)(*to_dev(x, y, b, g))
+    if M * N >= 1 << 28:
+        assert _last_meta("radial") == "1" and _path_status() == 0
+    rows = np.sort(rng.choice(M, 4000, replace=False)).astype(np.int64)
+    ref = cpu_reduc("gauss", [x, y, b, g], M, N, Dv, rows=rows)
+    out = got[torch.from_numpy(rows).cuda()].cpu().numpy().astype(np.float64)
+    live = ref.min(axis=1) > 1e-30                # (positive weights: the sum is its own scale)
+    assert live.sum() >= 50
+    deep = -np.log(ref[live].max(axis=1) / b.max()) # at least this deep in the tail
+    assert np.median(deep) > 10
+    worst = float(np.max(np.abs(out[live] - ref[live]) / ref[live]))
+    assert worst <= 1e-5, f"against the oracle: {worst:.3e}"
+    sel = torch.from_numpy(rows[live]).cuda()
+    xd, yd = torch.from_numpy(x).double().cuda(), torch.from_numpy(y).double().cuda()
+    d2 = ((xd[sel][:, None, :] - yd[None, :, :]) ** 2).sum(-1)
+    truth = (torch.exp(-float(g[0]) * d2) @ torch.from_numpy(b).double().cuda()).cpu().numpy()
+    own = float(np.max(np.abs(ref[live] - truth) / truth))
+    vs_truth = float(np.max(np.abs(out[live] - truth) / truth))
+    assert vs_truth <= own + 6e-6, f"against float64: {vs_truth:.3e} (the reference's own float32 evaluation: {own:.3e})"
+
+
 def test_small_calls_other_sum_schemes_and_dtypes_stay_on_the_general_purpose_kernel():
     rng = np.random.default_rng(4)
     x, y = rng.standard_normal((2000, 3)).astype(np.float32), rng.standard_normal((3000, 3)).astype(np.float32)
@@ -288,7 +330,7 @@ def test_gradients_wrt_points_and_weights_with_matrix_core_exponents(D):
 @pytest.mark.parametrize("seed", [0, 7])
 def test_random_clouds_and_kernel_widths_vs_oracle(seed):
     """Seeded sweep over dimensions, cloud shapes (anisotropic, two clumps, far from the origin), weight scales and
-    kernel widths from 5 times narrower to 30 times wider than the cloud: the device-side check sends each case to
+    kernel widths from 25 times narrower to 30 times wider than the cloud: the device-side check sends each case to
     the matrix-core exponents or to the exact differences, and every one meets the parity bar against the oracle
     (rows whose whole sum underflows in float32 are left out)."""
     rng = np.random.default_rng(seed)
@@ -307,9 +349,7 @@ def test_random_clouds_and_kernel_widths_vs_oracle(seed):
         b = rng.standard_normal((N, Dv)).astype(np.float32) * float(10 ** rng.uniform(-3, 3))
         if rng.random() < 0.3:
             b = np.abs(b)
-        # (not narrower than a fifth of the cloud: below, every row sums exponents of -50 and less, where the hardware
-        # exp2 of this build and the reference's own fast exponential are both beyond 1e-5 of the libm value)
-        width = float(10 ** rng.uniform(-0.7, 1.5)) * spread
+        width = float(10 ** rng.uniform(-1.4, 1.5)) * spread   # from 25 times narrower than the cloud to 30 times wider
         g = np.array([1.0 / (2 * width * width)], np.float32)
         got = _genred(D, Dv)(*to_dev(x, y, b, g))
         served += _path_status() == 1
@@ -325,7 +365,7 @@ def test_random_clouds_and_kernel_widths_vs_oracle(seed):
         except AssertionError as e:
             raise AssertionError(f"case {case}: D={D} Dv={Dv} M={M} N={N} spread={spread:.3g} offset={offset:.3g} "
                                  f"width={width:.3g}: {e}") from None
-    assert served >= 15
+    assert served >= 10
 
 
 @pytest.mark.parametrize("D,Dw", [(3, 4), (3, 8), (2, 13)])
