@@ -861,7 +861,7 @@ struct KnnHeader {
   void* logcount;
   void* overflow;
   int64_t logcap;
-  int32_t stage, pad_;
+  int32_t stage, fb;  // fb: device-side fallback of the two-phase schedule (see KnnParams)
   // filter on signed bytes (modules with knn_i8=1, two-phase launches; null otherwise)
   void *xq8, *yq8, *ykey_i, *xnorm_i, *xres, *thr_i, *scal;
   int64_t batch_rows, batch_cols;  // batches served as row ranges: indices relative to the batch
@@ -912,8 +912,9 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   if (nr > 2147483647LL) return fail(-1, "too many reference rows for 32-bit indices");
   // sampling step of the threshold estimate: every 16th reference for large sets, a sample of >= ~4096 rows otherwise
   const int64_t SAMPLE = std::max<int64_t>(2, std::min<int64_t>(m.meta_int("knn_sample", 16), nr / knn_min_sample()));
-  // the two-phase schedule reads a flag back from the device: not while the stream records into a HIP graph
-  const bool two_phase = nr >= knn_two_phase_min_refs() && nr / SAMPLE >= 8 * K && nq >= 1024 && !stream_is_capturing(stream);
+  // (the two-phase schedule needs no read-back: when a candidate log overflows, the adaptive kernel, launched behind
+  // it and idle otherwise, redoes the search, so the same sequence of launches also records into a HIP graph)
+  const bool two_phase = nr >= knn_two_phase_min_refs() && nr / SAMPLE >= 8 * K && nq >= 1024;
   const int64_t nsample = two_phase ? (nr + SAMPLE - 1) / SAMPLE : 0;
 
   // adaptive pass: over the sample (two-phase) or over everything
@@ -1015,7 +1016,6 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
     const int64_t qb = sampling ? SQB : QB;
     return run(kernel, (unsigned)((nq + qb - 1) / qb), (unsigned)slabs, (unsigned)(sampling ? SBLOCK : m.block), HS);
   };
-  bool done = false;
   if (two_phase) {
     // (a) thresholds from every SAMPLE-th reference
     void* gargs[3] = {ws + o_yhs, ws + o_ykeys, nullptr};
@@ -1046,17 +1046,21 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
       if (int rc = run("keops_knn_rerank", (unsigned)(f_qblocks * fb_slabs * FW), 1, 64, with_int((int)f_qblocks))) return rc;
       h.stage = 0;
     }
-    if (int rc = ensure_pinned(m, 64)) return rc;
-    HIP_TRY(hipMemcpyAsync(m.pinned, h.overflow, 4, hipMemcpyDeviceToHost, stream));
-    HIP_TRY(hipStreamSynchronize(stream));
-    done = *(volatile int*)m.pinned == 0;  // a log overflowed (pathological ties): redo adaptively
   }
-  if (!done) {
+  {
+    // adaptive schedule: the whole search when the call is too small for two phases, else the fallback that only
+    // runs when a log overflowed (pathological ties; decided on the device: the flag is never read back)
     int64_t slabs = pick_slabs((nq + QB - 1) / QB, nr, TJ, m.cu_count, main_per_cu, tag1D2D == 1 ? 2 : 1, main_min_tiles);
     slabs = std::min<int64_t>(slabs, list_slabs);
     int64_t len = ((nr + slabs - 1) / slabs + TJ - 1) / TJ * TJ;
     slabs = std::max<int64_t>(1, (nr + len - 1) / len);
+    h.fb = two_phase ? 1 : 0;
     if (int rc = adaptive("keops_knn_main", nr, ws + o_yh, ws + o_ykey, 1, slabs, len)) return rc;
+    if (two_phase) {
+      // the merge reads the lists of whichever pass produced them
+      h.nslabs = (int32_t)f_slabs;
+      h.fb = (int32_t)slabs;
+    }
   }
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
   if (int rc = run("keops_knn_merge", (unsigned)((nq + 255) / 256), 1, 256, HS)) return rc;

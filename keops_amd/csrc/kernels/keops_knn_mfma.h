@@ -40,7 +40,7 @@
 //      the same K-list insertion.  With enough slabs, (b)-(c) run twice: first on every 4th slab, whose
 //      replayed lists tighten the thresholds (K-th distance among a quarter of the references instead of
 //      among the sample), then on the other slabs, which then log about four times fewer survivors.
-//      If a log overflows (pathological ties) the host falls back to the adaptive kernel over all
+//      If a log overflows (pathological ties) the adaptive kernel, launched behind and idle otherwise, redoes all
 //      references.
 //
 // The plug-in defines: T (float), KEOPS_NARGS, KNN_D, KNN_DPAD (D rounded up to 16), KNN_K,
@@ -108,7 +108,9 @@ struct KnnParams {
   int* overflow;         // set to 1 when a log was too small
   i64 logcap;
   int stage;             // filter / replay: which slabs this launch covers (knn_stage_slab)
-  int pad_;
+  int fb;                // fallback of the two-phase schedule, decided on the device: keops_knn_main with fb = 1 runs only
+                         // when a candidate log overflowed (*overflow != 0); keops_knn_merge with fb > 0 then merges the
+                         // fb slabs of that pass instead of nslabs
   // filter on signed bytes (KNN_I8; null otherwise)
   signed char* xq8;      // [nq][KNN_DP8] minus the quantised centred queries
   signed char* yq8;      // [nr][KNN_DP8] quantised centred references
@@ -627,6 +629,9 @@ extern "C" __global__ void __launch_bounds__(64 * KNN_WAVES) keops_knn_main(cons
   __shared__ int owner[KNN_WAVES * 32 * KNN_QSETS];
   __shared__ int qq[KNN_WAVES][64];  // queued candidates: local query
   __shared__ int qj[KNN_WAVES][64];  //                    reference index
+#if !KNN_RANGES
+  if (P.fb == 1 && *P.overflow == 0) return;  // the two-phase schedule went through: nothing to redo
+#endif
   knn_sweep<0, KNN_WAVES, KNN_QSETS>(P, ys, ykey_s, lv, li, owner, qq, qj);
 }
 
@@ -932,7 +937,11 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_merge(const KnnParam
   if (q >= P.nq) return;
   float bv[KNN_K];
   int bi[KNN_K];
+#if KNN_RANGES
   knn_merge_lists(P, q, bv, bi, 0, 1, P.nslabs);
+#else
+  knn_merge_lists(P, q, bv, bi, 0, 1, (P.fb > 0 && *P.overflow != 0) ? P.fb : P.nslabs);
+#endif
   T* out = P.out + q * KEOPS_DIMOUT;
 #if KNN_RANGES
   if (P.batch_rows > 0) {

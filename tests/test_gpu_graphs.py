@@ -1,7 +1,7 @@
 """HIP graph capture of launches (torch.cuda.graph): after one eager call with the same shapes, which sizes the
 workspaces, a launch records kernels and copies only, so the replayed graph must reproduce the eager result bit for
-bit on new input values.  Launches that have to wait for the device adapt (the KNN scheme takes its adaptive
-schedule); block-sparse ranges are validated on the host once and then served without a read-back."""
+bit on new input values.  Nothing on the way waits for the device: the two-phase K-nearest-neighbour schedule keeps its
+fallback on the device, block-sparse ranges are validated on the host once and then served without a read-back."""
 import pytest
 import torch
 
@@ -73,9 +73,11 @@ def test_batched_reduction_under_graph_capture():
     assert _replays_like_eager(batched, [xb, yb, bb])
 
 
-def test_knn_scheme_takes_its_adaptive_schedule_under_capture():
-    """20000 x 40000 references would run the sampled two-phase schedule, which reads a flag back from the device;
-    under capture the launch uses the adaptive one: same neighbours, no wait."""
+def test_knn_two_phase_schedule_under_capture():
+    """20000 x 40000 references run the sampled two-phase schedule (thresholds from a sample, fixed-threshold filter,
+    exact replay of the survivors).  Its fallback for overflowing candidate logs is a kernel that is launched behind
+    it and returns at once unless the device raised the flag: no read-back, so the same launches record into a graph
+    and replay bit for bit on new data."""
     from keops_amd.torch import Genred
 
     gen = torch.Generator(device="cuda").manual_seed(3)

@@ -229,8 +229,9 @@ def test_knn_two_phase_with_massive_ties(D):
 
 
 def test_knn_two_phase_log_overflow_falls_back():
-    """All references identical: every pair passes any threshold, the candidate logs overflow and the launch
-    falls back to the adaptive schedule; the K lowest indices win the ties."""
+    """All references identical: every pair passes any threshold, the candidate logs overflow and the adaptive kernel
+    that is launched behind the two-phase schedule (idle otherwise; the flag stays on the device) redoes the search;
+    the K lowest indices win the ties."""
     M, N, D, K = 1100, 33000, 32, 6
     rng = np.random.default_rng(62)
     x = rng.random((M, D)).astype(np.float32)
