@@ -33,9 +33,9 @@ PUBLISHED_PAIRS_PER_S = 1e12 / 1.39
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/);
 # None until measured for a workload
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/keops_rad_main__gauss_1m_dv1.md: FETCH_SIZE 2302881 KiB x 2.0 (copy calibration) + WRITE_SIZE 11718.75 KiB
-    # (column slot vectors re-read by every row block, 98 % from L2 / Infinity Cache; 52 GB/s, not the limiter)
-    "gauss_1m_dv1": int((2302881 * 2.0 + 11718.75) * 1024),
+    # profiles/keops_rad_main__gauss_1m_dv1.md: FETCH_SIZE 2472982 KiB x 2.0 (copy calibration) + WRITE_SIZE 11718.75 KiB
+    # (column slot vectors re-read by every row block, 98 % from L2 / Infinity Cache; 55 GB/s, not the limiter)
+    "gauss_1m_dv1": int((2472982 * 2.0 + 11718.75) * 1024),
     # profiles/keops_knn_filter_i8__knn_d64.md: dominant kernel keops_knn_filter_i8 (two launches per call)
     "knn_d64": int(2 * (200093 * 2.0 + 45852) * 1024),
     # profiles/keops_chk_final__laplace_d256.md

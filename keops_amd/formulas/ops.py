@@ -1690,6 +1690,24 @@ def Divergence(formula, v):
     return acc
 
 
+def TraceOperator(formula, v):
+    """Trace of a formula that is linear in the variable v (LinearOperators/TraceOperator.py:27-101 with w = 1):
+    dim(F) = dim(v): sum_k M_kk of the matrix M of F; dim(F) = 1: sum_k M_k.  The Jacobian of a linear formula does not
+    depend on v, so v is absent from the result (a formula that still contains it was not linear)."""
+    formula, v = as_op(formula), as_op(v)
+    if not isinstance(v, Var):
+        raise FormulaError("TraceOperator(F, v): v must be a variable")
+    if formula.dim == v.dim:
+        res = Divergence(formula, v)
+    elif formula.dim == 1:
+        res = Diff(formula, v, SumT(IntCst(1), v.dim))
+    else:
+        raise FormulaError(f"TraceOperator: output dimension should be 1 or {v.dim} (got {formula.dim}).")
+    if v in res.variables:
+        raise FormulaError("TraceOperator: the formula must be a linear function of the variable")
+    return res
+
+
 def Laplacian(formula, v):
     """Divergence of the gradient of a scalar formula (autodiff/Laplacian.py:16-23)."""
     formula, v = as_op(formula), as_op(v)
@@ -1698,4 +1716,4 @@ def Laplacian(formula, v):
     return Divergence(formula.diff_t(v, IntCst(1)), v)
 
 
-FUNCTIONS.update(Diff=Diff, Divergence=Divergence, Laplacian=Laplacian)
+FUNCTIONS.update(Diff=Diff, Divergence=Divergence, Laplacian=Laplacian, TraceOperator=TraceOperator)

@@ -451,6 +451,17 @@ class LazyTensor:
         other = self._lift(other)
         return self._like(O.Divergence(self.formula, other.formula), other)
 
+    def trace_operator(self, var):
+        """Trace of self with respect to the variable ``var``, of which self must be a linear function
+        (lazy_tensor.py "trace_operator").  The variable leaves the formula: it needs no data when the result is reduced."""
+        var = self._lift(var)
+        if not isinstance(var.formula, O.Var):
+            raise ValueError("LazyTensor.trace_operator expects a variable")
+        res = self._like(O.TraceOperator(self.formula, var.formula), var)
+        res.variables.pop(var.formula.ind, None)
+        res.symbolic.discard(var.formula.ind)
+        return res
+
     def laplacian(self, other):
         """Symbolic Laplacian of a scalar formula with respect to ``other`` (lazy_tensor.py "laplacian")."""
         other = self._lift(other)

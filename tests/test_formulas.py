@@ -280,6 +280,26 @@ def test_forward_mode_diff_divergence_laplacian():
     _check("Laplacian(Exp(-g*SqDist(x,y)), x)", al, a, lap)
 
 
+def test_trace_operator_of_linear_formulas():
+    """TraceOperator(F, v) for F linear in v (keopscore/formulas/LinearOperators/TraceOperator.py:27-101): the trace of
+    the matrix of F when dim(F) = dim(v), the sum of its coefficients when dim(F) = 1; v leaves the formula."""
+    rng = np.random.default_rng(3)
+    A, x, p = rng.random((M, 9)), rng.random((N, 3)), rng.random(1)
+    al = ["A=Vi(0,9)", "x=Vj(1,3)", "p=Pm(2,1)", "v=Vj(3,3)"]
+    f = parse("TraceOperator(MatVecMult(A,v)*p + 2*v, v)", al)
+    assert f.dim == 1 and sorted(w.ind for w in f.variables) == [0, 2]
+    got = dense_eval(f, None, [A, x, p], M, N)
+    # MatVecMult(A, v)_i = sum_k A[3k + i] v_k: the diagonal is A[0], A[4], A[8]
+    assert np.allclose(got[:, :, 0], (A[:, 0] + A[:, 4] + A[:, 8])[:, None] * p + 6, rtol=1e-12)
+    g = parse("TraceOperator((A|Concat(Concat(v,v),v))*p + (x|v), v)", al)
+    got = dense_eval(g, None, [A, x, p], M, N)
+    assert np.allclose(got[:, :, 0], A.sum(1)[:, None] * p + x.sum(1)[None, :], rtol=1e-12)
+    with pytest.raises(FormulaError, match="linear"):
+        parse("TraceOperator(v*v, v)", al)
+    with pytest.raises(FormulaError, match="dimension"):
+        parse("TraceOperator(Concat(v,v), v)", al)
+
+
 def test_forward_mode_through_log_sum_exp_reduction():
     """Diff_WithSavedForward of a Max_SumShiftExpWeight reduction: [0, d(sum_j exp(F - m) G)] with the saved
     maximum m; flattened as the Python layer does (tangent of m + log s is ds / s) it must equal the jvp of a

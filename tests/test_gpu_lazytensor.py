@@ -214,3 +214,20 @@ def test_torch_func_transforms(which):
     assert close(torch.func.jacfwd(f_keops)(*args), torch.func.jacfwd(f_torch)(*args))
     assert close(torch.func.hessian(f_keops)(*args), torch.func.hessian(f_torch)(*args))
     assert close(torch.func.vmap(f_keops)(*args), torch.func.vmap(f_torch)(*args))
+
+
+def test_trace_operator_on_lazytensors():
+    """x.trace_operator(v) (pykeops/common/lazy_tensor.py:2007-2035): self must be linear in the symbolic variable v,
+    which leaves the formula and needs no data in the reduction."""
+    from keops_amd.torch import LazyTensor, Vi, Vj
+
+    gen = torch.Generator(device="cuda").manual_seed(12)
+    A = torch.rand(300, 9, device="cuda", generator=gen)
+    b = torch.rand(400, 1, device="cuda", generator=gen)
+    Ai, bj = Vi(A), Vj(b)
+    v = LazyTensor((7, 3, 1))                       # symbolic variable Var(7, 3, 1)
+    F = Ai.matvecmult(v) * bj + 2 * v               # linear in v: trace = b_j tr(A_i) + 6
+    T = F.trace_operator(v)
+    out = T.sum(dim=1)
+    tr = A[:, 0] + A[:, 4] + A[:, 8]
+    assert torch.allclose(out[:, 0], tr * b.sum() + 6 * 400, rtol=1e-5)
