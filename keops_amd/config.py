@@ -64,8 +64,9 @@ radial_bilinear_max_dw = int(os.environ.get("KEOPS_AMD_RADIAL_BILINEAR_MAX_DW", 
 radial_bilinear_max_nkb = int(os.environ.get("KEOPS_AMD_RADIAL_BILINEAR_MAX_NKB", 5))
 radial_mm_max_dv = 32               # ... when the weighted sum runs on the matrix cores (the three terms of the weights in up to three blocks of 32 operand columns)
 radial_rb2_max_dv = int(os.environ.get("KEOPS_AMD_RADIAL_RB2_MAX_DV", 4))  # two 32-row blocks per wavefront up to this many accumulated components
-# columns per staged tile (multiple of 32); auto: 128 up to two accumulated components per pair, 512 beyond (the
-# vector work of a sub-tile grows with the components while the cost of a tile change does not)
+# columns per staged tile (multiple of 32); auto: 512, and 256 when the weighted sum runs on the matrix cores too (a tile
+# change costs two barriers and the test of the tile's bound: 10^6 x 10^6 with one weight, 128 / 256 / 512 columns:
+# 95.9 / 93.4 / 93.0 ms; gradient with respect to the points, 256 / 512 / 1024: 182.6 / 180.0 / 187.3 ms)
 # accumulated components from which the weighted sum of the radial scheme runs on the matrix cores (per pair the vector
 # ALU then issues v_exp_f32 and a three-term split instead of one fused multiply-add per component); 99: never
 radial_mm_min_dv = int(os.environ.get("KEOPS_AMD_RADIAL_MM_MIN_DV", 7))

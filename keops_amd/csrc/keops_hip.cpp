@@ -687,6 +687,7 @@ struct RadHeader {
   void* gmax[2];
   void* out;
   void* partial;
+  void* yo;
   void* xpart;
   void* segmax;
   int64_t slab_len, seg_len;
@@ -737,6 +738,9 @@ int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* arg
   const int64_t seg_len = ((ny + nseg - 1) / nseg + TJ - 1) / TJ * TJ;
   nseg = std::max<int64_t>(1, (ny + seg_len - 1) / seg_len);
   const size_t o_xpart = take((size_t)nseg * nx * DV * 4), o_segmax = take((size_t)nseg * 4);
+  // what the exact kernel reads of a column, in sorted order: coordinates, centred coordinates (gradients), weights
+  const int64_t XW = m.meta_int("rad_exact_xw", 8);
+  const size_t o_yo = take((size_t)ncols * XW * 4);
   if (int rc = m.partial.reserve(off)) return rc;
   char* ws = (char*)m.partial.ptr;
   std::vector<char> buf(sizeof(RadHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs) + 16);
@@ -747,7 +751,7 @@ int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* arg
   h.perm[0] = ws + o_perm_r; h.perm[1] = ws + o_perm_c; h.qn[0] = ws + o_qn_r; h.qn[1] = ws + o_qn_c;
   h.gmax[0] = ws + o_gmax_r; h.gmax[1] = ws + o_gmax_c;
   h.out = out; h.partial = ws + o_part; h.slab_len = slab_len; h.nslabs = (int32_t)nslabs; h.nparts = nparts;
-  h.xpart = ws + o_xpart; h.segmax = ws + o_segmax; h.seg_len = seg_len; h.nseg = (int32_t)nseg;
+  h.yo = ws + o_yo; h.xpart = ws + o_xpart; h.segmax = ws + o_segmax; h.seg_len = seg_len; h.nseg = (int32_t)nseg;
   std::memcpy(buf.data(), &h, sizeof(h));
   for (int k = 0; k < m.nargs; k++) std::memcpy(buf.data() + sizeof(h) + sizeof(void*) * k, &args[k], sizeof(void*));
   const size_t psize = sizeof(RadHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs);

@@ -75,6 +75,7 @@ __device__ __forceinline__ double keops_fmax(double a, double b) { return __buil
 template <typename A> __device__ __forceinline__ A keops_inf() { return (A)__builtin_huge_valf(); }
 
 __device__ __forceinline__ i64 keops_min(i64 a, i64 b) { return a < b ? a : b; }
+__device__ __forceinline__ i64 keops_max(i64 a, i64 b) { return a > b ? a : b; }
 
 // ---- block-sparse / batched geometry of the matrix-core schemes ------------------------------------
 //

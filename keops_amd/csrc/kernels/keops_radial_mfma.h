@@ -97,6 +97,12 @@ typedef __bf16 rad_bf16x2 __attribute__((ext_vector_type(2)));
 #define RAD_TILEWISE (!RAD_RANGES)
 #define RAD_NBK 128                // buckets of the counting sort by |k| |x^|^2: [0, RAD_LIMIT) in equal parts, the last one open
 #define RAD_SORT_CHUNK 1024        // points per workgroup of the sort (4 rounds of 256)
+// keops_rad_exact: floats per column of its operand: original coordinates | centred coordinates (gradients with respect
+// to the points) | the weights as the formula gives them, each part padded to 16 bytes
+#define RADX_XD ((RAD_D + 3) / 4 * 4)
+#define RADX_XC (RAD_DIFF != 0 ? RADX_XD : 0)
+#define RADX_XWT ((RAD_DW + 3) / 4 * 4)
+#define RADX_XW (RADX_XD + RADX_XC + RADX_XWT)
 #ifndef RAD_EXACT_FRAC
 #define RAD_EXACT_FRAC 0.25f       // largest estimated share of pairs from exact differences for which this family still runs
 #endif
@@ -117,6 +123,7 @@ struct RadParams {
   float* gmax[2];     // largest qn of every group of sorted points: rows by 32 * RAD_RB (a wavefront's rows), columns by RAD_TJ (a tile)
   T* out;             // [nx][RAD_DOUT]
   float* partial;     // [nslabs][nx][RAD_DV], rows in sorted order
+  float* yo;          // [ntiles * RAD_TJ][RADX_XW] what keops_rad_exact needs of a column, columns in sorted order
   float* xpart;       // [nseg][nx][RAD_DV] sums of keops_rad_exact (only the rows that meet a tile beyond the bound are written)
   float* segmax;      // [nseg] largest qn of the columns of every segment
   i64 slab_len;       // reduced rows per slab (multiple of RAD_TJ)
@@ -435,6 +442,33 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_prep(const RadParams
     }
     P.perm[which][pos] = real ? (int)i : -1;
     P.qn[which][pos] = q;
+#if RAD_TILEWISE
+    if (which) {
+      // the column as keops_rad_exact reads it (zeros past the last column)
+      float* yo = P.yo + pos * RADX_XW;
+#pragma unroll
+      for (int d = 0; d < RADX_XW; d++) yo[d] = 0.f;
+      if (real) {
+        const T* src = P.arg[RAD_YARG] + i * RAD_D;
+#pragma unroll
+        for (int d = 0; d < RAD_D; d++) yo[d] = (float)src[d];
+#if RAD_DIFF != 0
+#pragma unroll
+        for (int d = 0; d < RAD_D; d++) yo[RADX_XD + d] = (float)((double)src[d] - (double)P.colsum[d]);
+#endif
+        T yj[RAD_DIMY > 0 ? RAD_DIMY : 1], wv[RAD_DW];
+#pragma unroll
+        for (int v = 0; v < RAD_NCOLVARS; v++) {
+          const T* a = P.arg[rad_col_arg[v]] + i * rad_col_dim[v];
+#pragma unroll
+          for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
+        }
+        KeopsRadFormula::weights(yj, p, wv);
+#pragma unroll
+        for (int d = 0; d < RAD_DW; d++) yo[RADX_XD + RADX_XC + d] = (float)wv[d];
+      }
+    }
+#endif
     if (!which) {
 #pragma unroll
       for (int c8 = 0; c8 < RAD_SLOTS / 8; c8++) {
@@ -1009,21 +1043,28 @@ extern "C" __global__ void __launch_bounds__(RAD_BLOCK, RAD_MIN_WAVES) keops_rad
 }
 
 // The tiles that the sweep left out, from exact differences.  RADX_LPR lanes share an output row (its original
-// coordinates in their registers) and take every RADX_LPR-th column of a staged chunk; the 256 columns of a chunk are
-// staged in LDS with everything a pair needs -- original coordinates, centred coordinates (gradients with respect to
-// the points) and the weights as the formula gives them -- and read back 16 bytes at a time.  The test of a
-// (wavefront of the sweep, tile) pair is the sweep's own, on the same numbers, so every pair is computed exactly once.
-// The work sits where both norms are large (the last rows against the last columns): it is cut finer than the sweep,
-// in workgroups of 256 / RADX_LPR rows and column segments of seg_len, heaviest first, and the sums of a segment go to
-// their own array, which keops_rad_reduce adds for the rows that have any (same test again).
+// coordinates in their registers) and take every RADX_LPR-th column of a staged chunk.  keops_rad_prep has written,
+// in sorted order, everything a pair needs of a column -- original coordinates, centred coordinates (gradients with
+// respect to the points) and the weights as the formula gives them: chunks of RADX_CHUNK columns travel through
+// registers into one of two LDS buffers while the previous chunk is computed (one barrier per chunk), and are read back
+// 16 bytes at a time.  The test of a (wavefront of the sweep, tile) pair is the sweep's own, on the same numbers, so
+// every pair is computed exactly once.  The work sits where both norms are large (the last rows against the last
+// columns): it is cut finer than the sweep, in workgroups of 256 / RADX_LPR rows and column segments of seg_len,
+// heaviest first, and the sums of a segment go to their own array, which keops_rad_reduce adds for the rows that
+// have any (same test again).
 #define RADX_LPR 4
 #define RADX_ROWS (256 / RADX_LPR)
+#define RADX_CHUNK (RADX_XW <= 16 ? (RAD_TJ < 256 ? RAD_TJ : 256) : (RAD_TJ < 128 ? RAD_TJ : 128))  // columns per staged chunk (divides RAD_TJ)
+#define RADX_MAXT 1024   // tiles of a segment whose numbers fit the workgroup's list (longer segments are walked in parts)
 extern "C" __global__ void __launch_bounds__(256) keops_rad_exact(const RadParams P) {
   if (P.scal[2] != 1u) return;
-  // floats per staged column: original coordinates | centred coordinates (RAD_DIFF) | weights, each padded to 16 bytes
-  constexpr int XD = (RAD_D + 3) / 4 * 4, XC = RAD_DIFF != 0 ? XD : 0, XWT = (RAD_DW + 3) / 4 * 4, XW = XD + XC + XWT;
-  __shared__ __attribute__((aligned(16))) float cs[256 * XW];
+  constexpr int XD = RADX_XD, XC = RADX_XC, XWT = RADX_XWT, XW = RADX_XW, CH = RADX_CHUNK, NF4 = XW / 4;
+  constexpr int CPT = RAD_TJ / CH;  // chunks per tile
+  __shared__ __attribute__((aligned(16))) float cs[2][CH * XW];
   __shared__ float wgmax[4];
+  __shared__ int slow_tile[RADX_MAXT];
+  __shared__ float slow_q[RADX_MAXT];
+  __shared__ int nslow_s;
   const int tid = threadIdx.x, lane = tid & 63, sub = tid % RADX_LPR;
   // (the last rows and the last segment hold the work: they are issued first)
   const i64 bx = (i64)gridDim.x - 1 - blockIdx.x, seg = (i64)gridDim.y - 1 - blockIdx.y;
@@ -1118,50 +1159,76 @@ extern "C" __global__ void __launch_bounds__(256) keops_rad_exact(const RadParam
 #endif
   };
 
-  // the tiles of the segment, 64 at a time: lane t looks at tile base + t, the workgroup visits those that some row needs
-  for (i64 base = 0; base < ntile; base += 64) {
-    const float tqv = base + lane < ntile ? P.gmax[1][tile0 + base + lane] : 0.f;
-    unsigned long long todo = __ballot(base + lane < ntile && !(tqv + xq_wg <= (float)RAD_LIMIT));
-    while (todo != 0ull) {
-      const int t = __builtin_ctzll(todo);
-      todo &= todo - 1ull;
-      const i64 j0 = (tile0 + base + t) * RAD_TJ;
-      const float tq = __shfl(tqv, t);
-      const bool mine = valid && !(tq + xq <= (float)RAD_LIMIT);  // the sweep's test for this row's wavefront
-      for (int c0 = 0; c0 < RAD_TJ; c0 += 256) {
-        const i64 ncol = keops_min((i64)256, keops_min((i64)RAD_TJ - c0, P.ny - (j0 + c0)));  // places past the last column are left out
-        if (ncol <= 0) break;
-        __syncthreads();
-        if (tid < ncol) {
-          const i64 j = (i64)P.perm[1][j0 + c0 + tid];
-          float* dst = cs + tid * XW;
-          const T* y = P.arg[RAD_YARG] + j * RAD_D;
-#pragma unroll
-          for (int d = 0; d < RAD_D; d++) dst[d] = (float)y[d];
-#if RAD_DIFF != 0
-#pragma unroll
-          for (int d = 0; d < RAD_D; d++) dst[XD + d] = (float)((double)y[d] - (double)P.colsum[d]);
-#endif
-          T yj[RAD_DIMY > 0 ? RAD_DIMY : 1], wv[RAD_DW];
-#pragma unroll
-          for (int v = 0; v < RAD_NCOLVARS; v++) {
-            const T* a = P.arg[rad_col_arg[v]] + j * rad_col_dim[v];
-#pragma unroll
-            for (int d = 0; d < rad_col_dim[v]; d++) yj[rad_col_off[v] + d] = a[d];
-          }
-          KeopsRadFormula::weights(yj, p, wv);
-#pragma unroll
-          for (int d = 0; d < RAD_DW; d++) dst[XD + XC + d] = (float)wv[d];
+  for (i64 part0 = 0; part0 < ntile; part0 += RADX_MAXT) {
+    const int npart = (int)keops_min((i64)RADX_MAXT, ntile - part0);
+    // the tiles that some row of the workgroup needs, in order (first wavefront: 64 tiles at a time)
+    __syncthreads();
+    if (tid < 64) {
+      int n = 0;
+      for (int base = 0; base < npart; base += 64) {
+        const int t = base + lane;
+        const float tq = t < npart ? P.gmax[1][tile0 + part0 + t] : 0.f;
+        const bool need = t < npart && !(tq + xq_wg <= (float)RAD_LIMIT);
+        const unsigned long long bal = __ballot(need);
+        if (need) {
+          const int at = n + __popcll(bal & ((1ull << lane) - 1ull));
+          slow_tile[at] = t;
+          slow_q[at] = tq;
         }
-        __syncthreads();
-        if (!mine) continue;
-        int c = sub;
-        for (; c + 3 * RADX_LPR < (int)ncol; c += 4 * RADX_LPR) {  // four independent pairs in flight
-#pragma unroll
-          for (int u = 0; u < 4; u++) pair(cs + (c + u * RADX_LPR) * XW);
-        }
-        for (; c < (int)ncol; c += RADX_LPR) pair(cs + c * XW);
+        n += __popcll(bal);
       }
+      if (lane == 0) nslow_s = n;
+    }
+    __syncthreads();
+    const int nitems = nslow_s * CPT;
+    // chunk `it` of the list: columns [col0, col0 + ncol) of the sorted operand
+    auto chunk_of = [&](int it, i64& col0, int& ncol) __attribute__((always_inline)) {
+      const i64 j0 = (tile0 + part0 + slow_tile[it / CPT]) * RAD_TJ + (i64)(it % CPT) * CH;
+      col0 = j0;
+      ncol = (int)keops_max((i64)0, keops_min((i64)CH, P.ny - j0));  // places past the last column are left out
+    };
+    float4 pf[NF4];
+    auto fetch = [&](int it) __attribute__((always_inline)) {
+      i64 col0;
+      int ncol;
+      chunk_of(it, col0, ncol);
+      // (a thread past the last column of the chunk reads a column it will not stash: yo is padded to whole tiles)
+      const float4* src = reinterpret_cast<const float4*>(P.yo + (col0 + (tid < CH ? tid : 0)) * XW);
+#pragma unroll
+      for (int q = 0; q < NF4; q++) pf[q] = src[q];
+    };
+    auto stash = [&](int it) __attribute__((always_inline)) {
+      i64 col0;
+      int ncol;
+      chunk_of(it, col0, ncol);
+      if (tid < ncol) {
+        float4* dst = reinterpret_cast<float4*>(cs[it & 1] + tid * XW);
+#pragma unroll
+        for (int q = 0; q < NF4; q++) dst[q] = pf[q];
+      }
+    };
+    if (nitems > 0) {
+      fetch(0);
+      stash(0);
+    }
+    __syncthreads();
+    for (int it = 0; it < nitems; it++) {
+      if (it + 1 < nitems) fetch(it + 1);  // in flight while this chunk is computed
+      i64 col0;
+      int ncol;
+      chunk_of(it, col0, ncol);
+      const bool mine = valid && !(slow_q[it / CPT] + xq <= (float)RAD_LIMIT);  // the sweep's test for this row's wavefront
+      if (mine) {
+        const float* buf = cs[it & 1];
+        int c = sub;
+        for (; c + 3 * RADX_LPR < ncol; c += 4 * RADX_LPR) {  // four independent pairs in flight
+#pragma unroll
+          for (int u = 0; u < 4; u++) pair(buf + (c + u * RADX_LPR) * XW);
+        }
+        for (; c < ncol; c += RADX_LPR) pair(buf + c * XW);
+      }
+      if (it + 1 < nitems) stash(it + 1);
+      __syncthreads();
     }
   }
   // the RADX_LPR lanes of a row are neighbours

@@ -977,7 +977,7 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     rb = (config.radial_mm_rb if mm else 2) if (mm or Dv <= config.radial_rb2_max_dv) else 1
     if upair:
         rb = 1  # 16 x dim(u) registers per 32-row block hold the row factors
-    tj = ((256 if mm else 128 if Dv <= 2 else 512) if config.radial_tile_j == "auto" else int(config.radial_tile_j))
+    tj = ((256 if mm else 512) if config.radial_tile_j == "auto" else int(config.radial_tile_j))
     if tj % 32 or not 32 <= tj <= 1024:
         raise ValueError("[KeOps] KEOPS_AMD_RADIAL_TJ must be a multiple of 32 between 32 and 1024")
     waves = 8
@@ -1017,7 +1017,8 @@ def generate_radial_section(red, match, nargs, rows_per_block=0):
     ca, cd, co = VarLayout.table(wl.colvars)
     ra, rd, ro = VarLayout.table(al.rowvars)
     meta = dict(radial=1, rad_ranges=int(bool(rows_per_block)), rad_mm=mm, rad_mm_nb=-(-3 * Dv // 32), rad_ws=(dimw + D + 1 if upair else Dv), rad_bil=bil, rad_d=D, rad_dv=Dv, rad_dout=dout, rad_nkb=nkb, rad_rb=rb, rad_waves=waves, rad_xarg=x.ind,
-                rad_yarg=y.ind, rad_tj=tj)
+                rad_yarg=y.ind, rad_tj=tj,
+                rad_exact_xw=-(-D // 4) * 4 * (2 if diff else 1) + -(-dimw // 4) * 4)
     src = ["", "// ---- exponents of the radial kernel on the matrix cores (kernels/keops_radial_mfma.h) ----"]
     defs = dict(RAD_RANGES=int(bool(rows_per_block)), RAD_MM=mm, RAD_MM_TERMS=int(config.radial_mm_terms), RAD_TJ=tj, RAD_D=D, RAD_DV=Dv, RAD_DW=dimw, RAD_DU=du, RAD_UPAIR=upair, RAD_BIL=bil, RAD_NKE=nke, RAD_DOUT=dout, RAD_DIFF=diff, RAD_SIGN=f"{float(sign)!r}f", RAD_NKB=nkb,
                 RAD_RB=rb, RAD_WAVES=waves, RAD_XARG=x.ind, RAD_YARG=y.ind, RAD_LIMIT=f"{float(config.radial_limit if not rows_per_block else config.radial_ranges_limit)!r}f", RAD_EXACT_FRAC=f"{float(config.radial_exact_frac)!r}f",
