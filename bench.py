@@ -33,9 +33,9 @@ PUBLISHED_PAIRS_PER_S = 1e12 / 1.39
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/);
 # None until measured for a workload
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/keops_rad_main__gauss_1m_dv1.md: FETCH_SIZE 2472982 KiB x 2.0 (copy calibration) + WRITE_SIZE 11718.75 KiB
+    # profiles/keops_rad_main__gauss_1m_dv1.md: FETCH_SIZE 2459909 KiB x 2.0 (copy calibration) + WRITE_SIZE 11718.75 KiB
     # (column slot vectors re-read by every row block, 98 % from L2 / Infinity Cache; 55 GB/s, not the limiter)
-    "gauss_1m_dv1": int((2472982 * 2.0 + 11718.75) * 1024),
+    "gauss_1m_dv1": int((2459909 * 2.0 + 11718.75) * 1024),
     # profiles/keops_knn_filter_i8__knn_d64.md: dominant kernel keops_knn_filter_i8 (two launches per call)
     "knn_d64": int(2 * (200093 * 2.0 + 45852) * 1024),
     # profiles/keops_chk_final__laplace_d256.md
@@ -43,7 +43,7 @@ MEASURED_TRAFFIC_BYTES = {
     # profiles/keops_chk_softmax__softmax_d64.md
     "softmax_d64": int((204925 * 2.0 + 33804) * 1024),
     # profiles/keops_fin_main3__gauss_dv256.md
-    "gauss_dv256": int((10715900 * 2.0 + 10797000) * 1024),
+    "gauss_dv256": int((6511553 * 2.0 + 3597770) * 1024),
     # profiles/keops_radr_main__sparse_100x10k.md (all kernels of a launch), keops_conv_ranges__lse_b16.md
     "sparse_100x10k": int((638070 * 2.0 + 179582) * 1024),
     "lse_b16": int((55625 * 2.0 + 6250) * 1024),
@@ -303,20 +303,25 @@ def calibration(mfma):
                  "through LDS, 48 v_mfma_f32_32x32x16_f16 per round (chains = 0: constant operands, 1: random)", (0, 1)),
              (5, "two chains of v_mfma_f32_32x32x16_bf16 with `chains` v_fmac_f32 after every matrix instruction", (0, 1, 2, 4, 8))] if mfma else [
         (0, "v_fmac_f32 chains", (1, 2, 4, 8)), (1, "Gaussian pair mix with v_exp_f32 (9 instr)", (1, 2, 4, 8)),
-        (2, "Gaussian pair mix without v_exp_f32 (8 instr)", (1, 2, 4, 8))]
+        (2, "Gaussian pair mix without v_exp_f32 (8 instr)", (1, 2, 4, 8)),
+        (10, "Gaussian pair, every operation rounded on its own (12 instr), `chains` pairs advanced statement by statement",
+         (1, 2, 4)),
+        (11, "written-out sequences, 8 wavefronts per SIMD (chains = sequence: 0 v_mul vgpr, 1 v_mul sgpr operand, 2 v_mul "
+             "literal, 3 v_add, 4 v_fmac, 5 v_fma three registers, 6 v_max, 7 v_perm_b32, 8 v_exp_f32, 9 v_exp_f32 alternating "
+             "with v_fmac, 10 rounded Gaussian pair (12 instr), 11 contracted pair (9 instr), 12 v_max3)", tuple(range(13)))]
     for kind, label, chain_set in kinds:
         for chains in chain_set:
             # one workgroup = 4 wavefronts = one per SIMD of a CU (kind 9: 8 wavefronts, at most two workgroups per CU)
             wg_waves = 8 if kind == 9 else 4
-            for wgs in ((1, 2) if kind == 9 else (1, 2, 4)):
+            for wgs in ((1, 2) if kind == 9 else (8,) if kind == 11 else (1, 2, 4)):
                 blocks, waves = cus * wgs, wgs * wg_waves // 4
-                iters = {7: 12_500, 8: 100_000, 5: 50_000, 9: 4_000}.get(kind) or (200_000 if kind < 3 else 100_000) // chains
+                iters = {7: 12_500, 8: 100_000, 5: 50_000, 9: 4_000, 11: 20_000}.get(kind) or (200_000 if kind < 3 or kind == 10 else 100_000) // chains
                 ms, ipw = binder.calibrate(kind, chains, blocks, iters)
                 total = ipw * blocks * wg_waves  # wavefront instructions
                 per_cycle = total / (ms * 1e-3) / simds / clock
                 row = dict(kind=label, chains=chains, waves_per_simd=waves, ms=round(ms, 3),
                            wave_instr_per_cycle_per_simd_at_2p4GHz=round(per_cycle, 4))
-                if kind >= 3:
+                if 3 <= kind <= 9:
                     # (kind 6: integer operations, 32 x 32 x 32 per instruction)
                     depth = 32 if kind in (6, 8) or (kind == 7 and chains == 2) else 16
                     row["PFLOP_per_s"] = round(total * 32 * 32 * depth * 2 / (ms * 1e-3) / 1e15, 3)

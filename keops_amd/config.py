@@ -87,10 +87,13 @@ radial_limit = float(os.environ.get("KEOPS_AMD_RADIAL_LIMIT", 30.0))
 radial_exact_frac = float(os.environ.get("KEOPS_AMD_RADIAL_EXACT_FRAC", 0.25))
 # block-sparse launches: one centre and one check per row range, |c| log2(e) (R_x^2 + min(R_y, R_x + reach)^2) <= this
 radial_ranges_limit = float(os.environ.get("KEOPS_AMD_RADIAL_RANGES_LIMIT", 128.0))
-# calls below 2**28 pairs (16384 x 16384) stay on the general-purpose kernel: measured 0.061 vs 0.074 ms at 12000^2, equal at
-# 16000^2, 0.150 vs 0.126 ms at 23000^2 (the pre-pass of the matrix-core scheme is seven small launches)
 radial_ranges = os.environ.get("KEOPS_AMD_RADIAL_RANGES", "1") != "0"  # block-sparse launches too (one centre per row range)
-radial_min_pairs_log2 = int(os.environ.get("KEOPS_AMD_RADIAL_MIN_PAIRS", 29))
+# calls below 2**29 pairs (23171 x 23171) stay on the general-purpose kernel: the sort, the per-tile maxima and the exact
+# kernel around the sweep are a dozen small launches, 0.12 ms together.  Measured, matrix-core scheme against the
+# general-purpose kernel: 16000^2 0.157 vs 0.103 ms, 23000^2 0.186 vs 0.174, 32000^2 0.252 vs 0.293, 50000^2 0.43 vs 0.64,
+# 100000^2 1.19 vs 2.47 ms.  Batches and block-sparse launches (their pre-pass is another one): from 2**28 pairs on
+radial_min_pairs_log2 = int(os.environ.get("KEOPS_AMD_RADIAL_MIN_PAIRS", 30))
+radial_ranges_min_pairs_log2 = int(os.environ.get("KEOPS_AMD_RADIAL_RANGES_MIN_PAIRS", 29))
 
 # matrix-core final-product scheme (csrc/kernels/keops_final_mfma.h): Sum_j f(x_i,y_j) * v_j with dim(v) large
 final_chunk_min_dim = int(os.environ.get("KEOPS_AMD_FINAL_MIN_DIM", 24))   # smallest dim(v) that selects the scheme
@@ -101,7 +104,7 @@ final_split3 = os.environ.get("KEOPS_AMD_FINAL_SPLIT3", "1") != "0"          # p
 # ... of the staged vectors and of the per-pair weights; 2: the weights in two terms, both rounded to nearest (off by up
 # to 2^-17 each, 2.4e-6 rms: not the float32 class; C5b 68.8 against 70.6 ms, softmax_d64 4.70 against 5.09 ms)
 final_weight_terms = int(os.environ.get("KEOPS_AMD_FINAL_WEIGHT_TERMS", 3))
-final_period = int(os.environ.get("KEOPS_AMD_FINAL_PERIOD", 4096))         # block-sum period in reduced rows
+final_period = int(os.environ.get("KEOPS_AMD_FINAL_PERIOD", 16384))        # block-sum period in reduced rows
 
 # matrix-core KNN kernel (csrc/kernels/keops_knn_mfma.h)
 knn_min_dim = int(os.environ.get("KEOPS_AMD_KNN_MIN_DIM", 2))         # smallest vector dimension served by the matrix-core KNN scheme

@@ -50,6 +50,108 @@ static __global__ void __launch_bounds__(256) keops_valu_loop(float* out, int it
   out[(size_t)blockIdx.x * 256 + threadIdx.x] = r;
 }
 
+// The Gaussian pair with every sum and product rounded on its own (no contraction: 3 subtractions, 3 multiplications,
+// 2 additions, the product with the coefficient, the product with log2(e), v_exp_f32, 1 fused multiply-add = 12
+// instructions per chain and round), W chains advanced statement by statement: W = 1 is one dependent chain, as a
+// formula evaluated pair after pair compiles; W = 2, 4 put independent instructions next to each other.
+template <int W, int SREG>
+static __global__ void __launch_bounds__(256) keops_valu_rounded_loop(float* out, int iters, float c0, float c1) {
+#pragma clang fp contract(off)
+  float l2e = -1.4426950408889634f;
+  if (SREG) asm volatile("" : "+s"(l2e));   // the constant in a scalar register instead of a literal operand
+  float a[W], acc[W];
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    a[k] = 1.0f + 1e-3f * (float)(threadIdx.x + k);
+    acc[k] = 0.f;
+  }
+  for (int it = 0; it < iters; it++) {
+    float d0[W], d1[W], d2[W], t[W];
+#pragma unroll
+    for (int k = 0; k < W; k++) d0[k] = a[k] - c0;
+#pragma unroll
+    for (int k = 0; k < W; k++) d1[k] = a[k] - c1;
+#pragma unroll
+    for (int k = 0; k < W; k++) d2[k] = c0 - a[k];
+#pragma unroll
+    for (int k = 0; k < W; k++) d0[k] = d0[k] * d0[k];
+#pragma unroll
+    for (int k = 0; k < W; k++) d1[k] = d1[k] * d1[k];
+#pragma unroll
+    for (int k = 0; k < W; k++) d2[k] = d2[k] * d2[k];
+#pragma unroll
+    for (int k = 0; k < W; k++) t[k] = d0[k] + d1[k];
+#pragma unroll
+    for (int k = 0; k < W; k++) t[k] = t[k] + d2[k];
+#pragma unroll
+    for (int k = 0; k < W; k++) t[k] = t[k] * c1;
+#pragma unroll
+    for (int k = 0; k < W; k++) t[k] = t[k] * l2e;
+#pragma unroll
+    for (int k = 0; k < W; k++) t[k] = __builtin_amdgcn_exp2f(t[k]);
+#pragma unroll
+    for (int k = 0; k < W; k++) acc[k] = __builtin_fmaf(t[k], c0, acc[k]);
+#pragma unroll
+    for (int k = 0; k < W; k++) asm volatile("" : "+v"(a[k]), "+v"(acc[k]));
+  }
+  float r = 0.f;
+#pragma unroll
+  for (int k = 0; k < W; k++) r += a[k] + acc[k];
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = r;
+}
+
+// Written-out instruction sequences (inline assembly, so the operands are what the text says): 8 blocks of 8 instructions
+// per round on 8 registers, SEQ selects the sequence.  64 counted instructions per round except SEQ 10 (96) and 11 (72).
+#define KEOPS_SEQ8(OP) asm volatile(OP(%0) OP(%1) OP(%2) OP(%3) OP(%4) OP(%5) OP(%6) OP(%7) \
+    : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7) : "v"(b0), "v"(b1), "v"(b2), "v"(b3), "s"(c0))
+#define KEOPS_OP_MUL_V(R) "v_mul_f32 " #R ", %8, " #R "\n"
+#define KEOPS_OP_MUL_S(R) "v_mul_f32 " #R ", %12, " #R "\n"
+#define KEOPS_OP_MUL_L(R) "v_mul_f32 " #R ", 0xbfb8aa3b, " #R "\n"
+#define KEOPS_OP_ADD_V(R) "v_add_f32 " #R ", %8, " #R "\n"
+#define KEOPS_OP_FMAC_V(R) "v_fmac_f32 " #R ", %8, %9\n"
+#define KEOPS_OP_FMA_V(R) "v_fma_f32 " #R ", " #R ", %8, %9\n"
+#define KEOPS_OP_MAX_V(R) "v_max_f32 " #R ", %8, " #R "\n"
+#define KEOPS_OP_MAX3_V(R) "v_max3_f32 " #R ", " #R ", %8, %9\n"
+#define KEOPS_OP_PERM_V(R) "v_perm_b32 " #R ", %8, " #R ", %9\n"
+#define KEOPS_OP_EXP(R) "v_exp_f32 " #R ", " #R "\n"
+template <int SEQ>
+static __global__ void __launch_bounds__(256) keops_valu_seq_loop(float* out, int iters, float c0) {
+  float a0 = threadIdx.x * 1e-3f + 1.f, a1 = a0 + 1, a2 = a0 + 2, a3 = a0 + 3, a4 = a0 + 4, a5 = a0 + 5, a6 = a0 + 6, a7 = a0 + 7;
+  float b0 = a0 * 0.5f, b1 = a1 * .5f, b2 = a2 * .5f, b3 = a3 * .5f;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      if (SEQ == 0) KEOPS_SEQ8(KEOPS_OP_MUL_V);
+      else if (SEQ == 1) KEOPS_SEQ8(KEOPS_OP_MUL_S);
+      else if (SEQ == 2) KEOPS_SEQ8(KEOPS_OP_MUL_L);
+      else if (SEQ == 3) KEOPS_SEQ8(KEOPS_OP_ADD_V);
+      else if (SEQ == 4) KEOPS_SEQ8(KEOPS_OP_FMAC_V);
+      else if (SEQ == 5) KEOPS_SEQ8(KEOPS_OP_FMA_V);
+      else if (SEQ == 6) KEOPS_SEQ8(KEOPS_OP_MAX_V);
+      else if (SEQ == 7) KEOPS_SEQ8(KEOPS_OP_PERM_V);
+      else if (SEQ == 8) KEOPS_SEQ8(KEOPS_OP_EXP);
+      else if (SEQ == 12) KEOPS_SEQ8(KEOPS_OP_MAX3_V);
+      else if (SEQ == 9)   // v_exp_f32 alternating with the v_fmac_f32 that consumes the exponential before the last one
+        asm volatile("v_exp_f32 %0, %0\n v_fmac_f32 %6, %8, %2\n v_exp_f32 %1, %1\n v_fmac_f32 %7, %8, %3\n"
+                     "v_exp_f32 %2, %2\n v_fmac_f32 %4, %8, %0\n v_exp_f32 %3, %3\n v_fmac_f32 %5, %8, %1\n"
+                     : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7) : "v"(b0));
+      else if (SEQ == 10)  // the Gaussian pair with every operation rounded on its own, as the general-purpose kernel compiles it
+        asm volatile("v_sub_f32 %4, %0, %8\n v_sub_f32 %5, %1, %9\n v_sub_f32 %6, %2, %10\n v_mul_f32 %4, %4, %4\n"
+                     "v_mul_f32 %5, %5, %5\n v_mul_f32 %6, %6, %6\n v_add_f32 %4, %4, %5\n v_add_f32 %4, %6, %4\n"
+                     "v_mul_f32 %4, %12, %4\n v_mul_f32 %4, 0xbfb8aa3b, %4\n v_exp_f32 %4, %4\n s_nop 0\n v_fmac_f32 %7, %11, %4\n"
+                     : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7)
+                     : "v"(b0), "v"(b1), "v"(b2), "v"(b3), "s"(c0));
+      else if (SEQ == 11)  // the contracted pair: 3 sub, 1 mul, 2 fmac, 1 mul, v_exp_f32, 1 fmac
+        asm volatile("v_sub_f32 %4, %0, %8\n v_sub_f32 %5, %1, %9\n v_sub_f32 %6, %2, %10\n v_mul_f32 %4, %4, %4\n"
+                     "v_fmac_f32 %4, %5, %5\n v_fmac_f32 %4, %6, %6\n v_mul_f32 %4, %12, %4\n v_exp_f32 %4, %4\n s_nop 0\n"
+                     "v_fmac_f32 %7, %11, %4\n"
+                     : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7)
+                     : "v"(b0), "v"(b1), "v"(b2), "v"(b3), "s"(c0));
+    }
+  }
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = a0 + a1 + a2 + a3 + a4 + a5 + a6 + a7;
+}
+
 typedef float keops_f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 keops_bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 keops_f16x8 __attribute__((ext_vector_type(8)));
@@ -365,6 +467,8 @@ static __global__ void __launch_bounds__(256) keops_mix_loop(float* out, int ite
 // instructions per round with `chains` v_fmac_f32 after each of them (0, 1, 2, 4, 8); kind 7: 32 matrix instructions
 // per round whose operands change with every instruction, `chains` = 0 bf16, 1 f16, 2 signed bytes; kind 8: the loop of
 // the signed-byte nearest-neighbour filter without memory traffic, `chains` = 0, 1, 2 (see keops_mfma_screen_loop);
+// kind 10: the Gaussian pair with separately rounded operations, `chains` chains side by side; kind 11: written-out
+// instruction sequences, `chains` = sequence of keops_valu_seq_loop;
 // kind 9: the contraction loop of the high-dimensional chunked kernel on its own (keops_stream_loop; workgroups of 8
 // wavefronts, `chains` = 0 constant / 1 random operands; out needs KEOPS_CALIBRATE_STREAM_BYTES more bytes).
 // chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
@@ -431,6 +535,25 @@ static int keops_calibrate_launch(int kind, int chains, int blocks, int iters, f
     else if (chains == 1) hipLaunchKernelGGL((keops_mfma_screen_loop<1>), g, b, 0, s, out, iters);
     else if (chains == 2) hipLaunchKernelGGL((keops_mfma_screen_loop<2>), g, b, 0, s, out, iters);
     else return (int)hipErrorInvalidValue;
+  } else if (kind == 11) {
+    // chains = the sequence of keops_valu_seq_loop
+    *instr_per_wave = (chains == 10 ? 96.0 : chains == 11 ? 72.0 : 64.0) * (double)iters;
+#define SEQ_CASE(Q) case Q: hipLaunchKernelGGL((keops_valu_seq_loop<Q>), g, b, 0, s, out, iters, 1.0009765625f); break
+    switch (chains) {
+      SEQ_CASE(0); SEQ_CASE(1); SEQ_CASE(2); SEQ_CASE(3); SEQ_CASE(4); SEQ_CASE(5); SEQ_CASE(6); SEQ_CASE(7); SEQ_CASE(8);
+      SEQ_CASE(9); SEQ_CASE(10); SEQ_CASE(11); SEQ_CASE(12);
+      default: return (int)hipErrorInvalidValue;
+    }
+#undef SEQ_CASE
+  } else if (kind == 10) {
+    // chains = chains advanced side by side: 1, 2, 4
+    *instr_per_wave = 12.0 * chains * (double)iters;
+#define ROUNDED_CASE(W, S) hipLaunchKernelGGL((keops_valu_rounded_loop<W, S>), g, b, 0, s, out, iters, 1.0009765625f, 0.99951171875f)
+    if (chains == 1) ROUNDED_CASE(1, 0); else if (chains == 2) ROUNDED_CASE(2, 0); else if (chains == 4) ROUNDED_CASE(4, 0);
+    else if (chains == 11) { ROUNDED_CASE(1, 1); *instr_per_wave = 12.0 * (double)iters; }
+    else if (chains == 12) { ROUNDED_CASE(2, 1); *instr_per_wave = 24.0 * (double)iters; }
+    else return (int)hipErrorInvalidValue;
+#undef ROUNDED_CASE
   } else if (kind == 5) {
     // chains = vector instructions per matrix instruction: 0, 1, 2, 4, 8
     *instr_per_wave = 8.0 * (double)iters;

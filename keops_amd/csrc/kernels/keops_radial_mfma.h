@@ -792,20 +792,29 @@ __device__ __forceinline__ void rad_sweep(const RadSweep& S, __bf16* ys, float* 
         }
     }
   }
-  // the 32 lanes of a half hold the same rows for different columns: shuffle sums, then one lane stores
+  // the 32 lanes of a half hold the same rows for different columns: shuffle sums; lane v of the half keeps the sum
+  // of row v, so that one store per row block covers its 32 rows
 #pragma unroll
-  for (int r = 0; r < RAD_RB; r++)
+  for (int r = 0; r < RAD_RB; r++) {
+    float keep[RAD_DV];
+#pragma unroll
+    for (int d = 0; d < RAD_DV; d++) keep[d] = 0.f;
 #pragma unroll
     for (int v = 0; v < 16; v++) {
-      const i64 i = r * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
 #pragma unroll
       for (int d = 0; d < RAD_DV; d++) {
         float s = acc[r][v][d];
 #pragma unroll
         for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o);
-        if (col == 0 && i < S.rows_store) S.part[i * RAD_DV + d] = s;
+        if (col == v) keep[d] = s;
       }
     }
+    const i64 i = r * 32 + 8 * (col >> 2) + 4 * half + (col & 3);
+    if (col < 16 && i < S.rows_store) {
+#pragma unroll
+      for (int d = 0; d < RAD_DV; d++) S.part[i * RAD_DV + d] = keep[d];
+    }
+  }
 }
 
 

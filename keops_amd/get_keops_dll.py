@@ -816,7 +816,7 @@ def match_radial(red, dtype, dtypeacc, sum_scheme, use_fast_math, map_reduce_id,
             return None
         if not block_sparse:
             pairs = batch_total
-    if pairs and int(pairs) < config.radial_min_pairs_log2:
+    if pairs and int(pairs) < (config.radial_ranges_min_pairs_log2 if "_ranges" in map_reduce_id else config.radial_min_pairs_log2):
         return None
     row_cat, col_cat = red.tagI, 1 - red.tagI
     # the factors of the product, signs and scalar constants pulled out
@@ -1087,7 +1087,7 @@ def get_keops_dll(
         rows_hint = nx if nx < 64 * 256 * config.block_size else None
     key = (map_reduce_id, repr(red), tuple(aliases), nargs, dtype, dtypeacc, sum_scheme_string, tag1D2D,
            use_fast_math, _rows_bucket(rows_hint), int(enable_chunks), bool(enable_finalchunks), int(batch_loop), int(pairs), int(batch_total),
-           binder.templates_digest(), bool(config.radial), float(config.radial_limit), float(config.radial_exact_frac), bool(config.radial_ranges), int(config.radial_mm_min_dv),
+           binder.templates_digest(), bool(config.radial), int(config.radial_min_pairs_log2), int(config.radial_ranges_min_pairs_log2), float(config.radial_limit), float(config.radial_exact_frac), bool(config.radial_ranges), int(config.radial_mm_min_dv),
            int(config.radial_mm_rb), int(config.radial_mm_terms), bool(config.radial_bilinear), bool(config.knn_i8), bool(use_half))
     with _lock:
         hit = _cache.get(key)

@@ -9,7 +9,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from . import binder
+from . import binder, config
 from .common.parse_type import parse_dtype_acc
 from .formulas.parse import parse_alias, parse_reduction
 from .get_keops_dll import get_keops_dll, plan_row_col_product
@@ -224,7 +224,8 @@ def load_keops_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_requ
     if pairs > 40:
         pairs = 0
     key = (tagCPUGPU, tag1D2D, tagHostDevice, bool(use_ranges), device_id_request, formula, tuple(aliases), nargs,
-           dtype, lang, tuple(sorted(optional_flags.items())), _rows_bucket(rows_hint), batch_loop, pairs, batch_total)
+           dtype, lang, tuple(sorted(optional_flags.items())), _rows_bucket(rows_hint), batch_loop, pairs, batch_total,
+           config.radial_min_pairs_log2, config.radial_ranges_min_pairs_log2)
     global last_loader
     obj = _loaders.get(key)
     if obj is None:

@@ -74,6 +74,25 @@ def test_large_rows_subset_and_exact_linearity():
     assert torch.equal(conv(xd, yd, bd, gd), got)          # and the result is reproducible bit for bit
 
 
+def test_long_all_positive_sums_stay_in_the_float32_class():
+    # 400 000 reduced rows, every term positive: the accumulation error cannot cancel, and a slab of the reduced
+    # axis spans several periods of the fold of the register tiles into the slab's partial sum
+    from keops_amd.torch import Genred
+
+    M, N, Dv = 4096, 400_000, 64
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.rand(M, 3, device="cuda", generator=gen)
+    y = torch.rand(N, 3, device="cuda", generator=gen)
+    b = torch.rand(N, Dv, device="cuda", generator=gen) + 0.5
+    g = torch.tensor([0.5], device="cuda")
+    got = Genred(FORMULA, _aliases(Dv), reduction_op="Sum", axis=1)(x, y, b, g)
+    assert _scheme_used("final")
+    rows = torch.arange(0, M, 16, device="cuda")
+    ref = torch.exp(-0.5 * torch.cdist(x[rows].double(), y.double()) ** 2) @ b.double()
+    rel = ((got[rows].double() - ref).abs() / ref).max().item()
+    assert rel <= 1e-5, rel          # measured 1.1e-6
+
+
 def test_axis0_gpu2d_and_gradient():
     from keops_amd.torch import Genred
 

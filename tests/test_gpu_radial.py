@@ -13,6 +13,15 @@ pytestmark = pytest.mark.gpu
 GAUSS = "Exp(-g*SqDist(x,y))*b"
 
 
+@pytest.fixture(autouse=True)
+def _scheme_from_2_to_the_28_pairs(monkeypatch):
+    """By default the scheme takes dense calls from 2**29 pairs on, where it is the faster one; the cases below are a
+    little above 2**28 pairs, which keeps their oracle comparisons short and exercises the same kernels."""
+    from keops_amd import config
+
+    monkeypatch.setattr(config, "radial_min_pairs_log2", 29)
+
+
 def _genred(D, Dv, axis=1, **kw):
     from keops_amd.torch import Genred
 
@@ -65,6 +74,20 @@ def test_gaussian_sums_with_matrix_core_exponents_vs_oracle(D, Dv, M, N):
     # exact linearity in the weights, deterministic from call to call
     assert torch.equal(_genred(D, Dv)(dev[0], dev[1], 2 * dev[2], dev[3]), 2 * got)
     assert torch.equal(_genred(D, Dv)(*dev), got)
+
+
+def test_default_threshold_of_the_scheme(monkeypatch):
+    from keops_amd import config
+
+    monkeypatch.setattr(config, "radial_min_pairs_log2", 30)      # the library's default
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for n, served in ((17000, None), (24000, "1")):                # 2**28.1 and 2**29.1 pairs
+        x, y = torch.randn(n, 3, device="cuda", generator=gen), torch.randn(n, 3, device="cuda", generator=gen)
+        b, g = torch.randn(n, 1, device="cuda", generator=gen), torch.tensor([0.7], device="cuda")
+        got = _genred(3, 1)(x, y, b, g)
+        assert _last_meta("radial") == served
+        ref = torch.exp(-0.7 * torch.cdist(x[:512].double(), y.double()) ** 2) @ b.double()
+        assert torch.allclose(got[:512].double(), ref, rtol=0, atol=1e-5 * float(ref.abs().max()))
 
 
 def test_reduction_over_i_and_formula_spellings():
