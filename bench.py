@@ -308,14 +308,16 @@ def calibration(mfma):
          (1, 2, 4)),
         (11, "written-out sequences, 8 wavefronts per SIMD (chains = sequence: 0 v_mul vgpr, 1 v_mul sgpr operand, 2 v_mul "
              "literal, 3 v_add, 4 v_fmac, 5 v_fma three registers, 6 v_max, 7 v_perm_b32, 8 v_exp_f32, 9 v_exp_f32 alternating "
-             "with v_fmac, 10 rounded Gaussian pair (12 instr), 11 contracted pair (9 instr), 12 v_max3)", tuple(range(13)))]
+             "with v_fmac, 10 rounded Gaussian pair (12 instr), 11 contracted pair (9 instr), 12 v_max3)", tuple(range(13))),
+        (12, "stream of the Gaussian sweep alone: 4 v_mfma_f32_32x32x16_bf16 per 32 pairs, v_exp_f32 and `chains` v_fmac_f32 "
+             "per pair; the rate counts pairs (v_exp_f32)", (1, 4, 8))]
     for kind, label, chain_set in kinds:
         for chains in chain_set:
             # one workgroup = 4 wavefronts = one per SIMD of a CU (kind 9: 8 wavefronts, at most two workgroups per CU)
-            wg_waves = 8 if kind == 9 else 4
-            for wgs in ((1, 2) if kind == 9 else (8,) if kind == 11 else (1, 2, 4)):
+            wg_waves = 8 if kind in (9, 12) else 4
+            for wgs in ((1, 2) if kind in (9, 12) else (8,) if kind == 11 else (1, 2, 4)):
                 blocks, waves = cus * wgs, wgs * wg_waves // 4
-                iters = {7: 12_500, 8: 100_000, 5: 50_000, 9: 4_000, 11: 20_000}.get(kind) or (200_000 if kind < 3 or kind == 10 else 100_000) // chains
+                iters = {7: 12_500, 8: 100_000, 5: 50_000, 9: 4_000, 11: 20_000, 12: 20_000}.get(kind) or (200_000 if kind < 3 or kind == 10 else 100_000) // chains
                 ms, ipw = binder.calibrate(kind, chains, blocks, iters)
                 total = ipw * blocks * wg_waves  # wavefront instructions
                 per_cycle = total / (ms * 1e-3) / simds / clock
@@ -327,6 +329,7 @@ def calibration(mfma):
                     row["PFLOP_per_s"] = round(total * 32 * 32 * depth * 2 / (ms * 1e-3) / 1e15, 3)
                 else:
                     row["lane_instr_per_s"] = total * 64 / (ms * 1e-3)
+                    row["ns_per_wave_instr_and_simd"] = round(ms * 1e6 / (total / simds), 4)
                 rows.append(row)
     return {"calibration": "mfma" if mfma else "valu", "cus": cus, "rows": rows}
 

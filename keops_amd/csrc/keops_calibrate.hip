@@ -156,6 +156,50 @@ typedef float keops_f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 keops_bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 keops_f16x8 __attribute__((ext_vector_type(8)));
 
+// The instruction stream of the Gaussian sweep on its own: per round four v_mfma_f32_32x32x16_bf16 (two exponent tiles of
+// two k blocks) and, for each of their 32 results, v_exp_f32 and NF v_fmac_f32 (NF accumulated components per pair);
+// no memory traffic.  Workgroups of 8 wavefronts, as the sweep's.
+template <int NF>
+static __global__ void __launch_bounds__(512, 2) keops_sweep_stream_loop(float* out, int iters, float w0) {
+  keops_bf16x8 a, b, a2, b2;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    a[e] = (__bf16)(1.0f + 0.01f * (float)(threadIdx.x + e));
+    b[e] = (__bf16)(0.5f - 0.001f * (float)e);
+    a2[e] = (__bf16)(0.7f + 0.02f * (float)(threadIdx.x + e));
+    b2[e] = (__bf16)(0.25f - 0.002f * (float)e);
+  }
+  float s[4][NF], w[NF];
+#pragma unroll
+  for (int d = 0; d < NF; d++) {
+    w[d] = w0 + (float)d;
+#pragma unroll
+    for (int e = 0; e < 4; e++) s[e][d] = 0.f;
+  }
+  keops_f32x16 z;
+#pragma unroll
+  for (int e = 0; e < 16; e++) z[e] = -1.0f * (float)e;
+  for (int it = 0; it < iters; it++) {
+    keops_f32x16 t0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, z, 0, 0, 0);
+    t0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, a, t0, 0, 0, 0);
+    keops_f32x16 t1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, b2, z, 0, 0, 0);
+    t1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b2, a2, t1, 0, 0, 0);
+#pragma unroll
+    for (int e = 0; e < 32; e++) {
+      const float x = __builtin_amdgcn_exp2f(e < 16 ? t0[e & 15] : t1[e & 15]);
+#pragma unroll
+      for (int d = 0; d < NF; d++) s[e & 3][d] = __builtin_fmaf(x, w[d], s[e & 3][d]);
+    }
+    asm volatile("" : "+v"(a), "+v"(b), "+v"(a2), "+v"(b2), "+v"(z));
+  }
+  float r = 0.f;
+#pragma unroll
+  for (int e = 0; e < 4; e++)
+#pragma unroll
+    for (int d = 0; d < NF; d++) r += s[e][d];
+  out[(size_t)blockIdx.x * 512 + threadIdx.x] = r;
+}
+
 // `iters` rounds of CHAINS independent v_mfma_f32_32x32x16_bf16 (HALF = 0) or _f16 (HALF = 1) accumulation chains per
 // wavefront; the operands carry full-width random significands (the power drawn, hence the sustained clock,
 // depends on the data)
@@ -468,7 +512,8 @@ static __global__ void __launch_bounds__(256) keops_mix_loop(float* out, int ite
 // per round whose operands change with every instruction, `chains` = 0 bf16, 1 f16, 2 signed bytes; kind 8: the loop of
 // the signed-byte nearest-neighbour filter without memory traffic, `chains` = 0, 1, 2 (see keops_mfma_screen_loop);
 // kind 10: the Gaussian pair with separately rounded operations, `chains` chains side by side; kind 11: written-out
-// instruction sequences, `chains` = sequence of keops_valu_seq_loop;
+// instruction sequences, `chains` = sequence of keops_valu_seq_loop; kind 12: the Gaussian sweep's stream (matrix
+// instructions, v_exp_f32 and `chains` v_fmac_f32 per pair);
 // kind 9: the contraction loop of the high-dimensional chunked kernel on its own (keops_stream_loop; workgroups of 8
 // wavefronts, `chains` = 0 constant / 1 random operands; out needs KEOPS_CALIBRATE_STREAM_BYTES more bytes).
 // chains: 1, 2, 4 or 8 (vector), 1, 2 or 4 (matrix).
@@ -535,6 +580,14 @@ static int keops_calibrate_launch(int kind, int chains, int blocks, int iters, f
     else if (chains == 1) hipLaunchKernelGGL((keops_mfma_screen_loop<1>), g, b, 0, s, out, iters);
     else if (chains == 2) hipLaunchKernelGGL((keops_mfma_screen_loop<2>), g, b, 0, s, out, iters);
     else return (int)hipErrorInvalidValue;
+  } else if (kind == 12) {
+    // chains = accumulated components per pair (1, 4, 8); workgroups of 8 wavefronts; counted: the v_exp_f32 (32 per round)
+    *instr_per_wave = 32.0 * (double)iters;
+    const dim3 b8(512);
+    if (chains == 1) hipLaunchKernelGGL((keops_sweep_stream_loop<1>), g, b8, 0, s, out, iters, 1.0009765625f);
+    else if (chains == 4) hipLaunchKernelGGL((keops_sweep_stream_loop<4>), g, b8, 0, s, out, iters, 1.0009765625f);
+    else if (chains == 8) hipLaunchKernelGGL((keops_sweep_stream_loop<8>), g, b8, 0, s, out, iters, 1.0009765625f);
+    else return (int)hipErrorInvalidValue;
   } else if (kind == 11) {
     // chains = the sequence of keops_valu_seq_loop
     *instr_per_wave = (chains == 10 ? 96.0 : chains == 11 ? 72.0 : 64.0) * (double)iters;
@@ -572,7 +625,7 @@ extern "C" int keops_calibrate(int device_id, int kind, int chains, int blocks, 
   if (!ms || !instr_per_wave || blocks <= 0 || iters <= 0) return -1;
   if (hipSetDevice(device_id < 0 ? 0 : device_id) != hipSuccess) return -2;
   float* out = nullptr;
-  if (hipMalloc((void**)&out, (size_t)blocks * 256 * sizeof(float) + KEOPS_CALIBRATE_STREAM_BYTES) != hipSuccess) return -3;
+  if (hipMalloc((void**)&out, (size_t)blocks * 512 * sizeof(float) + KEOPS_CALIBRATE_STREAM_BYTES) != hipSuccess) return -3;
   hipEvent_t e0 = nullptr, e1 = nullptr;
   int rc = 0;
   auto cleanup = [&] { if (e0) (void)hipEventDestroy(e0); if (e1) (void)hipEventDestroy(e1); (void)hipFree(out); };
