@@ -21,10 +21,10 @@ def _gauss_inputs(M, N, Dv, seed, dtype=np.float32):
     return x, y, b, np.array([1.0], dtype)
 
 
-def _genred_gauss(Dv, **kw):
+def _genred_gauss(Dv, D=3, **kw):
     from keops_amd.torch import Genred
 
-    return Genred(GAUSS, ["x=Vi(3)", "y=Vj(3)", f"b=Vj({Dv})", "g=Pm(1)"], reduction_op="Sum", axis=1, **kw)
+    return Genred(GAUSS, [f"x=Vi({D})", f"y=Vj({D})", f"b=Vj({Dv})", "g=Pm(1)"], reduction_op="Sum", axis=1, **kw)
 
 
 def test_config1_gaussian_10k_full_parity():
@@ -117,6 +117,9 @@ def test_sum_schemes(scheme):
     got = _genred_gauss(2, sum_scheme=scheme)(*to_dev(x, y, b, g)).cpu().numpy()
     ref = cpu_reduc("gauss", [x, y, b, g], M, N, 2, scheme=scheme)
     scale = cpu_reduc("gauss", [x, y, np.abs(b), g], M, N, 2)
+    # direct_sum: the oracle adds a row's 40 000 terms one after the other in float32, the kernel adds them in column
+    # slabs and tiles; two orders of an uncompensated float32 sum of that length differ by about sqrt(N) 2^-24 = 1.2e-5
+    # of sum |F_ij| whatever the kernel does, so the bar for this scheme is the sum's own accuracy
     assert_sum_parity(got, ref, scale, tol=1e-5 if scheme != "direct_sum" else 5e-5)
 
 
@@ -126,6 +129,21 @@ def test_no_fast_math_matches_libm_closely():
     got = _genred_gauss(1, use_fast_math=False)(*to_dev(x, y, b, g)).cpu().numpy()
     ref = cpu_reduc("gauss", [x, y, b, g], M, N, 1)
     assert rel_l2(got, ref) <= 2e-6
+
+
+def test_denormal_kernel_values_are_flushed_with_fast_math_and_kept_without():
+    """exp(-d^2) for d = 9.4 ... 10: values of 4e-39 ... 4e-44, below the smallest normal float32.  v_exp_f32 returns
+    zero there, as the reference's GPU build does under its default -use_fast_math (which implies -ftz=true,
+    keopscore/binders/nvrtc/nvrtc_jit.cpp:87-88); use_fast_math=False calls the library exponential."""
+    x = torch.zeros(4, 1, device="cuda")
+    y = torch.tensor([[9.4], [9.6], [9.8], [10.0]], device="cuda")
+    b, g = torch.ones(4, 1, device="cuda"), torch.tensor([1.0], device="cuda")
+    truth = float(torch.exp(-(y.double() ** 2)).sum())
+    assert 4e-39 < truth < 5e-39
+    fast = _genred_gauss(1, D=1)(x, y, b, g)
+    assert float(fast.abs().max()) == 0.0
+    kept = _genred_gauss(1, D=1, use_fast_math=False)(x, y, b, g)
+    assert abs(float(kept[0]) - truth) <= 1e-5 * truth + 2e-45      # one unit of the denormal grid
 
 
 @pytest.mark.parametrize("backend", ["GPU_1D", "GPU_2D", "GPU"])
