@@ -349,8 +349,15 @@ def measure(workload, steps, warmup):
     for _ in range(max(1, warmup)):
         step()
     torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+
     # kernel-only time: HIP events recorded by the library around the launch, on the launch stream; only the
-    # modules this workload loaded are asked
+    # modules this workload loaded are asked.  Taken right behind the timed steps, so that both figures see the same
+    # clocks (a pass that waits for its events after a pause runs up to a tenth slower on the short workloads)
     mods = [m for m in kernel_modules() if id(m) not in before] or kernel_modules()
     for m in mods:
         m.set_timing(True)
@@ -361,12 +368,6 @@ def measure(workload, steps, warmup):
     for m in mods:
         m.set_timing(False)
     torch.cuda.synchronize()
-
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / steps
 
     kms = sum(kernel_ms) / len(kernel_ms)
     achieved = pairs * flop_per_pair / (kms * 1e-3) / 1e12
