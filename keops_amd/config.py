@@ -105,6 +105,8 @@ final_split3 = os.environ.get("KEOPS_AMD_FINAL_SPLIT3", "1") != "0"          # p
 # to 2^-17 each, 2.4e-6 rms: not the float32 class; C5b 68.8 against 70.6 ms, softmax_d64 4.70 against 5.09 ms)
 final_weight_terms = int(os.environ.get("KEOPS_AMD_FINAL_WEIGHT_TERMS", 3))
 final_period = int(os.environ.get("KEOPS_AMD_FINAL_PERIOD", 16384))        # block-sum period in reduced rows
+# ... when the sums are kept in double (dtype_acc = float64, Kahan scheme): 64 matrix-instruction accumulations per fold
+final_period_acc64 = int(os.environ.get("KEOPS_AMD_FINAL_PERIOD_ACC64", 1024))
 
 # matrix-core KNN kernel (csrc/kernels/keops_knn_mfma.h)
 knn_min_dim = int(os.environ.get("KEOPS_AMD_KNN_MIN_DIM", 2))         # smallest vector dimension served by the matrix-core KNN scheme

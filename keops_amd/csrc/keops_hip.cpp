@@ -1353,11 +1353,14 @@ int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   const bool split3_kernel = m.meta_int("fin_split3", 0) != 0;  // three-term kernel; dense launches pre-split v
   const bool split3 = !rg && split3_kernel;
   const int64_t DVP = (DV + 31) / 32 * 32, ntiles = (ny + TJ - 1) / TJ;
-  const size_t part_bytes = nslabs > 1 ? align_up((size_t)nslabs * nx * DV * 4, 256) : 0;
+  // sums kept in double (meta fin_acc64): the folds always go to the partial buffer, keops_fin_reduce rounds once
+  const bool acc64 = m.meta_int("fin_acc64", 0) != 0;
+  if (acc64 && rg) return fail(-1, "corrupt final-product module metadata");
+  const size_t part_bytes = (nslabs > 1 || acc64) ? align_up((size_t)nslabs * nx * DV * (acc64 ? 8 : 4), 256) : 0;
   const size_t split_bytes = split3 ? (size_t)ntiles * 3 * DVP * TJ * 2 : 0;
   if (part_bytes + split_bytes > 0) {
     if (int rc = m.partial.reserve(part_bytes + split_bytes)) return rc;
-    if (nslabs > 1) h.partial = m.partial.ptr;
+    if (nslabs > 1 || acc64) h.partial = m.partial.ptr;
     if (split3) h.vsplit = (char*)m.partial.ptr + part_bytes;
   }
   std::vector<char> buf(sizeof(FinHeader) + sizeof(void*) * (size_t)std::max(1, m.nargs));
@@ -1370,7 +1373,7 @@ int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
   if (int rc = launch_raw3(m, split3_kernel ? "keops_fin_main3" : "keops_fin_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)NZ, (unsigned)m.block, buf.data(), buf.size(), stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
-  if (nslabs > 1) {
+  if (nslabs > 1 || acc64) {
     const int64_t gb = (nx * DV + 255) / 256;
     if (int rc = launch_raw(m, "keops_fin_reduce", (unsigned)gb, 1, 256, buf.data(), buf.size(), stream)) return rc;
   }

@@ -18,13 +18,19 @@
 //     output rows (owned by this workgroup, plain read-modify-write) and cleared, so rounding
 //     errors do not grow with the number of reduced rows;
 //   * few output rows: the reduced axis is cut in slabs (blockIdx.y) with one partial output per
-//     slab, summed in slab order by keops_fin_reduce (deterministic).
+//     slab, summed in slab order by keops_fin_reduce (deterministic);
+//   * FIN_ACC64 (dtype_acc = float64, or the Kahan scheme, whose compensated float32 sum this replaces): the folds
+//     and the slab sum run in double on a buffer of their own, with a short FIN_PERIOD, and keops_fin_reduce rounds
+//     once to float32 (sum_schemes.py:44-71 with a double accumulator).
 //
-// The plug-in defines: T (float), KEOPS_NARGS, FIN_DV, FIN_VARG, FIN_NB, FIN_WAVES, FIN_TJ,
+// The plug-in defines: T (float), TACC (float, double with FIN_ACC64), KEOPS_NARGS, FIN_DV, FIN_VARG, FIN_NB, FIN_WAVES, FIN_TJ,
 // FIN_PERIOD, FIN_BLOCKSUM, the KEOPS_DIM* macros and row/col/par variable tables of the scalar
 // kernel f, and KeopsFormula::eval(xi, yj, p, fout[1]).
 #pragma once
 #include "keops_common.h"
+#ifndef FIN_ACC64
+#define FIN_ACC64 0
+#endif
 
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float fin_f32x16;
 
@@ -37,7 +43,7 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float fin_f32x16;
 struct FinParams {
   i64 nx, ny;
   T* out;          // [nx][FIN_DV]
-  T* partial;      // [nslabs][nx][FIN_DV] when nslabs > 1
+  TACC* partial;   // [nslabs][nx][FIN_DV] when nslabs > 1, and always when the sums are kept in double (FIN_ACC64)
   i64 slab_len;    // reduced rows per slab (multiple of FIN_TJ)
   int nslabs;
   int pad_;
@@ -84,12 +90,12 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[b][r] = 0.f;
 
-  T* dst = P.nslabs > 1 ? P.partial + (i64)blockIdx.y * P.nx * FIN_DV : P.out;
+  TACC* dst = (P.nslabs > 1 || FIN_ACC64) ? P.partial + (i64)blockIdx.y * P.nx * FIN_DV : reinterpret_cast<TACC*>(P.out);
   bool first = true;
   // folds the register tiles into the output rows of this wavefront and clears them
   auto fold = [&]() {
     const i64 ibase = row0 + 4 * half;
-    T* o = dst + ibase * FIN_DV + c0 + col;
+    TACC* o = dst + ibase * FIN_DV + c0 + col;
     // folds are rare: keep their address arithmetic here instead of in registers across the sweep
     asm volatile("" : "+v"(o));
 #pragma unroll
@@ -99,8 +105,8 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main(const Fin
       for (int r = 0; r < 16; r++) {
         const int ir = 8 * (r >> 2) + (r & 3);
         if (ibase + ir < G.row_end && d < FIN_DV) {
-          T* oo = o + (i64)ir * FIN_DV + 32 * b;
-          *oo = first ? acc[b][r] : *oo + acc[b][r];
+          TACC* oo = o + (i64)ir * FIN_DV + 32 * b;
+          *oo = first ? (TACC)acc[b][r] : *oo + (TACC)acc[b][r];
         }
         acc[b][r] = 0.f;
       }
@@ -204,9 +210,9 @@ extern "C" __global__ void __launch_bounds__(256) keops_fin_reduce(const FinPara
   const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;
   const i64 total = P.nx * FIN_DV;
   if (e >= total) return;
-  T s = P.partial[e];
+  TACC s = P.partial[e];
   for (int k = 1; k < P.nslabs; k++) s += P.partial[(i64)k * total + e];
-  P.out[e] = s;
+  P.out[e] = (T)s;
 }
 
 #if KEOPS_MC_RANGES
@@ -295,12 +301,12 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[b][r] = 0.f;
 
-  T* dst = P.nslabs > 1 ? P.partial + (i64)blockIdx.y * P.nx * FIN_DV : P.out;
+  TACC* dst = (P.nslabs > 1 || FIN_ACC64) ? P.partial + (i64)blockIdx.y * P.nx * FIN_DV : reinterpret_cast<TACC*>(P.out);
   bool first = true;
   // folds the register tiles into the output rows of this wavefront and clears them
   auto fold = [&]() {
     const i64 ibase = row0 + 4 * half;
-    T* o = dst + ibase * FIN_DV + c0 + col;
+    TACC* o = dst + ibase * FIN_DV + c0 + col;
     asm volatile("" : "+v"(o));
 #pragma unroll
     for (int b = 0; b < FIN_NB; b++) {
@@ -309,8 +315,8 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
       for (int r = 0; r < 16; r++) {
         const int ir = 8 * (r >> 2) + (r & 3);
         if (ibase + ir < G.row_end && d < FIN_DV) {
-          T* oo = o + (i64)ir * FIN_DV + 32 * b;
-          *oo = first ? acc[b][r] : *oo + acc[b][r];
+          TACC* oo = o + (i64)ir * FIN_DV + 32 * b;
+          *oo = first ? (TACC)acc[b][r] : *oo + (TACC)acc[b][r];
         }
         acc[b][r] = 0.f;
       }

@@ -692,9 +692,12 @@ def match_final(red, dtype, dtypeacc, sum_scheme, map_reduce_id, use_fast_math=T
     from .formulas import ops as O
     from .formulas.reductions import KIND_SUM
 
-    if red.kind != KIND_SUM or dtype != "float" or dtypeacc != "float" or not use_fast_math:
+    if red.kind != KIND_SUM or dtype != "float" or dtypeacc not in ("float", "double") or not use_fast_math:
         return None
-    if sum_scheme not in ("block_sum", "direct_sum"):
+    if sum_scheme not in ("block_sum", "direct_sum", "kahan_scheme"):
+        return None
+    # sums kept in double (dtype_acc = float64; the Kahan scheme is served the same way): dense launches only
+    if (dtypeacc == "double" or sum_scheme == "kahan_scheme") and "_ranges" in map_reduce_id:
         return None
     F = red.formula
     if F.name != "Mult" or len(F.children) != 2:
@@ -709,10 +712,12 @@ def match_final(red, dtype, dtypeacc, sum_scheme, map_reduce_id, use_fast_math=T
     return None
 
 
-def generate_final_plugin(red, match, sum_scheme, nargs, irregular=False):
+def generate_final_plugin(red, match, sum_scheme, nargs, irregular=False, acc64=False):
     """Module source for the matrix-core final-product scheme (kernels/keops_final_mfma.h); ``irregular``: the
-    block-sparse / batched variant (GpuReduc1D_ranges_finalchunks.py:20-91)."""
+    block-sparse / batched variant (GpuReduc1D_ranges_finalchunks.py:20-91); ``acc64``: the register tiles are folded
+    into double sums every ``config.final_period_acc64`` reduced rows."""
     f, vvar = match
+    acc64 = bool(acc64) and not irregular
 
     class _Inner:  # what VarLayout needs: the scalar kernel with the reduction's orientation
         formula, tagI = f, red.tagI
@@ -732,16 +737,18 @@ def generate_final_plugin(red, match, sum_scheme, nargs, irregular=False):
     ca, cd, co = VarLayout.table(layout.colvars)
     pa, pd, po = VarLayout.table(layout.parvars)
     meta = dict(scheme="final", block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
-                sizeof_acc=4, nrowvars=len(layout.rowvars), ncolvars=len(layout.colvars) + (0 if vvar in layout.colvars else 1),
+                sizeof_acc=8 if acc64 else 4, nrowvars=len(layout.rowvars), ncolvars=len(layout.colvars) + (0 if vvar in layout.colvars else 1),
                 nparvars=len(layout.parvars), fin_dv=vvar.dim, fin_nb=nb, fin_nz=nz, fin_qb=32 * waves, ranges=int(irregular),
+                fin_acc64=int(acc64),
                 fin_split3=int(config.final_split3 and tj % 16 == 0),
                 nops=L.count_ops(outs))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
-           "typedef float T;\ntypedef float TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
+           f"typedef float T;\ntypedef {'double' if acc64 else 'float'} TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
            '#include "keops_common.h"']
     defs = dict(
         KEOPS_NARGS=nargs, FIN_DV=vvar.dim, FIN_VARG=vvar.ind, FIN_NB=nb, FIN_WAVES=waves, FIN_TJ=tj,
-        FIN_PERIOD=config.final_period, FIN_BLOCKSUM=int(sum_scheme == "block_sum"),
+        FIN_PERIOD=config.final_period_acc64 if acc64 else config.final_period,
+        FIN_BLOCKSUM=int(sum_scheme == "block_sum" or acc64), FIN_ACC64=int(acc64),
         FIN_SPLIT3=int(config.final_split3 and tj % 16 == 0),
         KEOPS_DIMX=layout.dimx, KEOPS_DIMY=layout.dimy, KEOPS_DIMY_PAD=dimy_pad, KEOPS_DIMP=layout.dimp,
         KEOPS_NROWVARS=len(layout.rowvars), KEOPS_NCOLVARS=len(layout.colvars), KEOPS_NPARVARS=len(layout.parvars),
@@ -1132,7 +1139,8 @@ def get_keops_dll(
             source, meta = generate_knn_plugin(red_k, knn[0], knn[1], nargs, block_sparse=(irregular and (batch_loop == -1 or knn_batches)))
             use_chunk_mode = 3  # matrix-core filter scheme (no counterpart among the reference's chunk modes)
         elif fin is not None:
-            source, meta = generate_final_plugin(red, fin, sum_scheme_string, nargs, irregular=irregular)
+            source, meta = generate_final_plugin(red, fin, sum_scheme_string, nargs, irregular=irregular,
+                                                 acc64=(dtypeacc == "double" or sum_scheme_string == "kahan_scheme"))
             use_chunk_mode = 2  # as the reference's final-chunk mode (get_keops_dll.py:101-108)
         elif chk is not None:
             source, meta = generate_chunk_plugin(red, chk, dtypeacc, sum_scheme_string, nargs, irregular=irregular,
