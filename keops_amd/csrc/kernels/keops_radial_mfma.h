@@ -616,7 +616,8 @@ __device__ __forceinline__ float rad_exp_of(float coef, float s) {
   const float th = u * 1.44269502162933349609375f;
   const float tl = __builtin_fmaf(u, 1.925963033500011e-08f, __builtin_fmaf(u, 1.44269502162933349609375f, -th));
   const float e = __builtin_amdgcn_exp2f(th);
-  return __builtin_fmaf(e, tl * 0.693147180559945f, e);
+  // (an infinite argument leaves tl undefined: exp2 has already given 0 or infinity)
+  return (e > 0.f && e < __builtin_inff()) ? __builtin_fmaf(e, tl * 0.693147180559945f, e) : e;
 }
 
 // squared distance in the reference's operation order (difference, square, sequential sum; no contraction)

@@ -234,6 +234,51 @@ def test_one_far_outlier_in_a_large_cloud_keeps_the_matrix_core_path():
     assert_sum_parity(got[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, scale)
 
 
+@pytest.mark.parametrize("case", ["nan_row", "inf_row", "huge_row", "inf_column", "huge_column", "nan_column", "nan_weight"])
+def test_values_that_are_not_finite_or_huge_behave_as_on_the_general_purpose_kernel(case):
+    """The reference's loops give a NaN or infinite coordinate of x_i to row i alone, an infinite or huge y_j a kernel
+    value of zero in every row, a NaN in y_j or b_j to every row: the sort, the centre and the device-side choice of
+    the matrix-core family must not change that."""
+    M, N, Dv = 17000, 16500, 2
+    gen = torch.Generator(device="cuda").manual_seed(12)
+    x, y = torch.randn(M, 3, device="cuda", generator=gen), torch.randn(N, 3, device="cuda", generator=gen)
+    b, g = torch.randn(N, Dv, device="cuda", generator=gen), torch.tensor([0.7], device="cuda")
+    if case == "nan_row":
+        x[4321, 1] = float("nan")
+    elif case == "inf_row":
+        x[4321, 1] = float("inf")
+    elif case == "huge_row":
+        x[4321, 1] = 3e19          # its square overflows float32
+    elif case == "inf_column":
+        y[1234, 2] = float("-inf")
+    elif case == "huge_column":
+        y[1234, 2] = 1e30
+    elif case == "nan_column":
+        y[1234, 0] = float("nan")
+    else:
+        b[1234, 1] = float("nan")
+    got = _genred(3, Dv)(x, y, b, g)
+    assert _last_meta("radial") == "1"
+    want = _plain(3, Dv)(x, y, b, g)
+    assert _last_meta("radial") is None
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    ok = ~torch.isnan(want)
+    if case in ("nan_row", "inf_row", "huge_row"):
+        assert int((~ok).any(dim=1).sum()) == (1 if case == "nan_row" else 0) and bool(ok[:4321].all()) and bool(ok[4322:].all())
+        if case != "nan_row":
+            assert float(got[4321].abs().max()) == 0.0     # exp(-inf): no neighbour
+    elif case in ("inf_column", "huge_column"):
+        assert bool(ok.all())
+    elif case == "nan_column":
+        assert not bool(ok.any())
+    else:
+        assert not bool(ok[:, 1].any()) and bool(ok[:, 0].all())
+    if ok.any():
+        scale = _plain(3, Dv)(x, y, torch.nan_to_num(b).abs(), g)
+        err = ((got - want).abs() / scale.clamp_min(1e-30))[ok]
+        assert float(err.max()) <= 1e-5
+
+
 @pytest.mark.parametrize("D,Dv,M,N,ratio,offset", [
     (7, 23, 24918, 13490, 0.101, 0.0),     # every live term of a row has an exponent of -50 ... -87
     (8, 20, 16004, 18283, 0.0448, 30.0),
