@@ -343,6 +343,9 @@ extern "C" __global__ void __launch_bounds__(256) keops_radr_decide(const RadRPa
       ry = ry < reach ? ry : reach;
     }
     if (!(ak * (rx2 + ry * ry) <= (float)RAD_LIMIT)) mine = 1;  // also for NaN
+    // a column so far out that the terms of its exponent overflow (they would cancel to NaN instead of a large negative
+    // number): the general-purpose kernel gives such pairs their zero
+    if (!(ak * ry2 <= 1e30f)) mine = 1;
   }
   bad[threadIdx.x] = mine;
   __syncthreads();

@@ -69,6 +69,34 @@ def test_block_sparse_gaussian_sums_on_the_matrix_cores_vs_oracle(D, Dv, sigma):
     assert torch.equal(conv(dev[0], dev[1], 2 * dev[2], dev[3], ranges=rd), 2 * got)   # exact linearity in b
 
 
+@pytest.mark.parametrize("case", ["inf_row", "nan_row", "huge_column"])
+def test_values_that_are_not_finite_or_huge_send_the_call_to_the_general_purpose_kernel(case):
+    """A row range that holds an infinite, NaN or huge coordinate fails the per-range check (its largest centred norm is
+    not finite, or far beyond the bound), so the general-purpose kernel serves the call: NaN where the reference's
+    loops give NaN and nowhere else."""
+    D, Dv = 3, 2
+    c, x, y, b, rx, ry = _clusters(D, Dv, 64, 23)
+    g = np.array([100.0], np.float32)
+    ranges, keep = _pattern(c, rx, ry)
+    i, j = int(rx[7, 0]) + 5, int(ry[9, 0]) + 3
+    if case == "inf_row":
+        x[i, 1] = np.inf
+    elif case == "nan_row":
+        x[i, 1] = np.nan
+    else:
+        y[j, 2] = 1e30
+    dev = to_dev(x, y, b, g)
+    rd = tuple(r.cuda() for r in ranges)
+    conv = _genred(D, Dv)
+    for _ in range(2):                                  # host-validated launch, then device-built tables
+        got = conv(*dev, ranges=rd)
+        assert _module().meta("rad_ranges") == "1" and _module().path_status() == 0
+        want = _genred(D, Dv, enable_chunks=False)(*dev, ranges=rd)
+        assert torch.equal(torch.isnan(got), torch.isnan(want))
+        assert int(torch.isnan(want).any(dim=1).sum()) == (1 if case == "nan_row" else 0)
+        assert torch.equal(torch.nan_to_num(got), torch.nan_to_num(want))
+
+
 def test_reduction_over_i_uses_the_last_three_ranges():
     D, Dv = 3, 2
     c, x, y, a, rx, ry = _clusters(D, Dv, 64, 5)
