@@ -41,6 +41,9 @@ chunk_min_dim = int(os.environ.get("KEOPS_AMD_CHUNK_MIN_DIM", 24))    # smallest
 # K-nearest-neighbour reductions with block-sparse ranges on the matrix-core scheme (0: the general-purpose ranges kernel)
 knn_ranges = os.environ.get("KEOPS_AMD_KNN_RANGES", "1") != "0"
 chunk_near = os.environ.get("KEOPS_AMD_CHUNK_NEAR", "auto")
+# squared distances on the matrix cores: operand scale from the bulk of the rows when a few rows hold components far
+# beyond the others', those rows (and rows with values that are not finite) computed pair by pair from the float32 data
+chunk_robust = os.environ.get("KEOPS_AMD_CHUNK_ROBUST", "1") != "0"
 # float64 contractions on the float64 matrix instruction (csrc/kernels/keops_chunk_f64.h)
 chunk64 = os.environ.get("KEOPS_AMD_CHUNK64", "1") != "0"
 chunk64_min_dim = int(os.environ.get("KEOPS_AMD_CHUNK64_MIN_DIM", 32))

@@ -1153,7 +1153,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
                            : "this module was compiled for float32 data: a use_half launch needs the module that get_keops_dll "
                              "returns for use_half = 1");
   const size_t o_xs = take((size_t)nxs * DP * (single ? 2 : 4)), o_ys = take((size_t)nys * DP * (single ? 2 : 4));
-  const size_t o_xn = take((size_t)nxs * 4), o_yn = take((size_t)nys * 4), o_scal = take(8);
+  const size_t o_xn = take((size_t)nxs * 4), o_yn = take((size_t)nys * 4), o_scal = take(16 + 2 * 256 * 4);
   // final-product variant: slabs over the reduced axis fill the chip and round the grid to whole
   // rounds of workgroups (one 8-wavefront workgroup per CU, all taking the same time)
   const bool softmax = m.meta_int("chk_softmax", 0) != 0;
@@ -1215,11 +1215,22 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
     if (int rc = launch_raw(m, "keops_chk_colsum_final", (unsigned)((DP + cw - 1) / cw), 1, 256, buf.data(), szp, stream)) return rc;
   }
   // power-of-two scales of the half-precision operands: largest |component| of both arguments
-  if (int e = keops_static_fill_zero(ws + o_scal, 8, stream)) return fail(e, std::string("zero fill failed: ") + hipGetErrorString((hipError_t)e));
+  if (int e = keops_static_fill_zero(ws + o_scal, 16 + 2 * 256 * 4, stream)) return fail(e, std::string("zero fill failed: ") + hipGetErrorString((hipError_t)e));
   {
     const int64_t elems = std::max(nxs, nys) * D;
     const unsigned gb = (unsigned)std::max<int64_t>(1, std::min<int64_t>(2048, (elems + 256 * 8 - 1) / (256 * 8)));
     if (int rc = launch_raw(m, "keops_chk_absmax", gb, 1, 256, buf.data(), psize, stream)) return rc;
+  }
+  // squared distances: when a few rows hold components far beyond the others', the scale follows the bulk of the rows
+  // and those rows are computed pair by pair from the float32 data (kernels/keops_chunk_mfma.h, keops_chk_robust)
+  if (mode == 0 && !single && m.meta_int("chk_robust", 0) != 0) {
+    for (int w = 0; w < 2; w++) {
+      const int64_t rows = w ? nys : nxs;
+      const unsigned gb = (unsigned)std::max<int64_t>(1, std::min<int64_t>(1024, (rows + 31) / 32));
+      const size_t szh = with_which(w);
+      if (int rc = launch_raw(m, "keops_chk_rowhist", gb, 1, 256, buf.data(), szh, stream)) return rc;
+    }
+    if (int rc = launch_raw(m, "keops_chk_robust", 1, 1, 64, buf.data(), psize, stream)) return rc;
   }
   const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
   size_t sz = with_which(0);

@@ -89,7 +89,8 @@ struct ChkParams {
   int pad_;
   i64 nxs, nys;         // rows of the chunked row / column arguments (fewer than nx, ny when a batch dimension is broadcast)
   __bf16* vsplit;       // CHK_SPLIT3: v as three bfloat16 terms, [tile][term][column][CHK_TS positions]
-  float* scal;          // [2] largest |component| of the chunked row / column arguments (bit patterns, keops_chk_absmax)
+  float* scal;          // [2] bound of the |components| of the chunked row / column arguments that sets their scale (keops_chk_absmax,
+                        // keops_chk_robust), then at byte 16 int[2][256]: rows per exponent of their largest component
   KeopsRangeTables rt;  // block-sparse / batch geometry (KEOPS_MC_RANGES)
   const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
 };
@@ -182,6 +183,66 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_absmax(const ChkPara
   }
 }
 
+// Outliers.  One scale per operand means that a single row with a component 2^k times the others' costs every other
+// row k bits, and one component of 1e30 (or an infinite one) leaves nothing of them.  For squared distances (CHK_MODE 0,
+// where single pairs can be recomputed from the float32 rows, chk_fix_near) the scale is therefore taken from the bulk
+// of the rows when the largest component is far beyond it: keops_chk_rowhist counts the rows by the exponent of their
+// largest component (integer atomics: the counts do not depend on the order), keops_chk_robust finds the exponent E
+// below which all but max(4, n / 1024) rows lie and, when the largest component exceeds 64 * 2^(E+1), replaces the bound
+// by 8 * 2^(E+1).  Rows that then leave the half-precision range get a NaN norm from keops_chk_prep, which sends every
+// pair they take part in through chk_fix_near: they cost D operations per pair, the other rows keep their accuracy.
+// Data without such rows (largest component within 64 times the bulk's) are scaled exactly as before.
+#ifndef CHK_ROBUST
+#define CHK_ROBUST 1
+#endif
+#define CHK_HIST(scal) (reinterpret_cast<int*>(scal) + 4)
+extern "C" __global__ void __launch_bounds__(256) keops_chk_rowhist(const ChkParams P, int which) {
+  __shared__ int h[256];
+  h[threadIdx.x] = 0;
+  __syncthreads();
+  const i64 n = which ? P.nys : P.nxs;
+  const T* src = P.arg[which ? CHK_YARG : CHK_XARG];
+  // one row per group of 8 lanes
+  const int q = threadIdx.x & 7;
+  for (i64 row = ((i64)blockIdx.x * 256 + threadIdx.x) >> 3; row < n; row += (i64)gridDim.x * 32) {
+    float m = 0.f;
+    bool odd = false;  // NaN or infinite
+    for (int c = q; c < CHK_D; c += 8) {
+      const float a = __builtin_fabsf((float)src[row * CHK_D + c]);
+      odd |= !(a < __builtin_inff());
+      m = __builtin_fmaxf(m, a);
+    }
+    unsigned key = odd ? 255u : ((__float_as_uint(m) >> 23) & 0xffu);
+#pragma unroll
+    for (int o = 4; o > 0; o >>= 1) {
+      const unsigned other = (unsigned)__shfl_xor((int)key, o, 8);
+      key = other > key ? other : key;
+    }
+    if (q == 0) atomicAdd(&h[key], 1);
+  }
+  __syncthreads();
+  if (h[threadIdx.x] != 0) atomicAdd(CHK_HIST(P.scal) + which * 256 + threadIdx.x, h[threadIdx.x]);
+}
+
+extern "C" __global__ void __launch_bounds__(64) keops_chk_robust(const ChkParams P) {
+  if (threadIdx.x >= 2) return;
+  const int which = threadIdx.x;
+  const i64 n = which ? P.nys : P.nxs;
+  const int* h = CHK_HIST(P.scal) + which * 256;
+  i64 budget = n / 1024 > 4 ? n / 1024 : 4;
+  if (budget > n / 2) budget = n / 2;
+  i64 cum = 0;
+  int E = 255;
+  for (int e = 0; e < 256; e++) {
+    cum += h[e];
+    if (cum >= n - budget) { E = e; break; }
+  }
+  if (E >= 254 - 7) return;  // the bulk itself is huge or not finite: nothing to protect
+  const float bulk = __uint_as_float((unsigned)(E + 1) << 23);  // every row but the budget has components below this
+  const float top = P.scal[which];
+  if (!(top <= 64.f * bulk)) P.scal[which] = 8.f * bulk;
+}
+
 // Power of two that brings components bounded by B into [2^12, 2^13) (1 for B = 0, clamped to 2^+-60): the split
 // terms then sit high in the half-precision range (lo terms stay normal down to components 2^-15 of the largest,
 // below that they lose absolute accuracy 2^-25 against a largest component of 2^12) and nothing can overflow
@@ -215,6 +276,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
   const float inv = 1.0f / (float)P.nys;
   const float scale = ((CHK_MODE == 0 && !which) ? -2.0f : 1.0f) * chk_operand_scale(P.scal, which);
   float nrm = 0.f;
+  bool over = false;
   for (int c0 = q * 4; c0 < CHK_DPAD && live; c0 += CHK_LPR * 4) {
     chk_h4 hi, lo;
 #pragma unroll
@@ -227,6 +289,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
       }
       nrm += v * v;
       v *= scale;
+      over |= !(__builtin_fabsf(v) < 65504.f);  // leaves the half-precision range (or is not a number)
       hi[e] = (_Float16)v;
       lo[e] = (_Float16)(v - (float)hi[e]);
     }
@@ -235,6 +298,12 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
   }
 #pragma unroll
   for (int o = CHK_LPR / 2; o > 0; o >>= 1) nrm += __shfl_xor(nrm, o, CHK_LPR);
+  // a row that does not fit the half-precision operand: its norm says so, and chk_fix_near computes its pairs from the
+  // float32 rows
+  int ov = over ? 1 : 0;
+#pragma unroll
+  for (int o = CHK_LPR / 2; o > 0; o >>= 1) ov |= __shfl_xor(ov, o, CHK_LPR);
+  if (ov && CHK_ROBUST) nrm = __builtin_nanf("");
   if (CHK_MODE == 0 && live && q == 0) (which ? P.yn : P.xn)[row] = nrm;
 }
 
@@ -263,12 +332,21 @@ __device__ __forceinline__ void chk_fix_near(const ChkParams& P, float (&sv)[NV]
   float m = sv[0];
 #pragma unroll
   for (int u = 1; u < NV; u++) m = __builtin_fminf(m, sv[u]);
+  // (comparisons written so that a NaN - a row that left the half-precision range, keops_chk_prep - takes the slow path)
+#if CHK_ROBUST
+  if (__builtin_expect(!keops_any(!(m >= near_bound)), 1)) return;
+#else
   if (__builtin_expect(!keops_any(m < near_bound), 1)) return;
+#endif
   unsigned mask = 0u;
 #pragma unroll
   for (int u = 0; u < NV; u++) {
     const int v = v0 + u, r = 8 * (v >> 2) + 4 * half + (v & 3);
+#if CHK_ROBUST
+    if (r < n && !(sv[u] >= CHK_NEAR * (xn + yn_s[r]))) mask |= 1u << u;
+#else
     if (r < n && sv[u] < CHK_NEAR * (xn + yn_s[r])) mask |= 1u << u;
+#endif
   }
   const T* x = P.arg[CHK_XARG] + ix * CHK_D;
   while (mask != 0u) {

@@ -584,12 +584,13 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
                 chk_mode=mode, chk_qb=32 * waves // nc, chk_final=int(final is not None), chk_softmax=int(softmax is not None),
                 chk_xarg=xvar.ind, chk_yarg=yvar.ind, ranges=int(irregular), chk_split3=int(split3 and config.chunk_presplit),
                 chk_vcols=0 if wvar is None else -(-wvar.dim // 32) * 32, nops=L.count_ops(outs),
-                chk_single=int(bool(half_data)))
+                chk_single=int(bool(half_data)), chk_robust=int(config.chunk_robust and mode == 0 and not half_data))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
            f"typedef float T;\ntypedef {dtypeacc} TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
            '#include "keops_common.h"']
     defs = dict(
         KEOPS_NARGS=nargs, CHK_D=D, CHK_DPAD=dpad, CHK_MODE=mode, CHK_XARG=xvar.ind, CHK_YARG=yvar.ind, CHK_WAVES=waves, CHK_NC=nc,
+        CHK_ROBUST=int(config.chunk_robust),
         KEOPS_DIMX=layout.dimx, KEOPS_DIMY=layout.dimy, KEOPS_DIMY_PAD=dimy_pad, KEOPS_DIMP=layout.dimp,
         KEOPS_DIMFOUT=post.dim, KEOPS_DIMRED=red.dimred, KEOPS_DIMOUT=red.dim, KEOPS_RED_KIND=red.kind,
         KEOPS_RED_KEEP=red.keep, KEOPS_RED_K=red.K, KEOPS_SUM_SCHEME=SUM_SCHEMES[sum_scheme],

@@ -429,6 +429,47 @@ def test_narrow_but_not_local_kernels_meet_parity_on_the_default_path(width, D, 
         assert np.max(np.abs(got - ref) / np.maximum(1, np.abs(ref))) <= 1e-5
 
 
+@pytest.mark.parametrize("case", ["huge_row", "inf_row", "nan_row", "huge_column", "inf_column", "nan_column", "large_rows"])
+@pytest.mark.parametrize("formula,D", [("Exp(-SqDist(x,y))*b", 64), ("Exp(-Norm2(x-y))*b", 256)])
+def test_rows_far_beyond_the_others_keep_to_themselves(formula, D, case):
+    """One operand scale for the whole cloud would let a single huge (or infinite, or NaN) component spoil every other
+    row.  The scale follows the bulk of the rows, and a row that then leaves the half-precision range is computed pair
+    by pair from the float32 data: the result is what the reference's loops give, row by row (zero kernel values for
+    infinitely distant points, NaN only where a NaN enters)."""
+    from keops_amd import keops_io
+    from keops_amd.torch import Genred
+
+    M, N, Dv = 3000, 4000, 4
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(M, D, device="cuda", generator=gen) / D ** 0.5
+    y = torch.randn(N, D, device="cuda", generator=gen) / D ** 0.5
+    b = torch.randn(N, Dv, device="cuda", generator=gen)
+    value = {"huge": 1e30, "inf": float("inf"), "nan": float("nan")}.get(case.split("_")[0])
+    if case == "large_rows":
+        x[70:73] *= 3e4          # three rows 30 000 times the others: finite, far away, kernel values zero
+        y[99] *= 1e5
+    elif case.endswith("row"):
+        x[77, 5] = value
+    else:
+        y[99, 5] = value
+    al = [f"x=Vi({D})", f"y=Vj({D})", f"b=Vj({Dv})"]
+    got = Genred(formula, al, reduction_op="Sum", axis=1)(x, y, b)
+    assert keops_io.last_loader.module.meta("scheme") == "chunk" and keops_io.last_loader.module.meta("chk_robust") == "1"
+    want = Genred(formula, al, reduction_op="Sum", axis=1, enable_chunks=False)(x, y, b)
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    nan_rows = int(torch.isnan(want).any(dim=1).sum())
+    assert nan_rows == {"nan_row": 1, "nan_column": M}.get(case, 0)
+    if nan_rows < M:
+        ok = ~torch.isnan(want)
+        scale = Genred(formula, al, reduction_op="Sum", axis=1, enable_chunks=False)(x, torch.nan_to_num(y), b.abs())
+        err = ((got - want).abs() / scale.clamp_min(1e-30))[ok]
+        assert float(err.max()) <= 1e-5
+        if case in ("huge_row", "inf_row"):
+            assert float(got[77].abs().max()) == 0.0
+        if case == "large_rows":
+            assert float(got[70:73].abs().max()) == 0.0
+
+
 def test_results_do_not_depend_on_what_the_workspace_held_before():
     """The pre-pass (column sums, operand copies) lives in a workspace that is reused from call to call: a call must
     give the same bits on a fresh workspace and after another call of the same module has left its data there."""
