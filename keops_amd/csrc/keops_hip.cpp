@@ -965,7 +965,8 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
   const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(512, nr / 64));
-  const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
+  // (two more rows of colpart: medians and flag of keops_knn_centre)
+  const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)(nparts + 2) * DP * 4);
   const int64_t RW = DP * (m.meta_int("knn_split", 0) ? 2 : 1);  // bf16 elements per stored row ([hi] or [hi | lo])
   const size_t o_xh = take((size_t)nq * RW * 2), o_yh = take((size_t)nr * RW * 2);
   const size_t o_xkey = take((size_t)nq * 4), o_ykey = take((size_t)nr * 4);
@@ -1003,6 +1004,8 @@ int launch_knn(Module& m, int64_t nq, int64_t nr, const void* xq, const void* yr
   // pre-pass: centring, bf16 copies, keys
   if (int rc = run("keops_knn_colsum", (unsigned)nparts, 1, 256, HS)) return rc;
   if (int rc = run("keops_knn_colsum_final", 1, 1, 256, with_int(nparts))) return rc;
+  if (int rc = run("keops_knn_centre", (unsigned)D, 1, 256, with_int(nparts))) return rc;
+  if (int rc = run("keops_knn_centre_apply", 1, 1, 256, with_int(nparts))) return rc;
   const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
   if (int rc = run("keops_knn_prep", (unsigned)((nq * lpr + 255) / 256), 1, 256, with_int(0))) return rc;
   if (int rc = run("keops_knn_prep", (unsigned)((nr * lpr + 255) / 256), 1, 256, with_int(1))) return rc;
@@ -1081,7 +1084,8 @@ int launch_knn_ranges(Module& m, int64_t nq, int64_t nr, const void* xq, const v
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
   const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(512, nr / 64));
-  const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
+  // (two more rows of colpart: medians and flag of keops_knn_centre)
+  const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)(nparts + 2) * DP * 4);
   const int64_t RW = DP * (m.meta_int("knn_split", 0) ? 2 : 1);
   const size_t o_xh = take((size_t)nq * RW * 2), o_yh = take((size_t)nr * RW * 2);
   const size_t o_xkey = take((size_t)nq * 4), o_ykey = take((size_t)nr * 4);
@@ -1101,6 +1105,8 @@ int launch_knn_ranges(Module& m, int64_t nq, int64_t nr, const void* xq, const v
   auto with_int = [&](int v) { std::memcpy(p.extra, &v, 4); return HS + 4; };
   if (int rc = run("keops_knn_colsum", (unsigned)nparts, 256, HS)) return rc;
   if (int rc = run("keops_knn_colsum_final", 1, 256, with_int(nparts))) return rc;
+  if (int rc = run("keops_knn_centre", (unsigned)D, 256, with_int(nparts))) return rc;
+  if (int rc = run("keops_knn_centre_apply", 1, 256, with_int(nparts))) return rc;
   const int64_t lpr = DP / 4 <= 4 ? 4 : (DP / 4 <= 8 ? 8 : (DP / 4 <= 16 ? 16 : (DP / 4 <= 32 ? 32 : 64)));
   if (int rc = run("keops_knn_prep", (unsigned)((nq * lpr + 255) / 256), 256, with_int(0))) return rc;
   if (int rc = run("keops_knn_prep", (unsigned)((nr * lpr + 255) / 256), 256, with_int(1))) return rc;

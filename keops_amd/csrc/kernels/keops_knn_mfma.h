@@ -172,6 +172,7 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_colsum(const KnnPara
 extern "C" __global__ void __launch_bounds__(256) keops_knn_colsum_final(const KnnParams P, int nparts) {
   __shared__ float part[256];
   if (KNN_I8 && P.scal != nullptr && threadIdx.x < 4) P.scal[threadIdx.x] = 0u;
+  if (threadIdx.x == 0) *reinterpret_cast<unsigned*>(P.colpart + (i64)(nparts + 1) * KNN_DPAD) = 0u;  // keops_knn_centre
   constexpr int RG = 256 / KNN_CW;
   const int cw = threadIdx.x % KNN_CW, rg = threadIdx.x / KNN_CW;
   for (int c0 = 0; c0 < KNN_DPAD; c0 += KNN_CW) {
@@ -189,6 +190,62 @@ extern "C" __global__ void __launch_bounds__(256) keops_knn_colsum_final(const K
     }
     __syncthreads();
   }
+}
+
+// The centre only has to lie inside the cloud: the filters' error bounds grow with the centred norms, the result does
+// not depend on it.  The mean does not when a few references are far away (one point at 1e30 moves it by 1e30 / n,
+// and every centred point is then that number: no neighbour would be found; one infinite component makes it NaN).
+// keops_knn_centre takes, per component, the median and the quartiles of 1024 evenly spaced references (bitonic sort
+// in LDS, values that are not finite last) and raises a flag when the mean is further than four interquartile ranges
+// from the median (or not a number); keops_knn_centre_apply then replaces every mean by the median.  Ordinary data keep
+// their mean, bit for bit.  Scratch: row nparts of colpart holds the medians, the first word of row nparts + 1 the flag.
+extern "C" __global__ void __launch_bounds__(256) keops_knn_centre(const KnnParams P, int nparts) {
+  __shared__ float v[1024];
+  __shared__ int nfin;
+  const int c = blockIdx.x, tid = threadIdx.x;
+  if (c >= KNN_D) return;
+  if (tid == 0) nfin = 0;
+  __syncthreads();
+  const i64 ns = P.nr < 1024 ? P.nr : 1024, step = P.nr / ns;
+  int mine = 0;
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    const int k = tid + 256 * t;
+    float a = __builtin_inff();
+    if (k < ns) {
+      const float y = P.yr[(i64)k * step * KNN_D + c];
+      if (__builtin_fabsf(y) < __builtin_inff()) { a = y; mine++; }
+    }
+    v[k] = a;
+  }
+  atomicAdd(&nfin, mine);
+  __syncthreads();
+  for (int k = 2; k <= 1024; k <<= 1)
+    for (int j = k >> 1; j > 0; j >>= 1) {
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+        const int i = tid + 256 * t, l = i ^ j;
+        if (l > i) {
+          const float a = v[i], b = v[l];
+          const bool up = (i & k) == 0;
+          if ((a > b) == up) { v[i] = b; v[l] = a; }
+        }
+      }
+      __syncthreads();
+    }
+  if (tid == 0) {
+    const int n = nfin;
+    const float med = n > 0 ? v[(n - 1) / 2] : 0.f, iqr = n > 0 ? v[(3 * n) / 4 < n ? (3 * n) / 4 : n - 1] - v[n / 4] : 0.f;
+    const float mean = P.colsum[c] / (float)P.nr;
+    P.colpart[(i64)nparts * KNN_DPAD + c] = med;
+    if (!(__builtin_fabsf(mean - med) <= 4.f * iqr + 1e-3f * __builtin_fabsf(med) + 1e-30f))
+      atomicOr(reinterpret_cast<unsigned*>(P.colpart + (i64)(nparts + 1) * KNN_DPAD), 1u);
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(256) keops_knn_centre_apply(const KnnParams P, int nparts) {
+  if (*reinterpret_cast<const unsigned*>(P.colpart + (i64)(nparts + 1) * KNN_DPAD) == 0u) return;
+  for (int c = threadIdx.x; c < KNN_D; c += 256) P.colsum[c] = P.colpart[(i64)nparts * KNN_DPAD + c] * (float)P.nr;
 }
 
 // which = 0: queries, 1: references.  One row per group of KNN_LPR lanes, 4 columns per lane.

@@ -75,6 +75,36 @@ def test_knn_gaussian_uncentred_data_and_axis0():
     assert np.array_equal(idx0.cpu().numpy(), ref0.astype(np.int64))
 
 
+@pytest.mark.parametrize("case", ["huge_reference", "infinite_reference", "nan_reference", "references_1e4_times_larger", "huge_query"])
+def test_a_far_or_non_finite_point_does_not_cost_the_others_their_neighbours(case):
+    """The filters work on points centred on the references' mean: one reference at 1e30 moved that mean by 1e30 / N and
+    every centred point became that number (no neighbour found for any query); an infinite one made it NaN.  The centre
+    is now the per-component median of a sample when the mean is far from it (keops_knn_centre): indices and distances
+    equal the reference's loops for every query (a query that is itself at 1e30 has all its distances infinite)."""
+    M, N, D, K = 3000, 40000, 64, 5
+    rng = np.random.default_rng(8)
+    x, y = rng.random((M, D), dtype=np.float32), rng.random((N, D), dtype=np.float32)
+    if case == "huge_reference":
+        y[99, 5] = 1e30
+    elif case == "infinite_reference":
+        y[99, 5] = np.inf
+    elif case == "nan_reference":
+        y[99, 5] = np.nan
+    elif case == "references_1e4_times_larger":
+        y[100:103] *= 1e4
+    else:
+        x[77, 5] = 1e30
+    vals, idx = _knn(D, K)(*to_dev(x, y))
+    assert _uses_mfma_module()
+    ref = cpu_reduc("sqdist", [x, y], M, N, 1, reduction="KMin_ArgKMin", K=K, scheme="direct_sum")
+    keep = np.ones(M, bool)
+    if case == "huge_query":
+        keep[77] = False
+        assert np.all(np.isinf(vals[77].cpu().numpy()))
+    assert np.array_equal(idx.cpu().numpy()[keep], ref[keep, 1::2].astype(np.int64))
+    assert np.array_equal(vals.cpu().numpy()[keep], ref[keep, 0::2])
+
+
 def test_knn_config3_query_subset():
     # headline configuration 3: M=100,000 queries, N=1,000,000 references, D=64, K=10, U[0,1), seed 2
     M, N, D, K = 100_000, 1_000_000, 64, 10
