@@ -25,16 +25,16 @@ def postprocess(out, binding, reduction_op, nout, opt_arg, dtype):
     if reduction_op in ("ArgMin", "ArgMax"):
         return out.long()
     if reduction_op in ("Min_ArgMin", "MinArgMin", "Max_ArgMax", "MaxArgMax"):
-        tmp = out.view(out.shape[:-1] + (2, -1))
+        tmp = out.view(out.shape[:-1] + (2, out.shape[-1] // 2))      # (explicit sizes: a view of no rows cannot infer one)
         return tmp[..., 0, :], tmp[..., 1, :].long()
     if reduction_op == "KMin":
-        out = out.view(out.shape[:-1] + (opt_arg, -1))
+        out = out.view(out.shape[:-1] + (opt_arg, out.shape[-1] // opt_arg))
         return out.squeeze(-1) if out.shape[-1] == 1 else out
     if reduction_op == "ArgKMin":
-        out = out.long().view(out.shape[:-1] + (opt_arg, -1))
+        out = out.long().view(out.shape[:-1] + (opt_arg, out.shape[-1] // opt_arg))
         return out.squeeze(-1) if out.shape[-1] == 1 else out
     if reduction_op in ("KMin_ArgKMin", "KMinArgKMin"):
-        tmp = out.view(out.shape[:-1] + (opt_arg, 2, -1))
+        tmp = out.view(out.shape[:-1] + (opt_arg, 2, out.shape[-1] // (2 * opt_arg)))
         vals, idx = tmp[..., 0, :], tmp[..., 1, :].long()
         if vals.shape[-1] == 1:
             return vals.squeeze(-1), idx.squeeze(-1)

@@ -1631,6 +1631,17 @@ static int launch_on_device(Module& m, int64_t nx, int64_t ny, int tagI, int tag
   h.nslabs = 1;
   h.slab_len = cols_total;
 
+  // nothing to reduce over: every output row is the reduction's neutral element (a sum of no terms, the log-sum-exp
+  // pair (-inf, 0), +inf for a minimum ...), as the reference's loops leave it
+  if (cols_total == 0) {
+    if (m.scheme != "conv")
+      return fail(-1, "the reduced axis is empty: only the general-purpose module (enable_chunks = 0) serves such a call");
+    const int64_t gb = (rows_total + m.block - 1) / m.block;
+    if (int rc = launch(m, "keops_fill_neutral", (unsigned)gb, 1, h, args, stream)) return rc;
+    if (sync) HIP_TRY(hipStreamSynchronize(stream));
+    return 0;
+  }
+
   if (m.scheme == "knn") {
     const bool built_for_ranges = m.meta_int("ranges", 0) != 0;
     const int rowarg = m.meta_int("rowarg", 0), colarg = m.meta_int("colarg", 1);

@@ -211,6 +211,10 @@ def load_keops_hip(tagCPUGPU, tag1D2D, tagHostDevice, use_ranges, device_id_requ
     from . import config
 
     rows_hint = nx if (nx is not None and nx < 64 * 256 * config.block_size) else None
+    if (nx is not None and nx == 0) or (ny is not None and ny == 0):
+        # no pair at all: the general-purpose module writes the reduction's neutral element (the other schemes assume
+        # at least one tile of work)
+        optional_flags = dict(optional_flags, enable_chunks=0)
     # log2 bucket of the pairs per batch when there are few batches: the engine weighs it against the formula
     batch_loop = int(batch[1] * batch[2]).bit_length() if (batch and 0 < batch[0] <= config.knn_batch_max) else 0
     if batch and batch[0] == 0:

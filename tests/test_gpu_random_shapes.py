@@ -62,3 +62,32 @@ def test_random_shape(seed):
         out = Genred("(x|y)*b", var + ["b=Vj(2)"], reduction_op="Sum", axis=1)(xd.double(), yd.double(), bd.double()).cpu()
         ref = (x64 @ y64.T) @ b64
         assert float((out - ref).abs().max()) < 1e-11 * max(1.0, float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("M,N", [(0, 5), (5, 0), (0, 0)])
+def test_no_rows_or_nothing_to_reduce_over(M, N):
+    """An empty output gives an empty result; an empty reduced axis gives every row the reduction's neutral element, as
+    the reference's loops leave it (CpuReduc.py:43-64: Initialize, no pair, Finalize): 0 for a sum, -inf for a
+    log-sum-exp, (+inf, 0) for a minimum with its index, index 0 for the K nearest neighbours.  (The library used to
+    divide by the number of column tiles.)"""
+    import torch
+
+    from keops_amd.torch import Genred
+
+    x, y = torch.randn(M, 3, device="cuda"), torch.randn(N, 3, device="cuda")
+    b, g = torch.randn(N, 2, device="cuda"), torch.tensor([0.5], device="cuda")
+    s = Genred("Exp(-g*SqDist(x,y))*b", ["x=Vi(3)", "y=Vj(3)", "b=Vj(2)", "g=Pm(1)"], reduction_op="Sum", axis=1)(x, y, b, g)
+    lse = Genred("-g*SqDist(x,y)", ["x=Vi(3)", "y=Vj(3)", "g=Pm(1)"], reduction_op="LogSumExp", axis=1)(x, y, g)
+    idx = Genred("SqDist(x,y)", ["x=Vi(3)", "y=Vj(3)"], reduction_op="ArgKMin", axis=1, opt_arg=3)(x, y)
+    vmin, imin = Genred("SqDist(x,y)", ["x=Vi(3)", "y=Vj(3)"], reduction_op="Min_ArgMin", axis=1)(x, y)
+    xh, yh = torch.randn(M, 64, device="cuda"), torch.randn(N, 64, device="cuda")
+    hd = Genred("Exp(-SqDist(x,y))*b", ["x=Vi(64)", "y=Vj(64)", "b=Vj(2)"], reduction_op="Sum", axis=1)(xh, yh, b)
+    kd = Genred("SqDist(x,y)", ["x=Vi(64)", "y=Vj(64)"], reduction_op="KMin_ArgKMin", axis=1, opt_arg=2)(xh, yh)
+    assert tuple(s.shape) == (M, 2) and tuple(lse.shape) == (M, 1) and tuple(idx.shape) == (M, 3)
+    assert tuple(vmin.shape) == (M, 1) and tuple(imin.shape) == (M, 1) and tuple(hd.shape) == (M, 2)
+    assert tuple(kd[0].shape) == (M, 2) and tuple(kd[1].shape) == (M, 2)
+    if M > 0:       # N = 0
+        assert bool((s == 0).all()) and bool((hd == 0).all()) and bool(torch.isneginf(lse).all())
+        assert bool((idx == 0).all()) and bool(torch.isposinf(vmin).all()) and bool((imin == 0).all())
+        assert bool(torch.isposinf(kd[0]).all()) and bool((kd[1] == 0).all())
+
