@@ -1149,7 +1149,8 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
   const int nparts = (int)std::max<int64_t>(1, std::min<int64_t>(128, nys / 64));
-  const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)nparts * DP * 4);
+  // (one more row of colpart: the medians of keops_chk_centre)
+  const size_t o_colsum = take((size_t)DP * 4), o_colpart = take((size_t)(nparts + 1) * DP * 4);
   // one half-precision term per component when the data are half-precision numbers (no lo parts, no centring)
   const bool single = m.meta_int("chk_single", 0) != 0;
   // one half-precision term per component is only exact for data that IS half precision
@@ -1226,6 +1227,12 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
     const int64_t elems = std::max(nxs, nys) * D;
     const unsigned gb = (unsigned)std::max<int64_t>(1, std::min<int64_t>(2048, (elems + 256 * 8 - 1) / (256 * 8)));
     if (int rc = launch_raw(m, "keops_chk_absmax", gb, 1, 256, buf.data(), psize, stream)) return rc;
+  }
+  // squared distances: the centre is the median of a sample when the mean is far from it (a few rows far away)
+  if (mode == 0 && !single && m.meta_int("chk_robust", 0) != 0) {
+    const size_t szc = with_which(nparts);
+    if (int rc = launch_raw(m, "keops_chk_centre", (unsigned)D, 1, 256, buf.data(), szc, stream)) return rc;
+    if (int rc = launch_raw(m, "keops_chk_centre_apply", 1, 1, 256, buf.data(), szc, stream)) return rc;
   }
   // squared distances: when a few rows hold components far beyond the others', the scale follows the bulk of the rows
   // and those rows are computed pair by pair from the float32 data (kernels/keops_chunk_mfma.h, keops_chk_robust)

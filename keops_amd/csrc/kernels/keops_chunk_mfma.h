@@ -163,6 +163,63 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_colsum_final(const C
   }
 }
 
+// The rows are centred to keep the norms, hence the error of the expansion, small: any point inside the cloud will do,
+// and the mean is not one when a few rows are far away (one component of 1e30 moves it by 1e30 / n: every centred row
+// would then leave the half-precision range and be computed pair by pair).  keops_chk_centre takes, per component, the
+// median and the quartiles of 1024 evenly spaced rows of the column variable (bitonic sort in LDS, values that are not
+// finite last) and raises a flag (fourth word of P.scal) when the mean is further than four interquartile ranges from
+// the median, or not a number; keops_chk_centre_apply then replaces every mean by the median.  Ordinary data keep their
+// mean, bit for bit.  Row nparts of colpart holds the medians.
+extern "C" __global__ void __launch_bounds__(256) keops_chk_centre(const ChkParams P, int nparts) {
+  __shared__ float v[1024];
+  __shared__ int nfin;
+  const int c = blockIdx.x, tid = threadIdx.x;
+  if (c >= CHK_D) return;
+  if (tid == 0) nfin = 0;
+  __syncthreads();
+  const T* y = P.arg[CHK_YARG];
+  const i64 ns = P.nys < 1024 ? P.nys : 1024, step = ns > 0 ? P.nys / ns : 1;
+  int mine = 0;
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    const int k = tid + 256 * t;
+    float a = __builtin_inff();
+    if (k < ns) {
+      const float w = (float)y[(i64)k * step * CHK_D + c];
+      if (__builtin_fabsf(w) < __builtin_inff()) { a = w; mine++; }
+    }
+    v[k] = a;
+  }
+  atomicAdd(&nfin, mine);
+  __syncthreads();
+  for (int k = 2; k <= 1024; k <<= 1)
+    for (int j = k >> 1; j > 0; j >>= 1) {
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+        const int i = tid + 256 * t, l = i ^ j;
+        if (l > i) {
+          const float a = v[i], b = v[l];
+          const bool up = (i & k) == 0;
+          if ((a > b) == up) { v[i] = b; v[l] = a; }
+        }
+      }
+      __syncthreads();
+    }
+  if (tid == 0) {
+    const int n = nfin;
+    const float med = n > 0 ? v[(n - 1) / 2] : 0.f, iqr = n > 0 ? v[(3 * n) / 4 < n ? (3 * n) / 4 : n - 1] - v[n / 4] : 0.f;
+    const float mean = P.colsum[c] / (float)P.nys;
+    P.colpart[(i64)nparts * CHK_DPAD + c] = med;
+    if (!(__builtin_fabsf(mean - med) <= 4.f * iqr + 1e-3f * __builtin_fabsf(med) + 1e-30f))
+      atomicOr(reinterpret_cast<unsigned*>(P.scal) + 3, 1u);
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(256) keops_chk_centre_apply(const ChkParams P, int nparts) {
+  if (reinterpret_cast<const unsigned*>(P.scal)[3] == 0u) return;
+  for (int c = threadIdx.x; c < CHK_D; c += 256) P.colsum[c] = P.colpart[(i64)nparts * CHK_DPAD + c] * (float)P.nys;
+}
+
 // Largest |component| of the two chunked arguments: atomic maximum on the bit patterns of non-negative floats
 // (order-independent, hence deterministic).  The host zeroes P.scal before the launch.
 extern "C" __global__ void __launch_bounds__(256) keops_chk_absmax(const ChkParams P) {
