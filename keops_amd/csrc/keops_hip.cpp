@@ -759,6 +759,7 @@ int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* arg
   auto with_nblk = [&]() { std::memcpy(buf.data() + psize, &nblk_r, 4); std::memcpy(buf.data() + psize + 4, &nblk_c, 4); return psize + 8; };
   if (int rc = launch_raw(m, "keops_rad_colsum", (unsigned)nparts, 1, 256, buf.data(), psize, stream)) return rc;
   if (int rc = launch_raw(m, "keops_rad_colsum_final", 1, 1, 64, buf.data(), psize, stream)) return rc;
+  if (int rc = launch_raw(m, "keops_rad_centre", (unsigned)D, 1, 256, buf.data(), psize, stream)) return rc;
   size_t sz = with_which(0);
   if (int rc = launch_raw(m, "keops_rad_bucket", (unsigned)nblk_r, 1, 256, buf.data(), sz, stream)) return rc;
   sz = with_which(1);

@@ -177,6 +177,54 @@ extern "C" __global__ void __launch_bounds__(64) keops_rad_colsum_final(const Ra
   if (c < 4) P.scal[c] = 0u;
 }
 
+// The centre only has to lie inside the cloud (the bound of a tile grows with the centred norms); the mean does not
+// when a few columns are very far away (one at 1e9 cloud radii among 1e6 moves it by 1e3 radii, and every tile is then
+// beyond the bound).  One workgroup per component: median and quartiles of 1024 evenly spaced columns (bitonic sort
+// in LDS, values that are not finite last); a mean further than four interquartile ranges from the median, or not a
+// number, is replaced by the median.  Ordinary data keep their mean.
+extern "C" __global__ void __launch_bounds__(256) keops_rad_centre(const RadParams P) {
+  __shared__ float v[1024];
+  __shared__ int nfin;
+  const int c = blockIdx.x, tid = threadIdx.x;
+  if (c >= RAD_D) return;
+  if (tid == 0) nfin = 0;
+  __syncthreads();
+  const T* y = P.arg[RAD_YARG];
+  const i64 ns = P.ny < 1024 ? P.ny : 1024, step = ns > 0 ? P.ny / ns : 1;
+  int mine = 0;
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    const int k = tid + 256 * t;
+    float a = __builtin_inff();
+    if (k < ns) {
+      const float w = (float)y[(i64)k * step * RAD_D + c];
+      if (__builtin_fabsf(w) < __builtin_inff()) { a = w; mine++; }
+    }
+    v[k] = a;
+  }
+  atomicAdd(&nfin, mine);
+  __syncthreads();
+  for (int k = 2; k <= 1024; k <<= 1)
+    for (int j = k >> 1; j > 0; j >>= 1) {
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+        const int i = tid + 256 * t, l = i ^ j;
+        if (l > i) {
+          const float a = v[i], b = v[l];
+          const bool up = (i & k) == 0;
+          if ((a > b) == up) { v[i] = b; v[l] = a; }
+        }
+      }
+      __syncthreads();
+    }
+  if (tid == 0) {
+    const int n = nfin;
+    const float med = n > 0 ? v[(n - 1) / 2] : 0.f, iqr = n > 0 ? v[(3 * n) / 4 < n ? (3 * n) / 4 : n - 1] - v[n / 4] : 0.f;
+    const float mean = P.colsum[c];
+    if (!(__builtin_fabsf(mean - med) <= 4.f * iqr + 1e-3f * __builtin_fabsf(med) + 1e-30f)) P.colsum[c] = med;
+  }
+}
+
 // |k| |x^|^2 of a point (x^: the point minus the mean of y, in double precision) and its bucket
 __device__ __forceinline__ double rad_centred_norm(const RadParams& P, const T* src) {
   double nrm = 0.0;
