@@ -90,7 +90,10 @@ template <typename A> struct KeopsAcc {
     const bool keep = m > (A)fm;  // false when equal or when m is still -inf
     // both sides still empty (-inf - -inf): the maximum with a finite bound drops the NaN, the factor is 0
     const A d = keops_fmax(keep ? (A)fm - m : m - (A)fm, (A)(-3.0e38f));
-    const A e = (A)keops_red_exp((T)d);
+    A e = (A)keops_red_exp((T)d);
+    // (the maximum above must not drop a value that is not a number: it makes the sums NaN for good, as the reference's
+    // update does, Max_SumShiftExpWeight_Reduction.py:35-61)
+    if (!((A)fm == (A)fm)) e = (A)fm;
 #pragma unroll
     for (int k = 0; k < KEOPS_FD - 1; k++) {
 #if KEOPS_SUM_SCHEME == 2

@@ -34,6 +34,24 @@ def test_logsumexp_sinkhorn_style(M, N, scheme):
     assert np.max(np.abs(got - ref) / np.maximum(1.0, np.abs(ref))) <= 1e-5
 
 
+@pytest.mark.parametrize("D", [3, 64])
+@pytest.mark.parametrize("scheme", ["block_sum", "kahan_scheme"])
+@pytest.mark.parametrize("where", [0, 5, 1000, 1019, 1022])
+def test_logsumexp_of_a_value_that_is_not_a_number_is_not_a_number(where, scheme, D):
+    """The reference's update (Max_SumShiftExpWeight_Reduction.py:35-61) turns the running sum into NaN for good when a
+    pair value is NaN, wherever the column sits: in a group of eight, among the last columns of a tile that are folded
+    one by one, first or last (the per-pair update used to drop such a value, and the sum so far with it)."""
+    from keops_amd.torch import Genred
+
+    M, N = 300, 1023
+    x, y, rng = _xy(M, N, D, 6)
+    x, y = x / np.sqrt(D), y / np.sqrt(D)
+    y[where, 1] = np.nan
+    lse = Genred("-SqDist(x,y)", [f"x=Vi({D})", f"y=Vj({D})"], reduction_op="LogSumExp", axis=1, sum_scheme=scheme)
+    got = lse(*to_dev(x, y))
+    assert bool(torch.isnan(got).all())
+
+
 def test_logsumexp_weighted_and_softmax():
     from keops_amd.torch import Genred
 
