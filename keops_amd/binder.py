@@ -86,6 +86,30 @@ def calibrate(kind, chains, blocks, iters, device_id=0):
     return ms.value, ipw.value
 
 
+def mfma_probe(a_bits, b_bits, acc0=0.0, device_id=0):
+    """out[32][32] = acc0 + a b^T of one v_mfma_f32_32x32x16_bf16 on bfloat16 bit patterns a_bits[32][16], b_bits[32][16]
+    (numpy uint16): keops_calibrate_mfma_probe of csrc/keops_calibrate.h."""
+    import numpy as np
+
+    global _calib
+    if _calib is None:
+        from .csrc import build_lib
+
+        if not os.path.exists(build_lib.CALIB_LIB):
+            build_lib.build()
+        _calib = ctypes.CDLL(build_lib.CALIB_LIB)
+        _calib.keops_calibrate.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 2
+    a = np.ascontiguousarray(a_bits, dtype=np.uint16).reshape(32, 16)
+    b = np.ascontiguousarray(b_bits, dtype=np.uint16).reshape(32, 16)
+    out = np.zeros((32, 32), np.float32)
+    fn = _calib.keops_calibrate_mfma_probe
+    fn.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]
+    rc = fn(int(device_id), a.ctypes.data, b.ctypes.data, float(acc0), out.ctypes.data)
+    if rc != 0:
+        raise KeOpsHipError(f"matrix-core probe failed (code {rc})")
+    return out
+
+
 def last_error():
     return lib().keops_hip_last_error().decode(errors="replace")
 

@@ -29,6 +29,14 @@ extern "C" {
  */
 int keops_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave);
 
+/*
+ * One v_mfma_f32_32x32x16_bf16 on operands given bit for bit (bfloat16 patterns): out[i * 32 + j] = acc0 +
+ * sum_k a[i][k] b[j][k] for a_bits[32][16], b_bits[32][16] (host arrays), as the matrix core adds it.  The tests use it
+ * to pin the model of that adder which the error bound of the matrix-core exponents rests on.  Returns 0 or a negative
+ * code.
+ */
+int keops_calibrate_mfma_probe(int device_id, const unsigned short* a_bits, const unsigned short* b_bits, float acc0, float* out);
+
 #ifdef __cplusplus
 }
 #endif

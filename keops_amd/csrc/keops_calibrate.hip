@@ -621,6 +621,43 @@ static int keops_calibrate_launch(int kind, int chains, int blocks, int iters, f
   return (int)hipGetLastError();
 }
 
+// One v_mfma_f32_32x32x16_bf16 on operands given bit for bit: out[i][j] = acc + sum_k a[i][k] b[j][k], one wavefront.
+// Operand layout of the instruction: lane l holds a[l % 32][8 (l / 32) .. +7] and b[l % 32][8 (l / 32) .. +7]; register v
+// of lane l receives row 8 (v / 4) + 4 (l / 32) + v % 4, column l % 32.
+static __global__ void __launch_bounds__(64) keops_mfma_probe_kernel(const unsigned short* a, const unsigned short* b, float acc0, float* out) {
+  const int lane = threadIdx.x, r = lane & 31, half = lane >> 5;
+  keops_bf16x8 av, bv;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    av[e] = __builtin_bit_cast(__bf16, a[r * 16 + 8 * half + e]);
+    bv[e] = __builtin_bit_cast(__bf16, b[r * 16 + 8 * half + e]);
+  }
+  keops_f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; v++) acc[v] = acc0;
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc, 0, 0, 0);
+#pragma unroll
+  for (int v = 0; v < 16; v++) out[(8 * (v >> 2) + 4 * half + (v & 3)) * 32 + r] = acc[v];
+}
+
+extern "C" int keops_calibrate_mfma_probe(int device_id, const unsigned short* a_bits, const unsigned short* b_bits, float acc0, float* out) {
+  if (!a_bits || !b_bits || !out) return -1;
+  if (hipSetDevice(device_id < 0 ? 0 : device_id) != hipSuccess) return -2;
+  unsigned short* d = nullptr;
+  float* o = nullptr;
+  if (hipMalloc((void**)&d, 2 * 512 * sizeof(unsigned short)) != hipSuccess) return -3;
+  if (hipMalloc((void**)&o, 1024 * sizeof(float)) != hipSuccess) { (void)hipFree(d); return -3; }
+  int rc = 0;
+  if (hipMemcpy(d, a_bits, 512 * 2, hipMemcpyHostToDevice) != hipSuccess || hipMemcpy(d + 512, b_bits, 512 * 2, hipMemcpyHostToDevice) != hipSuccess) rc = -4;
+  if (rc == 0) {
+    hipLaunchKernelGGL(keops_mfma_probe_kernel, dim3(1), dim3(64), 0, nullptr, d, d + 512, acc0, o);
+    if (hipGetLastError() != hipSuccess || hipMemcpy(out, o, 1024 * sizeof(float), hipMemcpyDeviceToHost) != hipSuccess) rc = -5;
+  }
+  (void)hipFree(d);
+  (void)hipFree(o);
+  return rc;
+}
+
 extern "C" int keops_calibrate(int device_id, int kind, int chains, int blocks, int iters, double* ms, double* instr_per_wave) {
   if (!ms || !instr_per_wave || blocks <= 0 || iters <= 0) return -1;
   if (hipSetDevice(device_id < 0 ? 0 : device_id) != hipSuccess) return -2;
