@@ -24,6 +24,11 @@ extern "C" {
  *   (workgroups of 8 wavefronts, 32 rows of 256 components per wavefront in registers as hi and lo half-precision
  *   operands, 32-row tiles streamed through LDS, 48 v_mfma_f32_32x32x16_f16 per round and wavefront, no vector
  *   work), chains = 0: every operand the same constant, 1: random operands with the magnitudes of real data.
+ *   kind 10: the Gaussian pair with every operation rounded on its own (12 instructions), `chains` = 1, 2, 4 pairs
+ *   advanced statement by statement (11, 12: one / two pairs with log2(e) in a scalar register); kind 11: written-out
+ *   instruction sequences at the rate of one kind of instruction each, `chains` = sequence 0 .. 12 (keops_valu_seq_loop);
+ *   kind 12: the stream of the Gaussian sweep alone (workgroups of 8 wavefronts: 4 v_mfma_f32_32x32x16_bf16 per 32
+ *   pairs, v_exp_f32 and `chains` = 1, 4, 8 v_fmac_f32 per pair; counted: the v_exp_f32).
  * Measurement aid without counterpart in the reference; used by bench.py --valu-calibration / --mfma-calibration.
  * Returns 0, or a negative code (bad arguments, device, allocation, events, kind or chains out of range).
  */
