@@ -1237,7 +1237,7 @@ int launch_chunk(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   }
   // squared distances: when a few rows hold components far beyond the others', the scale follows the bulk of the rows
   // and those rows are computed pair by pair from the float32 data (kernels/keops_chunk_mfma.h, keops_chk_robust)
-  if (mode == 0 && !single && m.meta_int("chk_robust", 0) != 0) {
+  if (!single && m.meta_int("chk_robust", 0) != 0) {
     for (int w = 0; w < 2; w++) {
       const int64_t rows = w ? nys : nxs;
       const unsigned gb = (unsigned)std::max<int64_t>(1, std::min<int64_t>(1024, (rows + 31) / 32));

@@ -297,7 +297,15 @@ extern "C" __global__ void __launch_bounds__(64) keops_chk_robust(const ChkParam
   if (E >= 254 - 7) return;  // the bulk itself is huge or not finite: nothing to protect
   const float bulk = __uint_as_float((unsigned)(E + 1) << 23);  // every row but the budget has components below this
   const float top = P.scal[which];
-  if (!(top <= 64.f * bulk)) P.scal[which] = 8.f * bulk;
+  // Squared distances: rows that leave the half-precision range are computed pair by pair, so the scale can follow
+  // the bulk closely.  Scalar products have no such path: there the scale only lets go of the largest component when
+  // it is 2^20 times the bulk's (the other rows would keep fewer than 17 bits), and rows up to that ratio stay
+  // representable; beyond it a row overflows to infinity in its own results and leaves the others theirs.
+  if (CHK_MODE == 0) {
+    if (!(top <= 64.f * bulk)) P.scal[which] = 8.f * bulk;
+  } else {
+    if (!(top <= 1048576.f * bulk)) P.scal[which] = 131072.f * bulk;
+  }
 }
 
 // Power of two that brings components bounded by B into [2^12, 2^13) (1 for B = 0, clamped to 2^+-60): the split
@@ -348,7 +356,8 @@ extern "C" __global__ void __launch_bounds__(256) keops_chk_prep(const ChkParams
       v *= scale;
       over |= !(__builtin_fabsf(v) < 65504.f);  // leaves the half-precision range (or is not a number)
       hi[e] = (_Float16)v;
-      lo[e] = (_Float16)(v - (float)hi[e]);
+      // (an infinite hi part has no remainder: infinity minus infinity would turn every product of the row into NaN)
+      lo[e] = __builtin_fabsf((float)hi[e]) < __builtin_inff() ? (_Float16)(v - (float)hi[e]) : (_Float16)0.0f;
     }
     *reinterpret_cast<chk_h4*>(dst + row * CHK_RW + c0) = hi;
     if (!CHK_SINGLE) *reinterpret_cast<chk_h4*>(dst + row * CHK_RW + CHK_DPAD + c0) = lo;

@@ -584,7 +584,7 @@ def generate_chunk_plugin(red, match, dtypeacc, sum_scheme, nargs, irregular=Fal
                 chk_mode=mode, chk_qb=32 * waves // nc, chk_final=int(final is not None), chk_softmax=int(softmax is not None),
                 chk_xarg=xvar.ind, chk_yarg=yvar.ind, ranges=int(irregular), chk_split3=int(split3 and config.chunk_presplit),
                 chk_vcols=0 if wvar is None else -(-wvar.dim // 32) * 32, nops=L.count_ops(outs),
-                chk_single=int(bool(half_data)), chk_robust=int(config.chunk_robust and mode == 0 and not half_data))
+                chk_single=int(bool(half_data)), chk_robust=int(config.chunk_robust and not half_data))
     src = ["//@keops " + " ".join(f"{k}={v}" for k, v in meta.items()), f"// reduction: {red!r}",
            f"typedef float T;\ntypedef {dtypeacc} TACC;", f"#define KEOPS_MC_RANGES {int(irregular)}",
            '#include "keops_common.h"']

@@ -470,6 +470,37 @@ def test_rows_far_beyond_the_others_keep_to_themselves(formula, D, case):
             assert float(got[70:73].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("case", ["row_1e4_times_larger", "huge_row", "infinite_row"])
+def test_scalar_product_formulas_keep_the_other_rows_when_one_row_is_far_larger(case):
+    """Scalar products have no pair-by-pair path: their operand scale lets go of the largest component only when it is
+    2^20 times the bulk's (one component of 1e30 used to leave every other row a quarter wrong); a row 10 000 times the
+    others is still represented, rows beyond the ratio overflow in their own results only."""
+    from keops_amd import keops_io
+    from keops_amd.torch import Genred
+
+    M, N, D, Dv = 3000, 4000, 64, 4
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(M, D, device="cuda", generator=gen) / 8
+    y = torch.randn(N, D, device="cuda", generator=gen) / 8
+    b = torch.randn(N, Dv, device="cuda", generator=gen)
+    if case == "row_1e4_times_larger":
+        x[77] *= 1e4
+    else:
+        x[77, 5] = 1e30 if case == "huge_row" else float("inf")
+    al = [f"x=Vi({D})", f"y=Vj({D})", f"b=Vj({Dv})"]
+    others = torch.ones(M, dtype=torch.bool, device="cuda")
+    others[77] = False
+    for formula, red, kw in (("Exp((x|y))*b", "Sum", {}), ("(x|y)", "SumSoftMaxWeight", dict(formula2="b"))):
+        got = Genred(formula, al, reduction_op=red, axis=1, **kw)(x, y, b)
+        assert keops_io.last_loader.module.meta("scheme") == "chunk"
+        want = Genred(formula, al, reduction_op=red, axis=1, enable_chunks=False, **kw)(x, y, b)
+        assert bool(torch.isfinite(want[others]).all()) and bool(torch.isfinite(got[others]).all())
+        rel = (got - want).abs().max(dim=1).values / want.abs().max(dim=1).values
+        assert float(rel[others].max()) <= 1e-5
+        if case == "row_1e4_times_larger" and red == "SumSoftMaxWeight":
+            assert float(rel[77]) <= 1e-5      # (the shift by the row maximum keeps this row finite)
+
+
 def test_results_do_not_depend_on_what_the_workspace_held_before():
     """The pre-pass (column sums, operand copies) lives in a workspace that is reused from call to call: a call must
     give the same bits on a fresh workspace and after another call of the same module has left its data there."""
