@@ -83,6 +83,19 @@ def choose_geometry(red, layout, nops, sizeof_t, nx=None, irregular=False):
     return dict(block=block, rows=rows, tile_j=tile_j, dimy_pad=dimy_pad, unroll=unroll)
 
 
+def _lse_group(red, geo, nops):
+    """Columns folded per running-maximum update of the log-sum-exp (KEOPS_LSE_GROUP).  A group inlines that many
+    evaluations of the formula per output row of a lane: worth it while the update (17.7 against 12.5 instructions
+    per pair) weighs against the formula, and a burden on the compiler when the formula is long (D = 100:
+    6 minutes of compilation with groups of 8, seconds with 1)."""
+    work = nops * geo["rows"]
+    if work > 640:
+        return 1
+    if work > 160:
+        return min(2, config.lse_group)
+    return config.lse_group if (red.formula.dim <= 2 and geo["rows"] <= 2) else min(4, config.lse_group)
+
+
 def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=None, geometry=None, irregular=False):
     """HIP source of the kernel module for a reduction; returns (source, meta dict)."""
     sizeof_t = 8 if dtype == "double" else 4
@@ -118,7 +131,7 @@ def generate_plugin(red, dtype, dtypeacc, sum_scheme, use_fast_math, nargs, nx=N
         KEOPS_DIMP=layout.dimp, KEOPS_DIMFOUT=red.formula.dim, KEOPS_DIMRED=red.dimred, KEOPS_DIMOUT=red.dim,
         KEOPS_RED_KIND=red.kind, KEOPS_RED_KEEP=red.keep, KEOPS_RED_K=red.K, KEOPS_SUM_SCHEME=SUM_SCHEMES[sum_scheme],
         KEOPS_BLOCK=geo["block"], KEOPS_ROWS=geo["rows"], KEOPS_TILE_J=geo["tile_j"], KEOPS_UNROLL_J=geo["unroll"],
-        KEOPS_LSE_GROUP=config.lse_group if (red.formula.dim <= 2 and geo["rows"] <= 2) else min(4, config.lse_group),
+        KEOPS_LSE_GROUP=_lse_group(red, geo, nops),
         KEOPS_NROWVARS=len(layout.rowvars), KEOPS_NCOLVARS=len(layout.colvars), KEOPS_NPARVARS=len(layout.parvars),
     )
     src += [f"#define {k} {v}" for k, v in defs.items()]
