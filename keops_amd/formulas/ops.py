@@ -1470,6 +1470,36 @@ def TensorProd(a, b):
     return TensorProdNode(as_op(a), as_op(b))
 
 
+class DifferenceMatrixNode(Op):
+    """DifferenceMatrix(x, y): out[j*dim(x)+i] = x_i - y_j, the table of differences that
+    LazyTensor.difference_matrix asks for (pykeops/common/lazy_tensor.py:1591-1597; the reference's formula layer holds
+    no such operation, its definition is the one of pykeops/sandbox/test_soft_dtw_kernel_dissmatrix.py:238-267)."""
+
+    name = "DifferenceMatrix"
+    __slots__ = ()
+
+    def __init__(self, x, y):
+        super().__init__((x, y), (), x.dim * y.dim)
+
+    def lower(self, L, kids):
+        x, y = kids
+        return [L.sub(s, t) for t in y for s in x]
+
+    def diff_t(self, v, gradin):
+        x, y = self.children
+        n, m = x.dim, y.dim
+        # gradin viewed as an (m x n) row-major table G: dx_i = sum_j G[j][i], dy_j = -sum_i G[j][i]
+        rows = [Extract(gradin, j * n, n) for j in range(m)]
+        gx, gy = rows[0], Sum(rows[0])
+        for r in rows[1:]:
+            gx, gy = Add(gx, r), Concat(gy, Sum(r))
+        return Add(x.diff_t(v, gx), y.diff_t(v, Minus(gy)))
+
+
+def DifferenceMatrix(x, y):
+    return DifferenceMatrixNode(as_op(x), as_op(y))
+
+
 def _ints(t, what):
     try:
         return tuple(int(x) for x in t)
@@ -1615,7 +1645,7 @@ BUILDERS = dict(
     IfElse=IfElse, Clamp=Clamp, ClampInt=ClampInt, DiffClampInt=DiffClampInt, Mod=Mod, Sum=Sum, SumT=SumT,
     Scalprod=Scalprod, Concat=Concat, Extract=Extract, ExtractT=ExtractT, OneHot=OneHot, Max=Max, Min=Min,
     ArgMax=ArgMax, ArgMin=ArgMin, MatVecMult=MatVecMult, VecMatMult=VecMatMult, TensorProd=TensorProd,
-    TensorDot=TensorDot, SoftDTW_SqDist=SoftDTW_SqDist,
+    TensorDot=TensorDot, SoftDTW_SqDist=SoftDTW_SqDist, DifferenceMatrix=DifferenceMatrix,
     GradSoftDTW_SqDist=lambda x, y, g: GradSoftDTWSqDistNode(as_op(x), as_op(y), as_op(g)),
     BSpline_Impl=lambda knots, x, order: BSplineImplNode(as_op(knots), as_op(x), order),
 )

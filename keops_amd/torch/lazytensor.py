@@ -439,6 +439,11 @@ class LazyTensor:
     def tensorprod(self, other):
         return self.binary(other, O.TensorProd)
 
+    def difference_matrix(self, other):
+        """Table of differences x_i - y_j of two vectors, of size dim(self) * dim(other), entry (j, i) at j*dim(self)+i
+        (lazy_tensor.py "difference_matrix")."""
+        return self.binary(other, O.DifferenceMatrix)
+
     def diff(self, other, diffin):
         """Symbolic forward-mode differential [d_other self] . diffin (lazy_tensor.py "diff")."""
         other, diffin = self._lift(other), self._lift(diffin)

@@ -131,7 +131,10 @@ def test_vector_ops():
            lambda A, v, w: (A.expand(M, N, 6).reshape(M, N, 2, 3) * w.expand(M, N, 3)[..., None, :]).sum(-1), (0, 2))
     _check("TensorProd(v, w)", al2, t2,
            lambda A, v, w: (v.expand(M, N, 2)[..., :, None] * w.expand(M, N, 3)[..., None, :]).reshape(M, N, 6), (1, 2))
-    _check("WeightedSqNorm(Concat(Concat(v,v),v)+1, v)" if False else "SqNorm2(MatVecMult(A, v))", al2, t2,
+    # entry (j, i) of the table of differences v_i - w_j sits at j*dim(v)+i
+    _check("DifferenceMatrix(v, w)*A", al2, t2,
+           lambda A, v, w: (v.expand(M, N, 2)[..., None, :] - w.expand(M, N, 3)[..., :, None]).reshape(M, N, 6) * A, (0, 1, 2))
+    _check("SqNorm2(MatVecMult(A, v))", al2, t2,
            lambda A, v, w: ((A.expand(M, N, 6).reshape(M, N, 2, 3) * v.expand(M, N, 2)[..., None]).sum(-2) ** 2).sum(-1, keepdim=True), (0, 1))
 
 

@@ -231,3 +231,22 @@ def test_trace_operator_on_lazytensors():
     out = T.sum(dim=1)
     tr = A[:, 0] + A[:, 4] + A[:, 8]
     assert torch.allclose(out[:, 0], tr * b.sum() + 6 * 400, rtol=1e-5)
+
+
+def test_difference_matrix_on_lazytensors():
+    """x.difference_matrix(y) (pykeops/common/lazy_tensor.py:1591-1597): the table x_i[a] - y_j[c] of size
+    dim(x) * dim(y), entry (c, a) at c*dim(x)+a, forward and both gradients against dense torch in float64."""
+    from keops_amd.torch import Vi, Vj
+
+    gen = torch.Generator(device="cuda").manual_seed(13)
+    x = torch.rand(300, 4, device="cuda", dtype=torch.float64, generator=gen, requires_grad=True)
+    y = torch.rand(400, 3, device="cuda", dtype=torch.float64, generator=gen, requires_grad=True)
+    w = torch.rand(400, 12, device="cuda", dtype=torch.float64, generator=gen)
+    D = Vi(x).difference_matrix(Vj(y))
+    assert D.ndim == 12
+    out = ((-(D ** 2)).exp() * Vj(w)).sum(dim=1)
+    dense = (torch.exp(-(x[:, None, None, :] - y[None, :, :, None]) ** 2).reshape(300, 400, 12) * w[None]).sum(1)
+    assert torch.allclose(out, dense, rtol=1e-12)
+    e = torch.rand(300, 12, device="cuda", dtype=torch.float64, generator=gen)
+    for got, ref in zip(torch.autograd.grad(out, [x, y], e), torch.autograd.grad(dense, [x, y], e)):
+        assert torch.allclose(got, ref, rtol=1e-10, atol=1e-12)

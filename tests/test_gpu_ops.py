@@ -93,6 +93,8 @@ CASES = {
     "VecMatMult": ("VecMatMult(w, A)", ALM, MAT, lambda A, v, w: (_mat(A) * w.expand(M, N, 3)[..., None, :]).sum(-1), (0, 2)),
     "TensorProd": ("TensorProd(v, w)+A", ALM, MAT,
                    lambda A, v, w: (v.expand(M, N, 2)[..., :, None] * w.expand(M, N, 3)[..., None, :]).reshape(M, N, 6) + A, (1, 2)),
+    "DifferenceMatrix": ("DifferenceMatrix(v, w)*A", ALM, MAT,
+                         lambda A, v, w: (v.expand(M, N, 2)[..., None, :] - w.expand(M, N, 3)[..., :, None]).reshape(M, N, 6) * A, (0, 1, 2)),
     "SqNormIsoDiag": ("SqNormIso(p, x-y)+SqNormDiag(y, x)", AL, STD,
                       lambda x, y, p, b: p * ((x - y) ** 2).sum(-1, keepdim=True) + (y * x * x).sum(-1, keepdim=True), (0, 1, 2)),
     "SymSqNorm": ("SymSqNorm(A, v)", ["A=Vi(0,4)", "v=Vj(1,2)"], [("i", 4, -1, 1), ("j", 2, -1, 1)],
