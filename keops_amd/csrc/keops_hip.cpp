@@ -1350,11 +1350,13 @@ struct FinHeader {
   int32_t nslabs;
   int32_t pad_;
   void* vsplit;
+  int64_t vrows;
   RangeHeader rt;
 };
 
+// vrows: rows of the array v (with batch dimensions: of all its batches; else the reduced size)
 int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args, int tag1D2D, hipStream_t stream,
-                 const RangeLaunch* rg) {
+                 const RangeLaunch* rg, int64_t vrows) {
   const int64_t DV = m.meta_int("fin_dv", 0), NZ = m.meta_int("fin_nz", 1), QB = m.meta_int("fin_qb", 256), TJ = m.tile_j;
   if (DV <= 0 || NZ <= 0 || QB <= 0 || TJ <= 0) return fail(-1, "corrupt final-product module metadata");
   const int64_t row_blocks = rg ? rg->tables.nblocks : (nx + QB - 1) / QB;
@@ -1374,10 +1376,11 @@ int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   FinHeader h{};
   h.nx = nx; h.ny = ny; h.out = out; h.slab_len = len; h.nslabs = (int32_t)nslabs;
   if (rg) h.rt = rg->header(m.nargs);
-  // split-operand variant (dense launches): v rewritten once as three bfloat16 terms, tile by tile
-  const bool split3_kernel = m.meta_int("fin_split3", 0) != 0;  // three-term kernel; dense launches pre-split v
-  const bool split3 = !rg && split3_kernel;
-  const int64_t DVP = (DV + 31) / 32 * 32, ntiles = (ny + TJ - 1) / TJ;
+  // split-operand variant: v rewritten once as three bfloat16 terms, tile by tile (tiles are counted along the
+  // array v, whatever the ranges and batches of the launch)
+  const bool split3 = m.meta_int("fin_split3", 0) != 0;
+  h.vrows = vrows;
+  const int64_t DVP = (DV + 31) / 32 * 32, ntiles = (vrows + TJ - 1) / TJ;
   // sums kept in double (meta fin_acc64): the folds always go to the partial buffer, keops_fin_reduce rounds once
   const bool acc64 = m.meta_int("fin_acc64", 0) != 0;
   if (acc64 && rg) return fail(-1, "corrupt final-product module metadata");
@@ -1396,7 +1399,7 @@ int launch_final(Module& m, int64_t nx, int64_t ny, void* out, void* const* args
   if (split3)
     if (int rc = launch_raw(m, "keops_fin_split", (unsigned)((ntiles * DVP * TJ + 255) / 256), 1, 256, buf.data(), buf.size(), stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev0, stream));
-  if (int rc = launch_raw3(m, split3_kernel ? "keops_fin_main3" : "keops_fin_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)NZ, (unsigned)m.block, buf.data(), buf.size(), stream)) return rc;
+  if (int rc = launch_raw3(m, split3 ? "keops_fin_main3" : "keops_fin_main", (unsigned)row_blocks, (unsigned)nslabs, (unsigned)NZ, (unsigned)m.block, buf.data(), buf.size(), stream)) return rc;
   if (m.timing) HIP_TRY(hipEventRecord(m.ev1, stream));
   if (nslabs > 1 || acc64) {
     const int64_t gb = (nx * DV + 255) / 256;
@@ -1739,7 +1742,10 @@ static int launch_on_device(Module& m, int64_t nx, int64_t ny, int tagI, int tag
       return n;
     };
     if (m.scheme == "final") {
-      if (int rc = launch_final(m, rows_total, cols_total, out, args, tag1D2D, stream, use_ranges ? &rg : nullptr)) return rc;
+      const int varg = m.meta_int("fin_varg", -1);
+      if (varg < 0 || varg >= m.nargs) return fail(-1, "corrupt final-product module metadata");
+      const int64_t vrows = nb > 0 ? arg_rows(varg, tagI == 0 ? S.N : S.M) : cols_total;
+      if (int rc = launch_final(m, rows_total, cols_total, out, args, tag1D2D, stream, use_ranges ? &rg : nullptr, vrows)) return rc;
     } else {
       const int xarg = m.meta_int("chk_xarg", -1), yarg = m.meta_int("chk_yarg", -1);
       if (xarg < 0 || yarg < 0 || xarg >= m.nargs || yarg >= m.nargs) return fail(-1, "corrupt chunk module metadata");

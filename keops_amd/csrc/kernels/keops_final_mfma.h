@@ -48,6 +48,7 @@ struct FinParams {
   int nslabs;
   int pad_;
   __bf16* vsplit;       // keops_fin_split: v as three bfloat16 terms, [tile][term][column][row in tile]
+  i64 vrows;            // rows of the array v (all batches)
   KeopsRangeTables rt;  // block-sparse / batch geometry (KEOPS_MC_RANGES)
   const T* arg[KEOPS_NARGS > 0 ? KEOPS_NARGS : 1];
 };
@@ -229,11 +230,12 @@ extern "C" __global__ void __launch_bounds__(256) keops_fin_fill_neutral(const F
 // float32, and f * v ~ hh + (hm + mh) + (hl + lh + mm) drops terms below 2^-24 |f v| only: float32 accuracy
 // from six v_mfma_f32_32x32x16_bf16 (6 x 32 cycles per 32 x 32 x 16 block) where the float32 instruction
 // v_mfma_f32_32x32x2_f32 needs 8 x 64 cycles.
-//   * Dense launches: keops_fin_split writes v once as [tile][term][column][row in tile] bfloat16, zero past the
-//     last row and column, so that a workgroup stages a tile with straight 16-byte copies.  Block-sparse and
-//     batched launches (ranges start anywhere) split the float32 tile while staging it, one column and 8 rows per
-//     task.  Either way a lane reads the 8 consecutive reduced rows of its B operand (column l % 32, rows
-//     8 (l / 32) ..) with one ds_read_b128 (columns padded to FIN_TS elements: conflict-free);
+//   * keops_fin_split writes v once as [tile][term][column][row in tile] bfloat16, zero past the last row and
+//     column, so that a workgroup stages a tile with straight 16-byte copies; a tile is FIN_TJ consecutive rows of
+//     the array v from a multiple of FIN_TJ on.  Block-sparse and batched launches (ranges start anywhere, a batch
+//     moves its arguments) sweep the tiles that cover a range and give the rows outside it the pair value 0.  A lane
+//     reads the 8 consecutive reduced rows of its B operand (column l % 32, rows 8 (l / 32) ..) with one
+//     ds_read_b128 (columns padded to FIN_TS elements: conflict-free);
 //   * lane l evaluates f for output row l % 32 and the 8 reduced rows 8 (l / 32) .. of a 16-row block -- the A
 //     operand layout -- and splits the 8 values in registers.
 // keops_fin_main above (float32 instruction) remains for modules built without FIN_SPLIT3.
@@ -241,18 +243,16 @@ extern "C" __global__ void __launch_bounds__(256) keops_fin_fill_neutral(const F
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 fin_bf16x8;
 #define FIN_TS (FIN_TJ + 8)            // bfloat16 elements per staged column (padded)
 #define FIN_DVP (FIN_NBTOT * 32)       // columns of the split copy
-#define FIN_PRESPLIT (!KEOPS_MC_RANGES)  // block-sparse / batched launches split the tile while staging it
 
-#if FIN_PRESPLIT
 extern "C" __global__ void __launch_bounds__(256) keops_fin_split(const FinParams P) {
   const i64 e = (i64)blockIdx.x * 256 + threadIdx.x;   // one (tile, column, row in tile)
-  const i64 ntiles = (P.ny + FIN_TJ - 1) / FIN_TJ;
+  const i64 ntiles = (P.vrows + FIN_TJ - 1) / FIN_TJ;
   if (e >= ntiles * FIN_DVP * FIN_TJ) return;
   const int r = (int)(e % FIN_TJ);
   const int c = (int)((e / FIN_TJ) % FIN_DVP);
   const i64 tile = e / ((i64)FIN_TJ * FIN_DVP);
   const i64 j = tile * FIN_TJ + r;
-  const float x = (j < P.ny && c < FIN_DV) ? P.arg[FIN_VARG][j * FIN_DV + c] : 0.f;
+  const float x = (j < P.vrows && c < FIN_DV) ? P.arg[FIN_VARG][j * FIN_DV + c] : 0.f;
   const __bf16 h = (__bf16)x;
   const float r1 = x - (float)h;
   const __bf16 m = (__bf16)r1;
@@ -262,11 +262,12 @@ extern "C" __global__ void __launch_bounds__(256) keops_fin_split(const FinParam
   dst[(i64)FIN_DVP * FIN_TJ] = m;
   dst[(i64)2 * FIN_DVP * FIN_TJ] = l;
 }
-#endif
 
-extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const FinParams P) {
-  __shared__ __attribute__((aligned(16))) __bf16 vt[3 * FIN_VS * FIN_TS];  // [term][column][row], this workgroup's column blocks
-  __shared__ __attribute__((aligned(16))) T ys[FIN_TJ * FIN_DY];            // reduced-index variables of f
+extern "C" __global__ void __launch_bounds__(FIN_BLOCK, 2) keops_fin_main3(const FinParams P) {
+  // two copies of a tile, [term][column][row] of this workgroup's column blocks and the reduced-index variables of f:
+  // a wavefront writes its share of the next tile while the others still read the current one
+  __shared__ __attribute__((aligned(16))) __bf16 vt2[2][3 * FIN_VS * FIN_TS];
+  __shared__ __attribute__((aligned(16))) T ys2[2][FIN_TJ * FIN_DY];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
@@ -324,14 +325,13 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
     first = false;
   };
 
-#if FIN_PRESPLIT
-  // a staged tile: per term FIN_VS columns of FIN_TJ rows, 16-byte chunks of the pre-split copy
+  // a staged tile: per term FIN_VS columns of FIN_TJ rows, 16-byte chunks of the split copy
   constexpr int CPC = FIN_TJ / 8;                         // chunks per column
   constexpr int NCH = 3 * FIN_VS * CPC;                   // chunks per tile
   constexpr int NPF = (NCH + FIN_BLOCK - 1) / FIN_BLOCK;
   uint4 pf[NPF];
-  auto prefetch = [&](i64 j0, i64 jend) {
-    const uint4* base = reinterpret_cast<const uint4*>(P.vsplit + (j0 / FIN_TJ) * 3 * FIN_DVP * FIN_TJ);
+  auto prefetch = [&](i64 tile) {
+    const uint4* base = reinterpret_cast<const uint4*>(P.vsplit + tile * 3 * FIN_DVP * FIN_TJ);
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * FIN_BLOCK;
@@ -341,7 +341,7 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
       pf[u] = (e < NCH && c0 + c < FIN_DVP) ? base[((i64)term * FIN_DVP + c0 + c) * CPC + part] : make_uint4(0u, 0u, 0u, 0u);
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](__bf16* vt) {
 #pragma unroll
     for (int u = 0; u < NPF; u++) {
       const int e = tid + u * FIN_BLOCK;
@@ -352,54 +352,8 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
       }
     }
   };
-#else
-  // no pre-split copy (reduced-index ranges start anywhere): a task is one column and 8 consecutive reduced rows,
-  // 8 coalesced float32 loads prefetched one tile ahead, split and written with one ds_write_b128 per term
-  constexpr int NTASK = FIN_VS * (FIN_TJ / 8);
-  constexpr int NT = (NTASK + FIN_BLOCK - 1) / FIN_BLOCK;
-  float pf[NT * 8];
-  const T* vsrc = P.arg[FIN_VARG];
-  auto prefetch = [&](i64 j0, i64 jend) {
-    const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
-    const i64 jv = G.col(FIN_VARG, j0);
-#pragma unroll
-    for (int u = 0; u < NT; u++) {
-      const int t = tid + u * FIN_BLOCK;
-      const int c = t % FIN_VS, g = t / FIN_VS;
-#pragma unroll
-      for (int e = 0; e < 8; e++) {
-        const int r = 8 * g + e;
-        pf[u * 8 + e] = (t < NTASK && r < n && c0 + c < FIN_DV) ? vsrc[(jv + r) * FIN_DV + c0 + c] : 0.f;
-      }
-    }
-  };
-  auto store_tile = [&]() {
-#pragma unroll
-    for (int u = 0; u < NT; u++) {
-      const int t = tid + u * FIN_BLOCK;
-      if (t < NTASK) {
-        const int c = t % FIN_VS, g = t / FIN_VS;
-        fin_bf16x8 h8, m8, l8;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-          const float x = pf[u * 8 + e];
-          const __bf16 h = (__bf16)x;
-          const float r1 = x - (float)h;
-          const __bf16 m = (__bf16)r1;
-          h8[e] = h;
-          m8[e] = m;
-          l8[e] = (__bf16)(r1 - (float)m);
-        }
-        __bf16* d = vt + c * FIN_TS + 8 * g;
-        *reinterpret_cast<fin_bf16x8*>(d) = h8;
-        *reinterpret_cast<fin_bf16x8*>(d + FIN_VS * FIN_TS) = m8;
-        *reinterpret_cast<fin_bf16x8*>(d + 2 * FIN_VS * FIN_TS) = l8;
-      }
-    }
-  };
-#endif
 
-  int since_fold = 0;
+  int since_fold = 0, cur = 0;
   // folds the reduced rows [jbeg, jend) into the register tiles
   i64 jbeg, jend;
 #if KEOPS_MC_RANGES
@@ -410,22 +364,36 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
   jend = keops_min(P.ny, ((i64)blockIdx.y + 1) * P.slab_len);
   {
 #endif
-  if (jbeg < jend) prefetch(jbeg, jend);
-  for (i64 j0 = jbeg; j0 < jend; j0 += FIN_TJ) {
+  // row of v that holds reduced row j: j + shift (a batch moves its arguments); tiles are counted along v
+  const i64 shift = G.col(FIN_VARG, 0);
+  i64 tile = (jbeg + shift) / FIN_TJ;
+  const i64 tile_end = (jend + shift + FIN_TJ - 1) / FIN_TJ;
+  if (tile < tile_end) prefetch(tile);
+  for (; tile < tile_end; tile++) {
+    const i64 j0 = tile * FIN_TJ - shift;  // reduced row of the tile's first row: before jbeg when the range starts inside
+#if KEOPS_MC_RANGES
+    const int lo = (int)keops_max((i64)0, jbeg - j0);
+#else
+    constexpr int lo = 0;                  // slabs start at multiples of FIN_TJ
+#endif
     const int n = (int)keops_min((i64)FIN_TJ, jend - j0);
-    __syncthreads();  // the previous tile has been consumed by every wavefront
-    store_tile();
+    // (the copy written here was last read two tiles ago, and every wavefront has passed the barrier of the
+    // previous tile since)
+    __bf16* vt = vt2[cur];
+    T* ys = ys2[cur];
+    cur ^= 1;
+    store_tile(vt);
 #pragma unroll
     for (int v = 0; v < KEOPS_NCOLVARS; v++) {
       const int dim = keops_col_dim[v];
-      const T* src = P.arg[keops_col_arg[v]] + G.col(keops_col_arg[v], j0) * dim;
+      const T* src = P.arg[keops_col_arg[v]] + G.col(keops_col_arg[v], j0) * dim;  // rows [lo, n) of it exist
       for (int e = tid; e < n * dim; e += FIN_BLOCK) {
         const int row = e / dim, c = e - row * dim;
-        ys[row * FIN_DY + keops_col_off[v] + c] = src[e];
+        if (row >= lo) ys[row * FIN_DY + keops_col_off[v] + c] = src[e];
       }
     }
     __syncthreads();
-    if (j0 + FIN_TJ < jend) prefetch(j0 + FIN_TJ, jend);
+    if (tile + 1 < tile_end) prefetch(tile + 1);
     if (!wave_live) continue;
 
 #pragma unroll
@@ -446,7 +414,8 @@ extern "C" __global__ void __launch_bounds__(FIN_BLOCK) keops_fin_main3(const Fi
         }
         T fout[1];
         KeopsFormula::eval(xi, yj, p, fout);
-        const float f = jr < n ? fout[0] : 0.f;  // select, never multiply: rows past the end hold garbage
+        // select, never multiply: rows outside the range hold garbage
+        const float f = (jr >= lo && jr < n) ? fout[0] : 0.f;
         const __bf16 h = (__bf16)f;
         const float r1 = f - (float)h;
         const __bf16 m = (__bf16)r1;

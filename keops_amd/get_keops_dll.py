@@ -752,7 +752,7 @@ def generate_final_plugin(red, match, sum_scheme, nargs, irregular=False, acc64=
     pa, pd, po = VarLayout.table(layout.parvars)
     meta = dict(scheme="final", block=64 * waves, rows=1, tile_j=tj, dimred=red.dimred, dimout=red.dim, sizeof_t=4,
                 sizeof_acc=8 if acc64 else 4, nrowvars=len(layout.rowvars), ncolvars=len(layout.colvars) + (0 if vvar in layout.colvars else 1),
-                nparvars=len(layout.parvars), fin_dv=vvar.dim, fin_nb=nb, fin_nz=nz, fin_qb=32 * waves, ranges=int(irregular),
+                nparvars=len(layout.parvars), fin_dv=vvar.dim, fin_varg=vvar.ind, fin_nb=nb, fin_nz=nz, fin_qb=32 * waves, ranges=int(irregular),
                 fin_acc64=int(acc64),
                 fin_split3=int(config.final_split3 and tj % 16 == 0),
                 nops=L.count_ops(outs))

@@ -166,3 +166,41 @@ def test_lazytensor_front_end_and_fallbacks():
     assert np.max(np.abs(got64 - (torch.exp(-0.75 * torch.cdist(xd.double().cpu(), yd.double().cpu()) ** 2) @ b64).numpy())) < 1e-10
     kahan = Genred(FORMULA, _aliases(Dv), reduction_op="Sum", axis=1, sum_scheme="kahan_scheme")(xd, yd, bd, gd)
     assert_sum_parity(kahan.cpu().numpy(), (K @ b64).numpy(), (K @ b64.abs()).numpy())
+
+
+def test_batches_and_ranges_that_start_inside_a_tile_of_the_split_copy():
+    """The staged tiles are cut along the array v from multiples of 32 rows on; a batch of 333 rows or a range
+    [77, 1201) starts and ends inside such a tile, and a broadcast batch dimension of v moves the tiles of a batch
+    without moving its rows of y."""
+    from keops_amd.torch import LazyTensor
+
+    gen = torch.Generator().manual_seed(31)
+    B, H, M, N, Dv = 2, 3, 210, 333, 40
+    x = torch.randn(B, H, M, 3, generator=gen)
+    y = torch.randn(B, H, N, 3, generator=gen)
+    v = torch.randn(B, 1, N, Dv, generator=gen)                      # shared by the second batch dimension
+    x_i, y_j = LazyTensor(x.cuda()[:, :, :, None, :]), LazyTensor(y.cuda()[:, :, None, :, :])
+    v_j = LazyTensor(v.cuda()[:, :, None, :, :])
+    got = ((-((x_i - y_j) ** 2).sum(-1)).exp() * v_j).sum(dim=3).cpu()
+    assert _scheme_used("final")
+    K = torch.exp(-torch.cdist(x.double(), y.double()) ** 2)
+    assert_sum_parity(got.numpy(), (K @ v.double()).numpy(), (K @ v.double().abs()).numpy())
+    # block-sparse: three row ranges, reduced ranges with odd ends, some of them adjacent
+    from keops_amd.torch import Genred
+
+    M, N, Dv = 700, 1500, 72
+    xs, ys, bs, gs = _inputs(M, N, Dv, 32)
+    ranges_i = torch.tensor([[0, 130], [130, 450], [450, 700]], dtype=torch.int32)
+    slices_i = torch.tensor([2, 3, 5], dtype=torch.int32)
+    ranges_j = torch.tensor([[77, 500], [500, 1201], [3, 29], [1000, 1033], [1299, 1500]], dtype=torch.int32)
+    ranges = (ranges_i, slices_i, ranges_j, ranges_j, torch.tensor([1, 2, 3, 4, 5], dtype=torch.int32),
+              torch.tensor([[0, 130], [0, 130], [130, 450], [450, 700], [450, 700]], dtype=torch.int32))
+    out = Genred(FORMULA, _aliases(Dv), reduction_op="Sum", axis=1)(*to_dev(xs, ys, bs, gs), ranges=ranges).cpu().numpy()
+    mask = torch.zeros(M, N, dtype=torch.float64)
+    mask[0:130, 77:1201] = 1
+    mask[130:450, 3:29] = 1
+    mask[450:700, 1000:1033] = 1
+    mask[450:700, 1299:1500] = 1
+    x64, y64, b64 = (torch.from_numpy(t).double() for t in (xs, ys, bs))
+    K = torch.exp(-0.75 * torch.cdist(x64, y64) ** 2) * mask
+    assert_sum_parity(out, (K @ b64).numpy(), (K @ b64.abs()).numpy())
