@@ -709,6 +709,8 @@ int launch_radial(Module& m, int64_t nx, int64_t ny, void* out, void* const* arg
   const int64_t ntiles = (ny + TJ - 1) / TJ, rows_per_wg = 32 * RB * WAVES, row_blocks = (nx + rows_per_wg - 1) / rows_per_wg;
   // slabs over the reduced axis: about 16 workgroups per compute unit, whole tiles per slab
   int64_t nslabs = std::max<int64_t>(1, (16 * (int64_t)m.cu_count + row_blocks - 1) / row_blocks);
+  static const int64_t slab_cols = [] { const char* e = getenv("KEOPS_HIP_RADIAL_SLAB_COLS"); return e ? atoll(e) : 0; }();
+  if (slab_cols > 0) nslabs = std::max<int64_t>(nslabs, (ny + slab_cols - 1) / slab_cols);
   nslabs = std::min<int64_t>(nslabs, std::max<int64_t>(1, ntiles / 8));
   int64_t slab_len = ((ny + nslabs - 1) / nslabs + TJ - 1) / TJ * TJ;
   nslabs = std::max<int64_t>(1, (ny + slab_len - 1) / slab_len);
