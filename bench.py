@@ -387,7 +387,7 @@ def measure(workload, steps, warmup):
                 achieved=achieved, peak=peak, note=note)
 
 
-def side_configs(steps=3, warmup=1):
+def side_configs(steps=3, warmup=2):
     """{workload: {ms, kernel_ms, pairs_per_s, frac, bound, peak}} for the other targets of the hot path, a few steps each."""
     import gc
 

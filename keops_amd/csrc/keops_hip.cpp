@@ -1508,6 +1508,14 @@ void* keops_hip_module_create(int device_id, int nargs, const char* target_file)
     delete m;
     return nullptr;
   }
+  {
+    // The library's own device code (fill, conversion and range-table kernels, the static scratch array) is loaded
+    // on a device at its first use, which takes about 50 ms (the array is 128 MiB): here, once per device, rather
+    // than inside some later launch -- the second call of a block-sparse launch, or one under graph capture.
+    void* sp = nullptr;
+    size_t sb = 0;
+    if (keops_static_scratch(m->device, &sp, &sb) != 0) (void)hipGetLastError();
+  }
   int cus = 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, m->device) == hipSuccess && cus > 0) m->cu_count = cus;
   m->block = m->meta_int("block", 256);
