@@ -1,5 +1,5 @@
 """Cases of the reference's own LazyTensor test files, run on the HIP backend with device tensors and compared
-with dense torch: pykeops/test/test_transpose.py, test_lazytensor_clamp.py, test_sinc.py,
+with dense torch: pykeops/test/test_transpose.py, conv2d.py, test_lazytensor_clamp.py, test_sinc.py,
 test_contiguous_torch.py, test_lazytensor_gaussian_inplace.py, test_lazytensor_grad.py (same shapes, seeds and
 tolerances)."""
 import math
@@ -238,3 +238,29 @@ def test_numpy_lazytensor_and_generic_ops():
     lse = ((Vi(x) * Vj(y)).sum(-1) * Pm(np.array([2.0]))).logsumexp(dim=1)
     refl = np.log(np.exp(2.0 * x @ y.T).sum(1))
     assert np.allclose(lse[:, 0], refl, rtol=1e-10)
+
+
+def test_matmul_with_the_2d_backend_and_two_orders_of_gradients():
+    """pykeops/test/conv2d.py: K @ b through LazyTensor.__matmul__(..., backend="GPU_2D") at 20000 x 30000, and the
+    first and second order gradients with respect to b, against dense torch (same shapes and draws)."""
+    import math
+
+    from keops_amd.torch import LazyTensor
+
+    M, N, D, DV = 20000, 30000, 3, 1
+    torch.manual_seed(0)
+    x = torch.rand(M, 1, D, device="cuda") / math.sqrt(D)
+    y = torch.rand(1, N, D, device="cuda") / math.sqrt(D)
+    b = torch.randn(N, DV, requires_grad=True, device="cuda")
+
+    def fun(keops):
+        if keops:
+            Kxy = (-((LazyTensor(x) - LazyTensor(y)) ** 2).sum(dim=2)).exp()
+            return LazyTensor.__matmul__(Kxy, b, backend="GPU_2D").squeeze()
+        return ((-((x.double() - y.double()) ** 2).sum(dim=2)).exp() @ b.double()).squeeze()
+
+    out = [fun(True), fun(False)]
+    g1 = [torch.autograd.grad((o ** 2).sum(), [b], create_graph=True)[0] for o in out]
+    g2 = [torch.autograd.grad((g ** 2).sum(), [b])[0] for g in g1]
+    for got, ref in zip((out[0], g1[0], g2[0]), (out[1], g1[1], g2[1])):
+        assert torch.allclose(got.double(), ref.double(), rtol=1e-4, atol=1e-5 * float(ref.detach().abs().max()))
